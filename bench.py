@@ -1,0 +1,209 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged decode step on one MI355X.
+
+One "step" is one pass of the decode hot path of a single layer over one batch:
+fused q/k RMSNorm + RoPE + KV-append (one launch), then paged GQA decode attention
+(split kernel + merge kernel).  The default workload is the Llama-3-8B shape:
+batch 64, 32 query / 8 KV heads, head dim 128, context lengths U[512, 8192], chunk 256,
+bf16, all inputs resident in HBM before timing starts.
+
+Prints ONE JSON line.  ``value`` is algorithmic decode-attention bytes divided by the step
+time; ``roofline`` prices the KV-streaming kernel alone, timed with HIP events recorded on
+the launch stream inside the same timed region; ``cpu_baseline`` is the CPU checker
+(``oracle/``) timed on the host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3_decode", "cfg4", "cfg5"])
+    ap.add_argument("--split-tokens", type=int, default=0)
+    ap.add_argument("--subtiles", type=int, default=0, help="16-token sub-tiles per loop iteration (1, 2 or 4)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--attention-only", action="store_true", help="time the attention call alone")
+    return ap.parse_args()
+
+
+def cpu_baseline(case, cfg, sample_requests: int):
+    """Time the CPU checker on the first ``sample_requests`` requests of the same seeded batch."""
+    import torch
+
+    from oracle import paged_attention as oa
+
+    n = min(sample_requests, case.q.size(0))
+    q = case.q[:n].cpu().squeeze(1)
+    rows = case.block_table[:n].cpu()
+    lens = case.kv_lens[:n].cpu()
+    used = rows[rows >= 0].unique().long()
+    # compact the sample's chunks into a small CPU cache (same logical contents)
+    remap = torch.full((case.k_cache.size(0),), -1, dtype=torch.int32)
+    remap[used] = torch.arange(used.numel(), dtype=torch.int32)
+    kc = case.k_cache[used.to(case.k_cache.device)].cpu()
+    vc = case.v_cache[used.to(case.k_cache.device)].cpu()
+    if kc.dtype == torch.uint8:
+        ks = case.k_scales[used.to(case.k_cache.device)].cpu()
+        vs = case.v_scales[used.to(case.k_cache.device)].cpu()
+    else:
+        ks = vs = None
+    bt = torch.where(rows >= 0, remap[rows.clamp(min=0).long()], rows)
+    torch.set_num_threads(os.cpu_count() or 1)
+    times = []
+    for i in range(4):
+        t0 = time.perf_counter()
+        oa.paged_decode_attention(q, kc, vc, lens, bt, k_scales=ks, v_scales=vs)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times[1:])[len(times[1:]) // 2]
+    nbytes = oa.decode_attention_bytes(lens.tolist(), cfg.Hq, cfg.Hkv, cfg.d, cfg.chunk,
+                                       kv_bytes=1 if cfg.fp8 else 2, fp8_scales=cfg.fp8)
+    return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first {n} of {case.q.size(0)} requests of the same seeded batch, fp32 gather + softmax "
+                      f"checker (oracle/paged_attention.py), median of 3 passes after 1 warm-up, {t * 1e3:.1f} ms/pass"}
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build's hot path is a single-GPU kernel path and --gpus "
+              f"{args.gpus} is not supported (no collectives are part of it).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from __graft_entry__ import load_package
+    from oracle import paged_attention as oa
+    from oracle import rope_norm as orn
+
+    mi = load_package()
+    lib = mi._lib.load()  # raises if the HIP library is missing: there is no fallback to measure
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    if args.subtiles:
+        mi.ops.set_tuning("decode_tile_subtiles", args.subtiles)
+
+    cfg = mi.synthetic.CONFIGS[args.workload]
+    case = mi.synthetic.make_decode_case(cfg, dev, on_device_rng=True)
+    if cfg.fp8:
+        k8 = torch.empty(case.k_cache.shape, dtype=torch.uint8, device=dev)
+        v8 = torch.empty_like(k8)
+        case.k_scales = torch.empty(case.k_cache.size(0), cfg.Hkv, dtype=torch.float32, device=dev)
+        case.v_scales = torch.empty_like(case.k_scales)
+        mi.ops.quantize_chunks_fp8(case.k_cache, k8, case.k_scales)
+        mi.ops.quantize_chunks_fp8(case.v_cache, v8, case.v_scales)
+        torch.cuda.synchronize()
+        case.k_cache, case.v_cache = k8, v8
+        torch.cuda.empty_cache()
+
+    lens_host = case.kv_lens.cpu()
+    max_len = int(lens_host.max())
+    gen = torch.Generator().manual_seed(cfg.seed + 1)
+    qw = (1 + 0.02 * torch.randn(cfg.d, generator=gen)).bfloat16().to(dev)
+    kw = (1 + 0.02 * torch.randn(cfg.d, generator=gen)).bfloat16().to(dev)
+    theta = cfg.rope_theta or 500000.0
+    table = orn.rotary_table(max_len + 1, cfg.d, base=theta).to(dev)
+    pos = (case.kv_lens.long() - 1).contiguous()
+    q_in = case.q.clone()
+    out = torch.empty_like(case.q)
+    use_norm = "rms"
+
+    def step():
+        if not args.attention_only:
+            q_in.copy_(case.q)  # the projection's fresh output each step (norm + RoPE work in place)
+            if cfg.fp8:
+                mi.ops.norm_rope_append(q_in, case.k_new, key_out=k_rot, q_weight=qw, k_weight=kw, eps=1e-5,
+                                        norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos)
+                mi.ops.kv_append_decode_fp8(k_rot, case.v_new, case.k_cache, case.v_cache, case.k_scales,
+                                            case.v_scales, case.block_table, case.kv_lens)
+            else:
+                mi.ops.norm_rope_append(q_in, case.k_new, value=case.v_new, q_weight=qw, k_weight=kw, eps=1e-5,
+                                        norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos,
+                                        k_cache=case.k_cache, v_cache=case.v_cache, block_table=case.block_table,
+                                        kv_lens=case.kv_lens)
+        mi.ops.paged_decode_attention(q_in, case.k_cache, case.v_cache, case.kv_lens, case.block_table, out=out,
+                                      max_kv_len=max_len, split_tokens=args.split_tokens,
+                                      k_scales=case.k_scales, v_scales=case.v_scales)
+
+    k_rot = torch.empty_like(case.k_new)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    lib.mi_profile_enable(1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    buf = (ctypes.c_float * args.steps)()
+    n_ev = lib.mi_profile_collect(buf, args.steps)
+    lib.mi_profile_enable(0)
+    kernel_ms = sum(buf[i] for i in range(min(n_ev, args.steps))) / max(1, min(n_ev, args.steps))
+
+    ms_per_step = elapsed * 1e3 / args.steps
+    nbytes = oa.decode_attention_bytes(lens_host.tolist(), cfg.Hq, cfg.Hkv, cfg.d, cfg.chunk,
+                                       kv_bytes=1 if cfg.fp8 else 2, fp8_scales=cfg.fp8)
+    value = nbytes / (ms_per_step * 1e-3) / 1e9
+    achieved = nbytes / (kernel_ms * 1e-3) / 1e9
+
+    result = {
+        "metric": "paged_decode_attention_hbm_GBps",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8-e4m3 KV, bf16 q/out, fp32 accumulate" if cfg.fp8 else "bf16 (fp32 accumulate)",
+        "data": "synthetic",
+        "config": {
+            "workload": cfg.name + (", attention call only" if args.attention_only
+                                    else ", step = fused RMSNorm+RoPE+KV-append then paged decode attention"),
+            "batch": case.q.size(0), "q_heads": cfg.Hq, "kv_heads": cfg.Hkv, "head_dim": cfg.d,
+            "chunk_tokens": cfg.chunk, "kv_tokens_total": int(lens_host.sum()), "kv_len_max": max_len,
+            "algorithmic_bytes_per_step": nbytes,
+        },
+        "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "decode_steps_per_sec": round(1e3 / ms_per_step, 1),
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "paged_decode_split_kernel",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "kernel_ms": round(kernel_ms, 5),
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline:
+        sample = {"cfg1": 4, "cfg2": 64, "cfg3_decode": 64, "cfg4": 1, "cfg5": 16}[args.workload]
+        result["cpu_baseline"] = cpu_baseline(case, cfg, sample)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,195 @@
+/*
+ * mi355_decode.h -- C ABI of libmi355_decode.so
+ *
+ * MI355X (gfx950) kernels for the decode-step hot path of Megatron-Core's dynamic
+ * inference engine: KV-append into the chunked ("paged") KV cache, paged GQA
+ * decode / chunked-prefill attention, and the fused q/k norm + rotary embedding.
+ *
+ * Conventions (all entry points)
+ *  - Every pointer except `stream`, names and returned strings is a DEVICE pointer
+ *    owned by the caller; the library allocates nothing and keeps no pointer.
+ *  - `stream` is a hipStream_t (null = the default stream).  Calls only enqueue
+ *    work: they never synchronise and never read device memory on the host, so they
+ *    can be recorded into a HIP graph.
+ *  - Strides are in ELEMENTS of the tensor they describe unless the name says bytes.
+ *  - Return value: 0 = enqueued; negative = rejected, nothing was launched
+ *    (MI_ERR_*); mi_last_error() gives the message of the calling thread's last
+ *    rejection.
+ *  - KV cache layout is the reference's: key cache = memory_buffer[0, layer],
+ *    value cache = memory_buffer[1, layer], each `[n_chunks, chunk_tokens, Hkv, d]`
+ *    (megatron/core/inference/contexts/dynamic_context.py:296-308,547-564).
+ */
+#ifndef MI355_DECODE_H
+#define MI355_DECODE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  MI_OK = 0,
+  MI_ERR_NULL = -1,
+  MI_ERR_SHAPE = -2,
+  MI_ERR_ALIGN = -3,
+  MI_ERR_UNSUPPORTED = -4,
+  MI_ERR_WORKSPACE = -5,
+  MI_ERR_LAUNCH = -6
+};
+
+enum { MI_KV_BF16 = 0, MI_KV_FP8_E4M3 = 1 };
+enum { MI_NORM_NONE = 0, MI_NORM_RMS = 1, MI_NORM_L2 = 2 };
+
+/* ABI revision of the loaded library. */
+int mi_version(void);
+
+/* Message of the calling thread's most recent rejected call ("" if none). */
+const char* mi_last_error(void);
+
+/* Experiment knobs ("decode_tile_subtiles" = 1|2|4, "prefill_tile_subtiles"). */
+int mi_set_tuning(const char* name, int32_t value);
+
+/*
+ * Kernel timing.  mi_profile_enable(1) makes mi_paged_decode_attention bracket its
+ * KV-streaming kernel with HIP events on the caller's stream; mi_profile_collect waits for
+ * the recorded pairs, writes their durations (milliseconds, HOST pointer) and returns how
+ * many there were.  Keep it off while capturing a graph.
+ */
+int mi_profile_enable(int32_t on);
+int32_t mi_profile_collect(float* out_ms_host, int32_t capacity);
+
+/*
+ * KV-append with explicit per-token slots.
+ * Replaces DynamicInferenceContext.append_key_value_cache
+ * (megatron/core/inference/contexts/dynamic_context.py:511-545):
+ *   k_cache[token_to_chunk_idx[t], token_to_local_pos[t]] = key[t]   (same for value)
+ * key/value: `[T, Hkv*d]` rows of `row_elems` contiguous elements, `src_stride_tok`
+ * apart.  Pure copy: the cache receives the source bits.  Tokens that share a slot
+ * (batch padding routed to the dummy chunk) race; any one of them wins.
+ */
+int mi_kv_append(const void* key, const void* value, int64_t src_stride_tok, void* k_cache,
+                 void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok,
+                 const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos, int32_t T,
+                 int32_t row_elems, int32_t elem_bytes, void* stream);
+
+/*
+ * KV-append for a decode step with the slot computed on the GPU: request r's new
+ * token goes to position kv_lens[r]-1 (kv_lens already counts it), i.e. chunk
+ * block_table[r][(kv_lens[r]-1) / chunk_tokens], local (kv_lens[r]-1) % chunk_tokens.
+ * Same result as mi_kv_append fed with the rows that
+ * DynamicInferenceContext.update_requests writes (dynamic_context.py:1283-1296),
+ * without materialising them.  Rows with kv_lens[r] <= 0 write nothing.
+ */
+int mi_kv_append_decode(const void* key, const void* value, int64_t src_stride_tok, void* k_cache,
+                        void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok,
+                        const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
+                        int32_t R, int32_t chunk_tokens, int32_t row_elems, int32_t elem_bytes,
+                        void* stream);
+
+/*
+ * fp8 KV storage (no counterpart in the reference, whose cache dtype is always
+ * params_dtype, dynamic_context.py:195,287-308).  OCP e4m3fn bytes, one fp32 scale
+ * per (chunk, KV head), value = byte * scale.
+ * mi_kv_quantize_chunks_fp8: whole chunks, scale = amax(chunk-head tile) / 448.
+ * mi_kv_append_decode_fp8  : one new token per request; a token that opens a chunk
+ *   sets scale = headroom * amax(token) / 448, later tokens reuse it (saturating).
+ */
+int mi_kv_quantize_chunks_fp8(const void* src_bf16, int64_t src_stride_chunk,
+                              int64_t src_stride_tok, void* dst_fp8, int64_t dst_stride_chunk,
+                              int64_t dst_stride_tok, float* scales, int32_t n_chunks,
+                              int32_t chunk_tokens, int32_t Hkv, int32_t head_dim, void* stream);
+
+int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_bf16, int64_t src_stride_tok,
+                            void* k_cache_fp8, void* v_cache_fp8, int64_t kv_stride_chunk,
+                            int64_t kv_stride_tok, float* k_scales, float* v_scales,
+                            const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
+                            int32_t R, int32_t chunk_tokens, int32_t Hkv, int32_t head_dim,
+                            float headroom, void* stream);
+
+/*
+ * Bytes of fp32 workspace mi_paged_decode_attention needs for these sizes
+ * (`split_tokens` = 0 lets the library choose, as the attention call will).
+ */
+int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
+                                  int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens);
+
+/*
+ * Paged GQA decode attention (one query token per request).
+ * Replaces flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=kv_lens,
+ * causal=True, block_table=...) as called from Attention.flash_decode_and_prefill
+ * (megatron/core/transformer/attention.py:589-600):
+ *   out[r,h] = softmax(q[r,h] . K_r[:len_r, h/G]^T * softmax_scale) . V_r[:len_r, h/G]
+ *   K_r[j] = k_cache[block_table[r, j / chunk_tokens], j % chunk_tokens], G = Hq/Hkv.
+ * q/out: bf16 `[R, Hq, d]` with the given token / head strides.  kv_lens int32 [R]
+ * (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] and sizes
+ * the grid (the reference passes max_sequence_length here, dynamic_context.py:791).
+ * kv_dtype MI_KV_FP8_E4M3 reads byte caches with k_scales/v_scales `[n_chunks, Hkv]`.
+ */
+int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
+                              const void* k_cache, const void* v_cache, int64_t kv_stride_chunk,
+                              int64_t kv_stride_tok, int64_t kv_stride_head,
+                              const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
+                              void* out, int64_t o_stride_tok, int64_t o_stride_head,
+                              void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq,
+                              int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
+                              int32_t max_kv_len, int32_t split_tokens, float softmax_scale,
+                              int32_t kv_dtype, const float* k_scales, const float* v_scales,
+                              void* stream);
+
+/*
+ * Paged varlen causal attention for prefill / mixed prefill+decode batches.
+ * Replaces flash_attn_varlen_func(q, k_cache, v_cache, cu_seqlens_q, cu_seqlens_k,
+ * max_seqlen_q, max_seqlen_k, softmax_scale, causal=True, block_table=...)
+ * (megatron/core/transformer/attention.py:546-557): request r owns query rows
+ * cu_seqlens_q[r]..cu_seqlens_q[r+1]-1 and kv_lens[r] keys; query i of Lq sees keys
+ * j <= i + (Lk - Lq) (bottom-right aligned causal mask).
+ */
+int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
+                                   int32_t max_kv_len, int32_t split_tokens);
+
+int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
+                               const void* k_cache, const void* v_cache, int64_t kv_stride_chunk,
+                               int64_t kv_stride_tok, int64_t kv_stride_head,
+                               const int32_t* block_table, int64_t bt_stride,
+                               const int32_t* cu_seqlens_q, const int32_t* kv_lens, void* out,
+                               int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
+                               int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq,
+                               int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
+                               int32_t max_kv_len, int32_t split_tokens, float softmax_scale,
+                               void* stream);
+
+/*
+ * Fused q/k head norm + rotary embedding (+ KV-append when k_cache is given).
+ * Replaces, per layer, q_layernorm/k_layernorm
+ * (megatron/core/transformer/attention.py:1026-1030), apply_rotary_emb_key /
+ * apply_rotary_emb_query (dynamic_context.py:566-631 ->
+ * megatron/core/models/common/embeddings/rope_utils.py:92-126) and, optionally,
+ * append_key_value_cache (dynamic_context.py:511-545).
+ *  q `[T,Hq,d]` bf16 is updated in place; k `[T,Hkv,d]` is read, the result goes to
+ *  k_out (if non-null) and to the cache slot (if k_cache non-null, together with v).
+ *  norm_kind: MI_NORM_NONE | MI_NORM_RMS (weights bf16 [d], may be null) | MI_NORM_L2.
+ *  rotary_angles: fp32 `[max_pos, rot_dim]` table of angles as built by
+ *  RotaryEmbedding.forward (rotary_pos_embedding.py:151-181), null = no rotary;
+ *  q_positions / k_positions int64 [T] index it.  rot_dim < head_dim leaves the tail
+ *  unrotated.  Cache slots: token_to_chunk_idx/token_to_local_pos (int64 [T]) if
+ *  given, else block_table + kv_lens as in mi_kv_append_decode (then T == R).
+ *  faithful_rounding != 0 rounds to bf16 wherever the unfused bf16 op chain does.
+ */
+int mi_norm_rope_append(void* q, int64_t q_stride_tok, const void* k, int64_t k_stride_tok,
+                        void* k_out, int64_t k_out_stride_tok, const void* v, int64_t v_stride_tok,
+                        const void* q_weight, const void* k_weight, float eps, int32_t norm_kind,
+                        const float* rotary_angles, int64_t angles_stride, int32_t rot_dim,
+                        int32_t rotary_interleaved, float mscale, const int64_t* q_positions,
+                        const int64_t* k_positions, void* k_cache, void* v_cache,
+                        int64_t kv_stride_chunk, int64_t kv_stride_tok,
+                        const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos,
+                        const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
+                        int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv, int32_t head_dim,
+                        int32_t faithful_rounding, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MI355_DECODE_H */

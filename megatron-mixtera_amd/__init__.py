@@ -1,0 +1,49 @@
+"""MI355X-native decode-step hot path of Megatron-Core's dynamic inference engine.
+
+Public surface (same names as the reference wherever one exists):
+
+* :class:`DynamicInferenceContext`, :class:`ChunkAllocator` and the overflow errors --
+  the chunked KV cache and in-flight batching state
+  (reference: megatron/core/inference/contexts/).
+* :func:`flash_attn_with_kvcache`, :func:`flash_attn_varlen_func` -- the two attention
+  calls ``Attention.flash_decode_and_prefill`` makes
+  (reference: megatron/core/transformer/attention.py:470-601).
+* :mod:`ops` -- thin torch wrappers over the C ABI (KV-append, paged attention,
+  fused norm + RoPE, fp8 KV).
+"""
+from . import ops, synthetic  # noqa: F401
+from .attention import (  # noqa: F401
+    PagedSelfAttentionCore,
+    adjust_key_value_for_inference,
+    flash_decode_and_prefill,
+)
+from .contexts import (  # noqa: F401
+    ActiveRequestCountOverflowError,
+    ChunkAllocator,
+    ChunkOverflowError,
+    ContextOverflowError,
+    DynamicInferenceContext,
+    MaxSequenceLengthOverflowError,
+    RequestOverflowError,
+    TokenOverflowError,
+    WarmupEngineMode,
+)
+from .flash_attn_interface import flash_attn_varlen_func, flash_attn_with_kvcache  # noqa: F401
+
+__all__ = [
+    "ops",
+    "DynamicInferenceContext",
+    "ChunkAllocator",
+    "WarmupEngineMode",
+    "ContextOverflowError",
+    "RequestOverflowError",
+    "TokenOverflowError",
+    "MaxSequenceLengthOverflowError",
+    "ChunkOverflowError",
+    "ActiveRequestCountOverflowError",
+    "flash_attn_with_kvcache",
+    "flash_attn_varlen_func",
+    "flash_decode_and_prefill",
+    "adjust_key_value_for_inference",
+    "PagedSelfAttentionCore",
+]

@@ -1,0 +1,110 @@
+"""Attention-side glue of the dynamic inference path, as free functions and a small module.
+
+Mirrors the pieces of ``Attention`` that run between the QKV projection and the output
+projection when ``inference_context`` is a dynamic context
+(megatron/core/transformer/attention.py:394-414 ``_adjust_key_value_for_inference`` dynamic
+branch, :470-601 ``flash_decode_and_prefill``, :740-790 rotary on the query), so a
+``SelfAttention`` subclass injected through a ModuleSpec only has to forward to them.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from .flash_attn_interface import flash_attn_varlen_func, flash_attn_with_kvcache
+
+
+def adjust_key_value_for_inference(inference_context, layer_number: int, query: Tensor, key: Tensor, value: Tensor,
+                                   rotary_pos_emb, config, cp_group=None):
+    """RoPE(K) -> append(K, V) -> fetch cache views, in the reference's order.
+
+    Returns ``(query, k_cache, v_cache, rotary_pos_emb, block_table)`` where the returned
+    ``rotary_pos_emb`` is ``(q_pos_emb, None)``: the key half has been applied.
+    """
+    if rotary_pos_emb is not None:
+        q_pos_emb, k_pos_emb = rotary_pos_emb
+        key = inference_context.apply_rotary_emb_key(key, k_pos_emb, config, cp_group)
+        rotary_pos_emb = (q_pos_emb, None)
+    inference_context.append_key_value_cache(layer_number, key, value)
+    k_cache, v_cache, block_table = inference_context.key_value_cache(layer_number)
+    return query, k_cache, v_cache, rotary_pos_emb, block_table
+
+
+def flash_decode_and_prefill(q: Tensor, k: Tensor, v: Tensor, max_seqlen_q, max_seqlen_k, cu_seqlens_q,
+                             cu_seqlens_k, seqlens_k, block_table, softmax_scale: Optional[float] = None) -> Tensor:
+    """Same contract as ``Attention.flash_decode_and_prefill`` (attention.py:470-601).
+
+    ``q`` is ``[T, 1, Hq, d]``; ``k`` / ``v`` are the paged caches.  ``max_seqlen_q == 1``
+    selects the decode kernel, anything else the varlen causal kernel.
+    """
+    if max_seqlen_q > 1:
+        out = flash_attn_varlen_func(q.squeeze(1), k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                     softmax_scale=softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5,
+                                     causal=True, block_table=block_table, seqused_k=seqlens_k)
+        return out.unsqueeze(1)
+    return flash_attn_with_kvcache(q=q, k_cache=k, v_cache=v, cache_seqlens=seqlens_k, causal=True,
+                                   block_table=block_table, softmax_scale=softmax_scale, max_seqlen_k=max_seqlen_k)
+
+
+class PagedSelfAttentionCore(torch.nn.Module):
+    """Everything between ``get_query_key_value_tensors`` and ``linear_proj`` for one layer.
+
+    ``forward(query, key, value, inference_context, rotary_pos_emb)`` takes the split,
+    per-head tensors ``[T, 1, H, d]`` and returns ``[T, 1, Hq*d]`` like
+    ``Attention.forward`` does before the output projection (attention.py:815-829).
+    With ``fused=True`` the q/k norm, both RoPE applications and the KV-append run as one
+    launch; otherwise the reference's call sequence on the context is kept.
+    """
+
+    def __init__(self, layer_number: int, head_dim: int, *, qk_norm: Optional[str] = None, eps: float = 1e-5,
+                 softmax_scale: Optional[float] = None, rotary_interleaved: bool = False, fused: bool = True,
+                 dtype: torch.dtype = torch.bfloat16, device=None):
+        super().__init__()
+        self.layer_number = layer_number
+        self.head_dim = head_dim
+        self.qk_norm = qk_norm
+        self.eps = eps
+        self.softmax_scale = softmax_scale
+        self.fused = fused
+        self.config = type("RopeConfig", (), {"rotary_interleaved": rotary_interleaved,
+                                                "multi_latent_attention": False})()
+        if qk_norm == "rms":
+            self.q_layernorm_weight = torch.nn.Parameter(torch.ones(head_dim, dtype=dtype, device=device))
+            self.k_layernorm_weight = torch.nn.Parameter(torch.ones(head_dim, dtype=dtype, device=device))
+        else:
+            self.q_layernorm_weight = self.k_layernorm_weight = None
+
+    def forward(self, query: Tensor, key: Tensor, value: Tensor, inference_context,
+                rotary_pos_emb: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
+        ctx = inference_context
+        q_emb = k_emb = None
+        if rotary_pos_emb is not None:
+            q_emb, k_emb = rotary_pos_emb if isinstance(rotary_pos_emb, tuple) else (rotary_pos_emb,) * 2
+        if self.fused:
+            assert q_emb is k_emb or q_emb is None or k_emb is None or q_emb.data_ptr() == k_emb.data_ptr(), \
+                "the fused path takes one rotary table for query and key"
+            ctx.fused_qk_norm_rope_append(
+                self.layer_number, query, key, value, rotary_pos_emb=q_emb if q_emb is not None else k_emb,
+                config=self.config, q_weight=None if self.q_layernorm_weight is None else self.q_layernorm_weight.data,
+                k_weight=None if self.k_layernorm_weight is None else self.k_layernorm_weight.data,
+                norm=self.qk_norm, eps=self.eps)
+        else:
+            from . import ops
+            if self.qk_norm is not None:
+                n = ctx.padded_active_token_count
+                ops.norm_rope_append(query[:n], key[:n], key_out=key[:n], norm=self.qk_norm, eps=self.eps,
+                                     q_weight=None if self.q_layernorm_weight is None else self.q_layernorm_weight.data,
+                                     k_weight=None if self.k_layernorm_weight is None else self.k_layernorm_weight.data)
+            if k_emb is not None:
+                key = ctx.apply_rotary_emb_key(key, k_emb, self.config, None)
+            ctx.append_key_value_cache(self.layer_number, key, value)
+            if q_emb is not None:
+                query = ctx.apply_rotary_emb_query(query, q_emb, self.config, None, None)
+        k_cache, v_cache, block_table = ctx.key_value_cache(self.layer_number)
+        cu_q, max_q = ctx.cu_query_lengths()
+        cu_k, kv_lens, max_k = ctx.cu_kv_lengths()
+        out = flash_decode_and_prefill(query, k_cache, v_cache, max_q, max_k, cu_q, cu_k, kv_lens, block_table,
+                                       softmax_scale=self.softmax_scale)
+        return out.reshape(out.size(0), out.size(1), -1)

@@ -1,0 +1,59 @@
+"""Build recipe for the C-ABI library: every ``csrc/*.hip`` file -> one shared object.
+
+``hipcc`` cross-compiles for gfx950 without a GPU, so this runs anywhere the ROCm
+toolchain is installed.  The result, ``libmi355_decode.so``, sits next to this file and
+is what :mod:`_lib` loads.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC = PKG_DIR / "csrc"
+LIB_NAME = "libmi355_decode.so"
+LIB_PATH = PKG_DIR / LIB_NAME
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # packed fp32 VALU forms are kept out of the generated code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc_path() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and Path(cand).exists():
+            return cand
+    raise RuntimeError("hipcc not found: the HIP kernels cannot be built")
+
+
+def sources() -> list[Path]:
+    return sorted(CSRC.glob("*.hip"))
+
+
+def build_library(verbose: bool = False) -> Path:
+    """Compile all kernels into ``libmi355_decode.so`` (always recompiles)."""
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(CSRC), *map(str, sources()), "-o", str(LIB_PATH)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    noise = ("packed-fp32-ops", "'-packed-fp32-ops' is not a recognized feature")
+    out = "\n".join(l for l in proc.stdout.splitlines() if not any(n in l for n in noise))
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
+    if verbose and out.strip():
+        print(out)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose="-v" in sys.argv))

@@ -1,0 +1,704 @@
+"""In-flight batching state and chunked KV cache for dynamic inference on MI355X.
+
+Drop-in for the reference's ``DynamicInferenceContext``
+(megatron/core/inference/contexts/dynamic_context.py:94-1365): same constructor keywords,
+attribute names, method signatures, tensor dtypes and exceptions, so the controller
+(text_generation_controller.py:411-555), the engine (dynamic_engine.py) and
+``Attention.forward`` can use it unchanged.  What differs is underneath the per-layer
+methods: ``append_key_value_cache`` and ``apply_rotary_emb_*`` enqueue the HIP kernels of
+``libmi355_decode.so`` instead of chains of torch indexing kernels, and
+:meth:`fused_qk_norm_rope_append` offers the whole norm -> RoPE -> append sequence of a
+layer as one launch.
+
+Request rows are laid out ``[paused | active | finished]``; ``paused_request_count`` and
+``total_request_count`` mark the boundaries.  Per-request rows are int32, per-token rows
+int64, exactly as in the reference, so states can be compared bit for bit.
+"""
+from __future__ import annotations
+
+import math
+import warnings
+from enum import Enum
+from typing import List, Optional, Tuple, Union
+
+import torch
+import torch.nn.functional as F
+from torch import Tensor
+
+from .. import ops
+from .dynamic_chunk_allocator import ChunkAllocator
+
+
+class ContextOverflowError(Exception):
+    """A request does not fit into the context (reference: dynamic_context.py:30-45).
+
+    ``is_transient`` tells the engine whether retrying later can succeed.
+    """
+
+    def __init__(self, request_id: Optional[int], message: Optional[str] = None, *, is_transient: bool = True):
+        rid = "--" if request_id is None else str(request_id)
+        tail = "" if message is None else f" | {message}"
+        super().__init__(f"request {rid}{tail}")
+        self.is_transient = is_transient
+
+
+class RequestOverflowError(ContextOverflowError):
+    """No free request row."""
+
+
+class TokenOverflowError(ContextOverflowError):
+    """No room left in the per-token rows."""
+
+
+class MaxSequenceLengthOverflowError(ContextOverflowError):
+    """Prompt + generation budget exceeds ``max_sequence_length`` (never transient)."""
+
+    def __init__(self, request_id, message: Optional[str] = None):
+        super().__init__(request_id, message=message, is_transient=False)
+
+
+class ChunkOverflowError(ContextOverflowError):
+    """Not enough free KV chunks."""
+
+
+class ActiveRequestCountOverflowError(ContextOverflowError):
+    """``initialize_attention_state`` was asked to warm up more tokens than ``max_requests``."""
+
+    def __init__(self, max_request_count, active_request_count):
+        assert active_request_count > max_request_count
+        super().__init__(
+            None,
+            "active_request_count (%d) > max_request_count (%d)." % (active_request_count, max_request_count),
+        )
+
+
+class WarmupEngineMode(Enum):
+    """Which attention path a graph warm-up step should exercise."""
+
+    DECODE = "decode"
+    NON_DECODE = "non_decode"
+
+
+def _ceil_to(value: int, multiple: int) -> int:
+    return multiple * int(math.ceil(int(value) / multiple))
+
+
+class DynamicInferenceContext:
+    """Chunked KV cache + batching bookkeeping; see the module docstring.
+
+    Keyword arguments are those of the reference constructor (dynamic_context.py:156-177);
+    ``device`` is an addition for host-side testing of the bookkeeping (the kernels need a
+    GPU).  ``num_attention_heads`` is the number of KV heads (query groups).
+    """
+
+    TOKEN_ROUNDER = 64
+    REQUEST_ROUNDER = 4
+
+    # ------------------------------------------------------------------ construction
+    def __init__(
+        self,
+        *,
+        params_dtype: torch.dtype,
+        num_layers: int,
+        kv_channels: int,
+        num_attention_heads: int,
+        max_sequence_length: int,
+        buffer_size_gb: float,
+        buffer_guaranteed_fraction: float,
+        chunk_size_tokens: int = 256,
+        buffer_overflow_factor: Optional[float] = None,
+        max_requests_override: Optional[int] = None,
+        max_tokens_override: Optional[int] = None,
+        tensor_model_parallel_size: Optional[int] = None,
+        cache_mla_latent: bool = False,
+        kv_lora_rank: Optional[int] = None,
+        qk_pos_emb_head_dim: Optional[int] = None,
+        num_cuda_graphs: Optional[int] = None,
+        materialize_only_last_token_logits: bool = True,
+        use_cuda_graphs_for_non_decode_steps: bool = True,
+        device: Optional[Union[torch.device, str, int]] = None,
+    ):
+        if cache_mla_latent:
+            raise NotImplementedError(
+                "the MLA latent cache (cache_mla_latent=True) is not part of the MI355X decode path")
+        self.materialize_only_last_token_logits = materialize_only_last_token_logits
+        self.cache_mla_latent = False
+        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+
+        tp = 1 if tensor_model_parallel_size is None else tensor_model_parallel_size
+        if num_attention_heads % tp:
+            raise ValueError(f"{num_attention_heads} KV heads are not divisible by tensor parallel size {tp}")
+        heads_here = num_attention_heads // tp
+
+        # ---- sizing (reference: dynamic_context.py:186-242) ----
+        self.chunk_size_tokens = chunk_size_tokens
+        self.chunk_size_bytes = params_dtype.itemsize * 2 * num_layers * chunk_size_tokens * heads_here * kv_channels
+        pool_bytes = int(buffer_size_gb * 1024**3)
+        pool_bytes -= pool_bytes % self.chunk_size_bytes
+        chunk_count_total = pool_bytes // self.chunk_size_bytes
+
+        token_capacity = pool_bytes / self.chunk_size_bytes * chunk_size_tokens
+        self.max_requests = self.round_up_requests(int(token_capacity / max_sequence_length), tp_size=tp)
+        self.max_tokens = self.round_up_tokens(int(token_capacity), tp_size=tp)
+        if buffer_overflow_factor is not None:
+            self.max_requests = self.round_up_requests(int(self.max_requests * buffer_overflow_factor), tp_size=tp)
+            self.max_tokens = self.round_up_tokens(int(self.max_tokens * buffer_overflow_factor / 50.0), tp_size=tp)
+        if max_requests_override is not None:
+            self.max_requests = self.round_up_requests(max_requests_override, tp_size=tp)
+        if max_tokens_override is not None:
+            self.max_tokens = self.round_up_tokens(max_tokens_override, tp_size=tp)
+        self.max_requests = min(self.max_requests, self.max_tokens)
+
+        self.params_dtype = params_dtype
+        self.num_layers = num_layers
+        self.max_sequence_length = max_sequence_length
+        self.num_kv_heads_per_partition = heads_here
+        self.kv_channels = kv_channels
+
+        self.total_request_count = 0
+        self.active_token_count = 0
+        self.paused_request_count = 0
+        self.padded_active_token_count = None
+        self.padded_active_request_count = None
+        self.paused_tokens = None
+
+        dev = self.device
+
+        def req_row(fill=None):
+            if fill is None:
+                return torch.empty(self.max_requests, dtype=torch.int32, device=dev)
+            return torch.full((self.max_requests,), fill, dtype=torch.int32, device=dev)
+
+        def tok_row(fill=None):
+            if fill is None:
+                return torch.empty(self.max_tokens, dtype=torch.long, device=dev)
+            return torch.full((self.max_tokens,), fill, dtype=torch.long, device=dev)
+
+        # ---- per-request rows (int32) ----
+        self.request_ids = req_row(-1)
+        self.request_query_lengths = req_row()
+        self.request_output_lengths = req_row()
+        self.request_kv_length_offsets = req_row()
+        self.request_kv_chunk_counts = req_row()
+        self.request_last_kv_chunk_id = req_row()
+        self.request_last_kv_chunk_offset = req_row()
+
+        # ---- per-token rows (int64) ----
+        self.token_to_input_ids = tok_row(0)
+        self.token_to_pos_ids = tok_row(0)
+        self.token_to_request_idx = tok_row()
+        self.token_to_chunk_idx = tok_row()
+        self.token_to_position_in_request = tok_row()
+        self.token_to_local_position_within_kv_chunk = tok_row()
+
+        # ---- the cache: [key|value, layer, chunk, token, head, channel] ----
+        self.memory_buffer = torch.full(
+            (2, num_layers, chunk_count_total, chunk_size_tokens, heads_here, kv_channels),
+            -1, dtype=params_dtype, device=dev)
+
+        self.max_kv_chunk_count = math.ceil(max_sequence_length / chunk_size_tokens)
+        self.request_to_kv_chunk_ids = torch.full(
+            (self.max_requests, self.max_kv_chunk_count), -1, dtype=torch.int, device=dev)
+
+        # ---- graph batch sizes (reference: dynamic_context.py:319-356) ----
+        self.cuda_graph_token_counts = None
+        if num_cuda_graphs is not None:
+            num_cuda_graphs = min(max(num_cuda_graphs, 1), self.max_requests)
+            step = math.ceil((self.max_requests / num_cuda_graphs) / 8) * 8
+            step = math.ceil(step / tp) * tp
+            self.cuda_graph_step_size = step
+            if num_cuda_graphs == 1:
+                counts = [self.max_requests]
+            else:
+                counts = list(range(step, self.max_requests, step))
+                if counts[-1] != self.max_requests:
+                    counts.append(self.max_requests)
+                counts.reverse()
+            self.cuda_graph_token_counts = counts
+            self.cuda_graph_token_counts_set = set(counts)
+            self.max_cuda_graph_token_count = max(counts)
+        self.cuda_graph_request_counts = self.cuda_graph_token_counts
+        self.non_decode_cuda_graphs = use_cuda_graphs_for_non_decode_steps and (num_cuda_graphs is not None)
+
+        # ---- fixed-address mirrors consumed by captured graphs ----
+        self.query_seq_lengths_cudagraph_only = torch.zeros(self.max_requests, dtype=torch.int32, device=dev)
+        self.cu_query_seq_lengths_cudagraph_only = torch.zeros(self.max_requests + 1, dtype=torch.int32, device=dev)
+        self.kv_seq_lengths_cudagraph_only = torch.zeros(self.max_requests, dtype=torch.int32, device=dev)
+        self.cu_kv_seq_lengths_cudagraph_only = torch.zeros(self.max_requests + 1, dtype=torch.int32, device=dev)
+        self.request_to_kv_chunk_ids_cudagraph_only = torch.zeros(
+            (self.max_requests, self.max_kv_chunk_count), dtype=torch.int, device=dev)
+
+        # ---- guaranteed-progress reserve (reference: dynamic_context.py:398-401) ----
+        reserve = min(int(buffer_guaranteed_fraction * chunk_count_total), chunk_count_total)
+        self.gtd_request_count = max(1, reserve // self.max_kv_chunk_count)
+        self.gtd_chunk_count = self.gtd_request_count * self.max_kv_chunk_count
+
+        self.chunk_allocator = ChunkAllocator(
+            chunk_count_total=chunk_count_total, gtd_chunk_count=self.gtd_chunk_count, device=dev)
+        self.dummy_chunk_idx = self.chunk_allocator.dummy_chunk_idx
+
+        self.reset_attention_state()
+
+    # ------------------------------------------------------------------ rounding helpers
+    @classmethod
+    def round_up_tokens(cls, value, tp_size=None):
+        """Next multiple of ``TOKEN_ROUNDER`` (itself rounded up to a multiple of the TP size)."""
+        tp = 1 if tp_size is None else tp_size
+        return _ceil_to(value, math.ceil(cls.TOKEN_ROUNDER / tp) * tp)
+
+    @classmethod
+    def round_up_requests(cls, value, tp_size=None):
+        """Next multiple of ``REQUEST_ROUNDER`` (itself rounded up to a multiple of the TP size)."""
+        tp = 1 if tp_size is None else tp_size
+        return _ceil_to(value, math.ceil(cls.REQUEST_ROUNDER / tp) * tp)
+
+    @classmethod
+    def round_up(cls, value):
+        """Deprecated single-rounder form kept for callers that still use it."""
+        warnings.warn("`round_up` is deprecated in favor of `round_up_tokens` or `round_up_requests`.")
+        return _ceil_to(value, getattr(cls, "ROUNDER", 64))
+
+    # ------------------------------------------------------------------ simple queries
+    def is_static_batching(self) -> bool:
+        return False
+
+    def is_dynamic_batching(self) -> bool:
+        return True
+
+    def increment_sequence_len_offset(self, increment: int) -> None:
+        """No-op for dynamic batching (static-context API)."""
+
+    def increment_batch_size_offset(self, increment: int) -> None:
+        """No-op for dynamic batching (static-context API)."""
+
+    def reset_batch_size_offset(self) -> None:
+        """No-op for dynamic batching (static-context API)."""
+
+    def _active(self) -> slice:
+        return slice(self.paused_request_count, self.total_request_count)
+
+    def is_decode_only(self) -> bool:
+        """Every active request contributes exactly one token this step."""
+        return self.total_request_count - self.paused_request_count == self.active_token_count
+
+    def has_unfinished_requests(self) -> bool:
+        return self.total_request_count > 0
+
+    def cu_query_lengths(self) -> Tuple[Optional[Tensor], int]:
+        return self.cu_query_seq_lengths, self.max_seqlen_q
+
+    def cu_kv_lengths(self) -> Tuple[Optional[Tensor], Tensor, int]:
+        return (self.cu_kv_seq_lengths, self.kv_seq_lengths, self.max_seqlen_k)
+
+    def get_active_sequence_lengths(self) -> Tensor:
+        return (self.request_kv_length_offsets + self.request_query_lengths)[self._active()]
+
+    def get_max_sequence_lengths(self) -> Tensor:
+        return self.request_output_lengths[self._active()]
+
+    def get_active_request_count(self):
+        unfinished = torch.less(self.get_active_sequence_lengths(), self.get_max_sequence_lengths())
+        return int(unfinished.sum().item())
+
+    # ------------------------------------------------------------------ per-layer hot path
+    def append_key_value_cache(self, layer_number: int, key: Tensor, value: Tensor) -> None:
+        """Scatter this step's K/V rows into the layer's chunks (bit-exact copy).
+
+        ``layer_number`` is 1-based.  Slots come from ``token_to_chunk_idx`` /
+        ``token_to_local_position_within_kv_chunk``; padded tokens land in the dummy chunk.
+        """
+        assert key.size(1) == 1 and value.size(1) == 1
+        n = self.padded_active_token_count
+        ops.kv_append(
+            key[:n], value[:n],
+            self.memory_buffer[0, layer_number - 1], self.memory_buffer[1, layer_number - 1],
+            self.token_to_chunk_idx, self.token_to_local_position_within_kv_chunk)
+
+    def key_value_cache(self, layer_number: int) -> Tuple[Tensor, Tensor, Tensor]:
+        """Views of the layer's key cache, value cache and this step's block table."""
+        return (self.memory_buffer[0, layer_number - 1], self.memory_buffer[1, layer_number - 1], self.block_table)
+
+    @staticmethod
+    def _rope_flags(config) -> bool:
+        if getattr(config, "multi_latent_attention", False):
+            raise NotImplementedError("multi-latent attention RoPE is not part of the MI355X decode path")
+        return bool(getattr(config, "rotary_interleaved", False))
+
+    def apply_rotary_emb_query(self, query: Tensor, query_emb: Tensor, config, cu_seqlens_q: Tensor,
+                               cp_group=None, mscale: float = 1.0) -> Tensor:
+        """Rotate the first ``padded_active_token_count`` query rows in place; positions = ``token_to_pos_ids``."""
+        n = self.padded_active_token_count
+        ops.norm_rope_append(query[:n], None, rotary_emb=query_emb, q_positions=self.token_to_pos_ids,
+                             rotary_interleaved=self._rope_flags(config), mscale=mscale)
+        return query
+
+    def apply_rotary_emb_key(self, key: Tensor, key_emb: Tensor, config, cp_group=None, mscale: float = 1.0) -> Tensor:
+        """Rotate key rows; positions = ``token_to_position_in_request``.
+
+        Decode-only steps return a fresh tensor, other steps update ``key[:n]`` in place
+        (the reference's behaviour, dynamic_context.py:619-631).
+        """
+        n = self.padded_active_token_count
+        interleaved = self._rope_flags(config)
+        if self.is_decode_only():
+            assert key.shape[0] == n
+            out = torch.empty_like(key)
+        else:
+            out = key
+        ops.norm_rope_append(None, key[:n], key_out=out[:n], rotary_emb=key_emb,
+                             k_positions=self.token_to_position_in_request,
+                             rotary_interleaved=interleaved, mscale=mscale)
+        return out
+
+    def fused_qk_norm_rope_append(self, layer_number: int, query: Tensor, key: Tensor, value: Tensor, *,
+                                  rotary_pos_emb: Optional[Tensor], config=None, q_weight: Optional[Tensor] = None,
+                                  k_weight: Optional[Tensor] = None, norm: Optional[str] = None, eps: float = 1e-5,
+                                  mscale: float = 1.0, faithful_rounding: bool = True) -> Tensor:
+        """One launch for q/k norm -> RoPE(q, k) -> append(k, v) of a layer.
+
+        Equivalent to q_layernorm/k_layernorm + ``apply_rotary_emb_key`` +
+        ``append_key_value_cache`` + ``apply_rotary_emb_query`` of the reference
+        (attention.py:1026-1030, 394-404, 766).  ``query`` is updated in place and returned.
+        """
+        n = self.padded_active_token_count
+        ops.norm_rope_append(
+            query[:n], key[:n], value=value[:n], q_weight=q_weight, k_weight=k_weight, eps=eps, norm=norm,
+            rotary_emb=rotary_pos_emb, q_positions=self.token_to_pos_ids,
+            k_positions=self.token_to_position_in_request,
+            rotary_interleaved=self._rope_flags(config) if config is not None else False, mscale=mscale,
+            k_cache=self.memory_buffer[0, layer_number - 1], v_cache=self.memory_buffer[1, layer_number - 1],
+            token_to_chunk_idx=self.token_to_chunk_idx,
+            token_to_local_pos=self.token_to_local_position_within_kv_chunk,
+            faithful_rounding=faithful_rounding)
+        return query
+
+    # ------------------------------------------------------------------ per-step attention state
+    def reset_attention_state(self) -> None:
+        """Forget the per-step attention metadata (the fixed-address mirrors are zeroed)."""
+        self.max_seqlen_q = None
+        self.max_seqlen_k = None
+        self.cu_query_seq_lengths = None
+        self.cu_kv_seq_lengths = None
+        self.kv_seq_lengths = None
+        self.block_table = None
+        self.cu_query_seq_lengths_cudagraph_only.fill_(0)
+        self.query_seq_lengths_cudagraph_only.fill_(0)
+        self.cu_kv_seq_lengths_cudagraph_only.fill_(0)
+        self.kv_seq_lengths_cudagraph_only.fill_(0)
+        self.request_to_kv_chunk_ids_cudagraph_only.fill_(0)
+
+    def using_cuda_graph_this_step(self) -> bool:
+        """Graph sizes exist, the step type may use them, and the batch fits the largest one."""
+        if self.cuda_graph_token_counts is None:
+            return False
+        if not (self.is_decode_only() or self.non_decode_cuda_graphs):
+            return False
+        return self.active_token_count <= self.max_cuda_graph_token_count
+
+    def initialize_attention_state(self, *, num_warmup_tokens: Optional[int] = None,
+                                   warmup_engine_mode: WarmupEngineMode = WarmupEngineMode.DECODE,
+                                   num_warmup_requests: Optional[int] = None) -> None:
+        """Prepare padding, sequence lengths and the block table for this step's forward pass.
+
+        Reference: dynamic_context.py:656-825.  Decode-only and graph steps publish their
+        lengths / block table through the fixed-address ``*_cudagraph_only`` buffers, with
+        padded rows holding kv-length 0 and block-table row 0.
+        """
+        if num_warmup_requests is not None:
+            warnings.warn("'num_warmup_requests' is deprecated; use 'num_warmup_tokens'.", DeprecationWarning)
+            if num_warmup_tokens is None:
+                num_warmup_tokens = num_warmup_requests
+
+        if num_warmup_tokens is not None:
+            if num_warmup_tokens > self.max_requests:
+                raise ActiveRequestCountOverflowError(self.max_requests, num_warmup_tokens)
+            if warmup_engine_mode == WarmupEngineMode.NON_DECODE:
+                assert self.non_decode_cuda_graphs, "Set non-decode cuda graphs to True"
+                # one request, zero tokens: makes is_decode_only() false for the warm-up
+                self.total_request_count = 1
+
+        token_count = self.active_token_count if num_warmup_tokens is None else num_warmup_tokens
+        graph_step = self.using_cuda_graph_this_step()
+        decode_only = self.is_decode_only()
+
+        if graph_step:
+            padded = _ceil_to(token_count, self.cuda_graph_step_size)
+            padded = min(padded, self.max_requests)
+            assert padded in self.cuda_graph_token_counts_set
+            assert padded >= token_count
+        else:
+            padded = self.round_up_tokens(self.active_token_count)
+            if decode_only:
+                padded = min(padded, self.max_requests)
+        self.padded_active_token_count = padded
+        n_active_req = self.total_request_count - self.paused_request_count
+        self.padded_active_request_count = padded if (graph_step or decode_only) else n_active_req
+
+        # padded token rows: write into the dummy chunk at position 0
+        pad = slice(self.active_token_count, padded)
+        self.token_to_chunk_idx[pad] = self.dummy_chunk_idx
+        self.token_to_local_position_within_kv_chunk[pad] = 0
+        self.token_to_position_in_request[pad] = 0
+
+        act = self._active()
+        q_lens = self.request_query_lengths[act]
+        kv_lens = (self.request_kv_length_offsets + self.request_query_lengths)[act]
+        R = self.padded_active_request_count
+        dev = self.device
+
+        if decode_only or graph_step:
+            self.query_seq_lengths_cudagraph_only[:n_active_req] = q_lens
+            self.kv_seq_lengths_cudagraph_only[:n_active_req] = kv_lens
+            self.kv_seq_lengths = self.kv_seq_lengths_cudagraph_only[:R]
+            self.max_seqlen_k = self.max_sequence_length
+            self.request_to_kv_chunk_ids_cudagraph_only[:n_active_req] = self.request_to_kv_chunk_ids[act]
+            self.block_table = self.request_to_kv_chunk_ids_cudagraph_only[:R]
+            if decode_only:
+                self.cu_query_seq_lengths = None
+                self.cu_kv_seq_lengths = None
+                self.max_seqlen_q = 1
+            else:
+                self.cu_query_seq_lengths_cudagraph_only[1 : R + 1] = torch.cumsum(
+                    self.query_seq_lengths_cudagraph_only[:R], dim=0)
+                self.cu_query_seq_lengths = self.cu_query_seq_lengths_cudagraph_only[: R + 1]
+                self.max_seqlen_q = padded
+                cu_kv = torch.cumsum(self.kv_seq_lengths, dim=0)
+                self.cu_kv_seq_lengths_cudagraph_only[1 : cu_kv.size(0) + 1] = cu_kv
+                self.cu_kv_seq_lengths = self.cu_kv_seq_lengths_cudagraph_only[: R + 1]
+        else:
+            self.cu_query_seq_lengths = torch.zeros(n_active_req + 1, dtype=torch.int32, device=dev)
+            self.cu_query_seq_lengths[1:] = torch.cumsum(q_lens, dim=0)
+            self.max_seqlen_q = q_lens.max().item()
+            self.kv_seq_lengths = kv_lens
+            self.cu_kv_seq_lengths = torch.zeros(n_active_req + 1, dtype=torch.int32, device=dev)
+            self.cu_kv_seq_lengths[1:] = torch.cumsum(kv_lens, dim=0)
+            self.max_seqlen_k = kv_lens.max().item()
+            self.block_table = self.request_to_kv_chunk_ids[act]
+
+    def reset(self) -> None:
+        """Return to the empty state without reallocating anything (graphs keep the addresses)."""
+        self.total_request_count = 0
+        self.active_token_count = 0
+        self.paused_request_count = 0
+        self.padded_active_token_count = 0
+        self.padded_active_request_count = 0
+        self.paused_tokens = None
+
+        self.request_ids.fill_(-1)
+        self.request_query_lengths.fill_(0)
+        self.request_output_lengths.fill_(0)
+        self.request_kv_length_offsets.fill_(0)
+        self.request_kv_chunk_counts.fill_(0)
+        self.request_last_kv_chunk_id.fill_(-1)
+        self.request_last_kv_chunk_offset.fill_(0)
+        self.request_to_kv_chunk_ids.fill_(-1)
+
+        self.token_to_input_ids.fill_(0)
+        self.token_to_pos_ids.fill_(0)
+        self.token_to_request_idx.fill_(-1)
+        self.token_to_position_in_request.fill_(0)
+        self.token_to_chunk_idx.fill_(-1)
+        self.token_to_local_position_within_kv_chunk.fill_(0)
+
+        self.reset_attention_state()
+        self.chunk_allocator.reset()
+
+    def current_input_and_position_ids(self, *, num_warmup_tokens: Optional[int] = None) -> Tuple[Tensor, Tensor]:
+        """``[1, T]`` views of this step's input ids and position ids."""
+        n = num_warmup_tokens or self.padded_active_token_count
+        return (self.token_to_input_ids[:n].unsqueeze(0), self.token_to_pos_ids[:n].unsqueeze(0))
+
+    def last_token_logits(self, logits: Tensor) -> Tensor:
+        """Rows of ``logits[0]`` at each active request's last token."""
+        assert logits.size(0) == 1
+        assert logits.size(1) == self.padded_active_token_count, (
+            f"logits.size(1) ({tuple(logits.shape)}) != "
+            f"padded_active_token_count ({self.padded_active_token_count}).")
+        last = torch.cumsum(self.request_query_lengths[self._active()], dim=0) - 1
+        return logits.squeeze(0)[last, :]
+
+    # ------------------------------------------------------------------ request lifecycle
+    def add_request(self, request_id: int, tokens: Tensor, num_tokens_to_generate: Optional[int] = None) -> None:
+        """Admit a prompt: reserve ``ceil(len/chunk)`` chunks and fill its request / token rows.
+
+        Raises the overflow errors of the reference in the reference's order
+        (dynamic_context.py:945-974).
+        """
+        length = tokens.numel()
+        if length > self.max_tokens:
+            raise TokenOverflowError(request_id, is_transient=True)
+        if self.active_token_count + length > self.max_tokens:
+            raise TokenOverflowError(request_id)
+        if self.total_request_count >= self.max_requests:
+            raise RequestOverflowError(request_id)
+
+        n_chunks = math.ceil(length / self.chunk_size_tokens)
+        chunk_ids = self.chunk_allocator.allocate_memory_chunks(n_chunks, safe=True)
+        if chunk_ids is None:
+            raise ChunkOverflowError(request_id)
+
+        if num_tokens_to_generate is None:
+            num_tokens_to_generate = self.max_sequence_length - length
+        elif length + num_tokens_to_generate > self.max_sequence_length:
+            raise MaxSequenceLengthOverflowError(request_id)
+
+        row = self.total_request_count
+        self.request_ids[row] = request_id
+        self.request_query_lengths[row] = length
+        self.request_output_lengths[row] = length + num_tokens_to_generate
+        self.request_kv_length_offsets[row] = 0
+        self.request_to_kv_chunk_ids[row][:n_chunks] = chunk_ids
+        self.request_kv_chunk_counts[row] = n_chunks
+        self.request_last_kv_chunk_id[row] = chunk_ids[-1]
+        self.request_last_kv_chunk_offset[row] = (length - 1) % self.chunk_size_tokens
+
+        span = slice(self.active_token_count, self.active_token_count + length)
+        pos = torch.arange(length, device=self.device)
+        self.token_to_pos_ids[span] = pos
+        self.token_to_input_ids[span] = tokens
+        self.token_to_request_idx[span] = row
+        self.token_to_position_in_request[span] = pos
+        self.token_to_chunk_idx[span] = chunk_ids[pos // self.chunk_size_tokens]
+        self.token_to_local_position_within_kv_chunk[span] = pos % self.chunk_size_tokens
+
+        self.total_request_count += 1
+        self.active_token_count += length
+
+    def _move_book_keeping_tensors(self, src_idxs, dst_idxs, next_tokens):
+        """``row[dst] = row[src]`` for every per-request row (right-hand sides gathered first)."""
+        for row in (self.request_kv_length_offsets, self.request_query_lengths, self.request_output_lengths,
+                    self.request_ids):
+            row[dst_idxs] = row[src_idxs]
+        next_tokens[dst_idxs] = next_tokens[src_idxs]
+        for row in (self.request_to_kv_chunk_ids, self.request_kv_chunk_counts, self.request_last_kv_chunk_id,
+                    self.request_last_kv_chunk_offset):
+            row[dst_idxs] = row[src_idxs]
+
+    def _release_chunks_of(self, rows: Tensor) -> None:
+        owned = self.request_to_kv_chunk_ids[rows]
+        self.chunk_allocator.release_memory_chunks(owned[owned != -1])
+
+    def update_requests(self, active_requests_mask: Tensor, new_tokens: Tensor) -> Optional[Tensor]:
+        """Advance every request by the token just sampled (reference: dynamic_context.py:1033-1298).
+
+        ``active_requests_mask[i]`` is 1 when active request i continues, 0 when it finished;
+        ``new_tokens[i]`` is its sampled token.  Finished requests give their chunks back and
+        move to the right; requests whose last chunk is full pause (move left) until a chunk
+        can be granted; resumed requests (LIFO) receive a fresh chunk; finally the per-token
+        rows are rewritten for a one-token-per-request decode step.  Returns the ids of
+        requests that were newly paused and stay paused, or ``None``.
+        """
+        n_continue = (active_requests_mask == 1).sum().item()
+        n_finished = (active_requests_mask == 0).sum().item()
+        assert n_continue + n_finished + self.paused_request_count == self.total_request_count
+
+        self.reset_attention_state()
+        paused0 = self.paused_request_count
+
+        # nothing left at all: give every chunk back and start over
+        if n_continue + paused0 == 0:
+            if n_finished > 0:
+                done = torch.nonzero(active_requests_mask == 0, as_tuple=True)[0] + paused0
+                self._release_chunks_of(done)
+            self.request_to_kv_chunk_ids.fill_(-1)
+            self.total_request_count = 0
+            self.active_token_count = 0
+            return None
+
+        if paused0 != 0:
+            assert self.paused_tokens is not None
+            next_tokens = torch.cat((self.paused_tokens, new_tokens))
+        else:
+            next_tokens = new_tokens
+
+        # finished requests: release chunks, then fill their holes from the right end
+        if n_finished > 0:
+            done = torch.nonzero(active_requests_mask == 0, as_tuple=True)[0] + paused0
+            self._release_chunks_of(done)
+            self.request_to_kv_chunk_ids[done] = -1
+            if n_continue > 0:
+                holes = torch.nonzero(active_requests_mask[:n_continue] == 0, as_tuple=True)[0] + paused0
+                movers = (torch.nonzero(active_requests_mask[n_continue:], as_tuple=True)[0]
+                          + n_continue + paused0)
+                self._move_book_keeping_tensors(src_idxs=movers, dst_idxs=holes, next_tokens=next_tokens)
+                self.request_to_kv_chunk_ids[movers] = -1
+
+        # requests sitting on a full last chunk pause until they get a new one
+        newly_paused_request_ids = None
+        if n_continue > 0:
+            fill = self.request_last_kv_chunk_offset[paused0 : paused0 + n_continue]
+            needs_chunk = (fill == self.chunk_size_tokens - 1).byte()
+            n_need = (needs_chunk == 1).sum().item()
+            if 0 < n_need != n_continue:
+                stay_left = torch.nonzero(needs_chunk[:n_need] == 0, as_tuple=True)[0] + paused0
+                need_right = torch.nonzero(needs_chunk[n_need:], as_tuple=True)[0] + n_need + paused0
+                dst = torch.cat((stay_left, need_right))
+                src = torch.cat((need_right, stay_left))
+                self._move_book_keeping_tensors(src_idxs=src, dst_idxs=dst, next_tokens=next_tokens)
+                newly_paused_request_ids = self.request_ids[dst]
+            self.paused_request_count += n_need
+            n_continue -= n_need
+
+        # how many paused requests can be given a chunk now
+        spare = max(0, self.chunk_allocator.chunk_count_avail - self.gtd_chunk_count)
+        if spare:
+            n_resume = min(spare, self.paused_request_count)
+        else:
+            n_resume = min(max(self.gtd_request_count - n_continue, 0), self.paused_request_count)
+        self.paused_request_count -= n_resume
+        n_continue += n_resume
+        assert n_continue > 0, "active_request_count == %d." % n_continue
+        if newly_paused_request_ids is not None and n_resume > 0:
+            newly_paused_request_ids = newly_paused_request_ids[:-n_resume]
+
+        # next step: one token per active request
+        self.total_request_count = n_continue + self.paused_request_count
+        self.active_token_count = n_continue
+        act = self._active()
+        self.token_to_input_ids[:n_continue] = next_tokens[act]
+        if self.paused_request_count > 0:
+            self.paused_tokens = next_tokens[: self.paused_request_count]
+
+        self.request_kv_length_offsets[act].add_(self.request_query_lengths[act])
+        self.request_query_lengths[act].fill_(1)
+        self.token_to_pos_ids[:n_continue] = self.request_kv_length_offsets[act]
+        self.request_last_kv_chunk_offset[act] = (self.request_last_kv_chunk_offset[act] + 1) % self.chunk_size_tokens
+
+        if n_resume > 0:
+            first = self.paused_request_count
+            resumed = slice(first, first + n_resume)
+            assert torch.all(self.request_last_kv_chunk_offset[resumed] == 0), (
+                "The request_last_kv_chunk_offset should be 0 for the requests that just got resumed this step. ")
+            chunk_ids = self.chunk_allocator.allocate_memory_chunks(n_resume)
+            rows = torch.arange(first, first + n_resume, device=self.device)
+            cols = self.request_kv_chunk_counts[resumed]
+            self.request_to_kv_chunk_ids[rows, cols] = chunk_ids
+            self.request_kv_chunk_counts[resumed] += 1
+            self.request_last_kv_chunk_id[resumed] = chunk_ids
+
+        self.token_to_request_idx[:n_continue] = torch.arange(
+            self.paused_request_count, self.total_request_count, device=self.device)
+        self.token_to_position_in_request[:n_continue] = self.request_kv_length_offsets[act]
+        self.token_to_chunk_idx[:n_continue] = self.request_last_kv_chunk_id[act]
+        self.token_to_local_position_within_kv_chunk[:n_continue] = self.request_last_kv_chunk_offset[act]
+        return newly_paused_request_ids
+
+    def calculate_log_probs(self, logits: Tensor, new_tokens: Tensor,
+                            only_last_token_logits: Optional[bool] = False) -> List[List[float]]:
+        """Log-probabilities of the tokens actually chosen, grouped per active request.
+
+        Reference: dynamic_context.py:1300-1365.  For prefill rows the chosen token of position
+        p is the prompt token at p+1; the last position of each request takes ``new_tokens``.
+        """
+        log_probs = F.log_softmax(logits.squeeze(0).float(), dim=-1)
+        if only_last_token_logits or self.is_decode_only():
+            idx = torch.arange(len(new_tokens), dtype=torch.int32, device=logits.device)
+            picked = log_probs[idx, new_tokens]
+            return [[lp] for lp in picked.flatten().tolist()]
+
+        chosen = self.token_to_input_ids[: self.active_token_count].roll(-1, 0)
+        q_lens = self.request_query_lengths[self._active()]
+        chosen[q_lens.cumsum(0) - 1] = new_tokens
+        idx = torch.arange(self.active_token_count, device=log_probs.device)
+        picked = log_probs[idx, chosen]
+        return [lp.tolist() for lp in picked.cpu().split(q_lens.tolist(), dim=0)]

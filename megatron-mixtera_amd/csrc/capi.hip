@@ -1,0 +1,95 @@
+// Error reporting, version and tuning entry points of the C-ABI library.
+#include "mi_capi_internal.h"
+
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+static thread_local char g_err[256] = "";
+
+int mi_fail(int code, const char* msg) {
+  snprintf(g_err, sizeof(g_err), "%s", msg);
+  return code;
+}
+
+int mi_check_launch(const char* where) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return MI_OK;
+  snprintf(g_err, sizeof(g_err), "%s: %s", where, hipGetErrorString(e));
+  return MI_ERR_LAUNCH;
+}
+
+static int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return (v && *v) ? atoi(v) : dflt;
+}
+
+MiTuning& mi_tuning() {
+  static MiTuning t = {env_int("MI355_DECODE_SUBTILES", 2), env_int("MI355_PREFILL_SUBTILES", 2)};
+  return t;
+}
+
+extern "C" int mi_version(void) { return 1; }
+
+extern "C" const char* mi_last_error(void) { return g_err; }
+
+extern "C" int mi_set_tuning(const char* name, int32_t value) {
+  if (!name) return mi_fail(MI_ERR_NULL, "mi_set_tuning: null name");
+  if (!strcmp(name, "decode_tile_subtiles")) {
+    if (value != 1 && value != 2 && value != 4) return mi_fail(MI_ERR_UNSUPPORTED, "decode_tile_subtiles must be 1, 2 or 4");
+    mi_tuning().decode_tile_subtiles = value;
+    return MI_OK;
+  }
+  if (!strcmp(name, "prefill_tile_subtiles")) {
+    mi_tuning().prefill_tile_subtiles = value;
+    return MI_OK;
+  }
+  return mi_fail(MI_ERR_UNSUPPORTED, "mi_set_tuning: unknown knob");
+}
+
+// ---- kernel timing with HIP events --------------------------------------------------
+// When enabled, mi_paged_decode_attention brackets its split kernel (the kernel that
+// streams the KV cache) with a start/stop event pair on the caller's stream; the pairs are
+// read back with mi_profile_collect.  Host objects only: nothing is allocated on the
+// device, and profiling must stay off while a stream is being captured into a graph.
+#include <vector>
+
+namespace {
+struct EventPair { hipEvent_t a, b; };
+std::vector<EventPair> g_pool;     // created once, reused
+size_t g_used = 0;
+bool g_profile = false;
+}  // namespace
+
+bool mi_profile_next(hipEvent_t* a, hipEvent_t* b) {
+  if (!g_profile) return false;
+  if (g_used == g_pool.size()) {
+    if (g_pool.size() >= 65536) return false;
+    EventPair p;
+    if (hipEventCreate(&p.a) != hipSuccess || hipEventCreate(&p.b) != hipSuccess) return false;
+    g_pool.push_back(p);
+  }
+  *a = g_pool[g_used].a;
+  *b = g_pool[g_used].b;
+  ++g_used;
+  return true;
+}
+
+extern "C" int mi_profile_enable(int32_t on) {
+  g_profile = on != 0;
+  g_used = 0;
+  return MI_OK;
+}
+
+extern "C" int32_t mi_profile_collect(float* out_ms, int32_t capacity) {
+  int32_t n = 0;
+  for (size_t i = 0; i < g_used; ++i) {
+    if (hipEventSynchronize(g_pool[i].b) != hipSuccess) break;
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, g_pool[i].a, g_pool[i].b) != hipSuccess) break;
+    if (out_ms && n < capacity) out_ms[n] = ms;
+    ++n;
+  }
+  g_used = 0;
+  return n;
+}

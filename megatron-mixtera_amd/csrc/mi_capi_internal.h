@@ -1,0 +1,38 @@
+// Host-side plumbing shared by the C-ABI entry points: error codes, the
+// per-thread error message, launch checking and the tuning knobs.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+// Return codes of every entry point (0 = enqueued, negative = rejected, nothing launched).
+enum {
+  MI_OK = 0,
+  MI_ERR_NULL = -1,         // a required pointer is null
+  MI_ERR_SHAPE = -2,        // sizes inconsistent with each other
+  MI_ERR_ALIGN = -3,        // pointer or stride breaks the 16-byte row alignment
+  MI_ERR_UNSUPPORTED = -4,  // valid request this build has no kernel for
+  MI_ERR_WORKSPACE = -5,    // caller-provided workspace too small
+  MI_ERR_LAUNCH = -6,       // the HIP runtime refused the launch
+};
+
+// KV storage formats.
+enum { MI_KV_BF16 = 0, MI_KV_FP8_E4M3 = 1 };
+
+// Norm applied to the head vectors before RoPE.
+enum { MI_NORM_NONE = 0, MI_NORM_RMS = 1, MI_NORM_L2 = 2 };
+
+struct MiTuning {
+  int decode_tile_subtiles;  // 16-token sub-tiles per loop iteration of the decode kernel: 1, 2 or 4
+  int prefill_tile_subtiles;
+};
+
+MiTuning& mi_tuning();
+int mi_fail(int code, const char* msg);
+int mi_check_launch(const char* where);
+// Next start/stop event pair when kernel timing is enabled (see mi_profile_enable).
+bool mi_profile_next(hipEvent_t* start, hipEvent_t* stop);
+
+namespace mi {
+int resolve_split_tokens(int R, int Hkv, int chunk, int max_kv_len, int split_tokens);
+}

@@ -1,0 +1,104 @@
+// Shared device helpers for the gfx950 (MI355X) paged-KV kernels.
+//
+// Conventions used by every kernel in this directory:
+//  * a wavefront is 64 lanes; `m16 = lane & 15` and `g = lane >> 4` are the two
+//    coordinates every MFMA operand layout is expressed in;
+//  * bf16 values travel as raw uint16_t / packed uint32_t pairs and are only
+//    reinterpreted at the MFMA call sites;
+//  * all kernels are enqueue-only: no host synchronisation, no device-side
+//    allocation, every buffer is owned by the caller.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+
+constexpr int kWave = 64;
+
+// D(16x16) += A(16x32) * B(32x16), bf16 inputs, fp32 accumulate.
+// Lane (m16, g) supplies A[m16][8g..8g+7] and B[8g..8g+7][m16]; it receives
+// D[4g+i][m16] in slot i.  Only the pairing "A slot j of group g meets B slot j
+// of group g" is relied upon, so any consistent assignment of contraction
+// indices to (g, j) gives the same dot products.
+static __device__ __forceinline__ f32x4_t mfma_16x16x32(uint4 a, uint4 b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+// D(16x16) += A(16x16) * B(16x16), bf16 inputs, fp32 accumulate.
+// Lane (m16, g) supplies A[m16][4g..4g+3] and B[4g..4g+3][m16]; D as above.
+static __device__ __forceinline__ f32x4_t mfma_16x16x16(uint2 a, uint2 b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a),
+                                                   __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+}
+
+// Two fp32 -> packed bf16 pair (round to nearest even), `lo` in bits 0..15.
+static __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2_t v = {lo, hi};
+  bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+static __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
+  return (uint16_t)(pack_bf16x2(x, 0.f) & 0xffffu);
+}
+
+static __device__ __forceinline__ float bf16_to_f32(uint16_t x) {
+  return __builtin_bit_cast(float, (uint32_t)x << 16);
+}
+static __device__ __forceinline__ float bf16lo_to_f32(uint32_t pair) {
+  return __builtin_bit_cast(float, pair << 16);
+}
+static __device__ __forceinline__ float bf16hi_to_f32(uint32_t pair) {
+  return __builtin_bit_cast(float, pair & 0xffff0000u);
+}
+
+// (hi16 of a | lo16 ... ) helpers for the in-register 4x4 bf16 transposes.
+// low_halves(a, b)  = (a.lo16 << 16) | b.lo16
+// high_halves(a, b) = (a.hi16 << 16) | b.hi16
+static __device__ __forceinline__ uint32_t low_halves(uint32_t a, uint32_t b) {
+  return __builtin_amdgcn_perm(a, b, 0x05040100u);
+}
+static __device__ __forceinline__ uint32_t high_halves(uint32_t a, uint32_t b) {
+  return __builtin_amdgcn_perm(a, b, 0x07060302u);
+}
+
+static __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+static __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Exchange with the lane 16 / 32 positions away (the two "g" bits).
+static __device__ __forceinline__ float xor16(float x) { return __shfl_xor(x, 16, 64); }
+static __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32, 64); }
+
+// 16-byte global loads / stores through plain pointers.
+static __device__ __forceinline__ uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+static __device__ __forceinline__ uint2 ld8(const void* p) { return *reinterpret_cast<const uint2*>(p); }
+static __device__ __forceinline__ void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
+static __device__ __forceinline__ void st8(void* p, uint2 v) { *reinterpret_cast<uint2*>(p) = v; }
+
+// OCP e4m3fn byte pairs -> fp32 (gfx950 converts OCP formats natively).
+static __device__ __forceinline__ f32x2_t fp8x2_lo_to_f32(uint32_t w) {
+  return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+}
+static __device__ __forceinline__ f32x2_t fp8x2_hi_to_f32(uint32_t w) {
+  return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+}
+// Four e4m3fn bytes -> two packed bf16 pairs (exact: every e4m3 value is a bf16 value, so
+// keeping the upper 16 bits of the fp32 conversion loses nothing).
+static __device__ __forceinline__ uint2 fp8x4_to_bf16x4(uint32_t w) {
+  const f32x2_t a = fp8x2_lo_to_f32(w), b = fp8x2_hi_to_f32(w);
+  const float a0 = a.x, a1 = a.y, b0 = b.x, b1 = b.y;
+  uint2 r;
+  r.x = high_halves(__float_as_uint(a1), __float_as_uint(a0));
+  r.y = high_halves(__float_as_uint(b1), __float_as_uint(b0));
+  return r;
+}
+
+}  // namespace mi

@@ -1,0 +1,242 @@
+// Fused q/k head norm + rotary embedding (+ optional KV-append) for the decode
+// and prefill Q/K of one layer.
+//
+// Replaces, in one launch, what the reference runs as ~20 small kernels per
+// layer:
+//   q_layernorm / k_layernorm over the head dim
+//       (megatron/core/transformer/attention.py:1026-1030; RMSNorm or L2Norm,
+//        megatron/core/transformer/torch_norm.py:15-96),
+//   apply_rotary_emb_key / apply_rotary_emb_query: gather emb[pos] and
+//       t*cos + rotate_half(t)*sin
+//       (megatron/core/inference/contexts/dynamic_context.py:566-631,
+//        megatron/core/models/common/embeddings/rope_utils.py:73-126),
+//   append_key_value_cache (dynamic_context.py:511-545) when a cache is given.
+//
+// Rounding: with `faithful != 0` every point where the unfused bf16 chain rounds
+// is rounded here too -- norm output, cos and sin, both products and their sum --
+// so the result equals the op-by-op bf16 evaluation; with `faithful == 0` the
+// whole expression is evaluated in fp32 and rounded once.
+//
+// One workgroup (4 waves) per token; each head vector is handled by d/2 lanes,
+// lane i owning elements i and i + d/2.  The normalised vector goes through a
+// few hundred bytes of LDS so that any rotary pairing (half-split, interleaved,
+// partial rotary width) reads its partner from there.
+#include "mi_common.h"
+#include "mi_capi_internal.h"
+
+namespace mi {
+
+struct NormRopeParams {
+  uint16_t* q;  // [T][Hq][d] in place
+  int64_t q_st;
+  const uint16_t* k;  // [T][Hkv][d]
+  int64_t k_st;
+  uint16_t* k_out;  // [T][Hkv][d] or null
+  int64_t ko_st;
+  const uint16_t* v;  // [T][Hkv][d] or null (append only)
+  int64_t v_st;
+  const uint16_t* q_w;  // [d] bf16 or null
+  const uint16_t* k_w;
+  const float* emb;  // [max_pos][rot] angles, or null for no rotary
+  int64_t emb_stride;
+  const int64_t* q_pos;  // [T]
+  const int64_t* k_pos;  // [T]
+  uint16_t* kc;  // cache or null
+  uint16_t* vc;
+  int64_t chunk_elems, tok_elems;
+  const int64_t* tok_chunk;  // slot mode A
+  const int64_t* tok_local;
+  const int32_t* bt;  // slot mode B (decode)
+  int64_t bt_stride;
+  const int32_t* lens;
+  int32_t T, Hq, Hkv, d, rot, chunk, norm, interleaved, faithful;
+  float eps, mscale;
+};
+
+static __device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+
+template <int D>
+__global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p) {
+  constexpr int LPV = D / 2;        // lanes per head vector
+  constexpr int VPW = 64 / LPV;     // head vectors per wave
+  constexpr int VPB = 4 * VPW;      // head vectors per workgroup pass
+  __shared__ float lds[VPB][D];
+
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = lane % LPV;
+  const int slot = wave * VPW + lane / LPV;
+  const int nvec = p.Hq + p.Hkv;
+  const bool faithful = p.faithful != 0;
+
+  // Destination slot of this token in the cache (wave-uniform).
+  int64_t cache_off = -1;
+  if (p.kc) {
+    if (p.tok_chunk) {
+      cache_off = p.tok_chunk[t] * p.chunk_elems + p.tok_local[t] * p.tok_elems;
+    } else {
+      const int len = p.lens[t];
+      if (len > 0) {
+        const int pos = len - 1, ci = pos / p.chunk;
+        cache_off = (int64_t)p.bt[(int64_t)t * p.bt_stride + ci] * p.chunk_elems +
+                    (int64_t)(pos - ci * p.chunk) * p.tok_elems;
+      }
+    }
+  }
+
+  for (int base = 0; base < nvec; base += VPB) {
+    const int vec = base + slot;
+    const bool active = vec < nvec;
+    const bool is_q = vec < p.Hq;
+    const int head = is_q ? vec : vec - p.Hq;
+    const uint16_t* src = is_q ? p.q + (int64_t)t * p.q_st + (int64_t)head * D
+                               : p.k + (int64_t)t * p.k_st + (int64_t)head * D;
+    float x0 = 0.f, x1 = 0.f;
+    if (active) {
+      x0 = bf16_to_f32(src[i]);
+      x1 = bf16_to_f32(src[i + LPV]);
+    }
+    float y0 = x0, y1 = x1;
+    if (p.norm != MI_NORM_NONE) {
+      float ss = x0 * x0 + x1 * x1;
+#pragma unroll
+      for (int o = LPV / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      const float rstd = rsqrtf(ss * (1.f / D) + p.eps);
+      y0 = x0 * rstd;
+      y1 = x1 * rstd;
+      const uint16_t* w = is_q ? p.q_w : p.k_w;
+      if (p.norm == MI_NORM_RMS && w) {
+        y0 *= bf16_to_f32(w[i]);
+        y1 *= bf16_to_f32(w[i + LPV]);
+      }
+      if (faithful) {
+        y0 = round_bf16(y0);
+        y1 = round_bf16(y1);
+      }
+    }
+    float o0 = y0, o1 = y1;
+    if (p.emb) {
+      lds[slot][i] = y0;
+      lds[slot][i + LPV] = y1;
+      __syncthreads();
+      const int64_t pos = active ? (is_q ? p.q_pos[t] : p.k_pos[t]) : 0;
+      const float* ang = p.emb + pos * p.emb_stride;
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const int e = i + w * LPV;
+        const float y = w ? y1 : y0;
+        if (active && e < p.rot) {
+          int partner;
+          float sign;
+          if (p.interleaved) {
+            partner = e ^ 1;
+            sign = (e & 1) ? 1.f : -1.f;
+          } else {
+            const int half = p.rot >> 1;
+            partner = e < half ? e + half : e - half;
+            sign = e < half ? -1.f : 1.f;
+          }
+          const float a = ang[e];
+          float c = cosf(a) * p.mscale, s = sinf(a) * p.mscale;
+          const float yp = lds[slot][partner] * sign;
+          float out;
+          if (faithful) {
+            c = round_bf16(c);
+            s = round_bf16(s);
+            out = round_bf16(y * c) + round_bf16(yp * s);
+          } else {
+            out = y * c + yp * s;
+          }
+          if (w) o1 = out; else o0 = out;
+        }
+      }
+      __syncthreads();
+    }
+    if (active) {
+      const uint16_t b0 = f32_to_bf16(o0), b1 = f32_to_bf16(o1);
+      if (is_q) {
+        uint16_t* dst = p.q + (int64_t)t * p.q_st + (int64_t)head * D;
+        dst[i] = b0;
+        dst[i + LPV] = b1;
+      } else {
+        if (p.k_out) {
+          uint16_t* dst = p.k_out + (int64_t)t * p.ko_st + (int64_t)head * D;
+          dst[i] = b0;
+          dst[i + LPV] = b1;
+        }
+        if (cache_off >= 0) {
+          uint16_t* dst = p.kc + cache_off + (int64_t)head * D;
+          dst[i] = b0;
+          dst[i + LPV] = b1;
+        }
+      }
+    }
+  }
+  // Value rows are copied unchanged.
+  if (cache_off >= 0 && p.v) {
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(p.v + (int64_t)t * p.v_st);
+    uint32_t* dst = reinterpret_cast<uint32_t*>(p.vc + cache_off);
+    for (int e = threadIdx.x; e < p.Hkv * D / 2; e += 256) dst[e] = src[e];
+  }
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" int mi_norm_rope_append(
+    void* q, int64_t q_stride_tok, const void* k, int64_t k_stride_tok, void* k_out,
+    int64_t k_out_stride_tok, const void* v, int64_t v_stride_tok, const void* q_weight,
+    const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles,
+    int64_t angles_stride, int32_t rot_dim, int32_t rotary_interleaved, float mscale,
+    const int64_t* q_positions, const int64_t* k_positions, void* k_cache, void* v_cache,
+    int64_t kv_stride_chunk, int64_t kv_stride_tok, const int64_t* token_to_chunk_idx,
+    const int64_t* token_to_local_pos, const int32_t* block_table, int64_t bt_stride,
+    const int32_t* kv_lens, int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv,
+    int32_t head_dim, int32_t faithful_rounding, void* stream) {
+  if (T == 0) return MI_OK;
+  if (T < 0 || Hq < 0 || Hkv < 0 || Hq + Hkv == 0)
+    return mi_fail(MI_ERR_SHAPE, "mi_norm_rope_append: bad sizes");
+  if ((Hq > 0 && !q) || (Hkv > 0 && !k))
+    return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: q / k missing");
+  if (head_dim != 64 && head_dim != 128)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_norm_rope_append: head_dim must be 64 or 128");
+  if (norm_kind != MI_NORM_NONE && norm_kind != MI_NORM_RMS && norm_kind != MI_NORM_L2)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_norm_rope_append: unknown norm kind");
+  if (rotary_angles) {
+    if (rot_dim <= 0 || rot_dim > head_dim || (rot_dim & 1) || angles_stride < rot_dim)
+      return mi_fail(MI_ERR_SHAPE, "mi_norm_rope_append: rot_dim must be even and within head_dim");
+    if ((Hq > 0 && !q_positions) || (Hkv > 0 && !k_positions))
+      return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: rotary positions missing");
+  }
+  const bool to_cache = k_cache != nullptr;
+  if (to_cache) {
+    if (!v_cache || !v) return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: append needs v and v_cache");
+    const bool mode_a = token_to_chunk_idx && token_to_local_pos;
+    const bool mode_b = block_table && kv_lens && chunk_tokens > 0;
+    if (!mode_a && !mode_b)
+      return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: append needs per-token slots or block table + lengths");
+    if ((((uintptr_t)v | (uintptr_t)v_cache) & 3) || (v_stride_tok & 1) || (kv_stride_chunk & 1) || (kv_stride_tok & 1))
+      return mi_fail(MI_ERR_ALIGN, "mi_norm_rope_append: value rows must be 4-byte aligned");
+  }
+  NormRopeParams p = {};
+  p.q = (uint16_t*)q; p.q_st = q_stride_tok;
+  p.k = (const uint16_t*)k; p.k_st = k_stride_tok;
+  p.k_out = (uint16_t*)k_out; p.ko_st = k_out_stride_tok;
+  p.v = (const uint16_t*)v; p.v_st = v_stride_tok;
+  p.q_w = (const uint16_t*)q_weight; p.k_w = (const uint16_t*)k_weight;
+  p.emb = rotary_angles; p.emb_stride = angles_stride;
+  p.q_pos = q_positions; p.k_pos = k_positions;
+  p.kc = (uint16_t*)k_cache; p.vc = (uint16_t*)v_cache;
+  p.chunk_elems = kv_stride_chunk; p.tok_elems = kv_stride_tok;
+  p.tok_chunk = (token_to_chunk_idx && token_to_local_pos) ? token_to_chunk_idx : nullptr;
+  p.tok_local = token_to_local_pos;
+  p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens;
+  p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.d = head_dim; p.rot = rot_dim; p.chunk = chunk_tokens;
+  p.norm = norm_kind; p.interleaved = rotary_interleaved; p.faithful = faithful_rounding;
+  p.eps = eps; p.mscale = mscale;
+  hipStream_t st = (hipStream_t)stream;
+  if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), dim3(T), dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((norm_rope_append_kernel<64>), dim3(T), dim3(256), 0, st, p);
+  return mi_check_launch("mi_norm_rope_append");
+}

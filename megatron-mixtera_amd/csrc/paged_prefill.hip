@@ -1,0 +1,306 @@
+// Paged varlen causal attention for chunked prefill and mixed prefill+decode
+// batches on gfx950.
+//
+// Replaces flash_attn_varlen_func(q, k_cache, v_cache, cu_seqlens_q, cu_seqlens_k,
+// max_seqlen_q, max_seqlen_k, softmax_scale, causal=True, block_table=...)
+// as called from Attention.flash_decode_and_prefill
+// (megatron/core/transformer/attention.py:546-557).  The new tokens' K/V are
+// already in the paged cache (append runs first), so keys are only ever read
+// through the block table.  Mask: query i (0-based among the request's Lq new
+// tokens) sees keys j <= i + (Lk - Lq).
+//
+// A wavefront owns 64 "rows" = (64/G query tokens) x (G query heads of one KV
+// head) and walks the keys 16 at a time with the same matrix-core scheme as the
+// decode kernel, reusing every K / V fragment for four 16-row tiles:
+//   S^T[tok][row] = K . Q^T   (mfma 16x16x32),   O^T[d][row] += V^T . P^T (16x16x16).
+// The four waves of a workgroup take four consecutive query blocks of the same
+// (request, KV head), so they pull identical K/V lines at about the same time.
+#include "mi_common.h"
+#include "mi_capi_internal.h"
+
+namespace mi {
+
+struct PrefillParams {
+  const uint16_t* q;
+  int64_t q_st, q_sh;
+  const uint8_t* kc;
+  const uint8_t* vc;
+  int64_t kv_sc;
+  int32_t kv_st, kv_sh;
+  const int32_t* bt;
+  int64_t bt_stride;
+  const int32_t* cu_q;
+  const int32_t* lens;
+  uint16_t* out;
+  int64_t o_st, o_sh;
+  int32_t T, R, Hq, Hkv, G, g_shift, chunk, chunk_shift;
+  float scale_log2;
+};
+
+template <int HD, int NT>
+__global__ __launch_bounds__(256) void paged_prefill_kernel(PrefillParams p) {
+  constexpr int KS = HD / 32;
+  constexpr int DV = HD / 16;
+  constexpr int NQ = 4;  // 16-row tiles per wave
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int m16 = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y;
+  const int G = p.G;
+  const int BQ = 64 >> p.g_shift;  // query tokens per wave
+  const int SBQ = 4 * BQ;          // query tokens per workgroup
+
+  // ---- which request does this workgroup belong to? ----------------------------
+  // Request r's workgroups start at pbs(r) = cu_q[r] / SBQ + r, a strictly
+  // increasing sequence that leaves at least ceil(Lq_r / SBQ) indices to r.
+  const int sb = blockIdx.x;
+  int lo = 0, hi = p.R - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (p.cu_q[mid] / SBQ + mid <= sb) lo = mid; else hi = mid - 1;
+  }
+  const int r = lo;
+  const int q_begin = p.cu_q[r];
+  const int Lq = p.cu_q[r + 1] - q_begin;
+  const int q0 = (sb - (q_begin / SBQ + r)) * SBQ + wave * BQ;  // first query of this wave
+  if (q0 >= Lq) return;
+  const int Lk = p.lens[r];
+  const int shift = Lk - Lq;  // key position of query 0
+  const int nq = min(BQ, Lq - q0);
+  const int kend = min(Lk, shift + q0 + nq);  // keys [0, kend) are visible to some row
+  const int last = Lk - 1;
+
+  // ---- query fragments and per-row causal limits ---------------------------------
+  uint4 qf[NQ][KS];
+  int qpos[NQ];
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    const int n = 16 * nt + m16;
+    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const bool valid = qi < nq;
+    qpos[nt] = valid ? shift + q0 + qi : last;
+    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      qf[nt][kk] = valid ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
+  }
+  const int ntiles = (nq * G + 15) >> 4;  // 16-row tiles that hold a valid row
+
+  const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * 2;
+  const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * 2;
+  const int64_t chunk_bytes = p.kv_sc * 2;
+  const int tok_bytes = p.kv_st * 2;
+
+  float m_run[NQ], l_run[NQ];
+  f32x4_t acc[NQ][DV];
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    m_run[nt] = -INFINITY;
+    l_run[nt] = 0.f;
+#pragma unroll
+    for (int e = 0; e < DV; ++e) acc[nt][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  if (kend <= 0) {
+    // No visible key (Lk == 0): rows are defined as zeros.
+#pragma unroll
+    for (int nt = 0; nt < NQ; ++nt) {
+      const int n = 16 * nt + m16;
+      const int qi = n >> p.g_shift, u = n & (G - 1);
+      if (qi < nq) {
+        uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
+        for (int i = 0; i < 4 * DV; i += 4) st8(o + i, make_uint2(0, 0));
+      }
+    }
+    return;
+  }
+
+  for (int T = 0; T < kend; T += 16 * NT) {
+    uint4 kf[NT][KS];
+    uint4 vf16[NT][4];
+    uint2 vf8[NT][4];
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      const int T0 = T + 16 * u;
+      const int tu = min(T0, last);
+      const int ci = p.chunk_shift >= 0 ? (tu >> p.chunk_shift) : (tu / p.chunk);
+      const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
+      const int cbase = ci * p.chunk;
+      const uint8_t* kc = kbase + (int64_t)pc * chunk_bytes;
+      const uint8_t* vc = vbase + (int64_t)pc * chunk_bytes;
+      const uint8_t* krow = kc + (min(T0 + m16, last) - cbase) * tok_bytes;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) kf[u][kk] = ld16(krow + (32 * kk + 8 * g) * 2);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint8_t* vrow = vc + (min(T0 + 4 * g + j, last) - cbase) * tok_bytes + DV * m16 * 2;
+        if (HD == 128) vf16[u][j] = ld16(vrow);
+        else vf8[u][j] = ld8(vrow);
+      }
+    }
+
+#pragma unroll
+    for (int nt = 0; nt < NQ; ++nt) {
+      if (nt >= ntiles) break;  // wave-uniform
+      // ---- scores of this 16-row tile against the NT key sub-tiles --------------
+      float sc[NT][4];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32(kf[u][kk], qf[nt][kk], sacc);
+        const int tok0 = T + 16 * u + 4 * g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = (tok0 + i <= qpos[nt]) ? sacc[i] * p.scale_log2 : -INFINITY;
+          sc[u][i] = v;
+          tmax = fmaxf(tmax, v);
+        }
+      }
+      tmax = fmaxf(tmax, xor16(tmax));
+      tmax = fmaxf(tmax, xor32(tmax));
+      // Key 0 is visible to every row of a well-formed request (Lk >= Lq), so m_run
+      // is finite after the first tile; a later tile that is fully masked for a row
+      // leaves it unchanged.
+      const float m_raw = fmaxf(m_run[nt], tmax);
+      const float m_new = m_raw == -INFINITY ? 0.f : m_raw;  // row with no visible key so far
+      const float alpha = fast_exp2(m_run[nt] - m_new);
+      m_run[nt] = m_raw;
+      float psum = 0.f;
+      uint2 pf[NT];
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        float pv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pv[i] = fast_exp2(sc[u][i] - m_new);
+          psum += pv[i];
+        }
+        pf[u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+      }
+      l_run[nt] = l_run[nt] * alpha + psum;
+#pragma unroll
+      for (int e = 0; e < DV; ++e) {
+        acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
+      }
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        if constexpr (HD == 128) {
+          const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0]);
+          const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1]);
+          const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2]);
+          const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3]);
+#pragma unroll
+          for (int pr = 0; pr < 4; ++pr) {
+            acc[nt][2 * pr] = mfma_16x16x16(
+                make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr])), pf[u], acc[nt][2 * pr]);
+            acc[nt][2 * pr + 1] = mfma_16x16x16(
+                make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr])), pf[u], acc[nt][2 * pr + 1]);
+          }
+        } else {
+          const uint2 a = vf8[u][0], b = vf8[u][1], c = vf8[u][2], d = vf8[u][3];
+          acc[nt][0] = mfma_16x16x16(make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x)), pf[u], acc[nt][0]);
+          acc[nt][1] = mfma_16x16x16(make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x)), pf[u], acc[nt][1]);
+          acc[nt][2] = mfma_16x16x16(make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y)), pf[u], acc[nt][2]);
+          acc[nt][3] = mfma_16x16x16(make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y)), pf[u], acc[nt][3]);
+        }
+      }
+    }
+  }
+
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    float l_tot = l_run[nt] + xor16(l_run[nt]);
+    l_tot += xor32(l_tot);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int n = 16 * nt + m16;
+    const int qi = n >> p.g_shift, u = n & (G - 1);
+    if (qi < nq) {
+      uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (DV == 8) {
+          st16(o + 8 * i, make_uint4(pack_bf16x2(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
+                                     pack_bf16x2(acc[nt][2][i] * inv, acc[nt][3][i] * inv),
+                                     pack_bf16x2(acc[nt][4][i] * inv, acc[nt][5][i] * inv),
+                                     pack_bf16x2(acc[nt][6][i] * inv, acc[nt][7][i] * inv)));
+        } else {
+          st8(o + 4 * i, make_uint2(pack_bf16x2(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
+                                    pack_bf16x2(acc[nt][2][i] * inv, acc[nt][3][i] * inv)));
+        }
+      }
+    }
+  }
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
+                                              int32_t head_dim, int32_t max_kv_len,
+                                              int32_t split_tokens) {
+  (void)T; (void)R; (void)Hq; (void)Hkv; (void)head_dim; (void)max_kv_len; (void)split_tokens;
+  return 0;  // the current kernel keeps every row's state in registers
+}
+
+extern "C" int mi_paged_prefill_attention(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
+    const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seqlens_q,
+    const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head,
+    void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
+    int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
+    float softmax_scale, void* stream) {
+  (void)workspace; (void)workspace_bytes; (void)max_kv_len; (void)split_tokens;
+  if (T == 0 || R == 0) return MI_OK;
+  if (!q || !k_cache || !v_cache || !block_table || !cu_seqlens_q || !kv_lens || !out)
+    return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention: null pointer argument");
+  if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: need T, R >= 0 and Hq a multiple of Hkv");
+  const int G = Hq / Hkv;
+  if (G > 16 || (G & (G - 1)))
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: query heads per KV head must be 1, 2, 4, 8 or 16");
+  if (head_dim != 64 && head_dim != 128)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: head_dim must be 64 or 128");
+  if (chunk_tokens <= 0 || chunk_tokens % 16)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: chunk size must be a positive multiple of 16");
+  if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention: q/k/v/out must be 16-byte aligned");
+  if ((q_stride_tok | q_stride_head | o_stride_tok | o_stride_head | kv_stride_chunk | kv_stride_tok | kv_stride_head) % 8)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention: strides must keep rows 16-byte aligned");
+  if (kv_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: one chunk must span less than 2 GiB");
+
+  PrefillParams p;
+  p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
+  p.kc = (const uint8_t*)k_cache; p.vc = (const uint8_t*)v_cache;
+  p.kv_sc = kv_stride_chunk; p.kv_st = (int32_t)kv_stride_tok; p.kv_sh = (int32_t)kv_stride_head;
+  p.bt = block_table; p.bt_stride = bt_stride; p.cu_q = cu_seqlens_q; p.lens = kv_lens;
+  p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
+  p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G;
+  p.g_shift = 0;
+  while ((1 << p.g_shift) < G) ++p.g_shift;
+  p.chunk = chunk_tokens;
+  p.chunk_shift = -1;
+  if (!(chunk_tokens & (chunk_tokens - 1))) {
+    p.chunk_shift = 0;
+    while ((1 << p.chunk_shift) < chunk_tokens) ++p.chunk_shift;
+  }
+  p.scale_log2 = softmax_scale * 1.4426950408889634f;
+
+  const int sbq = 4 * (64 / G);
+  dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  const int nt = mi_tuning().prefill_tile_subtiles;
+  if (head_dim == 128) {
+    if (nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<128, 1>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_kernel<128, 2>), grid, block, 0, st, p);
+  } else {
+    if (nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<64, 1>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_kernel<64, 2>), grid, block, 0, st, p);
+  }
+  return mi_check_launch("mi_paged_prefill_attention");
+}

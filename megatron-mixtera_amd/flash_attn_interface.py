@@ -1,0 +1,77 @@
+"""The two flash-attn entry points the reference's dynamic path calls, on MI355X kernels.
+
+``Attention.flash_decode_and_prefill`` (megatron/core/transformer/attention.py:470-601)
+resolves the module-level names ``flash_attn_with_kvcache`` and ``flash_attn_varlen_func``;
+these functions accept the keyword surface used there and run the paged kernels of
+``libmi355_decode.so``.  Arguments the reference never passes on this path (dropout,
+windows, alibi, rotary fusion, new-token append inside the call) are rejected rather than
+silently ignored.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch import Tensor
+
+from . import ops
+
+
+def _reject(**unsupported) -> None:
+    bad = [k for k, v in unsupported.items() if v not in (None, False, 0, 0.0, (-1, -1))]
+    if bad:
+        raise NotImplementedError(f"unsupported flash-attn arguments on the paged MI355X path: {bad}")
+
+
+def flash_attn_with_kvcache(q: Tensor, k_cache: Tensor, v_cache: Tensor, k: Optional[Tensor] = None,
+                            v: Optional[Tensor] = None, rotary_cos=None, rotary_sin=None,
+                            cache_seqlens: Optional[Tensor] = None, cache_batch_idx=None,
+                            cache_leftpad=None, block_table: Optional[Tensor] = None,
+                            softmax_scale: Optional[float] = None, causal: bool = False,
+                            window_size=(-1, -1), softcap: float = 0.0, rotary_interleaved: bool = True,
+                            alibi_slopes=None, num_splits: int = 0, return_softmax_lse: bool = False,
+                            *, page_table: Optional[Tensor] = None, k_scales: Optional[Tensor] = None,
+                            v_scales: Optional[Tensor] = None, max_seqlen_k: Optional[int] = None) -> Tensor:
+    """Paged decode attention: ``q`` is ``[batch, 1, Hq, d]``, one query token per request.
+
+    ``cache_seqlens`` (int32 ``[batch]``) already counts the token appended this step;
+    ``block_table`` / ``page_table`` is int32 ``[batch, max_chunks]``.  With a single query
+    token the causal mask is a no-op, so ``causal`` is accepted either way.
+    """
+    _reject(k=k, v=v, rotary_cos=rotary_cos, rotary_sin=rotary_sin, cache_batch_idx=cache_batch_idx,
+            cache_leftpad=cache_leftpad, window_size=window_size, softcap=softcap, alibi_slopes=alibi_slopes,
+            return_softmax_lse=return_softmax_lse)
+    table = block_table if block_table is not None else page_table
+    if table is None or cache_seqlens is None:
+        raise ValueError("the paged path needs block_table (or page_table) and cache_seqlens")
+    if q.dim() != 4 or q.size(1) != 1:
+        raise NotImplementedError("flash_attn_with_kvcache on this path takes one query token per request: q [B,1,Hq,d]")
+    return ops.paged_decode_attention(q, k_cache, v_cache, cache_seqlens, table, softmax_scale=softmax_scale,
+                                      max_kv_len=max_seqlen_k, k_scales=k_scales, v_scales=v_scales)
+
+
+def flash_attn_varlen_func(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor, cu_seqlens_k: Optional[Tensor],
+                           max_seqlen_q: int, max_seqlen_k: int, dropout_p: float = 0.0,
+                           softmax_scale: Optional[float] = None, causal: bool = False, window_size=(-1, -1),
+                           softcap: float = 0.0, alibi_slopes=None, deterministic: bool = False,
+                           return_attn_probs: bool = False, block_table: Optional[Tensor] = None,
+                           *, seqused_k: Optional[Tensor] = None) -> Tensor:
+    """Paged varlen causal attention: ``q`` is ``[T, Hq, d]``, ``k``/``v`` are the paged caches.
+
+    Per-request key counts come from ``seqused_k`` if given, else from the differences of
+    ``cu_seqlens_k``.  The mask is flash-attn's bottom-right aligned causal mask.
+    """
+    _reject(dropout_p=dropout_p, window_size=window_size, softcap=softcap, alibi_slopes=alibi_slopes,
+            return_attn_probs=return_attn_probs)
+    if block_table is None:
+        raise NotImplementedError("only the paged form (block_table given) exists on this path")
+    if not causal:
+        raise NotImplementedError("the paged prefill kernel is causal")
+    if seqused_k is not None:
+        kv_lens = seqused_k
+    elif cu_seqlens_k is not None:
+        kv_lens = (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).contiguous()
+    else:
+        raise ValueError("need cu_seqlens_k or seqused_k")
+    return ops.paged_prefill_attention(q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table,
+                                       softmax_scale=softmax_scale, max_kv_len=max_seqlen_k)

@@ -1,0 +1,318 @@
+"""Torch-level wrappers over the C ABI: tensors in, raw pointers + strides out.
+
+Each function validates what only the host can see (dtypes, devices, contiguity of
+the innermost dimension), then enqueues exactly one C-ABI call on torch's current
+stream.  Nothing here computes: without the HIP library these functions raise.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from ._lib import MI_KV_BF16, MI_KV_FP8_E4M3, MI_NORM_L2, MI_NORM_NONE, MI_NORM_RMS  # noqa: F401
+
+_NORM_KINDS = {None: MI_NORM_NONE, "none": MI_NORM_NONE, "rms": MI_NORM_RMS, "l2": MI_NORM_L2}
+
+
+def _stream(t: Tensor) -> int:
+    if t.device.type != "cuda":
+        raise RuntimeError(
+            f"the HIP kernels need device tensors, got a tensor on {t.device}; there is no CPU path")
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _require(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _cache_strides(cache: Tensor) -> Tuple[int, int, int]:
+    """(chunk, token, head) element strides of a ``[N, C, Hkv, d]`` cache view."""
+    _require(cache.dim() == 4 and cache.stride(3) == 1, "KV cache must be [N, C, Hkv, d] with contiguous d")
+    return cache.stride(0), cache.stride(1), cache.stride(2)
+
+
+# per-device split-K workspace, grown on demand (owned here, handed to the C ABI as caller memory)
+_workspaces: dict = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> Optional[Tensor]:
+    if nbytes <= 0:
+        return None
+    ws = _workspaces.get(device)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _workspaces[device] = ws
+    return ws
+
+
+def set_tuning(name: str, value: int) -> None:
+    lib = _lib.load()
+    _lib.check(lib.mi_set_tuning(name.encode(), int(value)), "mi_set_tuning")
+
+
+# ---------------------------------------------------------------------------------------------
+# KV append
+# ---------------------------------------------------------------------------------------------
+def _rows(x: Tensor, name: str) -> Tuple[Tensor, int, int]:
+    """View ``[T, (1,) Hkv, d]`` as T rows of Hkv*d contiguous elements."""
+    if x.dim() == 4:
+        _require(x.size(1) == 1, f"{name}.size(1) must be 1")
+        x = x.squeeze(1)
+    _require(x.dim() == 3, f"{name} must be [T, Hkv, d]")
+    _require(x.stride(2) == 1 and x.stride(1) == x.size(2), f"{name} rows must be contiguous")
+    return x, x.size(1) * x.size(2), x.stride(0)
+
+
+def kv_append(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor,
+              token_to_chunk_idx: Tensor, token_to_local_pos: Tensor) -> None:
+    """``k_cache[chunk_idx[t], local[t]] = key[t]`` (and value): bit-exact scatter."""
+    lib = _lib.load()
+    key, row, k_st = _rows(key, "key")
+    value, row_v, v_st = _rows(value, "value")
+    T = key.size(0)
+    _require(row == row_v and value.size(0) == T and k_st == v_st, "key/value shapes differ")
+    _require(key.dtype == k_cache.dtype == v_cache.dtype == value.dtype, "dtype mismatch between K/V and cache")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
+    _require(sh == k_cache.size(3) and row == k_cache.size(2) * k_cache.size(3), "cache rows must be contiguous [Hkv, d]")
+    _require(token_to_chunk_idx.dtype == torch.int64 and token_to_local_pos.dtype == torch.int64,
+             "slot index tensors must be int64")
+    _require(token_to_chunk_idx.numel() >= T and token_to_local_pos.numel() >= T, "slot index tensors too short")
+    _require(token_to_chunk_idx.is_contiguous() and token_to_local_pos.is_contiguous(), "slot index tensors must be contiguous")
+    _lib.check(lib.mi_kv_append(key.data_ptr(), value.data_ptr(), k_st, k_cache.data_ptr(), v_cache.data_ptr(),
+                                sc, st, token_to_chunk_idx.data_ptr(), token_to_local_pos.data_ptr(),
+                                T, row, key.element_size(), _stream(key)), "mi_kv_append")
+
+
+def kv_append_decode(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor,
+                     block_table: Tensor, kv_lens: Tensor) -> None:
+    """Decode-step append with the slot derived on the GPU from block table + kv length."""
+    lib = _lib.load()
+    key, row, k_st = _rows(key, "key")
+    value, row_v, v_st = _rows(value, "value")
+    R = key.size(0)
+    _require(row == row_v and value.size(0) == R and k_st == v_st, "key/value shapes differ")
+    _require(key.dtype == k_cache.dtype == v_cache.dtype == value.dtype, "dtype mismatch between K/V and cache")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
+    _require(sh == k_cache.size(3) and row == k_cache.size(2) * k_cache.size(3), "cache rows must be contiguous [Hkv, d]")
+    _require(block_table.dtype == torch.int32 and kv_lens.dtype == torch.int32, "block_table / kv_lens must be int32")
+    _require(block_table.dim() == 2 and block_table.stride(1) == 1 and block_table.size(0) >= R, "bad block_table")
+    _require(kv_lens.is_contiguous() and kv_lens.numel() >= R, "bad kv_lens")
+    _lib.check(lib.mi_kv_append_decode(key.data_ptr(), value.data_ptr(), k_st, k_cache.data_ptr(), v_cache.data_ptr(),
+                                       sc, st, block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(),
+                                       R, k_cache.size(1), row, key.element_size(), _stream(key)),
+               "mi_kv_append_decode")
+
+
+# ---------------------------------------------------------------------------------------------
+# fp8 KV storage
+# ---------------------------------------------------------------------------------------------
+def quantize_chunks_fp8(src: Tensor, dst: Tensor, scales: Tensor) -> None:
+    """Quantise whole bf16 chunks ``[N, C, Hkv, d]`` into an e4m3fn byte cache + ``[N, Hkv]`` scales."""
+    lib = _lib.load()
+    _require(src.dtype == torch.bfloat16, "source chunks must be bf16")
+    _require(dst.element_size() == 1, "destination cache must hold one byte per element")
+    _require(scales.dtype == torch.float32 and scales.is_contiguous(), "scales must be contiguous fp32")
+    ssc, sst, ssh = _cache_strides(src)
+    dsc, dst_t, dsh = _cache_strides(dst)
+    N, C, H, D = src.shape
+    _require(tuple(dst.shape) == (N, C, H, D) and tuple(scales.shape) == (N, H), "shape mismatch")
+    _require(ssh == D and dsh == D, "heads must be contiguous")
+    _lib.check(lib.mi_kv_quantize_chunks_fp8(src.data_ptr(), ssc, sst, dst.data_ptr(), dsc, dst_t,
+                                             scales.data_ptr(), N, C, H, D, _stream(src)),
+               "mi_kv_quantize_chunks_fp8")
+
+
+def kv_append_decode_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor, k_scales: Tensor,
+                         v_scales: Tensor, block_table: Tensor, kv_lens: Tensor, headroom: float = 2.0) -> None:
+    """Quantise and append one new bf16 token per request into an fp8 cache."""
+    lib = _lib.load()
+    key, row, k_st = _rows(key, "key")
+    value, _, v_st = _rows(value, "value")
+    _require(key.dtype == torch.bfloat16 and value.dtype == torch.bfloat16 and k_st == v_st, "K/V must be bf16 with equal strides")
+    _require(k_cache.element_size() == 1 and v_cache.element_size() == 1, "fp8 caches hold one byte per element")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh) and sh == k_cache.size(3), "cache layout")
+    _require(k_scales.dtype == torch.float32 and v_scales.dtype == torch.float32, "scales must be fp32")
+    _require(k_scales.is_contiguous() and v_scales.is_contiguous(), "scales must be contiguous")
+    _require(block_table.dtype == torch.int32 and kv_lens.dtype == torch.int32, "block_table / kv_lens must be int32")
+    _lib.check(lib.mi_kv_append_decode_fp8(key.data_ptr(), value.data_ptr(), k_st, k_cache.data_ptr(), v_cache.data_ptr(),
+                                           sc, st, k_scales.data_ptr(), v_scales.data_ptr(), block_table.data_ptr(),
+                                           block_table.stride(0), kv_lens.data_ptr(), key.size(0), k_cache.size(1),
+                                           k_cache.size(2), k_cache.size(3), float(headroom), _stream(key)),
+               "mi_kv_append_decode_fp8")
+
+
+# ---------------------------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------------------------
+def _qo_view(x: Tensor, name: str) -> Tensor:
+    if x.dim() == 4:
+        _require(x.size(1) == 1, f"{name} must be [T, 1, Hq, d] or [T, Hq, d]")
+        x = x.squeeze(1)
+    _require(x.dim() == 3 and x.stride(2) == 1, f"{name} must be [T, Hq, d] with contiguous d")
+    _require(x.dtype == torch.bfloat16, f"{name} must be bf16")
+    return x
+
+
+def decode_workspace_bytes(R: int, Hq: int, Hkv: int, head_dim: int, chunk: int, max_kv_len: int,
+                           split_tokens: int = 0) -> int:
+    return int(_lib.load().mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, chunk, max_kv_len, split_tokens))
+
+
+def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens: Tensor, block_table: Tensor,
+                           *, softmax_scale: Optional[float] = None, max_kv_len: Optional[int] = None,
+                           split_tokens: int = 0, out: Optional[Tensor] = None,
+                           workspace: Optional[Tensor] = None, k_scales: Optional[Tensor] = None,
+                           v_scales: Optional[Tensor] = None) -> Tensor:
+    """One query token per request against the paged cache; returns a tensor shaped like ``q``."""
+    lib = _lib.load()
+    q3 = _qo_view(q, "q")
+    R, Hq, D = q3.shape
+    N, C, Hkv, Dk = k_cache.shape
+    _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
+    fp8 = k_cache.element_size() == 1
+    _require(fp8 or k_cache.dtype == torch.bfloat16, "KV cache must be bf16 or a one-byte fp8 type")
+    _require(v_cache.dtype == k_cache.dtype, "k_cache / v_cache dtypes differ")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
+    _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
+    _require(kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "kv_lens must be contiguous int32")
+    _require(block_table.size(0) >= R and kv_lens.numel() >= R, "block_table / kv_lens shorter than the batch")
+    if fp8:
+        _require(k_scales is not None and v_scales is not None, "fp8 cache needs k_scales and v_scales")
+        _require(k_scales.dtype == torch.float32 and v_scales.dtype == torch.float32, "scales must be fp32")
+        _require(tuple(k_scales.shape) == (N, Hkv) and tuple(v_scales.shape) == (N, Hkv), "scales must be [N, Hkv]")
+        _require(k_scales.is_contiguous() and v_scales.is_contiguous(), "scales must be contiguous")
+    if max_kv_len is None:
+        max_kv_len = block_table.size(1) * C
+    if softmax_scale is None:
+        softmax_scale = D ** -0.5
+    if out is None:
+        out = torch.empty_like(q)
+    o3 = _qo_view(out, "out")
+    _require(tuple(o3.shape) == (R, Hq, D), "out shape mismatch")
+    need = lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, C, max_kv_len, split_tokens)
+    if workspace is None:
+        workspace = _workspace(q.device, need)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _lib.check(lib.mi_paged_decode_attention(
+        q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
+        block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
+        _ptr(workspace), ws_bytes, R, Hq, Hkv, D, C, int(max_kv_len), int(split_tokens), float(softmax_scale),
+        MI_KV_FP8_E4M3 if fp8 else MI_KV_BF16, _ptr(k_scales), _ptr(v_scales), _stream(q)),
+        "mi_paged_decode_attention")
+    return out
+
+
+def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
+                            block_table: Tensor, *, softmax_scale: Optional[float] = None,
+                            max_kv_len: Optional[int] = None, out: Optional[Tensor] = None) -> Tensor:
+    """Varlen causal attention of new tokens over the paged cache (bottom-right aligned mask)."""
+    lib = _lib.load()
+    q3 = _qo_view(q, "q")
+    T, Hq, D = q3.shape
+    N, C, Hkv, Dk = k_cache.shape
+    _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
+    _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16, "prefill needs a bf16 cache")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
+    _require(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.is_contiguous(), "cu_seqlens_q must be contiguous int32")
+    R = cu_seqlens_q.numel() - 1
+    _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
+    _require(kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "kv_lens must be contiguous int32")
+    _require(block_table.size(0) >= R and kv_lens.numel() >= R, "block_table / kv_lens shorter than the batch")
+    if max_kv_len is None:
+        max_kv_len = block_table.size(1) * C
+    if softmax_scale is None:
+        softmax_scale = D ** -0.5
+    if out is None:
+        out = torch.empty_like(q)
+    o3 = _qo_view(out, "out")
+    _require(tuple(o3.shape) == (T, Hq, D), "out shape mismatch")
+    _lib.check(lib.mi_paged_prefill_attention(
+        q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
+        block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),
+        o3.data_ptr(), o3.stride(0), o3.stride(1), None, 0, T, R, Hq, Hkv, D, C, int(max_kv_len), 0,
+        float(softmax_scale), _stream(q)), "mi_paged_prefill_attention")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# fused head norm + rotary embedding (+ append)
+# ---------------------------------------------------------------------------------------------
+def _angles(emb: Optional[Tensor]) -> Tuple[Optional[Tensor], int, int]:
+    """Accept the reference's ``[max_seq, 1, 1, rot]`` fp32 table (or ``[max_seq, rot]``)."""
+    if emb is None:
+        return None, 0, 0
+    _require(emb.dtype == torch.float32, "rotary table must be fp32 angles")
+    e2 = emb.reshape(emb.size(0), emb.size(-1)) if emb.dim() != 2 else emb
+    _require(e2.stride(1) == 1, "rotary table rows must be contiguous")
+    return e2, e2.stride(0), e2.size(1)
+
+
+def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: Optional[Tensor] = None,
+                     q_weight: Optional[Tensor] = None, k_weight: Optional[Tensor] = None,
+                     eps: float = 1e-5, norm: Optional[str] = None, rotary_emb: Optional[Tensor] = None,
+                     q_positions: Optional[Tensor] = None, k_positions: Optional[Tensor] = None,
+                     rotary_interleaved: bool = False, mscale: float = 1.0, key_out: Optional[Tensor] = None,
+                     k_cache: Optional[Tensor] = None, v_cache: Optional[Tensor] = None,
+                     token_to_chunk_idx: Optional[Tensor] = None, token_to_local_pos: Optional[Tensor] = None,
+                     block_table: Optional[Tensor] = None, kv_lens: Optional[Tensor] = None,
+                     faithful_rounding: bool = True) -> None:
+    """Norm (none / rms / l2) then RoPE on ``query`` (in place) and ``key`` (to ``key_out`` and/or cache)."""
+    lib = _lib.load()
+    ref = query if query is not None else key
+    _require(ref is not None, "need query and/or key")
+    T = Hq = Hkv = 0
+    D = ref.size(-1)
+    q3 = k3 = None
+    if query is not None:
+        q3 = _qo_view(query, "query")
+        _require(q3.stride(1) == D, "query heads must be contiguous")
+        T, Hq = q3.size(0), q3.size(1)
+    if key is not None:
+        k3 = _qo_view(key, "key")
+        _require(k3.stride(1) == D, "key heads must be contiguous")
+        T, Hkv = k3.size(0), k3.size(1)
+        _require(query is None or q3.size(0) == T, "query / key token counts differ")
+    ko3 = None
+    if key_out is not None:
+        ko3 = _qo_view(key_out, "key_out")
+        _require(tuple(ko3.shape) == tuple(k3.shape) and ko3.stride(1) == D, "key_out shape")
+    v3 = None
+    if value is not None:
+        v3 = _qo_view(value, "value")
+        _require(tuple(v3.shape) == tuple(k3.shape) and v3.stride(1) == D, "value shape")
+    ang, a_stride, rot = _angles(rotary_emb)
+    for w in (q_weight, k_weight):
+        _require(w is None or (w.dtype == torch.bfloat16 and w.numel() == D and w.is_contiguous()), "norm weights must be bf16 [d]")
+    for pz in (q_positions, k_positions, token_to_chunk_idx, token_to_local_pos):
+        _require(pz is None or (pz.dtype == torch.int64 and pz.is_contiguous() and pz.numel() >= T), "index rows must be int64 [>=T]")
+    sc = st = 0
+    chunk = 0
+    if k_cache is not None:
+        _require(k_cache.dtype == torch.bfloat16 and v_cache is not None and v_cache.dtype == torch.bfloat16, "bf16 caches")
+        sc, st, sh = _cache_strides(k_cache)
+        _require(_cache_strides(v_cache) == (sc, st, sh) and sh == D, "cache layout")
+        chunk = k_cache.size(1)
+        if block_table is not None:
+            _require(block_table.dtype == torch.int32 and block_table.stride(1) == 1, "bad block_table")
+            _require(kv_lens is not None and kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "bad kv_lens")
+    _lib.check(lib.mi_norm_rope_append(
+        _ptr(q3), 0 if q3 is None else q3.stride(0), _ptr(k3), 0 if k3 is None else k3.stride(0),
+        _ptr(ko3), 0 if ko3 is None else ko3.stride(0), _ptr(v3), 0 if v3 is None else v3.stride(0),
+        _ptr(q_weight), _ptr(k_weight), float(eps), _NORM_KINDS[norm], _ptr(ang), a_stride, rot,
+        int(bool(rotary_interleaved)), float(mscale), _ptr(q_positions), _ptr(k_positions),
+        _ptr(k_cache), _ptr(v_cache), sc, st, _ptr(token_to_chunk_idx), _ptr(token_to_local_pos),
+        _ptr(block_table), 0 if block_table is None else block_table.stride(0), _ptr(kv_lens), chunk,
+        T, Hq, Hkv, D, int(bool(faithful_rounding)), _stream(ref)), "mi_norm_rope_append")

@@ -1,0 +1,170 @@
+"""fp32 oracle for paged attention, KV append, LSE merge and fp8 KV storage.
+
+Restates, on CPU tensors:
+* ``key_value_cache`` + block-table addressing: ``K_r[j] = k_cache[block_table[r, j // C], j % C]``
+  (megatron/core/inference/contexts/dynamic_context.py:547-564, 811-825);
+* the unfused core attention the reference documents as its math -- GQA by repeating KV
+  heads, scores scaled by ``d**-0.5``, fp32 softmax, weighted sum of V
+  (megatron/core/transformer/dot_product_attention.py:159-235,
+  megatron/core/fusions/fused_softmax.py:299-342);
+* flash-attn's call contract at megatron/core/transformer/attention.py:546-557,589-600:
+  bottom-right aligned causal mask, kv length includes the token appended this step;
+* ``append_key_value_cache`` (dynamic_context.py:511-545).
+
+Pinned by (tests/test_oracle_attention.py): torch.nn.functional.scaled_dot_product_attention
+on gathered K/V (library routine, incl. an explicit bottom-right mask and GQA), fp64 brute
+force loops on tiny cases, invariance under chunk-id permutation, all-equal-K => mean of V,
+single-key => V itself, split + LSE merge == single pass, zero-length row => zeros.
+fp8: torch's own ``float8_e4m3fn`` cast is the rounding reference.
+"""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor
+
+E4M3_MAX = 448.0
+
+
+def gather_request_kv(cache: Tensor, block_table_row: Tensor, length: int) -> Tensor:
+    """Logical ``[length, Hkv, d]`` view of one request's keys (or values) as fp32."""
+    C = cache.size(1)
+    n_chunks = (length + C - 1) // C
+    ids = block_table_row[:n_chunks].long()
+    flat = cache[ids].reshape(n_chunks * C, cache.size(2), cache.size(3))
+    return flat[:length].float()
+
+
+def attention_one_request(q: Tensor, k: Tensor, v: Tensor, scale: float, causal_shift: Optional[int]) -> Tensor:
+    """``q`` [Lq,Hq,d], ``k``/``v`` [Lk,Hkv,d] fp32 -> [Lq,Hq,d] fp32.
+
+    ``causal_shift`` = Lk - Lq for the bottom-right aligned mask (query i sees keys
+    j <= i + shift); ``None`` disables masking.
+    """
+    Lq, Hq, d = q.shape
+    Lk, Hkv, _ = k.shape
+    G = Hq // Hkv
+    if Lk == 0:
+        return torch.zeros_like(q)
+    # Query head h reads KV head h // G: the same pairing as repeating every KV head G times
+    # (dot_product_attention.py:159-165), written without materialising the copies.
+    qg = q.reshape(Lq, Hkv, G, d)
+    scores = torch.einsum("qhgd,khd->hgqk", qg, k) * scale
+    if causal_shift is not None:
+        qi = torch.arange(Lq).view(Lq, 1)
+        kj = torch.arange(Lk).view(1, Lk)
+        scores = scores.masked_fill(kj > qi + causal_shift, float("-inf"))
+    probs = torch.softmax(scores, dim=-1)
+    probs = torch.nan_to_num(probs, nan=0.0)  # rows with no visible key
+    return torch.einsum("hgqk,khd->qhgd", probs, v).reshape(Lq, Hq, d)
+
+
+def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens: Tensor, block_table: Tensor,
+                           softmax_scale: Optional[float] = None, k_scales: Optional[Tensor] = None,
+                           v_scales: Optional[Tensor] = None) -> Tensor:
+    """Decode: ``q`` [R,Hq,d] (one token per request) -> fp32 [R,Hq,d]."""
+    R, Hq, d = q.shape
+    scale = d ** -0.5 if softmax_scale is None else softmax_scale
+    out = torch.zeros(R, Hq, d, dtype=torch.float32)
+    if k_scales is not None:
+        k_cache = dequantize_fp8(k_cache, k_scales)
+        v_cache = dequantize_fp8(v_cache, v_scales)
+    for r in range(R):
+        L = int(kv_lens[r])
+        if L <= 0:
+            continue
+        k = gather_request_kv(k_cache, block_table[r], L)
+        v = gather_request_kv(v_cache, block_table[r], L)
+        out[r] = attention_one_request(q[r : r + 1].float(), k, v, scale, None)[0]
+    return out
+
+
+def paged_varlen_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
+                           block_table: Tensor, softmax_scale: Optional[float] = None) -> Tensor:
+    """Prefill / mixed: ``q`` [T,Hq,d]; request r owns rows cu_q[r]:cu_q[r+1] and kv_lens[r] keys."""
+    T, Hq, d = q.shape
+    scale = d ** -0.5 if softmax_scale is None else softmax_scale
+    out = torch.zeros(T, Hq, d, dtype=torch.float32)
+    for r in range(cu_seqlens_q.numel() - 1):
+        a, b = int(cu_seqlens_q[r]), int(cu_seqlens_q[r + 1])
+        L = int(kv_lens[r])
+        if b <= a:
+            continue
+        if L <= 0:
+            continue
+        k = gather_request_kv(k_cache, block_table[r], L)
+        v = gather_request_kv(v_cache, block_table[r], L)
+        out[a:b] = attention_one_request(q[a:b].float(), k, v, scale, L - (b - a))
+    return out
+
+
+def kv_append(k_cache: Tensor, v_cache: Tensor, key: Tensor, value: Tensor, chunk_idx: Tensor,
+              local_pos: Tensor) -> None:
+    """In-place scatter ``cache[chunk_idx[t], local_pos[t]] = row[t]`` (token order; last writer wins)."""
+    for t in range(key.size(0)):
+        k_cache[int(chunk_idx[t]), int(local_pos[t])] = key[t]
+        v_cache[int(chunk_idx[t]), int(local_pos[t])] = value[t]
+
+
+def decode_slots(block_table: Tensor, kv_lens: Tensor, chunk: int) -> Tuple[Tensor, Tensor, Tensor]:
+    """(rows, chunk ids, local positions) of the token appended this step for rows with len > 0."""
+    rows = torch.nonzero(kv_lens > 0, as_tuple=True)[0]
+    pos = kv_lens[rows].long() - 1
+    ids = block_table[rows, pos // chunk].long()
+    return rows, ids, pos % chunk
+
+
+def lse_merge(partials: Sequence[Tensor], lses: Sequence[Tensor]) -> Tensor:
+    """o = sum_s e^{lse_s - m} o_s / sum_s e^{lse_s - m}; ``partials[s]`` [..., d], ``lses[s]`` [...]."""
+    lse = torch.stack(list(lses), dim=0).double()
+    o = torch.stack(list(partials), dim=0).double()
+    w = torch.exp(lse - lse.max(dim=0, keepdim=True).values)
+    return ((w.unsqueeze(-1) * o).sum(0) / w.sum(0).unsqueeze(-1)).float()
+
+
+def attention_with_lse(q: Tensor, k: Tensor, v: Tensor, scale: float) -> Tuple[Tensor, Tensor]:
+    """Unmasked single-request attention returning (out [Lq,Hq,d], natural-log LSE [Lq,Hq])."""
+    Lq, Hq, d = q.shape
+    Hkv = k.size(1)
+    qg = q.reshape(Lq, Hkv, Hq // Hkv, d)
+    s = torch.einsum("qhgd,khd->hgqk", qg, k) * scale
+    lse = torch.logsumexp(s, dim=-1)  # [Hkv, G, Lq]
+    out = torch.einsum("hgqk,khd->qhgd", torch.softmax(s, dim=-1), v).reshape(Lq, Hq, d)
+    return out, lse.permute(2, 0, 1).reshape(Lq, Hq)
+
+
+# --------------------------------------------------------------------------------------------
+# fp8 (OCP e4m3fn) KV storage with one fp32 scale per (chunk, KV head)
+# --------------------------------------------------------------------------------------------
+def quantize_chunks_fp8(cache: Tensor) -> Tuple[Tensor, Tensor]:
+    """``cache`` [N,C,Hkv,d] -> (uint8 e4m3fn bytes, fp32 scales [N,Hkv]); scale = amax / 448."""
+    x = cache.float()
+    amax = x.abs().amax(dim=(1, 3))
+    scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
+    y = (x / scale[:, None, :, None]).clamp(-E4M3_MAX, E4M3_MAX)
+    return y.to(torch.float8_e4m3fn).view(torch.uint8), scale
+
+
+def dequantize_fp8(cache_bytes: Tensor, scales: Tensor) -> Tensor:
+    return cache_bytes.view(torch.float8_e4m3fn).float() * scales[:, None, :, None]
+
+
+def quantize_token_fp8(row: Tensor, scale: Tensor) -> Tensor:
+    """``row`` [Hkv,d], ``scale`` [Hkv] -> uint8 e4m3fn bytes (saturating)."""
+    y = (row.float() / scale[:, None]).clamp(-E4M3_MAX, E4M3_MAX)
+    return y.to(torch.float8_e4m3fn).view(torch.uint8)
+
+
+def decode_attention_bytes(kv_lens: Sequence[int], Hq: int, Hkv: int, d: int, chunk: int, kv_bytes: int = 2,
+                           fp8_scales: bool = False) -> int:
+    """Algorithmic HBM bytes of one decode-attention call (KV once, q in, out, table, lengths)."""
+    lens = [int(x) for x in kv_lens]
+    total = sum(lens) * Hkv * d * 2 * kv_bytes
+    total += len(lens) * Hq * d * (2 + 2)
+    chunks = sum((l + chunk - 1) // chunk for l in lens)
+    total += chunks * 4 + len(lens) * 4
+    if fp8_scales:
+        total += chunks * Hkv * 2 * 4
+    return total

@@ -1,0 +1,105 @@
+"""GPU parity: fused head norm + rotary embedding (+ append) against the op-by-op CPU chain.
+
+Floating point: bf16 results within 2e-2 abs/rel of the fp32 formula; in the faithful
+rounding mode the kernel reproduces the bf16 op chain up to the last-place effects of
+cos/sin/rsqrt implementations (at most 2 bf16 ulps on a tiny fraction of elements).
+"""
+import pytest
+import torch
+
+from oracle import paged_attention as oa
+from oracle import rope_norm as orn
+
+pytestmark = pytest.mark.gpu
+
+
+def _ulp_diff(a, b):
+    a = a.view(torch.int16).to(torch.int32)
+    b = b.view(torch.int16).to(torch.int32)
+    # map sign-magnitude bf16 bit patterns to a monotone integer line
+    a = torch.where(a < 0, -(a & 0x7FFF), a)
+    b = torch.where(b < 0, -(b & 0x7FFF), b)
+    return (a - b).abs()
+
+
+@pytest.mark.parametrize("norm", [None, "rms", "l2"])
+@pytest.mark.parametrize("interleaved", [False, True])
+@pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64)])
+def test_norm_rope_matches_unfused_chain(mi, dev, norm, interleaved, d, rot):
+    gen = torch.Generator().manual_seed(d + rot + (7 if interleaved else 0))
+    T, Hq, Hkv = 37, 8, 2
+    q = torch.randn(T, 1, Hq, d, generator=gen).bfloat16()
+    k = torch.randn(T, 1, Hkv, d, generator=gen).bfloat16()
+    qw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16()
+    kw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16()
+    table = orn.rotary_table(9000, rot, base=500000.0, interleaved=interleaved)
+    qpos = torch.randint(0, 9000, (T,), generator=gen)
+    kpos = torch.randint(0, 9000, (T,), generator=gen)
+    eps = 1e-5 if norm == "rms" else 1e-6
+    q_ref = orn.norm_rope(q.squeeze(1), qpos, table, norm=norm, weight=qw if norm == "rms" else None, eps=eps,
+                          interleaved=interleaved)
+    k_ref = orn.norm_rope(k.squeeze(1), kpos, table, norm=norm, weight=kw if norm == "rms" else None, eps=eps,
+                          interleaved=interleaved)
+    for faithful in (True, False):
+        qd, kd = q.to(dev).clone(), k.to(dev)
+        k_out = torch.empty_like(kd)
+        mi.ops.norm_rope_append(qd, kd, key_out=k_out, q_weight=qw.to(dev), k_weight=kw.to(dev), eps=eps, norm=norm,
+                                rotary_emb=table.to(dev), q_positions=qpos.to(dev), k_positions=kpos.to(dev),
+                                rotary_interleaved=interleaved, faithful_rounding=faithful)
+        torch.cuda.synchronize()
+        for got, ref in ((qd.cpu().squeeze(1), q_ref), (k_out.cpu().squeeze(1), k_ref)):
+            err = (got.float() - ref.float()).abs()
+            assert (err <= 2e-2 + 2e-2 * ref.float().abs()).all(), f"max err {err.max().item()}"
+            if faithful:
+                ulps = _ulp_diff(got, ref)
+                assert ulps.max().item() <= 2
+                assert (ulps > 0).float().mean().item() < 0.01
+        assert torch.equal(kd.cpu(), k), "the key input must not be modified"
+
+
+def test_position_zero_is_identity_and_passthrough_tail(mi, dev):
+    T, H, d, rot = 5, 4, 128, 64
+    x = torch.randn(T, 1, H, d).bfloat16().to(dev)
+    table = orn.rotary_table(16, rot).to(dev)
+    y = x.clone()
+    pos = torch.zeros(T, dtype=torch.int64, device=dev)
+    mi.ops.norm_rope_append(y, None, rotary_emb=table, q_positions=pos)
+    torch.cuda.synchronize()
+    assert torch.equal(x, y)
+    pos = torch.arange(T, dtype=torch.int64, device=dev) + 3
+    mi.ops.norm_rope_append(y, None, rotary_emb=table, q_positions=pos)
+    torch.cuda.synchronize()
+    assert torch.equal(x[..., rot:], y[..., rot:]) and not torch.equal(x[..., :rot], y[..., :rot])
+
+
+@pytest.mark.parametrize("mode", ["token_rows", "block_table"])
+def test_fused_append_writes_rotated_key_and_raw_value(mi, dev, mode):
+    lens = torch.tensor([5, 256, 257, 1000, 0, 31], dtype=torch.int32)
+    cfg = mi.synthetic.DecodeConfig("fa", lens.numel(), 32, 8, 128, 0, 0, seed=4)
+    case = mi.synthetic.make_decode_case(cfg, dev, lens=lens)
+    kc0, vc0 = case.k_cache.cpu().clone(), case.v_cache.cpu().clone()
+    table = orn.rotary_table(2048, 128, base=500000.0)
+    pos = (lens.long() - 1).clamp(min=0)
+    w = (1 + 0.02 * torch.randn(128)).bfloat16()
+    q = case.q.clone()
+    k_out = torch.empty_like(case.k_new)
+    rows, ids, loc = oa.decode_slots(case.block_table.cpu(), lens, cfg.chunk)
+    kwargs = {}
+    if mode == "token_rows":
+        ci = torch.full((lens.numel(),), case.k_cache.size(0) - 1, dtype=torch.int64)
+        lo = torch.zeros(lens.numel(), dtype=torch.int64)
+        ci[rows], lo[rows] = ids, loc
+        kwargs = dict(token_to_chunk_idx=ci.to(dev), token_to_local_pos=lo.to(dev))
+    else:
+        kwargs = dict(block_table=case.block_table, kv_lens=case.kv_lens)
+    mi.ops.norm_rope_append(q, case.k_new, value=case.v_new, key_out=k_out, q_weight=w.to(dev), k_weight=w.to(dev),
+                            norm="rms", eps=1e-5, rotary_emb=table.to(dev), q_positions=pos.to(dev),
+                            k_positions=pos.to(dev), k_cache=case.k_cache, v_cache=case.v_cache, **kwargs)
+    torch.cuda.synchronize()
+    # append is bit-exact given the rotated key the kernel itself produced
+    oa.kv_append(kc0, vc0, k_out.cpu().squeeze(1)[rows], case.v_new.cpu().squeeze(1)[rows], ids, loc)
+    dummy = case.k_cache.size(0) - 1
+    assert torch.equal(case.k_cache.cpu()[:dummy], kc0[:dummy])
+    assert torch.equal(case.v_cache.cpu()[:dummy], vc0[:dummy])
+    k_ref = orn.norm_rope(case.k_new.cpu().squeeze(1), pos, table, norm="rms", weight=w, eps=1e-5)
+    assert (k_out.cpu().squeeze(1).float() - k_ref.float()).abs().max().item() <= 4e-2
