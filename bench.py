@@ -190,7 +190,7 @@ def main():
         "decode_steps_per_sec": round(1e3 / ms_per_step, 1),
         "roofline": {
             "bound": "hbm",
-            "kernel": "paged_decode_split_kernel",
+            "kernel": "paged_decode_stream_kernel",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

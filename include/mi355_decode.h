@@ -47,7 +47,8 @@ int mi_version(void);
 /* Message of the calling thread's most recent rejected call ("" if none). */
 const char* mi_last_error(void);
 
-/* Experiment knobs ("decode_tile_subtiles" = 1|2|4, "prefill_tile_subtiles"). */
+/* Experiment knobs: "decode_tile_subtiles" (1|2), "decode_min_waves" (3|4), "decode_wgs_per_cu",
+ * "decode_grid" (0 = automatic), "decode_waves_per_block", "prefill_tile_subtiles". */
 int mi_set_tuning(const char* name, int32_t value);
 
 /*
@@ -108,8 +109,8 @@ int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_bf16, int64_
                             float headroom, void* stream);
 
 /*
- * Bytes of fp32 workspace mi_paged_decode_attention needs for these sizes
- * (`split_tokens` = 0 lets the library choose, as the attention call will).
+ * Bytes of workspace mi_paged_decode_attention needs for these sizes on the current
+ * device (partials of the workgroups that share a request + per-request bookkeeping).
  */
 int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                   int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens);
@@ -122,8 +123,9 @@ int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t he
  *   out[r,h] = softmax(q[r,h] . K_r[:len_r, h/G]^T * softmax_scale) . V_r[:len_r, h/G]
  *   K_r[j] = k_cache[block_table[r, j / chunk_tokens], j % chunk_tokens], G = Hq/Hkv.
  * q/out: bf16 `[R, Hq, d]` with the given token / head strides.  kv_lens int32 [R]
- * (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] and sizes
- * the grid (the reference passes max_sequence_length here, dynamic_context.py:791).
+ * (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] (the reference
+ * passes max_sequence_length here, dynamic_context.py:791); the grid does not depend on
+ * it.  `split_tokens` = minimum tokens one workgroup streams (0 = default 256).
  * kv_dtype MI_KV_FP8_E4M3 reads byte caches with k_scales/v_scales `[n_chunks, Hkv]`.
  */
 int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_head,

@@ -26,6 +26,7 @@ HIPCC_FLAGS = [
     # packed fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    "-DMI_NT_LOADS",
 ]
 
 

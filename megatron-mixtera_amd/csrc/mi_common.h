@@ -80,6 +80,25 @@ static __device__ __forceinline__ float xor32(float x) { return __shfl_xor(x, 32
 // 16-byte global loads / stores through plain pointers.
 static __device__ __forceinline__ uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 static __device__ __forceinline__ uint2 ld8(const void* p) { return *reinterpret_cast<const uint2*>(p); }
+// Streaming variants: the data is read exactly once, so it is marked non-temporal.
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+static __device__ __forceinline__ uint4 ld16_stream(const void* p) {
+#ifdef MI_NT_LOADS
+  const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+#else
+  return ld16(p);
+#endif
+}
+static __device__ __forceinline__ uint2 ld8_stream(const void* p) {
+#ifdef MI_NT_LOADS
+  const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
+  return make_uint2(v.x, v.y);
+#else
+  return ld8(p);
+#endif
+}
 static __device__ __forceinline__ void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
 static __device__ __forceinline__ void st8(void* p, uint2 v) { *reinterpret_cast<uint2*>(p) = v; }
 

@@ -6,9 +6,15 @@
 // attends to the request's tokens scattered over fixed-size chunks of a
 // `[n_chunks, chunk, Hkv, d]` cache, addressed through a `[R, M]` block table.
 //
-// Work decomposition
-//   grid = (splits, R, Hkv / waves_per_block); one wavefront owns one
-//   (request, KV head, split) item and streams `split` tokens of K and V once.
+// Work decomposition ("flattened stream")
+//   Every request is cut into tiles of 16*NT tokens and the tiles of all requests are
+//   laid end to end.  A fixed grid of workgroups (a small multiple of the CU count)
+//   divides that sequence into equal contiguous spans, so every workgroup streams the
+//   same number of bytes whatever the mix of context lengths, and pays its start-up cost
+//   once.  A span that crosses a request boundary yields one segment per request; a
+//   segment that is a whole request writes bf16 output directly, any other segment
+//   writes a normalised fp32 partial + base-2 LSE into slot (workgroup index + request
+//   index), which is unique because both indices only grow along the sequence.
 //   The waves of a workgroup take neighbouring KV heads of the SAME tokens, so a
 //   workgroup as a whole reads each token's `Hkv*d` row contiguously.
 //
@@ -25,9 +31,9 @@
 //   Softmax statistics are per query row = per m16, so only the running max
 //   needs a cross-lane step (two exchanges across g).
 //
-// A split that is the only one of its request writes bf16 output directly; else
-// it writes a normalised fp32 partial and a base-2 LSE, merged by a second
-// kernel: o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max).
+// A second kernel merges the partials of each request,
+//   o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max),
+// and writes zeros for zero-length (padded) rows.
 #include "mi_common.h"
 #include "mi_capi_internal.h"
 
@@ -45,47 +51,33 @@ struct DecodeParams {
   const int32_t* lens;
   uint16_t* out;
   int64_t o_st, o_sh;
-  float* part_o;    // [R][Hq][max_splits][HD]
-  float* part_lse;  // [R][Hq][max_splits]
+  float* part_o;     // [slots][Hq][HD], slots = grid + R
+  float* part_lse;   // [slots][Hq]
+  int32_t* seg_info;  // [R][2]: first and last workgroup that touched request r
   const float* k_scale;  // fp8 only: [n_chunks][Hkv]
   const float* v_scale;
-  int32_t R, Hq, Hkv, G, chunk, chunk_shift, split, max_splits;
+  uint64_t chunk_magic;  // ceil(2^40 / chunk)
+  int32_t R, Hq, Hkv, G, chunk, min_span_tiles, grid;
   float scale_log2;
 };
 
-static __device__ __forceinline__ int chunk_of(int tok, int chunk, int shift) {
-  return shift >= 0 ? (tok >> shift) : (tok / chunk);
+// tok / chunk for 0 <= tok < 2^31 via a 40-bit reciprocal (exact while tok * chunk < 2^40).
+static __device__ __forceinline__ int chunk_of(int tok, uint64_t magic) {
+  return (int)(((uint64_t)(uint32_t)tok * magic) >> 40);
 }
 
+// One segment: tokens [start, end) of request r for KV head h (one wavefront).
+// `whole` = the segment is the entire request (write bf16 output, no partial).
 template <int HD, int NT, bool FP8>
-__global__ __launch_bounds__(512) void paged_decode_split_kernel(DecodeParams p) {
+static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int h, int len, int start,
+                                                      int end, bool whole, int slot, int lane) {
   constexpr int KS = HD / 32;
   constexpr int DV = HD / 16;
   static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
   constexpr int ESZ = FP8 ? 1 : 2;
-
-  const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
   const int m16 = lane & 15, g = lane >> 4;
-  const int s = blockIdx.x;
-  const int r = blockIdx.y;
-  const int h = __builtin_amdgcn_readfirstlane(blockIdx.z * (blockDim.x >> 6) + wave);
   const int G = p.G;
   const int hq = h * G + m16;  // query head of this lane's row (valid when m16 < G)
-
-  const int len = p.lens[r];
-  const int start = s * p.split;
-  if (len <= 0) {
-    // Padded batch rows carry kv-len 0: their output is defined as zeros.
-    if (s == 0 && m16 < G) {
-      uint16_t* o = p.out + (int64_t)r * p.o_st + (int64_t)hq * p.o_sh + (HD / 4) * g;
-      for (int i = 0; i < HD / 4; i += 8) st16(o + i, make_uint4(0, 0, 0, 0));
-    }
-    return;
-  }
-  if (start >= len) return;
-  const int end = min(start + p.split, len);
-  const int nsplit = (len + p.split - 1) / p.split;
   const int last = len - 1;
 
   // Query fragments: B operand rows are the G heads of this KV head.
@@ -112,45 +104,61 @@ __global__ __launch_bounds__(512) void paged_decode_split_kernel(DecodeParams p)
 #pragma unroll
   for (int e = 0; e < DV; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  for (int T = start; T < end; T += 16 * NT) {
-    // ---- issue every load of this tile first -------------------------------
-    uint4 kf[NT][FP8 ? KS / 2 : KS];
-    uint4 vf16[NT][4];  // bf16, HD=128 : 16 B per token
-    uint2 vf8[NT][4];   // bf16 HD=64 or fp8 HD=128 : 8 B per token
-    float ksc[NT], vsc[NT];
+  // Register staging of one tile (NT sub-tiles of 16 tokens).  The loop below is software
+  // pipelined with these registers alone: K of the next tile is requested as soon as the
+  // scores of the current one exist, V of the next tile as soon as the current P.V is done,
+  // so every wave keeps loads in flight while it computes.
+  uint4 kf[NT][FP8 ? KS / 2 : KS];
+  uint4 vf16[NT][4];  // bf16, HD=128 : 16 B per token
+  uint2 vf8[NT][4];   // bf16 HD=64 or fp8 HD=128 : 8 B per token
+  float ksc[NT], vsc[NT];
+
+  // Tokens past the end are clamped to the last valid one: the data stays finite and
+  // their probabilities are forced to zero below.  That also makes a request for a tile
+  // beyond `end` harmless (it re-reads the last token's rows).
+  auto load_k = [&](int T) {
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       const int T0 = T + 16 * u;
       const int tu = min(T0, last);  // wave-uniform
-      const int ci = chunk_of(tu, p.chunk, p.chunk_shift);
+      const int ci = chunk_of(tu, p.chunk_magic);
       const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
-      const int cbase = ci * p.chunk;
       const uint8_t* kc = kbase + (int64_t)pc * chunk_bytes;
-      const uint8_t* vc = vbase + (int64_t)pc * chunk_bytes;
-      if (FP8) {
-        ksc[u] = p.k_scale[(int64_t)pc * p.Hkv + h];
-        vsc[u] = p.v_scale[(int64_t)pc * p.Hkv + h];
-      }
-      // Tokens past the end are clamped to the last valid one: the data stays
-      // finite and their probabilities are forced to zero below.
-      const int tk = min(T0 + m16, last) - cbase;
+      if (FP8) ksc[u] = p.k_scale[(int64_t)pc * p.Hkv + h];
+      const int tk = min(T0 + m16, last) - ci * p.chunk;
       const uint8_t* krow = kc + tk * tok_bytes;
       if (FP8) {
 #pragma unroll
-        for (int kk = 0; kk < KS / 2; ++kk) kf[u][kk] = ld16(krow + 64 * kk + 16 * g);
+        for (int kk = 0; kk < KS / 2; ++kk) kf[u][kk] = ld16_stream(krow + 64 * kk + 16 * g);
       } else {
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk) kf[u][kk] = ld16(krow + (32 * kk + 8 * g) * 2);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int tv = min(T0 + 4 * g + j, last) - cbase;
-        const uint8_t* vrow = vc + tv * tok_bytes + DV * m16 * ESZ;
-        if (!FP8 && HD == 128) vf16[u][j] = ld16(vrow);
-        else vf8[u][j] = ld8(vrow);
+        for (int kk = 0; kk < KS; ++kk) kf[u][kk] = ld16_stream(krow + (32 * kk + 8 * g) * 2);
       }
     }
+  };
+  auto load_v = [&](int T) {
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      const int T0 = T + 16 * u;
+      const int tu = min(T0, last);
+      const int ci = chunk_of(tu, p.chunk_magic);
+      const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
+      const uint8_t* vc = vbase + (int64_t)pc * chunk_bytes;
+      if (FP8) vsc[u] = p.v_scale[(int64_t)pc * p.Hkv + h];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int tv = min(T0 + 4 * g + j, last) - ci * p.chunk;
+        const uint8_t* vrow = vc + tv * tok_bytes + DV * m16 * ESZ;
+        if (!FP8 && HD == 128) vf16[u][j] = ld16_stream(vrow);
+        else vf8[u][j] = ld8_stream(vrow);
+      }
+    }
+  };
 
+  load_k(start);
+  load_v(start);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int T = start; T < end; T += 16 * NT) {
     // ---- S^T = K Q^T ---------------------------------------------------------
     float sc[NT][4];
     float tmax = -INFINITY;
@@ -178,6 +186,14 @@ __global__ __launch_bounds__(512) void paged_decode_split_kernel(DecodeParams p)
         tmax = fmaxf(tmax, v);
       }
     }
+    float vmul[NT];
+#pragma unroll
+    for (int u = 0; u < NT; ++u) vmul[u] = FP8 ? vsc[u] : 1.f;
+    // The scheduling fences keep each batch of prefetch loads together at this point of the
+    // loop instead of letting the compiler sink them next to their uses one by one.
+    __builtin_amdgcn_sched_barrier(0);
+    load_k(T + 16 * NT);  // prefetch: the K registers are free again
+    __builtin_amdgcn_sched_barrier(0);
     tmax = fmaxf(tmax, xor16(tmax));
     tmax = fmaxf(tmax, xor32(tmax));
 
@@ -197,7 +213,7 @@ __global__ __launch_bounds__(512) void paged_decode_split_kernel(DecodeParams p)
       }
       if (FP8) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) pv[i] *= vsc[u];
+        for (int i = 0; i < 4; ++i) pv[i] *= vmul[u];
       }
       pf[u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
     }
@@ -248,15 +264,18 @@ __global__ __launch_bounds__(512) void paged_decode_split_kernel(DecodeParams p)
         }
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
+    load_v(T + 16 * NT);  // prefetch: the V registers are free again
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- epilogue ---------------------------------------------------------------
   float l_tot = l_run + xor16(l_run);
   l_tot += xor32(l_tot);
   const float inv = 1.f / l_tot;
-  if (m16 >= G) return;
+  if (m16 >= G) return;  // (no barrier follows inside a segment)
   // acc[e][i] holds d = DV*(4g+i) + e: DV*4 contiguous values per lane.
-  if (nsplit == 1) {
+  if (whole) {
     uint16_t* o = p.out + (int64_t)r * p.o_st + (int64_t)hq * p.o_sh + 4 * DV * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -271,7 +290,7 @@ __global__ __launch_bounds__(512) void paged_decode_split_kernel(DecodeParams p)
       }
     }
   } else {
-    const int64_t row = ((int64_t)r * p.Hq + hq) * p.max_splits + s;
+    const int64_t row = (int64_t)slot * p.Hq + hq;
     float* o = p.part_o + row * HD + 4 * DV * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -285,50 +304,122 @@ __global__ __launch_bounds__(512) void paged_decode_split_kernel(DecodeParams p)
   }
 }
 
-// One workgroup per (request, query head): merge the split partials.
+// Tiles (of TK tokens) of one request.
+static __device__ __forceinline__ int tiles_of(int len, int tk) { return len > 0 ? (len + tk - 1) / tk : 0; }
+
+template <int HD, int NT, bool FP8, int MINW>
+__global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
+  constexpr int TK = 16 * NT;
+  extern __shared__ int cum[];  // inclusive prefix sum of tiles per request, [R]
+
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x >> 6) + wave);
+
+  // ---- prefix sum of tiles over the batch (wave 0), shared through LDS -------------
+  if (wave == 0) {
+    int carry = 0;
+    for (int base = 0; base < p.R; base += 64) {
+      const int i = base + lane;
+      int v = i < p.R ? tiles_of(p.lens[i], TK) : 0;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(v, o, 64);
+        if (lane >= o) v += up;
+      }
+      if (i < p.R) cum[i] = carry + v;
+      carry += __shfl(v, 63, 64);
+    }
+  }
+  __syncthreads();
+  const int total = cum[p.R - 1];
+  const int per = max((total + p.grid - 1) / p.grid, p.min_span_tiles);
+  int t0 = blockIdx.x * per;
+  const int t1 = min(t0 + per, total);
+  if (t0 >= t1) return;
+
+  // first request whose tiles extend beyond t0
+  int lo = 0, hi = p.R - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi) >> 1;
+    if (cum[mid] > t0) hi = mid; else lo = mid + 1;
+  }
+  int r = lo;
+  while (t0 < t1) {
+    const int rb = r ? cum[r - 1] : 0;
+    const int re = cum[r];
+    if (re > t0) {  // requests without tiles (length 0) are skipped
+      const int len = p.lens[r];
+      const int tb = t0 - rb;             // first tile of the segment, within the request
+      const int te = min(t1, re) - rb;    // one past its last tile
+      const bool first = tb == 0, final = te == re - rb;
+      if (wave == 0 && lane == 0) {
+        if (first) p.seg_info[2 * r] = blockIdx.x;
+        if (final) p.seg_info[2 * r + 1] = blockIdx.x;
+      }
+      decode_segment<HD, NT, FP8>(p, r, h, len, tb * TK, min(te * TK, len), first && final,
+                                  (int)blockIdx.x + r, lane);
+      t0 = rb + te;
+    }
+    ++r;
+  }
+}
+
+// One workgroup per (request, query head): merge the partials of the workgroups that
+// shared the request; zero-length rows get zeros.
 template <int HD>
 __global__ __launch_bounds__(HD) void paged_decode_merge_kernel(DecodeParams p) {
   const int r = blockIdx.y, hq = blockIdx.x, d = threadIdx.x;
-  const int len = p.lens[r];
-  if (len <= 0) return;
-  const int nsplit = (len + p.split - 1) / p.split;
-  if (nsplit <= 1) return;
-  const int64_t row0 = ((int64_t)r * p.Hq + hq) * p.max_splits;
-  const float* lse = p.part_lse + row0;
-  const float* po = p.part_o + row0 * HD + d;
+  uint16_t* o = p.out + (int64_t)r * p.o_st + (int64_t)hq * p.o_sh + d;
+  if (p.lens[r] <= 0) {
+    *o = 0;
+    return;
+  }
+  const int first = p.seg_info[2 * r], last = p.seg_info[2 * r + 1];
+  if (first == last) return;  // written directly by the streaming kernel
   float mx = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) mx = fmaxf(mx, lse[s]);
+  for (int w = first; w <= last; ++w) mx = fmaxf(mx, p.part_lse[(int64_t)(w + r) * p.Hq + hq]);
   float num = 0.f, den = 0.f;
 #pragma unroll 4
-  for (int s = 0; s < nsplit; ++s) {
-    const float w = fast_exp2(lse[s] - mx);
-    num += w * po[(int64_t)s * HD];
-    den += w;
+  for (int w = first; w <= last; ++w) {
+    const int64_t row = (int64_t)(w + r) * p.Hq + hq;
+    const float wt = fast_exp2(p.part_lse[row] - mx);
+    num += wt * p.part_o[row * HD + d];
+    den += wt;
   }
-  p.out[(int64_t)r * p.o_st + (int64_t)hq * p.o_sh + d] = f32_to_bf16(num / den);
+  *o = f32_to_bf16(num / den);
 }
 
 static int pick_waves_per_block(int Hkv) {
-  for (int w = 8; w >= 1; --w)
+  int cap = mi_tuning().decode_waves_per_block;
+  if (cap < 1 || cap > 8) cap = 8;
+  for (int w = cap; w >= 1; --w)
     if (Hkv % w == 0) return w;
   return 1;
 }
 
-static int log2_exact(int x) {
-  if (x <= 0 || (x & (x - 1))) return -1;
-  int s = 0;
-  while ((1 << s) < x) ++s;
-  return s;
+static int device_cu_count() {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (!cus[dev]) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev] = n;
+  }
+  return cus[dev];
 }
 
-int resolve_split_tokens(int R, int Hkv, int chunk, int max_kv_len, int split_tokens) {
-  if (split_tokens > 0) return split_tokens;
-  int wpb = pick_waves_per_block(Hkv);
-  int split = chunk >= 256 ? 256 : chunk;
-  if (chunk > 256 && chunk % 256) split = chunk;
-  // Keep the grid (mostly early-exit workgroups when lengths are ragged) bounded.
-  while ((int64_t)R * (Hkv / wpb) * ((max_kv_len + split - 1) / split) > 16384 && split < 8192) split *= 2;
-  return split;
+// Workgroups along the flattened tile sequence: enough to put `decode_wgs_per_cu`
+// workgroups of 8 waves (or the equivalent in smaller workgroups) on every CU.
+int decode_grid_size(int Hkv) {
+  const int forced = mi_tuning().decode_grid;
+  if (forced > 0) return forced;
+  const int wpb = pick_waves_per_block(Hkv);
+  const int head_groups = Hkv / wpb;
+  int per_cu = mi_tuning().decode_wgs_per_cu * (8 / wpb);
+  int grid = device_cu_count() * per_cu / head_groups;
+  return grid < 1 ? 1 : grid;
 }
 
 }  // namespace mi
@@ -338,10 +429,10 @@ using namespace mi;
 extern "C" int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                              int32_t chunk_tokens, int32_t max_kv_len,
                                              int32_t split_tokens) {
-  if (R <= 0 || Hq <= 0 || Hkv <= 0 || head_dim <= 0 || chunk_tokens <= 0 || max_kv_len <= 0) return 0;
-  const int split = resolve_split_tokens(R, Hkv, chunk_tokens, max_kv_len, split_tokens);
-  const int64_t ms = (max_kv_len + split - 1) / split;
-  return (int64_t)R * Hq * ms * (head_dim + 1) * (int64_t)sizeof(float);
+  (void)chunk_tokens; (void)max_kv_len; (void)split_tokens;
+  if (R <= 0 || Hq <= 0 || Hkv <= 0 || head_dim <= 0) return 0;
+  const int64_t slots = (int64_t)decode_grid_size(Hkv) + R;
+  return slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
 
 extern "C" int mi_paged_decode_attention(
@@ -352,6 +443,7 @@ extern "C" int mi_paged_decode_attention(
     int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len,
     int32_t split_tokens, float softmax_scale, int32_t kv_dtype, const float* k_scales,
     const float* v_scales, void* stream) {
+  (void)max_kv_len;
   if (R == 0) return MI_OK;
   if (!q || !k_cache || !v_cache || !block_table || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_decode_attention: null pointer argument");
@@ -375,16 +467,23 @@ extern "C" int mi_paged_decode_attention(
     return mi_fail(MI_ERR_ALIGN, "mi_paged_decode_attention: strides must keep rows 16-byte aligned");
   if (kv_stride_tok * (int64_t)chunk_tokens * esz >= (int64_t)1 << 31)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: one chunk must span less than 2 GiB");
-  if (max_kv_len <= 0) return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: max_kv_len must be positive");
+  if (split_tokens < 0 || split_tokens % 16)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: split_tokens must be a non-negative multiple of 16");
+  if ((int64_t)R * sizeof(int32_t) > 60 * 1024)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: batch too large for the in-LDS prefix sum");
 
-  const int split = resolve_split_tokens(R, Hkv, chunk_tokens, max_kv_len, split_tokens);
-  if (split % 16) return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: split_tokens must be a multiple of 16");
-  const int max_splits = (max_kv_len + split - 1) / split;
-  const int64_t need = (int64_t)R * Hq * max_splits * (head_dim + 1) * (int64_t)sizeof(float);
-  if (max_splits > 1 && (!workspace || workspace_bytes < need))
+  const int grid_x = decode_grid_size(Hkv);
+  const int64_t slots = (int64_t)grid_x + R;
+  const int64_t need = slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
+  if (!workspace || workspace_bytes < need)
     return mi_fail(MI_ERR_WORKSPACE, "mi_paged_decode_attention: workspace too small (see mi_decode_workspace_bytes)");
-  if (max_splits > 1 && ((uintptr_t)workspace & 15))
+  if ((uintptr_t)workspace & 15)
     return mi_fail(MI_ERR_ALIGN, "mi_paged_decode_attention: workspace must be 16-byte aligned");
+
+  const int nt = mi_tuning().decode_tile_subtiles == 1 ? 1 : 2;
+  const int minw = mi_tuning().decode_min_waves;
+  const int tk = 16 * nt;
+  const int min_span_tokens = split_tokens > 0 ? split_tokens : 256;
 
   DecodeParams p;
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
@@ -393,37 +492,36 @@ extern "C" int mi_paged_decode_attention(
   p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens;
   p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
   p.part_o = (float*)workspace;
-  p.part_lse = p.part_o ? p.part_o + (int64_t)R * Hq * max_splits * head_dim : nullptr;
+  p.part_lse = p.part_o + slots * Hq * head_dim;
+  p.seg_info = (int32_t*)(p.part_lse + slots * Hq);
   p.k_scale = k_scales; p.v_scale = v_scales;
   p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G; p.chunk = chunk_tokens;
-  p.chunk_shift = log2_exact(chunk_tokens); p.split = split; p.max_splits = max_splits;
+  p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
+  p.min_span_tiles = (min_span_tokens + tk - 1) / tk;
+  p.grid = grid_x;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
 
   const int wpb = pick_waves_per_block(Hkv);
-  dim3 grid(max_splits, R, Hkv / wpb), block(64 * wpb);
+  dim3 grid(grid_x, Hkv / wpb), block(64 * wpb);
+  const size_t lds = (size_t)R * sizeof(int32_t);
   hipStream_t st = (hipStream_t)stream;
-  const int nt = mi_tuning().decode_tile_subtiles;
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
   if (timed) hipEventRecord(ev_a, st);
-  if (kv_dtype == MI_KV_FP8_E4M3) {
-    if (nt == 1) hipLaunchKernelGGL((paged_decode_split_kernel<128, 1, true>), grid, block, 0, st, p);
-    else if (nt == 4) hipLaunchKernelGGL((paged_decode_split_kernel<128, 4, true>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((paged_decode_split_kernel<128, 2, true>), grid, block, 0, st, p);
-  } else if (head_dim == 128) {
-    if (nt == 1) hipLaunchKernelGGL((paged_decode_split_kernel<128, 1, false>), grid, block, 0, st, p);
-    else if (nt == 4) hipLaunchKernelGGL((paged_decode_split_kernel<128, 4, false>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((paged_decode_split_kernel<128, 2, false>), grid, block, 0, st, p);
-  } else {
-    if (nt == 1) hipLaunchKernelGGL((paged_decode_split_kernel<64, 1, false>), grid, block, 0, st, p);
-    else if (nt == 4) hipLaunchKernelGGL((paged_decode_split_kernel<64, 4, false>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((paged_decode_split_kernel<64, 2, false>), grid, block, 0, st, p);
-  }
+#define MI_LAUNCH_DECODE(HD_, FP8_)                                                                             \
+  do {                                                                                                          \
+    if (nt == 1 && minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 4>), grid, block, lds, st, p); \
+    else if (nt == 1) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 3>), grid, block, lds, st, p);       \
+    else if (minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 4>), grid, block, lds, st, p);     \
+    else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 3>), grid, block, lds, st, p);                    \
+  } while (0)
+  if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true);
+  else if (head_dim == 128) MI_LAUNCH_DECODE(128, false);
+  else MI_LAUNCH_DECODE(64, false);
+#undef MI_LAUNCH_DECODE
   if (timed) hipEventRecord(ev_b, st);
-  if (max_splits > 1) {
-    dim3 mgrid(Hq, R);
-    if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p);
-    else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p);
-  }
+  dim3 mgrid(Hq, R);
+  if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p);
+  else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p);
   return mi_check_launch("mi_paged_decode_attention");
 }

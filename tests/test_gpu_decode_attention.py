@@ -52,21 +52,25 @@ def test_head_grouping(mi, dev, Hq, Hkv, d):
 
 
 @pytest.mark.parametrize("chunk", [16, 48, 128, 256])
-@pytest.mark.parametrize("subtiles", [1, 2, 4])
-def test_ragged_lengths_and_edges(mi, dev, chunk, subtiles):
-    """Lengths around every tile / chunk boundary, plus zero-length (padded) rows."""
+@pytest.mark.parametrize("subtiles", [1, 2])
+@pytest.mark.parametrize("grid", [0, 1, 7, 4096])
+def test_ragged_lengths_and_edges(mi, dev, chunk, subtiles, grid):
+    """Lengths around every tile / chunk boundary, plus zero-length (padded) rows, for several
+    ways of cutting the flattened tile sequence into workgroup spans (grid 0 = the default)."""
     lens = torch.tensor([0, 1, 2, 15, 16, 17, 31, 32, 33, chunk - 1, chunk, chunk + 1, 2 * chunk, 3 * chunk + 5, 0, 777],
                         dtype=torch.int32)
     cfg = mi.synthetic.DecodeConfig("edges", lens.numel(), 8, 2, 128, 0, 0, chunk=chunk, seed=chunk + subtiles)
     case = mi.synthetic.make_decode_case(cfg, dev, lens=lens)
     mi.ops.set_tuning("decode_tile_subtiles", subtiles)
+    mi.ops.set_tuning("decode_grid", grid)
     try:
-        for split in (0, 16, 64, chunk * 2):
+        for split in (0, 16, 64, 512):  # minimum tokens per workgroup span
             out = _run_case(mi, case, split_tokens=split, max_kv_len=int(lens.max()))
             _close(out, _ref(case), 2e-2)
-            assert (out[case.kv_lens.cpu() == 0] == 0).all(), "zero-length rows must be zeros"
+            assert (out[case.kv_lens == 0] == 0).all(), "zero-length rows must be zeros"
     finally:
         mi.ops.set_tuning("decode_tile_subtiles", 2)
+        mi.ops.set_tuning("decode_grid", 0)
 
 
 def test_block_table_width_and_padding_rows(mi, dev):
@@ -113,12 +117,16 @@ def test_all_equal_keys_give_mean_of_values(mi, dev):
 
 
 def test_split_invariance_cfg2_full_size(mi, dev):
-    """Full Llama-3-8B batch-64 size: different split sizes agree with each other (merge == single pass)."""
+    """Full Llama-3-8B batch-64 size: different span sizes agree with each other (merge == single pass)."""
     case = mi.synthetic.make_decode_case(mi.synthetic.CONFIGS["cfg2"], dev, on_device_rng=True)
     mx = int(case.kv_lens.max())
-    base = _run_case(mi, case, split_tokens=256, max_kv_len=mx).float()
-    for split in (512, 2048, 8192):
-        other = _run_case(mi, case, split_tokens=split, max_kv_len=mx).float()
+    base = _run_case(mi, case, max_kv_len=mx).float()
+    for split, grid in ((512, 4096), (2048, 0), (8192, 0), (1 << 20, 0)):  # the last one: no splitting at all
+        mi.ops.set_tuning("decode_grid", grid)
+        try:
+            other = _run_case(mi, case, split_tokens=split, max_kv_len=mx).float()
+        finally:
+            mi.ops.set_tuning("decode_grid", 0)
         assert (base - other).abs().max().item() < 8e-3
     # and a sample of rows against the checker
     rows = [0, 17, 63]
@@ -128,10 +136,10 @@ def test_split_invariance_cfg2_full_size(mi, dev):
 
 
 def test_long_context_split_merge(mi, dev):
-    """cfg4 shape (64/8 heads, 131072-token context, 512 splits per request) at batch 2."""
+    """cfg4 shape (64/8 heads, 131072-token context, hundreds of partials per request) at batch 2."""
     case = mi.synthetic.make_decode_case(mi.synthetic.CONFIGS["cfg4"], dev, batch=2, on_device_rng=True)
-    out = _run_case(mi, case, split_tokens=256).float()
-    out2 = _run_case(mi, case, split_tokens=4096).float()
+    out = _run_case(mi, case).float()
+    out2 = _run_case(mi, case, split_tokens=65536).float()
     assert (out - out2).abs().max().item() < 5e-3
     ref = oa.paged_decode_attention(case.q[:1].cpu().squeeze(1), case.k_cache.cpu(), case.v_cache.cpu(),
                                     case.kv_lens[:1].cpu(), case.block_table[:1].cpu())
