@@ -75,6 +75,7 @@ def kv_append(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor,
               token_to_chunk_idx: Tensor, token_to_local_pos: Tensor) -> None:
     """``k_cache[chunk_idx[t], local[t]] = key[t]`` (and value): bit-exact scatter."""
     lib = _lib.load()
+    _stream(key)  # device check first: there is no CPU path
     key, row, k_st = _rows(key, "key")
     value, row_v, v_st = _rows(value, "value")
     T = key.size(0)
@@ -96,6 +97,7 @@ def kv_append_decode(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tenso
                      block_table: Tensor, kv_lens: Tensor) -> None:
     """Decode-step append with the slot derived on the GPU from block table + kv length."""
     lib = _lib.load()
+    _stream(key)  # device check first: there is no CPU path
     key, row, k_st = _rows(key, "key")
     value, row_v, v_st = _rows(value, "value")
     R = key.size(0)
@@ -119,6 +121,7 @@ def kv_append_decode(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tenso
 def quantize_chunks_fp8(src: Tensor, dst: Tensor, scales: Tensor) -> None:
     """Quantise whole bf16 chunks ``[N, C, Hkv, d]`` into an e4m3fn byte cache + ``[N, Hkv]`` scales."""
     lib = _lib.load()
+    _stream(src)  # device check first: there is no CPU path
     _require(src.dtype == torch.bfloat16, "source chunks must be bf16")
     _require(dst.element_size() == 1, "destination cache must hold one byte per element")
     _require(scales.dtype == torch.float32 and scales.is_contiguous(), "scales must be contiguous fp32")
@@ -136,6 +139,7 @@ def kv_append_decode_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: T
                          v_scales: Tensor, block_table: Tensor, kv_lens: Tensor, headroom: float = 2.0) -> None:
     """Quantise and append one new bf16 token per request into an fp8 cache."""
     lib = _lib.load()
+    _stream(key)  # device check first: there is no CPU path
     key, row, k_st = _rows(key, "key")
     value, _, v_st = _rows(value, "value")
     _require(key.dtype == torch.bfloat16 and value.dtype == torch.bfloat16 and k_st == v_st, "K/V must be bf16 with equal strides")
@@ -176,6 +180,7 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
                            v_scales: Optional[Tensor] = None) -> Tensor:
     """One query token per request against the paged cache; returns a tensor shaped like ``q``."""
     lib = _lib.load()
+    _stream(q)  # device check first: there is no CPU path
     q3 = _qo_view(q, "q")
     R, Hq, D = q3.shape
     N, C, Hkv, Dk = k_cache.shape
@@ -219,6 +224,7 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
                             max_kv_len: Optional[int] = None, out: Optional[Tensor] = None) -> Tensor:
     """Varlen causal attention of new tokens over the paged cache (bottom-right aligned mask)."""
     lib = _lib.load()
+    _stream(q)  # device check first: there is no CPU path
     q3 = _qo_view(q, "q")
     T, Hq, D = q3.shape
     N, C, Hkv, Dk = k_cache.shape

@@ -1,0 +1,84 @@
+"""The C-ABI library loads and exports exactly what include/mi355_decode.h declares (no compute calls)."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = ROOT / "include" / "mi355_decode.h"
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    text = text[text.index('extern "C"'):]
+    return re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", text)
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_functions()
+    assert len(names) == len(set(names))
+    for must in ("mi_kv_append", "mi_kv_append_decode", "mi_paged_decode_attention", "mi_decode_workspace_bytes",
+                 "mi_paged_prefill_attention", "mi_norm_rope_append", "mi_kv_quantize_chunks_fp8",
+                 "mi_kv_append_decode_fp8", "mi_version", "mi_last_error"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol(mi):
+    lib = ctypes.CDLL(str(mi._lib.LIB_PATH))
+    for name in declared_functions():
+        assert hasattr(lib, name), f"{name} is declared in the header but missing from the library"
+
+
+def test_python_binding_covers_the_header(mi):
+    assert set(mi._lib.SIGNATURES) == set(declared_functions())
+    lib = mi._lib.load()
+    assert lib.mi_version() >= 1
+    assert lib.mi_last_error() == b"" or isinstance(lib.mi_last_error(), bytes)
+
+
+def test_argument_validation_needs_no_gpu(mi):
+    """Rejections happen on the host before anything is enqueued."""
+    lib = mi._lib.load()
+    assert lib.mi_set_tuning(b"no_such_knob", 1) < 0
+    assert b"unknown knob" in lib.mi_last_error()
+    assert lib.mi_set_tuning(b"decode_tile_subtiles", 3) < 0
+    # null pointers
+    rc = lib.mi_kv_append(None, None, 8, None, None, 8, 8, None, None, 4, 8, 2, None)
+    assert rc == -1 and b"null" in lib.mi_last_error()
+    # T == 0 is a no-op that succeeds
+    assert lib.mi_kv_append(None, None, 8, None, None, 8, 8, None, None, 0, 8, 2, None) == 0
+    # unsupported head_dim / grouping are refused with a message
+    one = ctypes.c_void_p(16)
+    rc = lib.mi_paged_decode_attention(one, 96, 96, one, one, 96, 96, 96, one, 1, one, one, 96, 96, one, 1 << 30,
+                                       1, 1, 1, 96, 16, 16, 0, 0.1, 0, None, None, None)
+    assert rc == -4 and b"head_dim" in lib.mi_last_error()
+    rc = lib.mi_paged_decode_attention(one, 128, 128, one, one, 128, 128, 128, one, 1, one, one, 128, 128, one,
+                                       1 << 30, 1, 34, 2, 128, 16, 16, 0, 0.1, 0, None, None, None)
+    assert rc == -4 and b"16 query heads" in lib.mi_last_error()
+    rc = lib.mi_paged_decode_attention(one, 128, 128, one, one, 128, 128, 128, one, 1, one, one, 128, 128, one,
+                                       1 << 30, 1, 8, 2, 128, 24, 16, 0, 0.1, 0, None, None, None)
+    assert rc == -2 and b"multiple of 16" in lib.mi_last_error()
+    assert lib.mi_decode_workspace_bytes(0, 8, 2, 128, 16, 16, 0) == 0
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="this checks the behaviour on a machine without a GPU")
+def test_ops_refuse_cpu_tensors_loudly(mi):
+    """No CPU fallback: handing the ops host tensors is an error, not a slow path."""
+    q = torch.zeros(2, 1, 8, 128, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 16, 2, 128, dtype=torch.bfloat16)
+    bt = torch.zeros(2, 2, dtype=torch.int32)
+    lens = torch.ones(2, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mi.ops.paged_decode_attention(q, kc, kc, lens, bt)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        mi.ops.kv_append(q[:, :, :2], q[:, :, :2], kc, kc, torch.zeros(2, dtype=torch.int64),
+                         torch.zeros(2, dtype=torch.int64))
+
+
+def test_missing_library_is_an_error(mi, tmp_path, monkeypatch):
+    monkeypatch.setattr(mi._lib, "_lib", None)
+    monkeypatch.setattr(mi._lib, "LIB_PATH", tmp_path / "libmi355_decode.so")
+    with pytest.raises(mi._lib.LibraryMissingError):
+        mi._lib.load()
