@@ -128,14 +128,13 @@ def main():
 
     def step():
         if not args.attention_only:
-            q_in.copy_(case.q)  # the projection's fresh output each step (norm + RoPE work in place)
             if cfg.fp8:
-                mi.ops.norm_rope_append(q_in, case.k_new, key_out=k_rot, q_weight=qw, k_weight=kw, eps=1e-5,
+                mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_in, key_out=k_rot, q_weight=qw, k_weight=kw, eps=1e-5,
                                         norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos)
                 mi.ops.kv_append_decode_fp8(k_rot, case.v_new, case.k_cache, case.v_cache, case.k_scales,
                                             case.v_scales, case.block_table, case.kv_lens)
             else:
-                mi.ops.norm_rope_append(q_in, case.k_new, value=case.v_new, q_weight=qw, k_weight=kw, eps=1e-5,
+                mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_in, value=case.v_new, q_weight=qw, k_weight=kw, eps=1e-5,
                                         norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos,
                                         k_cache=case.k_cache, v_cache=case.v_cache, block_table=case.block_table,
                                         kv_lens=case.kv_lens)

@@ -168,8 +168,9 @@ int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_st
  * apply_rotary_emb_query (dynamic_context.py:566-631 ->
  * megatron/core/models/common/embeddings/rope_utils.py:92-126) and, optionally,
  * append_key_value_cache (dynamic_context.py:511-545).
- *  q `[T,Hq,d]` bf16 is updated in place; k `[T,Hkv,d]` is read, the result goes to
- *  k_out (if non-null) and to the cache slot (if k_cache non-null, together with v).
+ *  q `[T,Hq,d]` bf16 is read and the result written to q_out (which may be q itself);
+ *  k `[T,Hkv,d]` is read, the result goes to k_out (if non-null) and to the cache slot
+ *  (if k_cache non-null, together with v).
  *  norm_kind: MI_NORM_NONE | MI_NORM_RMS (weights bf16 [d], may be null) | MI_NORM_L2.
  *  rotary_angles: fp32 `[max_pos, rot_dim]` table of angles as built by
  *  RotaryEmbedding.forward (rotary_pos_embedding.py:151-181), null = no rotary;
@@ -178,8 +179,8 @@ int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_st
  *  given, else block_table + kv_lens as in mi_kv_append_decode (then T == R).
  *  faithful_rounding != 0 rounds to bf16 wherever the unfused bf16 op chain does.
  */
-int mi_norm_rope_append(void* q, int64_t q_stride_tok, const void* k, int64_t k_stride_tok,
-                        void* k_out, int64_t k_out_stride_tok, const void* v, int64_t v_stride_tok,
+int mi_norm_rope_append(const void* q, int64_t q_stride_tok, void* q_out, int64_t q_out_stride_tok,
+                        const void* k, int64_t k_stride_tok, void* k_out, int64_t k_out_stride_tok, const void* v, int64_t v_stride_tok,
                         const void* q_weight, const void* k_weight, float eps, int32_t norm_kind,
                         const float* rotary_angles, int64_t angles_stride, int32_t rot_dim,
                         int32_t rotary_interleaved, float mscale, const int64_t* q_positions,

@@ -25,7 +25,7 @@ static int env_int(const char* name, int dflt) {
 }
 
 MiTuning& mi_tuning() {
-  static MiTuning t = {env_int("MI355_DECODE_SUBTILES", 2), env_int("MI355_PREFILL_SUBTILES", 2),
+  static MiTuning t = {env_int("MI355_DECODE_SUBTILES", 0), env_int("MI355_PREFILL_SUBTILES", 2),
                       env_int("MI355_DECODE_MIN_WAVES", 3),
                       env_int("MI355_DECODE_WGS_PER_CU", 1), env_int("MI355_DECODE_GRID", 0),
                       env_int("MI355_DECODE_WAVES_PER_BLOCK", 8)};
@@ -39,7 +39,8 @@ extern "C" const char* mi_last_error(void) { return g_err; }
 extern "C" int mi_set_tuning(const char* name, int32_t value) {
   if (!name) return mi_fail(MI_ERR_NULL, "mi_set_tuning: null name");
   if (!strcmp(name, "decode_tile_subtiles")) {
-    if (value != 1 && value != 2) return mi_fail(MI_ERR_UNSUPPORTED, "decode_tile_subtiles must be 1 or 2");
+    if (value != 0 && value != 1 && value != 2 && value != 4)
+      return mi_fail(MI_ERR_UNSUPPORTED, "decode_tile_subtiles must be 0 (automatic), 1, 2 or 4");
     mi_tuning().decode_tile_subtiles = value;
     return MI_OK;
   }
@@ -48,7 +49,7 @@ extern "C" int mi_set_tuning(const char* name, int32_t value) {
     return MI_OK;
   }
   if (!strcmp(name, "decode_min_waves")) {
-    if (value != 3 && value != 4) return mi_fail(MI_ERR_UNSUPPORTED, "decode_min_waves must be 3 or 4");
+    if (value < 2 || value > 4) return mi_fail(MI_ERR_UNSUPPORTED, "decode_min_waves must be 2, 3 or 4");
     mi_tuning().decode_min_waves = value;
     return MI_OK;
   }

@@ -23,9 +23,9 @@ enum { MI_KV_BF16 = 0, MI_KV_FP8_E4M3 = 1 };
 enum { MI_NORM_NONE = 0, MI_NORM_RMS = 1, MI_NORM_L2 = 2 };
 
 struct MiTuning {
-  int decode_tile_subtiles;  // 16-token sub-tiles per loop iteration of the decode kernel: 1 or 2
+  int decode_tile_subtiles;  // 16-token sub-tiles per loop iteration of the decode kernel: 0 = automatic, 1, 2, 4 (fp8)
   int prefill_tile_subtiles;
-  int decode_min_waves;        // occupancy target of the decode kernel, waves per SIMD: 3 or 4
+  int decode_min_waves;        // occupancy target of the decode kernel, waves per SIMD: 2, 3 or 4
   int decode_wgs_per_cu;       // decode workgroups (of 8 waves) per CU in the streaming grid
   int decode_grid;             // >0 forces the streaming grid size (tests)
   int decode_waves_per_block;  // cap on wavefronts (= KV heads) per decode workgroup, 1..8

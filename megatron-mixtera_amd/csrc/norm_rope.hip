@@ -17,8 +17,8 @@
 // so the result equals the op-by-op bf16 evaluation; with `faithful == 0` the
 // whole expression is evaluated in fp32 and rounded once.
 //
-// One workgroup (4 waves) per token; each head vector is handled by d/2 lanes,
-// lane i owning elements i and i + d/2.  The normalised vector goes through a
+// grid = (tokens, groups of head vectors); a workgroup of 4 waves handles 4 (d = 128) or 8
+// (d = 64) head vectors of one token, each by d/2 lanes, lane i owning elements i and i + d/2.  The normalised vector goes through a
 // few hundred bytes of LDS so that any rotary pairing (half-split, interleaved,
 // partial rotary width) reads its partner from there.
 #include "mi_common.h"
@@ -27,8 +27,10 @@
 namespace mi {
 
 struct NormRopeParams {
-  uint16_t* q;  // [T][Hq][d] in place
+  const uint16_t* q;  // [T][Hq][d]
   int64_t q_st;
+  uint16_t* q_out;  // [T][Hq][d]; may alias q
+  int64_t qo_st;
   const uint16_t* k;  // [T][Hkv][d]
   int64_t k_st;
   uint16_t* k_out;  // [T][Hkv][d] or null
@@ -84,8 +86,8 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
     }
   }
 
-  for (int base = 0; base < nvec; base += VPB) {
-    const int vec = base + slot;
+  {
+    const int vec = blockIdx.y * VPB + slot;
     const bool active = vec < nvec;
     const bool is_q = vec < p.Hq;
     const int head = is_q ? vec : vec - p.Hq;
@@ -155,7 +157,7 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
     if (active) {
       const uint16_t b0 = f32_to_bf16(o0), b1 = f32_to_bf16(o1);
       if (is_q) {
-        uint16_t* dst = p.q + (int64_t)t * p.q_st + (int64_t)head * D;
+        uint16_t* dst = p.q_out + (int64_t)t * p.qo_st + (int64_t)head * D;
         dst[i] = b0;
         dst[i + LPV] = b1;
       } else {
@@ -172,8 +174,8 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
       }
     }
   }
-  // Value rows are copied unchanged.
-  if (cache_off >= 0 && p.v) {
+  // Value rows are copied unchanged (by the first workgroup of the token).
+  if (blockIdx.y == 0 && cache_off >= 0 && p.v) {
     const uint32_t* src = reinterpret_cast<const uint32_t*>(p.v + (int64_t)t * p.v_st);
     uint32_t* dst = reinterpret_cast<uint32_t*>(p.vc + cache_off);
     for (int e = threadIdx.x; e < p.Hkv * D / 2; e += 256) dst[e] = src[e];
@@ -185,7 +187,8 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
 using namespace mi;
 
 extern "C" int mi_norm_rope_append(
-    void* q, int64_t q_stride_tok, const void* k, int64_t k_stride_tok, void* k_out,
+    const void* q, int64_t q_stride_tok, void* q_out, int64_t q_out_stride_tok, const void* k,
+    int64_t k_stride_tok, void* k_out,
     int64_t k_out_stride_tok, const void* v, int64_t v_stride_tok, const void* q_weight,
     const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles,
     int64_t angles_stride, int32_t rot_dim, int32_t rotary_interleaved, float mscale,
@@ -197,8 +200,8 @@ extern "C" int mi_norm_rope_append(
   if (T == 0) return MI_OK;
   if (T < 0 || Hq < 0 || Hkv < 0 || Hq + Hkv == 0)
     return mi_fail(MI_ERR_SHAPE, "mi_norm_rope_append: bad sizes");
-  if ((Hq > 0 && !q) || (Hkv > 0 && !k))
-    return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: q / k missing");
+  if ((Hq > 0 && (!q || !q_out)) || (Hkv > 0 && !k))
+    return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: q / q_out / k missing");
   if (head_dim != 64 && head_dim != 128)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_norm_rope_append: head_dim must be 64 or 128");
   if (norm_kind != MI_NORM_NONE && norm_kind != MI_NORM_RMS && norm_kind != MI_NORM_L2)
@@ -220,7 +223,8 @@ extern "C" int mi_norm_rope_append(
       return mi_fail(MI_ERR_ALIGN, "mi_norm_rope_append: value rows must be 4-byte aligned");
   }
   NormRopeParams p = {};
-  p.q = (uint16_t*)q; p.q_st = q_stride_tok;
+  p.q = (const uint16_t*)q; p.q_st = q_stride_tok;
+  p.q_out = (uint16_t*)q_out; p.qo_st = q_out_stride_tok;
   p.k = (const uint16_t*)k; p.k_st = k_stride_tok;
   p.k_out = (uint16_t*)k_out; p.ko_st = k_out_stride_tok;
   p.v = (const uint16_t*)v; p.v_st = v_stride_tok;
@@ -236,7 +240,10 @@ extern "C" int mi_norm_rope_append(
   p.norm = norm_kind; p.interleaved = rotary_interleaved; p.faithful = faithful_rounding;
   p.eps = eps; p.mscale = mscale;
   hipStream_t st = (hipStream_t)stream;
-  if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), dim3(T), dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((norm_rope_append_kernel<64>), dim3(T), dim3(256), 0, st, p);
+  const int vpb = head_dim == 128 ? 4 : 8;
+  dim3 grid(T, (Hq + Hkv + vpb - 1) / vpb);
+  if (grid.y > 65535) return mi_fail(MI_ERR_SHAPE, "mi_norm_rope_append: too many heads");
+  if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), grid, dim3(256), 0, st, p);
+  else hipLaunchKernelGGL((norm_rope_append_kernel<64>), grid, dim3(256), 0, st, p);
   return mi_check_launch("mi_norm_rope_append");
 }

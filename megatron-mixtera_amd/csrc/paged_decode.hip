@@ -480,7 +480,9 @@ extern "C" int mi_paged_decode_attention(
   if ((uintptr_t)workspace & 15)
     return mi_fail(MI_ERR_ALIGN, "mi_paged_decode_attention: workspace must be 16-byte aligned");
 
-  const int nt = mi_tuning().decode_tile_subtiles == 1 ? 1 : 2;
+  // 16-token sub-tiles per loop iteration (0 = automatic).
+  int nt = mi_tuning().decode_tile_subtiles;
+  if (nt != 1 && nt != 2 && nt != 4) nt = kv_dtype == MI_KV_FP8_E4M3 ? 4 : 2;
   const int minw = mi_tuning().decode_min_waves;
   const int tk = 16 * nt;
   const int min_span_tokens = split_tokens > 0 ? split_tokens : 256;
@@ -513,9 +515,16 @@ extern "C" int mi_paged_decode_attention(
     if (nt == 1 && minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 4>), grid, block, lds, st, p); \
     else if (nt == 1) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 3>), grid, block, lds, st, p);       \
     else if (minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 4>), grid, block, lds, st, p);     \
-    else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 3>), grid, block, lds, st, p);                    \
+    else if (minw == 3) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 3>), grid, block, lds, st, p);     \
+    else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 2>), grid, block, lds, st, p);                    \
   } while (0)
-  if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true);
+  if (kv_dtype == MI_KV_FP8_E4M3 && nt == 4)
+    hipLaunchKernelGGL((paged_decode_stream_kernel<128, 4, true, 2>), grid, block, lds, st, p);
+  else if (head_dim == 128 && nt == 4)
+    hipLaunchKernelGGL((paged_decode_stream_kernel<128, 4, false, 2>), grid, block, lds, st, p);
+  else if (nt == 4)
+    hipLaunchKernelGGL((paged_decode_stream_kernel<64, 4, false, 2>), grid, block, lds, st, p);
+  else if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true);
   else if (head_dim == 128) MI_LAUNCH_DECODE(128, false);
   else MI_LAUNCH_DECODE(64, false);
 #undef MI_LAUNCH_DECODE

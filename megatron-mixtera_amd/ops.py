@@ -270,12 +270,14 @@ def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: O
                      q_weight: Optional[Tensor] = None, k_weight: Optional[Tensor] = None,
                      eps: float = 1e-5, norm: Optional[str] = None, rotary_emb: Optional[Tensor] = None,
                      q_positions: Optional[Tensor] = None, k_positions: Optional[Tensor] = None,
-                     rotary_interleaved: bool = False, mscale: float = 1.0, key_out: Optional[Tensor] = None,
+                     rotary_interleaved: bool = False, mscale: float = 1.0, query_out: Optional[Tensor] = None,
+                     key_out: Optional[Tensor] = None,
                      k_cache: Optional[Tensor] = None, v_cache: Optional[Tensor] = None,
                      token_to_chunk_idx: Optional[Tensor] = None, token_to_local_pos: Optional[Tensor] = None,
                      block_table: Optional[Tensor] = None, kv_lens: Optional[Tensor] = None,
                      faithful_rounding: bool = True) -> None:
-    """Norm (none / rms / l2) then RoPE on ``query`` (in place) and ``key`` (to ``key_out`` and/or cache)."""
+    """Norm (none / rms / l2) then RoPE on ``query`` (in place unless ``query_out`` is given) and on
+    ``key`` (result to ``key_out`` and/or straight into the cache slot, together with ``value``)."""
     lib = _lib.load()
     ref = query if query is not None else key
     _require(ref is not None, "need query and/or key")
@@ -291,6 +293,10 @@ def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: O
         _require(k3.stride(1) == D, "key heads must be contiguous")
         T, Hkv = k3.size(0), k3.size(1)
         _require(query is None or q3.size(0) == T, "query / key token counts differ")
+    qo3 = q3
+    if query_out is not None:
+        qo3 = _qo_view(query_out, "query_out")
+        _require(q3 is not None and tuple(qo3.shape) == tuple(q3.shape) and qo3.stride(1) == D, "query_out shape")
     ko3 = None
     if key_out is not None:
         ko3 = _qo_view(key_out, "key_out")
@@ -315,7 +321,8 @@ def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: O
             _require(block_table.dtype == torch.int32 and block_table.stride(1) == 1, "bad block_table")
             _require(kv_lens is not None and kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "bad kv_lens")
     _lib.check(lib.mi_norm_rope_append(
-        _ptr(q3), 0 if q3 is None else q3.stride(0), _ptr(k3), 0 if k3 is None else k3.stride(0),
+        _ptr(q3), 0 if q3 is None else q3.stride(0), _ptr(qo3), 0 if qo3 is None else qo3.stride(0),
+        _ptr(k3), 0 if k3 is None else k3.stride(0),
         _ptr(ko3), 0 if ko3 is None else ko3.stride(0), _ptr(v3), 0 if v3 is None else v3.stride(0),
         _ptr(q_weight), _ptr(k_weight), float(eps), _NORM_KINDS[norm], _ptr(ang), a_stride, rot,
         int(bool(rotary_interleaved)), float(mscale), _ptr(q_positions), _ptr(k_positions),

@@ -44,6 +44,7 @@ def test_argument_validation_needs_no_gpu(mi):
     assert lib.mi_set_tuning(b"no_such_knob", 1) < 0
     assert b"unknown knob" in lib.mi_last_error()
     assert lib.mi_set_tuning(b"decode_tile_subtiles", 3) < 0
+    assert lib.mi_set_tuning(b"decode_tile_subtiles", 0) == 0
     # null pointers
     rc = lib.mi_kv_append(None, None, 8, None, None, 8, 8, None, None, 4, 8, 2, None)
     assert rc == -1 and b"null" in lib.mi_last_error()

@@ -69,7 +69,7 @@ def test_ragged_lengths_and_edges(mi, dev, chunk, subtiles, grid):
             _close(out, _ref(case), 2e-2)
             assert (out[case.kv_lens == 0] == 0).all(), "zero-length rows must be zeros"
     finally:
-        mi.ops.set_tuning("decode_tile_subtiles", 2)
+        mi.ops.set_tuning("decode_tile_subtiles", 0)
         mi.ops.set_tuning("decode_grid", 0)
 
 
