@@ -39,6 +39,9 @@ def parse_args():
     ap.add_argument("--subtiles", type=int, default=0, help="16-token sub-tiles per loop iteration (1, 2 or 4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--attention-only", action="store_true", help="time the attention call alone")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="also run a plain device copy of this many MiB (a known-size reference for "
+                         "scaling hardware traffic counters collected by an external profiler)")
     return ap.parse_args()
 
 
@@ -141,6 +144,14 @@ def main():
         mi.ops.paged_decode_attention(q_in, case.k_cache, case.v_cache, case.kv_lens, case.block_table, out=out,
                                       max_kv_len=max_len, split_tokens=args.split_tokens,
                                       k_scales=case.k_scales, v_scales=case.v_scales)
+
+    if args.calibrate_copy_mib:
+        src = torch.empty(args.calibrate_copy_mib << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     k_rot = torch.empty_like(case.k_new)
     for _ in range(args.warmup):

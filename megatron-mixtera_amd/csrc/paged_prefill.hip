@@ -51,6 +51,17 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(PrefillParams p) {
   const int BQ = 64 >> p.g_shift;  // query tokens per wave
   const int SBQ = 4 * BQ;          // query tokens per workgroup
 
+  // Rows beyond the last request (token padding of the batch) are defined as zeros; the first
+  // workgroup of every KV head clears its heads of those rows.
+  if (blockIdx.x == 0) {
+    const int tq = p.cu_q[p.R];
+    const int per_row = G * HD;  // contiguous elements of this head group in one row
+    for (int64_t i = (int64_t)threadIdx.x * 8; i < (int64_t)(p.T - tq) * per_row; i += 256 * 8) {
+      const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
+      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
+    }
+  }
+
   // ---- which request does this workgroup belong to? ----------------------------
   // Request r's workgroups start at pbs(r) = cu_q[r] / SBQ + r, a strictly
   // increasing sequence that leaves at least ceil(Lq_r / SBQ) indices to r.
