@@ -28,6 +28,12 @@ if str(ROOT) not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 
+# HBM bytes per launch of the streaming kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this same script, each counter scaled by what it reads for a plain 1 GiB device copy
+# (profiles/paged_decode_stream_kernel_cfg2_hbm_traffic.md).  Hardware counters cannot be read from
+# inside the benchmark, so the figure is recorded here per workload; None = not collected.
+MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_252_000_000}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -206,7 +212,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "kernel_ms": round(kernel_ms, 5),
-            "traffic": None,
+            "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
         },
     }
     if not args.no_cpu_baseline:

@@ -90,7 +90,10 @@ bool mi_profile_next(hipEvent_t* a, hipEvent_t* b) {
   if (g_used == g_pool.size()) {
     if (g_pool.size() >= 65536) return false;
     EventPair p;
-    if (hipEventCreate(&p.a) != hipSuccess || hipEventCreate(&p.b) != hipSuccess) return false;
+    // no system-scope fence: the events only time device work on one stream
+    if (hipEventCreateWithFlags(&p.a, hipEventDisableSystemFence) != hipSuccess ||
+        hipEventCreateWithFlags(&p.b, hipEventDisableSystemFence) != hipSuccess)
+      return false;
     g_pool.push_back(p);
   }
   *a = g_pool[g_used].a;
