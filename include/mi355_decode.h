@@ -145,7 +145,10 @@ int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_str
  * max_seqlen_q, max_seqlen_k, softmax_scale, causal=True, block_table=...)
  * (megatron/core/transformer/attention.py:546-557): request r owns query rows
  * cu_seqlens_q[r]..cu_seqlens_q[r+1]-1 and kv_lens[r] keys; query i of Lq sees keys
- * j <= i + (Lk - Lq) (bottom-right aligned causal mask).
+ * j <= i + (Lk - Lq) (bottom-right aligned causal mask).  Rows past cu_seqlens_q[R] (token
+ * padding) are zeroed.  With a workspace of mi_prefill_workspace_bytes() bytes, requests that
+ * have exactly one query row (the decode requests of a mixed batch) are streamed by the
+ * decode kernels at full bandwidth; with workspace == NULL one kernel handles every request.
  */
 int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                    int32_t max_kv_len, int32_t split_tokens);

@@ -39,4 +39,14 @@ bool mi_profile_next(hipEvent_t* start, hipEvent_t* stop);
 
 namespace mi {
 int decode_grid_size(int Hkv);
+// Shared by the decode entry point and by the mixed-batch path of the prefill entry point
+// (cu_seqlens_q non-null: only requests with one query row take part, at row cu_seqlens_q[r]).
+int launch_paged_decode(const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
+                        const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok,
+                        int64_t kv_stride_head, const int32_t* block_table, int64_t bt_stride,
+                        const int32_t* kv_lens, const int32_t* cu_seqlens_q, void* out, int64_t o_stride_tok,
+                        int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq,
+                        int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t split_tokens,
+                        float softmax_scale, int32_t kv_dtype, const float* k_scales, const float* v_scales,
+                        void* stream);
 }

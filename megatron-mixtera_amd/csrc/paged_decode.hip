@@ -49,6 +49,8 @@ struct DecodeParams {
   const int32_t* bt;
   int64_t bt_stride;
   const int32_t* lens;
+  const int32_t* cu_q;  // null: row r of q/out belongs to request r.  Else (mixed batches): only
+                        // requests with exactly one query row take part, at row cu_q[r].
   uint16_t* out;
   int64_t o_st, o_sh;
   float* part_o;     // [slots][Hq][HD], slots = grid + R
@@ -69,8 +71,8 @@ static __device__ __forceinline__ int chunk_of(int tok, uint64_t magic) {
 // One segment: tokens [start, end) of request r for KV head h (one wavefront).
 // `whole` = the segment is the entire request (write bf16 output, no partial).
 template <int HD, int NT, bool FP8>
-static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int h, int len, int start,
-                                                      int end, bool whole, int slot, int lane) {
+static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int row, int h, int len,
+                                                      int start, int end, bool whole, int slot, int lane) {
   constexpr int KS = HD / 32;
   constexpr int DV = HD / 16;
   static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
@@ -83,7 +85,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   // Query fragments: B operand rows are the G heads of this KV head.
   uint4 qf[KS];
   {
-    const uint16_t* qrow = p.q + (int64_t)r * p.q_st + (int64_t)hq * p.q_sh;
+    const uint16_t* qrow = p.q + (int64_t)row * p.q_st + (int64_t)hq * p.q_sh;
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) {
       // bf16 cache: lane g owns d = 32kk + 8g .. +7.
@@ -276,7 +278,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   if (m16 >= G) return;  // (no barrier follows inside a segment)
   // acc[e][i] holds d = DV*(4g+i) + e: DV*4 contiguous values per lane.
   if (whole) {
-    uint16_t* o = p.out + (int64_t)r * p.o_st + (int64_t)hq * p.o_sh + 4 * DV * g;
+    uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + 4 * DV * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if constexpr (DV == 8) {
@@ -307,6 +309,16 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
 // Tiles (of TK tokens) of one request.
 static __device__ __forceinline__ int tiles_of(int len, int tk) { return len > 0 ? (len + tk - 1) / tk : 0; }
 
+// Does request r take part in this launch, and which q/out row is its?
+static __device__ __forceinline__ bool decode_row(const DecodeParams& p, int r, int& row) {
+  if (!p.cu_q) {
+    row = r;
+    return true;
+  }
+  row = p.cu_q[r];
+  return p.cu_q[r + 1] - row == 1;
+}
+
 template <int HD, int NT, bool FP8, int MINW>
 __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
   constexpr int TK = 16 * NT;
@@ -321,7 +333,8 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
     int carry = 0;
     for (int base = 0; base < p.R; base += 64) {
       const int i = base + lane;
-      int v = i < p.R ? tiles_of(p.lens[i], TK) : 0;
+      int row_unused;
+      int v = (i < p.R && decode_row(p, i, row_unused)) ? tiles_of(p.lens[i], TK) : 0;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
         const int up = __shfl_up(v, o, 64);
@@ -357,7 +370,9 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
         if (first) p.seg_info[2 * r] = blockIdx.x;
         if (final) p.seg_info[2 * r + 1] = blockIdx.x;
       }
-      decode_segment<HD, NT, FP8>(p, r, h, len, tb * TK, min(te * TK, len), first && final,
+      int row;
+      decode_row(p, r, row);
+      decode_segment<HD, NT, FP8>(p, r, row, h, len, tb * TK, min(te * TK, len), first && final,
                                   (int)blockIdx.x + r, lane);
       t0 = rb + te;
     }
@@ -370,7 +385,9 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
 template <int HD>
 __global__ __launch_bounds__(HD) void paged_decode_merge_kernel(DecodeParams p) {
   const int r = blockIdx.y, hq = blockIdx.x, d = threadIdx.x;
-  uint16_t* o = p.out + (int64_t)r * p.o_st + (int64_t)hq * p.o_sh + d;
+  int row;
+  if (!decode_row(p, r, row)) return;
+  uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + d;
   if (p.lens[r] <= 0) {
     *o = 0;
     return;
@@ -435,15 +452,14 @@ extern "C" int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv,
   return slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
 
-extern "C" int mi_paged_decode_attention(
+int mi::launch_paged_decode(
     const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
     const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
-    const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
-    int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
-    int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, const int32_t* cu_seqlens_q,
+    void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
+    int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
     int32_t split_tokens, float softmax_scale, int32_t kv_dtype, const float* k_scales,
     const float* v_scales, void* stream) {
-  (void)max_kv_len;
   if (R == 0) return MI_OK;
   if (!q || !k_cache || !v_cache || !block_table || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_decode_attention: null pointer argument");
@@ -491,7 +507,7 @@ extern "C" int mi_paged_decode_attention(
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
   p.kc = (const uint8_t*)k_cache; p.vc = (const uint8_t*)v_cache;
   p.kv_sc = kv_stride_chunk; p.kv_st = (int32_t)kv_stride_tok; p.kv_sh = (int32_t)kv_stride_head;
-  p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens;
+  p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens; p.cu_q = cu_seqlens_q;
   p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
   p.part_o = (float*)workspace;
   p.part_lse = p.part_o + slots * Hq * head_dim;
@@ -533,4 +549,19 @@ extern "C" int mi_paged_decode_attention(
   if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p);
   else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p);
   return mi_check_launch("mi_paged_decode_attention");
+}
+
+extern "C" int mi_paged_decode_attention(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
+    const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
+    int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
+    int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len,
+    int32_t split_tokens, float softmax_scale, int32_t kv_dtype, const float* k_scales,
+    const float* v_scales, void* stream) {
+  (void)max_kv_len;
+  return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
+                             kv_stride_head, block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok,
+                             o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
+                             split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
 }

@@ -18,6 +18,8 @@
 #include "mi_common.h"
 #include "mi_capi_internal.h"
 
+extern "C" int64_t mi_decode_workspace_bytes(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t);
+
 namespace mi {
 
 struct PrefillParams {
@@ -34,6 +36,7 @@ struct PrefillParams {
   uint16_t* out;
   int64_t o_st, o_sh;
   int32_t T, R, Hq, Hkv, G, g_shift, chunk, chunk_shift;
+  int32_t skip_single;  // requests with exactly one query row are handled by the decode kernels
   float scale_log2;
 };
 
@@ -76,6 +79,7 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(PrefillParams p) {
   const int Lq = p.cu_q[r + 1] - q_begin;
   const int q0 = (sb - (q_begin / SBQ + r)) * SBQ + wave * BQ;  // first query of this wave
   if (q0 >= Lq) return;
+  if (p.skip_single && Lq == 1) return;
   const int Lk = p.lens[r];
   const int shift = Lk - Lq;  // key position of query 0
   const int nq = min(BQ, Lq - q0);
@@ -253,8 +257,10 @@ using namespace mi;
 extern "C" int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
                                               int32_t head_dim, int32_t max_kv_len,
                                               int32_t split_tokens) {
-  (void)T; (void)R; (void)Hq; (void)Hkv; (void)head_dim; (void)max_kv_len; (void)split_tokens;
-  return 0;  // the current kernel keeps every row's state in registers
+  (void)T;
+  // Only the one-row (decode) requests of a mixed batch need scratch: they are streamed by the
+  // decode kernels, whose partials live here.
+  return mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens);
 }
 
 extern "C" int mi_paged_prefill_attention(
@@ -265,7 +271,7 @@ extern "C" int mi_paged_prefill_attention(
     void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
     int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
     float softmax_scale, void* stream) {
-  (void)workspace; (void)workspace_bytes; (void)max_kv_len; (void)split_tokens;
+  (void)max_kv_len;
   if (T == 0 || R == 0) return MI_OK;
   if (!q || !k_cache || !v_cache || !block_table || !cu_seqlens_q || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention: null pointer argument");
@@ -301,6 +307,8 @@ extern "C" int mi_paged_prefill_attention(
     while ((1 << p.chunk_shift) < chunk_tokens) ++p.chunk_shift;
   }
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
+  // With a workspace, one-row requests go through the bandwidth-optimised decode kernels.
+  p.skip_single = workspace != nullptr;
 
   const int sbq = 4 * (64 / G);
   dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(256);
@@ -313,5 +321,10 @@ extern "C" int mi_paged_prefill_attention(
     if (nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<64, 1>), grid, block, 0, st, p);
     else hipLaunchKernelGGL((paged_prefill_kernel<64, 2>), grid, block, 0, st, p);
   }
-  return mi_check_launch("mi_paged_prefill_attention");
+  int rc = mi_check_launch("mi_paged_prefill_attention");
+  if (rc != MI_OK || !p.skip_single) return rc;
+  return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
+                             kv_stride_head, block_table, bt_stride, kv_lens, cu_seqlens_q, out, o_stride_tok,
+                             o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
+                             split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
 }

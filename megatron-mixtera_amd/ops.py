@@ -245,10 +245,13 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
         out = torch.empty_like(q)
     o3 = _qo_view(out, "out")
     _require(tuple(o3.shape) == (T, Hq, D), "out shape mismatch")
+    workspace = _workspace(q.device, lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, D, int(max_kv_len), 0))
+    ws_bytes = 0 if workspace is None else workspace.numel()
     _lib.check(lib.mi_paged_prefill_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
         block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),
-        o3.data_ptr(), o3.stride(0), o3.stride(1), None, 0, T, R, Hq, Hkv, D, C, int(max_kv_len), 0,
+        o3.data_ptr(), o3.stride(0), o3.stride(1), _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C,
+        int(max_kv_len), 0,
         float(softmax_scale), _stream(q)), "mi_paged_prefill_attention")
     return out
 
