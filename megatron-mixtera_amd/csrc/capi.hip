@@ -26,6 +26,7 @@ static int env_int(const char* name, int dflt) {
 
 MiTuning& mi_tuning() {
   static MiTuning t = {env_int("MI355_DECODE_SUBTILES", 0), env_int("MI355_PREFILL_SUBTILES", 2),
+                      env_int("MI355_PREFILL_LDS_ROW_TILES", 3), env_int("MI355_PREFILL_ROW_TILES", 2),
                       env_int("MI355_DECODE_MIN_WAVES", 3),
                       env_int("MI355_DECODE_WGS_PER_CU", 1), env_int("MI355_DECODE_GRID", 0),
                       env_int("MI355_DECODE_WAVES_PER_BLOCK", 8)};
@@ -42,6 +43,16 @@ extern "C" int mi_set_tuning(const char* name, int32_t value) {
     if (value != 0 && value != 1 && value != 2 && value != 4)
       return mi_fail(MI_ERR_UNSUPPORTED, "decode_tile_subtiles must be 0 (automatic), 1, 2 or 4");
     mi_tuning().decode_tile_subtiles = value;
+    return MI_OK;
+  }
+  if (!strcmp(name, "prefill_lds_row_tiles")) {
+    if (value != 0 && value != 2 && value != 3) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_lds_row_tiles must be 0, 2 or 3");
+    mi_tuning().prefill_lds_row_tiles = value;
+    return MI_OK;
+  }
+  if (!strcmp(name, "prefill_row_tiles")) {
+    if (value != 2 && value != 4) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_row_tiles must be 2 or 4");
+    mi_tuning().prefill_row_tiles = value;
     return MI_OK;
   }
   if (!strcmp(name, "prefill_tile_subtiles")) {

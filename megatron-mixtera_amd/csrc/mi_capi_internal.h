@@ -25,6 +25,8 @@ enum { MI_NORM_NONE = 0, MI_NORM_RMS = 1, MI_NORM_L2 = 2 };
 struct MiTuning {
   int decode_tile_subtiles;  // 16-token sub-tiles per loop iteration of the decode kernel: 0 = automatic, 1, 2, 4 (fp8)
   int prefill_tile_subtiles;
+  int prefill_lds_row_tiles;   // LDS-shared prefill kernel (head_dim 128): 16-row tiles per wave, 2 or 3; 0 = off
+  int prefill_row_tiles;       // 16-row tiles per wave in the prefill kernel: 2 (8 waves) or 4 (4 waves)
   int decode_min_waves;        // occupancy target of the decode kernel, waves per SIMD: 2, 3 or 4
   int decode_wgs_per_cu;       // decode workgroups (of 8 waves) per CU in the streaming grid
   int decode_grid;             // >0 forces the streaming grid size (tests)

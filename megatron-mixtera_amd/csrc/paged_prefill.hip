@@ -35,31 +35,33 @@ struct PrefillParams {
   const int32_t* lens;
   uint16_t* out;
   int64_t o_st, o_sh;
-  int32_t T, R, Hq, Hkv, G, g_shift, chunk, chunk_shift;
+  uint64_t chunk_magic;  // ceil(2^40 / chunk)
+  int32_t T, R, Hq, Hkv, G, g_shift, chunk;
   int32_t skip_single;  // requests with exactly one query row are handled by the decode kernels
   float scale_log2;
 };
 
-template <int HD, int NT>
-__global__ __launch_bounds__(256) void paged_prefill_kernel(PrefillParams p) {
+// NQ = 16-row tiles per wave; a workgroup always covers 256 rows (16 / NQ waves).
+template <int HD, int NT, int NQ>
+__global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillParams p) {
   constexpr int KS = HD / 32;
   constexpr int DV = HD / 16;
-  constexpr int NQ = 4;  // 16-row tiles per wave
+  constexpr int WAVES = 16 / NQ;
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int m16 = lane & 15, g = lane >> 4;
   const int h = blockIdx.y;
   const int G = p.G;
-  const int BQ = 64 >> p.g_shift;  // query tokens per wave
-  const int SBQ = 4 * BQ;          // query tokens per workgroup
+  const int BQ = (16 * NQ) >> p.g_shift;  // query tokens per wave
+  const int SBQ = WAVES * BQ;             // query tokens per workgroup
 
   // Rows beyond the last request (token padding of the batch) are defined as zeros; the first
   // workgroup of every KV head clears its heads of those rows.
   if (blockIdx.x == 0) {
     const int tq = p.cu_q[p.R];
     const int per_row = G * HD;  // contiguous elements of this head group in one row
-    for (int64_t i = (int64_t)threadIdx.x * 8; i < (int64_t)(p.T - tq) * per_row; i += 256 * 8) {
+    for (int64_t i = (int64_t)threadIdx.x * 8; i < (int64_t)(p.T - tq) * per_row; i += 64 * WAVES * 8) {
       const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
       st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
     }
@@ -131,98 +133,167 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(PrefillParams p) {
     return;
   }
 
-  for (int T = 0; T < kend; T += 16 * NT) {
-    uint4 kf[NT][KS];
-    uint4 vf16[NT][4];
-    uint2 vf8[NT][4];
+  // K / V staging registers of one tile of 16*NT keys; the loop is software pipelined on them
+  // (K of the next tile is requested once all scores of this one exist, V once P.V is done).
+  uint4 kf[NT][KS];
+  uint4 vf16[NT][4];
+  uint2 vf8[NT][4];
+  auto load_k = [&](int T) {
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       const int T0 = T + 16 * u;
       const int tu = min(T0, last);
-      const int ci = p.chunk_shift >= 0 ? (tu >> p.chunk_shift) : (tu / p.chunk);
+      const int ci = (int)(((uint64_t)(uint32_t)tu * p.chunk_magic) >> 40);
       const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
-      const int cbase = ci * p.chunk;
-      const uint8_t* kc = kbase + (int64_t)pc * chunk_bytes;
-      const uint8_t* vc = vbase + (int64_t)pc * chunk_bytes;
-      const uint8_t* krow = kc + (min(T0 + m16, last) - cbase) * tok_bytes;
+      const uint8_t* krow = kbase + (int64_t)pc * chunk_bytes + (min(T0 + m16, last) - ci * p.chunk) * tok_bytes;
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk) kf[u][kk] = ld16(krow + (32 * kk + 8 * g) * 2);
+    }
+  };
+  auto load_v = [&](int T) {
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      const int T0 = T + 16 * u;
+      const int tu = min(T0, last);
+      const int ci = (int)(((uint64_t)(uint32_t)tu * p.chunk_magic) >> 40);
+      const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
+      const uint8_t* vc = vbase + (int64_t)pc * chunk_bytes;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint8_t* vrow = vc + (min(T0 + 4 * g + j, last) - cbase) * tok_bytes + DV * m16 * 2;
+        const uint8_t* vrow = vc + (min(T0 + 4 * g + j, last) - ci * p.chunk) * tok_bytes + DV * m16 * 2;
         if (HD == 128) vf16[u][j] = ld16(vrow);
         else vf8[u][j] = ld8(vrow);
       }
     }
+  };
 
+  // Keys up to and including `full_until` are visible to every valid row of this wave, so a
+  // tile that ends there needs no masking.
+  const int full_until = shift + q0;
+  const float scale = p.scale_log2;
+
+  load_k(0);
+  load_v(0);
+  __builtin_amdgcn_sched_barrier(0);
+  for (int T = 0; T < kend; T += 16 * NT) {
+    // ---- S^T = K Q^T for every 16-row tile of the wave (raw, unscaled) ----------------
+    f32x4_t s[NQ][NT];
 #pragma unroll
     for (int nt = 0; nt < NQ; ++nt) {
       if (nt >= ntiles) break;  // wave-uniform
-      // ---- scores of this 16-row tile against the NT key sub-tiles --------------
-      float sc[NT][4];
-      float tmax = -INFINITY;
 #pragma unroll
       for (int u = 0; u < NT; ++u) {
         f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32(kf[u][kk], qf[nt][kk], sacc);
-        const int tok0 = T + 16 * u + 4 * g;
+        s[nt][u] = sacc;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    load_k(T + 16 * NT);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- online softmax per 16-row tile ----------------------------------------------
+    const bool need_mask = T + 16 * NT - 1 > full_until;  // wave-uniform
+    uint2 pf[NQ][NT];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float v = (tok0 + i <= qpos[nt]) ? sacc[i] * p.scale_log2 : -INFINITY;
-          sc[u][i] = v;
-          tmax = fmaxf(tmax, v);
+    for (int nt = 0; nt < NQ; ++nt) {
+      if (nt >= ntiles) break;
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        if (need_mask) {
+          const int tok0 = T + 16 * u + 4 * g;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (tok0 + i > qpos[nt]) s[nt][u][i] = -INFINITY;
         }
+        tmax = fmaxf(fmaxf(fmaxf(s[nt][u][0], s[nt][u][1]), fmaxf(s[nt][u][2], s[nt][u][3])), tmax);
       }
       tmax = fmaxf(tmax, xor16(tmax));
       tmax = fmaxf(tmax, xor32(tmax));
-      // Key 0 is visible to every row of a well-formed request (Lk >= Lq), so m_run
-      // is finite after the first tile; a later tile that is fully masked for a row
-      // leaves it unchanged.
+      // Key 0 is visible to every row of a well-formed request (Lk >= Lq), so m_run is finite
+      // after the first tile; a row with no visible key so far keeps m_run = -inf and p = 0.
       const float m_raw = fmaxf(m_run[nt], tmax);
-      const float m_new = m_raw == -INFINITY ? 0.f : m_raw;  // row with no visible key so far
-      const float alpha = fast_exp2(m_run[nt] - m_new);
+      const float m_use = m_raw == -INFINITY ? 0.f : m_raw;
+      const float alpha = fast_exp2((m_run[nt] - m_use) * scale);
+      const float neg = -m_use * scale;
       m_run[nt] = m_raw;
       float psum = 0.f;
-      uint2 pf[NT];
 #pragma unroll
       for (int u = 0; u < NT; ++u) {
         float pv[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          pv[i] = fast_exp2(sc[u][i] - m_new);
+          pv[i] = fast_exp2(__builtin_fmaf(s[nt][u][i], scale, neg));
           psum += pv[i];
         }
-        pf[u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+        pf[nt][u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
       }
       l_run[nt] = l_run[nt] * alpha + psum;
+      // The running max rarely moves once a few tiles have been seen: skip the rescale of the
+      // accumulators when no lane of the wave needs it.
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
-      for (int e = 0; e < DV; ++e) {
-        acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
-      }
-#pragma unroll
-      for (int u = 0; u < NT; ++u) {
-        if constexpr (HD == 128) {
-          const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0]);
-          const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1]);
-          const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2]);
-          const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3]);
-#pragma unroll
-          for (int pr = 0; pr < 4; ++pr) {
-            acc[nt][2 * pr] = mfma_16x16x16(
-                make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr])), pf[u], acc[nt][2 * pr]);
-            acc[nt][2 * pr + 1] = mfma_16x16x16(
-                make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr])), pf[u], acc[nt][2 * pr + 1]);
-          }
-        } else {
-          const uint2 a = vf8[u][0], b = vf8[u][1], c = vf8[u][2], d = vf8[u][3];
-          acc[nt][0] = mfma_16x16x16(make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x)), pf[u], acc[nt][0]);
-          acc[nt][1] = mfma_16x16x16(make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x)), pf[u], acc[nt][1]);
-          acc[nt][2] = mfma_16x16x16(make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y)), pf[u], acc[nt][2]);
-          acc[nt][3] = mfma_16x16x16(make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y)), pf[u], acc[nt][3]);
+        for (int e = 0; e < DV; ++e) {
+          acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
         }
       }
     }
+
+    // ---- O^T += V^T P^T: each transposed V fragment serves all row tiles ---------------
+    // Two 16-key sub-tiles are contracted by one mfma 16x16x32 (slots 0-3 = tokens 4g..4g+3 of
+    // the first sub-tile, slots 4-7 = the same of the second; P is packed the same way).
+    auto transpose_v = [&](int u, uint2 (&vt)[DV]) {
+      if constexpr (HD == 128) {
+        const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0]);
+        const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1]);
+        const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2]);
+        const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3]);
+#pragma unroll
+        for (int pr = 0; pr < 4; ++pr) {
+          vt[2 * pr] = make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr]));
+          vt[2 * pr + 1] = make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr]));
+        }
+      } else {
+        const uint2 a = vf8[u][0], b = vf8[u][1], c = vf8[u][2], d = vf8[u][3];
+        vt[0] = make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x));
+        vt[1] = make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x));
+        vt[2] = make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y));
+        vt[3] = make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y));
+      }
+    };
+    if constexpr (NT % 2 == 0) {
+#pragma unroll
+      for (int u = 0; u < NT; u += 2) {
+        uint2 va[DV], vb[DV];
+        transpose_v(u, va);
+        transpose_v(u + 1, vb);
+#pragma unroll
+        for (int nt = 0; nt < NQ; ++nt) {
+          if (nt >= ntiles) break;
+          const uint4 pp = make_uint4(pf[nt][u].x, pf[nt][u].y, pf[nt][u + 1].x, pf[nt][u + 1].y);
+#pragma unroll
+          for (int e = 0; e < DV; ++e)
+            acc[nt][e] = mfma_16x16x32(make_uint4(va[e].x, va[e].y, vb[e].x, vb[e].y), pp, acc[nt][e]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        uint2 vt[DV];
+        transpose_v(u, vt);
+#pragma unroll
+        for (int nt = 0; nt < NQ; ++nt) {
+          if (nt >= ntiles) break;
+#pragma unroll
+          for (int e = 0; e < DV; ++e) acc[nt][e] = mfma_16x16x16(vt[e], pf[nt][u], acc[nt][e]);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    load_v(T + 16 * NT);
+    __builtin_amdgcn_sched_barrier(0);
   }
 
 #pragma unroll
@@ -246,6 +317,237 @@ __global__ __launch_bounds__(256) void paged_prefill_kernel(PrefillParams p) {
                                     pack_bf16x2(acc[nt][2][i] * inv, acc[nt][3][i] * inv)));
         }
       }
+    }
+  }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// LDS-shared variant (head_dim 128): 8 waves x 48 rows = 384 rows per workgroup.  Each 32-key
+// K tile and V tile is fetched from HBM/L2 once per workgroup (one 16-byte piece per thread),
+// staged row-major in LDS with a 272-byte pitch (conflict-free for both read patterns), double
+// buffered with one barrier per tile; the waves read their MFMA operands from LDS.  The tile for
+// step t+1 is in flight in registers while step t computes.
+// ---------------------------------------------------------------------------------------------
+constexpr int kLdsPitch = 272;   // bytes per staged row (256 + 16 padding)
+constexpr int kLdsTile = 32;     // keys per staged tile
+
+template <int NQ>
+__global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams p) {
+  constexpr int HD = 128, KS = 4, DV = 8, NT = 2, WAVES = 8;
+  __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kLdsTile * kLdsPitch];
+  __shared__ __attribute__((aligned(16))) uint8_t Vs[2][kLdsTile * kLdsPitch];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int m16 = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y;
+  const int G = p.G;
+  const int BQ = (16 * NQ) >> p.g_shift;  // query tokens per wave
+  const int SBQ = WAVES * BQ;             // query tokens per workgroup
+
+  if (blockIdx.x == 0) {
+    const int tq = p.cu_q[p.R];
+    const int per_row = G * HD;
+    for (int64_t i = (int64_t)tid * 8; i < (int64_t)(p.T - tq) * per_row; i += 512 * 8) {
+      const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
+      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
+    }
+  }
+
+  const int sb = blockIdx.x;
+  int lo = 0, hi = p.R - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (p.cu_q[mid] / SBQ + mid <= sb) lo = mid; else hi = mid - 1;
+  }
+  const int r = lo;
+  const int q_begin = p.cu_q[r];
+  const int Lq = p.cu_q[r + 1] - q_begin;
+  const int q0_wg = (sb - (q_begin / SBQ + r)) * SBQ;
+  // Everything up to here is uniform over the workgroup: nobody is left behind at a barrier.
+  if (q0_wg >= Lq) return;
+  if (p.skip_single && Lq == 1) return;
+  const int Lk = p.lens[r];
+  const int shift = Lk - Lq;
+  const int last = Lk - 1;
+  const int kend_wg = min(Lk, shift + min(q0_wg + SBQ, Lq));  // keys some row of the workgroup sees
+
+  const int q0 = q0_wg + wave * BQ;
+  const int nq = max(0, min(BQ, Lq - q0));      // valid query tokens of this wave (may be 0)
+  const int kend = nq > 0 ? min(Lk, shift + q0 + nq) : 0;
+  const int ntiles = (nq * G + 15) >> 4;
+
+  uint4 qf[NQ][KS];
+  int qpos[NQ];
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    const int n = 16 * nt + m16;
+    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const bool valid = qi < nq;
+    qpos[nt] = valid ? shift + q0 + qi : last;
+    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      qf[nt][kk] = valid ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
+  }
+
+  float m_run[NQ], l_run[NQ];
+  f32x4_t acc[NQ][DV];
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    m_run[nt] = -INFINITY;
+    l_run[nt] = 0.f;
+#pragma unroll
+    for (int e = 0; e < DV; ++e) acc[nt][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  if (kend_wg > 0) {
+    const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * 2;
+    const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * 2;
+    const int64_t chunk_bytes = p.kv_sc * 2;
+    const int tok_bytes = p.kv_st * 2;
+    // loader role of this thread: one 16-byte piece of one key row, for K and for V
+    const int lkey = tid >> 4, lpiece = tid & 15;
+    const int lds_off = lkey * kLdsPitch + lpiece * 16;
+    uint4 kreg, vreg;
+    auto gload = [&](int T) {
+      const int tok = min(T + lkey, last);
+      const int ci = (int)(((uint64_t)(uint32_t)tok * p.chunk_magic) >> 40);
+      const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
+      const int64_t off = (int64_t)pc * chunk_bytes + (int64_t)(tok - ci * p.chunk) * tok_bytes + lpiece * 16;
+      kreg = ld16(kbase + off);
+      vreg = ld16(vbase + off);
+    };
+    auto lstore = [&](int buf) {
+      *reinterpret_cast<uint4*>(&Ks[buf][lds_off]) = kreg;
+      *reinterpret_cast<uint4*>(&Vs[buf][lds_off]) = vreg;
+    };
+    const int full_until = shift + q0;
+    const float scale = p.scale_log2;
+
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    int buf = 0;
+    for (int T = 0; T < kend_wg; T += kLdsTile, buf ^= 1) {
+      const bool more = T + kLdsTile < kend_wg;  // workgroup-uniform
+      if (more) gload(T + kLdsTile);
+      if (T < kend) {  // wave-uniform: this wave still has visible keys in the tile
+        const uint8_t* ks = Ks[buf];
+        const uint8_t* vs = Vs[buf];
+        // ---- S^T = K Q^T ---------------------------------------------------------------
+        f32x4_t s[NQ][NT];
+#pragma unroll
+        for (int u = 0; u < NT; ++u) {
+          uint4 kf[KS];
+#pragma unroll
+          for (int kk = 0; kk < KS; ++kk)
+            kf[kk] = *reinterpret_cast<const uint4*>(ks + (16 * u + m16) * kLdsPitch + (32 * kk + 8 * g) * 2);
+#pragma unroll
+          for (int nt = 0; nt < NQ; ++nt) {
+            if (nt >= ntiles) break;
+            f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32(kf[kk], qf[nt][kk], sacc);
+            s[nt][u] = sacc;
+          }
+        }
+        // ---- online softmax ---------------------------------------------------------------
+        const bool need_mask = T + kLdsTile - 1 > full_until;
+        uint2 pf[NQ][NT];
+#pragma unroll
+        for (int nt = 0; nt < NQ; ++nt) {
+          if (nt >= ntiles) break;
+          float tmax = -INFINITY;
+#pragma unroll
+          for (int u = 0; u < NT; ++u) {
+            if (need_mask) {
+              const int tok0 = T + 16 * u + 4 * g;
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (tok0 + i > qpos[nt]) s[nt][u][i] = -INFINITY;
+            }
+            tmax = fmaxf(fmaxf(fmaxf(s[nt][u][0], s[nt][u][1]), fmaxf(s[nt][u][2], s[nt][u][3])), tmax);
+          }
+          tmax = fmaxf(tmax, xor16(tmax));
+          tmax = fmaxf(tmax, xor32(tmax));
+          const float m_raw = fmaxf(m_run[nt], tmax);
+          const float m_use = m_raw == -INFINITY ? 0.f : m_raw;
+          const float alpha = fast_exp2((m_run[nt] - m_use) * scale);
+          const float neg = -m_use * scale;
+          m_run[nt] = m_raw;
+          float psum = 0.f;
+#pragma unroll
+          for (int u = 0; u < NT; ++u) {
+            float pv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              pv[i] = fast_exp2(__builtin_fmaf(s[nt][u][i], scale, neg));
+              psum += pv[i];
+            }
+            pf[nt][u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+          }
+          l_run[nt] = l_run[nt] * alpha + psum;
+          if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+            for (int e = 0; e < DV; ++e) {
+              acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
+            }
+          }
+        }
+        // ---- O^T += V^T P^T (k = 32: both 16-key sub-tiles in one mfma) -------------------
+        uint4 va[4], vb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          va[j] = *reinterpret_cast<const uint4*>(vs + (4 * g + j) * kLdsPitch + 16 * m16);
+          vb[j] = *reinterpret_cast<const uint4*>(vs + (16 + 4 * g + j) * kLdsPitch + 16 * m16);
+        }
+        const uint32_t* a0 = reinterpret_cast<const uint32_t*>(&va[0]);
+        const uint32_t* a1 = reinterpret_cast<const uint32_t*>(&va[1]);
+        const uint32_t* a2 = reinterpret_cast<const uint32_t*>(&va[2]);
+        const uint32_t* a3 = reinterpret_cast<const uint32_t*>(&va[3]);
+        const uint32_t* b0 = reinterpret_cast<const uint32_t*>(&vb[0]);
+        const uint32_t* b1 = reinterpret_cast<const uint32_t*>(&vb[1]);
+        const uint32_t* b2 = reinterpret_cast<const uint32_t*>(&vb[2]);
+        const uint32_t* b3 = reinterpret_cast<const uint32_t*>(&vb[3]);
+#pragma unroll
+        for (int pr = 0; pr < 4; ++pr) {
+          const uint4 lo4 = make_uint4(low_halves(a1[pr], a0[pr]), low_halves(a3[pr], a2[pr]),
+                                       low_halves(b1[pr], b0[pr]), low_halves(b3[pr], b2[pr]));
+          const uint4 hi4 = make_uint4(high_halves(a1[pr], a0[pr]), high_halves(a3[pr], a2[pr]),
+                                       high_halves(b1[pr], b0[pr]), high_halves(b3[pr], b2[pr]));
+#pragma unroll
+          for (int nt = 0; nt < NQ; ++nt) {
+            if (nt >= ntiles) break;
+            const uint4 pp = make_uint4(pf[nt][0].x, pf[nt][0].y, pf[nt][1].x, pf[nt][1].y);
+            acc[nt][2 * pr] = mfma_16x16x32(lo4, pp, acc[nt][2 * pr]);
+            acc[nt][2 * pr + 1] = mfma_16x16x32(hi4, pp, acc[nt][2 * pr + 1]);
+          }
+        }
+      }
+      if (more) lstore(buf ^ 1);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue (rows of a request without keys get zeros: l_tot == 0) -------------------
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    float l_tot = l_run[nt] + xor16(l_run[nt]);
+    l_tot += xor32(l_tot);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int n = 16 * nt + m16;
+    const int qi = n >> p.g_shift, u = n & (G - 1);
+    if (qi < nq) {
+      uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        st16(o + 8 * i, make_uint4(pack_bf16x2(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
+                                   pack_bf16x2(acc[nt][2][i] * inv, acc[nt][3][i] * inv),
+                                   pack_bf16x2(acc[nt][4][i] * inv, acc[nt][5][i] * inv),
+                                   pack_bf16x2(acc[nt][6][i] * inv, acc[nt][7][i] * inv)));
     }
   }
 }
@@ -301,26 +603,46 @@ extern "C" int mi_paged_prefill_attention(
   p.g_shift = 0;
   while ((1 << p.g_shift) < G) ++p.g_shift;
   p.chunk = chunk_tokens;
-  p.chunk_shift = -1;
-  if (!(chunk_tokens & (chunk_tokens - 1))) {
-    p.chunk_shift = 0;
-    while ((1 << p.chunk_shift) < chunk_tokens) ++p.chunk_shift;
-  }
+  p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   // With a workspace, one-row requests go through the bandwidth-optimised decode kernels.
   p.skip_single = workspace != nullptr;
 
-  const int sbq = 4 * (64 / G);
-  dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(256);
   hipStream_t st = (hipStream_t)stream;
-  const int nt = mi_tuning().prefill_tile_subtiles;
-  if (head_dim == 128) {
-    if (nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<128, 1>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((paged_prefill_kernel<128, 2>), grid, block, 0, st, p);
-  } else {
-    if (nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<64, 1>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((paged_prefill_kernel<64, 2>), grid, block, 0, st, p);
+  if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
+  const int lds_tiles = mi_tuning().prefill_lds_row_tiles;  // 0 = register-only kernel
+  if (head_dim == 128 && lds_tiles > 0) {
+    const int rows = 8 * 16 * (lds_tiles == 2 ? 2 : 3);
+    const int sbq_lds = rows / G;
+    dim3 lgrid((T + sbq_lds - 1) / sbq_lds + R, Hkv);
+    if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2>), lgrid, dim3(512), 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_lds_kernel<3>), lgrid, dim3(512), 0, st, p);
+    int rc0 = mi_check_launch("mi_paged_prefill_attention");
+    if (rc0 != MI_OK || !p.skip_single) return rc0;
+    return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
+                               kv_stride_head, block_table, bt_stride, kv_lens, cu_seqlens_q, out, o_stride_tok,
+                               o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
+                               split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
   }
+  const int nq = mi_tuning().prefill_row_tiles == 4 ? 4 : 2;
+  const int sbq = 256 / G;  // query tokens per workgroup (256 rows)
+  dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * (16 / nq));
+  const int nt = mi_tuning().prefill_tile_subtiles;
+#define MI_LAUNCH_PREFILL(HD_, NT_)                                                                        \
+  do {                                                                                                     \
+    if (nq == 4) hipLaunchKernelGGL((paged_prefill_kernel<HD_, NT_, 4>), grid, block, 0, st, p);           \
+    else hipLaunchKernelGGL((paged_prefill_kernel<HD_, NT_, 2>), grid, block, 0, st, p);                   \
+  } while (0)
+  if (head_dim == 128) {
+    if (nt == 1) MI_LAUNCH_PREFILL(128, 1);
+    else if (nt == 4) MI_LAUNCH_PREFILL(128, 4);
+    else MI_LAUNCH_PREFILL(128, 2);
+  } else {
+    if (nt == 1) MI_LAUNCH_PREFILL(64, 1);
+    else if (nt == 4) MI_LAUNCH_PREFILL(64, 4);
+    else MI_LAUNCH_PREFILL(64, 2);
+  }
+#undef MI_LAUNCH_PREFILL
   int rc = mi_check_launch("mi_paged_prefill_attention");
   if (rc != MI_OK || !p.skip_single) return rc;
   return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,

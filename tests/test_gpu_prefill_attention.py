@@ -25,12 +25,12 @@ def test_mixed_prefill_and_decode(mi, dev, Hq, Hkv, d):
     _check(mi, q, kc, vc, cu_q, lens, bt)
 
 
-@pytest.mark.parametrize("subtiles", [1, 2])
-def test_ragged_prefill_lengths(mi, dev, subtiles):
+@pytest.mark.parametrize("subtiles,lds_rows", [(1, 0), (2, 0), (2, 2), (2, 3)])
+def test_ragged_prefill_lengths(mi, dev, subtiles, lds_rows):
     """New-token counts around every block boundary, with and without existing context."""
     torch.manual_seed(0)
-    q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1]
-    ctx = [0, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0]
+    q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 500]
+    ctx = [0, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0, 40, 7]
     Hq, Hkv, d, chunk = 32, 8, 128, 32
     kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
     cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
@@ -41,10 +41,12 @@ def test_ragged_prefill_lengths(mi, dev, subtiles):
     kc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
     vc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
     mi.ops.set_tuning("prefill_tile_subtiles", subtiles)
+    mi.ops.set_tuning("prefill_lds_row_tiles", lds_rows)  # 0 = register-only kernel
     try:
         _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
     finally:
         mi.ops.set_tuning("prefill_tile_subtiles", 2)
+        mi.ops.set_tuning("prefill_lds_row_tiles", 3)
 
 
 def test_prefill_equals_decode_for_single_tokens(mi, dev):
