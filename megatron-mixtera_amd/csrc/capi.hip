@@ -25,8 +25,8 @@ static int env_int(const char* name, int dflt) {
 }
 
 MiTuning& mi_tuning() {
-  static MiTuning t = {env_int("MI355_DECODE_SUBTILES", 0), env_int("MI355_PREFILL_SUBTILES", 2),
-                      env_int("MI355_PREFILL_LDS_ROW_TILES", 3), env_int("MI355_PREFILL_ROW_TILES", 2),
+  static MiTuning t = {env_int("MI355_DECODE_SUBTILES", 0), env_int("MI355_PREFILL_SUBTILES", 4),
+                      env_int("MI355_PREFILL_LDS_ROW_TILES", 2), env_int("MI355_PREFILL_ROW_TILES", 2),
                       env_int("MI355_DECODE_MIN_WAVES", 3),
                       env_int("MI355_DECODE_WGS_PER_CU", 1), env_int("MI355_DECODE_GRID", 0),
                       env_int("MI355_DECODE_WAVES_PER_BLOCK", 8)};

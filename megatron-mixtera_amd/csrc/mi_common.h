@@ -102,6 +102,14 @@ static __device__ __forceinline__ uint2 ld8_stream(const void* p) {
 static __device__ __forceinline__ void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
 static __device__ __forceinline__ void st8(void* p, uint2 v) { *reinterpret_cast<uint2*>(p) = v; }
 
+// 16-byte LDS read that stays one ds_read_b128: the empty asm uses the whole vector, which keeps
+// the compiler from narrowing the load into strided dword reads (those conflict on the banks).
+static __device__ __forceinline__ uint4 lds_ld16(const void* p) {
+  u32x4_t v = *reinterpret_cast<const u32x4_t*>(p);
+  asm volatile("" : "+v"(v));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // OCP e4m3fn byte pairs -> fp32 (gfx950 converts OCP formats natively).
 static __device__ __forceinline__ f32x2_t fp8x2_lo_to_f32(uint32_t w) {
   return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);

@@ -330,11 +330,14 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 // step t+1 is in flight in registers while step t computes.
 // ---------------------------------------------------------------------------------------------
 constexpr int kLdsPitch = 272;   // bytes per staged row (256 + 16 padding)
-constexpr int kLdsTile = 32;     // keys per staged tile
 
-template <int NQ>
+// NQ = 16-row tiles per wave, NT = 16-key sub-tiles per staged tile (2 or 4).
+template <int NQ, int NT>
 __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams p) {
-  constexpr int HD = 128, KS = 4, DV = 8, NT = 2, WAVES = 8;
+  constexpr int HD = 128, KS = 4, DV = 8, WAVES = 8;
+  constexpr int kLdsTile = 16 * NT;  // keys per staged tile
+  constexpr int LP = NT / 2;         // loader passes (512 threads fetch 32 rows per pass)
+  static_assert(NT == 2 || NT == 4, "staged tile of 32 or 64 keys");
   __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kLdsTile * kLdsPitch];
   __shared__ __attribute__((aligned(16))) uint8_t Vs[2][kLdsTile * kLdsPitch];
 
@@ -411,18 +414,24 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
     // loader role of this thread: one 16-byte piece of one key row, for K and for V
     const int lkey = tid >> 4, lpiece = tid & 15;
     const int lds_off = lkey * kLdsPitch + lpiece * 16;
-    uint4 kreg, vreg;
+    uint4 kreg[LP], vreg[LP];
     auto gload = [&](int T) {
-      const int tok = min(T + lkey, last);
-      const int ci = (int)(((uint64_t)(uint32_t)tok * p.chunk_magic) >> 40);
-      const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
-      const int64_t off = (int64_t)pc * chunk_bytes + (int64_t)(tok - ci * p.chunk) * tok_bytes + lpiece * 16;
-      kreg = ld16(kbase + off);
-      vreg = ld16(vbase + off);
+#pragma unroll
+      for (int lp = 0; lp < LP; ++lp) {
+        const int tok = min(T + 32 * lp + lkey, last);
+        const int ci = (int)(((uint64_t)(uint32_t)tok * p.chunk_magic) >> 40);
+        const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
+        const int64_t off = (int64_t)pc * chunk_bytes + (int64_t)(tok - ci * p.chunk) * tok_bytes + lpiece * 16;
+        kreg[lp] = ld16(kbase + off);
+        vreg[lp] = ld16(vbase + off);
+      }
     };
     auto lstore = [&](int buf) {
-      *reinterpret_cast<uint4*>(&Ks[buf][lds_off]) = kreg;
-      *reinterpret_cast<uint4*>(&Vs[buf][lds_off]) = vreg;
+#pragma unroll
+      for (int lp = 0; lp < LP; ++lp) {
+        *reinterpret_cast<uint4*>(&Ks[buf][lds_off + 32 * lp * kLdsPitch]) = kreg[lp];
+        *reinterpret_cast<uint4*>(&Vs[buf][lds_off + 32 * lp * kLdsPitch]) = vreg[lp];
+      }
     };
     const int full_until = shift + q0;
     const float scale = p.scale_log2;
@@ -444,7 +453,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
           uint4 kf[KS];
 #pragma unroll
           for (int kk = 0; kk < KS; ++kk)
-            kf[kk] = *reinterpret_cast<const uint4*>(ks + (16 * u + m16) * kLdsPitch + (32 * kk + 8 * g) * 2);
+            kf[kk] = lds_ld16(ks + (16 * u + m16) * kLdsPitch + (32 * kk + 8 * g) * 2);
 #pragma unroll
           for (int nt = 0; nt < NQ; ++nt) {
             if (nt >= ntiles) break;
@@ -497,33 +506,36 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
             }
           }
         }
-        // ---- O^T += V^T P^T (k = 32: both 16-key sub-tiles in one mfma) -------------------
-        uint4 va[4], vb[4];
+        // ---- O^T += V^T P^T (k = 32: two 16-key sub-tiles per mfma) ------------------------
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          va[j] = *reinterpret_cast<const uint4*>(vs + (4 * g + j) * kLdsPitch + 16 * m16);
-          vb[j] = *reinterpret_cast<const uint4*>(vs + (16 + 4 * g + j) * kLdsPitch + 16 * m16);
-        }
-        const uint32_t* a0 = reinterpret_cast<const uint32_t*>(&va[0]);
-        const uint32_t* a1 = reinterpret_cast<const uint32_t*>(&va[1]);
-        const uint32_t* a2 = reinterpret_cast<const uint32_t*>(&va[2]);
-        const uint32_t* a3 = reinterpret_cast<const uint32_t*>(&va[3]);
-        const uint32_t* b0 = reinterpret_cast<const uint32_t*>(&vb[0]);
-        const uint32_t* b1 = reinterpret_cast<const uint32_t*>(&vb[1]);
-        const uint32_t* b2 = reinterpret_cast<const uint32_t*>(&vb[2]);
-        const uint32_t* b3 = reinterpret_cast<const uint32_t*>(&vb[3]);
+        for (int up = 0; up < NT; up += 2) {
+          uint4 va[4], vb[4];
 #pragma unroll
-        for (int pr = 0; pr < 4; ++pr) {
-          const uint4 lo4 = make_uint4(low_halves(a1[pr], a0[pr]), low_halves(a3[pr], a2[pr]),
-                                       low_halves(b1[pr], b0[pr]), low_halves(b3[pr], b2[pr]));
-          const uint4 hi4 = make_uint4(high_halves(a1[pr], a0[pr]), high_halves(a3[pr], a2[pr]),
-                                       high_halves(b1[pr], b0[pr]), high_halves(b3[pr], b2[pr]));
+          for (int j = 0; j < 4; ++j) {
+            va[j] = lds_ld16(vs + (16 * up + 4 * g + j) * kLdsPitch + 16 * m16);
+            vb[j] = lds_ld16(vs + (16 * up + 16 + 4 * g + j) * kLdsPitch + 16 * m16);
+          }
+          const uint32_t* a0 = reinterpret_cast<const uint32_t*>(&va[0]);
+          const uint32_t* a1 = reinterpret_cast<const uint32_t*>(&va[1]);
+          const uint32_t* a2 = reinterpret_cast<const uint32_t*>(&va[2]);
+          const uint32_t* a3 = reinterpret_cast<const uint32_t*>(&va[3]);
+          const uint32_t* b0 = reinterpret_cast<const uint32_t*>(&vb[0]);
+          const uint32_t* b1 = reinterpret_cast<const uint32_t*>(&vb[1]);
+          const uint32_t* b2 = reinterpret_cast<const uint32_t*>(&vb[2]);
+          const uint32_t* b3 = reinterpret_cast<const uint32_t*>(&vb[3]);
 #pragma unroll
-          for (int nt = 0; nt < NQ; ++nt) {
-            if (nt >= ntiles) break;
-            const uint4 pp = make_uint4(pf[nt][0].x, pf[nt][0].y, pf[nt][1].x, pf[nt][1].y);
-            acc[nt][2 * pr] = mfma_16x16x32(lo4, pp, acc[nt][2 * pr]);
-            acc[nt][2 * pr + 1] = mfma_16x16x32(hi4, pp, acc[nt][2 * pr + 1]);
+          for (int pr = 0; pr < 4; ++pr) {
+            const uint4 lo4 = make_uint4(low_halves(a1[pr], a0[pr]), low_halves(a3[pr], a2[pr]),
+                                         low_halves(b1[pr], b0[pr]), low_halves(b3[pr], b2[pr]));
+            const uint4 hi4 = make_uint4(high_halves(a1[pr], a0[pr]), high_halves(a3[pr], a2[pr]),
+                                         high_halves(b1[pr], b0[pr]), high_halves(b3[pr], b2[pr]));
+#pragma unroll
+            for (int nt = 0; nt < NQ; ++nt) {
+              if (nt >= ntiles) break;
+              const uint4 pp = make_uint4(pf[nt][up].x, pf[nt][up].y, pf[nt][up + 1].x, pf[nt][up + 1].y);
+              acc[nt][2 * pr] = mfma_16x16x32(lo4, pp, acc[nt][2 * pr]);
+              acc[nt][2 * pr + 1] = mfma_16x16x32(hi4, pp, acc[nt][2 * pr + 1]);
+            }
           }
         }
       }
@@ -615,8 +627,11 @@ extern "C" int mi_paged_prefill_attention(
     const int rows = 8 * 16 * (lds_tiles == 2 ? 2 : 3);
     const int sbq_lds = rows / G;
     dim3 lgrid((T + sbq_lds - 1) / sbq_lds + R, Hkv);
-    if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2>), lgrid, dim3(512), 0, st, p);
-    else hipLaunchKernelGGL((paged_prefill_lds_kernel<3>), lgrid, dim3(512), 0, st, p);
+    const bool wide = mi_tuning().prefill_tile_subtiles == 4;  // 64-key staged tiles
+    if (lds_tiles == 2 && wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 4>), lgrid, dim3(512), 0, st, p);
+    else if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 2>), lgrid, dim3(512), 0, st, p);
+    else if (wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 4>), lgrid, dim3(512), 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);
     int rc0 = mi_check_launch("mi_paged_prefill_attention");
     if (rc0 != MI_OK || !p.skip_single) return rc0;
     return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
@@ -627,7 +642,8 @@ extern "C" int mi_paged_prefill_attention(
   const int nq = mi_tuning().prefill_row_tiles == 4 ? 4 : 2;
   const int sbq = 256 / G;  // query tokens per workgroup (256 rows)
   dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * (16 / nq));
-  const int nt = mi_tuning().prefill_tile_subtiles;
+  // register-only kernel (head_dim 64, or LDS variant switched off): 16 or 32 keys per iteration
+  const int nt = mi_tuning().prefill_tile_subtiles == 1 ? 1 : 2;
 #define MI_LAUNCH_PREFILL(HD_, NT_)                                                                        \
   do {                                                                                                     \
     if (nq == 4) hipLaunchKernelGGL((paged_prefill_kernel<HD_, NT_, 4>), grid, block, 0, st, p);           \
@@ -635,11 +651,9 @@ extern "C" int mi_paged_prefill_attention(
   } while (0)
   if (head_dim == 128) {
     if (nt == 1) MI_LAUNCH_PREFILL(128, 1);
-    else if (nt == 4) MI_LAUNCH_PREFILL(128, 4);
     else MI_LAUNCH_PREFILL(128, 2);
   } else {
     if (nt == 1) MI_LAUNCH_PREFILL(64, 1);
-    else if (nt == 4) MI_LAUNCH_PREFILL(64, 4);
     else MI_LAUNCH_PREFILL(64, 2);
   }
 #undef MI_LAUNCH_PREFILL

@@ -25,7 +25,7 @@ def test_mixed_prefill_and_decode(mi, dev, Hq, Hkv, d):
     _check(mi, q, kc, vc, cu_q, lens, bt)
 
 
-@pytest.mark.parametrize("subtiles,lds_rows", [(1, 0), (2, 0), (2, 2), (2, 3)])
+@pytest.mark.parametrize("subtiles,lds_rows", [(1, 0), (2, 0), (2, 2), (2, 3), (4, 2), (4, 3)])
 def test_ragged_prefill_lengths(mi, dev, subtiles, lds_rows):
     """New-token counts around every block boundary, with and without existing context."""
     torch.manual_seed(0)
@@ -45,8 +45,8 @@ def test_ragged_prefill_lengths(mi, dev, subtiles, lds_rows):
     try:
         _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
     finally:
-        mi.ops.set_tuning("prefill_tile_subtiles", 2)
-        mi.ops.set_tuning("prefill_lds_row_tiles", 3)
+        mi.ops.set_tuning("prefill_tile_subtiles", 4)
+        mi.ops.set_tuning("prefill_lds_row_tiles", 2)
 
 
 def test_prefill_equals_decode_for_single_tokens(mi, dev):
