@@ -27,6 +27,7 @@ if str(ROOT) not in sys.path:
     sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 
 # HBM bytes per launch of the streaming kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this same script, each counter scaled by what it reads for a plain 1 GiB device copy
@@ -40,7 +41,8 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3_decode", "cfg4", "cfg5"])
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5"],
+                    help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch")
     ap.add_argument("--split-tokens", type=int, default=0)
     ap.add_argument("--subtiles", type=int, default=0, help="16-token sub-tiles per loop iteration (1, 2 or 4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -87,6 +89,81 @@ def cpu_baseline(case, cfg, sample_requests: int):
                       f"checker (oracle/paged_attention.py), median of 3 passes after 1 warm-up, {t * 1e3:.1f} ms/pass"}
 
 
+def run_mixed_batch(args, mi, lib, torch, dev):
+    """cfg3: 8 prefill requests x 2048 new tokens over U[0,4096] cached tokens + 120 decode requests
+    with U[512,8192] tokens, one varlen call.  Step = fused RMSNorm+RoPE+append of all new tokens,
+    then paged varlen attention (tile kernel for the prefill requests, streaming + merge kernels for
+    the one-token requests).  Two roofline objects: MFMA for the tile kernel, HBM for the stream."""
+    from oracle import rope_norm as orn
+
+    Hq, Hkv, d, chunk = 32, 8, 128, 256
+    q, kc, vc, cu_q, lens, bt = mi.synthetic.make_prefill_case(
+        dev, n_prefill=8, new_tokens=2048, ctx_lo=0, ctx_hi=4096, n_decode=120, dec_lo=512, dec_hi=8192,
+        Hq=Hq, Hkv=Hkv, d=d, chunk=chunk, seed=1003, on_device_rng=True)
+    T = q.size(0)
+    gen = torch.Generator().manual_seed(2003)
+    k_new = torch.randn(T, Hkv, d, generator=gen).bfloat16().to(dev)
+    v_new = torch.randn(T, Hkv, d, generator=gen).bfloat16().to(dev)
+    qw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16().to(dev)
+    kw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16().to(dev)
+    pos, tok_chunk, tok_local = mi.synthetic.prefill_token_rows(cu_q, lens, bt, chunk)
+    max_len = int(lens.max())
+    table = orn.rotary_table(max_len + 1, d, base=500000.0).to(dev)
+    q_rot = torch.empty_like(q)
+    out = torch.empty_like(q)
+
+    def step():
+        mi.ops.norm_rope_append(q, k_new, query_out=q_rot, value=v_new, q_weight=qw, k_weight=kw, eps=1e-5,
+                                norm="rms", rotary_emb=table, q_positions=pos, k_positions=pos, k_cache=kc,
+                                v_cache=vc, token_to_chunk_idx=tok_chunk, token_to_local_pos=tok_local)
+        mi.ops.paged_prefill_attention(q_rot, kc, vc, cu_q, lens, bt, max_kv_len=max_len, out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    lib.mi_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    buf = (ctypes.c_float * (2 * args.steps))()
+    n_ev = lib.mi_profile_collect(buf, 2 * args.steps)
+    lib.mi_profile_enable(0)
+    tile_ms = sum(buf[i] for i in range(0, n_ev, 2)) / max(1, n_ev // 2)
+    stream_ms = sum(buf[i] for i in range(1, n_ev, 2)) / max(1, n_ev // 2)
+
+    lq = (cu_q[1:] - cu_q[:-1]).cpu().long()
+    lk = lens.cpu().long()
+    pre = lq > 1
+    flops = 4 * Hq * d * int((lq[pre] * (lk - lq)[pre] + lq[pre] * (lq[pre] + 1) // 2).sum())
+    from oracle import paged_attention as oa
+    dec_bytes = oa.decode_attention_bytes(lk[~pre].tolist(), Hq, Hkv, d, chunk)
+    pre_kv_bytes = int(lk[pre].sum()) * Hkv * d * 2 * 2 + int(lq[pre].sum()) * Hq * d * 4
+    ms_per_step = elapsed * 1e3 / args.steps
+    total_bytes = dec_bytes + pre_kv_bytes
+    result = {
+        "metric": "paged_decode_attention_hbm_GBps",
+        "value": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 (fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "cfg3: mixed batch, 8 x 2048-token prefill over U[0,4096] + 120 decode U[512,8192], "
+                               "32/8 heads d128 chunk 256; step = fused RMSNorm+RoPE+append then paged varlen attention",
+                   "new_tokens": T, "requests": int(lens.numel()), "algorithmic_bytes_per_step": total_bytes,
+                   "prefill_flops_per_step": flops},
+        "roofline": {"bound": "mfma", "kernel": "paged_prefill_lds_kernel", "achieved": round(flops / tile_ms / 1e9, 1),
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(flops / tile_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "kernel_ms": round(tile_ms, 5),
+                     "traffic": None},
+        "roofline_decode_part": {"bound": "hbm", "kernel": "paged_decode_stream_kernel",
+                                 "achieved": round(dec_bytes / stream_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                                 "unit": "GB/s", "frac": round(dec_bytes / stream_ms / 1e6 / HBM_PEAK_GBPS, 4),
+                                 "kernel_ms": round(stream_ms, 5), "traffic": None},
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -109,6 +186,10 @@ def main():
     torch.cuda.set_device(dev)
     if args.subtiles:
         mi.ops.set_tuning("decode_tile_subtiles", args.subtiles)
+
+    if args.workload == "cfg3":
+        run_mixed_batch(args, mi, lib, torch, dev)
+        return
 
     cfg = mi.synthetic.CONFIGS[args.workload]
     case = mi.synthetic.make_decode_case(cfg, dev, on_device_rng=True)

@@ -52,8 +52,10 @@ const char* mi_last_error(void);
 int mi_set_tuning(const char* name, int32_t value);
 
 /*
- * Kernel timing.  mi_profile_enable(1) makes mi_paged_decode_attention bracket its
- * KV-streaming kernel with HIP events on the caller's stream; mi_profile_collect waits for
+ * Kernel timing.  mi_profile_enable(1) makes the attention entry points bracket their main
+ * kernel (decode: the KV-streaming kernel; prefill, head_dim 128: the tile kernel, followed by
+ * a second pair for the decode kernel of a mixed batch) with HIP events on the caller's
+ * stream; mi_profile_collect waits for
  * the recorded pairs, writes their durations (milliseconds, HOST pointer) and returns how
  * many there were.  Keep it off while capturing a graph.
  */

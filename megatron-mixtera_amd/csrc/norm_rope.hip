@@ -18,9 +18,9 @@
 // whole expression is evaluated in fp32 and rounded once.
 //
 // grid = (tokens, groups of head vectors); a workgroup of 4 waves handles 4 (d = 128) or 8
-// (d = 64) head vectors of one token, each by d/2 lanes, lane i owning elements i and i + d/2.  The normalised vector goes through a
-// few hundred bytes of LDS so that any rotary pairing (half-split, interleaved,
-// partial rotary width) reads its partner from there.
+// (d = 64) head vectors of one token per pass, each by d/2 lanes, lane i owning elements i and
+// i + d/2.  The normalised vector goes through a few hundred bytes of LDS so that any rotary
+// pairing (half-split, interleaved, partial rotary width) reads its partner from there.
 #include "mi_common.h"
 #include "mi_capi_internal.h"
 
@@ -86,8 +86,51 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
     }
   }
 
-  {
-    const int vec = blockIdx.y * VPB + slot;
+  // cos / sin of this lane's two elements depend only on the token position, not on the head:
+  // evaluate them once (twice if query and key positions differ) and reuse them for every head.
+  float cs[2][2][2] = {};  // [q|k][element][cos|sin]
+  int partner[2] = {0, 0};
+  float sign[2] = {0.f, 0.f};
+  bool rotate[2] = {false, false};
+  if (p.emb) {
+    const int64_t qp = p.q_pos ? p.q_pos[t] : 0;
+    const int64_t kp = p.k_pos ? p.k_pos[t] : qp;
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const int e = i + w * LPV;
+      rotate[w] = e < p.rot;
+      if (p.interleaved) {
+        partner[w] = e ^ 1;
+        sign[w] = (e & 1) ? 1.f : -1.f;
+      } else {
+        const int half = p.rot >> 1;
+        partner[w] = e < half ? e + half : e - half;
+        sign[w] = e < half ? -1.f : 1.f;
+      }
+      if (rotate[w]) {
+#pragma unroll
+        for (int which = 0; which < 2; ++which) {
+          if (which == 1 && kp == qp && p.Hq > 0) {
+            cs[1][w][0] = cs[0][w][0];
+            cs[1][w][1] = cs[0][w][1];
+            continue;
+          }
+          if ((which == 0 && p.Hq == 0) || (which == 1 && p.Hkv == 0)) continue;
+          const float a = p.emb[(which ? kp : qp) * p.emb_stride + e];
+          float c = cosf(a) * p.mscale, sn = sinf(a) * p.mscale;
+          if (faithful) {
+            c = round_bf16(c);
+            sn = round_bf16(sn);
+          }
+          cs[which][w][0] = c;
+          cs[which][w][1] = sn;
+        }
+      }
+    }
+  }
+
+  for (int vec0 = blockIdx.y * VPB; vec0 < nvec; vec0 += gridDim.y * VPB) {
+    const int vec = vec0 + slot;
     const bool active = vec < nvec;
     const bool is_q = vec < p.Hq;
     const int head = is_q ? vec : vec - p.Hq;
@@ -121,34 +164,13 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
       lds[slot][i] = y0;
       lds[slot][i + LPV] = y1;
       __syncthreads();
-      const int64_t pos = active ? (is_q ? p.q_pos[t] : p.k_pos[t]) : 0;
-      const float* ang = p.emb + pos * p.emb_stride;
 #pragma unroll
       for (int w = 0; w < 2; ++w) {
-        const int e = i + w * LPV;
-        const float y = w ? y1 : y0;
-        if (active && e < p.rot) {
-          int partner;
-          float sign;
-          if (p.interleaved) {
-            partner = e ^ 1;
-            sign = (e & 1) ? 1.f : -1.f;
-          } else {
-            const int half = p.rot >> 1;
-            partner = e < half ? e + half : e - half;
-            sign = e < half ? -1.f : 1.f;
-          }
-          const float a = ang[e];
-          float c = cosf(a) * p.mscale, s = sinf(a) * p.mscale;
-          const float yp = lds[slot][partner] * sign;
-          float out;
-          if (faithful) {
-            c = round_bf16(c);
-            s = round_bf16(s);
-            out = round_bf16(y * c) + round_bf16(yp * s);
-          } else {
-            out = y * c + yp * s;
-          }
+        if (active && rotate[w]) {
+          const float y = w ? y1 : y0;
+          const float c = cs[is_q ? 0 : 1][w][0], sn = cs[is_q ? 0 : 1][w][1];
+          const float yp = lds[slot][partner[w]] * sign[w];
+          const float out = faithful ? round_bf16(y * c) + round_bf16(yp * sn) : y * c + yp * sn;
           if (w) o1 = out; else o0 = out;
         }
       }
@@ -240,9 +262,13 @@ extern "C" int mi_norm_rope_append(
   p.norm = norm_kind; p.interleaved = rotary_interleaved; p.faithful = faithful_rounding;
   p.eps = eps; p.mscale = mscale;
   hipStream_t st = (hipStream_t)stream;
+  // Few tokens (decode): spread the heads of a token over several workgroups for latency.
+  // Many tokens (prefill): one workgroup per token loops over the heads and reuses cos / sin.
   const int vpb = head_dim == 128 ? 4 : 8;
-  dim3 grid(T, (Hq + Hkv + vpb - 1) / vpb);
-  if (grid.y > 65535) return mi_fail(MI_ERR_SHAPE, "mi_norm_rope_append: too many heads");
+  const int passes = (Hq + Hkv + vpb - 1) / vpb;
+  int gy = (2048 + T - 1) / T;
+  gy = gy < 1 ? 1 : (gy > passes ? passes : gy);
+  dim3 grid(T, gy);
   if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), grid, dim3(256), 0, st, p);
   else hipLaunchKernelGGL((norm_rope_append_kernel<64>), grid, dim3(256), 0, st, p);
   return mi_check_launch("mi_norm_rope_append");

@@ -628,10 +628,13 @@ extern "C" int mi_paged_prefill_attention(
     const int sbq_lds = rows / G;
     dim3 lgrid((T + sbq_lds - 1) / sbq_lds + R, Hkv);
     const bool wide = mi_tuning().prefill_tile_subtiles == 4;  // 64-key staged tiles
+    hipEvent_t ev_a, ev_b;
+    const bool timed = mi_profile_next(&ev_a, &ev_b);
+    if (timed) hipEventRecord(ev_a, st);
     if (lds_tiles == 2 && wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 4>), lgrid, dim3(512), 0, st, p);
     else if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 2>), lgrid, dim3(512), 0, st, p);
-    else if (wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 4>), lgrid, dim3(512), 0, st, p);
-    else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);  // (48 rows: 32-key tiles only)
+    if (timed) hipEventRecord(ev_b, st);
     int rc0 = mi_check_launch("mi_paged_prefill_attention");
     if (rc0 != MI_OK || !p.skip_single) return rc0;
     return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,

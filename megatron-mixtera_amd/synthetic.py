@@ -151,3 +151,16 @@ def make_prefill_case(device, *, n_prefill: int, new_tokens: int, ctx_lo: int, c
         k_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16), gen).to(device)
         v_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16), gen).to(device)
     return q.to(device), k_cache, v_cache, cu_q.to(device), kv_lens.to(device), table.to(device)
+
+
+def prefill_token_rows(cu_seqlens_q: Tensor, kv_lens: Tensor, block_table: Tensor, chunk: int):
+    """Per-token rows of a mixed batch, as the context would hold them: position in the request,
+    physical chunk id and position inside the chunk of every new token (int64, on the inputs' device).
+    Token i of request r (Lq new tokens over Lk - Lq cached ones) sits at position Lk - Lq + i."""
+    cu = cu_seqlens_q.long()
+    lq = cu[1:] - cu[:-1]
+    T = int(cu[-1])
+    req = torch.repeat_interleave(torch.arange(lq.numel(), device=cu.device), lq)
+    pos = torch.arange(T, device=cu.device) - cu[req] + (kv_lens.long() - lq)[req]
+    chunk_idx = block_table.long()[req, pos // chunk]
+    return pos.contiguous(), chunk_idx.contiguous(), (pos % chunk).contiguous()
