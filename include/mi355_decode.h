@@ -196,6 +196,56 @@ int mi_norm_rope_append(const void* q, int64_t q_stride_tok, void* q_out, int64_
                         int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv, int32_t head_dim,
                         int32_t faithful_rounding, void* stream);
 
+/*
+ * DynamicInferenceContext.update_requests as one kernel
+ * (megatron/core/inference/contexts/dynamic_context.py:1033-1298, allocator
+ * dynamic_chunk_allocator.py:56-86): same order of chunk releases, row moves, pauses, LIFO
+ * resumes and per-token row rewrites, so every state tensor ends up as the reference leaves
+ * it.  All state pointers are the context's own tensors (int32 request rows, int64 token rows,
+ * int32 chunk table with `table_stride` elements per row, int32 chunk stack).
+ * `active_requests_mask` int32 [total - paused], `new_tokens` int64 [total - paused];
+ * `paused_tokens` int64 [max_requests] holds the tokens of the paused rows on entry and on exit;
+ * `next_tokens_scratch` int64 [max_requests], `scratch` int32 [4 * max_requests].
+ * Results: `newly_paused_request_ids` int32 [max_requests] and `counters` int32 [8] =
+ * {total_request_count, paused_request_count, active_token_count, chunk_count_avail,
+ *  number of newly paused ids (-1 = none), status (0 ok, 1 mask/count mismatch - nothing was
+ *  changed, 2 no active request left, 3 resumed request not at a chunk start), 1 if the context
+ *  was emptied, 0}; the caller copies `counters` to the host after the call.
+ */
+int mi_update_requests(int32_t* request_ids, int32_t* request_query_lengths,
+                       int32_t* request_output_lengths, int32_t* request_kv_length_offsets,
+                       int32_t* request_kv_chunk_counts, int32_t* request_last_kv_chunk_id,
+                       int32_t* request_last_kv_chunk_offset, int32_t* request_to_kv_chunk_ids,
+                       int64_t table_stride, int32_t max_kv_chunk_count, int64_t* token_to_input_ids,
+                       int64_t* token_to_pos_ids, int64_t* token_to_request_idx,
+                       int64_t* token_to_position_in_request, int64_t* token_to_chunk_idx,
+                       int64_t* token_to_local_position_within_kv_chunk, int32_t* chunk_bag,
+                       const int32_t* active_requests_mask, const int64_t* new_tokens,
+                       int64_t* paused_tokens, int64_t* next_tokens_scratch, int32_t* scratch,
+                       int32_t* newly_paused_request_ids, int32_t* counters,
+                       int32_t total_request_count, int32_t paused_request_count,
+                       int32_t chunk_count_avail, int32_t gtd_chunk_count, int32_t gtd_request_count,
+                       int32_t chunk_size_tokens, int32_t max_requests, void* stream);
+
+/*
+ * The decode-only part of DynamicInferenceContext.initialize_attention_state
+ * (dynamic_context.py:733-741, 747-750, 785-787, 816-818) as one kernel: copies query lengths,
+ * kv lengths (offset + query length) and block-table rows of the active requests into the
+ * fixed-address mirrors, and points the padded token rows at the dummy chunk.  The mirrors'
+ * padded rows must already be zero (reset_attention_state does that).
+ */
+int mi_decode_attention_state(const int32_t* request_kv_length_offsets,
+                              const int32_t* request_query_lengths,
+                              const int32_t* request_to_kv_chunk_ids, int64_t table_stride,
+                              int32_t max_kv_chunk_count, int32_t* query_seq_lengths_out,
+                              int32_t* kv_seq_lengths_out, int32_t* block_table_out,
+                              int64_t block_table_out_stride, int64_t* token_to_chunk_idx,
+                              int64_t* token_to_local_position_within_kv_chunk,
+                              int64_t* token_to_position_in_request, int32_t paused_request_count,
+                              int32_t active_request_count, int32_t active_token_count,
+                              int32_t padded_active_token_count, int32_t dummy_chunk_idx,
+                              void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -117,6 +117,7 @@ class DynamicInferenceContext:
         materialize_only_last_token_logits: bool = True,
         use_cuda_graphs_for_non_decode_steps: bool = True,
         device: Optional[Union[torch.device, str, int]] = None,
+        fused_bookkeeping: Optional[bool] = None,
     ):
         if cache_mla_latent:
             raise NotImplementedError(
@@ -236,6 +237,18 @@ class DynamicInferenceContext:
         self.chunk_allocator = ChunkAllocator(
             chunk_count_total=chunk_count_total, gtd_chunk_count=self.gtd_chunk_count, device=dev)
         self.dummy_chunk_idx = self.chunk_allocator.dummy_chunk_idx
+
+        # ---- on-GPU bookkeeping: update_requests / decode attention state as single kernels ----
+        # (None = use them whenever the state lives on a GPU; the torch op sequence below is the
+        # host-side statement of the same steps and the only one available for device="cpu")
+        self.fused_bookkeeping = (dev.type == "cuda") if fused_bookkeeping is None else bool(fused_bookkeeping)
+        if self.fused_bookkeeping:
+            self._paused_tokens_buf = torch.zeros(self.max_requests, dtype=torch.long, device=dev)
+            self._next_tokens_buf = torch.zeros(self.max_requests, dtype=torch.long, device=dev)
+            self._update_scratch = torch.zeros(4 * self.max_requests, dtype=torch.int32, device=dev)
+            self._newly_paused_buf = torch.zeros(self.max_requests, dtype=torch.int32, device=dev)
+            self._counters = torch.zeros(8, dtype=torch.int32, device=dev)
+            self._counters_host = torch.zeros(8, dtype=torch.int32, pin_memory=True)
 
         self.reset_attention_state()
 
@@ -434,24 +447,31 @@ class DynamicInferenceContext:
         n_active_req = self.total_request_count - self.paused_request_count
         self.padded_active_request_count = padded if (graph_step or decode_only) else n_active_req
 
-        # padded token rows: write into the dummy chunk at position 0
-        pad = slice(self.active_token_count, padded)
-        self.token_to_chunk_idx[pad] = self.dummy_chunk_idx
-        self.token_to_local_position_within_kv_chunk[pad] = 0
-        self.token_to_position_in_request[pad] = 0
-
         act = self._active()
-        q_lens = self.request_query_lengths[act]
-        kv_lens = (self.request_kv_length_offsets + self.request_query_lengths)[act]
+        if self.fused_bookkeeping and (graph_step or decode_only):
+            # one kernel: padded token rows + fixed-address mirrors of lengths and block table
+            ops.decode_attention_state(self, n_active_req, padded)
+        else:
+            # padded token rows: write into the dummy chunk at position 0
+            pad = slice(self.active_token_count, padded)
+            self.token_to_chunk_idx[pad] = self.dummy_chunk_idx
+            self.token_to_local_position_within_kv_chunk[pad] = 0
+            self.token_to_position_in_request[pad] = 0
+
+        fused_mirrors = self.fused_bookkeeping and (graph_step or decode_only)
+        if not fused_mirrors:
+            q_lens = self.request_query_lengths[act]
+            kv_lens = (self.request_kv_length_offsets + self.request_query_lengths)[act]
         R = self.padded_active_request_count
         dev = self.device
 
         if decode_only or graph_step:
-            self.query_seq_lengths_cudagraph_only[:n_active_req] = q_lens
-            self.kv_seq_lengths_cudagraph_only[:n_active_req] = kv_lens
+            if not self.fused_bookkeeping:
+                self.query_seq_lengths_cudagraph_only[:n_active_req] = q_lens
+                self.kv_seq_lengths_cudagraph_only[:n_active_req] = kv_lens
+                self.request_to_kv_chunk_ids_cudagraph_only[:n_active_req] = self.request_to_kv_chunk_ids[act]
             self.kv_seq_lengths = self.kv_seq_lengths_cudagraph_only[:R]
             self.max_seqlen_k = self.max_sequence_length
-            self.request_to_kv_chunk_ids_cudagraph_only[:n_active_req] = self.request_to_kv_chunk_ids[act]
             self.block_table = self.request_to_kv_chunk_ids_cudagraph_only[:R]
             if decode_only:
                 self.cu_query_seq_lengths = None
@@ -588,6 +608,8 @@ class DynamicInferenceContext:
         rows are rewritten for a one-token-per-request decode step.  Returns the ids of
         requests that were newly paused and stay paused, or ``None``.
         """
+        if self.fused_bookkeeping:
+            return self._update_requests_fused(active_requests_mask, new_tokens)
         n_continue = (active_requests_mask == 1).sum().item()
         n_finished = (active_requests_mask == 0).sum().item()
         assert n_continue + n_finished + self.paused_request_count == self.total_request_count
@@ -682,6 +704,36 @@ class DynamicInferenceContext:
         self.token_to_chunk_idx[:n_continue] = self.request_last_kv_chunk_id[act]
         self.token_to_local_position_within_kv_chunk[:n_continue] = self.request_last_kv_chunk_offset[act]
         return newly_paused_request_ids
+
+    def _update_requests_fused(self, active_requests_mask: Tensor, new_tokens: Tensor) -> Optional[Tensor]:
+        """``update_requests`` as one kernel + one read-back of the new counters."""
+        dev = self.device
+        assert active_requests_mask.numel() + self.paused_request_count == self.total_request_count
+        mask = active_requests_mask.to(device=dev, dtype=torch.int32).contiguous()
+        tokens = new_tokens.to(device=dev, dtype=torch.long).contiguous()
+        assert tokens.numel() >= mask.numel()
+        if self.paused_request_count:
+            assert self.paused_tokens is not None
+            if self.paused_tokens.data_ptr() != self._paused_tokens_buf.data_ptr():
+                self._paused_tokens_buf[: self.paused_request_count] = self.paused_tokens[: self.paused_request_count]
+        ops.update_requests(self, mask, tokens)
+        self._counters_host.copy_(self._counters, non_blocking=True)
+        torch.cuda.current_stream(dev).synchronize()
+        total, paused, active, avail, n_newly, status, was_reset, _ = self._counters_host.tolist()
+        assert status != 1, "active + finished + paused requests != total_request_count"
+        self.reset_attention_state()
+        assert status != 2, "active_request_count == 0."
+        assert status != 3, (
+            "The request_last_kv_chunk_offset should be 0 for the requests that just got resumed this step. ")
+        self.chunk_allocator.chunk_count_avail = avail
+        self.total_request_count = total
+        self.active_token_count = active
+        if was_reset:
+            return None
+        self.paused_request_count = paused
+        if paused > 0:
+            self.paused_tokens = self._paused_tokens_buf[:paused]
+        return None if n_newly < 0 else self._newly_paused_buf[:n_newly].clone()
 
     def calculate_log_probs(self, logits: Tensor, new_tokens: Tensor,
                             only_last_token_logits: Optional[bool] = False) -> List[List[float]]:

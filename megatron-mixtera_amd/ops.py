@@ -332,3 +332,41 @@ def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: O
         _ptr(k_cache), _ptr(v_cache), sc, st, _ptr(token_to_chunk_idx), _ptr(token_to_local_pos),
         _ptr(block_table), 0 if block_table is None else block_table.stride(0), _ptr(kv_lens), chunk,
         T, Hq, Hkv, D, int(bool(faithful_rounding)), _stream(ref)), "mi_norm_rope_append")
+
+
+# ---------------------------------------------------------------------------------------------
+# context bookkeeping on the GPU
+# ---------------------------------------------------------------------------------------------
+def update_requests(ctx, mask_i32: Tensor, new_tokens_i64: Tensor) -> None:
+    """Enqueue the single-kernel ``update_requests`` on the state tensors of ``ctx`` (results land in
+    ``ctx._counters`` / ``ctx._newly_paused_buf`` / ``ctx._paused_tokens_buf``)."""
+    lib = _lib.load()
+    table = ctx.request_to_kv_chunk_ids
+    _require(table.stride(1) == 1, "request_to_kv_chunk_ids rows must be contiguous")
+    _lib.check(lib.mi_update_requests(
+        ctx.request_ids.data_ptr(), ctx.request_query_lengths.data_ptr(), ctx.request_output_lengths.data_ptr(),
+        ctx.request_kv_length_offsets.data_ptr(), ctx.request_kv_chunk_counts.data_ptr(),
+        ctx.request_last_kv_chunk_id.data_ptr(), ctx.request_last_kv_chunk_offset.data_ptr(),
+        table.data_ptr(), table.stride(0), table.size(1),
+        ctx.token_to_input_ids.data_ptr(), ctx.token_to_pos_ids.data_ptr(), ctx.token_to_request_idx.data_ptr(),
+        ctx.token_to_position_in_request.data_ptr(), ctx.token_to_chunk_idx.data_ptr(),
+        ctx.token_to_local_position_within_kv_chunk.data_ptr(), ctx.chunk_allocator.chunk_bag.data_ptr(),
+        mask_i32.data_ptr(), new_tokens_i64.data_ptr(), ctx._paused_tokens_buf.data_ptr(),
+        ctx._next_tokens_buf.data_ptr(), ctx._update_scratch.data_ptr(), ctx._newly_paused_buf.data_ptr(),
+        ctx._counters.data_ptr(), ctx.total_request_count, ctx.paused_request_count,
+        ctx.chunk_allocator.chunk_count_avail, ctx.gtd_chunk_count, ctx.gtd_request_count,
+        ctx.chunk_size_tokens, ctx.max_requests, _stream(table)), "mi_update_requests")
+
+
+def decode_attention_state(ctx, n_active_requests: int, padded_tokens: int) -> None:
+    """Fill the fixed-address length / block-table mirrors and the padded token rows in one launch."""
+    lib = _lib.load()
+    table = ctx.request_to_kv_chunk_ids
+    mirror = ctx.request_to_kv_chunk_ids_cudagraph_only
+    _lib.check(lib.mi_decode_attention_state(
+        ctx.request_kv_length_offsets.data_ptr(), ctx.request_query_lengths.data_ptr(), table.data_ptr(),
+        table.stride(0), table.size(1), ctx.query_seq_lengths_cudagraph_only.data_ptr(),
+        ctx.kv_seq_lengths_cudagraph_only.data_ptr(), mirror.data_ptr(), mirror.stride(0),
+        ctx.token_to_chunk_idx.data_ptr(), ctx.token_to_local_position_within_kv_chunk.data_ptr(),
+        ctx.token_to_position_in_request.data_ptr(), ctx.paused_request_count, n_active_requests,
+        ctx.active_token_count, padded_tokens, ctx.dummy_chunk_idx, _stream(table)), "mi_decode_attention_state")
