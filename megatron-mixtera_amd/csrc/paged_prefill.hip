@@ -345,12 +345,16 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int m16 = lane & 15, g = lane >> 4;
-  const int h = blockIdx.y;
+  // Heaviest workgroups first: within a request the visible keys grow with the query position, so
+  // the linear index walks the query blocks backwards; consecutive indices are the KV heads of
+  // one block (they land on different XCDs, each of which then keeps one head's K/V in its L2).
+  const int h = blockIdx.x % p.Hkv;
+  const int rank = blockIdx.x / p.Hkv;
   const int G = p.G;
   const int BQ = (16 * NQ) >> p.g_shift;  // query tokens per wave
   const int SBQ = WAVES * BQ;             // query tokens per workgroup
 
-  if (blockIdx.x == 0) {
+  if (rank == 0) {
     const int tq = p.cu_q[p.R];
     const int per_row = G * HD;
     for (int64_t i = (int64_t)tid * 8; i < (int64_t)(p.T - tq) * per_row; i += 512 * 8) {
@@ -359,7 +363,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
     }
   }
 
-  const int sb = blockIdx.x;
+  const int sb = (int)(gridDim.x / p.Hkv) - 1 - rank;
   int lo = 0, hi = p.R - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
@@ -564,7 +568,433 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Two-phase ("ping-pong") variant of the LDS kernel, head_dim 128.
+//
+// The per-tile work of a wave is split into a matrix phase  { O^T += V^T P^T of the previous tile,
+// S^T = K Q^T of this tile }  and a vector phase  { online softmax of this tile, staging of the
+// next tiles into LDS }.  The 8 waves form two groups of four (waves w and w+4 share a SIMD);
+// every phase ends in a workgroup barrier and the second group runs one phase behind the first,
+// so on every SIMD one wave is feeding the matrix cores while the other one runs the exp / max /
+// convert chain.  Because the groups read a staged tile one phase apart, the first group stages
+// one tile ahead of its own use and the second group two (see the table in the loop).
+//
+// Other differences to paged_prefill_lds_kernel: V fragments come out of LDS already transposed
+// (ds_read_b64_tr_b16, 288-byte V pitch), so there is no permute work; the softmax denominator is
+// accumulated by the matrix cores (an all-ones A fragment), and the cross-lane maximum uses the
+// lane-swap instructions instead of LDS permutes.
+// ---------------------------------------------------------------------------------------------
+constexpr int kKPitch = 288;  // bytes per staged K row: measured conflict-free for the 16-row x 64-byte fragment reads (272 is not)
+constexpr int kVPitch = 288;  // bytes per staged V row: 16 rows x 32 B tile the banks twice
+constexpr int kPPTile = 64;   // keys per staged tile
+
+typedef short s16x4v __attribute__((ext_vector_type(4)));
+
+// Transposing LDS read: within each block of 16 lanes, lane i supplies the address of 4 bf16
+// (row i/4, columns 4*(i%4)..+3 of a 4 x 16 matrix) and lane L receives column L of that matrix.
+static __device__ __forceinline__ uint2 lds_ld8_tr(const uint8_t* ptr) {
+  const s16x4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) s16x4v*)(uintptr_t)(uint32_t)(uintptr_t)ptr);
+  return __builtin_bit_cast(uint2, v);
+}
+
+// max over the four lanes {l, l^16, l^32, l^48} with two lane-swap instructions
+static __device__ __forceinline__ float rowgroup_max(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const uint32_t w = __float_as_uint(y);
+  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+
+#ifdef MI_PP_TRACE  // developer build only: per-phase cycle stamps of one heavy workgroup
+__device__ long long mi_pp_trace_buf[8 * 64 * 8];
+// stamps are parked in LDS (a global store here would sit in the queue the staging waits on)
+#define MI_PP_STAMP(slot)                                                                   \
+  do {                                                                                      \
+    if (rank == 1 && h == 0 && lane == 0 && it >= 8 && it < 72)                             \
+      trace_lds[(wave * 64 + (it - 8)) * 8 + (slot)] = (uint32_t)clock64();                 \
+  } while (0)
+#define MI_PP_CLOCK(var) const long long var = clock64()
+#define MI_PP_STAMP_AT(slot, var)                                                           \
+  do {                                                                                      \
+    if (rank == 1 && h == 0 && lane == 0 && it >= 8 && it < 72)                             \
+      trace_lds[(wave * 64 + (it - 8)) * 8 + (slot)] = (uint32_t)(var);                     \
+  } while (0)
+#else
+#define MI_PP_STAMP(slot) do { } while (0)
+#define MI_PP_CLOCK(var) do { } while (0)
+#define MI_PP_STAMP_AT(slot, var) do { } while (0)
+#endif
+
+template <bool STAGGER>
+__global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
+  constexpr int HD = 128, KS = 4, DV = 8, NQ = 2, NT = 4, WAVES = 8;
+  __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kPPTile * kKPitch];
+  __shared__ __attribute__((aligned(16))) uint8_t Vs[2][kPPTile * kVPitch];
+#ifdef MI_PP_TRACE
+  __shared__ uint32_t trace_lds[8 * 64 * 8];
+  for (int i = threadIdx.x; i < 8 * 64 * 8; i += 512) trace_lds[i] = 0;
+#endif
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform values stay in SGPRs
+  const int m16 = lane & 15, g = lane >> 4;
+  const int lead = STAGGER ? (wave >> 2) : 0;  // 0: first group, 1: second group (one phase behind)
+  const int h = blockIdx.x % p.Hkv;
+  const int rank = blockIdx.x / p.Hkv;
+  const int G = p.G;
+  const int BQ = (16 * NQ) >> p.g_shift;
+  const int SBQ = WAVES * BQ;
+
+  if (rank == 0) {
+    const int tq = p.cu_q[p.R];
+    const int per_row = G * HD;
+    for (int64_t i = (int64_t)tid * 8; i < (int64_t)(p.T - tq) * per_row; i += 512 * 8) {
+      const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
+      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
+    }
+  }
+
+  const int sb = (int)(gridDim.x / p.Hkv) - 1 - rank;
+  int lo = 0, hi = p.R - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (p.cu_q[mid] / SBQ + mid <= sb) lo = mid; else hi = mid - 1;
+  }
+  const int r = lo;
+  const int q_begin = p.cu_q[r];
+  const int Lq = p.cu_q[r + 1] - q_begin;
+  const int q0_wg = (sb - (q_begin / SBQ + r)) * SBQ;
+  if (q0_wg >= Lq) return;  // workgroup-uniform
+  if (p.skip_single && Lq == 1) return;
+  const int Lk = p.lens[r];
+  const int shift = Lk - Lq;
+  const int last = Lk - 1;
+  const int kend_wg = min(Lk, shift + min(q0_wg + SBQ, Lq));
+  const int ntl = (kend_wg + kPPTile - 1) / kPPTile;  // staged tiles of this workgroup
+
+  const int q0 = q0_wg + wave * BQ;
+  const int nq = max(0, min(BQ, Lq - q0));
+  const int kend = nq > 0 ? min(Lk, shift + q0 + nq) : 0;
+  const int full_until = shift + q0;
+
+  uint4 qf[NQ][KS];
+  int qpos[NQ];
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    const int n = 16 * nt + m16;
+    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const bool valid = qi < nq;
+    qpos[nt] = valid ? shift + q0 + qi : last;
+    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      qf[nt][kk] = valid ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
+  }
+
+  float m_run[NQ];
+  f32x4_t acc[NQ][DV], accl[NQ];
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    m_run[nt] = -INFINITY;
+    accl[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int e = 0; e < DV; ++e) acc[nt][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  if (ntl > 0) {
+    const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * 2;
+    const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * 2;
+    const int64_t chunk_bytes = p.kv_sc * 2;
+    const int tok_bytes = p.kv_st * 2;
+    // loader role: 16-byte piece `lpiece` of key rows `lkey` and `lkey + 32` of a tile
+    const int lkey = tid >> 4, lpiece = tid & 15;
+    const int k_off = lkey * kKPitch + lpiece * 16;
+    const int v_off = lkey * kVPitch + lpiece * 16;
+    uint4 kreg[2], vreg[2];
+    // Staged tiles never straddle a chunk (the launcher only picks this kernel when the chunk size
+    // is a multiple of 64), so a tile is addressed by scalars only -- physical chunk, tile index
+    // inside the chunk -- plus a per-lane row offset that is fixed for the whole kernel.  The
+    // fetch cursor below walks the tiles with adds and compares instead of divisions; it stops
+    // on the last tile, so the extra fetches and LDS stores at the end of the loop repeat that
+    // tile into a buffer nobody reads any more, which keeps the loop free of branches.
+    const int tiles_per_chunk = p.chunk / kPPTile;
+    const int tile_bytes = kPPTile * tok_bytes;
+    const uint32_t row_off0 = (uint32_t)(lkey * tok_bytes + lpiece * 16);
+    const uint32_t row_off1 = row_off0 + (uint32_t)(32 * tok_bytes);
+    const uint32_t piece_off = (uint32_t)(lpiece * 16);
+    const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
+    struct Cursor {   // all members are wave-uniform
+      int tile;       // tile index
+      int ci, tin;    // logical chunk of the tile and tile index inside the chunk
+      int room;       // bytes from the tile's first row to the request's last row (>= 0)
+    };
+    auto cursor_at = [&](int t) {
+      Cursor c;
+      c.tile = min(t, ntl - 1);
+      c.ci = c.tile / tiles_per_chunk;
+      c.tin = c.tile - c.ci * tiles_per_chunk;
+      c.room = (last - c.tile * kPPTile) * tok_bytes;
+      return c;
+    };
+    auto cursor_next = [&](Cursor& c) {  // one tile forward, sticking to the last tile
+      const bool adv = c.tile + 1 < ntl;
+      const bool wrap = adv && (c.tin + 1 == tiles_per_chunk);
+      c.tile += adv ? 1 : 0;
+      c.room -= adv ? tile_bytes : 0;
+      c.tin = wrap ? 0 : c.tin + (adv ? 1 : 0);
+      c.ci += wrap ? 1 : 0;
+    };
+    // byte offset of the cursor's tile inside a cache, given its physical chunk
+    auto tile_offset = [&](const Cursor& c, int pc_lane) -> int64_t {
+      const int pc = __builtin_amdgcn_readfirstlane(pc_lane);
+      return (int64_t)pc * chunk_bytes + (int64_t)c.tin * tile_bytes;
+    };
+    // this thread's two pieces of a tile (rows past the request's last key re-read the last row,
+    // which every query row masks)
+    auto tile_loads = [&](const uint8_t* base, int64_t off, int room, uint4 (&reg)[2]) {
+      const uint8_t* tb = base + off;
+      const uint32_t lim = (uint32_t)room + piece_off;
+      reg[0] = ld16(tb + min(row_off0, lim));
+      reg[1] = ld16(tb + min(row_off1, lim));
+    };
+    auto store_k = [&](int t) {
+      uint8_t* dst = &Ks[t & 1][k_off];
+      *reinterpret_cast<uint4*>(dst) = kreg[0];
+      *reinterpret_cast<uint4*>(dst + 32 * kKPitch) = kreg[1];
+    };
+    auto store_v = [&](int t) {
+      uint8_t* dst = &Vs[t & 1][v_off];
+      *reinterpret_cast<uint4*>(dst) = vreg[0];
+      *reinterpret_cast<uint4*>(dst + 32 * kVPitch) = vreg[1];
+    };
+
+    const float scale = p.scale_log2;
+    const uint4 ones = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+    f32x4_t s[NQ][NT];
+    uint2 pf[NQ][NT];
+    // fixed per-lane offsets of the fragment reads
+    const int kfrag_off = m16 * kKPitch + 16 * g;
+    const int vfrag_off = (4 * g + (m16 >> 2)) * kVPitch + 8 * (m16 & 3);
+
+    // ---- matrix phase pieces.  The work is cut into groups of 8-10 MFMAs; the LDS reads of a
+    // group are issued before the MFMAs of the previous group (scheduling barriers keep that
+    // order), so a read has ~130 cycles of matrix work to hide behind and only two groups of
+    // fragments are live at a time.
+    // S^T = K Q^T: group u = 16-key sub-tile u (4 K fragments, 8 MFMAs)
+    auto sc_load = [&](int t, int u, uint4 (&kf)[KS]) {
+      const uint8_t* ks = Ks[t & 1] + kfrag_off + 16 * u * kKPitch;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) kf[kk] = *reinterpret_cast<const uint4*>(ks + 64 * kk);
+    };
+    auto sc_mma = [&](int u, const uint4 (&kf)[KS]) {
+      s[0][u] = mfma_16x16x32(kf[0], qf[0][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
+      s[1][u] = mfma_16x16x32(kf[0], qf[1][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+      for (int kk = 1; kk < KS; ++kk) {
+        s[0][u] = mfma_16x16x32(kf[kk], qf[0][kk], s[0][u]);
+        s[1][u] = mfma_16x16x32(kf[kk], qf[1][kk], s[1][u]);
+      }
+    };
+    // O^T += V^T P^T: group grp = (32-key step grp / 2, output columns 64 * (grp % 2) ..+63):
+    // 8 transposed reads, 8 MFMAs (+2 for the denominators in the odd groups)
+    auto pv_load = [&](int t, int grp, uint2 (&af)[4][2]) {
+      const uint8_t* vs = Vs[t & 1] + vfrag_off + 32 * (grp >> 1) * kVPitch + 128 * (grp & 1);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        af[e][0] = lds_ld8_tr(vs + 32 * e);
+        af[e][1] = lds_ld8_tr(vs + 16 * kVPitch + 32 * e);
+      }
+    };
+    auto pv_mma = [&](int grp, const uint2 (&af)[4][2]) {
+      const int up = 2 * (grp >> 1), e0 = 4 * (grp & 1);
+      const uint4 pp0 = make_uint4(pf[0][up].x, pf[0][up].y, pf[0][up + 1].x, pf[0][up + 1].y);
+      const uint4 pp1 = make_uint4(pf[1][up].x, pf[1][up].y, pf[1][up + 1].x, pf[1][up + 1].y);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const uint4 a = make_uint4(af[e][0].x, af[e][0].y, af[e][1].x, af[e][1].y);
+        acc[0][e0 + e] = mfma_16x16x32(a, pp0, acc[0][e0 + e]);
+        acc[1][e0 + e] = mfma_16x16x32(a, pp1, acc[1][e0 + e]);
+      }
+      if (grp & 1) {
+        accl[0] = mfma_16x16x32(ones, pp0, accl[0]);
+        accl[1] = mfma_16x16x32(ones, pp1, accl[1]);
+      }
+    };
+#define MI_SB() __builtin_amdgcn_sched_barrier(0)
+    // The whole matrix phase of iteration it: O^T += V^T P^T of tile it-1, S^T = K Q^T of tile it,
+    // and -- spread over the first MFMA groups, whose shadow hides the address arithmetic --
+    // the staging: store K(it+1) and V(it) (fetched during the previous matrix phase) into LDS,
+    // then fetch K(it+2) and V(it+1).
+    Cursor cur = cursor_at(2);  // the K tile fetched during iteration 0
+    int pc_cur = 0;             // its block-table entry (a per-lane copy, made scalar at its use)
+    int64_t off_v = 0;          // offset and room of the V tile fetched during iteration 0: tile 1
+    int room_v = 0;
+    auto matrix_phase = [&](int it) {
+      uint2 a0[4][2], a1[4][2];
+      uint4 k0[KS], k1[KS];
+      const int ta = it - 1, ts = it;
+      pv_load(ta, 0, a0);
+      pv_load(ta, 1, a1); MI_SB();
+      MI_PP_CLOCK(c1);
+      pv_mma(0, a0); MI_SB();
+      MI_PP_CLOCK(c2);
+      store_k(it + 1);
+      store_v(it); MI_SB();
+      MI_PP_CLOCK(c3);
+      pv_load(ta, 2, a0); MI_SB();
+      pv_mma(1, a1);
+      // fetch K(it+2); its offset and room are kept for V(it+2), fetched one iteration later
+      const int64_t off_k = tile_offset(cur, pc_cur);
+      const int room_k = cur.room;
+      tile_loads(kbase, off_k, room_k, kreg);
+      cursor_next(cur);
+      pc_cur = bt_row[cur.ci];  // block-table entry of tile it+3, consumed one iteration from now
+      // spread the address arithmetic through the shadow of this group's MFMAs
+#pragma unroll
+      for (int i = 0; i < 10; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+        __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);  // up to three scalar / vector ALU instructions
+      }
+      MI_SB();
+      MI_PP_CLOCK(c4);
+      pv_load(ta, 3, a1); MI_SB();
+      pv_mma(2, a0);
+      tile_loads(vbase, off_v, room_v, vreg);  // V(it+1): same offset as K(it+1)
+      off_v = off_k;
+      room_v = room_k; MI_SB();
+      MI_PP_CLOCK(c5);
+      sc_load(ts, 0, k0); MI_SB();
+      pv_mma(3, a1); MI_SB();
+      MI_PP_CLOCK(c6);
+      sc_load(ts, 1, k1); MI_SB(); sc_mma(0, k0); MI_SB();
+      sc_load(ts, 2, k0); MI_SB(); sc_mma(1, k1); MI_SB();
+      MI_PP_CLOCK(c7);
+      sc_load(ts, 3, k1); MI_SB(); sc_mma(2, k0); MI_SB();
+      sc_mma(3, k1);
+      MI_PP_STAMP_AT(1, c1); MI_PP_STAMP_AT(2, c2); MI_PP_STAMP_AT(3, c3);
+      MI_PP_STAMP_AT(4, c4); MI_PP_STAMP_AT(5, c5); MI_PP_STAMP_AT(6, c6); MI_PP_STAMP_AT(7, c7);
+    };
+    // ---- online softmax of tile t: s -> pf, rescale of the accumulators when a maximum moved ----
+    auto softmax = [&](int t) {
+      const int T = t * kPPTile;
+      const bool need_mask = T + kPPTile - 1 > full_until;
+#pragma unroll
+      for (int nt = 0; nt < NQ; ++nt) {
+        if (need_mask) {
+#pragma unroll
+          for (int u = 0; u < NT; ++u) {
+            const int tok0 = T + 16 * u + 4 * g;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (tok0 + i > qpos[nt]) s[nt][u][i] = -INFINITY;
+          }
+        }
+        float tmax = fmaxf(fmaxf(s[nt][0][0], s[nt][0][1]), s[nt][0][2]);
+        tmax = fmaxf(fmaxf(tmax, s[nt][0][3]), s[nt][1][0]);
+        tmax = fmaxf(fmaxf(tmax, s[nt][1][1]), s[nt][1][2]);
+        tmax = fmaxf(fmaxf(tmax, s[nt][1][3]), s[nt][2][0]);
+        tmax = fmaxf(fmaxf(tmax, s[nt][2][1]), s[nt][2][2]);
+        tmax = fmaxf(fmaxf(tmax, s[nt][2][3]), s[nt][3][0]);
+        tmax = fmaxf(fmaxf(tmax, s[nt][3][1]), s[nt][3][2]);
+        tmax = fmaxf(tmax, s[nt][3][3]);
+        tmax = rowgroup_max(tmax);
+        const float m_raw = fmaxf(m_run[nt], tmax);
+        const float m_use = m_raw == -INFINITY ? 0.f : m_raw;
+        const float alpha = fast_exp2((m_run[nt] - m_use) * scale);
+        const float neg = -m_use * scale;
+        m_run[nt] = m_raw;
+#pragma unroll
+        for (int u = 0; u < NT; ++u) {
+          const float p0 = fast_exp2(__builtin_fmaf(s[nt][u][0], scale, neg));
+          const float p1 = fast_exp2(__builtin_fmaf(s[nt][u][1], scale, neg));
+          const float p2 = fast_exp2(__builtin_fmaf(s[nt][u][2], scale, neg));
+          const float p3 = fast_exp2(__builtin_fmaf(s[nt][u][3], scale, neg));
+          pf[nt][u] = make_uint2(pack_bf16x2(p0, p1), pack_bf16x2(p2, p3));
+        }
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+          for (int e = 0; e < DV; ++e) {
+            acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
+          }
+          accl[nt][0] *= alpha; accl[nt][1] *= alpha; accl[nt][2] *= alpha; accl[nt][3] *= alpha;
+        }
+      }
+    };
+    // Staging rides in the matrix phase (LDS-write and memory ports are idle there; the vector
+    // phase is the longer one).  Phase numbers: group 0 runs matrix(it) in phase 2it and vector(it)
+    // in 2it+1, group 1 one phase later.  matrix(it) reads K(it) and V(it-1); K(t) is therefore
+    // read in phases 2t and 2t+1, V(t) in 2t+2 and 2t+3.  Both groups store K(it+1) and V(it)
+    // during matrix(it): the buffers they overwrite held K(it-1) and V(it-2), last read in
+    // phase 2it-1, and the first reader of the new tiles is group 0 in phase 2it+2.
+#pragma unroll
+    for (int nt = 0; nt < NQ; ++nt)
+#pragma unroll
+      for (int u = 0; u < NT; ++u) pf[nt][u] = make_uint2(0u, 0u);
+    for (int i = tid * 16; i < kPPTile * kVPitch; i += 512 * 16)
+      *reinterpret_cast<uint4*>(&Vs[1][i]) = make_uint4(0u, 0u, 0u, 0u);
+    {
+      const Cursor c0 = cursor_at(0), c1 = cursor_at(1);
+      const int64_t off0 = tile_offset(c0, bt_row[c0.ci]);
+      tile_loads(kbase, off0, c0.room, kreg);
+      store_k(0);
+      __syncthreads();  // K(0) and the zero-filled V buffer 1 are visible; kreg is free again
+      off_v = tile_offset(c1, bt_row[c1.ci]);
+      room_v = c1.room;
+      tile_loads(kbase, off_v, room_v, kreg);  // K(1)
+      tile_loads(vbase, off0, c0.room, vreg);  // V(0)
+      pc_cur = bt_row[cur.ci];
+    }
+    if (lead) __syncthreads();  // second group idles through phase 0
+
+    // One code path for every iteration.  Every wave runs every staged tile of the workgroup (a
+    // wave whose rows cannot see a tile would only wait at the barriers instead; its scores there
+    // are all masked, p = 0).  Iteration 0 "accumulates" tile -1: zero probabilities times the
+    // zero-filled V buffer 1; iteration ntl computes scores of a stale K buffer that nobody uses.
+    for (int it = 0; it <= ntl; ++it) {
+      MI_PP_STAMP(0);
+      matrix_phase(it);
+      __syncthreads();
+      if (it < ntl) softmax(it);
+      __syncthreads();
+    }
+    if (!lead && STAGGER) __syncthreads();
+#undef MI_SB
+  }
+#ifdef MI_PP_TRACE
+  __syncthreads();
+  if (rank == 1 && h == 0)
+    for (int i = tid; i < 8 * 64 * 8; i += 512) mi_pp_trace_buf[i] = trace_lds[i];
+#endif
+
+  // ---- epilogue: acc[nt][e][i] is output element d = 16e + 4g + i of row (nt, m16) --------------
+#pragma unroll
+  for (int nt = 0; nt < NQ; ++nt) {
+    const float l_tot = accl[nt][0];
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int n = 16 * nt + m16;
+    const int qi = n >> p.g_shift, u = n & (G - 1);
+    if (qi < nq) {
+      uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * g;
+#pragma unroll
+      for (int e = 0; e < DV; ++e)
+        st8(o + 16 * e, make_uint2(pack_bf16x2(acc[nt][e][0] * inv, acc[nt][e][1] * inv),
+                                   pack_bf16x2(acc[nt][e][2] * inv, acc[nt][e][3] * inv)));
+    }
+  }
+}
+
 }  // namespace mi
+
+#ifdef MI_PP_TRACE
+extern "C" int mi_pp_trace_read(long long* dst, int n) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi::mi_pp_trace_buf), sizeof(long long) * n);
+}
+#endif
 
 using namespace mi;
 
@@ -624,14 +1054,17 @@ extern "C" int mi_paged_prefill_attention(
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
   const int lds_tiles = mi_tuning().prefill_lds_row_tiles;  // 0 = register-only kernel
   if (head_dim == 128 && lds_tiles > 0) {
-    const int rows = 8 * 16 * (lds_tiles == 2 ? 2 : 3);
+    const int rows = 8 * 16 * ((lds_tiles == 2 || (mi_tuning().prefill_pingpong && chunk_tokens % 64 == 0)) ? 2 : 3);
     const int sbq_lds = rows / G;
-    dim3 lgrid((T + sbq_lds - 1) / sbq_lds + R, Hkv);
+    dim3 lgrid(((T + sbq_lds - 1) / sbq_lds + R) * Hkv);
     const bool wide = mi_tuning().prefill_tile_subtiles == 4;  // 64-key staged tiles
     hipEvent_t ev_a, ev_b;
     const bool timed = mi_profile_next(&ev_a, &ev_b);
     if (timed) hipEventRecord(ev_a, st);
-    if (lds_tiles == 2 && wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 4>), lgrid, dim3(512), 0, st, p);
+    const int pp = (chunk_tokens % 64 == 0) ? mi_tuning().prefill_pingpong : 0;  // staged tiles must not straddle chunks
+    if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true>), lgrid, dim3(512), 0, st, p);
+    else if (pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false>), lgrid, dim3(512), 0, st, p);
+    else if (lds_tiles == 2 && wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 4>), lgrid, dim3(512), 0, st, p);
     else if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 2>), lgrid, dim3(512), 0, st, p);
     else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);  // (48 rows: 32-key tiles only)
     if (timed) hipEventRecord(ev_b, st);
