@@ -152,7 +152,7 @@ def run_mixed_batch(args, mi, lib, torch, dev):
                                "32/8 heads d128 chunk 256; step = fused RMSNorm+RoPE+append then paged varlen attention",
                    "new_tokens": T, "requests": int(lens.numel()), "algorithmic_bytes_per_step": total_bytes,
                    "prefill_flops_per_step": flops},
-        "roofline": {"bound": "mfma", "kernel": "paged_prefill_lds_kernel", "achieved": round(flops / tile_ms / 1e9, 1),
+        "roofline": {"bound": "mfma", "kernel": "paged_prefill_pp_kernel", "achieved": round(flops / tile_ms / 1e9, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / tile_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "kernel_ms": round(tile_ms, 5),
                      "traffic": None},

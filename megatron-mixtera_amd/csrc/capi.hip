@@ -29,7 +29,7 @@ MiTuning& mi_tuning() {
                       env_int("MI355_PREFILL_LDS_ROW_TILES", 2), env_int("MI355_PREFILL_ROW_TILES", 2),
                       env_int("MI355_DECODE_MIN_WAVES", 3),
                       env_int("MI355_DECODE_WGS_PER_CU", 1), env_int("MI355_DECODE_GRID", 0),
-                      env_int("MI355_DECODE_WAVES_PER_BLOCK", 8), env_int("MI355_PREFILL_PINGPONG", 0)};
+                      env_int("MI355_DECODE_WAVES_PER_BLOCK", 8), env_int("MI355_PREFILL_PINGPONG", 1)};
   return t;
 }
 

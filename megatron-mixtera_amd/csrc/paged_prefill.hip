@@ -633,7 +633,7 @@ template <bool STAGGER>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
   constexpr int HD = 128, KS = 4, DV = 8, NQ = 2, NT = 4, WAVES = 8;
   __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kPPTile * kKPitch];
-  __shared__ __attribute__((aligned(16))) uint8_t Vs[2][kPPTile * kVPitch];
+  __shared__ __attribute__((aligned(16))) uint8_t Vs[3][kPPTile * kVPitch];  // three: see the loop
 #ifdef MI_PP_TRACE
   __shared__ uint32_t trace_lds[8 * 64 * 8];
   for (int i = threadIdx.x; i < 8 * 64 * 8; i += 512) trace_lds[i] = 0;
@@ -767,8 +767,9 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       *reinterpret_cast<uint4*>(dst) = kreg[0];
       *reinterpret_cast<uint4*>(dst + 32 * kKPitch) = kreg[1];
     };
+    auto vbuf = [](int t) { return (unsigned)(t + 3) % 3u; };  // tile -1 lives in buffer 2
     auto store_v = [&](int t) {
-      uint8_t* dst = &Vs[t & 1][v_off];
+      uint8_t* dst = &Vs[vbuf(t)][v_off];
       *reinterpret_cast<uint4*>(dst) = vreg[0];
       *reinterpret_cast<uint4*>(dst + 32 * kVPitch) = vreg[1];
     };
@@ -803,7 +804,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // O^T += V^T P^T: group grp = (32-key step grp / 2, output columns 64 * (grp % 2) ..+63):
     // 8 transposed reads, 8 MFMAs (+2 for the denominators in the odd groups)
     auto pv_load = [&](int t, int grp, uint2 (&af)[4][2]) {
-      const uint8_t* vs = Vs[t & 1] + vfrag_off + 32 * (grp >> 1) * kVPitch + 128 * (grp & 1);
+      const uint8_t* vs = Vs[vbuf(t)] + vfrag_off + 32 * (grp >> 1) * kVPitch + 128 * (grp & 1);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         af[e][0] = lds_ld8_tr(vs + 32 * e);
@@ -828,30 +829,26 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 #define MI_SB() __builtin_amdgcn_sched_barrier(0)
     // The whole matrix phase of iteration it: O^T += V^T P^T of tile it-1, S^T = K Q^T of tile it,
     // and -- spread over the first MFMA groups, whose shadow hides the address arithmetic --
-    // the staging: store K(it+1) and V(it) (fetched during the previous matrix phase) into LDS,
-    // then fetch K(it+2) and V(it+1).
-    Cursor cur = cursor_at(2);  // the K tile fetched during iteration 0
+    // the staging: store K(it+1) and V(it+1) (fetched during the previous matrix phase) into
+    // LDS, then fetch K(it+2) and V(it+2).  (Reading fragments ahead during the vector phase, or
+    // moving score groups there, was measured slower: a wave sustains only ~32 B/clk of LDS reads
+    // and the vector phase has no issue slots to spare.)
+    Cursor cur = cursor_at(2);  // the tile fetched during iteration 0
     int pc_cur = 0;             // its block-table entry (a per-lane copy, made scalar at its use)
-    int64_t off_v = 0;          // offset and room of the V tile fetched during iteration 0: tile 1
-    int room_v = 0;
     auto matrix_phase = [&](int it) {
       uint2 a0[4][2], a1[4][2];
       uint4 k0[KS], k1[KS];
       const int ta = it - 1, ts = it;
       pv_load(ta, 0, a0);
       pv_load(ta, 1, a1); MI_SB();
-      MI_PP_CLOCK(c1);
-      pv_mma(0, a0); MI_SB();
-      MI_PP_CLOCK(c2);
+      pv_mma(0, a0);
       store_k(it + 1);
-      store_v(it); MI_SB();
-      MI_PP_CLOCK(c3);
+      store_v(it + 1); MI_SB();
       pv_load(ta, 2, a0); MI_SB();
       pv_mma(1, a1);
-      // fetch K(it+2); its offset and room are kept for V(it+2), fetched one iteration later
-      const int64_t off_k = tile_offset(cur, pc_cur);
-      const int room_k = cur.room;
-      tile_loads(kbase, off_k, room_k, kreg);
+      const int64_t off = tile_offset(cur, pc_cur);
+      const int room = cur.room;
+      tile_loads(kbase, off, room, kreg);
       cursor_next(cur);
       pc_cur = bt_row[cur.ci];  // block-table entry of tile it+3, consumed one iteration from now
       // spread the address arithmetic through the shadow of this group's MFMAs
@@ -861,23 +858,15 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);  // up to three scalar / vector ALU instructions
       }
       MI_SB();
-      MI_PP_CLOCK(c4);
       pv_load(ta, 3, a1); MI_SB();
       pv_mma(2, a0);
-      tile_loads(vbase, off_v, room_v, vreg);  // V(it+1): same offset as K(it+1)
-      off_v = off_k;
-      room_v = room_k; MI_SB();
-      MI_PP_CLOCK(c5);
+      tile_loads(vbase, off, room, vreg); MI_SB();
       sc_load(ts, 0, k0); MI_SB();
       pv_mma(3, a1); MI_SB();
-      MI_PP_CLOCK(c6);
       sc_load(ts, 1, k1); MI_SB(); sc_mma(0, k0); MI_SB();
       sc_load(ts, 2, k0); MI_SB(); sc_mma(1, k1); MI_SB();
-      MI_PP_CLOCK(c7);
       sc_load(ts, 3, k1); MI_SB(); sc_mma(2, k0); MI_SB();
       sc_mma(3, k1);
-      MI_PP_STAMP_AT(1, c1); MI_PP_STAMP_AT(2, c2); MI_PP_STAMP_AT(3, c3);
-      MI_PP_STAMP_AT(4, c4); MI_PP_STAMP_AT(5, c5); MI_PP_STAMP_AT(6, c6); MI_PP_STAMP_AT(7, c7);
     };
     // ---- online softmax of tile t: s -> pf, rescale of the accumulators when a maximum moved ----
     auto softmax = [&](int t) {
@@ -925,42 +914,56 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         }
       }
     };
-    // Staging rides in the matrix phase (LDS-write and memory ports are idle there; the vector
-    // phase is the longer one).  Phase numbers: group 0 runs matrix(it) in phase 2it and vector(it)
-    // in 2it+1, group 1 one phase later.  matrix(it) reads K(it) and V(it-1); K(t) is therefore
-    // read in phases 2t and 2t+1, V(t) in 2t+2 and 2t+3.  Both groups store K(it+1) and V(it)
-    // during matrix(it): the buffers they overwrite held K(it-1) and V(it-2), last read in
-    // phase 2it-1, and the first reader of the new tiles is group 0 in phase 2it+2.
+    // Staging rides in the matrix phase (LDS-write and memory ports are idle there).  Phase
+    // numbers: group 0 runs matrix(it) in phase 2it and vector(it) in 2it+1, group 1 one phase
+    // later.  matrix(it) reads K(it) and V(it-1), the vector phase reads no LDS; both groups store
+    // K(it+1) and V(it+1) during matrix(it), i.e. in phases 2it and 2it+1.
+    //   K(t): stored in phases 2t-2, 2t-1; read in 2t, 2t+1           -> two buffers
+    //   V(t): stored in phases 2t-2, 2t-1; read in 2t+2, 2t+3         -> three buffers
+    // (the tile that shares a buffer is stored from phase 2t+2 resp. 2t+4 on).
 #pragma unroll
     for (int nt = 0; nt < NQ; ++nt)
 #pragma unroll
       for (int u = 0; u < NT; ++u) pf[nt][u] = make_uint2(0u, 0u);
     for (int i = tid * 16; i < kPPTile * kVPitch; i += 512 * 16)
-      *reinterpret_cast<uint4*>(&Vs[1][i]) = make_uint4(0u, 0u, 0u, 0u);
+      *reinterpret_cast<uint4*>(&Vs[2][i]) = make_uint4(0u, 0u, 0u, 0u);  // "tile -1"
     {
       const Cursor c0 = cursor_at(0), c1 = cursor_at(1);
       const int64_t off0 = tile_offset(c0, bt_row[c0.ci]);
       tile_loads(kbase, off0, c0.room, kreg);
+      tile_loads(vbase, off0, c0.room, vreg);
       store_k(0);
-      __syncthreads();  // K(0) and the zero-filled V buffer 1 are visible; kreg is free again
-      off_v = tile_offset(c1, bt_row[c1.ci]);
-      room_v = c1.room;
-      tile_loads(kbase, off_v, room_v, kreg);  // K(1)
-      tile_loads(vbase, off0, c0.room, vreg);  // V(0)
+      store_v(0);
+      __syncthreads();  // K(0), V(0) and the zero-filled buffer are visible; the staging registers are free
+      const int64_t off1 = tile_offset(c1, bt_row[c1.ci]);
+      tile_loads(kbase, off1, c1.room, kreg);  // K(1), V(1): stored by matrix(0)
+      tile_loads(vbase, off1, c1.room, vreg);
       pc_cur = bt_row[cur.ci];
     }
     if (lead) __syncthreads();  // second group idles through phase 0
 
     // One code path for every iteration.  Every wave runs every staged tile of the workgroup (a
     // wave whose rows cannot see a tile would only wait at the barriers instead; its scores there
-    // are all masked, p = 0).  Iteration 0 "accumulates" tile -1: zero probabilities times the
-    // zero-filled V buffer 1; iteration ntl computes scores of a stale K buffer that nobody uses.
+    // are all masked, p = 0).  Iteration 0 "accumulates" tile -1: zero probabilities times a
+    // zero-filled V buffer; iteration ntl computes scores of a stale K buffer that nobody uses.
     for (int it = 0; it <= ntl; ++it) {
-      MI_PP_STAMP(0);
-      matrix_phase(it);
+      // (scheduling barriers: MFMAs touch no memory, so nothing else stops the compiler from
+      // sinking them past the workgroup barrier into the other phase)
+      MI_PP_CLOCK(c0);
+      __builtin_amdgcn_s_setprio(2);  // the matrix-phase wave issues first: its MFMAs are sparse
+      matrix_phase(it);               // and must never wait behind the other wave's ALU stream
+      __builtin_amdgcn_s_setprio(0);
+      MI_SB();
+      MI_PP_CLOCK(c1);
       __syncthreads();
+      MI_SB();
+      MI_PP_CLOCK(c2);
       if (it < ntl) softmax(it);
+      MI_PP_CLOCK(c3);
+      MI_PP_STAMP_AT(0, c0); MI_PP_STAMP_AT(1, c1); MI_PP_STAMP_AT(2, c2); MI_PP_STAMP_AT(3, c3);
+      MI_SB();
       __syncthreads();
+      MI_SB();
     }
     if (!lead && STAGGER) __syncthreads();
 #undef MI_SB
