@@ -29,6 +29,7 @@ from .contexts import (  # noqa: F401
     WarmupEngineMode,
 )
 from .flash_attn_interface import flash_attn_varlen_func, flash_attn_with_kvcache  # noqa: F401
+from .graphs import DecodeLayerGraphs  # noqa: F401
 
 __all__ = [
     "ops",
@@ -46,4 +47,5 @@ __all__ = [
     "flash_decode_and_prefill",
     "adjust_key_value_for_inference",
     "PagedSelfAttentionCore",
+    "DecodeLayerGraphs",
 ]

@@ -41,16 +41,40 @@ def _cache_strides(cache: Tensor) -> Tuple[int, int, int]:
 
 # per-device split-K workspace, grown on demand (owned here, handed to the C ABI as caller memory)
 _workspaces: dict = {}
+_retired_workspaces: list = []   # outgrown buffers stay alive: work already enqueued may still use them
+_workspace_override: list = []   # innermost ``use_workspace`` buffer
 
 
 def _workspace(device: torch.device, nbytes: int) -> Optional[Tensor]:
     if nbytes <= 0:
         return None
+    if _workspace_override:
+        ws = _workspace_override[-1]
+        _require(ws.device == device and ws.numel() >= nbytes, "the workspace given to use_workspace is too small")
+        return ws
     ws = _workspaces.get(device)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        if ws is not None:
+            _retired_workspaces.append(ws)
+        ws = torch.empty(max(nbytes, 2 * (0 if ws is None else ws.numel())), dtype=torch.uint8, device=device)
         _workspaces[device] = ws
     return ws
+
+
+class use_workspace:
+    """Context manager: attention calls inside use ``buffer`` as their scratch instead of the
+    per-device one (graph capture needs a buffer that is never re-allocated)."""
+
+    def __init__(self, buffer: Tensor):
+        self.buffer = buffer
+
+    def __enter__(self):
+        _workspace_override.append(self.buffer)
+        return self.buffer
+
+    def __exit__(self, *exc):
+        _workspace_override.pop()
+        return False
 
 
 def set_tuning(name: str, value: int) -> None:
