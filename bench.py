@@ -46,6 +46,7 @@ def parse_args():
     ap.add_argument("--split-tokens", type=int, default=0)
     ap.add_argument("--subtiles", type=int, default=0, help="16-token sub-tiles per loop iteration (1, 2 or 4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--hip-graph", action="store_true", help="replay the step as one captured HIP graph")
     ap.add_argument("--attention-only", action="store_true", help="time the attention call alone")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run a plain device copy of this many MiB (a known-size reference for "
@@ -245,6 +246,23 @@ def main():
         step()
     torch.cuda.synchronize()
 
+    graph = None
+    if args.hip_graph:
+        # the step as one HIP graph (the reference replays CUDA graphs for decode steps); the
+        # per-kernel events cannot be recorded inside a graph, so kernel_ms then comes from the
+        # eager steps timed right after the graph loop
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_elapsed = time.perf_counter() - t0
+
     lib.mi_profile_enable(1)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -252,6 +270,8 @@ def main():
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    if graph is not None:
+        elapsed = graph_elapsed
     buf = (ctypes.c_float * args.steps)()
     n_ev = lib.mi_profile_collect(buf, args.steps)
     lib.mi_profile_enable(0)
@@ -278,7 +298,8 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": cfg.name + (", attention call only" if args.attention_only
-                                    else ", step = fused RMSNorm+RoPE+KV-append then paged decode attention"),
+                                    else ", step = fused RMSNorm+RoPE+KV-append then paged decode attention")
+            + (", replayed as one HIP graph" if args.hip_graph else ""),
             "batch": case.q.size(0), "q_heads": cfg.Hq, "kv_heads": cfg.Hkv, "head_dim": cfg.d,
             "chunk_tokens": cfg.chunk, "kv_tokens_total": int(lens_host.sum()), "kv_len_max": max_len,
             "algorithmic_bytes_per_step": nbytes,
