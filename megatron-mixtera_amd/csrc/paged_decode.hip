@@ -319,10 +319,22 @@ static __device__ __forceinline__ bool decode_row(const DecodeParams& p, int r, 
   return p.cu_q[r + 1] - row == 1;
 }
 
+#ifdef MI_DECODE_TRACE  // developer build only: per-workgroup cycle stamps
+__device__ long long mi_decode_trace_buf[1024 * 4];
+#define MI_DECODE_STAMP(slot)                                                              \
+  do {                                                                                     \
+    if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 1024)                          \
+      mi_decode_trace_buf[blockIdx.x * 4 + (slot)] = (long long)wall_clock64();            \
+  } while (0)
+#else
+#define MI_DECODE_STAMP(slot) do { } while (0)
+#endif
+
 template <int HD, int NT, bool FP8, int MINW>
 __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
   constexpr int TK = 16 * NT;
   extern __shared__ int cum[];  // inclusive prefix sum of tiles per request, [R]
+  MI_DECODE_STAMP(0);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -345,10 +357,19 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
     }
   }
   __syncthreads();
+  MI_DECODE_STAMP(1);
   const int total = cum[p.R - 1];
-  const int per = max((total + p.grid - 1) / p.grid, p.min_span_tiles);
-  int t0 = blockIdx.x * per;
-  const int t1 = min(t0 + per, total);
+  // equal spans; the remainder goes one tile each to the first workgroups (rounding the span
+  // up instead would leave the last workgroups without work)
+  int t0, t1;
+  if (total >= p.grid * p.min_span_tiles) {
+    const int per = total / p.grid, rem = total - per * p.grid;
+    t0 = (int)blockIdx.x * per + min((int)blockIdx.x, rem);
+    t1 = t0 + per + ((int)blockIdx.x < rem ? 1 : 0);
+  } else {
+    t0 = blockIdx.x * p.min_span_tiles;
+    t1 = min(t0 + p.min_span_tiles, total);
+  }
   if (t0 >= t1) return;
 
   // first request whose tiles extend beyond t0
@@ -378,6 +399,7 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
     }
     ++r;
   }
+  MI_DECODE_STAMP(2);
 }
 
 // One workgroup per (request, query head): merge the partials of the workgroups that
@@ -550,6 +572,12 @@ int mi::launch_paged_decode(
   else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p);
   return mi_check_launch("mi_paged_decode_attention");
 }
+
+#ifdef MI_DECODE_TRACE
+extern "C" int mi_decode_trace_read(long long* dst, int n) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi::mi_decode_trace_buf), sizeof(long long) * n);
+}
+#endif
 
 extern "C" int mi_paged_decode_attention(
     const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
