@@ -991,6 +991,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   }
 }
 
+
 }  // namespace mi
 
 #ifdef MI_PP_TRACE
