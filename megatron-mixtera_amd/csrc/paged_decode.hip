@@ -319,22 +319,10 @@ static __device__ __forceinline__ bool decode_row(const DecodeParams& p, int r, 
   return p.cu_q[r + 1] - row == 1;
 }
 
-#ifdef MI_DECODE_TRACE  // developer build only: per-workgroup cycle stamps
-__device__ long long mi_decode_trace_buf[1024 * 4];
-#define MI_DECODE_STAMP(slot)                                                              \
-  do {                                                                                     \
-    if (threadIdx.x == 0 && blockIdx.y == 0 && blockIdx.x < 1024)                          \
-      mi_decode_trace_buf[blockIdx.x * 4 + (slot)] = (long long)wall_clock64();            \
-  } while (0)
-#else
-#define MI_DECODE_STAMP(slot) do { } while (0)
-#endif
-
 template <int HD, int NT, bool FP8, int MINW>
 __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
   constexpr int TK = 16 * NT;
   extern __shared__ int cum[];  // inclusive prefix sum of tiles per request, [R]
-  MI_DECODE_STAMP(0);
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -357,7 +345,6 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
     }
   }
   __syncthreads();
-  MI_DECODE_STAMP(1);
   const int total = cum[p.R - 1];
   // equal spans; the remainder goes one tile each to the first workgroups (rounding the span
   // up instead would leave the last workgroups without work)
@@ -399,7 +386,6 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
     }
     ++r;
   }
-  MI_DECODE_STAMP(2);
 }
 
 // One workgroup per (request, query head): merge the partials of the workgroups that
@@ -572,12 +558,6 @@ int mi::launch_paged_decode(
   else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p);
   return mi_check_launch("mi_paged_decode_attention");
 }
-
-#ifdef MI_DECODE_TRACE
-extern "C" int mi_decode_trace_read(long long* dst, int n) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi::mi_decode_trace_buf), sizeof(long long) * n);
-}
-#endif
 
 extern "C" int mi_paged_decode_attention(
     const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,

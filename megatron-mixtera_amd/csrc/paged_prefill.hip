@@ -609,35 +609,11 @@ static __device__ __forceinline__ float rowgroup_max(float x) {
   return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
-#ifdef MI_PP_TRACE  // developer build only: per-phase cycle stamps of one heavy workgroup
-__device__ long long mi_pp_trace_buf[8 * 64 * 8];
-// stamps are parked in LDS (a global store here would sit in the queue the staging waits on)
-#define MI_PP_STAMP(slot)                                                                   \
-  do {                                                                                      \
-    if (rank == 1 && h == 0 && lane == 0 && it >= 8 && it < 72)                             \
-      trace_lds[(wave * 64 + (it - 8)) * 8 + (slot)] = (uint32_t)clock64();                 \
-  } while (0)
-#define MI_PP_CLOCK(var) const long long var = clock64()
-#define MI_PP_STAMP_AT(slot, var)                                                           \
-  do {                                                                                      \
-    if (rank == 1 && h == 0 && lane == 0 && it >= 8 && it < 72)                             \
-      trace_lds[(wave * 64 + (it - 8)) * 8 + (slot)] = (uint32_t)(var);                     \
-  } while (0)
-#else
-#define MI_PP_STAMP(slot) do { } while (0)
-#define MI_PP_CLOCK(var) do { } while (0)
-#define MI_PP_STAMP_AT(slot, var) do { } while (0)
-#endif
-
 template <bool STAGGER>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
   constexpr int HD = 128, KS = 4, DV = 8, NQ = 2, NT = 4, WAVES = 8;
   __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kPPTile * kKPitch];
   __shared__ __attribute__((aligned(16))) uint8_t Vs[3][kPPTile * kVPitch];  // three: see the loop
-#ifdef MI_PP_TRACE
-  __shared__ uint32_t trace_lds[8 * 64 * 8];
-  for (int i = threadIdx.x; i < 8 * 64 * 8; i += 512) trace_lds[i] = 0;
-#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -949,18 +925,13 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     for (int it = 0; it <= ntl; ++it) {
       // (scheduling barriers: MFMAs touch no memory, so nothing else stops the compiler from
       // sinking them past the workgroup barrier into the other phase)
-      MI_PP_CLOCK(c0);
       __builtin_amdgcn_s_setprio(2);  // the matrix-phase wave issues first: its MFMAs are sparse
       matrix_phase(it);               // and must never wait behind the other wave's ALU stream
       __builtin_amdgcn_s_setprio(0);
       MI_SB();
-      MI_PP_CLOCK(c1);
       __syncthreads();
       MI_SB();
-      MI_PP_CLOCK(c2);
       if (it < ntl) softmax(it);
-      MI_PP_CLOCK(c3);
-      MI_PP_STAMP_AT(0, c0); MI_PP_STAMP_AT(1, c1); MI_PP_STAMP_AT(2, c2); MI_PP_STAMP_AT(3, c3);
       MI_SB();
       __syncthreads();
       MI_SB();
@@ -968,11 +939,6 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     if (!lead && STAGGER) __syncthreads();
 #undef MI_SB
   }
-#ifdef MI_PP_TRACE
-  __syncthreads();
-  if (rank == 1 && h == 0)
-    for (int i = tid; i < 8 * 64 * 8; i += 512) mi_pp_trace_buf[i] = trace_lds[i];
-#endif
 
   // ---- epilogue: acc[nt][e][i] is output element d = 16e + 4g + i of row (nt, m16) --------------
 #pragma unroll
@@ -993,12 +959,6 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 
 
 }  // namespace mi
-
-#ifdef MI_PP_TRACE
-extern "C" int mi_pp_trace_read(long long* dst, int n) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(mi::mi_pp_trace_buf), sizeof(long long) * n);
-}
-#endif
 
 using namespace mi;
 
