@@ -74,3 +74,78 @@ def test_padded_requests_with_zero_lengths(mi, dev):
     torch.cuda.synchronize()
     ref = oa.paged_varlen_attention(q.cpu(), kc.cpu(), vc.cpu(), cu_q.cpu(), lens.cpu(), bt.cpu())
     assert (out.float().cpu() - ref).abs().max().item() < 2e-2
+
+
+@pytest.mark.parametrize("pingpong", [1, 2])
+@pytest.mark.parametrize("chunk", [64, 128, 256])
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 1), (16, 2)])
+def test_two_phase_kernel_ragged_lengths(mi, dev, pingpong, chunk, Hq, Hkv):
+    """The two-phase tile kernel (head_dim 128, chunk a multiple of 64): new-token counts and cached
+    contexts around every tile (64 keys), workgroup (256 rows) and chunk boundary, for 1, 2, 4, 8
+    and 16 query heads per KV head, staggered and lock-step."""
+    q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 500, 256, 257, 3]
+    ctx = [0, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0, 40, 7, 64, 63, 1020]
+    d = 128
+    kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    gen = torch.Generator().manual_seed(chunk + Hq)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, gen)
+    q = torch.randn(int(cu_q[-1]), Hq, d, generator=gen).bfloat16().to(dev)
+    kc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
+    vc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
+    mi.ops.set_tuning("prefill_pingpong", pingpong)
+    try:
+        _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
+    finally:
+        mi.ops.set_tuning("prefill_pingpong", 1)
+
+
+def test_stale_cache_rows_beyond_the_length_do_not_leak(mi, dev):
+    """Slots past a request's last token may hold anything (NaN patterns included): the staged tiles
+    re-read the last valid row instead of them."""
+    q, kc, vc, cu_q, lens, bt = mi.synthetic.make_prefill_case(
+        dev, n_prefill=3, new_tokens=70, ctx_lo=3, ctx_hi=200, n_decode=0, dec_lo=1, dec_hi=2,
+        Hq=16, Hkv=4, d=128, chunk=64, seed=11)
+    ref = mi.ops.paged_prefill_attention(q, kc, vc, cu_q, lens, bt).clone()
+    kc2, vc2 = kc.clone(), vc.clone()
+    lens_h, bt_h = lens.cpu(), bt.cpu()
+    for r in range(lens.numel()):
+        L = int(lens_h[r])
+        ci, off = divmod(L, 64)
+        if off:  # poison the unused tail of the last chunk
+            pc = int(bt_h[r, ci])
+            kc2[pc, off:] = float("nan")
+            vc2[pc, off:] = float("nan")
+    out = mi.ops.paged_prefill_attention(q, kc2, vc2, cu_q, lens, bt)
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+
+
+def test_chunked_prefill_is_consistent_at_full_size(mi, dev):
+    """Size-independent property on the cfg3-sized prompts (8 x 2048 tokens over U[0,4096] cached):
+    the rows of the second half of every prompt, computed with the first half already counted as
+    cached context, equal the same rows of the single full call bit for bit (same tiles, same order),
+    and the block table can be permuted without changing a bit."""
+    q, kc, vc, cu_q, lens, bt = mi.synthetic.make_prefill_case(
+        dev, n_prefill=8, new_tokens=2048, ctx_lo=0, ctx_hi=4096, n_decode=0, dec_lo=1, dec_hi=2,
+        Hq=32, Hkv=8, d=128, chunk=256, seed=1003, on_device_rng=True)
+    full = mi.ops.paged_prefill_attention(q, kc, vc, cu_q, lens, bt, max_kv_len=int(lens.max()))
+    torch.cuda.synchronize()
+    assert torch.isfinite(full).all()
+    # second halves only: 1024 new tokens per request, same kv lengths
+    rows = torch.cat([torch.arange(int(cu_q[r]) + 1024, int(cu_q[r + 1]), device=dev) for r in range(8)])
+    cu_half = torch.arange(0, 8 * 1024 + 1, 1024, dtype=torch.int32, device=dev)
+    half = mi.ops.paged_prefill_attention(q[rows].contiguous(), kc, vc, cu_half, lens, bt, max_kv_len=int(lens.max()))
+    torch.cuda.synchronize()
+    assert torch.equal(half, full[rows])
+    # move every chunk to another physical slot
+    N = kc.size(0)
+    perm = torch.randperm(N, generator=torch.Generator().manual_seed(5)).to(dev)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(N, device=dev)
+    kc_p, vc_p = kc[perm], vc[perm]          # chunk i of the new pool is old chunk perm[i]
+    bt_p = inv[bt.long().clamp(min=0)].to(torch.int32)
+    moved = mi.ops.paged_prefill_attention(q, kc_p, vc_p, cu_q, lens, bt_p, max_kv_len=int(lens.max()))
+    torch.cuda.synchronize()
+    assert torch.equal(moved, full)
