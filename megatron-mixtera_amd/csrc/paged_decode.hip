@@ -194,7 +194,10 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     // The scheduling fences keep each batch of prefetch loads together at this point of the
     // loop instead of letting the compiler sink them next to their uses one by one.
     __builtin_amdgcn_sched_barrier(0);
-    load_k(T + 16 * NT);  // prefetch: the K registers are free again
+    // prefetch: the K registers are free again.  Not past the segment's end: that tile belongs to
+    // another workgroup (or does not exist) and would only be streamed from HBM a second time.
+    const bool more = T + 16 * NT < end;  // wave-uniform
+    if (more) load_k(T + 16 * NT);
     __builtin_amdgcn_sched_barrier(0);
     tmax = fmaxf(tmax, xor16(tmax));
     tmax = fmaxf(tmax, xor32(tmax));
@@ -267,7 +270,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    load_v(T + 16 * NT);  // prefetch: the V registers are free again
+    if (more) load_v(T + 16 * NT);  // prefetch: the V registers are free again
     __builtin_amdgcn_sched_barrier(0);
   }
 
