@@ -80,7 +80,10 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   const int m16 = lane & 15, g = lane >> 4;
   const int G = p.G;
   const int hq = h * G + m16;  // query head of this lane's row (valid when m16 < G)
-  const int last = len - 1;
+  // Loads are clamped to the last token of this segment (not of the request): the software
+  // pipeline requests one tile past the end, and that tile belongs to another workgroup's span --
+  // clamped, the request degenerates to re-reading one row instead of streaming 2 tiles from HBM.
+  const int last = min(end, len) - 1;
 
   // Query fragments: B operand rows are the G heads of this KV head.
   uint4 qf[KS];
@@ -194,10 +197,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     // The scheduling fences keep each batch of prefetch loads together at this point of the
     // loop instead of letting the compiler sink them next to their uses one by one.
     __builtin_amdgcn_sched_barrier(0);
-    // prefetch: the K registers are free again.  Not past the segment's end: that tile belongs to
-    // another workgroup (or does not exist) and would only be streamed from HBM a second time.
-    const bool more = T + 16 * NT < end;  // wave-uniform
-    if (more) load_k(T + 16 * NT);
+    load_k(T + 16 * NT);  // prefetch: the K registers are free again
     __builtin_amdgcn_sched_barrier(0);
     tmax = fmaxf(tmax, xor16(tmax));
     tmax = fmaxf(tmax, xor32(tmax));
@@ -270,7 +270,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (more) load_v(T + 16 * NT);  // prefetch: the V registers are free again
+    load_v(T + 16 * NT);  // prefetch: the V registers are free again
     __builtin_amdgcn_sched_barrier(0);
   }
 
