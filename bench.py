@@ -33,7 +33,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 # this same script, each counter scaled by what it reads for a plain 1 GiB device copy
 # (profiles/paged_decode_stream_kernel_cfg2_hbm_traffic.md).  Hardware counters cannot be read from
 # inside the benchmark, so the figure is recorded here per workload; None = not collected.
-MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_210_900_000}
+MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_218_600_000}
 
 
 def parse_args():
