@@ -28,10 +28,13 @@ class DecodeLayerGraphs:
     """Captured decode graphs for a list of :class:`PagedSelfAttentionCore` layers.
 
     ``capture()`` must run while the context is empty (as the reference's warm-up does, before
-    any request is admitted); it walks ``cuda_graph_token_counts`` from the largest size down.
+    any request is admitted); it walks ``cuda_graph_token_counts`` from the largest size down and,
+    when the context was built with ``use_cuda_graphs_for_non_decode_steps`` (the reference's
+    default), captures a second graph per size for prefill / mixed steps
+    (``WarmupEngineMode.NON_DECODE``: the varlen attention path over the padded mirrors).
     ``replay(layer_index, query, key, value)`` copies the step's tensors into the static inputs
-    of the graph for ``context.padded_active_token_count`` and returns the static output
-    ``[padded, 1, Hq*d]`` (valid until the next replay of the same layer and size).
+    of the graph for ``context.padded_active_token_count`` and the step's kind, and returns the
+    static output ``[padded, 1, Hq*d]`` (valid until the next replay of the same graph).
     """
 
     def __init__(self, context, layers: Sequence[torch.nn.Module], *, num_query_heads: int,
@@ -42,7 +45,8 @@ class DecodeLayerGraphs:
         self.layers = list(layers)
         self.num_query_heads = num_query_heads
         self.rotary_pos_emb = rotary_pos_emb
-        self._graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, Tensor, Tensor, Tensor, Tensor]] = {}
+        # (layer index, padded tokens, decode-only?) -> (graph, q, k, v, out)
+        self._graphs: Dict[Tuple[int, int, bool], Tuple[torch.cuda.CUDAGraph, Tensor, Tensor, Tensor, Tensor]] = {}
         self._pool = None
         # one workspace for every graph, sized for the largest decode batch and never re-allocated,
         # so no graph is left holding a pointer into freed memory
@@ -54,7 +58,7 @@ class DecodeLayerGraphs:
 
     @property
     def sizes(self) -> List[int]:
-        return sorted({n for (_, n) in self._graphs})
+        return sorted({n for (_, n, _) in self._graphs})
 
     def capture(self) -> None:
         ctx = self.context
@@ -63,23 +67,29 @@ class DecodeLayerGraphs:
         hkv, d = ctx.num_kv_heads_per_partition, ctx.kv_channels
         dtype = ctx.params_dtype
         side = torch.cuda.Stream(device=dev)
-        for n in ctx.cuda_graph_token_counts:  # largest first, as the reference warms up
-            ctx.initialize_attention_state(num_warmup_tokens=n, warmup_engine_mode=WarmupEngineMode.DECODE)
-            assert ctx.padded_active_token_count == n and ctx.is_decode_only()
-            for li, layer in enumerate(self.layers):
-                q = torch.zeros(n, 1, self.num_query_heads, d, dtype=dtype, device=dev)
-                k = torch.zeros(n, 1, hkv, d, dtype=dtype, device=dev)
-                v = torch.zeros(n, 1, hkv, d, dtype=dtype, device=dev)
-                side.wait_stream(torch.cuda.current_stream(dev))
-                with torch.cuda.stream(side):  # one eager run first (library handles, lazy initialisation)
-                    self._run(layer, q, k, v)
-                torch.cuda.current_stream(dev).wait_stream(side)
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph, pool=self._pool):
-                    out = self._run(layer, q, k, v)
-                if self._pool is None:
-                    self._pool = graph.pool()
-                self._graphs[(li, n)] = (graph, q, k, v, out)
+        modes = [WarmupEngineMode.DECODE]
+        if ctx.non_decode_cuda_graphs:
+            modes.append(WarmupEngineMode.NON_DECODE)
+        for mode in modes:
+            for n in ctx.cuda_graph_token_counts:  # largest first, as the reference warms up
+                ctx.initialize_attention_state(num_warmup_tokens=n, warmup_engine_mode=mode)
+                decode = mode == WarmupEngineMode.DECODE
+                assert ctx.padded_active_token_count == n and ctx.is_decode_only() == decode
+                for li, layer in enumerate(self.layers):
+                    q = torch.zeros(n, 1, self.num_query_heads, d, dtype=dtype, device=dev)
+                    k = torch.zeros(n, 1, hkv, d, dtype=dtype, device=dev)
+                    v = torch.zeros(n, 1, hkv, d, dtype=dtype, device=dev)
+                    side.wait_stream(torch.cuda.current_stream(dev))
+                    with torch.cuda.stream(side):  # one eager run first (library handles, lazy initialisation)
+                        self._run(layer, q, k, v)
+                    torch.cuda.current_stream(dev).wait_stream(side)
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, pool=self._pool):
+                        out = self._run(layer, q, k, v)
+                    if self._pool is None:
+                        self._pool = graph.pool()
+                    self._graphs[(li, n, decode)] = (graph, q, k, v, out)
+                ctx.reset()
         ctx.reset()
 
     def _run(self, layer, q: Tensor, k: Tensor, v: Tensor) -> Tensor:
@@ -89,9 +99,11 @@ class DecodeLayerGraphs:
     def replay(self, layer_index: int, query: Tensor, key: Tensor, value: Tensor) -> Tensor:
         ctx = self.context
         n = ctx.padded_active_token_count
-        entry = self._graphs.get((layer_index, n))
-        if entry is None or not ctx.using_cuda_graph_this_step() or not ctx.is_decode_only():
-            raise KeyError(f"no decode graph for layer {layer_index} and {n} tokens (captured sizes: {self.sizes})")
+        decode = ctx.is_decode_only()
+        entry = self._graphs.get((layer_index, n, decode)) if ctx.using_cuda_graph_this_step() else None
+        if entry is None:
+            raise KeyError(f"no {'decode' if decode else 'prefill'} graph for layer {layer_index} and {n} tokens "
+                           f"(captured sizes: {self.sizes})")
         graph, q, k, v, out = entry
         q.copy_(query[:n])
         k.copy_(key[:n])

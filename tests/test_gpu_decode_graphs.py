@@ -56,14 +56,17 @@ def test_graph_replays_match_eager_steps(mi, dev):
             for c in (ctx_g, ctx_e):
                 c.add_request(i, toks, num_tokens_to_generate=30)
         used = set()
+        kinds = set()
         for step in range(14):
             for c in (ctx_g, ctx_e):
                 c.initialize_attention_state()
             n = ctx_g.padded_active_token_count
-            # only decode-only steps have a captured graph here; prefill / mixed steps (step 0 and the
-            # step after the late admission) run eagerly, padded to a graph size by the context
-            graph_step = ctx_g.using_cuda_graph_this_step() and ctx_g.is_decode_only()
-            assert graph_step == (step not in (0, 10)), step
+            # step 0 (prefill of the prompts) is too large for any graph; every later step replays
+            # one: decode graphs, and the prefill-mode graph for the step after the late admission
+            graph_step = ctx_g.using_cuda_graph_this_step()
+            assert graph_step == (step != 0), step
+            assert ctx_g.is_decode_only() == (step not in (0, 10)), step
+            kinds.add((graph_step, ctx_g.is_decode_only()))
             ne = ctx_e.padded_active_token_count
             for l in range(L):
                 q = torch.randn(max(n, ne), 1, HQ, D, generator=gen).bfloat16().to(dev)
@@ -102,6 +105,7 @@ def test_graph_replays_match_eager_steps(mi, dev):
             for c in (ctx_g, ctx_e):
                 c.update_requests(mask, new)
         assert len(used) >= 2, used
+        assert (True, False) in kinds and (True, True) in kinds  # both kinds of graph were replayed
     finally:
         cls.TOKEN_ROUNDER, cls.REQUEST_ROUNDER = saved
 
