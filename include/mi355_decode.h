@@ -47,8 +47,11 @@ int mi_version(void);
 /* Message of the calling thread's most recent rejected call ("" if none). */
 const char* mi_last_error(void);
 
-/* Experiment knobs: "decode_tile_subtiles" (1|2), "decode_min_waves" (3|4), "decode_wgs_per_cu",
- * "decode_grid" (0 = automatic), "decode_waves_per_block", "prefill_tile_subtiles". */
+/* Experiment knobs (defaults are the measured best; out-of-range values are rejected):
+ * "decode_tile_subtiles" (0 = automatic, 1, 2, 4), "decode_min_waves" (2..4), "decode_wgs_per_cu",
+ * "decode_grid" (0 = automatic), "decode_waves_per_block" (1..8), "prefill_pingpong" (1 = two-phase
+ * tile kernel, 2 = the same kernel with its wave groups in lock-step, 0 = older LDS kernel),
+ * "prefill_tile_subtiles", "prefill_lds_row_tiles", "prefill_row_tiles" (the older kernels). */
 int mi_set_tuning(const char* name, int32_t value);
 
 /*
