@@ -398,22 +398,36 @@ __global__ __launch_bounds__(HD) void paged_decode_merge_kernel(DecodeParams p) 
   const int r = blockIdx.y, hq = blockIdx.x, d = threadIdx.x;
   int row;
   if (!decode_row(p, r, row)) return;
+  // The kernel is a chain of dependent memory round trips, so everything that does not depend
+  // on a loaded value is requested at once: length and segment range here, then LSE and partial
+  // of every segment together (the running-maximum form below needs no first pass over the LSEs).
+  const int len = p.lens[r];
+  const int first = p.seg_info[2 * r], last = p.seg_info[2 * r + 1];  // stale for len <= 0: not used then
   uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + d;
-  if (p.lens[r] <= 0) {
+  if (len <= 0) {
     *o = 0;
     return;
   }
-  const int first = p.seg_info[2 * r], last = p.seg_info[2 * r + 1];
   if (first == last) return;  // written directly by the streaming kernel
-  float mx = -INFINITY;
-  for (int w = first; w <= last; ++w) mx = fmaxf(mx, p.part_lse[(int64_t)(w + r) * p.Hq + hq]);
-  float num = 0.f, den = 0.f;
-#pragma unroll 4
-  for (int w = first; w <= last; ++w) {
-    const int64_t row = (int64_t)(w + r) * p.Hq + hq;
-    const float wt = fast_exp2(p.part_lse[row] - mx);
-    num += wt * p.part_o[row * HD + d];
-    den += wt;
+  float mx = -INFINITY, num = 0.f, den = 0.f;
+  for (int w0 = first; w0 <= last; w0 += 8) {
+    float lse[8], po[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int64_t slot = (int64_t)(min(w0 + j, last) + r) * p.Hq + hq;
+      lse[j] = p.part_lse[slot];
+      po[j] = p.part_o[slot * HD + d];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (w0 + j <= last) {
+        const float m_new = fmaxf(mx, lse[j]);
+        const float a = fast_exp2(mx - m_new), wt = fast_exp2(lse[j] - m_new);
+        num = num * a + wt * po[j];
+        den = den * a + wt;
+        mx = m_new;
+      }
+    }
   }
   *o = f32_to_bf16(num / den);
 }
