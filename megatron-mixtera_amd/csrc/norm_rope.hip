@@ -204,6 +204,169 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
   }
 }
 
+
+// Vectorised variant: a head vector is handled by d/8 lanes with 8 contiguous elements (one 16-byte
+// load / store) each.  The rotary partner of an element is in the same lane (interleaved pairs) or
+// one lane shuffle away (half-split pairs, when rot/2 is a multiple of 8).  Same rounding points as
+// norm_rope_append_kernel; only the order of the sum of squares differs.  grid = (tokens, groups of
+// head vectors) as above, 16 (d = 128) or 32 (d = 64) head vectors per workgroup pass.
+//
+// A token's work starts with a chain of dependent loads (position -> angle row -> cos / sin), so
+// the kernel is latency-bound unless enough workgroups are resident and independent loads are in
+// flight meanwhile: the first pass's head vector and the value row are requested before the chain,
+// and cos / sin / norm weights live in LDS or packed registers to stay within 64 VGPRs (8 waves per
+// SIMD).  Each angle's cos or sin is evaluated by exactly one thread of the workgroup.
+template <int D>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void norm_rope_append_vec_kernel(NormRopeParams p) {
+  constexpr int LPV = D / 8;        // lanes per head vector
+  constexpr int VPW = 64 / LPV;     // head vectors per wave
+  constexpr int VPB = 4 * VPW;      // head vectors per workgroup pass
+  const int t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int li = lane % LPV;
+  const int slot = wave * VPW + lane / LPV;
+  const int nvec = p.Hq + p.Hkv;
+  const bool faithful = p.faithful != 0;
+  const int e0 = 8 * li;  // first element of this lane
+
+  auto load_vec = [&](int vec) -> uint4 {
+    if (vec >= nvec) return make_uint4(0, 0, 0, 0);
+    const uint16_t* src = vec < p.Hq ? p.q + (int64_t)t * p.q_st + (int64_t)vec * D
+                                     : p.k + (int64_t)t * p.k_st + (int64_t)(vec - p.Hq) * D;
+    return ld16(src + e0);
+  };
+  // Independent of the position chain: first head vector, value row (first workgroup of the token).
+  uint4 raw = load_vec(blockIdx.y * VPB + slot);
+  const bool copy_v = blockIdx.y == 0 && p.kc && p.v;
+  const int v_vecs = p.Hkv * D / 8;  // 16-byte pieces of a value row
+  uint4 vraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  if (copy_v) {
+    const uint16_t* src = p.v + (int64_t)t * p.v_st;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+      if ((int)threadIdx.x + 256 * r < v_vecs) vraw[r] = ld16(src + 8 * (threadIdx.x + 256 * r));
+  }
+
+  int64_t cache_off = -1;
+  if (p.kc) {
+    if (p.tok_chunk) {
+      cache_off = p.tok_chunk[t] * p.chunk_elems + p.tok_local[t] * p.tok_elems;
+    } else {
+      const int len = p.lens[t];
+      if (len > 0) {
+        const int pos = len - 1, ci = pos / p.chunk;
+        cache_off = (int64_t)p.bt[(int64_t)t * p.bt_stride + ci] * p.chunk_elems +
+                    (int64_t)(pos - ci * p.chunk) * p.tok_elems;
+      }
+    }
+  }
+
+  __shared__ __align__(16) float cs_lds[2][2][D];  // [query | key position][cos | sin][element]
+  const int half = p.rot >> 1;
+  int src_lane = lane;   // lane holding the half-split partner elements (same j)
+  float psign = 0.f;     // sign of the partner term for half-split pairs
+  bool same = true;      // query and key positions agree (uniform over the workgroup)
+  if (p.emb) {
+    const int64_t qp = p.q_pos ? p.q_pos[t] : 0;
+    const int64_t kp = p.k_pos ? p.k_pos[t] : qp;
+    same = kp == qp && p.Hq > 0;
+    for (int job = threadIdx.x; job < 4 * D; job += 256) {
+      const int which = job / (2 * D), fn = (job / D) & 1, e = job % D;
+      if (which == 1 && same) break;
+      if ((which == 0 && p.Hq == 0) || (which == 1 && p.Hkv == 0)) continue;
+      float r = fn ? 0.f : 1.f;
+      if (e < p.rot) {
+        const float a = p.emb[(which ? kp : qp) * p.emb_stride + e];
+        r = (fn ? sinf(a) : cosf(a)) * p.mscale;
+        if (faithful) r = round_bf16(r);
+      }
+      cs_lds[which][fn][e] = r;
+    }
+    if (!p.interleaved) {
+      const int pe = e0 < half ? e0 + half : e0 - half;  // partner of this lane's first element
+      src_lane = lane - li + pe / 8;
+      psign = e0 < half ? -1.f : 1.f;
+    }
+  }
+  // norm weights of this lane's elements, kept packed
+  uint4 wq_raw = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u), wk_raw = wq_raw;
+  if (p.norm == MI_NORM_RMS) {
+    if (p.q_w) wq_raw = ld16(p.q_w + e0);
+    if (p.k_w) wk_raw = ld16(p.k_w + e0);
+  }
+  if (copy_v && cache_off >= 0) {
+    uint16_t* dst = p.vc + cache_off;
+#pragma unroll
+    for (int r = 0; r < 2; ++r)
+      if ((int)threadIdx.x + 256 * r < v_vecs) st16(dst + 8 * (threadIdx.x + 256 * r), vraw[r]);
+    for (int e = threadIdx.x + 512; e < v_vecs; e += 256)  // more than 32 KV heads of 128
+      st16(dst + 8 * e, ld16(p.v + (int64_t)t * p.v_st + 8 * e));
+  }
+  if (p.emb) __syncthreads();
+
+  for (int vec0 = blockIdx.y * VPB; vec0 < nvec; vec0 += gridDim.y * VPB) {
+    const int vec = vec0 + slot;
+    const bool active = vec < nvec;  // uniform over the LPV lanes of a vector
+    const bool is_q = vec < p.Hq;
+    const int head = is_q ? vec : vec - p.Hq;
+    float y[8];
+    {
+      const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { y[2 * j] = bf16lo_to_f32(w4[j]); y[2 * j + 1] = bf16hi_to_f32(w4[j]); }
+    }
+    raw = load_vec(vec + gridDim.y * VPB);  // next pass, in flight during this one
+    if (p.norm != MI_NORM_NONE) {
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss += y[j] * y[j];
+#pragma unroll
+      for (int o = LPV / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      const float rstd = rsqrtf(ss * (1.f / D) + p.eps);
+      const uint4 wr = is_q ? wq_raw : wk_raw;
+      const uint32_t w4[4] = {wr.x, wr.y, wr.z, wr.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float v = y[j] * rstd;
+        if (p.norm == MI_NORM_RMS) v *= (j & 1) ? bf16hi_to_f32(w4[j >> 1]) : bf16lo_to_f32(w4[j >> 1]);
+        y[j] = faithful ? round_bf16(v) : v;
+      }
+    }
+    float o[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = y[j];
+    if (p.emb) {
+      const int which = (is_q || same) ? 0 : 1;
+      float c[8], sn[8];
+#pragma unroll
+      for (int j = 0; j < 8; j += 4) {
+        const float4 c4 = *reinterpret_cast<const float4*>(&cs_lds[which][0][e0 + j]);
+        const float4 s4 = *reinterpret_cast<const float4*>(&cs_lds[which][1][e0 + j]);
+        c[j] = c4.x; c[j + 1] = c4.y; c[j + 2] = c4.z; c[j + 3] = c4.w;
+        sn[j] = s4.x; sn[j + 1] = s4.y; sn[j + 2] = s4.z; sn[j + 3] = s4.w;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float yp;
+        if (p.interleaved) yp = (j & 1) ? y[j ^ 1] : -y[j ^ 1];
+        else yp = __shfl(y[j], src_lane, 64) * psign;
+        // elements past the rotary width carry cos = 1, sin = 0 in the table
+        if (e0 + j < p.rot) o[j] = faithful ? round_bf16(y[j] * c[j]) + round_bf16(yp * sn[j]) : y[j] * c[j] + yp * sn[j];
+      }
+    }
+    if (active) {
+      const uint4 packed = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]),
+                                      pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+      if (is_q) {
+        st16(p.q_out + (int64_t)t * p.qo_st + (int64_t)head * D + e0, packed);
+      } else {
+        if (p.k_out) st16(p.k_out + (int64_t)t * p.ko_st + (int64_t)head * D + e0, packed);
+        if (cache_off >= 0) st16(p.kc + cache_off + (int64_t)head * D + e0, packed);
+      }
+    }
+  }
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -264,12 +427,26 @@ extern "C" int mi_norm_rope_append(
   hipStream_t st = (hipStream_t)stream;
   // Few tokens (decode): spread the heads of a token over several workgroups for latency.
   // Many tokens (prefill): one workgroup per token loops over the heads and reuses cos / sin.
-  const int vpb = head_dim == 128 ? 4 : 8;
+  // The vectorised kernel needs 16-byte rows and every rotary partner in the same lane or a whole
+  // number of lanes away; anything else takes the element-wise kernel.
+  const bool rot_ok = !rotary_angles || rotary_interleaved || (rot_dim % 16 == 0);
+  const uintptr_t ptrs = (uintptr_t)q | (uintptr_t)q_out | (uintptr_t)k | (uintptr_t)k_out | (uintptr_t)k_cache |
+                         (uintptr_t)q_weight | (uintptr_t)k_weight |
+                         (to_cache ? ((uintptr_t)v | (uintptr_t)v_cache) : 0);
+  const int64_t strides = q_stride_tok | q_out_stride_tok | k_stride_tok | k_out_stride_tok |
+                          (to_cache ? (kv_stride_chunk | kv_stride_tok | v_stride_tok) : 0);
+  const bool vec = rot_ok && (ptrs & 15) == 0 && (strides & 7) == 0 && mi_tuning().norm_rope_vectorised != 0;
+  const int vpb = vec ? (head_dim == 128 ? 16 : 32) : (head_dim == 128 ? 4 : 8);
   const int passes = (Hq + Hkv + vpb - 1) / vpb;
   int gy = (2048 + T - 1) / T;
   gy = gy < 1 ? 1 : (gy > passes ? passes : gy);
   dim3 grid(T, gy);
-  if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), grid, dim3(256), 0, st, p);
-  else hipLaunchKernelGGL((norm_rope_append_kernel<64>), grid, dim3(256), 0, st, p);
+  if (vec) {
+    if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_vec_kernel<128>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((norm_rope_append_vec_kernel<64>), grid, dim3(256), 0, st, p);
+  } else {
+    if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((norm_rope_append_kernel<64>), grid, dim3(256), 0, st, p);
+  }
   return mi_check_launch("mi_norm_rope_append");
 }

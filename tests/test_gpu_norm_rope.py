@@ -24,8 +24,19 @@ def _ulp_diff(a, b):
 
 @pytest.mark.parametrize("norm", [None, "rms", "l2"])
 @pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64)])
-def test_norm_rope_matches_unfused_chain(mi, dev, norm, interleaved, d, rot):
+@pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64), (128, 96), (64, 32), (128, 40)])
+@pytest.mark.parametrize("vectorised", [1, 0])
+def test_norm_rope_matches_unfused_chain(mi, dev, norm, interleaved, d, rot, vectorised):
+    """Both kernels: 16 bytes per lane (taken when every rotary partner is a whole number of lanes
+    away; rot 40 falls back for half-split pairs by itself) and the element-wise one."""
+    mi.ops.set_tuning("norm_rope_vectorised", vectorised)
+    try:
+        _norm_rope_case(mi, dev, norm, interleaved, d, rot)
+    finally:
+        mi.ops.set_tuning("norm_rope_vectorised", 1)
+
+
+def _norm_rope_case(mi, dev, norm, interleaved, d, rot):
     gen = torch.Generator().manual_seed(d + rot + (7 if interleaved else 0))
     T, Hq, Hkv = 37, 8, 2
     q = torch.randn(T, 1, Hq, d, generator=gen).bfloat16()
