@@ -202,6 +202,28 @@ int mi_norm_rope_append(const void* q, int64_t q_stride_tok, void* q_out, int64_
                         int32_t faithful_rounding, void* stream);
 
 /*
+ * The same launch reading the QKV projection's output directly: replaces the split of
+ * SelfAttention.get_query_key_value_tensors (megatron/core/transformer/attention.py:985-1030:
+ * view `[T, Hkv, (Hq/Hkv + 2) * d]`, split into G = Hq/Hkv query heads, one key head and one
+ * value head per query group, reshape of the query to `[T, Hq, d]`) together with everything
+ * mi_norm_rope_append replaces.  mixed_qkv is bf16 `[T][Hkv][(G + 2) * d]` with token stride
+ * qkv_stride_tok (elements); the normed / rotated query goes to q_out `[T, Hq, d]`, the key to
+ * k_out (if non-null) and to the cache slot (if k_cache non-null, together with the value
+ * heads); at least one key destination is required.  Remaining arguments as above.
+ */
+int mi_qkv_norm_rope_append(const void* mixed_qkv, int64_t qkv_stride_tok, void* q_out,
+                            int64_t q_out_stride_tok, void* k_out, int64_t k_out_stride_tok,
+                            const void* q_weight, const void* k_weight, float eps, int32_t norm_kind,
+                            const float* rotary_angles, int64_t angles_stride, int32_t rot_dim,
+                            int32_t rotary_interleaved, float mscale, const int64_t* q_positions,
+                            const int64_t* k_positions, void* k_cache, void* v_cache,
+                            int64_t kv_stride_chunk, int64_t kv_stride_tok,
+                            const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos,
+                            const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
+                            int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv, int32_t head_dim,
+                            int32_t faithful_rounding, void* stream);
+
+/*
  * DynamicInferenceContext.update_requests as one kernel
  * (megatron/core/inference/contexts/dynamic_context.py:1033-1298, allocator
  * dynamic_chunk_allocator.py:56-86): same order of chunk releases, row moves, pauses, LIFO

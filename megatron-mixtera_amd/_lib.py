@@ -49,6 +49,10 @@ SIGNATURES = {
         c_int,
         [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F,
          _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
+    "mi_qkv_norm_rope_append": (
+        c_int,
+        [_P, _I64, _P, _I64, _P, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F,
+         _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
 }
 
 

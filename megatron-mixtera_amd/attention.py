@@ -76,6 +76,25 @@ class PagedSelfAttentionCore(torch.nn.Module):
         else:
             self.q_layernorm_weight = self.k_layernorm_weight = None
 
+    def forward_mixed_qkv(self, mixed_qkv: Tensor, num_query_heads: int, inference_context,
+                          rotary_pos_emb: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
+        """Same as :meth:`forward`, starting from the QKV projection's output ``[T, 1, (Hq + 2 Hkv) d]``:
+        the split of ``get_query_key_value_tensors`` (attention.py:985-1030) is folded into the fused
+        norm / RoPE / append launch, so no per-head q / k / v tensors are materialised."""
+        ctx = inference_context
+        emb = None
+        if rotary_pos_emb is not None:
+            q_emb, k_emb = rotary_pos_emb if isinstance(rotary_pos_emb, tuple) else (rotary_pos_emb,) * 2
+            assert q_emb is k_emb or q_emb is None or k_emb is None or q_emb.data_ptr() == k_emb.data_ptr(), \
+                "the fused path takes one rotary table for query and key"
+            emb = q_emb if q_emb is not None else k_emb
+        query = ctx.fused_qkv_norm_rope_append(
+            self.layer_number, mixed_qkv, num_query_heads=num_query_heads, rotary_pos_emb=emb, config=self.config,
+            q_weight=None if self.q_layernorm_weight is None else self.q_layernorm_weight.data,
+            k_weight=None if self.k_layernorm_weight is None else self.k_layernorm_weight.data,
+            norm=self.qk_norm, eps=self.eps)
+        return self._attend(query, ctx)
+
     def forward(self, query: Tensor, key: Tensor, value: Tensor, inference_context,
                 rotary_pos_emb: Optional[Tuple[Tensor, Tensor]] = None) -> Tensor:
         ctx = inference_context
@@ -102,6 +121,9 @@ class PagedSelfAttentionCore(torch.nn.Module):
             ctx.append_key_value_cache(self.layer_number, key, value)
             if q_emb is not None:
                 query = ctx.apply_rotary_emb_query(query, q_emb, self.config, None, None)
+        return self._attend(query, ctx)
+
+    def _attend(self, query: Tensor, ctx) -> Tensor:
         k_cache, v_cache, block_table = ctx.key_value_cache(self.layer_number)
         cu_q, max_q = ctx.cu_query_lengths()
         cu_k, kv_lens, max_k = ctx.cu_kv_lengths()

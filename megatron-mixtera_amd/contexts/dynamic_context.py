@@ -385,6 +385,35 @@ class DynamicInferenceContext:
             faithful_rounding=faithful_rounding)
         return query
 
+    def fused_qkv_norm_rope_append(self, layer_number: int, mixed_qkv: Tensor, *, num_query_heads: int,
+                                   rotary_pos_emb: Optional[Tensor], config=None,
+                                   q_weight: Optional[Tensor] = None, k_weight: Optional[Tensor] = None,
+                                   norm: Optional[str] = None, eps: float = 1e-5, mscale: float = 1.0,
+                                   faithful_rounding: bool = True, query_out: Optional[Tensor] = None) -> Tensor:
+        """:meth:`fused_qk_norm_rope_append` starting from the QKV projection's output.
+
+        ``mixed_qkv`` is ``[T, 1, (Hq + 2 Hkv) * d]`` in the per-query-group order that
+        ``SelfAttention.get_query_key_value_tensors`` splits (attention.py:985-1030); the split, the
+        query reshape (a copy in the reference), both norms, both RoPE calls and the append run as one
+        launch.  Returns the query ``[T, 1, Hq, d]`` (``query_out`` if given, else a new tensor).
+        """
+        n = self.padded_active_token_count
+        hkv = self.num_kv_heads_per_partition
+        d = self.kv_channels
+        if query_out is None:
+            query_out = torch.empty((mixed_qkv.size(0), 1, num_query_heads, d), dtype=mixed_qkv.dtype,
+                                    device=mixed_qkv.device)
+        ops.qkv_norm_rope_append(
+            mixed_qkv[:n], num_query_heads=num_query_heads, num_kv_heads=hkv, query_out=query_out[:n],
+            q_weight=q_weight, k_weight=k_weight, eps=eps, norm=norm, rotary_emb=rotary_pos_emb,
+            q_positions=self.token_to_pos_ids, k_positions=self.token_to_position_in_request,
+            rotary_interleaved=self._rope_flags(config) if config is not None else False, mscale=mscale,
+            k_cache=self.memory_buffer[0, layer_number - 1], v_cache=self.memory_buffer[1, layer_number - 1],
+            token_to_chunk_idx=self.token_to_chunk_idx,
+            token_to_local_pos=self.token_to_local_position_within_kv_chunk,
+            faithful_rounding=faithful_rounding)
+        return query_out
+
     # ------------------------------------------------------------------ per-step attention state
     def reset_attention_state(self) -> None:
         """Forget the per-step attention metadata (the fixed-address mirrors are zeroed)."""

@@ -21,22 +21,24 @@
 // (d = 64) head vectors of one token per pass, each by d/2 lanes, lane i owning elements i and
 // i + d/2.  The normalised vector goes through a few hundred bytes of LDS so that any rotary
 // pairing (half-split, interleaved, partial rotary width) reads its partner from there.
+#include <stdio.h>
+
 #include "mi_common.h"
 #include "mi_capi_internal.h"
 
 namespace mi {
 
 struct NormRopeParams {
-  const uint16_t* q;  // [T][Hq][d]
-  int64_t q_st;
+  const uint16_t* q;  // [T][Hq][d]; head h at (h / q_group) * q_gst + (h % q_group) * d of its token
+  int64_t q_st, q_gst;
   uint16_t* q_out;  // [T][Hq][d]; may alias q
   int64_t qo_st;
-  const uint16_t* k;  // [T][Hkv][d]
-  int64_t k_st;
+  const uint16_t* k;  // [T][Hkv][d]; head h at h * k_hst of its token
+  int64_t k_st, k_hst;
   uint16_t* k_out;  // [T][Hkv][d] or null
   int64_t ko_st;
-  const uint16_t* v;  // [T][Hkv][d] or null (append only)
-  int64_t v_st;
+  const uint16_t* v;  // [T][Hkv][d] or null (append only); head h at h * v_hst of its token
+  int64_t v_st, v_hst;
   const uint16_t* q_w;  // [d] bf16 or null
   const uint16_t* k_w;
   const float* emb;  // [max_pos][rot] angles, or null for no rotary
@@ -51,11 +53,21 @@ struct NormRopeParams {
   const int32_t* bt;  // slot mode B (decode)
   int64_t bt_stride;
   const int32_t* lens;
-  int32_t T, Hq, Hkv, d, rot, chunk, norm, interleaved, faithful;
+  int32_t T, Hq, Hkv, d, rot, chunk, norm, interleaved, faithful, q_group;
   float eps, mscale;
 };
 
 static __device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+
+// First element of head vector `vec` (query heads first, then key heads) of token t.
+static __device__ __forceinline__ const uint16_t* head_vector(const NormRopeParams& p, int t, int vec) {
+  if (vec < p.Hq) {
+    if (p.q_gst == 0) return p.q + (int64_t)t * p.q_st + (int64_t)vec * p.d;  // one group: contiguous heads
+    const int g = vec / p.q_group;
+    return p.q + (int64_t)t * p.q_st + (int64_t)g * p.q_gst + (int64_t)(vec - g * p.q_group) * p.d;
+  }
+  return p.k + (int64_t)t * p.k_st + (int64_t)(vec - p.Hq) * p.k_hst;
+}
 
 template <int D>
 __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p) {
@@ -134,10 +146,9 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
     const bool active = vec < nvec;
     const bool is_q = vec < p.Hq;
     const int head = is_q ? vec : vec - p.Hq;
-    const uint16_t* src = is_q ? p.q + (int64_t)t * p.q_st + (int64_t)head * D
-                               : p.k + (int64_t)t * p.k_st + (int64_t)head * D;
     float x0 = 0.f, x1 = 0.f;
     if (active) {
+      const uint16_t* src = head_vector(p, t, vec);
       x0 = bf16_to_f32(src[i]);
       x1 = bf16_to_f32(src[i + LPV]);
     }
@@ -198,9 +209,11 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
   }
   // Value rows are copied unchanged (by the first workgroup of the token).
   if (blockIdx.y == 0 && cache_off >= 0 && p.v) {
-    const uint32_t* src = reinterpret_cast<const uint32_t*>(p.v + (int64_t)t * p.v_st);
     uint32_t* dst = reinterpret_cast<uint32_t*>(p.vc + cache_off);
-    for (int e = threadIdx.x; e < p.Hkv * D / 2; e += 256) dst[e] = src[e];
+    for (int e = threadIdx.x; e < p.Hkv * D / 2; e += 256) {
+      const int h = e / (D / 2);
+      dst[e] = *reinterpret_cast<const uint32_t*>(p.v + (int64_t)t * p.v_st + (int64_t)h * p.v_hst + 2 * (e - h * (D / 2)));
+    }
   }
 }
 
@@ -231,20 +244,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
 
   auto load_vec = [&](int vec) -> uint4 {
     if (vec >= nvec) return make_uint4(0, 0, 0, 0);
-    const uint16_t* src = vec < p.Hq ? p.q + (int64_t)t * p.q_st + (int64_t)vec * D
-                                     : p.k + (int64_t)t * p.k_st + (int64_t)(vec - p.Hq) * D;
-    return ld16(src + e0);
+    return ld16(head_vector(p, t, vec) + e0);
   };
   // Independent of the position chain: first head vector, value row (first workgroup of the token).
   uint4 raw = load_vec(blockIdx.y * VPB + slot);
   const bool copy_v = blockIdx.y == 0 && p.kc && p.v;
   const int v_vecs = p.Hkv * D / 8;  // 16-byte pieces of a value row
   uint4 vraw[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+  auto load_v = [&](int piece) -> uint4 {  // piece = 16 bytes of the token's value row
+    const int h = piece / LPV;
+    return ld16(p.v + (int64_t)t * p.v_st + (int64_t)h * p.v_hst + 8 * (piece - h * LPV));
+  };
   if (copy_v) {
-    const uint16_t* src = p.v + (int64_t)t * p.v_st;
 #pragma unroll
     for (int r = 0; r < 2; ++r)
-      if ((int)threadIdx.x + 256 * r < v_vecs) vraw[r] = ld16(src + 8 * (threadIdx.x + 256 * r));
+      if ((int)threadIdx.x + 256 * r < v_vecs) vraw[r] = load_v(threadIdx.x + 256 * r);
   }
 
   int64_t cache_off = -1;
@@ -300,7 +314,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
     for (int r = 0; r < 2; ++r)
       if ((int)threadIdx.x + 256 * r < v_vecs) st16(dst + 8 * (threadIdx.x + 256 * r), vraw[r]);
     for (int e = threadIdx.x + 512; e < v_vecs; e += 256)  // more than 32 KV heads of 128
-      st16(dst + 8 * e, ld16(p.v + (int64_t)t * p.v_st + 8 * e));
+      st16(dst + 8 * e, load_v(e));
   }
   if (p.emb) __syncthreads();
 
@@ -371,6 +385,64 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
 
 using namespace mi;
 
+namespace {
+
+// Argument checks shared by both entry points, kernel choice and launch.  `p` carries every pointer,
+// stride and size; `name` prefixes error messages.
+int norm_rope_launch(NormRopeParams& p, hipStream_t st, const char* name) {
+  char msg[160];
+  auto fail = [&](int code, const char* what) {
+    snprintf(msg, sizeof msg, "%s: %s", name, what);
+    return mi_fail(code, msg);
+  };
+  if (p.T == 0) return MI_OK;
+  if (p.T < 0 || p.Hq < 0 || p.Hkv < 0 || p.Hq + p.Hkv == 0) return fail(MI_ERR_SHAPE, "bad sizes");
+  if ((p.Hq > 0 && (!p.q || !p.q_out)) || (p.Hkv > 0 && !p.k)) return fail(MI_ERR_NULL, "q / q_out / k missing");
+  if (p.d != 64 && p.d != 128) return fail(MI_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
+  if (p.norm != MI_NORM_NONE && p.norm != MI_NORM_RMS && p.norm != MI_NORM_L2)
+    return fail(MI_ERR_UNSUPPORTED, "unknown norm kind");
+  if (p.emb) {
+    if (p.rot <= 0 || p.rot > p.d || (p.rot & 1) || p.emb_stride < p.rot)
+      return fail(MI_ERR_SHAPE, "rot_dim must be even and within head_dim");
+    if ((p.Hq > 0 && !p.q_pos) || (p.Hkv > 0 && !p.k_pos)) return fail(MI_ERR_NULL, "rotary positions missing");
+  }
+  const bool to_cache = p.kc != nullptr;
+  if (to_cache) {
+    if (!p.vc || !p.v) return fail(MI_ERR_NULL, "append needs v and v_cache");
+    const bool mode_a = p.tok_chunk && p.tok_local;
+    const bool mode_b = p.bt && p.lens && p.chunk > 0;
+    if (!mode_a && !mode_b) return fail(MI_ERR_NULL, "append needs per-token slots or block table + lengths");
+    if ((((uintptr_t)p.v | (uintptr_t)p.vc) & 3) || ((p.v_st | p.v_hst | p.chunk_elems | p.tok_elems) & 1))
+      return fail(MI_ERR_ALIGN, "value rows must be 4-byte aligned");
+  }
+  if (!(p.tok_chunk && p.tok_local)) p.tok_chunk = nullptr;
+  // Few tokens (decode): spread the heads of a token over several workgroups for latency.
+  // Many tokens (prefill): one workgroup per token loops over the heads and reuses cos / sin.
+  // The vectorised kernel needs 16-byte rows and every rotary partner in the same lane or a whole
+  // number of lanes away; anything else takes the element-wise kernel.
+  const bool rot_ok = !p.emb || p.interleaved || (p.rot % 16 == 0);
+  const uintptr_t ptrs = (uintptr_t)p.q | (uintptr_t)p.q_out | (uintptr_t)p.k | (uintptr_t)p.k_out | (uintptr_t)p.kc |
+                         (uintptr_t)p.q_w | (uintptr_t)p.k_w | (to_cache ? ((uintptr_t)p.v | (uintptr_t)p.vc) : 0);
+  const int64_t strides = p.q_st | p.q_gst | p.qo_st | p.k_st | p.k_hst | p.ko_st |
+                          (to_cache ? (p.chunk_elems | p.tok_elems | p.v_st | p.v_hst) : 0);
+  const bool vec = rot_ok && (ptrs & 15) == 0 && (strides & 7) == 0 && mi_tuning().norm_rope_vectorised != 0;
+  const int vpb = vec ? (p.d == 128 ? 16 : 32) : (p.d == 128 ? 4 : 8);
+  const int passes = (p.Hq + p.Hkv + vpb - 1) / vpb;
+  int gy = (2048 + p.T - 1) / p.T;
+  gy = gy < 1 ? 1 : (gy > passes ? passes : gy);
+  dim3 grid(p.T, gy);
+  if (vec) {
+    if (p.d == 128) hipLaunchKernelGGL((norm_rope_append_vec_kernel<128>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((norm_rope_append_vec_kernel<64>), grid, dim3(256), 0, st, p);
+  } else {
+    if (p.d == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((norm_rope_append_kernel<64>), grid, dim3(256), 0, st, p);
+  }
+  return mi_check_launch(name);
+}
+
+}  // namespace
+
 extern "C" int mi_norm_rope_append(
     const void* q, int64_t q_stride_tok, void* q_out, int64_t q_out_stride_tok, const void* k,
     int64_t k_stride_tok, void* k_out,
@@ -382,71 +454,60 @@ extern "C" int mi_norm_rope_append(
     const int64_t* token_to_local_pos, const int32_t* block_table, int64_t bt_stride,
     const int32_t* kv_lens, int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv,
     int32_t head_dim, int32_t faithful_rounding, void* stream) {
-  if (T == 0) return MI_OK;
-  if (T < 0 || Hq < 0 || Hkv < 0 || Hq + Hkv == 0)
-    return mi_fail(MI_ERR_SHAPE, "mi_norm_rope_append: bad sizes");
-  if ((Hq > 0 && (!q || !q_out)) || (Hkv > 0 && !k))
-    return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: q / q_out / k missing");
-  if (head_dim != 64 && head_dim != 128)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_norm_rope_append: head_dim must be 64 or 128");
-  if (norm_kind != MI_NORM_NONE && norm_kind != MI_NORM_RMS && norm_kind != MI_NORM_L2)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_norm_rope_append: unknown norm kind");
-  if (rotary_angles) {
-    if (rot_dim <= 0 || rot_dim > head_dim || (rot_dim & 1) || angles_stride < rot_dim)
-      return mi_fail(MI_ERR_SHAPE, "mi_norm_rope_append: rot_dim must be even and within head_dim");
-    if ((Hq > 0 && !q_positions) || (Hkv > 0 && !k_positions))
-      return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: rotary positions missing");
-  }
-  const bool to_cache = k_cache != nullptr;
-  if (to_cache) {
-    if (!v_cache || !v) return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: append needs v and v_cache");
-    const bool mode_a = token_to_chunk_idx && token_to_local_pos;
-    const bool mode_b = block_table && kv_lens && chunk_tokens > 0;
-    if (!mode_a && !mode_b)
-      return mi_fail(MI_ERR_NULL, "mi_norm_rope_append: append needs per-token slots or block table + lengths");
-    if ((((uintptr_t)v | (uintptr_t)v_cache) & 3) || (v_stride_tok & 1) || (kv_stride_chunk & 1) || (kv_stride_tok & 1))
-      return mi_fail(MI_ERR_ALIGN, "mi_norm_rope_append: value rows must be 4-byte aligned");
-  }
   NormRopeParams p = {};
-  p.q = (const uint16_t*)q; p.q_st = q_stride_tok;
+  p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_gst = 0; p.q_group = Hq > 0 ? Hq : 1;
   p.q_out = (uint16_t*)q_out; p.qo_st = q_out_stride_tok;
-  p.k = (const uint16_t*)k; p.k_st = k_stride_tok;
+  p.k = (const uint16_t*)k; p.k_st = k_stride_tok; p.k_hst = head_dim;
   p.k_out = (uint16_t*)k_out; p.ko_st = k_out_stride_tok;
-  p.v = (const uint16_t*)v; p.v_st = v_stride_tok;
+  p.v = (const uint16_t*)v; p.v_st = v_stride_tok; p.v_hst = head_dim;
   p.q_w = (const uint16_t*)q_weight; p.k_w = (const uint16_t*)k_weight;
   p.emb = rotary_angles; p.emb_stride = angles_stride;
   p.q_pos = q_positions; p.k_pos = k_positions;
   p.kc = (uint16_t*)k_cache; p.vc = (uint16_t*)v_cache;
   p.chunk_elems = kv_stride_chunk; p.tok_elems = kv_stride_tok;
-  p.tok_chunk = (token_to_chunk_idx && token_to_local_pos) ? token_to_chunk_idx : nullptr;
-  p.tok_local = token_to_local_pos;
+  p.tok_chunk = token_to_chunk_idx; p.tok_local = token_to_local_pos;
   p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens;
   p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.d = head_dim; p.rot = rot_dim; p.chunk = chunk_tokens;
   p.norm = norm_kind; p.interleaved = rotary_interleaved; p.faithful = faithful_rounding;
   p.eps = eps; p.mscale = mscale;
-  hipStream_t st = (hipStream_t)stream;
-  // Few tokens (decode): spread the heads of a token over several workgroups for latency.
-  // Many tokens (prefill): one workgroup per token loops over the heads and reuses cos / sin.
-  // The vectorised kernel needs 16-byte rows and every rotary partner in the same lane or a whole
-  // number of lanes away; anything else takes the element-wise kernel.
-  const bool rot_ok = !rotary_angles || rotary_interleaved || (rot_dim % 16 == 0);
-  const uintptr_t ptrs = (uintptr_t)q | (uintptr_t)q_out | (uintptr_t)k | (uintptr_t)k_out | (uintptr_t)k_cache |
-                         (uintptr_t)q_weight | (uintptr_t)k_weight |
-                         (to_cache ? ((uintptr_t)v | (uintptr_t)v_cache) : 0);
-  const int64_t strides = q_stride_tok | q_out_stride_tok | k_stride_tok | k_out_stride_tok |
-                          (to_cache ? (kv_stride_chunk | kv_stride_tok | v_stride_tok) : 0);
-  const bool vec = rot_ok && (ptrs & 15) == 0 && (strides & 7) == 0 && mi_tuning().norm_rope_vectorised != 0;
-  const int vpb = vec ? (head_dim == 128 ? 16 : 32) : (head_dim == 128 ? 4 : 8);
-  const int passes = (Hq + Hkv + vpb - 1) / vpb;
-  int gy = (2048 + T - 1) / T;
-  gy = gy < 1 ? 1 : (gy > passes ? passes : gy);
-  dim3 grid(T, gy);
-  if (vec) {
-    if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_vec_kernel<128>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((norm_rope_append_vec_kernel<64>), grid, dim3(256), 0, st, p);
-  } else {
-    if (head_dim == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((norm_rope_append_kernel<64>), grid, dim3(256), 0, st, p);
-  }
-  return mi_check_launch("mi_norm_rope_append");
+  return norm_rope_launch(p, (hipStream_t)stream, "mi_norm_rope_append");
+}
+
+extern "C" int mi_qkv_norm_rope_append(
+    const void* mixed_qkv, int64_t qkv_stride_tok, void* q_out, int64_t q_out_stride_tok, void* k_out,
+    int64_t k_out_stride_tok, const void* q_weight, const void* k_weight, float eps, int32_t norm_kind,
+    const float* rotary_angles, int64_t angles_stride, int32_t rot_dim, int32_t rotary_interleaved,
+    float mscale, const int64_t* q_positions, const int64_t* k_positions, void* k_cache, void* v_cache,
+    int64_t kv_stride_chunk, int64_t kv_stride_tok, const int64_t* token_to_chunk_idx,
+    const int64_t* token_to_local_pos, const int32_t* block_table, int64_t bt_stride,
+    const int32_t* kv_lens, int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv,
+    int32_t head_dim, int32_t faithful_rounding, void* stream) {
+  if (T == 0) return MI_OK;
+  if (!mixed_qkv) return mi_fail(MI_ERR_NULL, "mi_qkv_norm_rope_append: mixed_qkv missing");
+  if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0)
+    return mi_fail(MI_ERR_SHAPE, "mi_qkv_norm_rope_append: query heads must be a positive multiple of KV heads");
+  if (!k_cache && !k_out)
+    return mi_fail(MI_ERR_NULL, "mi_qkv_norm_rope_append: the key needs a destination (k_out and/or the cache)");
+  const int G = Hq / Hkv;
+  const int64_t group = (int64_t)(G + 2) * head_dim;  // elements of one query group: G q heads, k, v
+  if (qkv_stride_tok < group * Hkv)
+    return mi_fail(MI_ERR_SHAPE, "mi_qkv_norm_rope_append: token stride smaller than (Hq + 2 Hkv) * head_dim");
+  const uint16_t* base = (const uint16_t*)mixed_qkv;
+  NormRopeParams p = {};
+  p.q = base; p.q_st = qkv_stride_tok; p.q_gst = group; p.q_group = G;
+  p.q_out = (uint16_t*)q_out; p.qo_st = q_out_stride_tok;
+  p.k = base + (int64_t)G * head_dim; p.k_st = qkv_stride_tok; p.k_hst = group;
+  p.k_out = (uint16_t*)k_out; p.ko_st = k_out_stride_tok;
+  p.v = k_cache ? base + (int64_t)(G + 1) * head_dim : nullptr; p.v_st = qkv_stride_tok; p.v_hst = group;
+  p.q_w = (const uint16_t*)q_weight; p.k_w = (const uint16_t*)k_weight;
+  p.emb = rotary_angles; p.emb_stride = angles_stride;
+  p.q_pos = q_positions; p.k_pos = k_positions;
+  p.kc = (uint16_t*)k_cache; p.vc = (uint16_t*)v_cache;
+  p.chunk_elems = kv_stride_chunk; p.tok_elems = kv_stride_tok;
+  p.tok_chunk = token_to_chunk_idx; p.tok_local = token_to_local_pos;
+  p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens;
+  p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.d = head_dim; p.rot = rot_dim; p.chunk = chunk_tokens;
+  p.norm = norm_kind; p.interleaved = rotary_interleaved; p.faithful = faithful_rounding;
+  p.eps = eps; p.mscale = mscale;
+  return norm_rope_launch(p, (hipStream_t)stream, "mi_qkv_norm_rope_append");
 }

@@ -358,6 +358,59 @@ def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: O
         T, Hq, Hkv, D, int(bool(faithful_rounding)), _stream(ref)), "mi_norm_rope_append")
 
 
+def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_heads: int, query_out: Tensor,
+                         key_out: Optional[Tensor] = None, q_weight: Optional[Tensor] = None,
+                         k_weight: Optional[Tensor] = None, eps: float = 1e-5, norm: Optional[str] = None,
+                         rotary_emb: Optional[Tensor] = None, q_positions: Optional[Tensor] = None,
+                         k_positions: Optional[Tensor] = None, rotary_interleaved: bool = False,
+                         mscale: float = 1.0, k_cache: Optional[Tensor] = None, v_cache: Optional[Tensor] = None,
+                         token_to_chunk_idx: Optional[Tensor] = None, token_to_local_pos: Optional[Tensor] = None,
+                         block_table: Optional[Tensor] = None, kv_lens: Optional[Tensor] = None,
+                         faithful_rounding: bool = True) -> None:
+    """:func:`norm_rope_append` reading the QKV projection's output ``[T, (1,) (Hq + 2 Hkv) * d]`` (per
+    query group: its query heads, then its key head, then its value head -- the layout that
+    ``get_query_key_value_tensors`` splits, attention.py:985-1030) without materialising the split."""
+    lib = _lib.load()
+    _require(mixed_qkv.is_cuda and mixed_qkv.dtype == torch.bfloat16, "mixed_qkv must be a bf16 device tensor")
+    if mixed_qkv.dim() == 3:
+        _require(mixed_qkv.size(1) == 1, "mixed_qkv must be [T, 1, W]")
+        mixed_qkv = mixed_qkv[:, 0]
+    _require(mixed_qkv.dim() == 2 and mixed_qkv.stride(1) == 1, "mixed_qkv must be [T, W] with contiguous rows")
+    T, W = mixed_qkv.shape
+    Hq, Hkv = int(num_query_heads), int(num_kv_heads)
+    _require(Hq > 0 and Hkv > 0 and Hq % Hkv == 0 and W % (Hq + 2 * Hkv) == 0, "mixed_qkv width / head counts")
+    D = W // (Hq + 2 * Hkv)
+    qo3 = _qo_view(query_out, "query_out")
+    _require(tuple(qo3.shape) == (T, Hq, D) and qo3.stride(1) == D, "query_out must be [T, Hq, d]")
+    ko3 = None
+    if key_out is not None:
+        ko3 = _qo_view(key_out, "key_out")
+        _require(tuple(ko3.shape) == (T, Hkv, D) and ko3.stride(1) == D, "key_out must be [T, Hkv, d]")
+    _require(ko3 is not None or k_cache is not None, "the key needs a destination: key_out and/or the cache")
+    ang, a_stride, rot = _angles(rotary_emb)
+    for w in (q_weight, k_weight):
+        _require(w is None or (w.dtype == torch.bfloat16 and w.numel() == D and w.is_contiguous()), "norm weights must be bf16 [d]")
+    for pz in (q_positions, k_positions, token_to_chunk_idx, token_to_local_pos):
+        _require(pz is None or (pz.dtype == torch.int64 and pz.is_contiguous() and pz.numel() >= T), "index rows must be int64 [>=T]")
+    sc = st = 0
+    chunk = 0
+    if k_cache is not None:
+        _require(k_cache.dtype == torch.bfloat16 and v_cache is not None and v_cache.dtype == torch.bfloat16, "bf16 caches")
+        sc, st, sh = _cache_strides(k_cache)
+        _require(_cache_strides(v_cache) == (sc, st, sh) and sh == D, "cache layout")
+        chunk = k_cache.size(1)
+        if block_table is not None:
+            _require(block_table.dtype == torch.int32 and block_table.stride(1) == 1, "bad block_table")
+            _require(kv_lens is not None and kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "bad kv_lens")
+    _lib.check(lib.mi_qkv_norm_rope_append(
+        _ptr(mixed_qkv), mixed_qkv.stride(0), _ptr(qo3), qo3.stride(0), _ptr(ko3), 0 if ko3 is None else ko3.stride(0),
+        _ptr(q_weight), _ptr(k_weight), float(eps), _NORM_KINDS[norm], _ptr(ang), a_stride, rot,
+        int(bool(rotary_interleaved)), float(mscale), _ptr(q_positions), _ptr(k_positions),
+        _ptr(k_cache), _ptr(v_cache), sc, st, _ptr(token_to_chunk_idx), _ptr(token_to_local_pos),
+        _ptr(block_table), 0 if block_table is None else block_table.stride(0), _ptr(kv_lens), chunk,
+        T, Hq, Hkv, D, int(bool(faithful_rounding)), _stream(mixed_qkv)), "mi_qkv_norm_rope_append")
+
+
 # ---------------------------------------------------------------------------------------------
 # context bookkeeping on the GPU
 # ---------------------------------------------------------------------------------------------

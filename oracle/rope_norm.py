@@ -9,12 +9,15 @@ Restates:
   (megatron/core/models/common/embeddings/rope_utils.py:73-126);
 * gather of the table by per-token positions (dynamic_context.py:587-589, 619-621);
 * q/k layernorm = torch RMSNorm over the head dim or L2Norm
-  (megatron/core/transformer/attention.py:1026-1030, torch_norm.py:15-96).
+  (megatron/core/transformer/attention.py:1026-1030, torch_norm.py:15-96);
+* the split of the QKV projection's output into per-head query / key / value
+  (``SelfAttention.get_query_key_value_tensors``, megatron/core/transformer/attention.py:985-1024).
 
 Pinned by (tests/test_oracle_rope_norm.py): position 0 is the identity; fp64 complex
 multiplication by e^{i theta}; pairwise norm preservation; torch.nn.functional.rms_norm
 (library routine); llama-3 scaling against the published three-band formula evaluated in
-fp64 for a low, a medium and a high frequency.
+fp64 for a low, a medium and a high frequency; the QKV split against hand-computed element
+offsets of an ``arange`` row and a scalar triple loop.
 """
 from __future__ import annotations
 
@@ -109,3 +112,19 @@ def norm_rope(x: Tensor, positions: Tensor, table: Optional[Tensor], *, norm: Op
         return x
     tab = table.reshape(table.shape[0], table.shape[-1])
     return apply_rope(x, tab[positions.long()], interleaved, mscale)
+
+
+def split_mixed_qkv(mixed_qkv: Tensor, num_query_heads: int, num_kv_heads: int):
+    """``[T, 1, (Hq + 2 Hkv) d]`` -> query ``[T, 1, Hq, d]``, key and value ``[T, 1, Hkv, d]``.
+
+    The projection's columns are ordered by query group: the G = Hq/Hkv query heads of the group,
+    then its key head, then its value head (attention.py:989-1024: view as
+    ``[sq, b, ng, (np/ng + 2) hn]``, split ``[np/ng * hn, hn, hn]`` along the last dim, reshape the
+    query to ``[sq, b, np, hn]``).
+    """
+    t, b, w = mixed_qkv.shape
+    g = num_query_heads // num_kv_heads
+    d = w // (num_query_heads + 2 * num_kv_heads)
+    grouped = mixed_qkv.view(t, b, num_kv_heads, (g + 2) * d)
+    query, key, value = torch.split(grouped, [g * d, d, d], dim=3)
+    return query.reshape(t, b, num_query_heads, d), key, value

@@ -137,3 +137,42 @@ def test_fused_and_unfused_paths_write_identical_caches(mi, dev):
             assert torch.equal(a, b)
     finally:
         mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER = saved
+
+
+def test_mixed_qkv_entry_matches_split_entry(mi, dev):
+    """``forward_mixed_qkv`` on the projection output == ``forward`` on the tensors the reference's split
+    (attention.py:985-1024) would hand over: same attention output, same cache bits, prefill and decode."""
+    saved = (mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER)
+    try:
+        outs, bufs = [], []
+        for use_mixed in (True, False):
+            gen = torch.Generator().manual_seed(21)
+            ctx = _make_ctx(mi, dev)
+            table_d = orn.rotary_table(96, D, base=10000.0).to(dev)
+            core = mi.PagedSelfAttentionCore(1, D, qk_norm="rms", fused=True, device=dev)
+            core.q_layernorm_weight.data.copy_((1 + 0.02 * torch.randn(D, generator=gen)).bfloat16())
+            core.k_layernorm_weight.data.copy_((1 + 0.02 * torch.randn(D, generator=gen)).bfloat16())
+            for i, n in enumerate([9, 18, 3]):
+                ctx.add_request(i, torch.randint(0, 100, (n,), generator=gen).to(dev), num_tokens_to_generate=8)
+            step_out = []
+            for step in range(3):
+                ctx.initialize_attention_state()
+                n = ctx.padded_active_token_count
+                mixed = torch.randn(n, 1, (HQ + 2 * HKV) * D, generator=gen).bfloat16()
+                if use_mixed:
+                    out = core.forward_mixed_qkv(mixed.to(dev), HQ, ctx, (table_d, table_d))
+                else:
+                    q, k, v = orn.split_mixed_qkv(mixed, HQ, HKV)
+                    out = core(q.contiguous().to(dev), k.contiguous().to(dev), v.contiguous().to(dev), ctx,
+                               (table_d, table_d))
+                step_out.append(out[: ctx.active_token_count].clone())
+                ctx.update_requests(torch.ones(3, dtype=torch.int32, device=dev),
+                                    torch.randint(0, 100, (3,), generator=gen).to(dev))
+            torch.cuda.synchronize()
+            outs.append(step_out)
+            bufs.append(ctx.memory_buffer[:, 0, : ctx.dummy_chunk_idx].clone())
+        assert torch.equal(bufs[0], bufs[1])
+        for a, b in zip(*outs):
+            assert torch.equal(a, b)
+    finally:
+        mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER = saved

@@ -114,3 +114,76 @@ def test_fused_append_writes_rotated_key_and_raw_value(mi, dev, mode):
     assert torch.equal(case.v_cache.cpu()[:dummy], vc0[:dummy])
     k_ref = orn.norm_rope(case.k_new.cpu().squeeze(1), pos, table, norm="rms", weight=w, eps=1e-5)
     assert (k_out.cpu().squeeze(1).float() - k_ref.float()).abs().max().item() <= 4e-2
+
+
+@pytest.mark.parametrize("d,hq,hkv", [(128, 32, 8), (128, 8, 8), (64, 12, 4), (128, 5, 1)])
+@pytest.mark.parametrize("vectorised", [1, 0])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_mixed_qkv_input_equals_split_inputs(mi, dev, d, hq, hkv, vectorised, interleaved):
+    """Reading the QKV projection's output directly gives the bits the same launch produces from the
+    split tensors (attention.py:985-1024), for query, key output, key cache and value cache, and
+    agrees with the op-by-op chain on the checker's split."""
+    mi.ops.set_tuning("norm_rope_vectorised", vectorised)
+    try:
+        gen = torch.Generator().manual_seed(11 + d + hq)
+        T, C = 45, 16
+        mixed = torch.randn(T, 1, (hq + 2 * hkv) * d, generator=gen).bfloat16()
+        q, k, v = orn.split_mixed_qkv(mixed, hq, hkv)
+        qw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16().to(dev)
+        kw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16().to(dev)
+        table = orn.rotary_table(500, d, base=10000.0, interleaved=interleaved)
+        pos = torch.randint(0, 500, (T,), generator=gen)
+        n_chunks = (T + C - 1) // C + 1
+        ci = (torch.randperm(T, generator=gen) // C).long()
+        lo = torch.empty(T, dtype=torch.int64)
+        for c in range(n_chunks):  # distinct slots inside each chunk
+            idx = (ci == c).nonzero().flatten()
+            lo[idx] = torch.randperm(C, generator=gen)[: idx.numel()]
+        common = dict(q_weight=qw, k_weight=kw, norm="rms", eps=1e-5, rotary_emb=table.to(dev), q_positions=pos.to(dev),
+                      k_positions=pos.to(dev), rotary_interleaved=interleaved, token_to_chunk_idx=ci.to(dev),
+                      token_to_local_pos=lo.to(dev))
+        res = []
+        for use_mixed in (True, False):
+            kc = torch.full((n_chunks, C, hkv, d), -1.0, dtype=torch.bfloat16, device=dev)
+            vc = torch.full_like(kc, -1.0)
+            qo = torch.empty(T, 1, hq, d, dtype=torch.bfloat16, device=dev)
+            ko = torch.empty(T, 1, hkv, d, dtype=torch.bfloat16, device=dev)
+            if use_mixed:
+                md = mixed.to(dev)
+                mi.ops.qkv_norm_rope_append(md, num_query_heads=hq, num_kv_heads=hkv, query_out=qo, key_out=ko,
+                                            k_cache=kc, v_cache=vc, **common)
+                torch.cuda.synchronize()
+                assert torch.equal(md.cpu(), mixed), "the projection output must not be modified"
+            else:
+                mi.ops.norm_rope_append(q.contiguous().to(dev), k.contiguous().to(dev), value=v.contiguous().to(dev),
+                                        query_out=qo, key_out=ko, k_cache=kc, v_cache=vc, **common)
+                torch.cuda.synchronize()
+            res.append((qo.cpu(), ko.cpu(), kc.cpu(), vc.cpu()))
+        for a, b in zip(*res):
+            assert torch.equal(a, b)
+        qo, ko, kc, vc = res[0]
+        # value rows are copied bit for bit into their slots, other slots keep the fill
+        vc_ref = torch.full_like(vc, -1.0)
+        vc_ref[ci, lo] = v.squeeze(1)
+        assert torch.equal(vc, vc_ref)
+        assert torch.equal(kc[ci, lo], ko.squeeze(1))
+        q_ref = orn.norm_rope(q.squeeze(1), pos, table, norm="rms", weight=qw.cpu(), eps=1e-5, interleaved=interleaved)
+        k_ref = orn.norm_rope(k.squeeze(1), pos, table, norm="rms", weight=kw.cpu(), eps=1e-5, interleaved=interleaved)
+        for got, ref in ((qo.squeeze(1), q_ref), (ko.squeeze(1), k_ref)):
+            # a last-place difference in cos / sin is many ulps of a result that nearly cancels, so
+            # bound the error absolutely and the number of differing elements
+            err = (got.float() - ref.float()).abs()
+            assert (err <= 2e-2 + 2e-2 * ref.float().abs()).all(), f"max err {err.max().item()}"
+            assert (_ulp_diff(got, ref) > 0).float().mean().item() < 0.01
+    finally:
+        mi.ops.set_tuning("norm_rope_vectorised", 1)
+
+
+def test_mixed_qkv_argument_errors(mi, dev):
+    mixed = torch.zeros(4, 1, (8 + 4) * 128, dtype=torch.bfloat16, device=dev)
+    qo = torch.empty(4, 1, 8, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(ValueError):  # no destination for the key
+        mi.ops.qkv_norm_rope_append(mixed, num_query_heads=8, num_kv_heads=2, query_out=qo)
+    with pytest.raises(ValueError):  # width does not match the head counts
+        mi.ops.qkv_norm_rope_append(mixed, num_query_heads=7, num_kv_heads=2, query_out=qo,
+                                    key_out=torch.empty(4, 1, 2, 128, dtype=torch.bfloat16, device=dev))

@@ -97,3 +97,28 @@ def test_rms_norm_equals_library_routine_and_fp64():
     assert (orn.rms_norm(x, w, 1e-5).double() - ref).abs().max() < 2e-2
     l2 = orn.l2_norm(x, 1e-6).double()
     assert torch.allclose(l2.pow(2).mean(-1), torch.ones(64, 4, dtype=torch.float64), atol=2e-2)
+
+
+def test_split_mixed_qkv_offsets():
+    """Hand-computed column offsets: Hq=4, Hkv=2, d=2 -> per group [q q k v] of width 2 each, so a
+    row 0..15 splits into q = [0 1 | 2 3 | 8 9 | 10 11], k = [4 5 | 12 13], v = [6 7 | 14 15]."""
+    row = torch.arange(16.0).view(1, 1, 16)
+    q, k, v = orn.split_mixed_qkv(row, 4, 2)
+    assert q.flatten().tolist() == [0, 1, 2, 3, 8, 9, 10, 11]
+    assert k.flatten().tolist() == [4, 5, 12, 13]
+    assert v.flatten().tolist() == [6, 7, 14, 15]
+
+
+def test_split_mixed_qkv_scalar_loop():
+    t, hq, hkv, d = 3, 6, 2, 4
+    g = hq // hkv
+    x = torch.randn(t, 1, (hq + 2 * hkv) * d)
+    q, k, v = orn.split_mixed_qkv(x, hq, hkv)
+    assert q.shape == (t, 1, hq, d) and k.shape == (t, 1, hkv, d) and v.shape == (t, 1, hkv, d)
+    for ti in range(t):
+        for grp in range(hkv):
+            base = grp * (g + 2) * d
+            for j in range(g):
+                assert torch.equal(q[ti, 0, grp * g + j], x[ti, 0, base + j * d: base + (j + 1) * d])
+            assert torch.equal(k[ti, 0, grp], x[ti, 0, base + g * d: base + (g + 1) * d])
+            assert torch.equal(v[ti, 0, grp], x[ti, 0, base + (g + 1) * d: base + (g + 2) * d])
