@@ -273,6 +273,49 @@ int mi_decode_attention_state(const int32_t* request_kv_length_offsets,
                               int32_t padded_active_token_count, int32_t dummy_chunk_idx,
                               void* stream);
 
+/*
+ * DynamicInferenceContext.last_token_logits (dynamic_context.py:890-918) as one launch:
+ *   dst[r] = src[cumsum(request_query_lengths)[r] - 1],  r < R
+ * with the running sum taken on the GPU.  src `[T, row_elems]`, dst `[R, row_elems]`, row strides
+ * in elements, 2- or 4-byte elements (logits or hidden states); request_query_lengths points at
+ * the first ACTIVE request's entry.  A bit-exact row copy.
+ */
+int mi_last_token_gather(const void* src, int64_t src_stride_row, void* dst, int64_t dst_stride_row,
+                         const int32_t* request_query_lengths, int32_t R, int32_t row_elems,
+                         int32_t elem_bytes, void* stream);
+
+/*
+ * TextGenerationController.sample_from_logits and the finished-request test that follows it
+ * (megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315,
+ * 503-512) as one launch, one workgroup per row of `logits` `[R, vocab]` (logits_dtype 0 = fp32,
+ * 1 = bf16; row stride in elements):
+ *   top_k == 1             : samples[r] = argmax (lowest index among equal maxima);
+ *   otherwise              : x = logits * (1 / temperature) (rounded to bf16 for bf16 logits, as the
+ *                            reference's in-place division rounds), then
+ *     top_k > 1            : keep x >= the top_k-th largest value (ties kept, as `logits < kth`),
+ *     top_p > 0 (top_k 0)  : order by value, keep the shortest prefix whose softmax mass exceeds
+ *                            top_p (the reference's shifted `cumsum > top_p` rule); values equal to
+ *                            the last kept one are all kept (the reference keeps an unspecified
+ *                            subset of them, torch.sort being unstable),
+ *     softmax over the kept values and ONE draw by inverse CDF in vocabulary order:
+ *     samples[r] = min{ j : sum_{i<=j} p_i > uniform[r] * sum_i p_i },  uniform[r] in [0, 1)
+ *     (the reference draws with torch.multinomial from its own generator: same distribution,
+ *     different stream of random numbers), clamped to [0, vocab_clamp-1] when vocab_clamp > 0.
+ *   Probability mass is summed as 2^-40 fixed point, so a call is reproducible bit for bit.
+ *   cut_values (optional, fp32 [R]) receives the smallest kept value (-inf: nothing filtered).
+ *   active_request_mask (optional, uint8 [R]) = (samples[r] != termination_id) &&
+ *     (request_kv_length_offsets[r] + request_query_lengths[r] + 1 < request_output_lengths[r]);
+ *     the three length rows (optional, all or none) point at the first ACTIVE request's entries.
+ *   A row whose maximum is not finite yields its argmax.
+ */
+int mi_sample_from_logits(const void* logits, int64_t stride_row, int32_t logits_dtype, int32_t R,
+                          int32_t vocab, int32_t top_k, float top_p, float temperature,
+                          const float* uniform, int32_t vocab_clamp, int64_t* samples,
+                          float* cut_values, const int32_t* request_kv_length_offsets,
+                          const int32_t* request_query_lengths,
+                          const int32_t* request_output_lengths, int64_t termination_id,
+                          uint8_t* active_request_mask, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

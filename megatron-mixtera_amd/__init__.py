@@ -9,9 +9,11 @@ Public surface (same names as the reference wherever one exists):
   calls ``Attention.flash_decode_and_prefill`` makes
   (reference: megatron/core/transformer/attention.py:470-601).
 * :mod:`ops` -- thin torch wrappers over the C ABI (KV-append, paged attention,
-  fused norm + RoPE, fp8 KV).
+  fused norm + RoPE, fp8 KV, last-token gather, sampling).
+* :mod:`sampling` -- ``sample_from_logits`` and the finished-request mask on one kernel
+  (reference: megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315).
 """
-from . import ops, synthetic  # noqa: F401
+from . import ops, sampling, synthetic  # noqa: F401
 from .attention import (  # noqa: F401
     PagedSelfAttentionCore,
     adjust_key_value_for_inference,
@@ -33,6 +35,7 @@ from .graphs import DecodeLayerGraphs  # noqa: F401
 
 __all__ = [
     "ops",
+    "sampling",
     "DynamicInferenceContext",
     "ChunkAllocator",
     "WarmupEngineMode",

@@ -563,6 +563,9 @@ class DynamicInferenceContext:
         assert logits.size(1) == self.padded_active_token_count, (
             f"logits.size(1) ({tuple(logits.shape)}) != "
             f"padded_active_token_count ({self.padded_active_token_count}).")
+        if logits.device.type == "cuda" and logits.element_size() in (2, 4) and logits.stride(-1) == 1:
+            # running sum and row copy in one launch
+            return ops.last_token_gather(logits.squeeze(0), self.request_query_lengths[self._active()])
         last = torch.cumsum(self.request_query_lengths[self._active()], dim=0) - 1
         return logits.squeeze(0)[last, :]
 

@@ -1,0 +1,429 @@
+// Tail of a decode step: last-token gather, token sampling and the finished-request mask.
+//
+// What the reference does with torch ops after the forward pass
+// (megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315,
+// 503-530 and megatron/core/inference/contexts/dynamic_context.py:890-918):
+//   * last_token_logits: rows  cumsum(request_query_lengths) - 1  of the `[T, V]` logits;
+//   * sample_from_logits: argmax (top_k == 1), or  logits / temperature -> top-k filter (keep
+//     values >= the k-th largest) or top-p filter (sort descending, keep the shortest prefix
+//     whose softmax mass exceeds top_p) -> softmax -> one multinomial draw per row;
+//   * active_request_mask = (sample != termination_id) & (sequence length + 1 < maximum length).
+//
+// Here a row is never sorted.  One workgroup of 16 wavefronts owns a row and finds the cut
+// value of the filter by selection: a 256-bin histogram over the value range followed by four
+// 8-bit digit passes over the order-preserving integer image of the floats, each pass a re-read
+// of the (cache-resident) row.  Probability mass is carried as 64-bit fixed point
+// (exp(x - max) * 2^40), so every sum is an integer sum: the result does not depend on the
+// order of the atomic additions and a replay of the same call gives the same token.  The draw
+// itself is an inverse-CDF lookup in vocabulary order driven by one caller-supplied uniform
+// number per row (three levels: 16 ranges -> 16 sub-ranges -> elements).
+#include "mi_common.h"
+#include "mi_capi_internal.h"
+
+namespace mi {
+
+struct SampleParams {
+  const void* logits; int64_t stride;  // row stride in elements
+  int32_t R, V;
+  int32_t top_k; float top_p; float inv_temperature;
+  const float* uniform;      // [R], unused for top_k == 1
+  int32_t vocab_clamp;       // > 0: samples are clamped to [0, vocab_clamp - 1]
+  int64_t* samples;          // [R]
+  float* cut_out;            // optional [R]: smallest kept (scaled) logit value, -inf = nothing filtered
+  const int32_t* kv_off; const int32_t* q_len; const int32_t* out_len;  // optional, [R] each
+  int64_t termination_id;
+  uint8_t* active_mask;      // optional [R]
+};
+
+constexpr int kSampleThreads = 1024;
+constexpr int kSampleWaves = kSampleThreads / 64;
+constexpr float kMassOne = 1099511627776.0f;  // 2^40
+
+// float -> uint32 with the same ordering (and back)
+static __device__ __forceinline__ uint32_t order_key(float x) {
+  const uint32_t u = __float_as_uint(x);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+static __device__ __forceinline__ float order_key_value(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+static __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
+  const uint32_t lo = __shfl_xor((uint32_t)v, m, 64), hi = __shfl_xor((uint32_t)(v >> 32), m, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+static __device__ __forceinline__ uint64_t shfl_up_u64(uint64_t v, int d) {
+  const uint32_t lo = __shfl_up((uint32_t)v, d, 64), hi = __shfl_up((uint32_t)(v >> 32), d, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+static __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_u64(v, m);
+  return v;
+}
+static __device__ __forceinline__ uint64_t wave_scan_incl_u64(uint64_t v, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint64_t o = shfl_up_u64(v, d);
+    if (lane >= d) v += o;
+  }
+  return v;
+}
+
+template <bool BF16>
+struct RowReader {
+  const void* row; float inv_t; bool scale;
+  // the value the filters see: logit * (1 / temperature), rounded to the logits' dtype as the
+  // in-place division of the reference rounds it; -0 becomes +0 so that equal values share a key
+  __device__ __forceinline__ float operator()(int i) const {
+    float x;
+    if (BF16) x = bf16_to_f32(reinterpret_cast<const uint16_t*>(row)[i]);
+    else x = reinterpret_cast<const float*>(row)[i];
+    if (scale) {
+      x *= inv_t;
+      if (BF16) x = bf16_to_f32(f32_to_bf16(x));
+    }
+    return x + 0.0f;
+  }
+};
+
+// exp(x - mx) as 2^-40 fixed point; 0 for anything that is not a number below the maximum
+static __device__ __forceinline__ uint64_t mass_of(float x, float mx) {
+  float e = fast_exp2((x - mx) * 1.4426950408889634f);
+  e = e >= 0.f ? e : 0.f;
+  e = e <= 1.f ? e : 1.f;
+  return (uint64_t)(e * kMassOne);
+}
+
+// Adds w to hist[bin] for the active lanes.  When every active lane of the wavefront hits the same
+// bin (values clustered in one bin would otherwise serialise 64 atomics on one address) the
+// wavefront adds its sum once.
+static __device__ __forceinline__ void hist_add(uint64_t* hist, int bin, uint64_t w, bool active, int lane) {
+  const uint64_t m = __builtin_amdgcn_ballot_w64(active);
+  if (m == 0) return;
+  const int first = __builtin_ctzll(m);
+  const int b0 = __builtin_amdgcn_readlane(bin, first);
+  const uint64_t same = __builtin_amdgcn_ballot_w64(active && bin == b0);
+  if (same == m) {
+    const uint64_t s = wave_sum_u64(active ? w : 0);
+    if (lane == first && s) atomicAdd(reinterpret_cast<unsigned long long*>(&hist[b0]), (unsigned long long)s);
+  } else if (active && w) {
+    atomicAdd(reinterpret_cast<unsigned long long*>(&hist[bin]), (unsigned long long)w);
+  }
+}
+
+// Wave 0: first bin b (ascending) whose inclusive running sum, started at `above`, exceeds
+// `target`.  Writes {bin or -1, running sum before that bin} to res[0..1].
+static __device__ void find_crossing(const uint64_t* hist, uint64_t above, uint64_t target, uint64_t* res, int lane) {
+  uint64_t h[4], loc = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) { h[j] = hist[4 * lane + j]; loc += h[j]; }
+  const uint64_t incl = wave_scan_incl_u64(loc, lane) + above;
+  const bool cross = incl > target;
+  const uint64_t m = __builtin_amdgcn_ballot_w64(cross);
+  if (m == 0) {
+    if (lane == 63) { res[0] = (uint64_t)-1; res[1] = incl; }
+    return;
+  }
+  if (lane == __builtin_ctzll(m)) {
+    uint64_t run = incl - loc;
+    int b = 4 * lane;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (run + h[j] > target) break;
+      run += h[j];
+      ++b;
+    }
+    res[0] = (uint64_t)b;
+    res[1] = run;
+  }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) {
+  __shared__ uint64_t hist[256];
+  __shared__ uint64_t res[2];
+  __shared__ uint64_t wsum[kSampleWaves];
+  __shared__ uint32_t red_key[kSampleWaves];
+  __shared__ int32_t red_idx[kSampleWaves];
+  __shared__ float red_min[kSampleWaves];
+  __shared__ int32_t pick[2];
+
+  const int r = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int V = p.V;
+  const bool greedy = p.top_k == 1;
+  RowReader<BF16> val{reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)r * p.stride * (BF16 ? 2 : 4),
+                      p.inv_temperature, !greedy && p.inv_temperature != 1.0f};
+
+  // ---- pass A: maximum (lowest index among equals, NaN counts as largest) and finite minimum ----
+  uint32_t bk = 0; int bi = 0x7fffffff; float mn = INFINITY;
+#pragma unroll 4
+  for (int i = tid; i < V; i += kSampleThreads) {
+    const float x = val(i);
+    const uint32_t k = order_key(x);
+    if (k > bk) { bk = k; bi = i; }
+    if (x > -INFINITY) mn = fminf(mn, x);
+  }
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) {
+    const uint32_t ok = __shfl_xor(bk, m, 64); const int oi = __shfl_xor(bi, m, 64);
+    if (ok > bk || (ok == bk && oi < bi)) { bk = ok; bi = oi; }
+    mn = fminf(mn, __shfl_xor(mn, m, 64));
+  }
+  if (lane == 0) { red_key[wave] = bk; red_idx[wave] = bi; red_min[wave] = mn; }
+  __syncthreads();
+  bk = red_key[0]; bi = red_idx[0]; mn = red_min[0];
+#pragma unroll
+  for (int w = 1; w < kSampleWaves; ++w) {
+    const uint32_t ok = red_key[w]; const int oi = red_idx[w];
+    if (ok > bk || (ok == bk && oi < bi)) { bk = ok; bi = oi; }
+    mn = fminf(mn, red_min[w]);
+  }
+  if (bi >= V) bi = 0;  // only when no element compared greater than the start value
+  const float mx = order_key_value(bk);
+  int sample = bi;
+  uint32_t cut_key = 0;  // keep everything
+
+  // A maximum that is not a finite number leaves no distribution to draw from: take the argmax.
+  const bool drawable = !greedy && fabsf(mx) < INFINITY;
+  if (drawable) {
+    const bool by_count = p.top_k > 1;
+    const bool filtered = by_count || p.top_p > 0.f;
+    if (filtered) {
+      // ---- pass B: 256 linear bins over [mx - range, mx], bin 0 = largest values ----
+      float range = mx - mn;
+      if (!by_count) range = fminf(range, 32.f);  // mass below exp(-32) cannot move a top-p cut
+      const float inv_w = range > 0.f ? 256.f / range : 0.f;
+      auto lin_bin = [&](float x) {
+        const float f = (mx - x) * inv_w;
+        int b = f >= 255.f ? 255 : (int)f;  // NaN (inf * 0) compares false and converts to 0
+        return b < 0 ? 0 : b;
+      };
+      if (tid < 256) hist[tid] = 0;
+      __syncthreads();
+#pragma unroll 4
+      for (int i0 = 0; i0 < V; i0 += kSampleThreads) {
+        const int i = i0 + tid;
+        const bool in = i < V;
+        const float x = in ? val(i) : mx;
+        hist_add(hist, lin_bin(x), by_count ? 1 : mass_of(x, mx), in, lane);
+      }
+      __syncthreads();
+      uint64_t target;
+      if (by_count) {
+        target = (uint64_t)(p.top_k - 1);
+      } else {
+        uint64_t z = 0;
+        for (int j = 0; j < 256; ++j) z += hist[j];  // same LDS words for every lane: broadcast reads
+        target = (uint64_t)((double)p.top_p * (double)z);
+      }
+      if (wave == 0) find_crossing(hist, 0, target, res, lane);
+      __syncthreads();
+      const int lbin = (int)(int64_t)res[0];
+      uint64_t above = res[1];
+      if (lbin >= 0) {
+        // ---- four digit passes over the members of the chosen linear bin ----
+        uint32_t pmask = 0, pval = 0;
+        for (int d = 3; d >= 0; --d) {
+          __syncthreads();
+          if (tid < 256) hist[tid] = 0;
+          __syncthreads();
+#pragma unroll 4
+          for (int i0 = 0; i0 < V; i0 += kSampleThreads) {
+            const int i = i0 + tid;
+            const bool in = i < V;
+            const float x = in ? val(i) : mx;
+            const uint32_t k = order_key(x);
+            const bool member = in && lin_bin(x) == lbin && (k & pmask) == pval;
+            hist_add(hist, 255 - (int)((k >> (8 * d)) & 255u), by_count ? 1 : mass_of(x, mx), member, lane);
+          }
+          __syncthreads();
+          if (wave == 0) find_crossing(hist, above, target, res, lane);
+          __syncthreads();
+          // the crossing lies inside the chosen bin, so a bin is always found
+          const uint32_t digit = 255u - (uint32_t)res[0];
+          above = res[1];
+          pmask |= 0xffu << (8 * d);
+          pval |= digit << (8 * d);
+        }
+        cut_key = pval;
+      }
+    }
+
+    // ---- draw: inverse CDF over the kept elements in vocabulary order ----
+    auto kept_mass = [&](int i) -> uint64_t {
+      const float x = val(i);
+      return order_key(x) >= cut_key ? mass_of(x, mx) : 0;
+    };
+    const int L1 = ((V + kSampleWaves - 1) / kSampleWaves + 63) & ~63;  // elements per first-level range
+    {
+      const int a = wave * L1, b = min(a + L1, V);
+      uint64_t s = 0;
+#pragma unroll 4
+      for (int i = a + lane; i < b; i += 64) s += kept_mass(i);
+      s = wave_sum_u64(s);
+      if (lane == 0) wsum[wave] = s;
+    }
+    __syncthreads();
+    uint64_t total = 0;
+#pragma unroll
+    for (int w = 0; w < kSampleWaves; ++w) total += wsum[w];
+    // total >= 2^40: the maximum itself is always kept
+    uint64_t want = (uint64_t)((double)p.uniform[r] * (double)total);
+    want = want < total ? want : total - 1;
+    int w1 = 0;
+#pragma unroll
+    for (int w = 0; w < kSampleWaves - 1; ++w) {
+      const bool pass = w == w1 && want >= wsum[w];
+      want -= pass ? wsum[w] : 0;
+      w1 += pass ? 1 : 0;
+    }
+    // (ranges after the last non-empty one hold no mass, so w1 stops inside the vocabulary)
+    const int a1 = w1 * L1, b1 = min(a1 + L1, V);
+    const int L2 = (L1 / kSampleWaves + 63) & ~63;  // elements per second-level range
+    __syncthreads();
+    {
+      const int a = min(a1 + wave * L2, b1), b = min(a + L2, b1);
+      uint64_t s = 0;
+      for (int i = a + lane; i < b; i += 64) s += kept_mass(i);
+      s = wave_sum_u64(s);
+      if (lane == 0) wsum[wave] = s;
+    }
+    __syncthreads();
+    int w2 = 0;
+#pragma unroll
+    for (int w = 0; w < kSampleWaves - 1; ++w) {
+      const bool pass = w == w2 && want >= wsum[w];
+      want -= pass ? wsum[w] : 0;
+      w2 += pass ? 1 : 0;
+    }
+    const int a2 = min(a1 + w2 * L2, b1), b2 = min(a2 + L2, b1);
+    if (wave == 0) {
+      // third level: each lane owns a contiguous run of the sub-range
+      const int per = L2 / 64;
+      const int a = min(a2 + lane * per, b2), b = min(a + per, b2);
+      uint64_t s = 0;
+      for (int i = a; i < b; ++i) s += kept_mass(i);
+      const uint64_t incl = wave_scan_incl_u64(s, lane);
+      const uint64_t m = __builtin_amdgcn_ballot_w64(incl > want);
+      const int owner = m ? __builtin_ctzll(m) : 63;
+      if (lane == owner) {
+        uint64_t run = incl - s;
+        int found = b > a ? b - 1 : bi;
+        for (int i = a; i < b; ++i) {
+          run += kept_mass(i);
+          if (run > want) { found = i; break; }
+        }
+        pick[0] = found;
+      }
+    }
+    __syncthreads();
+    sample = pick[0];
+    if (p.vocab_clamp > 0) sample = min(max(sample, 0), p.vocab_clamp - 1);
+  }
+
+  if (tid == 0) {
+    p.samples[r] = sample;
+    if (p.cut_out) p.cut_out[r] = cut_key ? order_key_value(cut_key) : -INFINITY;
+    if (p.active_mask) {
+      bool active = (int64_t)sample != p.termination_id;
+      if (p.kv_off) active = active && (p.kv_off[r] + p.q_len[r] + 1 < p.out_len[r]);
+      p.active_mask[r] = active ? 1 : 0;
+    }
+  }
+}
+
+struct GatherParams {
+  const uint8_t* src; int64_t src_stride_bytes;
+  uint8_t* dst; int64_t dst_stride_bytes;
+  const int32_t* q_len; int32_t R; int64_t row_bytes; int32_t vec;
+};
+
+// dst[r] = src[sum(q_len[0..r]) - 1]; grid = (R, column blocks)
+__global__ __launch_bounds__(256) void last_token_gather_kernel(GatherParams p) {
+  __shared__ int32_t part[4];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  int s = 0;
+  for (int i = tid; i <= r; i += 256) s += p.q_len[i];
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) s += __shfl_xor(s, m, 64);
+  if ((tid & 63) == 0) part[tid >> 6] = s;
+  __syncthreads();
+  const int64_t row = (int64_t)part[0] + part[1] + part[2] + part[3] - 1;
+  if (row < 0) return;
+  const uint8_t* src = p.src + row * p.src_stride_bytes;
+  uint8_t* dst = p.dst + (int64_t)r * p.dst_stride_bytes;
+  const int64_t step = (int64_t)gridDim.y * 256 * p.vec;
+  for (int64_t o = ((int64_t)blockIdx.y * 256 + tid) * p.vec; o < p.row_bytes; o += step) {
+    if (p.vec == 16) st16(dst + o, ld16(src + o));
+    else if (p.vec == 4) *reinterpret_cast<uint32_t*>(dst + o) = *reinterpret_cast<const uint32_t*>(src + o);
+    else *reinterpret_cast<uint16_t*>(dst + o) = *reinterpret_cast<const uint16_t*>(src + o);
+  }
+}
+
+}  // namespace mi
+
+using namespace mi;
+
+extern "C" int mi_last_token_gather(const void* src, int64_t src_stride_row, void* dst, int64_t dst_stride_row,
+                                    const int32_t* request_query_lengths, int32_t R, int32_t row_elems,
+                                    int32_t elem_bytes, void* stream) {
+  if (R == 0 || row_elems == 0) return MI_OK;
+  if (!src || !dst || !request_query_lengths) return mi_fail(MI_ERR_NULL, "mi_last_token_gather: null pointer argument");
+  if (R < 0 || row_elems < 0 || (elem_bytes != 2 && elem_bytes != 4))
+    return mi_fail(MI_ERR_SHAPE, "mi_last_token_gather: need R, row_elems >= 0 and 2- or 4-byte elements");
+  if (src_stride_row < row_elems || dst_stride_row < row_elems)
+    return mi_fail(MI_ERR_SHAPE, "mi_last_token_gather: row strides are shorter than a row");
+  GatherParams p;
+  p.src = (const uint8_t*)src; p.src_stride_bytes = src_stride_row * elem_bytes;
+  p.dst = (uint8_t*)dst; p.dst_stride_bytes = dst_stride_row * elem_bytes;
+  p.q_len = request_query_lengths; p.R = R; p.row_bytes = (int64_t)row_elems * elem_bytes;
+  const bool wide = !(((uintptr_t)src | (uintptr_t)dst | (uintptr_t)p.src_stride_bytes | (uintptr_t)p.dst_stride_bytes |
+                       (uintptr_t)p.row_bytes) & 15);
+  p.vec = wide ? 16 : elem_bytes;
+  const int64_t per_block = 256 * (int64_t)p.vec;
+  int ny = (int)((p.row_bytes + per_block - 1) / per_block);
+  ny = ny < 1 ? 1 : (ny > 64 ? 64 : ny);
+  hipLaunchKernelGGL(last_token_gather_kernel, dim3(R, ny), dim3(256), 0, (hipStream_t)stream, p);
+  return mi_check_launch("mi_last_token_gather");
+}
+
+extern "C" int mi_sample_from_logits(const void* logits, int64_t stride_row, int32_t logits_dtype, int32_t R,
+                                     int32_t vocab, int32_t top_k, float top_p, float temperature,
+                                     const float* uniform, int32_t vocab_clamp, int64_t* samples,
+                                     float* cut_values, const int32_t* request_kv_length_offsets,
+                                     const int32_t* request_query_lengths, const int32_t* request_output_lengths,
+                                     int64_t termination_id, uint8_t* active_request_mask, void* stream) {
+  if (R == 0) return MI_OK;
+  if (!logits || !samples) return mi_fail(MI_ERR_NULL, "mi_sample_from_logits: null pointer argument");
+  if (R < 0 || vocab <= 0 || stride_row < vocab)
+    return mi_fail(MI_ERR_SHAPE, "mi_sample_from_logits: need R >= 0, vocab > 0 and a row stride of at least vocab");
+  if (logits_dtype != 0 && logits_dtype != 1)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_sample_from_logits: logits must be fp32 (0) or bf16 (1)");
+  if (top_k < 0 || !(top_p >= 0.f && top_p <= 1.f))
+    return mi_fail(MI_ERR_SHAPE, "mi_sample_from_logits: need top_k >= 0 and top_p in [0, 1]");
+  if (top_k > 0 && top_p > 0.f)
+    return mi_fail(MI_ERR_SHAPE, "mi_sample_from_logits: cannot have top-p and top-k both greater than zero");
+  if (top_k > vocab) return mi_fail(MI_ERR_SHAPE, "mi_sample_from_logits: top-k is larger than logit size");
+  if (top_k != 1 && !(temperature > 0.f))
+    return mi_fail(MI_ERR_SHAPE, "mi_sample_from_logits: temperature must be positive");
+  if (top_k != 1 && !uniform)
+    return mi_fail(MI_ERR_NULL, "mi_sample_from_logits: sampling needs one uniform number per row");
+  const bool any_len = request_kv_length_offsets || request_query_lengths || request_output_lengths;
+  if (any_len && !(request_kv_length_offsets && request_query_lengths && request_output_lengths))
+    return mi_fail(MI_ERR_NULL, "mi_sample_from_logits: the three request length rows go together");
+  if (any_len && !active_request_mask)
+    return mi_fail(MI_ERR_NULL, "mi_sample_from_logits: request lengths were given without a mask to write");
+  SampleParams p;
+  p.logits = logits; p.stride = stride_row; p.R = R; p.V = vocab;
+  p.top_k = top_k; p.top_p = top_p; p.inv_temperature = top_k == 1 ? 1.0f : 1.0f / temperature;
+  p.uniform = uniform; p.vocab_clamp = vocab_clamp; p.samples = samples; p.cut_out = cut_values;
+  p.kv_off = request_kv_length_offsets; p.q_len = request_query_lengths; p.out_len = request_output_lengths;
+  p.termination_id = termination_id; p.active_mask = active_request_mask;
+  if (logits_dtype == 1)
+    hipLaunchKernelGGL(sample_kernel<true>, dim3(R), dim3(kSampleThreads), 0, (hipStream_t)stream, p);
+  else
+    hipLaunchKernelGGL(sample_kernel<false>, dim3(R), dim3(kSampleThreads), 0, (hipStream_t)stream, p);
+  return mi_check_launch("mi_sample_from_logits");
+}

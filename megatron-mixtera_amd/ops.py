@@ -447,3 +447,66 @@ def decode_attention_state(ctx, n_active_requests: int, padded_tokens: int) -> N
         ctx.token_to_chunk_idx.data_ptr(), ctx.token_to_local_position_within_kv_chunk.data_ptr(),
         ctx.token_to_position_in_request.data_ptr(), ctx.paused_request_count, n_active_requests,
         ctx.active_token_count, padded_tokens, ctx.dummy_chunk_idx, _stream(table)), "mi_decode_attention_state")
+
+
+# ---------------------------------------------------------------------------------------------
+# tail of a decode step: last-token rows, sampling, finished-request mask
+# ---------------------------------------------------------------------------------------------
+def last_token_gather(rows: Tensor, request_query_lengths: Tensor, out: Optional[Tensor] = None) -> Tensor:
+    """``rows[cumsum(request_query_lengths) - 1]`` in one launch (``rows`` is ``[T, E]``; the
+    lengths are those of the active requests, int32)."""
+    lib = _lib.load()
+    stream = _stream(rows)
+    _require(rows.dim() == 2 and rows.stride(1) == 1, "rows must be [T, E] with contiguous E")
+    _require(rows.element_size() in (2, 4), "rows must have 2- or 4-byte elements")
+    _require(request_query_lengths.dtype == torch.int32 and request_query_lengths.dim() == 1
+             and request_query_lengths.is_contiguous(), "request_query_lengths must be a contiguous int32 row")
+    R, E = request_query_lengths.numel(), rows.size(1)
+    if out is None:
+        out = torch.empty(R, E, dtype=rows.dtype, device=rows.device)
+    _require(out.dtype == rows.dtype and tuple(out.shape) == (R, E) and out.stride(1) == 1, "out must be [R, E]")
+    _lib.check(lib.mi_last_token_gather(rows.data_ptr(), rows.stride(0), out.data_ptr(), out.stride(0),
+                                        request_query_lengths.data_ptr(), R, E, rows.element_size(), stream),
+               "mi_last_token_gather")
+    return out
+
+
+def sample_from_logits(logits: Tensor, *, top_k: int = 0, top_p: float = 0.0, temperature: float = 1.0,
+                       uniform: Optional[Tensor] = None, vocab_size: Optional[int] = None,
+                       termination_id: Optional[int] = None, kv_length_offsets: Optional[Tensor] = None,
+                       query_lengths: Optional[Tensor] = None, output_lengths: Optional[Tensor] = None,
+                       return_cut: bool = False):
+    """One launch: filter + draw per row of ``logits`` ``[R, V]`` (fp32 or bf16) and, when
+    ``termination_id`` is given, the uint8 mask of requests that go on generating.
+
+    Returns ``(samples int64 [R], mask uint8 [R] or None)`` and, with ``return_cut``, also the
+    smallest kept value per row (fp32, -inf where nothing was filtered)."""
+    lib = _lib.load()
+    stream = _stream(logits)
+    _require(logits.dim() == 2 and logits.stride(1) == 1, "logits must be [R, V] with contiguous V")
+    _require(logits.dtype in (torch.float32, torch.bfloat16), "logits must be fp32 or bf16")
+    R, V = logits.shape
+    dev = logits.device
+    if top_k != 1:
+        _require(uniform is not None, "sampling needs one uniform number per row")
+        _require(uniform.dtype == torch.float32 and uniform.is_contiguous() and uniform.numel() >= R
+                 and uniform.device == dev, "uniform must be a contiguous fp32 row of at least R numbers")
+    samples = torch.empty(R, dtype=torch.int64, device=dev)
+    mask = None
+    lens = (kv_length_offsets, query_lengths, output_lengths)
+    if termination_id is not None:
+        mask = torch.empty(R, dtype=torch.uint8, device=dev)
+        _require(all(t is None for t in lens) or all(t is not None for t in lens),
+                 "the three request length rows go together")
+        for t in lens:
+            _require(t is None or (t.dtype == torch.int32 and t.is_contiguous() and t.numel() >= R and t.device == dev),
+                     "request length rows must be contiguous int32 rows of at least R entries")
+    else:
+        _require(all(t is None for t in lens), "request lengths without a termination id")
+    cut = torch.empty(R, dtype=torch.float32, device=dev) if return_cut else None
+    _lib.check(lib.mi_sample_from_logits(
+        logits.data_ptr(), logits.stride(0), 1 if logits.dtype == torch.bfloat16 else 0, R, V, int(top_k),
+        float(top_p), float(temperature), _ptr(uniform), int(vocab_size or 0), samples.data_ptr(), _ptr(cut),
+        _ptr(kv_length_offsets), _ptr(query_lengths), _ptr(output_lengths),
+        int(termination_id) if termination_id is not None else -1, _ptr(mask), stream), "mi_sample_from_logits")
+    return (samples, mask, cut) if return_cut else (samples, mask)
