@@ -10,9 +10,9 @@
 //   * active_request_mask = (sample != termination_id) & (sequence length + 1 < maximum length).
 //
 // Here a row is never sorted.  One workgroup of 16 wavefronts owns a row and finds the cut
-// value of the filter by selection: a 256-bin histogram over the value range followed by four
-// 8-bit digit passes over the order-preserving integer image of the floats, each pass a re-read
-// of the (cache-resident) row.  Probability mass is carried as 64-bit fixed point
+// value of the filter by selection: a 256-bin histogram over the value range, then four 8-bit
+// digit passes over the order-preserving integer image of the floats in the chosen bin (its
+// members are listed in LDS; the row is re-read instead when they do not fit).  Probability mass is carried as 64-bit fixed point
 // (exp(x - max) * 2^40), so every sum is an integer sum: the result does not depend on the
 // order of the atomic additions and a replay of the same call gives the same token.  The draw
 // itself is an inverse-CDF lookup in vocabulary order driven by one caller-supplied uniform
@@ -70,22 +70,70 @@ static __device__ __forceinline__ uint64_t wave_scan_incl_u64(uint64_t v, int la
   return v;
 }
 
-template <bool BF16>
+// One row of logits.  VEC = elements per 16-byte load (4 fp32, 8 bf16) when the row is 16-byte
+// aligned, 1 otherwise.
+template <bool BF16, int VEC>
 struct RowReader {
-  const void* row; float inv_t; bool scale;
+  const uint8_t* row; int V; float inv_t; bool scale;
   // the value the filters see: logit * (1 / temperature), rounded to the logits' dtype as the
   // in-place division of the reference rounds it; -0 becomes +0 so that equal values share a key
-  __device__ __forceinline__ float operator()(int i) const {
-    float x;
-    if (BF16) x = bf16_to_f32(reinterpret_cast<const uint16_t*>(row)[i]);
-    else x = reinterpret_cast<const float*>(row)[i];
+  __device__ __forceinline__ float finish(float x) const {
     if (scale) {
       x *= inv_t;
       if (BF16) x = bf16_to_f32(f32_to_bf16(x));
     }
     return x + 0.0f;
   }
+  __device__ __forceinline__ float at(int i) const {
+    return finish(BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(row)[i]) : reinterpret_cast<const float*>(row)[i]);
+  }
+  // elements i0 .. i0+VEC-1 (i0 a multiple of VEC); slots at or past V are left unset
+  __device__ __forceinline__ void load(int i0, float (&x)[VEC]) const {
+    if (VEC > 1 && i0 + VEC <= V) {
+      const uint4 w = ld16(row + (int64_t)i0 * (BF16 ? 2 : 4));
+      const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        float v;
+        if (BF16) v = (j & 1) ? bf16hi_to_f32(u[(j >> 1) & 3]) : bf16lo_to_f32(u[(j >> 1) & 3]);
+        else v = __uint_as_float(u[j & 3]);
+        x[j] = finish(v);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) x[j] = i0 + j < V ? at(i0 + j) : 0.f;
+    }
+  }
 };
+
+// Calls f(i, x, i < end) for every slot of [begin, end) rounded up to whole strides: `nthreads`
+// threads (this one is `t`) take VEC consecutive elements each, U loads in flight.  Every thread
+// makes the same number of calls, so f may use wavefront-wide operations.  begin % VEC == 0.
+template <int U, bool BF16, int VEC, typename F>
+static __device__ __forceinline__ void sweep(const RowReader<BF16, VEC>& rd, int begin, int end, int t, int nthreads, F f) {
+  const int stride = nthreads * VEC;
+  for (int base = begin; base < end; base += U * stride) {
+    float x[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i0 = base + u * stride + t * VEC;
+      if (i0 < end) {
+        rd.load(i0, x[u]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) x[u][j] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i0 = base + u * stride + t * VEC;
+      if (base + u * stride < end) {  // uniform over the participating threads
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) f(i0 + j, x[u][j], i0 + j < end);
+      }
+    }
+  }
+}
 
 // exp(x - mx) as 2^-40 fixed point; 0 for anything that is not a number below the maximum
 static __device__ __forceinline__ uint64_t mass_of(float x, float mx) {
@@ -95,17 +143,19 @@ static __device__ __forceinline__ uint64_t mass_of(float x, float mx) {
   return (uint64_t)(e * kMassOne);
 }
 
-// Adds w to hist[bin] for the active lanes.  When every active lane of the wavefront hits the same
-// bin (values clustered in one bin would otherwise serialise 64 atomics on one address) the
-// wavefront adds its sum once.
-static __device__ __forceinline__ void hist_add(uint64_t* hist, int bin, uint64_t w, bool active, int lane) {
+// Adds weight() to hist[bin] for the active lanes (weight is only evaluated when some lane of the
+// wavefront is active).  When every active lane hits the same bin -- values clustered in one bin
+// would otherwise serialise 64 atomics on one address -- the wavefront adds its sum once.
+template <typename W>
+static __device__ __forceinline__ void hist_add(uint64_t* hist, int bin, bool active, int lane, W weight) {
   const uint64_t m = __builtin_amdgcn_ballot_w64(active);
   if (m == 0) return;
+  const uint64_t w = active ? weight() : 0;
   const int first = __builtin_ctzll(m);
   const int b0 = __builtin_amdgcn_readlane(bin, first);
   const uint64_t same = __builtin_amdgcn_ballot_w64(active && bin == b0);
   if (same == m) {
-    const uint64_t s = wave_sum_u64(active ? w : 0);
+    const uint64_t s = wave_sum_u64(w);
     if (lane == first && s) atomicAdd(reinterpret_cast<unsigned long long*>(&hist[b0]), (unsigned long long)s);
   } else if (active && w) {
     atomicAdd(reinterpret_cast<unsigned long long*>(&hist[bin]), (unsigned long long)w);
@@ -139,7 +189,9 @@ static __device__ void find_crossing(const uint64_t* hist, uint64_t above, uint6
   }
 }
 
-template <bool BF16>
+constexpr int kMemberCap = 4096;  // members of the chosen value bin that fit the LDS list
+
+template <bool BF16, int VEC>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) {
   __shared__ uint64_t hist[256];
   __shared__ uint64_t res[2];
@@ -148,23 +200,25 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   __shared__ int32_t red_idx[kSampleWaves];
   __shared__ float red_min[kSampleWaves];
   __shared__ int32_t pick[2];
+  __shared__ uint32_t member_count;
+  __shared__ uint32_t member_key[kMemberCap];
+  __shared__ uint64_t member_mass[kMemberCap];
 
   const int r = blockIdx.x;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int V = p.V;
   const bool greedy = p.top_k == 1;
-  RowReader<BF16> val{reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)r * p.stride * (BF16 ? 2 : 4),
-                      p.inv_temperature, !greedy && p.inv_temperature != 1.0f};
+  const RowReader<BF16, VEC> rd{reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)r * p.stride * (BF16 ? 2 : 4), V,
+                                p.inv_temperature, !greedy && p.inv_temperature != 1.0f};
+  constexpr int U = VEC > 1 ? 4 : 8;  // loads in flight per thread
 
   // ---- pass A: maximum (lowest index among equals, NaN counts as largest) and finite minimum ----
   uint32_t bk = 0; int bi = 0x7fffffff; float mn = INFINITY;
-#pragma unroll 4
-  for (int i = tid; i < V; i += kSampleThreads) {
-    const float x = val(i);
+  sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
     const uint32_t k = order_key(x);
-    if (k > bk) { bk = k; bi = i; }
-    if (x > -INFINITY) mn = fminf(mn, x);
-  }
+    if (in && (k > bk || (k == bk && i < bi))) { bk = k; bi = i; }
+    if (in && x > -INFINITY) mn = fminf(mn, x);
+  });
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) {
     const uint32_t ok = __shfl_xor(bk, m, 64); const int oi = __shfl_xor(bi, m, 64);
@@ -200,15 +254,13 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
         int b = f >= 255.f ? 255 : (int)f;  // NaN (inf * 0) compares false and converts to 0
         return b < 0 ? 0 : b;
       };
+      auto weight_of = [&](float x) -> uint64_t { return by_count ? (uint64_t)1 : mass_of(x, mx); };
       if (tid < 256) hist[tid] = 0;
+      if (tid == 0) member_count = 0;
       __syncthreads();
-#pragma unroll 4
-      for (int i0 = 0; i0 < V; i0 += kSampleThreads) {
-        const int i = i0 + tid;
-        const bool in = i < V;
-        const float x = in ? val(i) : mx;
-        hist_add(hist, lin_bin(x), by_count ? 1 : mass_of(x, mx), in, lane);
-      }
+      sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int, float x, bool in) {
+        hist_add(hist, lin_bin(x), in, lane, [&] { return weight_of(x); });
+      });
       __syncthreads();
       uint64_t target;
       if (by_count) {
@@ -223,25 +275,49 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
       const int lbin = (int)(int64_t)res[0];
       uint64_t above = res[1];
       if (lbin >= 0) {
-        // ---- four digit passes over the members of the chosen linear bin ----
+        // ---- pass C: list the members of the chosen bin in LDS (wavefront-aggregated append) ----
+        sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int, float x, bool in) {
+          const bool member = in && lin_bin(x) == lbin;
+          const uint64_t m = __builtin_amdgcn_ballot_w64(member);
+          if (m == 0) return;
+          uint32_t base = 0;
+          const int first = __builtin_ctzll(m);
+          if (lane == first) base = atomicAdd(&member_count, (uint32_t)__builtin_popcountll(m));
+          base = __builtin_amdgcn_readlane(base, first);
+          const uint32_t at = base + (uint32_t)__builtin_popcountll(m & (((uint64_t)1 << lane) - 1));
+          if (member && at < (uint32_t)kMemberCap) {
+            member_key[at] = order_key(x);
+            member_mass[at] = weight_of(x);
+          }
+        });
+        __syncthreads();
+        const int n_members = (int)member_count;
+        const bool listed = n_members <= kMemberCap;
+        // ---- four 8-bit digit passes over the members (the LDS list, or the row when it overflowed) ----
         uint32_t pmask = 0, pval = 0;
         for (int d = 3; d >= 0; --d) {
           __syncthreads();
           if (tid < 256) hist[tid] = 0;
           __syncthreads();
-#pragma unroll 4
-          for (int i0 = 0; i0 < V; i0 += kSampleThreads) {
-            const int i = i0 + tid;
-            const bool in = i < V;
-            const float x = in ? val(i) : mx;
-            const uint32_t k = order_key(x);
-            const bool member = in && lin_bin(x) == lbin && (k & pmask) == pval;
-            hist_add(hist, 255 - (int)((k >> (8 * d)) & 255u), by_count ? 1 : mass_of(x, mx), member, lane);
+          if (listed) {
+            for (int j0 = 0; j0 < n_members; j0 += kSampleThreads) {
+              const int j = j0 + tid;
+              const bool in = j < n_members;
+              const uint32_t k = in ? member_key[j] : 0;
+              hist_add(hist, 255 - (int)((k >> (8 * d)) & 255u), in && (k & pmask) == pval, lane,
+                       [&] { return member_mass[j]; });
+            }
+          } else {
+            sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int, float x, bool in) {
+              const uint32_t k = order_key(x);
+              hist_add(hist, 255 - (int)((k >> (8 * d)) & 255u), in && lin_bin(x) == lbin && (k & pmask) == pval, lane,
+                       [&] { return weight_of(x); });
+            });
           }
           __syncthreads();
           if (wave == 0) find_crossing(hist, above, target, res, lane);
           __syncthreads();
-          // the crossing lies inside the chosen bin, so a bin is always found
+          // the crossing lies inside the chosen bin, so a digit is always found
           const uint32_t digit = 255u - (uint32_t)res[0];
           above = res[1];
           pmask |= 0xffu << (8 * d);
@@ -252,16 +328,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
     }
 
     // ---- draw: inverse CDF over the kept elements in vocabulary order ----
-    auto kept_mass = [&](int i) -> uint64_t {
-      const float x = val(i);
-      return order_key(x) >= cut_key ? mass_of(x, mx) : 0;
-    };
+    auto kept_mass = [&](float x) -> uint64_t { return order_key(x) >= cut_key ? mass_of(x, mx) : 0; };
     const int L1 = ((V + kSampleWaves - 1) / kSampleWaves + 63) & ~63;  // elements per first-level range
     {
-      const int a = wave * L1, b = min(a + L1, V);
+      const int a = min(wave * L1, V), b = min(a + L1, V);
       uint64_t s = 0;
-#pragma unroll 4
-      for (int i = a + lane; i < b; i += 64) s += kept_mass(i);
+      sweep<U>(rd, a, b, lane, 64, [&](int, float x, bool in) { s += in ? kept_mass(x) : 0; });
       s = wave_sum_u64(s);
       if (lane == 0) wsum[wave] = s;
     }
@@ -280,13 +352,13 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
       w1 += pass ? 1 : 0;
     }
     // (ranges after the last non-empty one hold no mass, so w1 stops inside the vocabulary)
-    const int a1 = w1 * L1, b1 = min(a1 + L1, V);
+    const int a1 = min(w1 * L1, V), b1 = min(a1 + L1, V);
     const int L2 = (L1 / kSampleWaves + 63) & ~63;  // elements per second-level range
     __syncthreads();
     {
       const int a = min(a1 + wave * L2, b1), b = min(a + L2, b1);
       uint64_t s = 0;
-      for (int i = a + lane; i < b; i += 64) s += kept_mass(i);
+      sweep<1>(rd, a, b, lane, 64, [&](int, float x, bool in) { s += in ? kept_mass(x) : 0; });
       s = wave_sum_u64(s);
       if (lane == 0) wsum[wave] = s;
     }
@@ -304,7 +376,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
       const int per = L2 / 64;
       const int a = min(a2 + lane * per, b2), b = min(a + per, b2);
       uint64_t s = 0;
-      for (int i = a; i < b; ++i) s += kept_mass(i);
+      for (int i = a; i < b; ++i) s += kept_mass(rd.at(i));
       const uint64_t incl = wave_scan_incl_u64(s, lane);
       const uint64_t m = __builtin_amdgcn_ballot_w64(incl > want);
       const int owner = m ? __builtin_ctzll(m) : 63;
@@ -312,7 +384,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
         uint64_t run = incl - s;
         int found = b > a ? b - 1 : bi;
         for (int i = a; i < b; ++i) {
-          run += kept_mass(i);
+          run += kept_mass(rd.at(i));
           if (run > want) { found = i; break; }
         }
         pick[0] = found;
@@ -421,9 +493,16 @@ extern "C" int mi_sample_from_logits(const void* logits, int64_t stride_row, int
   p.uniform = uniform; p.vocab_clamp = vocab_clamp; p.samples = samples; p.cut_out = cut_values;
   p.kv_off = request_kv_length_offsets; p.q_len = request_query_lengths; p.out_len = request_output_lengths;
   p.termination_id = termination_id; p.active_mask = active_request_mask;
-  if (logits_dtype == 1)
-    hipLaunchKernelGGL(sample_kernel<true>, dim3(R), dim3(kSampleThreads), 0, (hipStream_t)stream, p);
-  else
-    hipLaunchKernelGGL(sample_kernel<false>, dim3(R), dim3(kSampleThreads), 0, (hipStream_t)stream, p);
+  const int esize = logits_dtype == 1 ? 2 : 4;
+  const bool wide = !(((uintptr_t)logits | (uintptr_t)(stride_row * esize)) & 15);  // 16-byte loads
+  const dim3 grid(R), block(kSampleThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (logits_dtype == 1) {
+    if (wide) hipLaunchKernelGGL((sample_kernel<true, 8>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((sample_kernel<true, 1>), grid, block, 0, st, p);
+  } else {
+    if (wide) hipLaunchKernelGGL((sample_kernel<false, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((sample_kernel<false, 1>), grid, block, 0, st, p);
+  }
   return mi_check_launch("mi_sample_from_logits");
 }
