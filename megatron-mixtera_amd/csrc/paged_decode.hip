@@ -77,6 +77,14 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   constexpr int DV = HD / 16;
   static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
   constexpr int ESZ = FP8 ? 1 : 2;
+  // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
+  // tile base addresses below run on the scalar unit instead of costing vector instructions.
+  r = __builtin_amdgcn_readfirstlane(r);
+  row = __builtin_amdgcn_readfirstlane(row);
+  len = __builtin_amdgcn_readfirstlane(len);
+  start = __builtin_amdgcn_readfirstlane(start);
+  end = __builtin_amdgcn_readfirstlane(end);
+  slot = __builtin_amdgcn_readfirstlane(slot);
   const int m16 = lane & 15, g = lane >> 4;
   const int G = p.G;
   const int hq = h * G + m16;  // query head of this lane's row (valid when m16 < G)
@@ -102,7 +110,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * ESZ;
   const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * ESZ;
   const int64_t chunk_bytes = p.kv_sc * ESZ;
-  const int tok_bytes = p.kv_st * ESZ;
+  const uint32_t tok_bytes = (uint32_t)(p.kv_st * ESZ);
 
   float m_run = -INFINITY, l_run = 0.f;
   f32x4_t acc[DV];
@@ -118,42 +126,98 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   uint2 vf8[NT][4];   // bf16 HD=64 or fp8 HD=128 : 8 B per token
   float ksc[NT], vsc[NT];
 
-  // Tokens past the end are clamped to the last valid one: the data stays finite and
-  // their probabilities are forced to zero below.  That also makes a request for a tile
-  // beyond `end` harmless (it re-reads the last token's rows).
-  auto load_k = [&](int T) {
+  // Addressing.  A tile of 16*NT tokens never straddles a chunk (the launcher picks NT so that the
+  // tile size divides the chunk size), so its address is
+  //   cache + table entry * chunk_bytes + (token inside the chunk) * tok_bytes        -- all scalar --
+  // plus a per-lane byte offset that is fixed for the whole kernel:
+  //   K: lane (m16, g) reads 16 B at column 16g (+64 per step) of row m16 of a sub-tile;
+  //   V: lane (m16, g) reads its DV values of rows 4g .. 4g+3.
+  // Tokens past the end are clamped to the last valid one (row offset min(row, rows left)): the
+  // data stays finite and their probabilities are forced to zero below.  That also makes a request
+  // for a tile beyond `end` harmless (it re-reads the last token's rows).
+  const uint32_t k_col = 16u * (uint32_t)g, v_col = (uint32_t)(DV * m16 * ESZ);
+  const uint32_t k_lane = (uint32_t)m16 * tok_bytes + k_col;
+  uint32_t v_lane[4];
 #pragma unroll
-    for (int u = 0; u < NT; ++u) {
-      const int T0 = T + 16 * u;
-      const int tu = min(T0, last);  // wave-uniform
-      const int ci = chunk_of(tu, p.chunk_magic);
-      const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
-      const uint8_t* kc = kbase + (int64_t)pc * chunk_bytes;
-      if (FP8) ksc[u] = p.k_scale[(int64_t)pc * p.Hkv + h];
-      const int tk = min(T0 + m16, last) - ci * p.chunk;
-      const uint8_t* krow = kc + tk * tok_bytes;
+  for (int j = 0; j < 4; ++j) v_lane[j] = (uint32_t)(4 * g + j) * tok_bytes + v_col;
+
+  // Block-table cursor: the entries of the current chunk and of the next one as scalars, the one
+  // after that still in flight; with fp8 the scale of the next chunk is in flight too.  An entry is
+  // requested two chunks (its scale one chunk) before its first use, so after the start of a
+  // segment the stream never waits for the table.  One cursor each for K and V (V runs half an
+  // iteration behind K).
+  const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
+  const int ci_last = chunk_of(last, p.chunk_magic);
+  struct Cursor {
+    int ci;            // chunk the scalars describe
+    int pc, pc_next;   // its table entry and the next chunk's
+    int pc_after;      // per-lane copy of the entry two chunks ahead (load may be in flight)
+    float sc;          // fp8: scale of (pc, h)
+    float sc_next;     // per-lane copy of the next chunk's scale (load may be in flight)
+  };
+  auto entry_load = [&](int ci) { return bt_row[min(ci, ci_last)]; };
+  auto scale_load = [&](const float* scales, int pc) { return scales[(int64_t)pc * p.Hkv + h]; };
+  auto uniform_f = [](float x) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(x))); };
+  auto cursor_open = [&](Cursor& c, const float* scales, int ci) {
+    c.ci = ci;
+    c.pc = __builtin_amdgcn_readfirstlane(entry_load(ci));
+    c.pc_next = __builtin_amdgcn_readfirstlane(entry_load(ci + 1));
+    c.pc_after = entry_load(ci + 2);
+    c.sc = FP8 ? uniform_f(scale_load(scales, c.pc)) : 1.f;
+    c.sc_next = FP8 ? scale_load(scales, c.pc_next) : 1.f;
+  };
+  // the clamped tile start only ever moves forward, by at most one chunk per tile
+  auto cursor_follow = [&](Cursor& c, const float* scales, int ci) {
+    if (ci != c.ci) {
+      c.ci = ci;
+      c.pc = c.pc_next;
+      c.pc_next = __builtin_amdgcn_readfirstlane(c.pc_after);
+      c.pc_after = entry_load(ci + 2);
       if (FP8) {
-#pragma unroll
-        for (int kk = 0; kk < KS / 2; ++kk) kf[u][kk] = ld16_stream(krow + 64 * kk + 16 * g);
-      } else {
-#pragma unroll
-        for (int kk = 0; kk < KS; ++kk) kf[u][kk] = ld16_stream(krow + (32 * kk + 8 * g) * 2);
+        c.sc = uniform_f(c.sc_next);
+        c.sc_next = scale_load(scales, c.pc_next);
       }
     }
   };
-  auto load_v = [&](int T) {
+  Cursor kcur, vcur;
+  {
+    const int ci0 = chunk_of(min(start, last), p.chunk_magic);
+    cursor_open(kcur, p.k_scale, ci0);
+    cursor_open(vcur, p.v_scale, ci0);
+  }
+
+  // chunk base (scalar) of the tile that starts at T; `row0` = chunk-relative row of token 0 of the chunk
+  auto tile_chunk = [&](Cursor& c, const float* scales, const uint8_t* base, int T, int& tok0) {
+    const int ci = chunk_of(min(T, last), p.chunk_magic);
+    cursor_follow(c, scales, ci);
+    tok0 = ci * p.chunk;
+    return base + (int64_t)c.pc * chunk_bytes;
+  };
+  auto load_k = [&](int T) {
+    int tok0;
+    const uint8_t* chunk = tile_chunk(kcur, p.k_scale, kbase, T, tok0);
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
-      const int T0 = T + 16 * u;
-      const int tu = min(T0, last);
-      const int ci = chunk_of(tu, p.chunk_magic);
-      const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
-      const uint8_t* vc = vbase + (int64_t)pc * chunk_bytes;
-      if (FP8) vsc[u] = p.v_scale[(int64_t)pc * p.Hkv + h];
+      const int t0 = min(T + 16 * u, last);
+      const uint32_t lim = (uint32_t)min(last - t0, 15) * tok_bytes;
+      const uint8_t* krow = chunk + (uint32_t)(t0 - tok0) * tok_bytes + min(k_lane, lim + k_col);
+      if (FP8) ksc[u] = kcur.sc;
+#pragma unroll
+      for (int kk = 0; kk < (FP8 ? KS / 2 : KS); ++kk) kf[u][kk] = ld16_stream(krow + 64 * kk);
+    }
+  };
+  auto load_v = [&](int T) {
+    int tok0;
+    const uint8_t* chunk = tile_chunk(vcur, p.v_scale, vbase, T, tok0);
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      const int t0 = min(T + 16 * u, last);
+      const uint32_t cap = (uint32_t)min(last - t0, 15) * tok_bytes + v_col;
+      const uint8_t* tile = chunk + (uint32_t)(t0 - tok0) * tok_bytes;
+      if (FP8) vsc[u] = vcur.sc;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int tv = min(T0 + 4 * g + j, last) - ci * p.chunk;
-        const uint8_t* vrow = vc + tv * tok_bytes + DV * m16 * ESZ;
+        const uint8_t* vrow = tile + min(v_lane[j], cap);
         if (!FP8 && HD == 128) vf16[u][j] = ld16_stream(vrow);
         else vf8[u][j] = ld8_stream(vrow);
       }
@@ -524,6 +588,7 @@ int mi::launch_paged_decode(
   // 16-token sub-tiles per loop iteration (0 = automatic).
   int nt = mi_tuning().decode_tile_subtiles;
   if (nt != 1 && nt != 2 && nt != 4) nt = kv_dtype == MI_KV_FP8_E4M3 ? 4 : 2;
+  while (chunk_tokens % (16 * nt)) nt >>= 1;  // a tile must not straddle two chunks
   const int minw = mi_tuning().decode_min_waves;
   const int tk = 16 * nt;
   const int min_span_tokens = split_tokens > 0 ? split_tokens : 256;
