@@ -29,7 +29,8 @@
 //       fully coalesced row loads) and transposes the 4 x (d/16) block in
 //       registers with byte permutes to build the A operand.
 //   Softmax statistics are per query row = per m16, so only the running max
-//   needs a cross-lane step (two exchanges across g).
+//   needs a cross-lane step (two exchanges across g); the row sums are one more
+//   16x16x16 product with an all-ones A operand.
 //
 // A second kernel merges the partials of each request,
 //   o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max),
@@ -227,8 +228,13 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   load_k(start);
   load_v(start);
   __builtin_amdgcn_sched_barrier(0);
+  const uint2 ones = make_uint2(0x3f803f80u, 0x3f803f80u);  // four bf16 1.0
   for (int T = start; T < end; T += 16 * NT) {
     // ---- S^T = K Q^T ---------------------------------------------------------
+    // The tile lies in one chunk, so one K scale and one V scale hold for all of it; the score
+    // multiplier is positive and wave-uniform, so the maximum is taken over the raw products.
+    const float mul = FP8 ? p.scale_log2 * ksc[0] : p.scale_log2;
+    const bool ragged = T + 16 * NT > end;  // only the last tile of a segment has masked tokens
     float sc[NT][4];
     float tmax = -INFINITY;
 #pragma unroll
@@ -246,18 +252,17 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32(kf[u][kk], qf[kk], sacc);
       }
-      const float mul = FP8 ? p.scale_log2 * ksc[u] : p.scale_log2;
-      const int tok0 = T + 16 * u + 4 * g;
+      if (ragged) {
+        const int tok0 = T + 16 * u + 4 * g;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float v = (tok0 + i < end) ? sacc[i] * mul : -INFINITY;
-        sc[u][i] = v;
-        tmax = fmaxf(tmax, v);
+        for (int i = 0; i < 4; ++i)
+          if (tok0 + i >= end) sacc[i] = -INFINITY;
       }
-    }
-    float vmul[NT];
 #pragma unroll
-    for (int u = 0; u < NT; ++u) vmul[u] = FP8 ? vsc[u] : 1.f;
+      for (int i = 0; i < 4; ++i) sc[u][i] = sacc[i];
+      tmax = fmaxf(fmaxf(tmax, sacc[0]), fmaxf(sacc[1], fmaxf(sacc[2], sacc[3])));
+    }
+    const float vscale = FP8 ? vsc[0] : 1.f;
     // The scheduling fences keep each batch of prefetch loads together at this point of the
     // loop instead of letting the compiler sink them next to their uses one by one.
     __builtin_amdgcn_sched_barrier(0);
@@ -267,29 +272,30 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     tmax = fmaxf(tmax, xor32(tmax));
 
     // ---- online softmax (row = m16, all lane-local after the max) -----------
-    const float m_new = fmaxf(m_run, tmax);
+    // p = 2^(s * mul - m) [* V scale, folded into the exponent]; the row sums come from the
+    // matrix cores (an all-ones A operand), complete over the 16 tokens of a sub-tile.
+    const float m_new = fmaxf(m_run, tmax * mul);
     const float alpha = fast_exp2(m_run - m_new);
     m_run = m_new;
-    float psum = 0.f;
+    const float neg = FP8 ? fast_log2(vscale) - m_new : -m_new;
     uint2 pf[NT];
+    f32x4_t psum4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
-      float pv[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        pv[i] = fast_exp2(sc[u][i] - m_new);
-        psum += pv[i];
-      }
-      if (FP8) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) pv[i] *= vmul[u];
-      }
-      pf[u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+      const float p0 = fast_exp2(__builtin_fmaf(sc[u][0], mul, neg));
+      const float p1 = fast_exp2(__builtin_fmaf(sc[u][1], mul, neg));
+      const float p2 = fast_exp2(__builtin_fmaf(sc[u][2], mul, neg));
+      const float p3 = fast_exp2(__builtin_fmaf(sc[u][3], mul, neg));
+      pf[u] = make_uint2(pack_bf16x2(p0, p1), pack_bf16x2(p2, p3));
+      psum4 = mfma_16x16x16(ones, pf[u], psum4);
     }
-    l_run = l_run * alpha + psum;
+    // (every slot of psum4 holds the row sum of this lane's query row)
+    l_run = l_run * alpha + (FP8 ? psum4[0] * __builtin_amdgcn_rcpf(vscale) : psum4[0]);
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {  // the running maximum rarely moves after the first tiles
 #pragma unroll
-    for (int e = 0; e < DV; ++e) {
-      acc[e][0] *= alpha; acc[e][1] *= alpha; acc[e][2] *= alpha; acc[e][3] *= alpha;
+      for (int e = 0; e < DV; ++e) {
+        acc[e][0] *= alpha; acc[e][1] *= alpha; acc[e][2] *= alpha; acc[e][3] *= alpha;
+      }
     }
 
     // ---- O^T += V^T P^T --------------------------------------------------------
@@ -339,8 +345,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   }
 
   // ---- epilogue ---------------------------------------------------------------
-  float l_tot = l_run + xor16(l_run);
-  l_tot += xor32(l_tot);
+  const float l_tot = l_run;  // already summed over the lanes of a row (matrix-core row sums)
   const float inv = 1.f / l_tot;
   if (m16 >= G) return;  // (no barrier follows inside a segment)
   // acc[e][i] holds d = DV*(4g+i) + e: DV*4 contiguous values per lane.
