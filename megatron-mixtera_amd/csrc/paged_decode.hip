@@ -159,14 +159,6 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   auto entry_load = [&](int ci) { return bt_row[min(ci, ci_last)]; };
   auto scale_load = [&](const float* scales, int pc) { return scales[(int64_t)pc * p.Hkv + h]; };
   auto uniform_f = [](float x) { return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(x))); };
-  auto cursor_open = [&](Cursor& c, const float* scales, int ci) {
-    c.ci = ci;
-    c.pc = __builtin_amdgcn_readfirstlane(entry_load(ci));
-    c.pc_next = __builtin_amdgcn_readfirstlane(entry_load(ci + 1));
-    c.pc_after = entry_load(ci + 2);
-    c.sc = FP8 ? uniform_f(scale_load(scales, c.pc)) : 1.f;
-    c.sc_next = FP8 ? scale_load(scales, c.pc_next) : 1.f;
-  };
   // the clamped tile start only ever moves forward, by at most one chunk per tile
   auto cursor_follow = [&](Cursor& c, const float* scales, int ci) {
     if (ci != c.ci) {
@@ -180,11 +172,25 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       }
     }
   };
+  // Opening: one round trip for the three table entries, shared by both cursors; the scales are
+  // requested next and only waited for after the first tiles' loads have been issued.
   Cursor kcur, vcur;
+  float ksc_first = 1.f, vsc_first = 1.f;  // per-lane copies, loads in flight
   {
     const int ci0 = chunk_of(min(start, last), p.chunk_magic);
-    cursor_open(kcur, p.k_scale, ci0);
-    cursor_open(vcur, p.v_scale, ci0);
+    const int e0 = entry_load(ci0), e1 = entry_load(ci0 + 1), e2 = entry_load(ci0 + 2);
+    kcur.ci = ci0;
+    kcur.pc = __builtin_amdgcn_readfirstlane(e0);
+    kcur.pc_next = __builtin_amdgcn_readfirstlane(e1);
+    kcur.pc_after = e2;
+    kcur.sc = kcur.sc_next = 1.f;
+    vcur = kcur;
+    if (FP8) {
+      ksc_first = scale_load(p.k_scale, kcur.pc);
+      vsc_first = scale_load(p.v_scale, kcur.pc);
+      kcur.sc_next = scale_load(p.k_scale, kcur.pc_next);
+      vcur.sc_next = scale_load(p.v_scale, kcur.pc_next);
+    }
   }
 
   // chunk base (scalar) of the tile that starts at T; `row0` = chunk-relative row of token 0 of the chunk
@@ -228,6 +234,12 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   load_k(start);
   load_v(start);
   __builtin_amdgcn_sched_barrier(0);
+  if (FP8) {  // the first tile lies in the opening chunk
+    kcur.sc = uniform_f(ksc_first);
+    vcur.sc = uniform_f(vsc_first);
+#pragma unroll
+    for (int u = 0; u < NT; ++u) { ksc[u] = kcur.sc; vsc[u] = vcur.sc; }
+  }
   const uint2 ones = make_uint2(0x3f803f80u, 0x3f803f80u);  // four bf16 1.0
   for (int T = start; T < end; T += 16 * NT) {
     // ---- S^T = K Q^T ---------------------------------------------------------
@@ -394,7 +406,8 @@ static __device__ __forceinline__ bool decode_row(const DecodeParams& p, int r, 
 template <int HD, int NT, bool FP8, int MINW>
 __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
   constexpr int TK = 16 * NT;
-  extern __shared__ int cum[];  // inclusive prefix sum of tiles per request, [R]
+  extern __shared__ int cum[];  // inclusive prefix sum of tiles per request, [R], then the lengths, [R]
+  int* const len_s = cum + p.R;
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -406,13 +419,17 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
     for (int base = 0; base < p.R; base += 64) {
       const int i = base + lane;
       int row_unused;
-      int v = (i < p.R && decode_row(p, i, row_unused)) ? tiles_of(p.lens[i], TK) : 0;
+      const int len_i = i < p.R ? p.lens[i] : 0;
+      int v = (i < p.R && decode_row(p, i, row_unused)) ? tiles_of(len_i, TK) : 0;
 #pragma unroll
       for (int o = 1; o < 64; o <<= 1) {
         const int up = __shfl_up(v, o, 64);
         if (lane >= o) v += up;
       }
-      if (i < p.R) cum[i] = carry + v;
+      if (i < p.R) {
+        cum[i] = carry + v;
+        len_s[i] = len_i;  // a segment start then costs no trip to memory for the length
+      }
       carry += __shfl(v, 63, 64);
     }
   }
@@ -442,7 +459,7 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
     const int rb = r ? cum[r - 1] : 0;
     const int re = cum[r];
     if (re > t0) {  // requests without tiles (length 0) are skipped
-      const int len = p.lens[r];
+      const int len = len_s[r];
       const int tb = t0 - rb;             // first tile of the segment, within the request
       const int te = min(t1, re) - rb;    // one past its last tile
       const bool first = tb == 0, final = te == re - rb;
@@ -579,8 +596,8 @@ int mi::launch_paged_decode(
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: one chunk must span less than 2 GiB");
   if (split_tokens < 0 || split_tokens % 16)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: split_tokens must be a non-negative multiple of 16");
-  if ((int64_t)R * sizeof(int32_t) > 60 * 1024)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: batch too large for the in-LDS prefix sum");
+  if ((int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: batch too large for the in-LDS prefix sum (7680 requests)");
 
   const int grid_x = decode_grid_size(Hkv);
   const int64_t slots = (int64_t)grid_x + R;
@@ -616,7 +633,7 @@ int mi::launch_paged_decode(
 
   const int wpb = pick_waves_per_block(Hkv);
   dim3 grid(grid_x, Hkv / wpb), block(64 * wpb);
-  const size_t lds = (size_t)R * sizeof(int32_t);
+  const size_t lds = (size_t)R * 2 * sizeof(int32_t);
   hipStream_t st = (hipStream_t)stream;
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
