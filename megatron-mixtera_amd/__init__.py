@@ -12,8 +12,10 @@ Public surface (same names as the reference wherever one exists):
   fused norm + RoPE, fp8 KV, last-token gather, sampling).
 * :mod:`sampling` -- ``sample_from_logits`` and the finished-request mask on one kernel
   (reference: megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315).
+* :mod:`step` -- ``generate_output_tokens_dynamic_batch``: one engine step on a context with the
+  model behind a callable (reference: the same file, :411-546).
 """
-from . import ops, sampling, synthetic  # noqa: F401
+from . import ops, sampling, step, synthetic  # noqa: F401
 from .attention import (  # noqa: F401
     PagedSelfAttentionCore,
     adjust_key_value_for_inference,
@@ -36,6 +38,7 @@ from .graphs import DecodeLayerGraphs  # noqa: F401
 __all__ = [
     "ops",
     "sampling",
+    "step",
     "DynamicInferenceContext",
     "ChunkAllocator",
     "WarmupEngineMode",
