@@ -31,9 +31,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 
 # HBM bytes per launch of the streaming kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this same script, each counter scaled by what it reads for a plain 1 GiB device copy
-# (profiles/paged_decode_stream_kernel_cfg2_hbm_traffic.md).  Hardware counters cannot be read from
-# inside the benchmark, so the figure is recorded here per workload; None = not collected.
-MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_218_600_000}
+# (profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md).  Hardware counters cannot be
+# read from inside the benchmark, so the figure is recorded here per workload; None = not collected.
+MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_226_800_000, "cfg4": 8_724_000_000, "cfg5": 9_070_100_000}
 
 
 def parse_args():
