@@ -301,7 +301,7 @@ int mi_last_token_gather(const void* src, int64_t src_stride_row, void* dst, int
  *     samples[r] = min{ j : sum_{i<=j} p_i > uniform[r] * sum_i p_i },  uniform[r] in [0, 1)
  *     (the reference draws with torch.multinomial from its own generator: same distribution,
  *     different stream of random numbers), clamped to [0, vocab_clamp-1] when vocab_clamp > 0.
- *   Probability mass is summed as 2^-40 fixed point, so a call is reproducible bit for bit.
+ *   Probability mass is summed as fixed point (each term rounded to 2^-32), so a call is reproducible bit for bit.
  *   cut_values (optional, fp32 [R]) receives the smallest kept value (-inf: nothing filtered).
  *   active_request_mask (optional, uint8 [R]) = (samples[r] != termination_id) &&
  *     (request_kv_length_offsets[r] + request_query_lengths[r] + 1 < request_output_lengths[r]);

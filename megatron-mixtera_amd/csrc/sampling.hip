@@ -13,7 +13,7 @@
 // value of the filter by selection: a 256-bin histogram over the value range, then four 8-bit
 // digit passes over the order-preserving integer image of the floats in the chosen bin (its
 // members are listed in LDS; the row is re-read instead when they do not fit).  Probability mass is carried as 64-bit fixed point
-// (exp(x - max) * 2^40), so every sum is an integer sum: the result does not depend on the
+// (exp(x - max) rounded to 2^-32), so every sum is an integer sum: the result does not depend on the
 // order of the atomic additions and a replay of the same call gives the same token.  The draw
 // itself is an inverse-CDF lookup in vocabulary order driven by one caller-supplied uniform
 // number per row (three levels: 16 ranges -> 16 sub-ranges -> elements).
@@ -37,7 +37,6 @@ struct SampleParams {
 
 constexpr int kSampleThreads = 1024;
 constexpr int kSampleWaves = kSampleThreads / 64;
-constexpr float kMassOne = 1099511627776.0f;  // 2^40
 
 // float -> uint32 with the same ordering (and back)
 static __device__ __forceinline__ uint32_t order_key(float x) {
@@ -87,7 +86,23 @@ struct RowReader {
   __device__ __forceinline__ float at(int i) const {
     return finish(BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(row)[i]) : reinterpret_cast<const float*>(row)[i]);
   }
-  // elements i0 .. i0+VEC-1 (i0 a multiple of VEC); slots at or past V are left unset
+  // elements i0 .. i0+VEC-1 (i0 a multiple of VEC), all inside the row
+  __device__ __forceinline__ void load_full(int i0, float (&x)[VEC]) const {
+    if (VEC > 1) {
+      const uint4 w = ld16(row + (int64_t)i0 * (BF16 ? 2 : 4));
+      const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) {
+        float v;
+        if (BF16) v = (j & 1) ? bf16hi_to_f32(u[(j >> 1) & 3]) : bf16lo_to_f32(u[(j >> 1) & 3]);
+        else v = __uint_as_float(u[j & 3]);
+        x[j] = finish(v);
+      }
+    } else {
+      x[0] = at(i0);
+    }
+  }
+  // the same with slots at or past V set to 0
   __device__ __forceinline__ void load(int i0, float (&x)[VEC]) const {
     if (VEC > 1 && i0 + VEC <= V) {
       const uint4 w = ld16(row + (int64_t)i0 * (BF16 ? 2 : 4));
@@ -109,10 +124,24 @@ struct RowReader {
 // Calls f(i, x, i < end) for every slot of [begin, end) rounded up to whole strides: `nthreads`
 // threads (this one is `t`) take VEC consecutive elements each, U loads in flight.  Every thread
 // makes the same number of calls, so f may use wavefront-wide operations.  begin % VEC == 0.
+// Whole blocks of U strides run without any bounds test (the flag is the constant true there);
+// only the rest of the range pays for guards.
 template <int U, bool BF16, int VEC, typename F>
 static __device__ __forceinline__ void sweep(const RowReader<BF16, VEC>& rd, int begin, int end, int t, int nthreads, F f) {
   const int stride = nthreads * VEC;
-  for (int base = begin; base < end; base += U * stride) {
+  const int row_end = rd.V - (rd.V % VEC);  // whole 16-byte groups of the row end here
+  int base = begin;
+  for (; base + U * stride <= min(end, row_end); base += U * stride) {
+    float x[U][VEC];
+#pragma unroll
+    for (int u = 0; u < U; ++u) rd.load_full(base + u * stride + t * VEC, x[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int j = 0; j < VEC; ++j) f(base + u * stride + t * VEC + j, x[u][j], true);
+    }
+  }
+  if (base < end) {  // the rest: fewer than U strides, guarded, loads still issued together
     float x[U][VEC];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -135,12 +164,12 @@ static __device__ __forceinline__ void sweep(const RowReader<BF16, VEC>& rd, int
   }
 }
 
-// exp(x - mx) as 2^-40 fixed point; 0 for anything that is not a number below the maximum
-static __device__ __forceinline__ uint64_t mass_of(float x, float mx) {
-  float e = fast_exp2((x - mx) * 1.4426950408889634f);
-  e = e >= 0.f ? e : 0.f;
-  e = e <= 1.f ? e : 1.f;
-  return (uint64_t)(e * kMassOne);
+// exp(x - mx) as fixed point, rounded to the nearest 2^-32: one 32-bit conversion per element
+// (sums are carried in 64 bits).  0 for anything that is not a number at or below the maximum.
+constexpr float kMassOne = 4294967040.0f;  // largest fp32 below 2^32
+static __device__ __forceinline__ uint64_t mass_of(float x, float neg_mx_log2e) {
+  const float e = fmaxf(fast_exp2(__builtin_fmaf(x, 1.4426950408889634f, neg_mx_log2e)), 0.f);  // NaN -> 0
+  return (uint64_t)(uint32_t)__builtin_fmaf(e, kMassOne, 0.5f);  // the conversion saturates
 }
 
 // Adds weight() to hist[bin] for the active lanes (weight is only evaluated when some lane of the
@@ -210,15 +239,26 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   const bool greedy = p.top_k == 1;
   const RowReader<BF16, VEC> rd{reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)r * p.stride * (BF16 ? 2 : 4), V,
                                 p.inv_temperature, !greedy && p.inv_temperature != 1.0f};
-  constexpr int U = VEC > 1 ? 4 : 8;  // loads in flight per thread
+  constexpr int U = 8;  // loads in flight per thread
 
   // ---- pass A: maximum (lowest index among equals, NaN counts as largest) and finite minimum ----
+  // (a thread meets its elements in rising index order, so "strictly greater" keeps the first)
   uint32_t bk = 0; int bi = 0x7fffffff; float mn = INFINITY;
-  sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
-    const uint32_t k = order_key(x);
-    if (in && (k > bk || (k == bk && i < bi))) { bk = k; bi = i; }
-    if (in && x > -INFINITY) mn = fminf(mn, x);
-  });
+  const bool filtering = !greedy && (p.top_k > 1 || p.top_p > 0.f);
+  if (filtering) {
+    sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
+      const uint32_t k = order_key(x);
+      const bool up = in && k > bk;
+      bk = up ? k : bk; bi = up ? i : bi;
+      mn = (in && x > -INFINITY) ? fminf(mn, x) : mn;
+    });
+  } else {
+    sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
+      const uint32_t k = order_key(x);
+      const bool up = in && k > bk;
+      bk = up ? k : bk; bi = up ? i : bi;
+    });
+  }
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) {
     const uint32_t ok = __shfl_xor(bk, m, 64); const int oi = __shfl_xor(bi, m, 64);
@@ -241,6 +281,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
 
   // A maximum that is not a finite number leaves no distribution to draw from: take the argmax.
   const bool drawable = !greedy && fabsf(mx) < INFINITY;
+  const float neg_mx = -mx * 1.4426950408889634f;
   if (drawable) {
     const bool by_count = p.top_k > 1;
     const bool filtered = by_count || p.top_p > 0.f;
@@ -254,7 +295,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
         int b = f >= 255.f ? 255 : (int)f;  // NaN (inf * 0) compares false and converts to 0
         return b < 0 ? 0 : b;
       };
-      auto weight_of = [&](float x) -> uint64_t { return by_count ? (uint64_t)1 : mass_of(x, mx); };
+      auto weight_of = [&](float x) -> uint64_t { return by_count ? (uint64_t)1 : mass_of(x, neg_mx); };
       if (tid < 256) hist[tid] = 0;
       if (tid == 0) member_count = 0;
       __syncthreads();
@@ -328,7 +369,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
     }
 
     // ---- draw: inverse CDF over the kept elements in vocabulary order ----
-    auto kept_mass = [&](float x) -> uint64_t { return order_key(x) >= cut_key ? mass_of(x, mx) : 0; };
+    auto kept_mass = [&](float x) -> uint64_t { return order_key(x) >= cut_key ? mass_of(x, neg_mx) : 0; };
     const int L1 = ((V + kSampleWaves - 1) / kSampleWaves + 63) & ~63;  // elements per first-level range
     {
       const int a = min(wave * L1, V), b = min(a + L1, V);
@@ -341,7 +382,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
     uint64_t total = 0;
 #pragma unroll
     for (int w = 0; w < kSampleWaves; ++w) total += wsum[w];
-    // total >= 2^40: the maximum itself is always kept
+    // total > 0: the maximum itself is always kept and has the largest mass
     uint64_t want = (uint64_t)((double)p.uniform[r] * (double)total);
     want = want < total ? want : total - 1;
     int w1 = 0;

@@ -2,7 +2,7 @@
 
 Bars.  The gather, the argmax, the top-k cut and the mask are integer / selection work: equality
 with the checker.  The top-p cut and the draw depend on sums of exponentials, which the kernel
-carries as 2^-40 fixed point and the checker in fp64: a result must equal the checker's whenever
+carries as 2^-32 fixed point and the checker in fp64: a result must equal the checker's whenever
 the checker's decision has a margin (2e-6 of the total mass: the
 kernel's exponentials are fp32), and must in every case satisfy the definition within that margin
 (mass strictly above the cut <= top_p < mass down to the cut; CDF bracket of the drawn index).
