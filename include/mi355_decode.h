@@ -116,6 +116,19 @@ int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_bf16, int64_
                             float headroom, void* stream);
 
 /*
+ * fp8 append with explicit per-token slots (prefill / mixed steps; no counterpart in the reference).
+ * The tokens a call writes into one chunk must be neighbours in the token dimension with rising
+ * local positions, as DynamicInferenceContext lays them out (dynamic_context.py:982-1005,1283-1296).
+ * A run that starts at local position 0 opens its chunk: scale = amax(run) / 448, times `headroom`
+ * unless the run fills the chunk; any other run reuses the stored scale (saturating).
+ */
+int mi_kv_append_fp8(const void* key_bf16, const void* value_bf16, int64_t src_stride_tok,
+                     void* k_cache_fp8, void* v_cache_fp8, int64_t kv_stride_chunk,
+                     int64_t kv_stride_tok, float* k_scales, float* v_scales,
+                     const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos, int32_t T,
+                     int32_t chunk_tokens, int32_t Hkv, int32_t head_dim, float headroom, void* stream);
+
+/*
  * Bytes of workspace mi_paged_decode_attention needs for these sizes on the current
  * device (partials of the workgroups that share a request + per-request bookkeeping).
  */
@@ -170,6 +183,24 @@ int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_st
                                int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
                                int32_t max_kv_len, int32_t split_tokens, float softmax_scale,
                                void* stream);
+
+/*
+ * The same call over an fp8-e4m3 cache (byte caches `[n_chunks, chunk_tokens, Hkv, d]`, strides in
+ * elements = bytes, fp32 scales `[n_chunks, Hkv]`; no counterpart in the reference).  Tiles are
+ * multiplied by their chunk's scale and rounded to bf16 on their way into LDS.  Needs head_dim 128
+ * and a chunk size that is a multiple of 64.
+ */
+int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
+                                   const void* k_cache_fp8, const void* v_cache_fp8,
+                                   int64_t kv_stride_chunk, int64_t kv_stride_tok,
+                                   int64_t kv_stride_head, const float* k_scales,
+                                   const float* v_scales, const int32_t* block_table,
+                                   int64_t bt_stride, const int32_t* cu_seqlens_q,
+                                   const int32_t* kv_lens, void* out, int64_t o_stride_tok,
+                                   int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
+                                   int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
+                                   int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
+                                   float softmax_scale, void* stream);
 
 /*
  * Fused q/k head norm + rotary embedding (+ KV-append when k_cache is given).

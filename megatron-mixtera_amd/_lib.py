@@ -31,6 +31,8 @@ SIGNATURES = {
         c_int, [_P, _I64, _I64, _P, _I64, _I64, _P, _I32, _I32, _I32, _I32, _P]),
     "mi_kv_append_decode_fp8": (
         c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _F, _P]),
+    "mi_kv_append_fp8": (
+        c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _F, _P]),
     "mi_decode_workspace_bytes": (_I64, [_I32, _I32, _I32, _I32, _I32, _I32, _I32]),
     "mi_paged_decode_attention": (
         c_int,
@@ -40,6 +42,10 @@ SIGNATURES = {
     "mi_paged_prefill_attention": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _P, _I64,
+         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
+    "mi_paged_prefill_attention_fp8": (
+        c_int,
+        [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _P, _P, _I64, _P, _P, _P, _I64, _I64, _P, _I64,
          _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
     "mi_update_requests": (
         c_int, [_P] * 8 + [_I64, _I32] + [_P] * 14 + [_I32] * 7 + [_P]),

@@ -138,6 +138,73 @@ __global__ __launch_bounds__(64) void kv_append_decode_fp8_kernel(QuantParams p)
   for (int e = threadIdx.x; e < p.d; e += 64) dst[e] = (uint8_t)f32_to_e4m3_sat(bf16_to_f32(src[e]) / scale);
 }
 
+// ---- fp8 append of many tokens per request (prefill / mixed steps) ----------------------------
+// Slots come from the per-token rows.  Tokens of one chunk are neighbours in the token dimension
+// with rising local positions (that is how the context lays requests out), so the tokens a call
+// writes into a chunk form one run.  A run that starts at local position 0 opens the chunk and fixes
+// the scale of each of its heads: amax over the whole run / 448, times `headroom` unless the run
+// fills the chunk (later tokens of a partly filled chunk reuse the scale and saturate).  A run that
+// starts further in reuses the stored scale.
+struct AppendFp8Params {
+  const uint16_t* src[2];   // key, value rows (bf16)
+  int64_t src_stride;       // elements between tokens
+  uint8_t* dst[2];          // fp8 caches
+  int64_t chunk_bytes, tok_bytes;
+  float* scale[2];          // [n_chunks][Hkv] each
+  const int64_t* tok_chunk;
+  const int64_t* tok_local;
+  int32_t T, chunk, Hkv, d;
+  float headroom;
+};
+
+// grid = (T, Hkv, 2): the workgroup of a run's first token computes the scale of (chunk, head).
+__global__ __launch_bounds__(256) void kv_append_fp8_scales_kernel(AppendFp8Params p) {
+  const int t = blockIdx.x, h = blockIdx.y, kv = blockIdx.z;
+  if (p.tok_local[t] != 0) return;  // not the opening token of a chunk
+  const int64_t c = p.tok_chunk[t];
+  __shared__ int run_s[256];
+  __shared__ float red[256];
+  // run length: first i >= 1 where token t+i is not (chunk c, local i)
+  int first_bad = p.chunk;
+  for (int i = 1 + threadIdx.x; i < p.chunk; i += 256) {
+    const bool ok = t + i < p.T && p.tok_chunk[t + i] == c && p.tok_local[t + i] == i;
+    if (!ok) { first_bad = i; break; }
+  }
+  run_s[threadIdx.x] = first_bad;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) run_s[threadIdx.x] = min(run_s[threadIdx.x], run_s[threadIdx.x + s]);
+    __syncthreads();
+  }
+  const int n = run_s[0];
+  const uint16_t* src = p.src[kv] + (int64_t)t * p.src_stride + (int64_t)h * p.d;
+  float amax = 0.f;
+  for (int i = threadIdx.x; i < n * p.d; i += 256) {
+    const int tok = i / p.d, e = i - tok * p.d;
+    amax = fmaxf(amax, fabsf(bf16_to_f32(src[(int64_t)tok * p.src_stride + e])));
+  }
+  red[threadIdx.x] = amax;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if ((int)threadIdx.x < s) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    const float hr = n == p.chunk ? 1.f : p.headroom;
+    p.scale[kv][c * p.Hkv + h] = red[0] > 0.f ? hr * red[0] / 448.f : 1.f;
+  }
+}
+
+// grid = (T, Hkv, 2): quantise one head row of one token with its chunk's scale.
+__global__ __launch_bounds__(64) void kv_append_fp8_rows_kernel(AppendFp8Params p) {
+  const int t = blockIdx.x, h = blockIdx.y, kv = blockIdx.z;
+  const int64_t c = p.tok_chunk[t], l = p.tok_local[t];
+  const float scale = p.scale[kv][c * p.Hkv + h];
+  const uint16_t* src = p.src[kv] + (int64_t)t * p.src_stride + (int64_t)h * p.d;
+  uint8_t* dst = p.dst[kv] + c * p.chunk_bytes + l * p.tok_bytes + (int64_t)h * p.d;
+  for (int e = threadIdx.x; e < p.d; e += 64) dst[e] = (uint8_t)f32_to_e4m3_sat(bf16_to_f32(src[e]) / scale);
+}
+
 template <bool DECODE>
 static int launch_append(AppendParams& p, hipStream_t st) {
   const uintptr_t bits = (uintptr_t)p.key | (uintptr_t)p.value | (uintptr_t)p.kc | (uintptr_t)p.vc |
@@ -237,4 +304,30 @@ extern "C" int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_b
   p.src = (const uint16_t*)value_bf16; p.dst = (uint8_t*)v_cache_fp8; p.scale = v_scales;
   hipLaunchKernelGGL(kv_append_decode_fp8_kernel, dim3(R, Hkv), dim3(64), 0, (hipStream_t)stream, p);
   return mi_check_launch("mi_kv_append_decode_fp8");
+}
+
+extern "C" int mi_kv_append_fp8(const void* key_bf16, const void* value_bf16, int64_t src_stride_tok,
+                                void* k_cache_fp8, void* v_cache_fp8, int64_t kv_stride_chunk,
+                                int64_t kv_stride_tok, float* k_scales, float* v_scales,
+                                const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos,
+                                int32_t T, int32_t chunk_tokens, int32_t Hkv, int32_t head_dim,
+                                float headroom, void* stream) {
+  if (T == 0) return MI_OK;
+  if (!key_bf16 || !value_bf16 || !k_cache_fp8 || !v_cache_fp8 || !k_scales || !v_scales || !token_to_chunk_idx ||
+      !token_to_local_pos)
+    return mi_fail(MI_ERR_NULL, "mi_kv_append_fp8: null pointer argument");
+  if (T < 0 || chunk_tokens <= 0 || Hkv <= 0 || head_dim <= 0 || Hkv > 65535 || !(headroom > 0.f) ||
+      src_stride_tok < (int64_t)Hkv * head_dim || kv_stride_tok < (int64_t)Hkv * head_dim)
+    return mi_fail(MI_ERR_SHAPE, "mi_kv_append_fp8: bad sizes or strides");
+  AppendFp8Params p = {};
+  p.src[0] = (const uint16_t*)key_bf16; p.src[1] = (const uint16_t*)value_bf16; p.src_stride = src_stride_tok;
+  p.dst[0] = (uint8_t*)k_cache_fp8; p.dst[1] = (uint8_t*)v_cache_fp8;
+  p.chunk_bytes = kv_stride_chunk; p.tok_bytes = kv_stride_tok;
+  p.scale[0] = k_scales; p.scale[1] = v_scales;
+  p.tok_chunk = token_to_chunk_idx; p.tok_local = token_to_local_pos;
+  p.T = T; p.chunk = chunk_tokens; p.Hkv = Hkv; p.d = head_dim; p.headroom = headroom;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(kv_append_fp8_scales_kernel, dim3(T, Hkv, 2), dim3(256), 0, st, p);
+  hipLaunchKernelGGL(kv_append_fp8_rows_kernel, dim3(T, Hkv, 2), dim3(64), 0, st, p);
+  return mi_check_launch("mi_kv_append_fp8");
 }

@@ -637,7 +637,7 @@ int mi::launch_paged_decode(
   hipStream_t st = (hipStream_t)stream;
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
-  if (timed) hipEventRecord(ev_a, st);
+  if (timed) (void)hipEventRecord(ev_a, st);
 #define MI_LAUNCH_DECODE(HD_, FP8_)                                                                             \
   do {                                                                                                          \
     if (nt == 1 && minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 4>), grid, block, lds, st, p); \
@@ -656,7 +656,7 @@ int mi::launch_paged_decode(
   else if (head_dim == 128) MI_LAUNCH_DECODE(128, false);
   else MI_LAUNCH_DECODE(64, false);
 #undef MI_LAUNCH_DECODE
-  if (timed) hipEventRecord(ev_b, st);
+  if (timed) (void)hipEventRecord(ev_b, st);
   dim3 mgrid(Hq, R);
   if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p);
   else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p);

@@ -39,6 +39,8 @@ struct PrefillParams {
   int32_t T, R, Hq, Hkv, G, g_shift, chunk;
   int32_t skip_single;  // requests with exactly one query row are handled by the decode kernels
   float scale_log2;
+  const float* k_scale;  // fp8 KV only: [n_chunks][Hkv]
+  const float* v_scale;
 };
 
 // NQ = 16-row tiles per wave; a workgroup always covers 256 rows (16 / NQ waves).
@@ -609,9 +611,13 @@ static __device__ __forceinline__ float rowgroup_max(float x) {
   return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
-template <bool STAGGER>
+// FP8: the cache holds e4m3 bytes with one fp32 scale per (chunk, KV head); a piece is multiplied by
+// its chunk's scale and rounded to bf16 on its way into LDS, so both matrix phases are the bf16 ones.
+template <bool STAGGER, bool FP8>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
   constexpr int HD = 128, KS = 4, DV = 8, NQ = 2, NT = 4, WAVES = 8;
+  constexpr int ESZ = FP8 ? 1 : 2;       // bytes per cache element
+  constexpr int PIECE = FP8 ? 8 : 16;    // bytes one loader thread fetches of a row (8 elements)
   __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kPPTile * kKPitch];
   __shared__ __attribute__((aligned(16))) uint8_t Vs[3][kPPTile * kVPitch];  // three: see the loop
 
@@ -683,11 +689,11 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   }
 
   if (ntl > 0) {
-    const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * 2;
-    const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * 2;
-    const int64_t chunk_bytes = p.kv_sc * 2;
-    const int tok_bytes = p.kv_st * 2;
-    // loader role: 16-byte piece `lpiece` of key rows `lkey` and `lkey + 32` of a tile
+    const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * ESZ;
+    const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * ESZ;
+    const int64_t chunk_bytes = p.kv_sc * ESZ;
+    const int tok_bytes = p.kv_st * ESZ;
+    // loader role: piece `lpiece` (8 elements) of key rows `lkey` and `lkey + 32` of a tile
     const int lkey = tid >> 4, lpiece = tid & 15;
     const int k_off = lkey * kKPitch + lpiece * 16;
     const int v_off = lkey * kVPitch + lpiece * 16;
@@ -700,9 +706,10 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // tile into a buffer nobody reads any more, which keeps the loop free of branches.
     const int tiles_per_chunk = p.chunk / kPPTile;
     const int tile_bytes = kPPTile * tok_bytes;
-    const uint32_t row_off0 = (uint32_t)(lkey * tok_bytes + lpiece * 16);
+    const uint32_t row_off0 = (uint32_t)(lkey * tok_bytes + lpiece * PIECE);
     const uint32_t row_off1 = row_off0 + (uint32_t)(32 * tok_bytes);
-    const uint32_t piece_off = (uint32_t)(lpiece * 16);
+    const uint32_t piece_off = (uint32_t)(lpiece * PIECE);
+    float ksc_staged = 1.f, vsc_staged = 1.f;  // fp8: scales of the tile held in kreg / vreg (per-lane copies)
     const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
     struct Cursor {   // all members are wave-uniform
       int tile;       // tile index
@@ -725,9 +732,17 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       c.tin = wrap ? 0 : c.tin + (adv ? 1 : 0);
       c.ci += wrap ? 1 : 0;
     };
+    // fp8: the scales of a tile's chunk, requested when the tile's loads are issued
+    auto tile_scales = [&](int pc) {
+      if (FP8) {
+        ksc_staged = p.k_scale[(int64_t)pc * p.Hkv + h];
+        vsc_staged = p.v_scale[(int64_t)pc * p.Hkv + h];
+      }
+    };
     // byte offset of the cursor's tile inside a cache, given its physical chunk
     auto tile_offset = [&](const Cursor& c, int pc_lane) -> int64_t {
       const int pc = __builtin_amdgcn_readfirstlane(pc_lane);
+      tile_scales(pc);
       return (int64_t)pc * chunk_bytes + (int64_t)c.tin * tile_bytes;
     };
     // this thread's two pieces of a tile (rows past the request's last key re-read the last row,
@@ -735,19 +750,33 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     auto tile_loads = [&](const uint8_t* base, int64_t off, int room, uint4 (&reg)[2]) {
       const uint8_t* tb = base + off;
       const uint32_t lim = (uint32_t)room + piece_off;
-      reg[0] = ld16(tb + min(row_off0, lim));
-      reg[1] = ld16(tb + min(row_off1, lim));
+      if (FP8) {
+        const uint2 a = ld8(tb + min(row_off0, lim)), b = ld8(tb + min(row_off1, lim));
+        reg[0] = make_uint4(a.x, a.y, 0u, 0u);
+        reg[1] = make_uint4(b.x, b.y, 0u, 0u);
+      } else {
+        reg[0] = ld16(tb + min(row_off0, lim));
+        reg[1] = ld16(tb + min(row_off1, lim));
+      }
+    };
+    // what goes into LDS for one staged piece: the bf16 bits, or (fp8) 8 bytes -> 8 bf16 of byte * scale
+    auto lds_piece = [&](uint4 raw, float scale) {
+      if (!FP8) return raw;
+      const f32x2_t a = fp8x2_lo_to_f32(raw.x), b = fp8x2_hi_to_f32(raw.x);
+      const f32x2_t c = fp8x2_lo_to_f32(raw.y), d = fp8x2_hi_to_f32(raw.y);
+      return make_uint4(pack_bf16x2(a.x * scale, a.y * scale), pack_bf16x2(b.x * scale, b.y * scale),
+                        pack_bf16x2(c.x * scale, c.y * scale), pack_bf16x2(d.x * scale, d.y * scale));
     };
     auto store_k = [&](int t) {
       uint8_t* dst = &Ks[t & 1][k_off];
-      *reinterpret_cast<uint4*>(dst) = kreg[0];
-      *reinterpret_cast<uint4*>(dst + 32 * kKPitch) = kreg[1];
+      *reinterpret_cast<uint4*>(dst) = lds_piece(kreg[0], ksc_staged);
+      *reinterpret_cast<uint4*>(dst + 32 * kKPitch) = lds_piece(kreg[1], ksc_staged);
     };
     auto vbuf = [](int t) { return (unsigned)(t + 3) % 3u; };  // tile -1 lives in buffer 2
     auto store_v = [&](int t) {
       uint8_t* dst = &Vs[vbuf(t)][v_off];
-      *reinterpret_cast<uint4*>(dst) = vreg[0];
-      *reinterpret_cast<uint4*>(dst + 32 * kVPitch) = vreg[1];
+      *reinterpret_cast<uint4*>(dst) = lds_piece(vreg[0], vsc_staged);
+      *reinterpret_cast<uint4*>(dst + 32 * kVPitch) = lds_piece(vreg[1], vsc_staged);
     };
 
     const float scale = p.scale_log2;
@@ -971,15 +1000,15 @@ extern "C" int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, 
   return mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens);
 }
 
-extern "C" int mi_paged_prefill_attention(
+static int launch_paged_prefill(
     const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
     const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
     const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seqlens_q,
     const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head,
     void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
-    int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
-    float softmax_scale, void* stream) {
-  (void)max_kv_len;
+    int32_t head_dim, int32_t chunk_tokens, int32_t split_tokens, float softmax_scale,
+    int32_t kv_dtype, const float* k_scales, const float* v_scales, void* stream) {
+  const bool fp8 = kv_dtype == MI_KV_FP8_E4M3;
   if (T == 0 || R == 0) return MI_OK;
   if (!q || !k_cache || !v_cache || !block_table || !cu_seqlens_q || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention: null pointer argument");
@@ -998,6 +1027,15 @@ extern "C" int mi_paged_prefill_attention(
     return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention: strides must keep rows 16-byte aligned");
   if (kv_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: one chunk must span less than 2 GiB");
+  if (kv_dtype != MI_KV_BF16 && !fp8)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: unknown kv_dtype");
+  if (fp8 && (!k_scales || !v_scales))
+    return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_fp8: both scale arrays are required");
+  if (fp8 && (head_dim != 128 || chunk_tokens % 64 || mi_tuning().prefill_pingpong == 0 ||
+              mi_tuning().prefill_lds_row_tiles == 0))
+    return mi_fail(MI_ERR_UNSUPPORTED,
+                   "mi_paged_prefill_attention_fp8: fp8 KV needs head_dim 128, a chunk size that is a multiple "
+                   "of 64 and the two-phase tile kernel");
 
   PrefillParams p;
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
@@ -1013,6 +1051,7 @@ extern "C" int mi_paged_prefill_attention(
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   // With a workspace, one-row requests go through the bandwidth-optimised decode kernels.
   p.skip_single = workspace != nullptr;
+  p.k_scale = k_scales; p.v_scale = v_scales;
 
   hipStream_t st = (hipStream_t)stream;
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
@@ -1024,20 +1063,22 @@ extern "C" int mi_paged_prefill_attention(
     const bool wide = mi_tuning().prefill_tile_subtiles == 4;  // 64-key staged tiles
     hipEvent_t ev_a, ev_b;
     const bool timed = mi_profile_next(&ev_a, &ev_b);
-    if (timed) hipEventRecord(ev_a, st);
+    if (timed) (void)hipEventRecord(ev_a, st);
     const int pp = (chunk_tokens % 64 == 0) ? mi_tuning().prefill_pingpong : 0;  // staged tiles must not straddle chunks
-    if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true>), lgrid, dim3(512), 0, st, p);
-    else if (pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false>), lgrid, dim3(512), 0, st, p);
+    if (fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true>), lgrid, dim3(512), 0, st, p);
+    else if (fp8) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, true>), lgrid, dim3(512), 0, st, p);
+    else if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false>), lgrid, dim3(512), 0, st, p);
+    else if (pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false>), lgrid, dim3(512), 0, st, p);
     else if (lds_tiles == 2 && wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 4>), lgrid, dim3(512), 0, st, p);
     else if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 2>), lgrid, dim3(512), 0, st, p);
     else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);  // (48 rows: 32-key tiles only)
-    if (timed) hipEventRecord(ev_b, st);
+    if (timed) (void)hipEventRecord(ev_b, st);
     int rc0 = mi_check_launch("mi_paged_prefill_attention");
     if (rc0 != MI_OK || !p.skip_single) return rc0;
     return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
                                kv_stride_head, block_table, bt_stride, kv_lens, cu_seqlens_q, out, o_stride_tok,
                                o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
-                               split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
+                               split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
   }
   const int nq = mi_tuning().prefill_row_tiles == 4 ? 4 : 2;
   const int sbq = 256 / G;  // query tokens per workgroup (256 rows)
@@ -1063,4 +1104,34 @@ extern "C" int mi_paged_prefill_attention(
                              kv_stride_head, block_table, bt_stride, kv_lens, cu_seqlens_q, out, o_stride_tok,
                              o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
                              split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
+}
+
+extern "C" int mi_paged_prefill_attention(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
+    const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seqlens_q,
+    const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head,
+    void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
+    int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
+    float softmax_scale, void* stream) {
+  (void)max_kv_len;
+  return launch_paged_prefill(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
+                              kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out, o_stride_tok,
+                              o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim, chunk_tokens,
+                              split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
+}
+
+extern "C" int mi_paged_prefill_attention_fp8(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache_fp8,
+    const void* v_cache_fp8, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
+    const float* k_scales, const float* v_scales, const int32_t* block_table, int64_t bt_stride,
+    const int32_t* cu_seqlens_q, const int32_t* kv_lens, void* out, int64_t o_stride_tok,
+    int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq,
+    int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
+    float softmax_scale, void* stream) {
+  (void)max_kv_len;
+  return launch_paged_prefill(q, q_stride_tok, q_stride_head, k_cache_fp8, v_cache_fp8, kv_stride_chunk,
+                              kv_stride_tok, kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out,
+                              o_stride_tok, o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim,
+                              chunk_tokens, split_tokens, softmax_scale, MI_KV_FP8_E4M3, k_scales, v_scales, stream);
 }

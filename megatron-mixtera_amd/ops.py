@@ -180,6 +180,30 @@ def kv_append_decode_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: T
                "mi_kv_append_decode_fp8")
 
 
+def kv_append_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor, k_scales: Tensor, v_scales: Tensor,
+                  token_to_chunk_idx: Tensor, token_to_local_pos: Tensor, headroom: float = 2.0) -> None:
+    """Quantise and append bf16 tokens with explicit slots into an fp8 cache (prefill / mixed steps)."""
+    lib = _lib.load()
+    _stream(key)  # device check first: there is no CPU path
+    key, row, k_st = _rows(key, "key")
+    value, _, v_st = _rows(value, "value")
+    T = key.size(0)
+    _require(key.dtype == torch.bfloat16 and value.dtype == torch.bfloat16 and k_st == v_st and value.size(0) == T,
+             "K/V must be bf16 with equal shapes and strides")
+    _require(k_cache.element_size() == 1 and v_cache.element_size() == 1, "fp8 caches hold one byte per element")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh) and sh == k_cache.size(3) and row == k_cache.size(2) * sh,
+             "cache layout")
+    _require(k_scales.dtype == torch.float32 and v_scales.dtype == torch.float32, "scales must be fp32")
+    _require(k_scales.is_contiguous() and v_scales.is_contiguous(), "scales must be contiguous")
+    for rows in (token_to_chunk_idx, token_to_local_pos):
+        _require(rows.dtype == torch.int64 and rows.is_contiguous() and rows.numel() >= T, "slot rows must be int64 [>=T]")
+    _lib.check(lib.mi_kv_append_fp8(key.data_ptr(), value.data_ptr(), k_st, k_cache.data_ptr(), v_cache.data_ptr(),
+                                    sc, st, k_scales.data_ptr(), v_scales.data_ptr(), token_to_chunk_idx.data_ptr(),
+                                    token_to_local_pos.data_ptr(), T, k_cache.size(1), k_cache.size(2),
+                                    k_cache.size(3), float(headroom), _stream(key)), "mi_kv_append_fp8")
+
+
 # ---------------------------------------------------------------------------------------------
 # attention
 # ---------------------------------------------------------------------------------------------
@@ -245,15 +269,25 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
 
 def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
                             block_table: Tensor, *, softmax_scale: Optional[float] = None,
-                            max_kv_len: Optional[int] = None, out: Optional[Tensor] = None) -> Tensor:
-    """Varlen causal attention of new tokens over the paged cache (bottom-right aligned mask)."""
+                            max_kv_len: Optional[int] = None, out: Optional[Tensor] = None,
+                            k_scales: Optional[Tensor] = None, v_scales: Optional[Tensor] = None) -> Tensor:
+    """Varlen causal attention of new tokens over the paged cache (bottom-right aligned mask).
+    Byte caches with ``k_scales`` / ``v_scales`` ``[N, Hkv]`` select the fp8-e4m3 path."""
     lib = _lib.load()
     _stream(q)  # device check first: there is no CPU path
     q3 = _qo_view(q, "q")
     T, Hq, D = q3.shape
     N, C, Hkv, Dk = k_cache.shape
     _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
-    _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16, "prefill needs a bf16 cache")
+    fp8 = k_scales is not None
+    if fp8:
+        _require(k_cache.element_size() == 1 and v_cache.element_size() == 1, "fp8 caches hold one byte per element")
+        _require(v_scales is not None and k_scales.dtype == torch.float32 and v_scales.dtype == torch.float32
+                 and k_scales.is_contiguous() and v_scales.is_contiguous() and tuple(k_scales.shape) == (N, Hkv)
+                 and tuple(v_scales.shape) == (N, Hkv), "scales must be contiguous fp32 [N, Hkv]")
+    else:
+        _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16,
+                 "the cache must be bf16, or bytes with scales")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
     _require(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.is_contiguous(), "cu_seqlens_q must be contiguous int32")
@@ -271,6 +305,14 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
     _require(tuple(o3.shape) == (T, Hq, D), "out shape mismatch")
     workspace = _workspace(q.device, lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, D, int(max_kv_len), 0))
     ws_bytes = 0 if workspace is None else workspace.numel()
+    if fp8:
+        _lib.check(lib.mi_paged_prefill_attention_fp8(
+            q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
+            k_scales.data_ptr(), v_scales.data_ptr(), block_table.data_ptr(), block_table.stride(0),
+            cu_seqlens_q.data_ptr(), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
+            _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C, int(max_kv_len), 0, float(softmax_scale), _stream(q)),
+            "mi_paged_prefill_attention_fp8")
+        return out
     _lib.check(lib.mi_paged_prefill_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
         block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),

@@ -82,8 +82,13 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
 
 
 def paged_varlen_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
-                           block_table: Tensor, softmax_scale: Optional[float] = None) -> Tensor:
-    """Prefill / mixed: ``q`` [T,Hq,d]; request r owns rows cu_q[r]:cu_q[r+1] and kv_lens[r] keys."""
+                           block_table: Tensor, softmax_scale: Optional[float] = None,
+                           k_scales: Optional[Tensor] = None, v_scales: Optional[Tensor] = None) -> Tensor:
+    """Prefill / mixed: ``q`` [T,Hq,d]; request r owns rows cu_q[r]:cu_q[r+1] and kv_lens[r] keys.
+    With scales the caches are e4m3fn bytes, dequantised to fp32 first."""
+    if k_scales is not None:
+        k_cache = dequantize_fp8(k_cache, k_scales)
+        v_cache = dequantize_fp8(v_cache, v_scales)
     T, Hq, d = q.shape
     scale = d ** -0.5 if softmax_scale is None else softmax_scale
     out = torch.zeros(T, Hq, d, dtype=torch.float32)
@@ -155,6 +160,34 @@ def quantize_token_fp8(row: Tensor, scale: Tensor) -> Tensor:
     """``row`` [Hkv,d], ``scale`` [Hkv] -> uint8 e4m3fn bytes (saturating)."""
     y = (row.float() / scale[:, None]).clamp(-E4M3_MAX, E4M3_MAX)
     return y.to(torch.float8_e4m3fn).view(torch.uint8)
+
+
+def kv_append_fp8(cache_bytes: Tensor, scales: Tensor, rows: Tensor, chunk_idx: Tensor, local: Tensor,
+                  headroom: float = 2.0) -> None:
+    """The library's fp8 append policy for many tokens per call, in scalar loops (in place).
+
+    ``cache_bytes`` uint8 [N,C,Hkv,d], ``scales`` fp32 [N,Hkv], ``rows`` bf16 [T,Hkv,d]; token t goes to
+    (chunk_idx[t], local[t]).  Consecutive tokens of one chunk with rising local positions form a run.
+    A run starting at local 0 opens the chunk: per head, scale = amax(run) / 448, times ``headroom`` unless
+    the run fills the chunk (zero amax -> scale 1); a run starting further in reuses the stored scale.
+    Values are divided by the scale in fp32, clamped to +-448 and rounded to e4m3fn (nearest even).
+    This policy has no counterpart in the reference (its cache is never quantised)."""
+    C = cache_bytes.size(1)
+    T = rows.size(0)
+    t = 0
+    while t < T:
+        c, l0 = int(chunk_idx[t]), int(local[t])
+        n = 1
+        while t + n < T and int(chunk_idx[t + n]) == c and int(local[t + n]) == l0 + n and l0 + n < C:
+            n += 1
+        if l0 == 0:
+            amax = rows[t:t + n].float().abs().amax(dim=(0, 2))
+            hr = 1.0 if n == C else headroom
+            scales[c] = torch.where(amax > 0, (torch.tensor(hr, dtype=torch.float32) * amax) / E4M3_MAX,
+                                    torch.ones_like(amax))
+        for i in range(n):
+            cache_bytes[c, l0 + i] = quantize_token_fp8(rows[t + i], scales[c])
+        t += n
 
 
 def decode_attention_bytes(kv_lens: Sequence[int], Hq: int, Hkv: int, d: int, chunk: int, kv_bytes: int = 2,

@@ -182,3 +182,29 @@ def test_decode_attention_bytes_formula():
     assert n == (300 + 256) * 8 * 128 * 2 * 2 + 2 * 32 * 128 * 4 + (2 + 1) * 4 + 2 * 4
     n8 = oa.decode_attention_bytes([300, 256], 32, 8, 128, 256, kv_bytes=1, fp8_scales=True)
     assert n8 == (300 + 256) * 8 * 128 * 2 + 2 * 32 * 128 * 4 + 3 * 4 + 2 * 4 + 3 * 8 * 2 * 4
+
+
+def test_fp8_append_policy_pins():
+    """The many-token append policy: a run that fills a chunk is the whole-chunk quantiser; a run that
+    stops short gets headroom; a run that continues a chunk keeps the stored scale and saturates."""
+    g = torch.Generator().manual_seed(12)
+    C, Hkv, d = 16, 2, 8
+    rows = (torch.randn(40, Hkv, d, generator=g) * 2).bfloat16()
+    cache = torch.zeros(4, C, Hkv, d, dtype=torch.uint8)
+    scales = torch.full((4, Hkv), 0.125)
+    chunk_idx = torch.tensor([2] * 16 + [0] * 10 + [3] * 14)
+    local = torch.tensor(list(range(16)) + list(range(10)) + list(range(2, 16)))
+    oa.kv_append_fp8(cache, scales, rows, chunk_idx, local, headroom=2.0)
+    full = rows[:16].reshape(1, C, Hkv, d)
+    b, s = oa.quantize_chunks_fp8(full)
+    assert torch.equal(cache[2], b[0]) and torch.equal(scales[2], s[0])
+    amax = rows[16:26].float().abs().amax(dim=(0, 2))
+    assert torch.equal(scales[0], 2.0 * amax / 448.0)            # opened but not filled: headroom 2
+    assert (cache[0, 10:] == 0).all()                            # slots after the run untouched
+    assert torch.equal(scales[3], torch.full((Hkv,), 0.125))     # continued chunk: scale kept
+    want = oa.quantize_token_fp8(rows[26], scales[3])
+    assert torch.equal(cache[3, 2], want) and (cache[3, :2] == 0).all()
+    # 448 * 0.125 = 56 is the largest magnitude the kept scale can hold: larger values saturate to 0x7e / 0xfe
+    big = torch.full((1, Hkv, d), 100.0).bfloat16()
+    oa.kv_append_fp8(cache, scales, big, torch.tensor([3]), torch.tensor([0 + 1]), headroom=2.0)
+    assert (cache[3, 1] == 0x7E).all()
