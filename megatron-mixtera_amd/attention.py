@@ -33,19 +33,23 @@ def adjust_key_value_for_inference(inference_context, layer_number: int, query: 
 
 
 def flash_decode_and_prefill(q: Tensor, k: Tensor, v: Tensor, max_seqlen_q, max_seqlen_k, cu_seqlens_q,
-                             cu_seqlens_k, seqlens_k, block_table, softmax_scale: Optional[float] = None) -> Tensor:
+                             cu_seqlens_k, seqlens_k, block_table, softmax_scale: Optional[float] = None, *,
+                             k_scales: Optional[Tensor] = None, v_scales: Optional[Tensor] = None) -> Tensor:
     """Same contract as ``Attention.flash_decode_and_prefill`` (attention.py:470-601).
 
     ``q`` is ``[T, 1, Hq, d]``; ``k`` / ``v`` are the paged caches.  ``max_seqlen_q == 1``
-    selects the decode kernel, anything else the varlen causal kernel.
+    selects the decode kernel, anything else the varlen causal kernel.  ``k_scales`` / ``v_scales``
+    (an addition) go with byte caches holding e4m3 values.
     """
     if max_seqlen_q > 1:
         out = flash_attn_varlen_func(q.squeeze(1), k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                                      softmax_scale=softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5,
-                                     causal=True, block_table=block_table, seqused_k=seqlens_k)
+                                     causal=True, block_table=block_table, seqused_k=seqlens_k,
+                                     k_scales=k_scales, v_scales=v_scales)
         return out.unsqueeze(1)
     return flash_attn_with_kvcache(q=q, k_cache=k, v_cache=v, cache_seqlens=seqlens_k, causal=True,
-                                   block_table=block_table, softmax_scale=softmax_scale, max_seqlen_k=max_seqlen_k)
+                                   block_table=block_table, softmax_scale=softmax_scale, max_seqlen_k=max_seqlen_k,
+                                   k_scales=k_scales, v_scales=v_scales)
 
 
 class PagedSelfAttentionCore(torch.nn.Module):
@@ -127,6 +131,7 @@ class PagedSelfAttentionCore(torch.nn.Module):
         k_cache, v_cache, block_table = ctx.key_value_cache(self.layer_number)
         cu_q, max_q = ctx.cu_query_lengths()
         cu_k, kv_lens, max_k = ctx.cu_kv_lengths()
+        k_scales, v_scales = ctx.key_value_scales(self.layer_number) if hasattr(ctx, "key_value_scales") else (None, None)
         out = flash_decode_and_prefill(query, k_cache, v_cache, max_q, max_k, cu_q, cu_k, kv_lens, block_table,
-                                       softmax_scale=self.softmax_scale)
+                                       softmax_scale=self.softmax_scale, k_scales=k_scales, v_scales=v_scales)
         return out.reshape(out.size(0), out.size(1), -1)

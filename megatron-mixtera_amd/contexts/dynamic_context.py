@@ -118,6 +118,8 @@ class DynamicInferenceContext:
         use_cuda_graphs_for_non_decode_steps: bool = True,
         device: Optional[Union[torch.device, str, int]] = None,
         fused_bookkeeping: Optional[bool] = None,
+        kv_cache_dtype: Optional[Union[str, torch.dtype]] = None,
+        fp8_append_headroom: float = 2.0,
     ):
         if cache_mla_latent:
             raise NotImplementedError(
@@ -131,9 +133,24 @@ class DynamicInferenceContext:
             raise ValueError(f"{num_attention_heads} KV heads are not divisible by tensor parallel size {tp}")
         heads_here = num_attention_heads // tp
 
+        # ---- KV storage format: params_dtype as in the reference, or (an addition) e4m3 bytes with one
+        # fp32 scale per (key|value, layer, chunk, head) ----
+        if kv_cache_dtype in (None, params_dtype):
+            self.kv_cache_fp8 = False
+        elif kv_cache_dtype in ("fp8", "fp8_e4m3", "float8_e4m3fn", torch.float8_e4m3fn):
+            if params_dtype != torch.bfloat16:
+                raise ValueError("the fp8 KV cache quantises bf16 keys and values: params_dtype must be bfloat16")
+            self.kv_cache_fp8 = True
+        else:
+            raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r} (None or 'fp8_e4m3')")
+        self.fp8_append_headroom = float(fp8_append_headroom)
+
         # ---- sizing (reference: dynamic_context.py:186-242) ----
         self.chunk_size_tokens = chunk_size_tokens
-        self.chunk_size_bytes = params_dtype.itemsize * 2 * num_layers * chunk_size_tokens * heads_here * kv_channels
+        kv_itemsize = 1 if self.kv_cache_fp8 else params_dtype.itemsize
+        self.chunk_size_bytes = kv_itemsize * 2 * num_layers * chunk_size_tokens * heads_here * kv_channels
+        if self.kv_cache_fp8:
+            self.chunk_size_bytes += 4 * 2 * num_layers * heads_here  # its scales
         pool_bytes = int(buffer_size_gb * 1024**3)
         pool_bytes -= pool_bytes % self.chunk_size_bytes
         chunk_count_total = pool_bytes // self.chunk_size_bytes
@@ -193,9 +210,17 @@ class DynamicInferenceContext:
         self.token_to_local_position_within_kv_chunk = tok_row()
 
         # ---- the cache: [key|value, layer, chunk, token, head, channel] ----
-        self.memory_buffer = torch.full(
-            (2, num_layers, chunk_count_total, chunk_size_tokens, heads_here, kv_channels),
-            -1, dtype=params_dtype, device=dev)
+        if self.kv_cache_fp8:
+            # bytes (0 = +0.0 in e4m3; the reference's -1 fill would read as NaN here) and their scales
+            self.memory_buffer = torch.zeros(
+                (2, num_layers, chunk_count_total, chunk_size_tokens, heads_here, kv_channels),
+                dtype=torch.uint8, device=dev)
+            self.kv_scales = torch.ones((2, num_layers, chunk_count_total, heads_here), dtype=torch.float32, device=dev)
+        else:
+            self.memory_buffer = torch.full(
+                (2, num_layers, chunk_count_total, chunk_size_tokens, heads_here, kv_channels),
+                -1, dtype=params_dtype, device=dev)
+            self.kv_scales = None
 
         self.max_kv_chunk_count = math.ceil(max_sequence_length / chunk_size_tokens)
         self.request_to_kv_chunk_ids = torch.full(
@@ -322,6 +347,14 @@ class DynamicInferenceContext:
         """
         assert key.size(1) == 1 and value.size(1) == 1
         n = self.padded_active_token_count
+        if self.kv_cache_fp8:
+            ops.kv_append_fp8(
+                key[:n], value[:n],
+                self.memory_buffer[0, layer_number - 1], self.memory_buffer[1, layer_number - 1],
+                self.kv_scales[0, layer_number - 1], self.kv_scales[1, layer_number - 1],
+                self.token_to_chunk_idx, self.token_to_local_position_within_kv_chunk,
+                headroom=self.fp8_append_headroom)
+            return
         ops.kv_append(
             key[:n], value[:n],
             self.memory_buffer[0, layer_number - 1], self.memory_buffer[1, layer_number - 1],
@@ -330,6 +363,12 @@ class DynamicInferenceContext:
     def key_value_cache(self, layer_number: int) -> Tuple[Tensor, Tensor, Tensor]:
         """Views of the layer's key cache, value cache and this step's block table."""
         return (self.memory_buffer[0, layer_number - 1], self.memory_buffer[1, layer_number - 1], self.block_table)
+
+    def key_value_scales(self, layer_number: int) -> Tuple[Optional[Tensor], Optional[Tensor]]:
+        """fp8 cache: the layer's key and value scales ``[chunks, heads]``; otherwise ``(None, None)``."""
+        if not self.kv_cache_fp8:
+            return None, None
+        return self.kv_scales[0, layer_number - 1], self.kv_scales[1, layer_number - 1]
 
     @staticmethod
     def _rope_flags(config) -> bool:
@@ -374,6 +413,17 @@ class DynamicInferenceContext:
         (attention.py:1026-1030, 394-404, 766).  ``query`` is updated in place and returned.
         """
         n = self.padded_active_token_count
+        if self.kv_cache_fp8:
+            # norm + RoPE in one launch, then the quantising append (the roped key passes through memory)
+            key_out = torch.empty_like(key[:n])
+            ops.norm_rope_append(
+                query[:n], key[:n], key_out=key_out, q_weight=q_weight, k_weight=k_weight, eps=eps, norm=norm,
+                rotary_emb=rotary_pos_emb, q_positions=self.token_to_pos_ids,
+                k_positions=self.token_to_position_in_request,
+                rotary_interleaved=self._rope_flags(config) if config is not None else False, mscale=mscale,
+                faithful_rounding=faithful_rounding)
+            self.append_key_value_cache(layer_number, key_out, value[:n])
+            return query
         ops.norm_rope_append(
             query[:n], key[:n], value=value[:n], q_weight=q_weight, k_weight=k_weight, eps=eps, norm=norm,
             rotary_emb=rotary_pos_emb, q_positions=self.token_to_pos_ids,
@@ -403,6 +453,18 @@ class DynamicInferenceContext:
         if query_out is None:
             query_out = torch.empty((mixed_qkv.size(0), 1, num_query_heads, d), dtype=mixed_qkv.dtype,
                                     device=mixed_qkv.device)
+        if self.kv_cache_fp8:
+            key_out = torch.empty((n, 1, hkv, d), dtype=mixed_qkv.dtype, device=mixed_qkv.device)
+            ops.qkv_norm_rope_append(
+                mixed_qkv[:n], num_query_heads=num_query_heads, num_kv_heads=hkv, query_out=query_out[:n],
+                key_out=key_out, q_weight=q_weight, k_weight=k_weight, eps=eps, norm=norm, rotary_emb=rotary_pos_emb,
+                q_positions=self.token_to_pos_ids, k_positions=self.token_to_position_in_request,
+                rotary_interleaved=self._rope_flags(config) if config is not None else False, mscale=mscale,
+                faithful_rounding=faithful_rounding)
+            group = num_query_heads // hkv
+            value = mixed_qkv[:n].reshape(n, hkv, (group + 2) * d)[:, :, (group + 1) * d:].contiguous()
+            self.append_key_value_cache(layer_number, key_out, value.unsqueeze(1))
+            return query_out
         ops.qkv_norm_rope_append(
             mixed_qkv[:n], num_query_heads=num_query_heads, num_kv_heads=hkv, query_out=query_out[:n],
             q_weight=q_weight, k_weight=k_weight, eps=eps, norm=norm, rotary_emb=rotary_pos_emb,

@@ -55,7 +55,8 @@ def flash_attn_varlen_func(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor
                            softmax_scale: Optional[float] = None, causal: bool = False, window_size=(-1, -1),
                            softcap: float = 0.0, alibi_slopes=None, deterministic: bool = False,
                            return_attn_probs: bool = False, block_table: Optional[Tensor] = None,
-                           *, seqused_k: Optional[Tensor] = None) -> Tensor:
+                           *, seqused_k: Optional[Tensor] = None, k_scales: Optional[Tensor] = None,
+                           v_scales: Optional[Tensor] = None) -> Tensor:
     """Paged varlen causal attention: ``q`` is ``[T, Hq, d]``, ``k``/``v`` are the paged caches.
 
     Per-request key counts come from ``seqused_k`` if given, else from the differences of
@@ -74,4 +75,5 @@ def flash_attn_varlen_func(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor
     else:
         raise ValueError("need cu_seqlens_k or seqused_k")
     return ops.paged_prefill_attention(q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table,
-                                       softmax_scale=softmax_scale, max_kv_len=max_seqlen_k)
+                                       softmax_scale=softmax_scale, max_kv_len=max_seqlen_k,
+                                       k_scales=k_scales, v_scales=v_scales)

@@ -508,3 +508,26 @@ def test_random_request_streams_match_restatement(mi, Ctx, seed):
     assert {"added", "finished"} <= events
     if seed == 0:
         assert "paused" in events and "resumed" in events
+
+
+def test_fp8_cache_sizing_counts_bytes_and_scales(mi):
+    """An fp8 KV cache (an addition to the reference's constructor) sizes its pool from one byte per
+    element plus one fp32 scale per (key|value, layer, chunk, head): 512 KiB + 64 B for the
+    Mixtral-shape single-layer chunk of 256 tokens x 8 heads x 128."""
+    Ctx = mi.DynamicInferenceContext
+    c = Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=128, num_attention_heads=8,
+            max_sequence_length=1024, buffer_size_gb=8 * (512 * 1024 + 64) / 1024**3, buffer_guaranteed_fraction=0.1,
+            chunk_size_tokens=256, kv_cache_dtype="fp8_e4m3", device="cpu")
+    assert c.chunk_size_bytes == 512 * 1024 + 64
+    assert c.chunk_allocator.chunk_count_total == 8
+    assert c.memory_buffer.dtype == torch.uint8 and c.memory_buffer.numel() == 8 * 512 * 1024
+    assert c.kv_scales.shape == (2, 1, 8, 8)
+    assert c.key_value_scales(1)[0].shape == (8, 8)
+    b = Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=128, num_attention_heads=8,
+            max_sequence_length=1024, buffer_size_gb=8 * 1024 * 1024 / 1024**3, buffer_guaranteed_fraction=0.1,
+            chunk_size_tokens=256, device="cpu")
+    assert b.chunk_size_bytes == 1024 * 1024 and b.kv_scales is None and b.key_value_scales(1) == (None, None)
+    with pytest.raises(ValueError, match="kv_cache_dtype"):
+        Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=128, num_attention_heads=8,
+            max_sequence_length=1024, buffer_size_gb=0.01, buffer_guaranteed_fraction=0.1, kv_cache_dtype="int4",
+            device="cpu")
