@@ -48,6 +48,7 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--hip-graph", action="store_true", help="replay the step as one captured HIP graph")
     ap.add_argument("--attention-only", action="store_true", help="time the attention call alone")
+    ap.add_argument("--fp8-kv", action="store_true", help="cfg3 only: run the mixed batch over an fp8-e4m3 KV cache")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run a plain device copy of this many MiB (a known-size reference for "
                          "scaling hardware traffic counters collected by an external profiler)")
@@ -114,12 +115,27 @@ def run_mixed_batch(args, mi, lib, torch, dev):
     table = orn.rotary_table(max_len + 1, d, base=500000.0).to(dev)
     q_rot = torch.empty_like(q)
     out = torch.empty_like(q)
+    ks = vs = None
+    if args.fp8_kv:
+        k8, v8 = torch.empty(kc.shape, dtype=torch.uint8, device=dev), torch.empty(kc.shape, dtype=torch.uint8, device=dev)
+        ks = torch.empty(kc.size(0), Hkv, dtype=torch.float32, device=dev)
+        vs = torch.empty_like(ks)
+        mi.ops.quantize_chunks_fp8(kc, k8, ks)
+        mi.ops.quantize_chunks_fp8(vc, v8, vs)
+        kc, vc = k8, v8
+        k_rot = torch.empty_like(k_new)
 
     def step():
-        mi.ops.norm_rope_append(q, k_new, query_out=q_rot, value=v_new, q_weight=qw, k_weight=kw, eps=1e-5,
-                                norm="rms", rotary_emb=table, q_positions=pos, k_positions=pos, k_cache=kc,
-                                v_cache=vc, token_to_chunk_idx=tok_chunk, token_to_local_pos=tok_local)
-        mi.ops.paged_prefill_attention(q_rot, kc, vc, cu_q, lens, bt, max_kv_len=max_len, out=out)
+        if args.fp8_kv:
+            mi.ops.norm_rope_append(q, k_new, query_out=q_rot, key_out=k_rot, q_weight=qw, k_weight=kw, eps=1e-5,
+                                    norm="rms", rotary_emb=table, q_positions=pos, k_positions=pos)
+            mi.ops.kv_append_fp8(k_rot, v_new, kc, vc, ks, vs, tok_chunk, tok_local)
+        else:
+            mi.ops.norm_rope_append(q, k_new, query_out=q_rot, value=v_new, q_weight=qw, k_weight=kw, eps=1e-5,
+                                    norm="rms", rotary_emb=table, q_positions=pos, k_positions=pos, k_cache=kc,
+                                    v_cache=vc, token_to_chunk_idx=tok_chunk, token_to_local_pos=tok_local)
+        mi.ops.paged_prefill_attention(q_rot, kc, vc, cu_q, lens, bt, max_kv_len=max_len, out=out,
+                                       k_scales=ks, v_scales=vs)
 
     for _ in range(args.warmup):
         step()
@@ -141,8 +157,9 @@ def run_mixed_batch(args, mi, lib, torch, dev):
     pre = lq > 1
     flops = 4 * Hq * d * int((lq[pre] * (lk - lq)[pre] + lq[pre] * (lq[pre] + 1) // 2).sum())
     from oracle import paged_attention as oa
-    dec_bytes = oa.decode_attention_bytes(lk[~pre].tolist(), Hq, Hkv, d, chunk)
-    pre_kv_bytes = int(lk[pre].sum()) * Hkv * d * 2 * 2 + int(lq[pre].sum()) * Hq * d * 4
+    kvb = 1 if args.fp8_kv else 2
+    dec_bytes = oa.decode_attention_bytes(lk[~pre].tolist(), Hq, Hkv, d, chunk, kv_bytes=kvb, fp8_scales=args.fp8_kv)
+    pre_kv_bytes = int(lk[pre].sum()) * Hkv * d * 2 * kvb + int(lq[pre].sum()) * Hq * d * 4
     ms_per_step = elapsed * 1e3 / args.steps
     total_bytes = dec_bytes + pre_kv_bytes
     result = {
@@ -150,9 +167,11 @@ def run_mixed_batch(args, mi, lib, torch, dev):
         "value": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
         "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 (fp32 accumulate)", "data": "synthetic",
+        "dtype": "fp8-e4m3 KV, bf16 q/out, fp32 accumulate" if args.fp8_kv else "bf16 (fp32 accumulate)",
+        "data": "synthetic",
         "config": {"workload": "cfg3: mixed batch, 8 x 2048-token prefill over U[0,4096] + 120 decode U[512,8192], "
-                               "32/8 heads d128 chunk 256; step = fused RMSNorm+RoPE+append then paged varlen attention",
+                               "32/8 heads d128 chunk 256; step = fused RMSNorm+RoPE+append then paged varlen attention"
+                               + (" (fp8-e4m3 KV cache, quantising append)" if args.fp8_kv else ""),
                    "new_tokens": T, "requests": int(lens.numel()), "algorithmic_bytes_per_step": total_bytes,
                    "prefill_flops_per_step": flops},
         "roofline": {"bound": "mfma", "kernel": "paged_prefill_pp_kernel", "achieved": round(flops / tile_ms / 1e9, 1),

@@ -157,52 +157,101 @@ struct AppendFp8Params {
   float headroom;
 };
 
-// grid = (T, Hkv, 2): the workgroup of a run's first token computes the scale of (chunk, head).
+// grid = (ceil(T / 64), Hkv, 2): a workgroup looks at 64 tokens and, for each of them that opens a
+// chunk (local position 0), computes the scale of (chunk, head) of the key (z = 0) or value (z = 1)
+// cache from the whole run that starts there.
 __global__ __launch_bounds__(256) void kv_append_fp8_scales_kernel(AppendFp8Params p) {
-  const int t = blockIdx.x, h = blockIdx.y, kv = blockIdx.z;
-  if (p.tok_local[t] != 0) return;  // not the opening token of a chunk
-  const int64_t c = p.tok_chunk[t];
+  const int t0 = blockIdx.x * 64, h = blockIdx.y, kv = blockIdx.z;
+  __shared__ int open_s[64];
+  __shared__ int n_open_s;
   __shared__ int run_s[256];
   __shared__ float red[256];
-  // run length: first i >= 1 where token t+i is not (chunk c, local i)
-  int first_bad = p.chunk;
-  for (int i = 1 + threadIdx.x; i < p.chunk; i += 256) {
-    const bool ok = t + i < p.T && p.tok_chunk[t + i] == c && p.tok_local[t + i] == i;
-    if (!ok) { first_bad = i; break; }
+  if (threadIdx.x < 64) {
+    const int t = t0 + threadIdx.x;
+    const bool opens = t < p.T && p.tok_local[t] == 0;
+    const uint64_t m = __builtin_amdgcn_ballot_w64(opens);
+    if (opens) open_s[__builtin_popcountll(m & (((uint64_t)1 << threadIdx.x) - 1))] = t;
+    if (threadIdx.x == 0) n_open_s = __builtin_popcountll(m);
   }
-  run_s[threadIdx.x] = first_bad;
   __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if ((int)threadIdx.x < s) run_s[threadIdx.x] = min(run_s[threadIdx.x], run_s[threadIdx.x + s]);
+  const int n_open = n_open_s;
+  // 8 elements (16 bytes) per thread step when the rows allow it
+  const bool wide = !((p.d | p.src_stride) & 7) && !((uintptr_t)p.src[kv] & 15);
+  for (int k = 0; k < n_open; ++k) {
+    const int t = open_s[k];
+    const int64_t c = p.tok_chunk[t];
+    // run length: first i >= 1 where token t+i is not (chunk c, local i)
+    int first_bad = p.chunk;
+    for (int i = 1 + threadIdx.x; i < p.chunk; i += 256) {
+      const bool ok = t + i < p.T && p.tok_chunk[t + i] == c && p.tok_local[t + i] == i;
+      if (!ok) { first_bad = i; break; }
+    }
     __syncthreads();
-  }
-  const int n = run_s[0];
-  const uint16_t* src = p.src[kv] + (int64_t)t * p.src_stride + (int64_t)h * p.d;
-  float amax = 0.f;
-  for (int i = threadIdx.x; i < n * p.d; i += 256) {
-    const int tok = i / p.d, e = i - tok * p.d;
-    amax = fmaxf(amax, fabsf(bf16_to_f32(src[(int64_t)tok * p.src_stride + e])));
-  }
-  red[threadIdx.x] = amax;
-  __syncthreads();
-  for (int s = 128; s > 0; s >>= 1) {
-    if ((int)threadIdx.x < s) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+    run_s[threadIdx.x] = first_bad;
     __syncthreads();
-  }
-  if (threadIdx.x == 0) {
-    const float hr = n == p.chunk ? 1.f : p.headroom;
-    p.scale[kv][c * p.Hkv + h] = red[0] > 0.f ? hr * red[0] / 448.f : 1.f;
+    for (int s = 128; s > 0; s >>= 1) {
+      if ((int)threadIdx.x < s) run_s[threadIdx.x] = min(run_s[threadIdx.x], run_s[threadIdx.x + s]);
+      __syncthreads();
+    }
+    const int n = run_s[0];
+    const uint16_t* src = p.src[kv] + (int64_t)t * p.src_stride + (int64_t)h * p.d;
+    float amax = 0.f;
+    if (wide) {
+      const int per_row = p.d >> 3;
+      for (int i = threadIdx.x; i < n * per_row; i += 256) {
+        const int tok = i / per_row, e = (i - tok * per_row) << 3;
+        const uint4 w = ld16(src + (int64_t)tok * p.src_stride + e);
+        const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          amax = fmaxf(amax, fmaxf(fabsf(bf16lo_to_f32(u[j])), fabsf(bf16hi_to_f32(u[j]))));
+      }
+    } else {
+      for (int i = threadIdx.x; i < n * p.d; i += 256) {
+        const int tok = i / p.d, e = i - tok * p.d;
+        amax = fmaxf(amax, fabsf(bf16_to_f32(src[(int64_t)tok * p.src_stride + e])));
+      }
+    }
+    red[threadIdx.x] = amax;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+      if ((int)threadIdx.x < s) red[threadIdx.x] = fmaxf(red[threadIdx.x], red[threadIdx.x + s]);
+      __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+      const float hr = n == p.chunk ? 1.f : p.headroom;
+      p.scale[kv][c * p.Hkv + h] = red[0] > 0.f ? hr * red[0] / 448.f : 1.f;
+    }
   }
 }
 
-// grid = (T, Hkv, 2): quantise one head row of one token with its chunk's scale.
-__global__ __launch_bounds__(64) void kv_append_fp8_rows_kernel(AppendFp8Params p) {
-  const int t = blockIdx.x, h = blockIdx.y, kv = blockIdx.z;
+// grid = (T, 2): quantise the key (y = 0) or value (y = 1) row of one token with its chunk's scales.
+__global__ __launch_bounds__(256) void kv_append_fp8_rows_kernel(AppendFp8Params p) {
+  const int t = blockIdx.x, kv = blockIdx.y;
   const int64_t c = p.tok_chunk[t], l = p.tok_local[t];
-  const float scale = p.scale[kv][c * p.Hkv + h];
-  const uint16_t* src = p.src[kv] + (int64_t)t * p.src_stride + (int64_t)h * p.d;
-  uint8_t* dst = p.dst[kv] + c * p.chunk_bytes + l * p.tok_bytes + (int64_t)h * p.d;
-  for (int e = threadIdx.x; e < p.d; e += 64) dst[e] = (uint8_t)f32_to_e4m3_sat(bf16_to_f32(src[e]) / scale);
+  const uint16_t* src = p.src[kv] + (int64_t)t * p.src_stride;
+  uint8_t* dst = p.dst[kv] + c * p.chunk_bytes + l * p.tok_bytes;
+  const float* scales = p.scale[kv] + c * p.Hkv;
+  const int row = p.Hkv * p.d;
+  const bool wide = !((p.d | p.src_stride) & 7) && !((uintptr_t)p.src[kv] & 15) &&
+                    !(((uintptr_t)p.dst[kv] | (uintptr_t)p.chunk_bytes | (uintptr_t)p.tok_bytes) & 7);
+  if (wide) {
+    for (int e = threadIdx.x * 8; e < row; e += 256 * 8) {
+      const float scale = scales[e / p.d];
+      const uint4 w = ld16(src + e);
+      const uint32_t u[4] = {w.x, w.y, w.z, w.w};
+      uint32_t out[2] = {0u, 0u};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = f32_to_e4m3_sat(bf16lo_to_f32(u[j]) / scale), hi = f32_to_e4m3_sat(bf16hi_to_f32(u[j]) / scale);
+        out[j >> 1] |= (lo | (hi << 8)) << (16 * (j & 1));
+      }
+      st8(dst + e, make_uint2(out[0], out[1]));
+    }
+  } else {
+    for (int e = threadIdx.x; e < row; e += 256)
+      dst[e] = (uint8_t)f32_to_e4m3_sat(bf16_to_f32(src[e]) / scales[e / p.d]);
+  }
 }
 
 template <bool DECODE>
@@ -327,7 +376,7 @@ extern "C" int mi_kv_append_fp8(const void* key_bf16, const void* value_bf16, in
   p.tok_chunk = token_to_chunk_idx; p.tok_local = token_to_local_pos;
   p.T = T; p.chunk = chunk_tokens; p.Hkv = Hkv; p.d = head_dim; p.headroom = headroom;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(kv_append_fp8_scales_kernel, dim3(T, Hkv, 2), dim3(256), 0, st, p);
-  hipLaunchKernelGGL(kv_append_fp8_rows_kernel, dim3(T, Hkv, 2), dim3(64), 0, st, p);
+  hipLaunchKernelGGL(kv_append_fp8_scales_kernel, dim3((T + 63) / 64, Hkv, 2), dim3(256), 0, st, p);
+  hipLaunchKernelGGL(kv_append_fp8_rows_kernel, dim3(T, 2), dim3(256), 0, st, p);
   return mi_check_launch("mi_kv_append_fp8");
 }
