@@ -52,8 +52,8 @@ const char* mi_last_error(void);
  * "decode_grid" (0 = automatic), "decode_waves_per_block" (1..8), "prefill_pingpong" (1 = two-phase
  * tile kernel, 2 = the same kernel with its wave groups in lock-step, 0 = older LDS kernel),
  * "prefill_tile_subtiles", "prefill_lds_row_tiles", "prefill_row_tiles" (the older kernels),
- * "norm_rope_vectorised" (1 = 16-byte-per-lane norm / rotary kernel where alignment and the rotary
- * width allow it, 0 = element-wise kernel always). */
+ * "norm_rope_vectorised" (16-byte-per-lane norm / rotary kernel: 1 = wherever alignment and the rotary
+ * width allow it, 2 = the same but only from 256 tokens up (default), 0 = element-wise kernel always). */
 int mi_set_tuning(const char* name, int32_t value);
 
 /*

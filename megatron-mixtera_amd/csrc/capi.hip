@@ -29,7 +29,7 @@ MiTuning& mi_tuning() {
                       env_int("MI355_PREFILL_LDS_ROW_TILES", 2), env_int("MI355_PREFILL_ROW_TILES", 2),
                       env_int("MI355_DECODE_MIN_WAVES", 3),
                       env_int("MI355_DECODE_WGS_PER_CU", 1), env_int("MI355_DECODE_GRID", 0),
-                      env_int("MI355_DECODE_WAVES_PER_BLOCK", 8), env_int("MI355_NORM_ROPE_VECTORISED", 1),
+                      env_int("MI355_DECODE_WAVES_PER_BLOCK", 8), env_int("MI355_NORM_ROPE_VECTORISED", 2),
                       env_int("MI355_PREFILL_PINGPONG", 1)};
   return t;
 }
@@ -76,7 +76,7 @@ extern "C" int mi_set_tuning(const char* name, int32_t value) {
     return MI_OK;
   }
   if (!strcmp(name, "norm_rope_vectorised")) {
-    if (value != 0 && value != 1) return mi_fail(MI_ERR_UNSUPPORTED, "norm_rope_vectorised must be 0 or 1");
+    if (value < 0 || value > 2) return mi_fail(MI_ERR_UNSUPPORTED, "norm_rope_vectorised must be 0, 1 or 2");
     mi_tuning().norm_rope_vectorised = value;
     return MI_OK;
   }

@@ -31,7 +31,7 @@ struct MiTuning {
   int decode_wgs_per_cu;       // decode workgroups (of 8 waves) per CU in the streaming grid
   int decode_grid;             // >0 forces the streaming grid size (tests)
   int decode_waves_per_block;  // cap on wavefronts (= KV heads) per decode workgroup, 1..8
-  int norm_rope_vectorised;    // 1 = 16-byte-per-lane norm/RoPE kernel when shapes allow, 0 = element-wise kernel
+  int norm_rope_vectorised;    // 16-byte-per-lane norm/RoPE kernel: 1 = whenever shapes allow, 2 = and T >= 256 (default), 0 = never
   int prefill_pingpong;        // head_dim-128 prefill: 1 = two wave groups one phase apart, 2 = same kernel in lock-step, 0 = off
 };
 

@@ -425,7 +425,10 @@ int norm_rope_launch(NormRopeParams& p, hipStream_t st, const char* name) {
                          (uintptr_t)p.q_w | (uintptr_t)p.k_w | (to_cache ? ((uintptr_t)p.v | (uintptr_t)p.vc) : 0);
   const int64_t strides = p.q_st | p.q_gst | p.qo_st | p.k_st | p.k_hst | p.ko_st |
                           (to_cache ? (p.chunk_elems | p.tok_elems | p.v_st | p.v_hst) : 0);
-  const bool vec = rot_ok && (ptrs & 15) == 0 && (strides & 7) == 0 && mi_tuning().norm_rope_vectorised != 0;
+  // The 16-byte-per-lane kernel wins on many tokens; on a decode batch (a few hundred rows at most) the
+  // element-wise kernel's shorter dependent chain does (4.8 against 5.7 us at 64 tokens).
+  const int mode = mi_tuning().norm_rope_vectorised;  // 0 never, 1 whenever the shapes allow, 2 automatic
+  const bool vec = rot_ok && (ptrs & 15) == 0 && (strides & 7) == 0 && (mode == 1 || (mode == 2 && p.T >= 256));
   const int vpb = vec ? (p.d == 128 ? 16 : 32) : (p.d == 128 ? 4 : 8);
   const int passes = (p.Hq + p.Hkv + vpb - 1) / vpb;
   int gy = (2048 + p.T - 1) / p.T;

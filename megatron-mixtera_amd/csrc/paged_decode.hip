@@ -125,7 +125,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   uint4 kf[NT][FP8 ? KS / 2 : KS];
   uint4 vf16[NT][4];  // bf16, HD=128 : 16 B per token
   uint2 vf8[NT][4];   // bf16 HD=64 or fp8 HD=128 : 8 B per token
-  float ksc[NT], vsc[NT];
+  float ksc_tile = 1.f, vsc_tile = 1.f;  // fp8: scales of the chunk the staged K / V tile lies in
 
   // Addressing.  A tile of 16*NT tokens never straddles a chunk (the launcher picks NT so that the
   // tile size divides the chunk size), so its address is
@@ -203,12 +203,12 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   auto load_k = [&](int T) {
     int tok0;
     const uint8_t* chunk = tile_chunk(kcur, p.k_scale, kbase, T, tok0);
+    if (FP8) ksc_tile = kcur.sc;
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       const int t0 = min(T + 16 * u, last);
       const uint32_t lim = (uint32_t)min(last - t0, 15) * tok_bytes;
       const uint8_t* krow = chunk + (uint32_t)(t0 - tok0) * tok_bytes + min(k_lane, lim + k_col);
-      if (FP8) ksc[u] = kcur.sc;
 #pragma unroll
       for (int kk = 0; kk < (FP8 ? KS / 2 : KS); ++kk) kf[u][kk] = ld16_stream(krow + 64 * kk);
     }
@@ -216,12 +216,12 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   auto load_v = [&](int T) {
     int tok0;
     const uint8_t* chunk = tile_chunk(vcur, p.v_scale, vbase, T, tok0);
+    if (FP8) vsc_tile = vcur.sc;
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       const int t0 = min(T + 16 * u, last);
       const uint32_t cap = (uint32_t)min(last - t0, 15) * tok_bytes + v_col;
       const uint8_t* tile = chunk + (uint32_t)(t0 - tok0) * tok_bytes;
-      if (FP8) vsc[u] = vcur.sc;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint8_t* vrow = tile + min(v_lane[j], cap);
@@ -235,17 +235,15 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   load_v(start);
   __builtin_amdgcn_sched_barrier(0);
   if (FP8) {  // the first tile lies in the opening chunk
-    kcur.sc = uniform_f(ksc_first);
-    vcur.sc = uniform_f(vsc_first);
-#pragma unroll
-    for (int u = 0; u < NT; ++u) { ksc[u] = kcur.sc; vsc[u] = vcur.sc; }
+    kcur.sc = ksc_tile = uniform_f(ksc_first);
+    vcur.sc = vsc_tile = uniform_f(vsc_first);
   }
   const uint2 ones = make_uint2(0x3f803f80u, 0x3f803f80u);  // four bf16 1.0
   for (int T = start; T < end; T += 16 * NT) {
     // ---- S^T = K Q^T ---------------------------------------------------------
     // The tile lies in one chunk, so one K scale and one V scale hold for all of it; the score
     // multiplier is positive and wave-uniform, so the maximum is taken over the raw products.
-    const float mul = FP8 ? p.scale_log2 * ksc[0] : p.scale_log2;
+    const float mul = FP8 ? p.scale_log2 * ksc_tile : p.scale_log2;
     const bool ragged = T + 16 * NT > end;  // only the last tile of a segment has masked tokens
     float sc[NT][4];
     float tmax = -INFINITY;
@@ -274,7 +272,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       for (int i = 0; i < 4; ++i) sc[u][i] = sacc[i];
       tmax = fmaxf(fmaxf(tmax, sacc[0]), fmaxf(sacc[1], fmaxf(sacc[2], sacc[3])));
     }
-    const float vscale = FP8 ? vsc[0] : 1.f;
+    const float vscale = FP8 ? vsc_tile : 1.f;
     // The scheduling fences keep each batch of prefetch loads together at this point of the
     // loop instead of letting the compiler sink them next to their uses one by one.
     __builtin_amdgcn_sched_barrier(0);

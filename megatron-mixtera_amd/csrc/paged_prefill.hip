@@ -661,7 +661,6 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 
   const int q0 = q0_wg + wave * BQ;
   const int nq = max(0, min(BQ, Lq - q0));
-  const int kend = nq > 0 ? min(Lk, shift + q0 + nq) : 0;
   const int full_until = shift + q0;
 
   uint4 qf[NQ][KS];

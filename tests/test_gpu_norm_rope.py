@@ -33,7 +33,7 @@ def test_norm_rope_matches_unfused_chain(mi, dev, norm, interleaved, d, rot, vec
     try:
         _norm_rope_case(mi, dev, norm, interleaved, d, rot)
     finally:
-        mi.ops.set_tuning("norm_rope_vectorised", 1)
+        mi.ops.set_tuning("norm_rope_vectorised", 2)
 
 
 def _norm_rope_case(mi, dev, norm, interleaved, d, rot):
@@ -176,7 +176,7 @@ def test_mixed_qkv_input_equals_split_inputs(mi, dev, d, hq, hkv, vectorised, in
             assert (err <= 2e-2 + 2e-2 * ref.float().abs()).all(), f"max err {err.max().item()}"
             assert (_ulp_diff(got, ref) > 0).float().mean().item() < 0.01
     finally:
-        mi.ops.set_tuning("norm_rope_vectorised", 1)
+        mi.ops.set_tuning("norm_rope_vectorised", 2)
 
 
 def test_mixed_qkv_argument_errors(mi, dev):
