@@ -160,6 +160,28 @@ int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_str
                               void* stream);
 
 /*
+ * Decode attention over the latent cache of multi-latent attention (absorbed form).
+ * Replaces flash_mla_with_kvcache(q, kv_cache.unsqueeze(-2), block_table, cache_seqlens, head_dim_v,
+ * tile_scheduler_metadata, num_splits, softmax_scale=, causal=True) together with get_mla_metadata
+ * as called from Attention.flash_decode_and_prefill
+ * (megatron/core/transformer/attention.py:561-587): the cache holds one row of head_dim_k = 576
+ * values per token (kv_lora_rank 512 + rotary 64; dynamic_context.py:288-294,533-538), shared by
+ * all query heads:
+ *   out[r,h] = softmax(q[r,h] . KV_r[:len_r, :576]^T * softmax_scale) . KV_r[:len_r, :512]
+ * q bf16 `[R, Hq, 576]`, out bf16 `[R, Hq, 512]`, kv_cache bf16 `[n_chunks, chunk_tokens, 576]` with
+ * the given chunk / token strides (elements).  Hq: 1, 2, 4, 8 or a multiple of 16.
+ */
+int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v);
+
+int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
+                                  const void* kv_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok,
+                                  const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
+                                  void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
+                                  int64_t workspace_bytes, int32_t R, int32_t Hq, int32_t head_dim_k,
+                                  int32_t head_dim_v, int32_t chunk_tokens, int32_t max_kv_len,
+                                  float softmax_scale, void* stream);
+
+/*
  * Paged varlen causal attention for prefill / mixed prefill+decode batches.
  * Replaces flash_attn_varlen_func(q, k_cache, v_cache, cu_seqlens_q, cu_seqlens_k,
  * max_seqlen_q, max_seqlen_k, softmax_scale, causal=True, block_table=...)

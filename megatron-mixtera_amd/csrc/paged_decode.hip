@@ -71,12 +71,17 @@ static __device__ __forceinline__ int chunk_of(int tok, uint64_t magic) {
 
 // One segment: tokens [start, end) of request r for KV head h (one wavefront).
 // `whole` = the segment is the entire request (write bf16 output, no partial).
-template <int HD, int NT, bool FP8>
+// HDK = width of the keys (and queries), HDV = width of the values (and of the output).  They differ
+// only for the latent cache of multi-latent attention (576 / 512: the value is the first 512 of the
+// shared 576-wide row, the caller points both cache arguments at the same buffer).
+template <int HDK, int HDV, int NT, bool FP8>
 static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int row, int h, int len,
                                                       int start, int end, bool whole, int slot, int lane) {
-  constexpr int KS = HD / 32;
-  constexpr int DV = HD / 16;
-  static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
+  constexpr int KS = HDK / 32;
+  constexpr int DV = HDV / 16;
+  constexpr int VW = DV * (FP8 ? 1 : 2) / 16;  // 16-byte loads per token and lane of the value operand (0: 8 bytes)
+  static_assert((HDK == 64 || HDK == 128 || HDK == 576) && (HDV == 64 || HDV == 128 || HDV == 512), "head widths");
+  static_assert(!FP8 || (HDK == 128 && HDV == 128), "fp8 KV: head_dim 128");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
   // tile base addresses below run on the scalar unit instead of costing vector instructions.
@@ -123,8 +128,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   // scores of the current one exist, V of the next tile as soon as the current P.V is done,
   // so every wave keeps loads in flight while it computes.
   uint4 kf[NT][FP8 ? KS / 2 : KS];
-  uint4 vf16[NT][4];  // bf16, HD=128 : 16 B per token
-  uint2 vf8[NT][4];   // bf16 HD=64 or fp8 HD=128 : 8 B per token
+  uint4 vf16[NT][4][VW > 0 ? VW : 1];  // bf16, value width 128 (512): 16 (64) bytes per token and lane
+  uint2 vf8[NT][4];                    // bf16 width 64 or fp8 width 128: 8 bytes per token and lane
   float ksc_tile = 1.f, vsc_tile = 1.f;  // fp8: scales of the chunk the staged K / V tile lies in
 
   // Addressing.  A tile of 16*NT tokens never straddles a chunk (the launcher picks NT so that the
@@ -225,8 +230,12 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint8_t* vrow = tile + min(v_lane[j], cap);
-        if (!FP8 && HD == 128) vf16[u][j] = ld16_stream(vrow);
-        else vf8[u][j] = ld8_stream(vrow);
+        if (VW > 0) {
+#pragma unroll
+          for (int w = 0; w < VW; ++w) vf16[u][j][w] = ld16_stream(vrow + 16 * w);
+        } else {
+          vf8[u][j] = ld8_stream(vrow);
+        }
       }
     }
   };
@@ -311,25 +320,28 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     // ---- O^T += V^T P^T --------------------------------------------------------
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
-      if (!FP8 && HD == 128) {
-        const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0]);
-        const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1]);
-        const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2]);
-        const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3]);
+      if (VW > 0) {  // bf16, 8 * VW values per token per lane
 #pragma unroll
-        for (int pr = 0; pr < 4; ++pr) {
-          acc[2 * pr] = mfma_16x16x16(
-              make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr])), pf[u], acc[2 * pr]);
-          acc[2 * pr + 1] = mfma_16x16x16(
-              make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr])), pf[u], acc[2 * pr + 1]);
+        for (int w = 0; w < VW; ++w) {
+          const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0][w]);
+          const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1][w]);
+          const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2][w]);
+          const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3][w]);
+#pragma unroll
+          for (int pr = 0; pr < 4; ++pr) {
+            acc[8 * w + 2 * pr] = mfma_16x16x16(
+                make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr])), pf[u], acc[8 * w + 2 * pr]);
+            acc[8 * w + 2 * pr + 1] = mfma_16x16x16(
+                make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr])), pf[u], acc[8 * w + 2 * pr + 1]);
+          }
         }
-      } else if (!FP8) {  // bf16, HD == 64: four values per token per lane
+      } else if (!FP8) {  // bf16, value width 64: four values per token per lane
         const uint2 a = vf8[u][0], b = vf8[u][1], c = vf8[u][2], d = vf8[u][3];
         acc[0] = mfma_16x16x16(make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x)), pf[u], acc[0]);
         acc[1] = mfma_16x16x16(make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x)), pf[u], acc[1]);
         acc[2] = mfma_16x16x16(make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y)), pf[u], acc[2]);
         acc[3] = mfma_16x16x16(make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y)), pf[u], acc[3]);
-      } else {  // fp8, HD == 128: eight bytes per token per lane
+      } else {  // fp8, width 128: eight bytes per token per lane
         uint2 w[4][2];  // [token j][half] -> two packed bf16 pairs (4 d values)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -363,11 +375,14 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + 4 * DV * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if constexpr (DV == 8) {
-        st16(o + 8 * i, make_uint4(pack_bf16x2(acc[0][i] * inv, acc[1][i] * inv),
-                                   pack_bf16x2(acc[2][i] * inv, acc[3][i] * inv),
-                                   pack_bf16x2(acc[4][i] * inv, acc[5][i] * inv),
-                                   pack_bf16x2(acc[6][i] * inv, acc[7][i] * inv)));
+      if constexpr (DV >= 8) {
+#pragma unroll
+        for (int w = 0; w < DV / 8; ++w)
+          st16(o + DV * i + 8 * w,
+               make_uint4(pack_bf16x2(acc[8 * w + 0][i] * inv, acc[8 * w + 1][i] * inv),
+                          pack_bf16x2(acc[8 * w + 2][i] * inv, acc[8 * w + 3][i] * inv),
+                          pack_bf16x2(acc[8 * w + 4][i] * inv, acc[8 * w + 5][i] * inv),
+                          pack_bf16x2(acc[8 * w + 6][i] * inv, acc[8 * w + 7][i] * inv)));
       } else {
         st8(o + 4 * i, make_uint2(pack_bf16x2(acc[0][i] * inv, acc[1][i] * inv),
                                   pack_bf16x2(acc[2][i] * inv, acc[3][i] * inv)));
@@ -375,7 +390,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     }
   } else {
     const int64_t row = (int64_t)slot * p.Hq + hq;
-    float* o = p.part_o + row * HD + 4 * DV * g;
+    float* o = p.part_o + row * HDV + 4 * DV * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
 #pragma unroll
@@ -401,8 +416,9 @@ static __device__ __forceinline__ bool decode_row(const DecodeParams& p, int r, 
   return p.cu_q[r + 1] - row == 1;
 }
 
-template <int HD, int NT, bool FP8, int MINW>
-__global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
+// The body of the streaming kernels: span of this workgroup, then its segments one after the other.
+template <int HDK, int HDV, int NT, bool FP8>
+static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p) {
   constexpr int TK = 16 * NT;
   extern __shared__ int cum[];  // inclusive prefix sum of tiles per request, [R], then the lengths, [R]
   int* const len_s = cum + p.R;
@@ -467,12 +483,25 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
       }
       int row;
       decode_row(p, r, row);
-      decode_segment<HD, NT, FP8>(p, r, row, h, len, tb * TK, min(te * TK, len), first && final,
-                                  (int)blockIdx.x + r, lane);
+      decode_segment<HDK, HDV, NT, FP8>(p, r, row, h, len, tb * TK, min(te * TK, len), first && final,
+                                        (int)blockIdx.x + r, lane);
       t0 = rb + te;
     }
     ++r;
   }
+}
+
+template <int HD, int NT, bool FP8, int MINW>
+__global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
+  decode_stream_body<HD, HD, NT, FP8>(p);
+}
+
+// Multi-latent attention, absorbed form: every query head attends to the same 576-wide latent rows
+// (scores over all 576 values, output = weighted sum of the first 512).  A wavefront takes 16 query
+// heads; with 128 accumulator registers per lane a SIMD holds one wavefront, hence at most four per
+// workgroup.
+__global__ __launch_bounds__(256, 1) void paged_mla_decode_stream_kernel(DecodeParams p) {
+  decode_stream_body<576, 512, 1, false>(p);
 }
 
 // One workgroup per (request, query head): merge the partials of the workgroups that
@@ -674,4 +703,96 @@ extern "C" int mi_paged_decode_attention(
                              kv_stride_head, block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok,
                              o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
                              split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Multi-latent attention (absorbed decode): one shared latent row per token, every query head
+// attends to it.  The streaming kernel sees the 16-head query groups as "KV heads" whose cache
+// head stride is zero, and is handed the same buffer as key and value cache.
+// ---------------------------------------------------------------------------------------------
+namespace mi {
+// query groups (wavefronts) per workgroup: at most four, one per SIMD
+static int mla_waves_per_block(int groups) {
+  for (int w = 4; w >= 1; --w)
+    if (groups % w == 0) return w;
+  return 1;
+}
+// spans along the flattened tile sequence: four wavefronts on every CU in total
+static int mla_grid_size(int groups) {
+  const int forced = mi_tuning().decode_grid;
+  if (forced > 0) return forced;
+  const int grid = device_cu_count() * 4 / groups;
+  return grid < 1 ? 1 : grid;
+}
+static int mla_groups(int Hq) { return Hq <= 16 ? 1 : Hq / 16; }
+}  // namespace mi
+
+extern "C" int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v) {
+  if (R <= 0 || Hq <= 0 || head_dim_v <= 0) return 0;
+  const int64_t slots = (int64_t)mla_grid_size(mla_groups(Hq)) + R;
+  return slots * Hq * (head_dim_v + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
+}
+
+extern "C" int mi_paged_mla_decode_attention(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* kv_cache, int64_t kv_stride_chunk,
+    int64_t kv_stride_tok, const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
+    int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq,
+    int32_t head_dim_k, int32_t head_dim_v, int32_t chunk_tokens, int32_t max_kv_len, float softmax_scale,
+    void* stream) {
+  (void)max_kv_len;
+  if (R == 0) return MI_OK;
+  if (!q || !kv_cache || !block_table || !kv_lens || !out)
+    return mi_fail(MI_ERR_NULL, "mi_paged_mla_decode_attention: null pointer argument");
+  if (R < 0 || Hq <= 0) return mi_fail(MI_ERR_SHAPE, "mi_paged_mla_decode_attention: need R >= 0 and Hq > 0");
+  if (head_dim_k != 576 || head_dim_v != 512)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: latent rows of 576 values (512 + 64) only");
+  if ((Hq > 16 && Hq % 16) || (Hq < 16 && (Hq & (Hq - 1))))
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: Hq must be 1, 2, 4, 8 or a multiple of 16");
+  if (chunk_tokens <= 0 || chunk_tokens % 16)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_mla_decode_attention: chunk size must be a positive multiple of 16");
+  if (((uintptr_t)q | (uintptr_t)kv_cache | (uintptr_t)out) & 15)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_mla_decode_attention: q / cache / out must be 16-byte aligned");
+  if ((q_stride_tok | q_stride_head | o_stride_tok | o_stride_head | kv_stride_chunk | kv_stride_tok) % 8)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_mla_decode_attention: strides must keep rows 16-byte aligned");
+  if (kv_stride_tok < head_dim_k || kv_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_mla_decode_attention: bad token stride, or a chunk of 2 GiB or more");
+  if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_mla_decode_attention: softmax_scale must be positive");
+  if ((int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: batch too large for the in-LDS prefix sum (7680 requests)");
+
+  const int groups = mla_groups(Hq);
+  const int grid_x = mla_grid_size(groups);
+  const int64_t slots = (int64_t)grid_x + R;
+  const int64_t need = slots * Hq * (head_dim_v + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
+  if (!workspace || workspace_bytes < need)
+    return mi_fail(MI_ERR_WORKSPACE, "mi_paged_mla_decode_attention: workspace too small (see mi_mla_decode_workspace_bytes)");
+  if ((uintptr_t)workspace & 15)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_mla_decode_attention: workspace must be 16-byte aligned");
+
+  DecodeParams p;
+  p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
+  p.kc = (const uint8_t*)kv_cache; p.vc = (const uint8_t*)kv_cache;  // value = first head_dim_v values of the row
+  p.kv_sc = kv_stride_chunk; p.kv_st = (int32_t)kv_stride_tok; p.kv_sh = 0;
+  p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens; p.cu_q = nullptr;
+  p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
+  p.part_o = (float*)workspace;
+  p.part_lse = p.part_o + slots * Hq * head_dim_v;
+  p.seg_info = (int32_t*)(p.part_lse + slots * Hq);
+  p.k_scale = nullptr; p.v_scale = nullptr;
+  p.R = R; p.Hq = Hq; p.Hkv = groups; p.G = Hq < 16 ? Hq : 16; p.chunk = chunk_tokens;
+  p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
+  p.min_span_tiles = 256 / 16;
+  p.grid = grid_x;
+  p.scale_log2 = softmax_scale * 1.4426950408889634f;
+
+  const int wpb = mla_waves_per_block(groups);
+  hipStream_t st = (hipStream_t)stream;
+  hipEvent_t ev_a, ev_b;
+  const bool timed = mi_profile_next(&ev_a, &ev_b);
+  if (timed) (void)hipEventRecord(ev_a, st);
+  hipLaunchKernelGGL(paged_mla_decode_stream_kernel, dim3(grid_x, groups / wpb), dim3(64 * wpb),
+                     (size_t)R * 2 * sizeof(int32_t), st, p);
+  if (timed) (void)hipEventRecord(ev_b, st);
+  hipLaunchKernelGGL((paged_decode_merge_kernel<512>), dim3(Hq, R), dim3(512), 0, st, p);
+  return mi_check_launch("mi_paged_mla_decode_attention");
 }

@@ -267,6 +267,38 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
     return out
 
 
+def paged_mla_decode_attention(q: Tensor, kv_cache: Tensor, kv_lens: Tensor, block_table: Tensor, *,
+                               softmax_scale: float, head_dim_v: int = 512, max_kv_len: Optional[int] = None,
+                               out: Optional[Tensor] = None) -> Tensor:
+    """Absorbed multi-latent decode attention: ``q`` ``[R, (1,) Hq, 576]`` over the latent cache
+    ``[N, C, 576]`` (or ``[N, C, 1, 576]``); returns ``[R, (1,) Hq, head_dim_v]``."""
+    lib = _lib.load()
+    stream = _stream(q)
+    q3 = _qo_view(q, "q")
+    R, Hq, Dk = q3.shape
+    if kv_cache.dim() == 4:
+        _require(kv_cache.size(2) == 1, "the latent cache has one row per token")
+        kv_cache = kv_cache.squeeze(2)
+    _require(kv_cache.dim() == 3 and kv_cache.stride(2) == 1 and kv_cache.size(2) == Dk
+             and kv_cache.dtype == torch.bfloat16, "kv_cache must be bf16 [N, C, 576] with contiguous rows")
+    _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
+    _require(kv_lens.dtype == torch.int32 and kv_lens.is_contiguous() and kv_lens.numel() >= R, "bad kv_lens")
+    C = kv_cache.size(1)
+    if max_kv_len is None:
+        max_kv_len = block_table.size(1) * C
+    if out is None:
+        out = torch.empty(q.shape[:-1] + (head_dim_v,), dtype=q.dtype, device=q.device)
+    o3 = _qo_view(out, "out")
+    _require(tuple(o3.shape) == (R, Hq, head_dim_v), "out shape mismatch")
+    workspace = _workspace(q.device, lib.mi_mla_decode_workspace_bytes(R, Hq, head_dim_v))
+    _lib.check(lib.mi_paged_mla_decode_attention(
+        q3.data_ptr(), q3.stride(0), q3.stride(1), kv_cache.data_ptr(), kv_cache.stride(0), kv_cache.stride(1),
+        block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
+        _ptr(workspace), 0 if workspace is None else workspace.numel(), R, Hq, Dk, head_dim_v, C, int(max_kv_len),
+        float(softmax_scale), stream), "mi_paged_mla_decode_attention")
+    return out
+
+
 def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
                             block_table: Tensor, *, softmax_scale: Optional[float] = None,
                             max_kv_len: Optional[int] = None, out: Optional[Tensor] = None,

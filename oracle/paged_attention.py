@@ -81,6 +81,26 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
     return out
 
 
+def mla_decode_attention(q: Tensor, latent_cache: Tensor, kv_lens: Tensor, block_table: Tensor,
+                         softmax_scale: float, head_dim_v: int) -> Tensor:
+    """Absorbed multi-latent decode attention, the arithmetic flash_mla_with_kvcache is called for at
+    megatron/core/transformer/attention.py:561-587: ``q`` [R,Hq,dk]; ``latent_cache`` [N,C,dk] holds one
+    row per token shared by every head; scores over all dk values, output = weighted sum of the first
+    ``head_dim_v`` values of the rows.  fp32 [R,Hq,head_dim_v]."""
+    R, Hq, dk = q.shape
+    C = latent_cache.size(1)
+    out = torch.zeros(R, Hq, head_dim_v, dtype=torch.float32)
+    for r in range(R):
+        L = int(kv_lens[r])
+        if L <= 0:
+            continue
+        n = (L + C - 1) // C
+        rows = latent_cache[block_table[r, :n].long()].reshape(n * C, dk)[:L].float()
+        probs = torch.softmax(q[r].float() @ rows.T * softmax_scale, dim=-1)
+        out[r] = probs @ rows[:, :head_dim_v]
+    return out
+
+
 def paged_varlen_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
                            block_table: Tensor, softmax_scale: Optional[float] = None,
                            k_scales: Optional[Tensor] = None, v_scales: Optional[Tensor] = None) -> Tensor:

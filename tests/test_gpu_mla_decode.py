@@ -1,0 +1,78 @@
+"""GPU parity: absorbed multi-latent decode attention over the latent cache (through the C ABI),
+against the fp32 checker: 2e-2 abs/rel as for the other bf16 attention paths."""
+import pytest
+import torch
+
+from oracle import paged_attention as oa
+
+pytestmark = pytest.mark.gpu
+
+DK, DV = 576, 512
+
+
+def _case(mi, dev, lens, Hq, chunk, seed, pool_extra=3):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.tensor(lens, dtype=torch.int32)
+    bt, N = mi.synthetic.build_block_table(lens, chunk, g)
+    cache = (torch.randn(N + pool_extra, chunk, DK, generator=g) * 0.5).bfloat16()
+    q = torch.randn(lens.numel(), 1, Hq, DK, generator=g).bfloat16()
+    return q, cache, lens, bt
+
+
+def _check(mi, dev, q, cache, lens, bt, scale):
+    out = mi.ops.paged_mla_decode_attention(q.to(dev), cache.to(dev), lens.to(dev), bt.to(dev), softmax_scale=scale)
+    torch.cuda.synchronize()
+    ref = oa.mla_decode_attention(q.squeeze(1), cache, lens, bt, scale, DV)
+    got = out.float().cpu().squeeze(1)
+    assert got.shape == ref.shape and torch.isfinite(got).all()
+    err = (got - ref).abs()
+    assert (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
+    return out
+
+
+@pytest.mark.parametrize("Hq", [1, 8, 16, 32, 128])
+@pytest.mark.parametrize("chunk", [16, 64, 256])
+def test_mla_decode_matches_checker(mi, dev, Hq, chunk):
+    lens = [0, 1, 15, 16, 17, chunk - 1, chunk, chunk + 1, 3 * chunk + 5, 700, 0, 2049]
+    q, cache, lens, bt = _case(mi, dev, lens, Hq, chunk, seed=Hq + chunk)
+    out = _check(mi, dev, q, cache, lens, bt, scale=(128 + 64) ** -0.5)
+    assert (out.cpu()[lens == 0] == 0).all()
+
+
+def test_mla_decode_long_contexts_and_splits(mi, dev):
+    """Enough tokens that every request is cut over many workgroups and merged."""
+    q, cache, lens, bt = _case(mi, dev, [20000, 4097, 12345, 1], 16, 64, seed=9)
+    _check(mi, dev, q, cache, lens, bt, scale=0.07)
+    for grid in (3, 37):
+        mi.ops.set_tuning("decode_grid", grid)
+        try:
+            _check(mi, dev, q, cache, lens, bt, scale=0.07)
+        finally:
+            mi.ops.set_tuning("decode_grid", 0)
+
+
+def test_mla_decode_chunk_permutation_and_cache_view(mi, dev):
+    """Moving the rows to other physical chunks changes nothing; a [N, C, 1, 576] cache view is accepted."""
+    q, cache, lens, bt = _case(mi, dev, [100, 333, 64], 32, 64, seed=4)
+    a = mi.ops.paged_mla_decode_attention(q.to(dev), cache.to(dev), lens.to(dev), bt.to(dev), softmax_scale=0.1)
+    N = cache.size(0)
+    perm = torch.randperm(N, generator=torch.Generator().manual_seed(1))
+    moved = torch.empty_like(cache)
+    moved[perm] = cache
+    bt2 = torch.where(bt >= 0, perm[bt.clamp(min=0).long()].int(), bt)
+    b = mi.ops.paged_mla_decode_attention(q.to(dev), moved.unsqueeze(2).to(dev), lens.to(dev), bt2.to(dev),
+                                          softmax_scale=0.1)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_mla_decode_argument_errors(mi, dev):
+    q, cache, lens, bt = _case(mi, dev, [10, 20], 24, 16, seed=2)
+    with pytest.raises(mi._lib.KernelError, match="multiple of 16"):
+        mi.ops.paged_mla_decode_attention(q.to(dev), cache.to(dev), lens.to(dev), bt.to(dev), softmax_scale=0.1)
+    q, cache, lens, bt = _case(mi, dev, [10, 20], 16, 16, seed=2)
+    with pytest.raises(ValueError, match="576"):
+        mi.ops.paged_mla_decode_attention(q.to(dev)[..., :512].contiguous(), cache.to(dev), lens.to(dev), bt.to(dev),
+                                          softmax_scale=0.1)
+    with pytest.raises(mi._lib.KernelError, match="softmax_scale"):
+        mi.ops.paged_mla_decode_attention(q.to(dev), cache.to(dev), lens.to(dev), bt.to(dev), softmax_scale=0.0)

@@ -208,3 +208,31 @@ def test_fp8_append_policy_pins():
     big = torch.full((1, Hkv, d), 100.0).bfloat16()
     oa.kv_append_fp8(cache, scales, big, torch.tensor([3]), torch.tensor([0 + 1]), headroom=2.0)
     assert (cache[3, 1] == 0x7E).all()
+
+
+def test_mla_decode_checker_against_library_attention_and_brute_force():
+    """Latent-cache decode: scores over the whole shared row, values = its first dv columns.  Pinned by the
+    library's scaled_dot_product_attention (which takes a narrower value) and by fp64 loops."""
+    g = torch.Generator().manual_seed(31)
+    R, Hq, dk, dv, C = 3, 5, 24, 16, 8
+    lens = torch.tensor([13, 1, 0], dtype=torch.int32)
+    N = 6
+    cache = torch.randn(N, C, dk, generator=g)
+    bt = torch.tensor([[4, 1, -1], [2, -1, -1], [-1, -1, -1]], dtype=torch.int32)
+    q = torch.randn(R, Hq, dk, generator=g)
+    scale = 0.37
+    out = oa.mla_decode_attention(q, cache, lens, bt, scale, dv)
+    assert out.shape == (R, Hq, dv) and (out[2] == 0).all()
+    for r in range(2):
+        L = int(lens[r])
+        rows = torch.cat([cache[int(c)] for c in bt[r, : (L + C - 1) // C]])[:L]
+        want = F.scaled_dot_product_attention(q[r][None, :, None, :], rows[None, None].expand(1, Hq, L, dk),
+                                              rows[None, None, :, :dv].expand(1, Hq, L, dv), scale=scale)[0, :, 0]
+        assert torch.allclose(out[r], want, atol=1e-5)
+        for h in range(Hq):  # brute force
+            s = [sum(float(q[r, h, i]) * float(rows[j, i]) for i in range(dk)) * scale for j in range(L)]
+            m = max(s)
+            w = [math.exp(x - m) for x in s]
+            for e in (0, dv - 1):
+                ref = sum(w[j] * float(rows[j, e]) for j in range(L)) / sum(w)
+                assert abs(float(out[r, h, e]) - ref) < 1e-5
