@@ -76,8 +76,17 @@ static __device__ __forceinline__ int chunk_of(int tok, uint64_t magic) {
 // shared 576-wide row, the caller points both cache arguments at the same buffer).
 template <int HDK, int HDV, int NT, bool FP8>
 static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int row, int h, int len,
-                                                      int start, int end, bool whole, int slot, int lane) {
+                                                      int start, int end, bool whole, int slot, int lane,
+                                                      uint8_t* q_lds) {
   constexpr int KS = HDK / 32;
+  // Wide keys (the 576-wide latent rows): the query fragments would take 72 registers per lane next
+  // to 128 accumulator registers, so they live in this wavefront's piece of LDS instead (16 rows with
+  // a pitch that spreads the 16 rows of a fragment read over all banks).
+  constexpr bool Q_IN_LDS = HDK > 128;
+  // The latent rows are read twice (as keys, then their first part as values) and by every query
+  // group: those loads stay cacheable; an ordinary KV cache is read exactly once and streams past.
+  constexpr bool SHARED_KV = HDK != HDV;
+  constexpr int kQPitch = HDK * 2 + 16;
   constexpr int DV = HDV / 16;
   constexpr int VW = DV * (FP8 ? 1 : 2) / 16;  // 16-byte loads per token and lane of the value operand (0: 8 bytes)
   static_assert((HDK == 64 || HDK == 128 || HDK == 576) && (HDV == 64 || HDV == 128 || HDV == 512), "head widths");
@@ -100,16 +109,25 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   const int last = min(end, len) - 1;
 
   // Query fragments: B operand rows are the G heads of this KV head.
-  uint4 qf[KS];
+  uint4 qf[Q_IN_LDS ? 1 : KS];
+  const uint8_t* q_frag = q_lds + m16 * kQPitch + 16 * g;  // this lane's fragment of step kk: + 64 kk
   {
     const uint16_t* qrow = p.q + (int64_t)row * p.q_st + (int64_t)hq * p.q_sh;
+    if (Q_IN_LDS) {
 #pragma unroll
-    for (int kk = 0; kk < KS; ++kk) {
-      // bf16 cache: lane g owns d = 32kk + 8g .. +7.
-      // fp8 cache : K bytes are loaded 16 per lane, d = 64u + 16g + 8half .. +7
-      //             for mfma step kk = 2u + half.
-      const int d0 = FP8 ? (64 * (kk >> 1) + 16 * g + 8 * (kk & 1)) : (32 * kk + 8 * g);
-      qf[kk] = (m16 < G) ? ld16(qrow + d0) : make_uint4(0, 0, 0, 0);
+      for (int kk = 0; kk < KS; ++kk)
+        *reinterpret_cast<uint4*>(q_lds + m16 * kQPitch + 16 * g + 64 * kk) =
+            (m16 < G) ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
+      // (every lane reads back exactly what it wrote, so no cross-lane ordering is needed)
+    } else {
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) {
+        // bf16 cache: lane g owns d = 32kk + 8g .. +7.
+        // fp8 cache : K bytes are loaded 16 per lane, d = 64u + 16g + 8half .. +7
+        //             for mfma step kk = 2u + half.
+        const int d0 = FP8 ? (64 * (kk >> 1) + 16 * g + 8 * (kk & 1)) : (32 * kk + 8 * g);
+        qf[kk] = (m16 < G) ? ld16(qrow + d0) : make_uint4(0, 0, 0, 0);
+      }
     }
   }
 
@@ -215,7 +233,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       const uint32_t lim = (uint32_t)min(last - t0, 15) * tok_bytes;
       const uint8_t* krow = chunk + (uint32_t)(t0 - tok0) * tok_bytes + min(k_lane, lim + k_col);
 #pragma unroll
-      for (int kk = 0; kk < (FP8 ? KS / 2 : KS); ++kk) kf[u][kk] = ld16_stream(krow + 64 * kk);
+      for (int kk = 0; kk < (FP8 ? KS / 2 : KS); ++kk)
+        kf[u][kk] = SHARED_KV ? ld16(krow + 64 * kk) : ld16_stream(krow + 64 * kk);
     }
   };
   auto load_v = [&](int T) {
@@ -232,7 +251,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
         const uint8_t* vrow = tile + min(v_lane[j], cap);
         if (VW > 0) {
 #pragma unroll
-          for (int w = 0; w < VW; ++w) vf16[u][j][w] = ld16_stream(vrow + 16 * w);
+          for (int w = 0; w < VW; ++w) vf16[u][j][w] = SHARED_KV ? ld16(vrow + 16 * w) : ld16_stream(vrow + 16 * w);
         } else {
           vf8[u][j] = ld8_stream(vrow);
         }
@@ -269,7 +288,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
         }
       } else {
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32(kf[u][kk], qf[kk], sacc);
+        for (int kk = 0; kk < KS; ++kk)
+          sacc = mfma_16x16x32(kf[u][kk], Q_IN_LDS ? lds_ld16(q_frag + 64 * kk) : qf[Q_IN_LDS ? 0 : kk], sacc);
       }
       if (ragged) {
         const int tok0 = T + 16 * u + 4 * g;
@@ -426,6 +446,9 @@ static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p)
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x >> 6) + wave);
+  // wide keys: 16 query rows per wavefront behind the two integer arrays (see decode_segment)
+  uint8_t* const q_lds = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15) +
+                         (size_t)wave * 16 * (HDK * 2 + 16);
 
   // ---- prefix sum of tiles over the batch (wave 0), shared through LDS -------------
   if (wave == 0) {
@@ -484,7 +507,7 @@ static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p)
       int row;
       decode_row(p, r, row);
       decode_segment<HDK, HDV, NT, FP8>(p, r, row, h, len, tb * TK, min(te * TK, len), first && final,
-                                        (int)blockIdx.x + r, lane);
+                                        (int)blockIdx.x + r, lane, q_lds);
       t0 = rb + te;
     }
     ++r;
@@ -790,8 +813,17 @@ extern "C" int mi_paged_mla_decode_attention(
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
   if (timed) (void)hipEventRecord(ev_a, st);
-  hipLaunchKernelGGL(paged_mla_decode_stream_kernel, dim3(grid_x, groups / wpb), dim3(64 * wpb),
-                     (size_t)R * 2 * sizeof(int32_t), st, p);
+  const size_t lds = (((size_t)R * 2 * sizeof(int32_t) + 15) & ~(size_t)15) + (size_t)wpb * 16 * (576 * 2 + 16);
+  static bool lds_limit_raised[64] = {false};  // per device: more than the default 64 KB of dynamic LDS
+  int dev_id = 0;
+  if (hipGetDevice(&dev_id) != hipSuccess || dev_id < 0 || dev_id >= 64) dev_id = 0;
+  if (!lds_limit_raised[dev_id]) {
+    if (hipFuncSetAttribute((const void*)paged_mla_decode_stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            128 * 1024) != hipSuccess)
+      return mi_fail(MI_ERR_LAUNCH, "mi_paged_mla_decode_attention: cannot raise the dynamic LDS limit");
+    lds_limit_raised[dev_id] = true;
+  }
+  hipLaunchKernelGGL(paged_mla_decode_stream_kernel, dim3(grid_x, groups / wpb), dim3(64 * wpb), lds, st, p);
   if (timed) (void)hipEventRecord(ev_b, st);
   hipLaunchKernelGGL((paged_decode_merge_kernel<512>), dim3(Hq, R), dim3(512), 0, st, p);
   return mi_check_launch("mi_paged_mla_decode_attention");
