@@ -225,6 +225,26 @@ int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t 
                                    float softmax_scale, void* stream);
 
 /*
+ * Paged varlen causal attention with keys wider than values: the prefill / mixed step of
+ * multi-latent attention, where the reference decompresses the latent cache into a key cache
+ * `[n_chunks, chunk_tokens, H, 192]` (128 + the 64 shared rotary values) and a value cache
+ * `[.., H, 128]` (MLASelfAttention.uncompress_kv_from_cache,
+ * megatron/core/transformer/multi_latent_attention.py:801-825, called from
+ * attention.py:406-411) and hands them to flash_attn_varlen_func (attention.py:546-557).
+ * Same mask and padding rules as mi_paged_prefill_attention; each cache has its own strides
+ * (elements); q `[T, Hq, 192]`, out `[T, Hq, 128]`.  One kernel serves every request.
+ */
+int mi_paged_prefill_attention_mla(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
+                                   const void* k_cache, int64_t k_stride_chunk, int64_t k_stride_tok,
+                                   int64_t k_stride_head, const void* v_cache, int64_t v_stride_chunk,
+                                   int64_t v_stride_tok, int64_t v_stride_head,
+                                   const int32_t* block_table, int64_t bt_stride,
+                                   const int32_t* cu_seqlens_q, const int32_t* kv_lens, void* out,
+                                   int64_t o_stride_tok, int64_t o_stride_head, int32_t T, int32_t R,
+                                   int32_t Hq, int32_t Hkv, int32_t head_dim_k, int32_t head_dim_v,
+                                   int32_t chunk_tokens, float softmax_scale, void* stream);
+
+/*
  * Fused q/k head norm + rotary embedding (+ KV-append when k_cache is given).
  * Replaces, per layer, q_layernorm/k_layernorm
  * (megatron/core/transformer/attention.py:1026-1030), apply_rotary_emb_key /

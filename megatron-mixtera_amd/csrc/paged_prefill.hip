@@ -29,6 +29,8 @@ struct PrefillParams {
   const uint8_t* vc;
   int64_t kv_sc;
   int32_t kv_st, kv_sh;
+  int64_t v_sc;          // value cache strides (register-only kernel; equal to the key cache's otherwise)
+  int32_t v_st, v_sh;
   const int32_t* bt;
   int64_t bt_stride;
   const int32_t* cu_q;
@@ -44,10 +46,12 @@ struct PrefillParams {
 };
 
 // NQ = 16-row tiles per wave; a workgroup always covers 256 rows (16 / NQ waves).
-template <int HD, int NT, int NQ>
+// HDK = width of queries and keys, HDV = width of values and of the output (they differ for the
+// decompressed caches of multi-latent attention: 192 / 128); the value cache has its own strides.
+template <int HDK, int HDV, int NT, int NQ>
 __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillParams p) {
-  constexpr int KS = HD / 32;
-  constexpr int DV = HD / 16;
+  constexpr int KS = HDK / 32;
+  constexpr int DV = HDV / 16;
   constexpr int WAVES = 16 / NQ;
 
   const int lane = threadIdx.x & 63;
@@ -62,10 +66,10 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
   // workgroup of every KV head clears its heads of those rows.
   if (blockIdx.x == 0) {
     const int tq = p.cu_q[p.R];
-    const int per_row = G * HD;  // contiguous elements of this head group in one row
+    const int per_row = G * HDV;  // contiguous elements of this head group in one row
     for (int64_t i = (int64_t)threadIdx.x * 8; i < (int64_t)(p.T - tq) * per_row; i += 64 * WAVES * 8) {
       const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
-      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
+      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HDV) * p.o_sh + (e % HDV), make_uint4(0, 0, 0, 0));
     }
   }
 
@@ -107,9 +111,11 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
   const int ntiles = (nq * G + 15) >> 4;  // 16-row tiles that hold a valid row
 
   const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * 2;
-  const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * 2;
+  const uint8_t* vbase = p.vc + (int64_t)h * p.v_sh * 2;
   const int64_t chunk_bytes = p.kv_sc * 2;
   const int tok_bytes = p.kv_st * 2;
+  const int64_t v_chunk_bytes = p.v_sc * 2;
+  const int v_tok_bytes = p.v_st * 2;
 
   float m_run[NQ], l_run[NQ];
   f32x4_t acc[NQ][DV];
@@ -159,11 +165,11 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
       const int tu = min(T0, last);
       const int ci = (int)(((uint64_t)(uint32_t)tu * p.chunk_magic) >> 40);
       const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
-      const uint8_t* vc = vbase + (int64_t)pc * chunk_bytes;
+      const uint8_t* vc = vbase + (int64_t)pc * v_chunk_bytes;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint8_t* vrow = vc + (min(T0 + 4 * g + j, last) - ci * p.chunk) * tok_bytes + DV * m16 * 2;
-        if (HD == 128) vf16[u][j] = ld16(vrow);
+        const uint8_t* vrow = vc + (min(T0 + 4 * g + j, last) - ci * p.chunk) * v_tok_bytes + DV * m16 * 2;
+        if (HDV == 128) vf16[u][j] = ld16(vrow);
         else vf8[u][j] = ld8(vrow);
       }
     }
@@ -247,7 +253,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
     // Two 16-key sub-tiles are contracted by one mfma 16x16x32 (slots 0-3 = tokens 4g..4g+3 of
     // the first sub-tile, slots 4-7 = the same of the second; P is packed the same way).
     auto transpose_v = [&](int u, uint2 (&vt)[DV]) {
-      if constexpr (HD == 128) {
+      if constexpr (HDV == 128) {
         const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0]);
         const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1]);
         const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2]);
@@ -1040,6 +1046,7 @@ static int launch_paged_prefill(
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
   p.kc = (const uint8_t*)k_cache; p.vc = (const uint8_t*)v_cache;
   p.kv_sc = kv_stride_chunk; p.kv_st = (int32_t)kv_stride_tok; p.kv_sh = (int32_t)kv_stride_head;
+  p.v_sc = p.kv_sc; p.v_st = p.kv_st; p.v_sh = p.kv_sh;
   p.bt = block_table; p.bt_stride = bt_stride; p.cu_q = cu_seqlens_q; p.lens = kv_lens;
   p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
   p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G;
@@ -1086,8 +1093,8 @@ static int launch_paged_prefill(
   const int nt = mi_tuning().prefill_tile_subtiles == 1 ? 1 : 2;
 #define MI_LAUNCH_PREFILL(HD_, NT_)                                                                        \
   do {                                                                                                     \
-    if (nq == 4) hipLaunchKernelGGL((paged_prefill_kernel<HD_, NT_, 4>), grid, block, 0, st, p);           \
-    else hipLaunchKernelGGL((paged_prefill_kernel<HD_, NT_, 2>), grid, block, 0, st, p);                   \
+    if (nq == 4) hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, NT_, 4>), grid, block, 0, st, p);      \
+    else hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, NT_, 2>), grid, block, 0, st, p);              \
   } while (0)
   if (head_dim == 128) {
     if (nt == 1) MI_LAUNCH_PREFILL(128, 1);
@@ -1133,4 +1140,53 @@ extern "C" int mi_paged_prefill_attention_fp8(
                               kv_stride_tok, kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out,
                               o_stride_tok, o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim,
                               chunk_tokens, split_tokens, softmax_scale, MI_KV_FP8_E4M3, k_scales, v_scales, stream);
+}
+
+extern "C" int mi_paged_prefill_attention_mla(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache, int64_t k_stride_chunk,
+    int64_t k_stride_tok, int64_t k_stride_head, const void* v_cache, int64_t v_stride_chunk, int64_t v_stride_tok,
+    int64_t v_stride_head, const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seqlens_q,
+    const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head, int32_t T, int32_t R,
+    int32_t Hq, int32_t Hkv, int32_t head_dim_k, int32_t head_dim_v, int32_t chunk_tokens, float softmax_scale,
+    void* stream) {
+  if (T == 0 || R == 0) return MI_OK;
+  if (!q || !k_cache || !v_cache || !block_table || !cu_seqlens_q || !kv_lens || !out)
+    return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_mla: null pointer argument");
+  if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention_mla: need T, R >= 0 and Hq a multiple of Hkv");
+  const int G = Hq / Hkv;
+  if (G > 16 || (G & (G - 1)))
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: query heads per KV head must be 1, 2, 4, 8 or 16");
+  if (head_dim_k != 192 || head_dim_v != 128)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: key width 192 (128 + 64) and value width 128 only");
+  if (chunk_tokens <= 0 || chunk_tokens % 16)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention_mla: chunk size must be a positive multiple of 16");
+  if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention_mla: q/k/v/out must be 16-byte aligned");
+  if ((q_stride_tok | q_stride_head | o_stride_tok | o_stride_head | k_stride_chunk | k_stride_tok | k_stride_head |
+       v_stride_chunk | v_stride_tok | v_stride_head) % 8)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention_mla: strides must keep rows 16-byte aligned");
+  if (k_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31 || v_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31)
+    return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention_mla: one chunk must span less than 2 GiB");
+  if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention_mla: softmax_scale must be positive");
+
+  PrefillParams p;
+  p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
+  p.kc = (const uint8_t*)k_cache; p.vc = (const uint8_t*)v_cache;
+  p.kv_sc = k_stride_chunk; p.kv_st = (int32_t)k_stride_tok; p.kv_sh = (int32_t)k_stride_head;
+  p.v_sc = v_stride_chunk; p.v_st = (int32_t)v_stride_tok; p.v_sh = (int32_t)v_stride_head;
+  p.bt = block_table; p.bt_stride = bt_stride; p.cu_q = cu_seqlens_q; p.lens = kv_lens;
+  p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
+  p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G;
+  p.g_shift = 0;
+  while ((1 << p.g_shift) < G) ++p.g_shift;
+  p.chunk = chunk_tokens;
+  p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
+  p.scale_log2 = softmax_scale * 1.4426950408889634f;
+  p.skip_single = 0;  // one kernel serves every request, one-row requests included
+  p.k_scale = nullptr; p.v_scale = nullptr;
+  const int sbq = 256 / G;  // query tokens per workgroup (256 rows)
+  dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * 8);
+  hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2>), grid, block, 0, (hipStream_t)stream, p);
+  return mi_check_launch("mi_paged_prefill_attention_mla");
 }

@@ -299,6 +299,39 @@ def paged_mla_decode_attention(q: Tensor, kv_cache: Tensor, kv_lens: Tensor, blo
     return out
 
 
+def paged_prefill_attention_mla(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
+                                block_table: Tensor, *, softmax_scale: float, out: Optional[Tensor] = None) -> Tensor:
+    """Varlen causal attention over the decompressed caches of multi-latent attention: ``q`` ``[T, Hq, 192]``,
+    ``k_cache`` ``[N, C, H, 192]``, ``v_cache`` ``[N, C, H, 128]`` (each with its own strides) -> ``[T, Hq, 128]``."""
+    lib = _lib.load()
+    stream = _stream(q)
+    q3 = _qo_view(q, "q")
+    T, Hq, Dk = q3.shape
+    _require(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[:3] == v_cache.shape[:3],
+             "key / value caches must be [N, C, H, d] with equal leading dimensions")
+    _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16, "the caches must be bf16")
+    N, C, Hkv, _ = k_cache.shape
+    Dv = v_cache.size(3)
+    _require(k_cache.size(3) == Dk, "query and key widths differ")
+    ksc, kst, ksh = _cache_strides(k_cache)
+    vsc, vst, vsh = _cache_strides(v_cache)
+    _require(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.is_contiguous(), "cu_seqlens_q must be contiguous int32")
+    R = cu_seqlens_q.numel() - 1
+    _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
+    _require(kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "kv_lens must be contiguous int32")
+    _require(block_table.size(0) >= R and kv_lens.numel() >= R, "block_table / kv_lens shorter than the batch")
+    if out is None:
+        out = torch.empty(q.shape[:-1] + (Dv,), dtype=q.dtype, device=q.device)
+    o3 = _qo_view(out, "out")
+    _require(tuple(o3.shape) == (T, Hq, Dv), "out shape mismatch")
+    _lib.check(lib.mi_paged_prefill_attention_mla(
+        q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), ksc, kst, ksh, v_cache.data_ptr(), vsc, vst, vsh,
+        block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),
+        o3.data_ptr(), o3.stride(0), o3.stride(1), T, R, Hq, Hkv, Dk, Dv, C, float(softmax_scale), stream),
+        "mi_paged_prefill_attention_mla")
+    return out
+
+
 def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
                             block_table: Tensor, *, softmax_scale: Optional[float] = None,
                             max_kv_len: Optional[int] = None, out: Optional[Tensor] = None,

@@ -38,7 +38,8 @@ def gather_request_kv(cache: Tensor, block_table_row: Tensor, length: int) -> Te
 
 
 def attention_one_request(q: Tensor, k: Tensor, v: Tensor, scale: float, causal_shift: Optional[int]) -> Tensor:
-    """``q`` [Lq,Hq,d], ``k``/``v`` [Lk,Hkv,d] fp32 -> [Lq,Hq,d] fp32.
+    """``q`` [Lq,Hq,d], ``k`` [Lk,Hkv,d], ``v`` [Lk,Hkv,dv] fp32 -> [Lq,Hq,dv] fp32 (dv = d except for the
+    decompressed caches of multi-latent attention, whose keys are wider than their values).
 
     ``causal_shift`` = Lk - Lq for the bottom-right aligned mask (query i sees keys
     j <= i + shift); ``None`` disables masking.
@@ -47,7 +48,7 @@ def attention_one_request(q: Tensor, k: Tensor, v: Tensor, scale: float, causal_
     Lk, Hkv, _ = k.shape
     G = Hq // Hkv
     if Lk == 0:
-        return torch.zeros_like(q)
+        return torch.zeros(Lq, Hq, v.size(-1))
     # Query head h reads KV head h // G: the same pairing as repeating every KV head G times
     # (dot_product_attention.py:159-165), written without materialising the copies.
     qg = q.reshape(Lq, Hkv, G, d)
@@ -58,7 +59,7 @@ def attention_one_request(q: Tensor, k: Tensor, v: Tensor, scale: float, causal_
         scores = scores.masked_fill(kj > qi + causal_shift, float("-inf"))
     probs = torch.softmax(scores, dim=-1)
     probs = torch.nan_to_num(probs, nan=0.0)  # rows with no visible key
-    return torch.einsum("hgqk,khd->qhgd", probs, v).reshape(Lq, Hq, d)
+    return torch.einsum("hgqk,khd->qhgd", probs, v).reshape(Lq, Hq, v.size(-1))
 
 
 def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens: Tensor, block_table: Tensor,
@@ -111,7 +112,7 @@ def paged_varlen_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqle
         v_cache = dequantize_fp8(v_cache, v_scales)
     T, Hq, d = q.shape
     scale = d ** -0.5 if softmax_scale is None else softmax_scale
-    out = torch.zeros(T, Hq, d, dtype=torch.float32)
+    out = torch.zeros(T, Hq, v_cache.size(-1), dtype=torch.float32)
     for r in range(cu_seqlens_q.numel() - 1):
         a, b = int(cu_seqlens_q[r]), int(cu_seqlens_q[r + 1])
         L = int(kv_lens[r])
