@@ -75,6 +75,9 @@ int32_t mi_profile_collect(float* out_ms_host, int32_t capacity);
  * key/value: `[T, Hkv*d]` rows of `row_elems` contiguous elements, `src_stride_tok`
  * apart.  Pure copy: the cache receives the source bits.  Tokens that share a slot
  * (batch padding routed to the dummy chunk) race; any one of them wins.
+ * value == NULL and v_cache == NULL: only the key rows are written -- the latent cache of
+ * multi-latent attention, memory_buffer[layer, chunk_idx, local] = kv_concat
+ * (dynamic_context.py:533-538), `row_elems` = kv_lora_rank + qk_pos_emb_head_dim.
  */
 int mi_kv_append(const void* key, const void* value, int64_t src_stride_tok, void* k_cache,
                  void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok,

@@ -32,7 +32,12 @@ from .contexts import (  # noqa: F401
     TokenOverflowError,
     WarmupEngineMode,
 )
-from .flash_attn_interface import flash_attn_varlen_func, flash_attn_with_kvcache  # noqa: F401
+from .flash_attn_interface import (  # noqa: F401
+    flash_attn_varlen_func,
+    flash_attn_with_kvcache,
+    flash_mla_with_kvcache,
+    get_mla_metadata,
+)
 from .graphs import DecodeLayerGraphs  # noqa: F401
 
 __all__ = [
@@ -50,6 +55,8 @@ __all__ = [
     "ActiveRequestCountOverflowError",
     "flash_attn_with_kvcache",
     "flash_attn_varlen_func",
+    "flash_mla_with_kvcache",
+    "get_mla_metadata",
     "flash_decode_and_prefill",
     "adjust_key_value_for_inference",
     "PagedSelfAttentionCore",

@@ -13,7 +13,12 @@ from typing import Optional, Tuple
 import torch
 from torch import Tensor
 
-from .flash_attn_interface import flash_attn_varlen_func, flash_attn_with_kvcache
+from .flash_attn_interface import (
+    flash_attn_varlen_func,
+    flash_attn_with_kvcache,
+    flash_mla_with_kvcache,
+    get_mla_metadata,
+)
 
 
 def adjust_key_value_for_inference(inference_context, layer_number: int, query: Tensor, key: Tensor, value: Tensor,
@@ -34,12 +39,15 @@ def adjust_key_value_for_inference(inference_context, layer_number: int, query: 
 
 def flash_decode_and_prefill(q: Tensor, k: Tensor, v: Tensor, max_seqlen_q, max_seqlen_k, cu_seqlens_q,
                              cu_seqlens_k, seqlens_k, block_table, softmax_scale: Optional[float] = None, *,
-                             k_scales: Optional[Tensor] = None, v_scales: Optional[Tensor] = None) -> Tensor:
+                             k_scales: Optional[Tensor] = None, v_scales: Optional[Tensor] = None,
+                             mla_head_dim_v: Optional[int] = None) -> Tensor:
     """Same contract as ``Attention.flash_decode_and_prefill`` (attention.py:470-601).
 
     ``q`` is ``[T, 1, Hq, d]``; ``k`` / ``v`` are the paged caches.  ``max_seqlen_q == 1``
     selects the decode kernel, anything else the varlen causal kernel.  ``k_scales`` / ``v_scales``
-    (an addition) go with byte caches holding e4m3 values.
+    (an addition) go with byte caches holding e4m3 values.  ``mla_head_dim_v`` (the reference tests
+    ``isinstance(self.config, MLATransformerConfig)`` and reads ``config.kv_lora_rank`` instead) selects the
+    absorbed multi-latent decode: ``k`` is then the latent cache and ``v`` is ``None``.
     """
     if max_seqlen_q > 1:
         out = flash_attn_varlen_func(q.squeeze(1), k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
@@ -47,6 +55,11 @@ def flash_decode_and_prefill(q: Tensor, k: Tensor, v: Tensor, max_seqlen_q, max_
                                      causal=True, block_table=block_table, seqused_k=seqlens_k,
                                      k_scales=k_scales, v_scales=v_scales)
         return out.unsqueeze(1)
+    if mla_head_dim_v is not None:
+        metadata, num_splits = get_mla_metadata(seqlens_k, q.size(2), 1)
+        out, _ = flash_mla_with_kvcache(q, k.unsqueeze(-2), block_table, seqlens_k, mla_head_dim_v, metadata,
+                                        num_splits, softmax_scale=softmax_scale, causal=True)
+        return out
     return flash_attn_with_kvcache(q=q, k_cache=k, v_cache=v, cache_seqlens=seqlens_k, causal=True,
                                    block_table=block_table, softmax_scale=softmax_scale, max_seqlen_k=max_seqlen_k,
                                    k_scales=k_scales, v_scales=v_scales)

@@ -121,11 +121,16 @@ class DynamicInferenceContext:
         kv_cache_dtype: Optional[Union[str, torch.dtype]] = None,
         fp8_append_headroom: float = 2.0,
     ):
-        if cache_mla_latent:
-            raise NotImplementedError(
-                "the MLA latent cache (cache_mla_latent=True) is not part of the MI355X decode path")
         self.materialize_only_last_token_logits = materialize_only_last_token_logits
-        self.cache_mla_latent = False
+        self.cache_mla_latent = bool(cache_mla_latent)
+        if self.cache_mla_latent:
+            assert (
+                chunk_size_tokens == 64
+            ), "Flash MLA requires a block size of 64. Set --inference-dynamic-batching-chunk-size 64 to fix this assert"
+            if kv_lora_rank is None or qk_pos_emb_head_dim is None:
+                raise ValueError("cache_mla_latent=True needs kv_lora_rank and qk_pos_emb_head_dim")
+            if kv_cache_dtype not in (None, params_dtype):
+                raise NotImplementedError("the MLA latent cache is kept in params_dtype (no fp8 variant)")
         self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
 
         tp = 1 if tensor_model_parallel_size is None else tensor_model_parallel_size
@@ -148,7 +153,12 @@ class DynamicInferenceContext:
         # ---- sizing (reference: dynamic_context.py:186-242) ----
         self.chunk_size_tokens = chunk_size_tokens
         kv_itemsize = 1 if self.kv_cache_fp8 else params_dtype.itemsize
-        self.chunk_size_bytes = kv_itemsize * 2 * num_layers * chunk_size_tokens * heads_here * kv_channels
+        if self.cache_mla_latent:
+            # one vector c_t (rank) + the shared RoPE slice per token and layer (reference: :197-203)
+            self.kv_reduced_dim = kv_lora_rank + qk_pos_emb_head_dim
+            self.chunk_size_bytes = kv_itemsize * num_layers * chunk_size_tokens * self.kv_reduced_dim
+        else:
+            self.chunk_size_bytes = kv_itemsize * 2 * num_layers * chunk_size_tokens * heads_here * kv_channels
         if self.kv_cache_fp8:
             self.chunk_size_bytes += 4 * 2 * num_layers * heads_here  # its scales
         pool_bytes = int(buffer_size_gb * 1024**3)
@@ -210,7 +220,13 @@ class DynamicInferenceContext:
         self.token_to_local_position_within_kv_chunk = tok_row()
 
         # ---- the cache: [key|value, layer, chunk, token, head, channel] ----
-        if self.kv_cache_fp8:
+        if self.cache_mla_latent:
+            # [layer, chunk, token, rank + rope]: one row per token, shared by all heads (reference: :288-294)
+            self.memory_buffer = torch.full(
+                (num_layers, chunk_count_total, chunk_size_tokens, self.kv_reduced_dim),
+                -1, dtype=params_dtype, device=dev)
+            self.kv_scales = None
+        elif self.kv_cache_fp8:
             # bytes (0 = +0.0 in e4m3; the reference's -1 fill would read as NaN here) and their scales
             self.memory_buffer = torch.zeros(
                 (2, num_layers, chunk_count_total, chunk_size_tokens, heads_here, kv_channels),
@@ -345,8 +361,14 @@ class DynamicInferenceContext:
         ``layer_number`` is 1-based.  Slots come from ``token_to_chunk_idx`` /
         ``token_to_local_position_within_kv_chunk``; padded tokens land in the dummy chunk.
         """
-        assert key.size(1) == 1 and value.size(1) == 1
         n = self.padded_active_token_count
+        if self.cache_mla_latent:
+            # the caller passes kv_concat as the key; there is no value cache (reference: :533-538)
+            latent = key.squeeze(1) if key.dim() == 3 else key
+            ops.kv_append(latent[:n].unsqueeze(1), None, self.memory_buffer[layer_number - 1].unsqueeze(2), None,
+                          self.token_to_chunk_idx, self.token_to_local_position_within_kv_chunk)
+            return
+        assert key.size(1) == 1 and value.size(1) == 1
         if self.kv_cache_fp8:
             ops.kv_append_fp8(
                 key[:n], value[:n],
@@ -361,7 +383,10 @@ class DynamicInferenceContext:
             self.token_to_chunk_idx, self.token_to_local_position_within_kv_chunk)
 
     def key_value_cache(self, layer_number: int) -> Tuple[Tensor, Tensor, Tensor]:
-        """Views of the layer's key cache, value cache and this step's block table."""
+        """Views of the layer's key cache, value cache and this step's block table (latent cache: the
+        layer's ``[chunks, tokens, rank + rope]`` buffer and ``None``)."""
+        if self.cache_mla_latent:
+            return (self.memory_buffer[layer_number - 1], None, self.block_table)
         return (self.memory_buffer[0, layer_number - 1], self.memory_buffer[1, layer_number - 1], self.block_table)
 
     def key_value_scales(self, layer_number: int) -> Tuple[Optional[Tensor], Optional[Tensor]]:
@@ -413,6 +438,8 @@ class DynamicInferenceContext:
         (attention.py:1026-1030, 394-404, 766).  ``query`` is updated in place and returned.
         """
         n = self.padded_active_token_count
+        if self.cache_mla_latent:
+            raise NotImplementedError("the fused q/k norm + RoPE + append launch serves per-head KV caches, not MLA latents")
         if self.kv_cache_fp8:
             # norm + RoPE in one launch, then the quantising append (the roped key passes through memory)
             key_out = torch.empty_like(key[:n])
@@ -448,6 +475,8 @@ class DynamicInferenceContext:
         launch.  Returns the query ``[T, 1, Hq, d]`` (``query_out`` if given, else a new tensor).
         """
         n = self.padded_active_token_count
+        if self.cache_mla_latent:
+            raise NotImplementedError("the fused QKV launch serves per-head KV caches, not MLA latents")
         hkv = self.num_kv_heads_per_partition
         d = self.kv_channels
         if query_out is None:

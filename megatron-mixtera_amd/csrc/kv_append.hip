@@ -254,12 +254,13 @@ __global__ __launch_bounds__(256) void kv_append_fp8_rows_kernel(AppendFp8Params
   }
 }
 
+// n_tensors = 2: key and value; 1: the key alone (a cache with one row per token, e.g. MLA latents)
 template <bool DECODE>
-static int launch_append(AppendParams& p, hipStream_t st) {
+static int launch_append(AppendParams& p, hipStream_t st, int n_tensors = 2) {
   const uintptr_t bits = (uintptr_t)p.key | (uintptr_t)p.value | (uintptr_t)p.kc | (uintptr_t)p.vc |
                          (uintptr_t)p.src_stride | (uintptr_t)p.chunk_bytes | (uintptr_t)p.tok_bytes |
                          (uintptr_t)p.row_bytes;
-  dim3 grid(p.T, 2), block(256);
+  dim3 grid(p.T, n_tensors), block(256);
   if (!(bits & 15)) hipLaunchKernelGGL((kv_append_kernel<16, DECODE>), grid, block, 0, st, p);
   else if (!(bits & 3)) hipLaunchKernelGGL((kv_append_kernel<4, DECODE>), grid, block, 0, st, p);
   else if (!(bits & 1)) hipLaunchKernelGGL((kv_append_kernel<2, DECODE>), grid, block, 0, st, p);
@@ -277,8 +278,8 @@ extern "C" int mi_kv_append(const void* key, const void* value, int64_t src_stri
                             const int64_t* token_to_local_pos, int32_t T, int32_t row_elems,
                             int32_t elem_bytes, void* stream) {
   if (T == 0) return MI_OK;
-  if (!key || !value || !k_cache || !v_cache || !token_to_chunk_idx || !token_to_local_pos)
-    return mi_fail(MI_ERR_NULL, "mi_kv_append: null pointer argument");
+  if (!key || !k_cache || !token_to_chunk_idx || !token_to_local_pos || (value == nullptr) != (v_cache == nullptr))
+    return mi_fail(MI_ERR_NULL, "mi_kv_append: null pointer argument (value and v_cache go together)");
   if (T < 0 || row_elems <= 0 || elem_bytes <= 0 || src_stride_tok < row_elems || kv_stride_tok < row_elems)
     return mi_fail(MI_ERR_SHAPE, "mi_kv_append: bad sizes or strides");
   AppendParams p = {};
@@ -288,7 +289,7 @@ extern "C" int mi_kv_append(const void* key, const void* value, int64_t src_stri
   p.chunk_bytes = kv_stride_chunk * elem_bytes; p.tok_bytes = kv_stride_tok * elem_bytes;
   p.tok_chunk = token_to_chunk_idx; p.tok_local = token_to_local_pos;
   p.row_bytes = row_elems * elem_bytes; p.T = T; p.chunk = 1;
-  launch_append<false>(p, (hipStream_t)stream);
+  launch_append<false>(p, (hipStream_t)stream, value ? 2 : 1);
   return mi_check_launch("mi_kv_append");
 }
 

@@ -74,6 +74,35 @@ def flash_attn_varlen_func(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor
         kv_lens = (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).contiguous()
     else:
         raise ValueError("need cu_seqlens_k or seqused_k")
+    if k.size(-1) != v.size(-1):
+        # decompressed multi-latent caches: keys carry the shared rotary slice, values do not
+        if k_scales is not None or v_scales is not None:
+            raise NotImplementedError("no fp8 variant for caches with different key / value widths")
+        return ops.paged_prefill_attention_mla(
+            q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table,
+            softmax_scale=softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
     return ops.paged_prefill_attention(q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table,
                                        softmax_scale=softmax_scale, max_kv_len=max_seqlen_k,
                                        k_scales=k_scales, v_scales=v_scales)
+
+
+def get_mla_metadata(cache_seqlens: Tensor, num_heads_per_head_k: int, num_heads_k: int):
+    """Counterpart of ``flash_mla.get_mla_metadata`` (called at attention.py:571-575): the streaming
+    kernel splits the work on the GPU by itself, so there is no schedule to precompute."""
+    return None, None
+
+
+def flash_mla_with_kvcache(q: Tensor, k_cache: Tensor, block_table: Tensor, cache_seqlens: Tensor, head_dim_v: int,
+                           tile_scheduler_metadata=None, num_splits=None, softmax_scale: Optional[float] = None,
+                           causal: bool = False):
+    """Absorbed multi-latent decode attention with flash_mla's call shape (attention.py:576-587):
+    ``q`` ``[batch, 1, Hq, 576]``, ``k_cache`` ``[chunks, chunk_tokens, 1, 576]`` (the latent cache with a
+    head dimension added), ``cache_seqlens`` int32 ``[batch]`` counting this step's token.  Returns
+    ``(out [batch, 1, Hq, head_dim_v], None)``: the log-sum-exp the reference discards is not produced."""
+    if q.dim() != 4 or q.size(1) != 1:
+        raise NotImplementedError("flash_mla_with_kvcache on this path takes one query token per request: q [B,1,Hq,d]")
+    if softmax_scale is None:
+        softmax_scale = q.shape[-1] ** -0.5
+    out = ops.paged_mla_decode_attention(q, k_cache, cache_seqlens, block_table, softmax_scale=softmax_scale,
+                                         head_dim_v=head_dim_v)
+    return out, None

@@ -95,24 +95,28 @@ def _rows(x: Tensor, name: str) -> Tuple[Tensor, int, int]:
     return x, x.size(1) * x.size(2), x.stride(0)
 
 
-def kv_append(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor,
+def kv_append(key: Tensor, value: Optional[Tensor], k_cache: Tensor, v_cache: Optional[Tensor],
               token_to_chunk_idx: Tensor, token_to_local_pos: Tensor) -> None:
-    """``k_cache[chunk_idx[t], local[t]] = key[t]`` (and value): bit-exact scatter."""
+    """``k_cache[chunk_idx[t], local[t]] = key[t]`` (and value): bit-exact scatter.  ``value`` and
+    ``v_cache`` may both be ``None`` (a cache with one tensor, e.g. MLA latents ``[N, C, 1, r]``)."""
     lib = _lib.load()
     _stream(key)  # device check first: there is no CPU path
     key, row, k_st = _rows(key, "key")
-    value, row_v, v_st = _rows(value, "value")
     T = key.size(0)
-    _require(row == row_v and value.size(0) == T and k_st == v_st, "key/value shapes differ")
-    _require(key.dtype == k_cache.dtype == v_cache.dtype == value.dtype, "dtype mismatch between K/V and cache")
+    _require((value is None) == (v_cache is None), "value and v_cache go together")
     sc, st, sh = _cache_strides(k_cache)
-    _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
+    _require(key.dtype == k_cache.dtype, "dtype mismatch between K/V and cache")
+    if value is not None:
+        value, row_v, v_st = _rows(value, "value")
+        _require(row == row_v and value.size(0) == T and k_st == v_st, "key/value shapes differ")
+        _require(key.dtype == v_cache.dtype == value.dtype, "dtype mismatch between K/V and cache")
+        _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
     _require(sh == k_cache.size(3) and row == k_cache.size(2) * k_cache.size(3), "cache rows must be contiguous [Hkv, d]")
     _require(token_to_chunk_idx.dtype == torch.int64 and token_to_local_pos.dtype == torch.int64,
              "slot index tensors must be int64")
     _require(token_to_chunk_idx.numel() >= T and token_to_local_pos.numel() >= T, "slot index tensors too short")
     _require(token_to_chunk_idx.is_contiguous() and token_to_local_pos.is_contiguous(), "slot index tensors must be contiguous")
-    _lib.check(lib.mi_kv_append(key.data_ptr(), value.data_ptr(), k_st, k_cache.data_ptr(), v_cache.data_ptr(),
+    _lib.check(lib.mi_kv_append(key.data_ptr(), _ptr(value), k_st, k_cache.data_ptr(), _ptr(v_cache),
                                 sc, st, token_to_chunk_idx.data_ptr(), token_to_local_pos.data_ptr(),
                                 T, row, key.element_size(), _stream(key)), "mi_kv_append")
 

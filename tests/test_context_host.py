@@ -531,3 +531,28 @@ def test_fp8_cache_sizing_counts_bytes_and_scales(mi):
         Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=128, num_attention_heads=8,
             max_sequence_length=1024, buffer_size_gb=0.01, buffer_guaranteed_fraction=0.1, kv_cache_dtype="int4",
             device="cpu")
+
+
+def test_mla_latent_cache_sizing_and_views(mi):
+    """cache_mla_latent=True (dynamic_context.py:180-203,288-294,547-557): one row of
+    kv_lora_rank + qk_pos_emb_head_dim values per token and layer, no value cache, chunk size 64."""
+    Ctx = mi.DynamicInferenceContext
+    chunk_bytes = 2 * 3 * 64 * (512 + 64)  # bf16 x layers x tokens x (rank + rope) = 221 184
+    c = Ctx(params_dtype=torch.bfloat16, num_layers=3, kv_channels=128, num_attention_heads=16,
+            max_sequence_length=256, buffer_size_gb=10 * chunk_bytes / 1024**3, buffer_guaranteed_fraction=0.1,
+            chunk_size_tokens=64, cache_mla_latent=True, kv_lora_rank=512, qk_pos_emb_head_dim=64, device="cpu")
+    assert c.cache_mla_latent and c.kv_reduced_dim == 576
+    assert c.chunk_size_bytes == chunk_bytes == 221184
+    assert c.chunk_allocator.chunk_count_total == 10
+    assert c.memory_buffer.shape == (3, 10, 64, 576) and bool((c.memory_buffer == -1).all())
+    k, v, bt = c.key_value_cache(2)
+    assert v is None and k.shape == (10, 64, 576) and k.data_ptr() == c.memory_buffer[1].data_ptr()
+    assert c.key_value_scales(1) == (None, None)
+    with pytest.raises(AssertionError, match="block size of 64"):
+        Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=128, num_attention_heads=16,
+            max_sequence_length=256, buffer_size_gb=0.001, buffer_guaranteed_fraction=0.1, chunk_size_tokens=128,
+            cache_mla_latent=True, kv_lora_rank=512, qk_pos_emb_head_dim=64, device="cpu")
+    with pytest.raises(ValueError, match="kv_lora_rank"):
+        Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=128, num_attention_heads=16,
+            max_sequence_length=256, buffer_size_gb=0.001, buffer_guaranteed_fraction=0.1, chunk_size_tokens=64,
+            cache_mla_latent=True, device="cpu")
