@@ -53,7 +53,10 @@ const char* mi_last_error(void);
  * tile kernel, 2 = the same kernel with its wave groups in lock-step, 0 = older LDS kernel),
  * "prefill_tile_subtiles", "prefill_lds_row_tiles", "prefill_row_tiles" (the older kernels),
  * "norm_rope_vectorised" (16-byte-per-lane norm / rotary kernel: 1 = wherever alignment and the rotary
- * width allow it, 2 = the same but only from 256 tokens up (default), 0 = element-wise kernel always). */
+ * width allow it, 2 = the same but only from 256 tokens up (default), 0 = element-wise kernel always),
+ * "mla_decode_lds" (multi-latent decode: 1 = latent tiles shared through LDS by the wavefronts of a
+ * workgroup when the chunk size is a multiple of 64 and at most 768 requests are in the call (default),
+ * 0 = one streaming wavefront per 16-head group always). */
 int mi_set_tuning(const char* name, int32_t value);
 
 /*

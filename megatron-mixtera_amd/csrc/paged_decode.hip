@@ -436,19 +436,16 @@ static __device__ __forceinline__ bool decode_row(const DecodeParams& p, int r, 
   return p.cu_q[r + 1] - row == 1;
 }
 
-// The body of the streaming kernels: span of this workgroup, then its segments one after the other.
-template <int HDK, int HDV, int NT, bool FP8>
-static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p) {
-  constexpr int TK = 16 * NT;
-  extern __shared__ int cum[];  // inclusive prefix sum of tiles per request, [R], then the lengths, [R]
+// Span of this workgroup along the flattened sequence of TK-token tiles, then its segments one after
+// the other: seg(r, row, len, first token, one past the last token, whole request?, partial slot).
+// Every wavefront of the workgroup walks the same segments.  Dynamic LDS starts with the inclusive
+// prefix sums of tiles per request [R] and the request lengths [R].
+template <int TK, typename Seg>
+static __device__ __forceinline__ void walk_segments(const DecodeParams& p, Seg seg) {
+  extern __shared__ int cum[];
   int* const len_s = cum + p.R;
-
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x >> 6) + wave);
-  // wide keys: 16 query rows per wavefront behind the two integer arrays (see decode_segment)
-  uint8_t* const q_lds = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15) +
-                         (size_t)wave * 16 * (HDK * 2 + 16);
 
   // ---- prefix sum of tiles over the batch (wave 0), shared through LDS -------------
   if (wave == 0) {
@@ -506,12 +503,26 @@ static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p)
       }
       int row;
       decode_row(p, r, row);
-      decode_segment<HDK, HDV, NT, FP8>(p, r, row, h, len, tb * TK, min(te * TK, len), first && final,
-                                        (int)blockIdx.x + r, lane, q_lds);
+      seg(r, row, len, tb * TK, min(te * TK, len), first && final, (int)blockIdx.x + r);
       t0 = rb + te;
     }
     ++r;
   }
+}
+
+// The body of the register-streaming kernels: one wavefront per (virtual) KV head.
+template <int HDK, int HDV, int NT, bool FP8>
+static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p) {
+  extern __shared__ int cum[];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x >> 6) + wave);
+  // wide keys: 16 query rows per wavefront behind the two integer arrays (see decode_segment)
+  uint8_t* const q_lds = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15) +
+                         (size_t)wave * 16 * (HDK * 2 + 16);
+  walk_segments<16 * NT>(p, [&](int r, int row, int len, int start, int end, bool whole, int slot) {
+    decode_segment<HDK, HDV, NT, FP8>(p, r, row, h, len, start, end, whole, slot, lane, q_lds);
+  });
 }
 
 template <int HD, int NT, bool FP8, int MINW>
@@ -525,6 +536,195 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
 // workgroup.
 __global__ __launch_bounds__(256, 1) void paged_mla_decode_stream_kernel(DecodeParams p) {
   decode_stream_body<576, 512, 1, false>(p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Multi-latent attention decode with the latent tile shared through LDS.
+//
+// A workgroup of 8 wavefronts streams 64-token tiles of the latent rows (64 x 576 bf16 = 72 KB) into
+// LDS, double buffered, each row fetched from memory once per workgroup.  Wavefront w works for
+// query-head group w / PARTS (16 heads).  Scores: the PARTS wavefronts of a group share the work --
+// each takes one of the four 16-token sub-tiles (and, with PARTS = 8, one half of the 576 key
+// values), writes its raw partial scores to LDS, and after a barrier every wavefront reads the whole
+// 16 x 64 score tile back and runs the (cheap) softmax for itself.  Values: wavefront w owns output
+// columns part w % PARTS of the 512 and reads their fragments with transposing LDS reads.
+// PARTS = 8 serves one head group per workgroup (up to 16 heads per rank), PARTS = 4 two groups.
+// Two barriers per tile; the global loads of tile t+1 are in flight in registers while tile t computes.
+// ---------------------------------------------------------------------------------------------
+constexpr int kMlaTile = 64;                 // tokens per staged tile
+constexpr int kMlaPitch = 576 * 2 + 16;      // LDS bytes per staged row: 16 rows of a fragment read cover all banks
+
+template <int PARTS>
+__global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodeParams p) {
+  constexpr int HDK = 576, HDV = 512, KS = HDK / 32;
+  constexpr int NG = 8 / PARTS;               // head groups per workgroup
+  constexpr int DVW = HDV / PARTS / 16;       // 16-column output blocks per wavefront
+  constexpr int KH = PARTS / 4;               // wavefronts that share the key values of one sub-tile
+  constexpr int KSW = KS / KH;                // 32-value steps of the score product per wavefront
+  extern __shared__ int cum[];
+  uint8_t* const tiles = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m16 = lane & 15, g = lane >> 4;
+  const int group = blockIdx.y * NG + wave / PARTS;   // 16-head query group of this wavefront
+  const int c0 = (wave % PARTS) * (HDV / PARTS);      // its first output column
+  const int su = wave & 3;                            // sub-tile whose scores it computes
+  const int k0 = ((wave % PARTS) >> 2) * KSW;         // first 32-value step of its share of the keys
+  // partial scores of this wavefront's group: [key part][sub-tile][lane] float4, behind the two tile buffers
+  float4* const sbuf = reinterpret_cast<float4*>(tiles + 2 * kMlaTile * kMlaPitch) + (wave / PARTS) * (KH * 4 * 64);
+  const int G = p.G;
+  const int hq = group * G + m16;                     // query head of this lane's row (valid when m16 < G)
+  const int64_t chunk_bytes = p.kv_sc * 2;
+  const uint32_t tok_bytes = (uint32_t)(p.kv_st * 2);
+  // loader role: row tid / 8 of a tile, 16-byte pieces (tid % 8) + 8 i, i < 9, of that row
+  const int lrow = tid >> 3, lpiece = tid & 7;
+  const uint32_t l_src = (uint32_t)lrow * tok_bytes + 16u * lpiece;
+  uint8_t* const l_dst = tiles + lrow * kMlaPitch + 16 * lpiece;
+  // fragment reads: keys as the A operand of the scores, values transposed as the A operand of P.V
+  const int kfrag_off = m16 * kMlaPitch + 16 * g;
+  const int vfrag_off = (4 * g + (m16 >> 2)) * kMlaPitch + 2 * c0 + 8 * (m16 & 3);
+  const uint4 ones = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+
+  walk_segments<kMlaTile>(p, [&](int r, int row, int len, int start, int end, bool whole, int slot) {
+    r = __builtin_amdgcn_readfirstlane(r);
+    row = __builtin_amdgcn_readfirstlane(row);
+    len = __builtin_amdgcn_readfirstlane(len);
+    start = __builtin_amdgcn_readfirstlane(start);
+    end = __builtin_amdgcn_readfirstlane(end);
+    slot = __builtin_amdgcn_readfirstlane(slot);
+    const int last = min(end, len) - 1;
+    const int ntile = (end - start + kMlaTile - 1) / kMlaTile;
+    const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
+
+    uint4 qf[KSW];
+    {
+      const uint16_t* qrow = p.q + (int64_t)row * p.q_st + (int64_t)hq * p.q_sh + 32 * k0;
+#pragma unroll
+      for (int kk = 0; kk < KSW; ++kk) qf[kk] = (m16 < G) ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
+    }
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4_t acc[DVW];
+#pragma unroll
+    for (int e = 0; e < DVW; ++e) acc[e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    // A tile lies in one chunk (the launcher requires a chunk size that is a multiple of 64); rows past
+    // the segment's last token re-read that token's row (their probabilities are forced to zero).
+    uint4 stage[9];
+    auto fetch = [&](int t) {
+      const int T = start + t * kMlaTile;
+      const int ci = chunk_of(T, p.chunk_magic);
+      const int pc = __builtin_amdgcn_readfirstlane(bt_row[ci]);
+      const uint8_t* src = p.kc + (int64_t)pc * chunk_bytes + (int64_t)(uint32_t)(T - ci * p.chunk) * tok_bytes;
+      const uint32_t lim = (uint32_t)min(last - T, kMlaTile - 1) * tok_bytes + 16u * lpiece;
+      const uint8_t* rowp = src + min(l_src, lim);
+#pragma unroll
+      for (int i = 0; i < 9; ++i) stage[i] = ld16(rowp + 128 * i);
+    };
+    auto store = [&](int t) {
+      uint8_t* dst = l_dst + (t & 1) * (kMlaTile * kMlaPitch);
+#pragma unroll
+      for (int i = 0; i < 9; ++i) *reinterpret_cast<uint4*>(dst + 128 * i) = stage[i];
+    };
+
+    fetch(0);
+    store(0);
+    __syncthreads();
+    for (int t = 0; t < ntile; ++t) {
+      if (t + 1 < ntile) fetch(t + 1);  // workgroup-uniform
+      const uint8_t* buf = tiles + (t & 1) * (kMlaTile * kMlaPitch);
+      const int T = start + t * kMlaTile;
+      // ---- S^T = K Q^T: this wavefront's share, then the whole tile through LDS -----------
+      {
+        const uint8_t* ks = buf + kfrag_off + 16 * su * kMlaPitch + 64 * k0;
+        f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KSW; ++kk) sacc = mfma_16x16x32(lds_ld16(ks + 64 * kk), qf[kk], sacc);
+        sbuf[((k0 ? 1 : 0) * 4 + su) * 64 + lane] = make_float4(sacc[0], sacc[1], sacc[2], sacc[3]);
+      }
+      __syncthreads();
+      f32x4_t sc[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        float4 a = sbuf[u * 64 + lane];
+        if (KH == 2) {
+          const float4 b = sbuf[(4 + u) * 64 + lane];
+          a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w;
+        }
+        sc[u] = f32x4_t{a.x, a.y, a.z, a.w};
+      }
+      if (T + kMlaTile > end) {  // only the last tile of a segment has masked tokens
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int tok0 = T + 16 * u + 4 * g;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (tok0 + i >= end) sc[u][i] = -INFINITY;
+        }
+      }
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) tmax = fmaxf(fmaxf(tmax, sc[u][0]), fmaxf(sc[u][1], fmaxf(sc[u][2], sc[u][3])));
+      tmax = rowgroup_max(tmax);
+      // ---- online softmax (row = m16) ----------------------------------------------------
+      const float mul = p.scale_log2;
+      const float m_new = fmaxf(m_run, tmax * mul);
+      const float alpha = fast_exp2(m_run - m_new);
+      m_run = m_new;
+      uint2 pf[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float p0 = fast_exp2(__builtin_fmaf(sc[u][0], mul, -m_new));
+        const float p1 = fast_exp2(__builtin_fmaf(sc[u][1], mul, -m_new));
+        const float p2 = fast_exp2(__builtin_fmaf(sc[u][2], mul, -m_new));
+        const float p3 = fast_exp2(__builtin_fmaf(sc[u][3], mul, -m_new));
+        pf[u] = make_uint2(pack_bf16x2(p0, p1), pack_bf16x2(p2, p3));
+      }
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+        for (int e = 0; e < DVW; ++e) {
+          acc[e][0] *= alpha; acc[e][1] *= alpha; acc[e][2] *= alpha; acc[e][3] *= alpha;
+        }
+      }
+      // ---- O^T += V^T P^T, 32 tokens per product; row sums from an all-ones A operand -----
+      f32x4_t psum4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const uint4 pp = make_uint4(pf[2 * s2].x, pf[2 * s2].y, pf[2 * s2 + 1].x, pf[2 * s2 + 1].y);
+        const uint8_t* vs = buf + vfrag_off + 32 * s2 * kMlaPitch;
+#pragma unroll
+        for (int e = 0; e < DVW; ++e) {
+          const uint2 a0 = lds_ld8_tr(vs + 32 * e), a1 = lds_ld8_tr(vs + 16 * kMlaPitch + 32 * e);
+          acc[e] = mfma_16x16x32(make_uint4(a0.x, a0.y, a1.x, a1.y), pp, acc[e]);
+        }
+        psum4 = mfma_16x16x32(ones, pp, psum4);
+      }
+      l_run = l_run * alpha + psum4[0];
+      if (t + 1 < ntile) store(t + 1);
+      __syncthreads();
+    }
+
+    // ---- epilogue: acc[e][i] is output column c0 + 16 e + 4 g + i of row m16 ------------------
+    const float inv = 1.f / l_run;
+    if (m16 < G) {
+      if (whole) {
+        uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + c0 + 4 * g;
+#pragma unroll
+        for (int e = 0; e < DVW; ++e)
+          st8(o + 16 * e, make_uint2(pack_bf16x2(acc[e][0] * inv, acc[e][1] * inv),
+                                     pack_bf16x2(acc[e][2] * inv, acc[e][3] * inv)));
+      } else {
+        const int64_t prow = (int64_t)slot * p.Hq + hq;
+        float* o = p.part_o + prow * HDV + c0 + 4 * g;
+#pragma unroll
+        for (int e = 0; e < DVW; ++e)
+          *reinterpret_cast<float4*>(o + 16 * e) =
+              make_float4(acc[e][0] * inv, acc[e][1] * inv, acc[e][2] * inv, acc[e][3] * inv);
+        if (g == 0 && c0 == 0) p.part_lse[prow] = m_run + fast_log2(l_run);
+      }
+    }
+  });
 }
 
 // One workgroup per (request, query head): merge the partials of the workgroups that
@@ -752,6 +952,7 @@ static int mla_groups(int Hq) { return Hq <= 16 ? 1 : Hq / 16; }
 
 extern "C" int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v) {
   if (R <= 0 || Hq <= 0 || head_dim_v <= 0) return 0;
+  // (the per-wavefront kernel uses the larger grid of the two: enough for either)
   const int64_t slots = (int64_t)mla_grid_size(mla_groups(Hq)) + R;
   return slots * Hq * (head_dim_v + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
@@ -784,7 +985,18 @@ extern "C" int mi_paged_mla_decode_attention(
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: batch too large for the in-LDS prefix sum (7680 requests)");
 
   const int groups = mla_groups(Hq);
-  const int grid_x = mla_grid_size(groups);
+  // Two kernels: the latent tile shared through LDS by the eight wavefronts of a workgroup (needs tiles
+  // of 64 tokens that do not straddle chunks), or one wavefront per head group streaming on its own.
+  const size_t lds_head = ((size_t)R * 2 * sizeof(int32_t) + 15) & ~(size_t)15;
+  const size_t lds_shared = lds_head + (size_t)2 * kMlaTile * kMlaPitch + 8 * 1024;  // tiles + partial scores
+  const bool shared_tile = chunk_tokens % kMlaTile == 0 && mi_tuning().mla_decode_lds != 0 && lds_shared <= 160 * 1024;
+  const int parts = (groups % 2 == 0) ? 4 : 8;            // output-column parts per head group
+  const int wg_y = shared_tile ? groups / (8 / parts) : 0;  // workgroups per span (shared-tile kernel)
+  int grid_x = mla_grid_size(groups);
+  if (shared_tile && mi_tuning().decode_grid <= 0) {
+    grid_x = device_cu_count() / wg_y;
+    if (grid_x < 1) grid_x = 1;
+  }
   const int64_t slots = (int64_t)grid_x + R;
   const int64_t need = slots * Hq * (head_dim_v + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
   if (!workspace || workspace_bytes < need)
@@ -804,26 +1016,35 @@ extern "C" int mi_paged_mla_decode_attention(
   p.k_scale = nullptr; p.v_scale = nullptr;
   p.R = R; p.Hq = Hq; p.Hkv = groups; p.G = Hq < 16 ? Hq : 16; p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
-  p.min_span_tiles = 256 / 16;
+  p.min_span_tiles = shared_tile ? 256 / kMlaTile : 256 / 16;
   p.grid = grid_x;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
 
-  const int wpb = mla_waves_per_block(groups);
   hipStream_t st = (hipStream_t)stream;
-  hipEvent_t ev_a, ev_b;
-  const bool timed = mi_profile_next(&ev_a, &ev_b);
-  if (timed) (void)hipEventRecord(ev_a, st);
-  const size_t lds = (((size_t)R * 2 * sizeof(int32_t) + 15) & ~(size_t)15) + (size_t)wpb * 16 * (576 * 2 + 16);
+  const int wpb = mla_waves_per_block(groups);
+  const size_t lds = shared_tile ? lds_shared : lds_head + (size_t)wpb * 16 * (576 * 2 + 16);
+  if (lds > 160 * 1024)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: batch too large for the LDS of one workgroup");
   static bool lds_limit_raised[64] = {false};  // per device: more than the default 64 KB of dynamic LDS
   int dev_id = 0;
   if (hipGetDevice(&dev_id) != hipSuccess || dev_id < 0 || dev_id >= 64) dev_id = 0;
   if (!lds_limit_raised[dev_id]) {
-    if (hipFuncSetAttribute((const void*)paged_mla_decode_stream_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                            128 * 1024) != hipSuccess)
+    const hipFuncAttribute attr = hipFuncAttributeMaxDynamicSharedMemorySize;
+    if (hipFuncSetAttribute((const void*)paged_mla_decode_stream_kernel, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<4>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8>, attr, 160 * 1024) != hipSuccess)
       return mi_fail(MI_ERR_LAUNCH, "mi_paged_mla_decode_attention: cannot raise the dynamic LDS limit");
     lds_limit_raised[dev_id] = true;
   }
-  hipLaunchKernelGGL(paged_mla_decode_stream_kernel, dim3(grid_x, groups / wpb), dim3(64 * wpb), lds, st, p);
+  hipEvent_t ev_a, ev_b;
+  const bool timed = mi_profile_next(&ev_a, &ev_b);
+  if (timed) (void)hipEventRecord(ev_a, st);
+  if (shared_tile && parts == 4)
+    hipLaunchKernelGGL(paged_mla_decode_lds_kernel<4>, dim3(grid_x, wg_y), dim3(512), lds, st, p);
+  else if (shared_tile)
+    hipLaunchKernelGGL(paged_mla_decode_lds_kernel<8>, dim3(grid_x, wg_y), dim3(512), lds, st, p);
+  else
+    hipLaunchKernelGGL(paged_mla_decode_stream_kernel, dim3(grid_x, groups / wpb), dim3(64 * wpb), lds, st, p);
   if (timed) (void)hipEventRecord(ev_b, st);
   hipLaunchKernelGGL((paged_decode_merge_kernel<512>), dim3(Hq, R), dim3(512), 0, st, p);
   return mi_check_launch("mi_paged_mla_decode_attention");

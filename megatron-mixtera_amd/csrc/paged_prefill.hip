@@ -597,26 +597,6 @@ constexpr int kKPitch = 288;  // bytes per staged K row: measured conflict-free 
 constexpr int kVPitch = 288;  // bytes per staged V row: 16 rows x 32 B tile the banks twice
 constexpr int kPPTile = 64;   // keys per staged tile
 
-typedef short s16x4v __attribute__((ext_vector_type(4)));
-
-// Transposing LDS read: within each block of 16 lanes, lane i supplies the address of 4 bf16
-// (row i/4, columns 4*(i%4)..+3 of a 4 x 16 matrix) and lane L receives column L of that matrix.
-static __device__ __forceinline__ uint2 lds_ld8_tr(const uint8_t* ptr) {
-  const s16x4v v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-      (__attribute__((address_space(3))) s16x4v*)(uintptr_t)(uint32_t)(uintptr_t)ptr);
-  return __builtin_bit_cast(uint2, v);
-}
-
-// max over the four lanes {l, l^16, l^32, l^48} with two lane-swap instructions
-static __device__ __forceinline__ float rowgroup_max(float x) {
-  const uint32_t u = __float_as_uint(x);
-  const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
-  const uint32_t w = __float_as_uint(y);
-  const auto b = __builtin_amdgcn_permlane32_swap(w, w, false, false);
-  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
-}
-
 // FP8: the cache holds e4m3 bytes with one fp32 scale per (chunk, KV head); a piece is multiplied by
 // its chunk's scale and rounded to bf16 on its way into LDS, so both matrix phases are the bf16 ones.
 template <bool STAGGER, bool FP8>

@@ -30,18 +30,30 @@ def _check(mi, dev, q, cache, lens, bt, scale):
     return out
 
 
-@pytest.mark.parametrize("Hq", [1, 8, 16, 32, 128])
+@pytest.fixture(params=[1, 0], ids=["lds_tile", "streaming"])
+def kernel_choice(request, mi):
+    """Both decode kernels: latent tiles shared through LDS (chunk sizes that are multiples of 64 only;
+    other sizes stream either way) and one streaming wavefront per head group."""
+    mi.ops.set_tuning("mla_decode_lds", request.param)
+    yield request.param
+    mi.ops.set_tuning("mla_decode_lds", 1)
+
+
+@pytest.mark.parametrize("Hq", [1, 8, 16, 32, 48, 128])
 @pytest.mark.parametrize("chunk", [16, 64, 256])
-def test_mla_decode_matches_checker(mi, dev, Hq, chunk):
+def test_mla_decode_matches_checker(mi, dev, Hq, chunk, kernel_choice):
+    if chunk == 16 and kernel_choice == 0:
+        pytest.skip("chunk 16 always streams")
     lens = [0, 1, 15, 16, 17, chunk - 1, chunk, chunk + 1, 3 * chunk + 5, 700, 0, 2049]
     q, cache, lens, bt = _case(mi, dev, lens, Hq, chunk, seed=Hq + chunk)
     out = _check(mi, dev, q, cache, lens, bt, scale=(128 + 64) ** -0.5)
     assert (out.cpu()[lens == 0] == 0).all()
 
 
-def test_mla_decode_long_contexts_and_splits(mi, dev):
+@pytest.mark.parametrize("Hq", [16, 64])
+def test_mla_decode_long_contexts_and_splits(mi, dev, Hq, kernel_choice):
     """Enough tokens that every request is cut over many workgroups and merged."""
-    q, cache, lens, bt = _case(mi, dev, [20000, 4097, 12345, 1], 16, 64, seed=9)
+    q, cache, lens, bt = _case(mi, dev, [20000, 4097, 12345, 1], Hq, 64, seed=9)
     _check(mi, dev, q, cache, lens, bt, scale=0.07)
     for grid in (3, 37):
         mi.ops.set_tuning("decode_grid", grid)
@@ -49,6 +61,14 @@ def test_mla_decode_long_contexts_and_splits(mi, dev):
             _check(mi, dev, q, cache, lens, bt, scale=0.07)
         finally:
             mi.ops.set_tuning("decode_grid", 0)
+
+
+def test_mla_decode_many_requests_fall_back_to_streaming(mi, dev):
+    """More requests than the LDS-tile kernel has room for next to its tiles: the call still succeeds."""
+    g = torch.Generator().manual_seed(12)
+    lens = torch.randint(0, 200, (1000,), generator=g).tolist()
+    q, cache, lens, bt = _case(mi, dev, lens, 16, 64, seed=13)
+    _check(mi, dev, q, cache, lens, bt, scale=0.07)
 
 
 def test_mla_decode_chunk_permutation_and_cache_view(mi, dev):
