@@ -364,9 +364,20 @@ int mi_last_token_gather(const void* src, int64_t src_stride_row, void* dst, int
                          int32_t elem_bytes, void* stream);
 
 /*
+ * The arithmetic of DynamicInferenceContext.calculate_log_probs (dynamic_context.py:1300-1365):
+ *   log_probs[t] = log_softmax(float(logits[t, :]))[token_ids[t]],  t < T
+ * without materialising the `[T, vocab]` fp32 log-softmax matrix: one read of each row.  logits
+ * `[T, vocab]` fp32 (0) or bf16 (1), row stride in elements; token_ids int64 `[T]` (the caller builds
+ * them as the reference does: the prompt token that follows each position, the newly sampled token at
+ * the last position of each request); an id outside [0, vocab) yields NaN.  fp32 results.
+ */
+int mi_selected_log_probs(const void* logits, int64_t stride_row, int32_t logits_dtype, int32_t T,
+                          int32_t vocab, const int64_t* token_ids, float* log_probs, void* stream);
+
+/*
  * TextGenerationController.sample_from_logits and the finished-request test that follows it
  * (megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315,
- * 503-512) as one launch, one workgroup per row of `logits` `[R, vocab]` (logits_dtype 0 = fp32,
+ * 519-530) as one launch, one workgroup per row of `logits` `[R, vocab]` (logits_dtype 0 = fp32,
  * 1 = bf16; row stride in elements):
  *   top_k == 1             : samples[r] = argmax (lowest index among equal maxima);
  *   otherwise              : x = logits * (1 / temperature) (rounded to bf16 for bf16 logits, as the

@@ -60,6 +60,7 @@ SIGNATURES = {
     "mi_decode_attention_state": (
         c_int, [_P, _P, _P, _I64, _I32, _P, _P, _P, _I64, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P]),
     "mi_last_token_gather": (c_int, [_P, _I64, _P, _I64, _P, _I32, _I32, _I32, _P]),
+    "mi_selected_log_probs": (c_int, [_P, _I64, _I32, _I32, _I32, _P, _P, _P]),
     "mi_sample_from_logits": (
         c_int, [_P, _I64, _I32, _I32, _I32, _I32, _F, _F, _P, _I32, _P, _P, _P, _P, _P, _I64, _P, _P]),
     "mi_norm_rope_append": (

@@ -865,15 +865,20 @@ class DynamicInferenceContext:
         Reference: dynamic_context.py:1300-1365.  For prefill rows the chosen token of position
         p is the prompt token at p+1; the last position of each request takes ``new_tokens``.
         """
-        log_probs = F.log_softmax(logits.squeeze(0).float(), dim=-1)
+        rows = logits.squeeze(0)
+        if rows.is_cuda:
+            # one read of every row, no [T, V] fp32 intermediate
+            def pick(ids):
+                return ops.selected_log_probs(rows[: ids.numel()], ids.to(torch.int64).contiguous())
+        else:
+            def pick(ids):
+                log_probs = F.log_softmax(rows.float(), dim=-1)
+                return log_probs[torch.arange(ids.numel(), device=rows.device), ids]
         if only_last_token_logits or self.is_decode_only():
-            idx = torch.arange(len(new_tokens), dtype=torch.int32, device=logits.device)
-            picked = log_probs[idx, new_tokens]
-            return [[lp] for lp in picked.flatten().tolist()]
+            return [[lp] for lp in pick(new_tokens).flatten().tolist()]
 
         chosen = self.token_to_input_ids[: self.active_token_count].roll(-1, 0)
         q_lens = self.request_query_lengths[self._active()]
         chosen[q_lens.cumsum(0) - 1] = new_tokens
-        idx = torch.arange(self.active_token_count, device=log_probs.device)
-        picked = log_probs[idx, chosen]
+        picked = pick(chosen)
         return [lp.tolist() for lp in picked.cpu().split(q_lens.tolist(), dim=0)]

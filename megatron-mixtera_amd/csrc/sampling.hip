@@ -2,7 +2,7 @@
 //
 // What the reference does with torch ops after the forward pass
 // (megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315,
-// 503-530 and megatron/core/inference/contexts/dynamic_context.py:890-918):
+// 519-530 and megatron/core/inference/contexts/dynamic_context.py:890-918):
 //   * last_token_logits: rows  cumsum(request_query_lengths) - 1  of the `[T, V]` logits;
 //   * sample_from_logits: argmax (top_k == 1), or  logits / temperature -> top-k filter (keep
 //     values >= the k-th largest) or top-p filter (sort descending, keep the shortest prefix
@@ -475,6 +475,91 @@ __global__ __launch_bounds__(256) void last_token_gather_kernel(GatherParams p) 
   }
 }
 
+struct LogProbParams {
+  const void* logits; int64_t stride; int32_t T, V;
+  const int64_t* token_ids; float* out;
+};
+
+constexpr int kLogProbThreads = 512;
+
+// out[t] = log_softmax(logits[t])[token_ids[t]] in fp32: one pass over the row with a running
+// (maximum, sum of exp(x - maximum)) pair per thread, merged over the workgroup.  One workgroup per row.
+template <bool BF16, int VEC>
+__global__ __launch_bounds__(kLogProbThreads) void selected_log_probs_kernel(LogProbParams p) {
+  __shared__ float red_m[kLogProbThreads / 64], red_s[kLogProbThreads / 64];
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  RowReader<BF16, VEC> rd;
+  rd.row = reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)t * p.stride * (BF16 ? 2 : 4);
+  rd.V = p.V; rd.inv_t = 1.f; rd.scale = false;
+  constexpr float kLog2e = 1.4426950408889634f;
+  // a finite start keeps exp(-inf - m) = 0 for masked (-inf) logits
+  float m = -3.0e38f, sum = 0.f;
+  // Whole batches of U 16-byte groups per thread: the batch maximum first (one three-way maximum per
+  // two elements), a rescale only when it raises the running maximum (rare after a thread's first
+  // batches), then one fused multiply-add, one exp2 and one add per element.
+  constexpr int U = 4;
+  const int stride = kLogProbThreads * VEC;
+  const int row_end = p.V - (p.V % VEC);
+  int base = 0;
+  if (VEC > 1) {
+    for (; base + U * stride <= row_end; base += U * stride) {
+      float x[U * VEC];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint4 w = ld16(rd.row + (int64_t)(base + u * stride + tid * VEC) * (BF16 ? 2 : 4));
+        const uint32_t q[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < VEC; ++j)
+          x[u * VEC + j] = BF16 ? ((j & 1) ? bf16hi_to_f32(q[(j >> 1) & 3]) : bf16lo_to_f32(q[(j >> 1) & 3]))
+                                : __uint_as_float(q[j & 3]);
+      }
+      float bm = x[0];
+#pragma unroll
+      for (int j = 1; j + 1 < U * VEC; j += 2) bm = fmaxf(fmaxf(bm, x[j]), x[j + 1]);
+      bm = fmaxf(bm, x[U * VEC - 1]);
+      if (bm > m) {
+        sum *= fast_exp2((m - bm) * kLog2e);
+        m = bm;
+      }
+      const float nm = -m * kLog2e;
+      float part = 0.f;
+#pragma unroll
+      for (int j = 0; j < U * VEC; ++j) part += fast_exp2(__builtin_fmaf(x[j], kLog2e, nm));
+      sum += part;
+    }
+  }
+  sweep<U>(rd, base, p.V, tid, kLogProbThreads, [&](int, float x, bool valid) {
+    if (valid) {
+      if (x > m) {
+        sum *= fast_exp2((m - x) * kLog2e);
+        m = x;
+      }
+      sum += fast_exp2((x - m) * kLog2e);
+    }
+  });
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    const float m2 = __shfl_xor(m, d, 64), s2 = __shfl_xor(sum, d, 64);
+    const float mm = fmaxf(m, m2);
+    sum = sum * fast_exp2((m - mm) * kLog2e) + s2 * fast_exp2((m2 - mm) * kLog2e);
+    m = mm;
+  }
+  if (lane == 0) { red_m[wave] = m; red_s[wave] = sum; }
+  __syncthreads();
+  if (tid == 0) {
+    float mm = red_m[0];
+#pragma unroll
+    for (int w = 1; w < kLogProbThreads / 64; ++w) mm = fmaxf(mm, red_m[w]);
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < kLogProbThreads / 64; ++w) total += red_s[w] * fast_exp2((red_m[w] - mm) * kLog2e);
+    const int64_t id = p.token_ids[t];
+    float r = __builtin_nanf("");
+    if (id >= 0 && id < p.V) r = (rd.at((int)id) - mm) - __logf(total);
+    p.out[t] = r;
+  }
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -546,4 +631,28 @@ extern "C" int mi_sample_from_logits(const void* logits, int64_t stride_row, int
     else hipLaunchKernelGGL((sample_kernel<false, 1>), grid, block, 0, st, p);
   }
   return mi_check_launch("mi_sample_from_logits");
+}
+
+extern "C" int mi_selected_log_probs(const void* logits, int64_t stride_row, int32_t logits_dtype, int32_t T,
+                                     int32_t vocab, const int64_t* token_ids, float* log_probs, void* stream) {
+  if (T == 0) return MI_OK;
+  if (!logits || !token_ids || !log_probs) return mi_fail(MI_ERR_NULL, "mi_selected_log_probs: null pointer argument");
+  if (T < 0 || vocab <= 0 || stride_row < vocab)
+    return mi_fail(MI_ERR_SHAPE, "mi_selected_log_probs: need T >= 0, vocab > 0 and a row stride of at least vocab");
+  if (logits_dtype != 0 && logits_dtype != 1)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_selected_log_probs: logits must be fp32 (0) or bf16 (1)");
+  LogProbParams p;
+  p.logits = logits; p.stride = stride_row; p.T = T; p.V = vocab; p.token_ids = token_ids; p.out = log_probs;
+  const int esize = logits_dtype == 1 ? 2 : 4;
+  const bool wide = !(((uintptr_t)logits | (uintptr_t)(stride_row * esize)) & 15);  // 16-byte loads
+  const dim3 grid(T), block(kLogProbThreads);
+  hipStream_t st = (hipStream_t)stream;
+  if (logits_dtype == 1) {
+    if (wide) hipLaunchKernelGGL((selected_log_probs_kernel<true, 8>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((selected_log_probs_kernel<true, 1>), grid, block, 0, st, p);
+  } else {
+    if (wide) hipLaunchKernelGGL((selected_log_probs_kernel<false, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((selected_log_probs_kernel<false, 1>), grid, block, 0, st, p);
+  }
+  return mi_check_launch("mi_selected_log_probs");
 }

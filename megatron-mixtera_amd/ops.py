@@ -582,6 +582,24 @@ def last_token_gather(rows: Tensor, request_query_lengths: Tensor, out: Optional
     return out
 
 
+def selected_log_probs(logits: Tensor, token_ids: Tensor) -> Tensor:
+    """``log_softmax(logits.float(), -1)[arange(T), token_ids]`` (fp32 ``[T]``) with one read of each row of
+    ``logits`` ``[T, V]`` (fp32 or bf16) and no ``[T, V]`` intermediate."""
+    lib = _lib.load()
+    stream = _stream(logits)
+    _require(logits.dim() == 2 and logits.stride(1) == 1, "logits must be [T, V] with contiguous V")
+    _require(logits.dtype in (torch.float32, torch.bfloat16), "logits must be fp32 or bf16")
+    T, V = logits.shape
+    _require(token_ids.dtype == torch.int64 and token_ids.dim() == 1 and token_ids.numel() == T
+             and token_ids.is_contiguous() and token_ids.device == logits.device,
+             "token_ids must be a contiguous int64 row with one id per row of logits")
+    out = torch.empty(T, dtype=torch.float32, device=logits.device)
+    _lib.check(lib.mi_selected_log_probs(logits.data_ptr(), logits.stride(0),
+                                         1 if logits.dtype == torch.bfloat16 else 0, T, V,
+                                         token_ids.data_ptr(), out.data_ptr(), stream), "mi_selected_log_probs")
+    return out
+
+
 def sample_from_logits(logits: Tensor, *, top_k: int = 0, top_p: float = 0.0, temperature: float = 1.0,
                        uniform: Optional[Tensor] = None, vocab_size: Optional[int] = None,
                        termination_id: Optional[int] = None, kv_length_offsets: Optional[Tensor] = None,

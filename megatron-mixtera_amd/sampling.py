@@ -4,7 +4,7 @@
 ``TextGenerationController.sample_from_logits``
 (megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315);
 ``sample_and_finish_mask`` adds what ``async_generate_output_tokens_dynamic_batch`` computes
-right after it (:503-512), so a decode step needs one launch between the logits and
+right after it (:519-530), so a decode step needs one launch between the logits and
 ``DynamicInferenceContext.update_requests``.
 
 The reference draws with ``torch.multinomial(probabilities, 1, generator=sampling_rng)``; here

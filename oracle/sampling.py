@@ -7,13 +7,15 @@ Restates, on CPU tensors:
   (megatron/core/inference/contexts/dynamic_context.py:890-918);
 * ``TextGenerationController.sample_from_logits``
   (megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315):
-  greedy argmax (:297-298), division by the temperature (:300-302), the top-k filter
+  greedy argmax (:289-290), division by the temperature (:292-294), the top-k filter
   ``logits < topk(logits, k)[0][..., -1]`` (:216-219), the top-p filter -- descending sort, softmax,
   cumsum, ``cumulative > top_p`` shifted right by one with the first column cleared (:221-240);
 * the finished-request test ``(sample != termination_id) & (length + 1 < maximum length)``
-  (text_generation_controller.py:503-512).
+  (text_generation_controller.py:519-530);
+* ``DynamicInferenceContext.calculate_log_probs`` (dynamic_context.py:1300-1365): which token id each
+  logits row is scored on (:1326-1355) and ``log_softmax(logits.float())[row, id]`` (:1317-1322,1357-1359).
 
-The reference then draws with ``torch.multinomial`` from its own generator (:311-313); a stream of
+The reference then draws with ``torch.multinomial`` from its own generator (:307-309); a stream of
 random numbers cannot be reproduced by another implementation, so the draw restated here is the
 inverse CDF over the kept probabilities in vocabulary order for a GIVEN uniform number -- the same
 distribution.  Temperature: the reference divides in place on the device, where torch evaluates a
@@ -23,7 +25,9 @@ dtype; :func:`scaled_logits` does exactly that.
 Pinned by (tests/test_oracle_sampling.py): ``torch.topk`` / ``torch.sort`` library routines, a
 hand-worked top-p example, the set definition "shortest prefix whose mass exceeds p" by brute
 force, limiting cases (p -> 0 keeps the argmax, p = 1 keeps all, k = V keeps all),
-``numpy.searchsorted`` for the draw, and an empirical-frequency check of the draw.
+``numpy.searchsorted`` for the draw, and an empirical-frequency check of the draw; the log-prob
+functions by ``torch.log_softmax`` / ``torch.logsumexp`` and by the worked example in the reference's
+own comment (dynamic_context.py:1331-1349).
 """
 from __future__ import annotations
 
@@ -105,3 +109,22 @@ def active_request_mask(sample: Tensor, termination_id: int, kv_length_offsets: 
     """uint8 mask of the requests that go on generating."""
     lengths = kv_length_offsets.long() + query_lengths.long() + 1
     return ((sample != termination_id).byte() & torch.less(lengths, output_lengths.long()).byte())
+
+
+def scored_token_ids(token_to_input_ids: Tensor, query_lengths: Tensor, new_tokens: Tensor) -> Tensor:
+    """Id each active token row is scored on: the next prompt token inside a request, the newly
+    sampled token at its last position (dynamic_context.py:1326-1355), by an explicit loop."""
+    ids, row = [], 0
+    flat = token_to_input_ids.tolist()
+    for n, new in zip(query_lengths.tolist(), new_tokens.tolist()):
+        ids += flat[row + 1: row + n] + [new]
+        row += n
+    return torch.tensor(ids, dtype=torch.int64)
+
+
+def selected_log_probs(logits: Tensor, token_ids: Tensor) -> Tensor:
+    """fp64 ``x[id] - log(sum(exp(x)))`` per row of the fp32-converted logits (:1317, :1357-1359)."""
+    x = logits.float().double()
+    mx = x.max(dim=-1, keepdim=True).values
+    lse = (x - mx).exp().sum(-1).log() + mx.squeeze(-1)
+    return x.gather(1, token_ids.view(-1, 1).long()).squeeze(1) - lse

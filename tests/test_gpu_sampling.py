@@ -281,3 +281,77 @@ def test_decode_step_tail_on_a_context(mi, dev):
         if step == 1:
             assert not c.has_unfinished_requests()
             break
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("V", [1, 7, 4096, 32003, 131072])
+def test_selected_log_probs_match_fp64_checker(mi, dev, dtype, V):
+    """log_softmax(row)[id] with one read of the row: 2e-5 absolute against fp64 (fp32 sums of up to
+    131 072 terms, hardware exp2 / log)."""
+    g = torch.Generator().manual_seed(V)
+    T = 37
+    x = (torch.randn(T, V, generator=g) * 5).to(dtype)
+    if V > 64:
+        x[1, 10:40] = float("-inf")
+        x[2, :] = 3.0                         # uniform row: -log V
+        x[3, V // 2] = 60.0                   # one dominant entry
+    ids = torch.randint(0, V, (T,), generator=g)
+    if V > 64:
+        ids[3] = V // 2
+    got = mi.ops.selected_log_probs(x.to(dev), ids.to(dev)).cpu()
+    want = osm.selected_log_probs(x, ids)
+    assert torch.isfinite(got).all()
+    assert (got.double() - want).abs().max().item() <= 2e-5
+    if V > 64:
+        assert abs(got[2].item() + float(torch.tensor(float(V)).log())) <= 2e-5
+        assert abs(got[3].item()) <= 2e-5
+
+
+def test_selected_log_probs_unaligned_rows_and_bad_ids(mi, dev):
+    g = torch.Generator().manual_seed(5)
+    big = torch.randn(6, 1003, generator=g)
+    x = big[:, 1:1002]                         # rows neither 16-byte aligned nor a multiple of 4 wide
+    ids = torch.randint(0, 1001, (6,), generator=g)
+    got = mi.ops.selected_log_probs(x.to(dev)[:, :], ids.to(dev)).cpu()
+    xd = big.to(dev)[:, 1:1002]
+    got2 = mi.ops.selected_log_probs(xd, ids.to(dev)).cpu()
+    want = osm.selected_log_probs(x, ids)
+    assert (got.double() - want).abs().max().item() <= 2e-5
+    assert (got2.double() - want).abs().max().item() <= 2e-5
+    ids[4] = 1001
+    ids[5] = -1
+    bad = mi.ops.selected_log_probs(xd, ids.to(dev)).cpu()
+    assert torch.isnan(bad[4]) and torch.isnan(bad[5]) and torch.isfinite(bad[:4]).all()
+
+
+def test_context_log_probs_through_the_kernel(mi, dev):
+    """calculate_log_probs on a mixed step: ids from the shifted prompt, grouped per request."""
+    Ctx = mi.DynamicInferenceContext
+    saved = (Ctx.TOKEN_ROUNDER, Ctx.REQUEST_ROUNDER)
+    try:
+        Ctx.TOKEN_ROUNDER, Ctx.REQUEST_ROUNDER = 4, 4
+        ctx = Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=64, num_attention_heads=2,
+                  max_sequence_length=64, buffer_size_gb=0.01, buffer_guaranteed_fraction=0.1, chunk_size_tokens=16,
+                  max_requests_override=16, max_tokens_override=256, device=dev)
+        g = torch.Generator().manual_seed(8)
+        V = 300
+        prompts = [torch.randint(0, V, (n,), generator=g) for n in (5, 1, 9)]
+        for rid, pr in enumerate(prompts):
+            ctx.add_request(rid, pr.to(dev), num_tokens_to_generate=4)
+        ctx.initialize_attention_state()
+        T = ctx.padded_active_token_count        # 15 active rows padded to 16
+        logits = torch.randn(1, T, V, generator=g)
+        new = torch.randint(0, V, (3,), generator=g)
+        got = ctx.calculate_log_probs(logits.to(dev), new.to(dev))
+        ids = osm.scored_token_ids(torch.cat(prompts), torch.tensor([5, 1, 9]), new)
+        want = osm.selected_log_probs(logits[0][: ctx.active_token_count], ids)
+        assert [len(r) for r in got] == [5, 1, 9]
+        flat = torch.tensor([v for r in got for v in r], dtype=torch.float64)
+        assert (flat - want).abs().max().item() <= 2e-5
+        # last-token rows only
+        rows = ctx.last_token_logits(logits.to(dev))
+        got_last = ctx.calculate_log_probs(rows.unsqueeze(0), new.to(dev), only_last_token_logits=True)
+        want_last = osm.selected_log_probs(logits[0][osm.last_token_indices(torch.tensor([5, 1, 9]))], new)
+        assert (torch.tensor(got_last, dtype=torch.float64).flatten() - want_last).abs().max().item() <= 2e-5
+    finally:
+        Ctx.TOKEN_ROUNDER, Ctx.REQUEST_ROUNDER = saved

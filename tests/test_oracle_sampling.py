@@ -115,3 +115,35 @@ def test_active_request_mask_vector():
     m = osm.active_request_mask(sample, 2, torch.tensor([3, 3, 8, 8]), torch.tensor([1, 1, 1, 1]),
                                 torch.tensor([10, 10, 10, 11]))
     assert m.dtype == torch.uint8 and m.tolist() == [1, 0, 0, 0]
+
+
+def test_scored_token_ids_reference_comment_example():
+    # the worked example in the reference's comment (dynamic_context.py:1331-1349)
+    ids = osm.scored_token_ids(torch.tensor([31, 75, 45, 16, 90, 12, 72, 24, 88]), torch.tensor([1, 1, 2, 5]),
+                               torch.tensor([52, 12, 3, 86]))
+    assert ids.tolist() == [52, 12, 16, 3, 12, 72, 24, 88, 86]
+    # and the roll / index-assign formulation the reference uses (:1350-1355)
+    g = torch.Generator().manual_seed(11)
+    q = torch.randint(1, 9, (13,), generator=g)
+    tok = torch.randint(0, 1000, (int(q.sum()),), generator=g)
+    new = torch.randint(0, 1000, (13,), generator=g)
+    rolled = tok.roll(-1, 0)
+    rolled[q.cumsum(0) - 1] = new
+    assert torch.equal(osm.scored_token_ids(tok, q, new), rolled)
+
+
+def test_selected_log_probs_matches_library_log_softmax():
+    g = torch.Generator().manual_seed(12)
+    for dtype in (torch.float32, torch.bfloat16):
+        x = (torch.randn(9, 777, generator=g) * 6).to(dtype)
+        x[2, 5:50] = float("-inf")      # masked entries carry no mass
+        ids = torch.randint(0, 777, (9,), generator=g)
+        ids[2] = 3
+        want = torch.log_softmax(x.float().double(), dim=-1)[torch.arange(9), ids]
+        got = osm.selected_log_probs(x, ids)
+        assert torch.allclose(got, want, rtol=0, atol=1e-12)
+        lse = torch.logsumexp(x.float().double(), dim=-1)
+        assert torch.allclose(got, x.float().double()[torch.arange(9), ids] - lse, rtol=0, atol=1e-12)
+    # probabilities of a row sum to one
+    row = torch.randn(1, 50, generator=g).expand(50, 50)
+    assert abs(osm.selected_log_probs(row, torch.arange(50)).exp().sum().item() - 1.0) < 1e-12
