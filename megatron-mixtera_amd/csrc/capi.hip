@@ -103,6 +103,7 @@ extern "C" int mi_set_tuning(const char* name, int32_t value) {
 // streams the KV cache) with a start/stop event pair on the caller's stream; the pairs are
 // read back with mi_profile_collect.  Host objects only: nothing is allocated on the
 // device, and profiling must stay off while a stream is being captured into a graph.
+#include <mutex>
 #include <vector>
 
 namespace {
@@ -110,9 +111,11 @@ struct EventPair { hipEvent_t a, b; };
 std::vector<EventPair> g_pool;     // created once, reused
 size_t g_used = 0;
 bool g_profile = false;
+std::mutex g_profile_mutex;        // entry points may be called from several host threads
 }  // namespace
 
 bool mi_profile_next(hipEvent_t* a, hipEvent_t* b) {
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
   if (!g_profile) return false;
   if (g_used == g_pool.size()) {
     if (g_pool.size() >= 65536) return false;
@@ -130,12 +133,14 @@ bool mi_profile_next(hipEvent_t* a, hipEvent_t* b) {
 }
 
 extern "C" int mi_profile_enable(int32_t on) {
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
   g_profile = on != 0;
   g_used = 0;
   return MI_OK;
 }
 
 extern "C" int32_t mi_profile_collect(float* out_ms, int32_t capacity) {
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
   int32_t n = 0;
   for (size_t i = 0; i < g_used; ++i) {
     if (hipEventSynchronize(g_pool[i].b) != hipSuccess) break;

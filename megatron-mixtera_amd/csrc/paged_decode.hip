@@ -36,6 +36,8 @@
 //   o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max),
 // and writes zeros for zero-length (padded) rows.
 #include "mi_common.h"
+
+#include <atomic>
 #include "mi_capi_internal.h"
 
 namespace mi {
@@ -777,15 +779,15 @@ static int pick_waves_per_block(int Hkv) {
 }
 
 static int device_cu_count() {
-  static int cus[64] = {0};
+  static std::atomic<int> cus[64];  // zero-initialised; callers on several host threads may race to fill a slot
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-  if (!cus[dev]) {
-    int n = 0;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (!n) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-    cus[dev] = n;
+    cus[dev].store(n, std::memory_order_relaxed);
   }
-  return cus[dev];
+  return n;
 }
 
 // Workgroups along the flattened tile sequence: enough to put `decode_wgs_per_cu`
@@ -1025,16 +1027,16 @@ extern "C" int mi_paged_mla_decode_attention(
   const size_t lds = shared_tile ? lds_shared : lds_head + (size_t)wpb * 16 * (576 * 2 + 16);
   if (lds > 160 * 1024)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: batch too large for the LDS of one workgroup");
-  static bool lds_limit_raised[64] = {false};  // per device: more than the default 64 KB of dynamic LDS
+  static std::atomic<bool> lds_limit_raised[64];  // per device: more than the default 64 KB of dynamic LDS
   int dev_id = 0;
   if (hipGetDevice(&dev_id) != hipSuccess || dev_id < 0 || dev_id >= 64) dev_id = 0;
-  if (!lds_limit_raised[dev_id]) {
+  if (!lds_limit_raised[dev_id].load(std::memory_order_acquire)) {
     const hipFuncAttribute attr = hipFuncAttributeMaxDynamicSharedMemorySize;
     if (hipFuncSetAttribute((const void*)paged_mla_decode_stream_kernel, attr, 160 * 1024) != hipSuccess ||
         hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<4>, attr, 160 * 1024) != hipSuccess ||
         hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8>, attr, 160 * 1024) != hipSuccess)
       return mi_fail(MI_ERR_LAUNCH, "mi_paged_mla_decode_attention: cannot raise the dynamic LDS limit");
-    lds_limit_raised[dev_id] = true;
+    lds_limit_raised[dev_id].store(true, std::memory_order_release);
   }
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);

@@ -8,7 +8,9 @@ Three layers of evidence:
 2. the two implementations against each other on random request streams;
 3. invariants (every chunk id is either free or owned exactly once, padded rows, ...).
 """
+import json
 import math
+import os
 import random
 
 import numpy as np
@@ -16,6 +18,10 @@ import pytest
 import torch
 
 from oracle import context as oc
+
+# expected values held by the reference's own tests (data only; each entry names its source)
+with open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")) as _f:
+    GOLD = json.load(_f)
 
 
 @pytest.fixture()
@@ -56,11 +62,12 @@ def engine_ctx(Ctx, **over):
 # --------------------------------------------------------------------------- sizing constants
 def test_sizing_constants_of_the_reference_tests(Ctx):
     c = small_ctx(Ctx)
-    assert c.gtd_chunk_count == 48
-    assert c.gtd_request_count == 12
-    assert c.chunk_allocator.chunk_count_total == 491
-    assert c.max_requests == 128
-    assert c.max_tokens == 62848
+    want = GOLD["sizing_small_context"]["expected"]
+    assert c.gtd_chunk_count == want["gtd_chunk_count"] == 48
+    assert c.gtd_request_count == want["gtd_request_count"] == 12
+    assert c.chunk_allocator.chunk_count_total == want["chunk_count_total"] == 491
+    assert c.max_requests == want["max_requests"] == 128
+    assert c.max_tokens == want["max_tokens"] == 62848
     assert torch.all(c.request_ids == -1)
     assert c.memory_buffer.shape == (2, 4, 491, 128, 2, 8) and (c.memory_buffer == -1).all()
     assert c.request_to_kv_chunk_ids.shape == (128, 4) and c.request_to_kv_chunk_ids.dtype == torch.int32
@@ -68,20 +75,20 @@ def test_sizing_constants_of_the_reference_tests(Ctx):
     ref = oc.sizing(itemsize=4, num_layers=4, kv_channels=8, num_heads=2, max_sequence_length=512,
                     buffer_size_gb=0.03, buffer_guaranteed_fraction=0.1, chunk_size_tokens=128,
                     token_rounder=64, request_rounder=64)
-    assert (ref["gtd_chunk_count"], ref["gtd_request_count"], ref["chunk_count_total"], ref["max_requests"],
-            ref["max_tokens"]) == (48, 12, 491, 128, 62848)
+    assert {k: ref[k] for k in want} == want
 
 
 def test_engine_sizing_constants(Ctx):
+    gold = GOLD["sizing_engine_context"]
     c = engine_ctx(Ctx, max_requests_override=32, max_tokens_override=8 * 20)
-    assert (c.max_requests, c.max_tokens) == (32, 160)
+    assert [c.max_requests, c.max_tokens] == gold["overrides"]["expected"]
     c = engine_ctx(Ctx, buffer_overflow_factor=0.1)
-    assert (c.max_requests, c.max_tokens) == (420, 420)
+    assert [c.max_requests, c.max_tokens] == gold["overflow_factor"]["expected"]
     ref = oc.sizing(itemsize=2, num_layers=4, kv_channels=8, num_heads=4, max_sequence_length=20,
                     buffer_size_gb=0.1, buffer_guaranteed_fraction=0.01, chunk_size_tokens=256,
                     buffer_overflow_factor=0.1, token_rounder=4, request_rounder=4)
-    assert (ref["max_requests"], ref["max_tokens"], ref["chunk_size_bytes"], ref["chunk_count_total"]) == (
-        420, 420, 131072, 819)
+    assert [ref["max_requests"], ref["max_tokens"]] == gold["overflow_factor"]["expected"]
+    assert (ref["chunk_size_bytes"], ref["chunk_count_total"]) == (131072, 819)
 
 
 def test_tensor_parallel_divides_heads_and_rounders(Ctx):
@@ -98,10 +105,7 @@ def test_tensor_parallel_divides_heads_and_rounders(Ctx):
     assert c.chunk_size_bytes == 2 * 2 * 1 * 16 * 2 * 16
 
 
-@pytest.mark.parametrize("num_cuda_graphs,expected", [
-    (0, [64]), (1, [64]), (2, [64, 32]), (4, [64, 48, 32, 16]), (8, [64, 56, 48, 40, 32, 24, 16, 8]),
-    (16, [64, 56, 48, 40, 32, 24, 16, 8]), (64, [64, 56, 48, 40, 32, 24, 16, 8]),
-    (1024, [64, 56, 48, 40, 32, 24, 16, 8])])
+@pytest.mark.parametrize("num_cuda_graphs,expected", [tuple(row) for row in GOLD["cuda_graph_token_counts"]["table"]])
 def test_cuda_graph_token_counts(Ctx, num_cuda_graphs, expected):
     c = engine_ctx(Ctx, max_requests_override=64, max_tokens_override=64 * 20, num_cuda_graphs=num_cuda_graphs)
     assert c.cuda_graph_token_counts == expected
@@ -110,14 +114,13 @@ def test_cuda_graph_token_counts(Ctx, num_cuda_graphs, expected):
 
 
 @pytest.mark.parametrize("mode", ["DECODE", "NON_DECODE"])
-@pytest.mark.parametrize("warm,expected", [(1, 8), (2, 8), (4, 8), (8, 8), (10, 16), (12, 16), (16, 16), (20, 24),
-                                           (24, 24), (28, 32), (32, 32)])
+@pytest.mark.parametrize("warm,expected", [tuple(row) for row in GOLD["cuda_graph_warmup_padding"]["table"]])
 def test_cuda_graph_warmup_padding(mi, Ctx, mode, warm, expected):
     if warm == 1 and mode == "NON_DECODE":
         pytest.skip("not supported by the reference either")
     c = engine_ctx(Ctx, max_sequence_length=17, max_requests_override=32, max_tokens_override=32 * 17,
                    num_cuda_graphs=8)
-    assert c.is_decode_only() and c.cuda_graph_token_counts == [32, 24, 16, 8]
+    assert c.is_decode_only() and c.cuda_graph_token_counts == GOLD["cuda_graph_warmup_padding"]["token_counts"]
     c.initialize_attention_state(num_warmup_tokens=warm, warmup_engine_mode=getattr(mi.WarmupEngineMode, mode))
     assert expected == c.padded_active_request_count == c.padded_active_token_count
     ids, pos = c.current_input_and_position_ids()
@@ -140,19 +143,21 @@ def test_cuda_graph_warmup_padding(mi, Ctx, mode, warm, expected):
 def test_allocator_vectors(Ctx):
     c = small_ctx(Ctx)
     a = c.chunk_allocator
-    assert a.allocate_memory_chunks(4).tolist() == [486, 487, 488, 489]
-    assert a.chunk_count_avail == 486
-    a.release_memory_chunks(torch.tensor([488, 489], dtype=torch.int32))
-    assert a.chunk_count_avail == 488
-    assert a.allocate_memory_chunks(1).item() == 489
-    assert a.chunk_count_avail == 487
+    gold = GOLD["allocator"]
+    assert a.allocate_memory_chunks(4).tolist() == gold["allocate_4"]
+    assert a.chunk_count_avail == gold["avail_after_allocate_4"]
+    a.release_memory_chunks(torch.tensor(gold["release"], dtype=torch.int32))
+    assert a.chunk_count_avail == gold["avail_after_release"]
+    assert a.allocate_memory_chunks(1).item() == gold["allocate_1"]
+    assert a.chunk_count_avail == gold["avail_after_allocate_1"]
     assert a.allocate_memory_chunks(a.chunk_count_avail + 100) is None
-    assert a.dummy_chunk_idx == 490 == c.dummy_chunk_idx
+    assert a.dummy_chunk_idx == gold["dummy_chunk_idx"] == c.dummy_chunk_idx
     r = oc.RefContext(max_requests=128, max_tokens=62848, chunk_count_total=491, chunk_size_tokens=128,
                       max_kv_chunk_count=4, gtd_request_count=12, gtd_chunk_count=48, max_sequence_length=512)
-    assert r.alloc(4) == [486, 487, 488, 489] and r.avail == 486
-    r.release([488, 489])
-    assert r.alloc(1) == [489] and r.avail == 487 and r.alloc(r.avail + 100) is None
+    assert r.alloc(4) == gold["allocate_4"] and r.avail == gold["avail_after_allocate_4"]
+    r.release(gold["release"])
+    assert r.alloc(1) == [gold["allocate_1"]] and r.avail == gold["avail_after_allocate_1"]
+    assert r.alloc(r.avail + 100) is None
 
 
 def test_is_memory_available_truth_table(Ctx):
@@ -223,14 +228,15 @@ def test_reset_restores_every_row(Ctx):
 # --------------------------------------------------------------------------- add_request vector
 def test_add_request_vector(Ctx):
     c = small_ctx(Ctx)
-    n = 144
+    gold = GOLD["add_request"]
+    n = gold["prompt_length"]
     c.add_request(request_id=0, tokens=torch.arange(0, n, dtype=torch.long))
     assert c.total_request_count == 1 and c.active_token_count == n
     assert c.request_ids[0] == 0 and torch.all(c.request_ids[1:] == -1)
     assert c.request_query_lengths[0] == n and c.request_kv_length_offsets[0] == 0
-    assert c.request_to_kv_chunk_ids[0].tolist() == [488, 489, -1, -1]
-    assert c.request_kv_chunk_counts[0] == 2 and c.request_last_kv_chunk_id[0] == 489
-    assert c.request_last_kv_chunk_offset[0].item() == 15
+    assert c.request_to_kv_chunk_ids[0].tolist() == gold["block_row"]
+    assert c.request_kv_chunk_counts[0] == gold["chunk_count"] and c.request_last_kv_chunk_id[0] == gold["last_chunk_id"]
+    assert c.request_last_kv_chunk_offset[0].item() == gold["last_chunk_offset"]
     ar = torch.arange(0, n)
     assert torch.equal(c.token_to_pos_ids[:n], ar) and torch.equal(c.token_to_input_ids[:n], ar)
     assert torch.equal(c.token_to_position_in_request[:n], ar)
@@ -279,8 +285,9 @@ def test_update_requests_all_finished_resets(Ctx):
 def test_update_requests_pause_finish_resume_scenario(Ctx):
     """The reference's full scenario: 2 paused, 3 finished, 2 newly paused, 4 resumed (LIFO)."""
     c = small_ctx(Ctx)
-    mask = torch.tensor([1, 0, 1, 1, 1, 0, 0, 1], dtype=torch.int32)
-    new = torch.arange(2, 10, dtype=torch.int32)
+    gold = GOLD["update_requests_scenario"]
+    mask = torch.tensor(gold["active_requests_mask"], dtype=torch.int32)
+    new = torch.tensor(gold["new_tokens"], dtype=torch.int32)
     c.paused_request_count = 2
     c.paused_tokens = torch.tensor([0, 1], dtype=torch.int32)
     c.total_request_count = 5
@@ -290,15 +297,14 @@ def test_update_requests_pause_finish_resume_scenario(Ctx):
     c = small_ctx(Ctx)
     _setup_big_scenario(c)
     newly = c.update_requests(active_requests_mask=mask, new_tokens=new)
-    assert c.request_ids[0:7].tolist() == [0, 1, 5, 6, 4, 2, 9]
-    assert (c.paused_request_count, c.total_request_count, c.active_token_count) == (0, 7, 7)
-    assert c.request_last_kv_chunk_offset[0:10].tolist() == [0, 0, 0, 0, 11, 11, 11, 10, 10, 10]
-    assert c.token_to_input_ids[:7].tolist() == [0, 1, 5, 6, 4, 2, 9]
-    assert c.token_to_pos_ids[:7].tolist() == [128, 128, 128, 128, 11, 11, 11]
-    assert c.request_to_kv_chunk_ids[0:10].tolist() == [
-        [479, 482, -1, -1], [480, 479, -1, -1], [484, 486, -1, -1], [485, 487, -1, -1], [483, -1, -1, -1],
-        [481, -1, -1, -1], [488, -1, -1, -1], [-1, -1, -1, -1], [-1, -1, -1, -1], [-1, -1, -1, -1]]
-    assert c.chunk_allocator.chunk_count_avail == 479
+    assert c.request_ids[0:7].tolist() == gold["request_ids"]
+    assert (c.paused_request_count, c.total_request_count, c.active_token_count) == (
+        gold["paused_request_count"], gold["total_request_count"], gold["active_token_count"])
+    assert c.request_last_kv_chunk_offset[0:10].tolist() == gold["request_last_kv_chunk_offset"]
+    assert c.token_to_input_ids[:7].tolist() == gold["token_to_input_ids"]
+    assert c.token_to_pos_ids[:7].tolist() == gold["token_to_pos_ids"]
+    assert c.request_to_kv_chunk_ids[0:10].tolist() == gold["request_to_kv_chunk_ids"]
+    assert c.chunk_allocator.chunk_count_avail == gold["chunk_count_avail"]
     # (the scenario stores synthetic last-chunk ids 0..9 for the rows that were not resumed)
     assert c.token_to_chunk_idx[:7].tolist() == [482, 479, 486, 487, 4, 2, 9]
     assert c.token_to_local_position_within_kv_chunk[:7].tolist() == [0, 0, 0, 0, 11, 11, 11]
@@ -319,9 +325,9 @@ def test_update_requests_pause_finish_resume_scenario(Ctx):
         r.kv_off[i] = r.last_off[i] = 127
     r.kv_off[3], r.n_chunks[3], r.last_chunk[3] = 16384 + 10, 2, 11
     assert r.update_requests(mask.tolist(), new.tolist()) == []
-    assert r.ids[:7].tolist() == [0, 1, 5, 6, 4, 2, 9] and r.avail == 479
-    assert r.table[:10].tolist() == c.request_to_kv_chunk_ids[0:10].tolist()
-    assert r.tok_pos[:7].tolist() == [128, 128, 128, 128, 11, 11, 11]
+    assert r.ids[:7].tolist() == gold["request_ids"] and r.avail == gold["chunk_count_avail"]
+    assert r.table[:10].tolist() == gold["request_to_kv_chunk_ids"]
+    assert r.tok_pos[:7].tolist() == gold["token_to_pos_ids"]
 
 
 def test_release_chunks_of_finished_requests(Ctx):

@@ -13,7 +13,7 @@ import pytest
 import torch
 
 from oracle import context as oc
-from test_context_host import _setup_big_scenario, _snapshot_product, _snapshot_ref, set_rounder
+from test_context_host import GOLD, _setup_big_scenario, _snapshot_product, _snapshot_ref, set_rounder
 
 pytestmark = pytest.mark.gpu
 
@@ -79,20 +79,20 @@ def test_count_mismatch_raises_and_changes_nothing(Ctx, dev):
 def test_pause_finish_resume_scenario(Ctx, dev, fused):
     """2 paused, 3 finished, 2 newly paused, 4 resumed (LIFO): the constants of the reference's test."""
     c = small_ctx(Ctx, dev, fused_bookkeeping=fused)
-    mask = torch.tensor([1, 0, 1, 1, 1, 0, 0, 1], dtype=torch.int32)
-    new = torch.arange(2, 10, dtype=torch.int32)
+    gold = GOLD["update_requests_scenario"]          # tests/golden/reference_vectors.json
+    mask = torch.tensor(gold["active_requests_mask"], dtype=torch.int32)
+    new = torch.tensor(gold["new_tokens"], dtype=torch.int32)
     _setup_big_scenario(c)
     c.paused_tokens = c.paused_tokens.to(dev)
     newly = c.update_requests(active_requests_mask=mask.to(dev), new_tokens=new.to(dev))
-    assert c.request_ids[0:7].tolist() == [0, 1, 5, 6, 4, 2, 9]
-    assert (c.paused_request_count, c.total_request_count, c.active_token_count) == (0, 7, 7)
-    assert c.request_last_kv_chunk_offset[0:10].tolist() == [0, 0, 0, 0, 11, 11, 11, 10, 10, 10]
-    assert c.token_to_input_ids[:7].tolist() == [0, 1, 5, 6, 4, 2, 9]
-    assert c.token_to_pos_ids[:7].tolist() == [128, 128, 128, 128, 11, 11, 11]
-    assert c.request_to_kv_chunk_ids[0:10].tolist() == [
-        [479, 482, -1, -1], [480, 479, -1, -1], [484, 486, -1, -1], [485, 487, -1, -1], [483, -1, -1, -1],
-        [481, -1, -1, -1], [488, -1, -1, -1], [-1, -1, -1, -1], [-1, -1, -1, -1], [-1, -1, -1, -1]]
-    assert c.chunk_allocator.chunk_count_avail == 479
+    assert c.request_ids[0:7].tolist() == gold["request_ids"]
+    assert (c.paused_request_count, c.total_request_count, c.active_token_count) == (
+        gold["paused_request_count"], gold["total_request_count"], gold["active_token_count"])
+    assert c.request_last_kv_chunk_offset[0:10].tolist() == gold["request_last_kv_chunk_offset"]
+    assert c.token_to_input_ids[:7].tolist() == gold["token_to_input_ids"]
+    assert c.token_to_pos_ids[:7].tolist() == gold["token_to_pos_ids"]
+    assert c.request_to_kv_chunk_ids[0:10].tolist() == gold["request_to_kv_chunk_ids"]
+    assert c.chunk_allocator.chunk_count_avail == gold["chunk_count_avail"]
     assert c.token_to_chunk_idx[:7].tolist() == [482, 479, 486, 487, 4, 2, 9]
     assert c.token_to_local_position_within_kv_chunk[:7].tolist() == [0, 0, 0, 0, 11, 11, 11]
     assert c.token_to_request_idx[:7].tolist() == list(range(7))

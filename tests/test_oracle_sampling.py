@@ -118,10 +118,13 @@ def test_active_request_mask_vector():
 
 
 def test_scored_token_ids_reference_comment_example():
-    # the worked example in the reference's comment (dynamic_context.py:1331-1349)
-    ids = osm.scored_token_ids(torch.tensor([31, 75, 45, 16, 90, 12, 72, 24, 88]), torch.tensor([1, 1, 2, 5]),
-                               torch.tensor([52, 12, 3, 86]))
-    assert ids.tolist() == [52, 12, 16, 3, 12, 72, 24, 88, 86]
+    # the worked example in the reference's comment (dynamic_context.py:1331-1349), kept as data
+    import json, os
+    with open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")) as f:
+        gold = json.load(f)["log_probs_token_shift"]
+    ids = osm.scored_token_ids(torch.tensor(gold["active_token_ids"]), torch.tensor(gold["active_query_lengths"]),
+                               torch.tensor(gold["new_tokens"]))
+    assert ids.tolist() == gold["scored_token_ids"] == [52, 12, 16, 3, 12, 72, 24, 88, 86]
     # and the roll / index-assign formulation the reference uses (:1350-1355)
     g = torch.Generator().manual_seed(11)
     q = torch.randint(1, 9, (13,), generator=g)
