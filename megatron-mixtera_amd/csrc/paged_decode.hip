@@ -730,10 +730,15 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
 }
 
 // One workgroup per (request, query head): merge the partials of the workgroups that
-// shared the request; zero-length rows get zeros.
+// shared the request; zero-length rows get zeros.  blockDim.x = HD * S: S groups of HD threads take the
+// segments round-robin in batches of 8 (a request cut over hundreds of workgroups is a chain of dependent
+// memory round trips otherwise) and group 0 folds the S running (maximum, numerator, denominator) triples.
 template <int HD>
-__global__ __launch_bounds__(HD) void paged_decode_merge_kernel(DecodeParams p) {
-  const int r = blockIdx.y, hq = blockIdx.x, d = threadIdx.x;
+__global__ __launch_bounds__(1024) void paged_decode_merge_kernel(DecodeParams p) {
+  constexpr int kMaxGroups = 1024 / HD;
+  __shared__ float red[3][kMaxGroups > 1 ? 1024 : 1];
+  const int r = blockIdx.y, hq = blockIdx.x, d = threadIdx.x % HD, grp = threadIdx.x / HD;
+  const int groups = blockDim.x / HD;
   int row;
   if (!decode_row(p, r, row)) return;
   // The kernel is a chain of dependent memory round trips, so everything that does not depend
@@ -742,13 +747,13 @@ __global__ __launch_bounds__(HD) void paged_decode_merge_kernel(DecodeParams p) 
   const int len = p.lens[r];
   const int first = p.seg_info[2 * r], last = p.seg_info[2 * r + 1];  // stale for len <= 0: not used then
   uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + d;
-  if (len <= 0) {
-    *o = 0;
+  if (len <= 0) {  // (uniform over the workgroup, like the two returns around it)
+    if (grp == 0) *o = 0;
     return;
   }
   if (first == last) return;  // written directly by the streaming kernel
   float mx = -INFINITY, num = 0.f, den = 0.f;
-  for (int w0 = first; w0 <= last; w0 += 8) {
+  for (int w0 = first + 8 * grp; w0 <= last; w0 += 8 * groups) {
     float lse[8], po[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -767,7 +772,31 @@ __global__ __launch_bounds__(HD) void paged_decode_merge_kernel(DecodeParams p) 
       }
     }
   }
+  if (kMaxGroups > 1 && groups > 1) {
+    red[0][threadIdx.x] = mx; red[1][threadIdx.x] = num; red[2][threadIdx.x] = den;
+    __syncthreads();
+    if (grp != 0) return;
+    for (int g2 = 1; g2 < groups; ++g2) {
+      const float m2 = red[0][g2 * HD + d];
+      if (m2 == -INFINITY) continue;  // that group had no segment
+      const float m_new = fmaxf(mx, m2);
+      const float a = fast_exp2(mx - m_new), wt = fast_exp2(m2 - m_new);
+      num = num * a + wt * red[1][g2 * HD + d];
+      den = den * a + wt * red[2][g2 * HD + d];
+      mx = m_new;
+    }
+  }
   *o = f32_to_bf16(num / den);
+}
+
+// Thread groups per merge workgroup: one per 8 segments a request is expected to be cut into.
+static int merge_groups(int grid_x, int R, int head_dim) {
+  const int per_request = grid_x / (R > 0 ? R : 1) + 2;
+  int g = (per_request + 7) / 8;
+  const int cap = 1024 / head_dim;
+  if (g > cap) g = cap;
+  if (g > 8) g = 8;
+  return g < 1 ? 1 : g;
 }
 
 static int pick_waves_per_block(int Hkv) {
@@ -910,8 +939,9 @@ int mi::launch_paged_decode(
 #undef MI_LAUNCH_DECODE
   if (timed) (void)hipEventRecord(ev_b, st);
   dim3 mgrid(Hq, R);
-  if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128>), mgrid, dim3(128), 0, st, p);
-  else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, dim3(64), 0, st, p);
+  const dim3 mblock(head_dim * merge_groups(p.grid, R, head_dim));
+  if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128>), mgrid, mblock, 0, st, p);
+  else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, mblock, 0, st, p);
   return mi_check_launch("mi_paged_decode_attention");
 }
 
@@ -1048,6 +1078,6 @@ extern "C" int mi_paged_mla_decode_attention(
   else
     hipLaunchKernelGGL(paged_mla_decode_stream_kernel, dim3(grid_x, groups / wpb), dim3(64 * wpb), lds, st, p);
   if (timed) (void)hipEventRecord(ev_b, st);
-  hipLaunchKernelGGL((paged_decode_merge_kernel<512>), dim3(Hq, R), dim3(512), 0, st, p);
+  hipLaunchKernelGGL((paged_decode_merge_kernel<512>), dim3(Hq, R), dim3(512 * merge_groups(grid_x, R, 512)), 0, st, p);
   return mi_check_launch("mi_paged_mla_decode_attention");
 }
