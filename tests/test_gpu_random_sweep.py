@@ -22,6 +22,13 @@ def _note(text):
     _last_case[0] = text
 
 
+def poison(dev):
+    """Fill the memory the allocator is about to hand out again with NaN, so that an output row or a
+    partial result that a kernel fails to write cannot pass as a plausible number."""
+    junk = torch.full((32 << 20,), float("nan"), device=dev)
+    del junk
+
+
 def close(out, ref, tol, what):
     out = out.float().cpu().reshape(ref.shape)
     if not torch.isfinite(out).all():
@@ -91,6 +98,7 @@ def case_decode(mi, dev, rng, seed, fp8):
             vs = torch.empty_like(ks)
             mi.ops.quantize_chunks_fp8(kc.contiguous(), k8, ks)
             mi.ops.quantize_chunks_fp8(vc.contiguous(), v8, vs)
+            poison(dev)
             out = mi.ops.paged_decode_attention(qd, k8, v8, lens_t.to(dev), bt.to(dev), split_tokens=split,
                                                 k_scales=ks, v_scales=vs)
             torch.cuda.synchronize()
@@ -98,6 +106,7 @@ def case_decode(mi, dev, rng, seed, fp8):
                                             v_scales=vs.cpu())
             close(out, ref, 2.5e-2, "decode fp8")
         else:
+            poison(dev)
             out = mi.ops.paged_decode_attention(qd, kc, vc, lens_t.to(dev), bt.to(dev), split_tokens=split)
             torch.cuda.synchronize()
             ref = oa.paged_decode_attention(q.squeeze(1), buf[0, layer], buf[1, layer], lens_t, bt)
@@ -151,13 +160,16 @@ def case_prefill(mi, dev, rng, seed, fp8):
             vs = torch.empty_like(ks)
             mi.ops.quantize_chunks_fp8(kc.to(dev), k8, ks)
             mi.ops.quantize_chunks_fp8(vc.to(dev), v8, vs)
+            poison(dev)
             out = mi.ops.paged_prefill_attention(q.to(dev), k8, v8, cu_q.to(dev), kv_lens.to(dev), bt.to(dev),
                                                  k_scales=ks, v_scales=vs)
             torch.cuda.synchronize()
             ref = oa.paged_varlen_attention(q, k8.cpu(), v8.cpu(), cu_q, kv_lens, bt, k_scales=ks.cpu(), v_scales=vs.cpu())
             close(out, ref, 2.5e-2, "prefill fp8")
         else:
-            out = mi.ops.paged_prefill_attention(q.to(dev), kc.to(dev), vc.to(dev), cu_q.to(dev), kv_lens.to(dev),
+            qd_, kd_, vd_ = q.to(dev), kc.to(dev), vc.to(dev)
+            poison(dev)
+            out = mi.ops.paged_prefill_attention(qd_, kd_, vd_, cu_q.to(dev), kv_lens.to(dev),
                                                  bt.to(dev))
             torch.cuda.synchronize()
             ref = oa.paged_varlen_attention(q, kc, vc, cu_q, kv_lens, bt)
@@ -182,7 +194,9 @@ def case_mla_decode(mi, dev, rng, seed):
     mi.ops.set_tuning("decode_grid", grid)
     mi.ops.set_tuning("mla_decode_lds", lds)
     try:
-        out = mi.ops.paged_mla_decode_attention(q.to(dev), cache.to(dev), lens_t.to(dev), bt.to(dev), softmax_scale=0.07)
+        qd_, cd_ = q.to(dev), cache.to(dev)
+        poison(dev)
+        out = mi.ops.paged_mla_decode_attention(qd_, cd_, lens_t.to(dev), bt.to(dev), softmax_scale=0.07)
         torch.cuda.synchronize()
     finally:
         mi.ops.set_tuning("decode_grid", 0)
