@@ -1,5 +1,7 @@
 """GPU parity on seeded random cases: decode (bf16 / fp8 cache), prefill and mixed batches (bf16 / fp8),
-multi-latent decode -- random head counts, head widths, chunk sizes, lengths around every tile / chunk
+multi-latent decode, and the write side (scatter append in three dtypes, the quantising fp8 append of
+token runs, fused norm + rotary + append from split or mixed QKV input) -- random head counts, head
+widths, chunk sizes, lengths around every tile / chunk
 boundary, zero-length rows, strided query views, caches that are layer views of a bigger buffer, wider
 block tables, and random settings of the grid / tile / kernel-choice knobs -- each compared with the CPU
 checker at the bars of the dedicated tests (2e-2 abs/rel bf16; 2.5e-2 for an fp8 cache against the checker
@@ -12,6 +14,7 @@ import pytest
 import torch
 
 from oracle import paged_attention as oa
+from oracle import rope_norm as orn
 
 pytestmark = pytest.mark.gpu
 
@@ -232,3 +235,158 @@ def test_random_cases_match_the_checker(mi, dev, block):
         except AssertionError as e:
             raise AssertionError(f"{_last_case[0]}: {e}") from None
     assert rejected < 30
+
+
+# ---------------------------------------------------------------------------------------------- write side
+def mixed_batch(mi, rng, gen, chunk, max_req=8):
+    """Requests with q_len new tokens over ctx cached ones -> cu_q, kv_lens, block table, per-token rows."""
+    R = rng.randint(1, max_req)
+    q_lens, ctx = [], []
+    for _ in range(R):
+        k = rng.random()
+        if k < 0.4:
+            q_lens.append(1)
+            ctx.append(rng.randint(0, 700))
+        else:
+            q_lens.append(rng.choice([2, 15, 16, 17, 63, 64, 65, chunk - 1, chunk, chunk + 1, 2 * chunk + 3,
+                                      rng.randint(1, 500)]))
+            ctx.append(rng.choice([0, 0, 5, chunk - 1, chunk, rng.randint(0, 600)]))
+    kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.zeros(R + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, gen)
+    pos, ci, lo = mi.synthetic.prefill_token_rows(cu_q, kv_lens, bt, chunk)
+    return q_lens, ctx, cu_q, kv_lens, bt, N, pos, ci, lo
+
+
+def case_append(mi, dev, rng, seed):
+    gen = torch.Generator().manual_seed(seed)
+    chunk = rng.choice([16, 32, 64, 128, 256])
+    Hkv = rng.choice([1, 2, 3, 8])
+    d = rng.choice([8, 64, 128, 5])
+    dtype = rng.choice([torch.bfloat16, torch.float32, torch.float16])
+    q_lens, ctx, cu_q, kv_lens, bt, N, pos, ci, lo = mixed_batch(mi, rng, gen, chunk)
+    _note(f"append seed={seed} chunk={chunk} Hkv={Hkv} d={d} dtype={dtype} q_lens={q_lens} ctx={ctx}")
+    T = int(cu_q[-1])
+    k = torch.randn(T, 1, Hkv, d, generator=gen).to(dtype)
+    v = torch.randn(T, 1, Hkv, d, generator=gen).to(dtype)
+    kc = torch.full((N + 1, chunk, Hkv, d), -1.0).to(dtype)
+    vc = kc.clone()
+    kcd, vcd = kc.to(dev), vc.to(dev)
+    poison(dev)
+    mi.ops.kv_append(k.to(dev), v.to(dev), kcd, vcd, ci.to(dev), lo.to(dev))
+    torch.cuda.synchronize()
+    oa.kv_append(kc, vc, k.squeeze(1), v.squeeze(1), ci, lo)
+    assert torch.equal(kcd.cpu().view(torch.uint8), kc.view(torch.uint8)), "K cache differs"
+    assert torch.equal(vcd.cpu().view(torch.uint8), vc.view(torch.uint8)), "V cache differs"
+
+
+def case_append_fp8(mi, dev, rng, seed):
+    gen = torch.Generator().manual_seed(seed)
+    chunk = rng.choice([64, 128, 256])
+    Hkv = rng.choice([1, 2, 8])
+    d = 128
+    q_lens, ctx, cu_q, kv_lens, bt, N, pos, ci, lo = mixed_batch(mi, rng, gen, chunk, max_req=5)
+    headroom = rng.choice([1.0, 2.0, 1.5])
+    _note(f"append_fp8 seed={seed} chunk={chunk} Hkv={Hkv} q_lens={q_lens} ctx={ctx} headroom={headroom}")
+    T = int(cu_q[-1])
+    scale_mag = torch.rand(T, 1, Hkv, 1, generator=gen) * 3 + 0.05
+    k = (torch.randn(T, 1, Hkv, d, generator=gen) * scale_mag).bfloat16()
+    v = (torch.randn(T, 1, Hkv, d, generator=gen) * scale_mag).bfloat16()
+    # existing content: chunks quantised from random data (so that runs continuing a chunk reuse a real scale)
+    base_k = torch.randn(N + 1, chunk, Hkv, d, generator=gen).bfloat16()
+    base_v = torch.randn(N + 1, chunk, Hkv, d, generator=gen).bfloat16()
+    k8, ks = oa.quantize_chunks_fp8(base_k)
+    v8, vs = oa.quantize_chunks_fp8(base_v)
+    k8d, v8d, ksd, vsd = k8.to(dev), v8.to(dev), ks.to(dev), vs.to(dev)
+    poison(dev)
+    mi.ops.kv_append_fp8(k.to(dev), v.to(dev), k8d, v8d, ksd, vsd, ci.to(dev), lo.to(dev), headroom=headroom)
+    torch.cuda.synchronize()
+    oa.kv_append_fp8(k8, ks, k.squeeze(1), ci, lo, headroom=headroom)
+    oa.kv_append_fp8(v8, vs, v.squeeze(1), ci, lo, headroom=headroom)
+    assert torch.equal(ksd.cpu(), ks) and torch.equal(vsd.cpu(), vs), "scales differ"
+    assert torch.equal(k8d.cpu(), k8) and torch.equal(v8d.cpu(), v8), "bytes differ"
+
+
+def case_norm_rope(mi, dev, rng, seed):
+    gen = torch.Generator().manual_seed(seed)
+    chunk = rng.choice([16, 64, 256])
+    d = rng.choice([64, 128])
+    rot = rng.choice([d, d // 2, d, 32])
+    Hkv = rng.choice([1, 2, 4, 8])
+    Hq = Hkv * rng.choice([1, 2, 4])
+    norm = rng.choice([None, "rms", "l2"])
+    interleaved = rng.random() < 0.3
+    vec = rng.choice([0, 1, 2])
+    mixed = rng.random() < 0.5
+    q_lens, ctx, cu_q, kv_lens, bt, N, pos, ci, lo = mixed_batch(mi, rng, gen, chunk)
+    _note(f"norm_rope seed={seed} chunk={chunk} d={d} rot={rot} Hq={Hq} Hkv={Hkv} norm={norm} il={interleaved} "
+          f"vec={vec} mixed={mixed} q_lens={q_lens} ctx={ctx}")
+    T = int(cu_q[-1])
+    G = Hq // Hkv
+    mixed_qkv = torch.randn(T, 1, Hkv * (G + 2) * d, generator=gen).bfloat16()
+    q, k, v = orn.split_mixed_qkv(mixed_qkv, Hq, Hkv)
+    qw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16()
+    kw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16()
+    table = orn.rotary_table(int(kv_lens.max()) + 2, rot, base=10000.0, interleaved=interleaved)
+    eps = 1e-5
+    q_ref = orn.norm_rope(q.squeeze(1), pos, table, norm=norm, weight=qw if norm == "rms" else None, eps=eps,
+                          interleaved=interleaved)
+    k_ref = orn.norm_rope(k.squeeze(1), pos, table, norm=norm, weight=kw if norm == "rms" else None, eps=eps,
+                          interleaved=interleaved)
+    kc = torch.full((N + 1, chunk, Hkv, d), -1.0).bfloat16()
+    vc = kc.clone()
+    kcd, vcd = kc.to(dev), vc.to(dev)
+    mi.ops.set_tuning("norm_rope_vectorised", vec)
+    try:
+        poison(dev)
+        if mixed:
+            q_out = torch.empty(T, 1, Hq, d, dtype=torch.bfloat16, device=dev)
+            mi.ops.qkv_norm_rope_append(mixed_qkv.to(dev), num_query_heads=Hq, num_kv_heads=Hkv, query_out=q_out,
+                                        q_weight=qw.to(dev), k_weight=kw.to(dev), eps=eps, norm=norm,
+                                        rotary_emb=table.to(dev), q_positions=pos.to(dev),
+                                        k_positions=pos.to(dev), rotary_interleaved=interleaved, k_cache=kcd, v_cache=vcd,
+                                        token_to_chunk_idx=ci.to(dev), token_to_local_pos=lo.to(dev))
+        else:
+            q_out = q.to(dev).clone()
+            mi.ops.norm_rope_append(q_out, k.to(dev), value=v.to(dev), q_weight=qw.to(dev), k_weight=kw.to(dev), eps=eps,
+                                    norm=norm, rotary_emb=table.to(dev), q_positions=pos.to(dev), k_positions=pos.to(dev),
+                                    rotary_interleaved=interleaved, k_cache=kcd, v_cache=vcd,
+                                    token_to_chunk_idx=ci.to(dev), token_to_local_pos=lo.to(dev))
+        torch.cuda.synchronize()
+    finally:
+        mi.ops.set_tuning("norm_rope_vectorised", 2)
+    got_q = q_out.cpu().view(T, Hq, d)
+    err = (got_q.float() - q_ref.float()).abs()
+    assert torch.isfinite(got_q.float()).all()
+    assert (err <= 2e-2 + 2e-2 * q_ref.float().abs()).all(), f"q err {err.max().item()}"
+    # cache: rotated key rows (within tolerance) and raw value rows (bit-exact) at the right slots, -1 elsewhere
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    oa.kv_append(kc_ref, vc_ref, k_ref, v.squeeze(1), ci, lo)
+    gk, gv = kcd.cpu(), vcd.cpu()
+    assert torch.equal(gv.view(torch.int16), vc_ref.view(torch.int16)), "V cache differs"
+    errk = (gk.float() - kc_ref.float()).abs()
+    assert (errk <= 2e-2 + 2e-2 * kc_ref.float().abs()).all(), f"K cache err {errk.max().item()}"
+    untouched = torch.ones(N + 1, chunk, dtype=torch.bool)
+    untouched[ci, lo] = False
+    assert (gk[untouched] == -1).all(), "rows outside the appended slots changed"
+
+
+WRITE_KINDS = {"append": case_append, "append_fp8": case_append_fp8, "norm_rope": case_norm_rope}
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_random_append_cases_match_the_checker(mi, dev, block):
+    rejected = 0
+    for seed in range(70_000 + 60 * block, 70_000 + 60 * (block + 1)):
+        rng = random.Random(seed)
+        kind = rng.choice(["append", "append_fp8", "norm_rope", "norm_rope"])
+        try:
+            WRITE_KINDS[kind](mi, dev, rng, seed)
+        except ValueError as e:
+            # a key that is a strided view of the mixed projection is refused by the split-input entry point
+            assert "contiguous" in str(e), f"{_last_case[0]}: {e}"
+            rejected += 1
+        except AssertionError as e:
+            raise AssertionError(f"{_last_case[0]}: {e}") from None
+    assert rejected < 10
