@@ -1,11 +1,12 @@
 """GPU parity on seeded random cases: decode (bf16 / fp8 cache), prefill and mixed batches (bf16 / fp8),
 multi-latent decode, and the write side (scatter append in three dtypes, the quantising fp8 append of
 token runs, fused norm + rotary + append from split or mixed QKV input) -- random head counts, head
-widths, chunk sizes, lengths around every tile / chunk
-boundary, zero-length rows, strided query views, caches that are layer views of a bigger buffer, wider
-block tables, and random settings of the grid / tile / kernel-choice knobs -- each compared with the CPU
-checker at the bars of the dedicated tests (2e-2 abs/rel bf16; 2.5e-2 for an fp8 cache against the checker
-run on the same bytes).  A case outside what the kernels support must be rejected with an error, never
+widths, chunk sizes, lengths around every tile / chunk boundary, zero-length rows, strided query views,
+caches that are layer views of a bigger buffer, wider block tables, and random settings of the grid /
+tile / kernel-choice knobs -- each compared with the CPU checker at the bars of the dedicated tests
+(2e-2 abs/rel bf16; 2.5e-2 for an fp8 cache against the checker run on the same bytes; appended bytes
+bit-exact).  Before every call the device memory that the allocator is about to reuse is filled with NaN,
+so an output row or a partial result that a kernel leaves unwritten cannot pass.  A case outside what the kernels support must be rejected with an error, never
 computed wrongly.  The generator is seeded per case, so a failure names the seed that rebuilds it.
 """
 import random
