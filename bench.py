@@ -36,13 +36,110 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_226_800_000, "cfg4": 8_724_000_000, "cfg5": 9_070_100_000}
 
 
+# Single-kernel workloads for the rows built around the path (multi-latent decode, the tail of a step).
+SECONDARY_WORKLOADS = {
+    # name: (kind, parameters)
+    "mla_decode_h16": ("mla", dict(Hq=16, B=64, lo=512, hi=8192)),
+    "mla_decode_h128": ("mla", dict(Hq=128, B=64, lo=512, hi=8192)),
+    "mla_decode_h16_long": ("mla", dict(Hq=16, B=16, lo=65536, hi=65536)),
+    "mla_decode_h128_long": ("mla", dict(Hq=128, B=16, lo=65536, hi=65536)),
+    "sampling_top_k": ("sampling", dict(R=64, V=128256, top_k=50, top_p=0.0)),
+    "sampling_top_p": ("sampling", dict(R=64, V=128256, top_k=0, top_p=0.9)),
+    "sampling_greedy": ("sampling", dict(R=64, V=128256, top_k=1, top_p=0.0)),
+    "log_probs_bf16": ("log_probs", dict(T=4096, V=131072, bf16=True)),
+    "log_probs_fp32": ("log_probs", dict(T=4096, V=131072, bf16=False)),
+}
+
+
+def run_secondary(args, mi, lib, torch, dev):
+    """One kernel per step; HIP events on the launch stream around every call give the kernel time."""
+    kind, prm = SECONDARY_WORKLOADS[args.workload]
+    gen = torch.Generator().manual_seed(7)
+    flops = None
+    if kind == "mla":
+        Hq, B = prm["Hq"], prm["B"]
+        lens = torch.randint(prm["lo"], prm["hi"] + 1, (B,), generator=gen, dtype=torch.int32)
+        bt, N = mi.synthetic.build_block_table(lens, 256, gen)
+        cache = torch.empty(N + 1, 256, 576, dtype=torch.bfloat16, device=dev).normal_(0, 0.5)
+        q = torch.randn(B, 1, Hq, 576, device=dev).bfloat16()
+        lens_d, bt_d = lens.to(dev), bt.to(dev)
+        out = torch.empty(B, 1, Hq, 512, dtype=torch.bfloat16, device=dev)
+        step = lambda: mi.ops.paged_mla_decode_attention(q, cache, lens_d, bt_d, softmax_scale=0.072, out=out)
+        nbytes = int(lens.sum()) * 576 * 2 + B * Hq * (576 + 512) * 2 + int(((lens + 255) // 256).sum()) * 4 + B * 4
+        flops = int(lens.sum()) * Hq * (576 + 512) * 2
+        kernel = "paged_mla_decode_lds_kernel"
+        what = (f"absorbed multi-latent decode attention, {Hq} query heads, batch {B}, latent rows of 576 bf16, "
+                f"context U[{prm['lo']},{prm['hi']}], chunk 256")
+        dtype = "bf16 (fp32 accumulate)"
+        timed_by_library = True
+    elif kind == "sampling":
+        R, V = prm["R"], prm["V"]
+        logits = (torch.randn(R, V, generator=gen) * 3).to(dev)
+        u = torch.rand(R, generator=gen).to(dev)
+        step = lambda: mi.ops.sample_from_logits(logits, top_k=prm["top_k"], top_p=prm["top_p"], temperature=0.8,
+                                                 uniform=u)
+        nbytes = R * V * 4 + R * 12
+        kernel = "sample_kernel"
+        what = f"sampling of {R} rows of {V} fp32 logits, top_k {prm['top_k']}, top_p {prm['top_p']}, temperature 0.8"
+        dtype = "fp32 logits, 2^-32 fixed-point mass"
+        timed_by_library = False
+    else:
+        T, V = prm["T"], prm["V"]
+        logits = torch.empty(T, V, dtype=torch.bfloat16 if prm["bf16"] else torch.float32, device=dev).normal_(0, 3)
+        ids = torch.randint(0, V, (T,), generator=gen).to(dev)
+        step = lambda: mi.ops.selected_log_probs(logits, ids)
+        nbytes = T * V * logits.element_size() + T * 12
+        kernel = "selected_log_probs_kernel"
+        what = f"log-probabilities of the chosen tokens, {T} rows of {V} {'bf16' if prm['bf16'] else 'fp32'} logits"
+        dtype = "fp32 accumulation"
+        timed_by_library = False
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    if timed_by_library:
+        lib.mi_profile_enable(1)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in events:
+        a.record()   # (these ops launch on torch's current stream, which is the stream the events see)
+        step()
+        b.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    call_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    kernel_ms = call_ms
+    if timed_by_library:
+        buf = (ctypes.c_float * args.steps)()
+        n_ev = lib.mi_profile_collect(buf, args.steps)
+        lib.mi_profile_enable(0)
+        kernel_ms = sum(buf[i] for i in range(min(n_ev, args.steps))) / max(1, min(n_ev, args.steps))
+    ms_per_step = elapsed * 1e3 / args.steps
+    mfma_bound = kind == "mla" and prm["Hq"] >= 64
+    roofline = ({"bound": "mfma", "kernel": kernel, "achieved": round(flops / kernel_ms / 1e9, 1),
+                 "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                 "frac": round(flops / kernel_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)} if mfma_bound else
+                {"bound": "hbm", "kernel": kernel, "achieved": round(nbytes / kernel_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                 "unit": "GB/s", "frac": round(nbytes / kernel_ms / 1e6 / HBM_PEAK_GBPS, 4)})
+    roofline.update({"kernel_ms": round(kernel_ms, 5), "traffic": None})
+    print(json.dumps({
+        "metric": f"{args.workload}_GBps", "value": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": what, "algorithmic_bytes_per_step": nbytes, "flops_per_step": flops,
+                   "call_ms_by_events": round(call_ms, 5)},
+        "roofline": roofline}), flush=True)
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5"],
-                    help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch")
+    ap.add_argument("--workload", default="cfg2",
+                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", *SECONDARY_WORKLOADS],
+                    help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch; the "
+                         "mla_* / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
     ap.add_argument("--split-tokens", type=int, default=0)
     ap.add_argument("--subtiles", type=int, default=0, help="16-token sub-tiles per loop iteration (1, 2 or 4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -211,6 +308,9 @@ def main():
 
     if args.workload == "cfg3":
         run_mixed_batch(args, mi, lib, torch, dev)
+        return
+    if args.workload in SECONDARY_WORKLOADS:
+        run_secondary(args, mi, lib, torch, dev)
         return
 
     cfg = mi.synthetic.CONFIGS[args.workload]
