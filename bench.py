@@ -33,7 +33,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 # this same script, each counter scaled by what it reads for a plain 1 GiB device copy
 # (profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md).  Hardware counters cannot be
 # read from inside the benchmark, so the figure is recorded here per workload; None = not collected.
-MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_226_800_000, "cfg4": 8_724_000_000, "cfg5": 9_070_100_000}
+MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_226_800_000, "cfg4": 8_724_000_000, "cfg5": 9_070_100_000,
+                              # the mixed step (profiles/paged_prefill_pp_kernel_cfg3_mfma.md): tile kernel, stream kernel
+                              "cfg3_tile": 402_300_000, "cfg3_stream": 2_195_700_000}
 
 
 # Single-kernel workloads for the rows built around the path (multi-latent decode, the tail of a step).
@@ -234,6 +236,13 @@ def run_mixed_batch(args, mi, lib, torch, dev):
         mi.ops.paged_prefill_attention(q_rot, kc, vc, cu_q, lens, bt, max_kv_len=max_len, out=out,
                                        k_scales=ks, v_scales=vs)
 
+    if args.calibrate_copy_mib:  # a copy of known size for scaling an external profiler's traffic counters
+        src = torch.empty(args.calibrate_copy_mib << 20, dtype=torch.uint8, device=dev).random_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -274,11 +283,12 @@ def run_mixed_batch(args, mi, lib, torch, dev):
         "roofline": {"bound": "mfma", "kernel": "paged_prefill_pp_kernel", "achieved": round(flops / tile_ms / 1e9, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / tile_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "kernel_ms": round(tile_ms, 5),
-                     "traffic": None},
+                     "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_tile"]},
         "roofline_decode_part": {"bound": "hbm", "kernel": "paged_decode_stream_kernel",
                                  "achieved": round(dec_bytes / stream_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
                                  "unit": "GB/s", "frac": round(dec_bytes / stream_ms / 1e6 / HBM_PEAK_GBPS, 4),
-                                 "kernel_ms": round(stream_ms, 5), "traffic": None},
+                                 "kernel_ms": round(stream_ms, 5),
+                                 "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_stream"]},
     }
     print(json.dumps(result), flush=True)
 
