@@ -151,7 +151,7 @@ int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t he
  * q/out: bf16 `[R, Hq, d]` with the given token / head strides.  kv_lens int32 [R]
  * (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] (the reference
  * passes max_sequence_length here, dynamic_context.py:791); the grid does not depend on
- * it.  `split_tokens` = minimum tokens one workgroup streams (0 = default 256).
+ * it.  `split_tokens` = minimum tokens one workgroup streams (0 = default 64).
  * kv_dtype MI_KV_FP8_E4M3 reads byte caches with k_scales/v_scales `[n_chunks, Hkv]`.
  */
 int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_head,

@@ -894,7 +894,9 @@ int mi::launch_paged_decode(
   while (chunk_tokens % (16 * nt)) nt >>= 1;  // a tile must not straddle two chunks
   const int minw = mi_tuning().decode_min_waves;
   const int tk = 16 * nt;
-  const int min_span_tokens = split_tokens > 0 ? split_tokens : 256;
+  // a small batch is cut finer than a large one needs: 64 tokens per workgroup put a single 8 192-token
+  // request on 128 CUs (17.8 us against 33 us with 256-token spans); large batches get equal spans anyway
+  const int min_span_tokens = split_tokens > 0 ? split_tokens : 64;
 
   DecodeParams p;
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
@@ -1048,7 +1050,7 @@ extern "C" int mi_paged_mla_decode_attention(
   p.k_scale = nullptr; p.v_scale = nullptr;
   p.R = R; p.Hq = Hq; p.Hkv = groups; p.G = Hq < 16 ? Hq : 16; p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
-  p.min_span_tiles = shared_tile ? 256 / kMlaTile : 256 / 16;
+  p.min_span_tiles = shared_tile ? 64 / kMlaTile : 64 / 16;
   p.grid = grid_x;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
 
