@@ -54,6 +54,8 @@ const char* mi_last_error(void);
  * "prefill_tile_subtiles", "prefill_lds_row_tiles", "prefill_row_tiles" (the older kernels),
  * "norm_rope_vectorised" (16-byte-per-lane norm / rotary kernel: 1 = wherever alignment and the rotary
  * width allow it, 2 = the same but only from 256 tokens up (default), 0 = element-wise kernel always),
+ * "prefill_kv_split" (key ranges per request in the head_dim-128 tile kernel: 1 = chosen from T and
+ * max_kv_len (default), 0 = never, 2..64 = forced where the workspace allows it),
  * "mla_decode_lds" (multi-latent decode: 1 = latent tiles shared through LDS by the wavefronts of a
  * workgroup when the chunk size is a multiple of 64 and at most 768 requests are in the call (default),
  * 0 = one streaming wavefront per 16-head group always). */
@@ -197,6 +199,12 @@ int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q
  * padding) are zeroed.  With a workspace of mi_prefill_workspace_bytes() bytes, requests that
  * have exactly one query row (the decode requests of a mixed batch) are streamed by the
  * decode kernels at full bandwidth; with workspace == NULL one kernel handles every request.
+ * The same workspace lets the head_dim-128 tile kernel cut the keys of every request into ranges when
+ * the batch has few query rows over long contexts (a chunk of a prompt, a short turn after a long
+ * history: without it a handful of workgroups would walk thousands of keys each): the ranges are
+ * computed by separate workgroups and merged by log-sum-exp, as in the decode path.  `max_kv_len` (an
+ * upper bound of kv_lens; 0 = unknown, no splitting) and T decide the number of ranges, so pass the same
+ * values to mi_prefill_workspace_bytes and to the attention call.
  */
 int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                    int32_t max_kv_len, int32_t split_tokens);

@@ -30,7 +30,8 @@ MiTuning& mi_tuning() {
                       env_int("MI355_DECODE_MIN_WAVES", 3),
                       env_int("MI355_DECODE_WGS_PER_CU", 1), env_int("MI355_DECODE_GRID", 0),
                       env_int("MI355_DECODE_WAVES_PER_BLOCK", 8), env_int("MI355_NORM_ROPE_VECTORISED", 2),
-                      env_int("MI355_MLA_DECODE_LDS", 1), env_int("MI355_PREFILL_PINGPONG", 1)};
+                      env_int("MI355_MLA_DECODE_LDS", 1), env_int("MI355_PREFILL_KV_SPLIT", 1),
+                      env_int("MI355_PREFILL_PINGPONG", 1)};
   return t;
 }
 
@@ -83,6 +84,11 @@ extern "C" int mi_set_tuning(const char* name, int32_t value) {
   if (!strcmp(name, "prefill_pingpong")) {
     if (value < 0 || value > 2) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_pingpong must be 0, 1 or 2");
     mi_tuning().prefill_pingpong = value;
+    return MI_OK;
+  }
+  if (!strcmp(name, "prefill_kv_split")) {
+    if (value < 0 || value > 64) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_kv_split must be 0 (never), 1 (automatic) or 2..64");
+    mi_tuning().prefill_kv_split = value;
     return MI_OK;
   }
   if (!strcmp(name, "mla_decode_lds")) {

@@ -33,6 +33,7 @@ struct MiTuning {
   int decode_waves_per_block;  // cap on wavefronts (= KV heads) per decode workgroup, 1..8
   int norm_rope_vectorised;    // 16-byte-per-lane norm/RoPE kernel: 1 = whenever shapes allow, 2 = and T >= 256 (default), 0 = never
   int mla_decode_lds;          // MLA decode: 1 = latent tile shared through LDS when the chunk size allows, 0 = per-wavefront streaming
+  int prefill_kv_split;        // two-phase prefill kernel: key ranges per request, 1 = automatic (default), 0 = never, n > 1 = forced
   int prefill_pingpong;        // head_dim-128 prefill: 1 = two wave groups one phase apart, 2 = same kernel in lock-step, 0 = off
 };
 

@@ -43,6 +43,11 @@ struct PrefillParams {
   float scale_log2;
   const float* k_scale;  // fp8 KV only: [n_chunks][Hkv]
   const float* v_scale;
+  // Two-phase tile kernel only: the keys of a request cut into gridDim.y ranges, one workgroup each;
+  // with more than one range the workgroups write fp32 partials [range][T][Hq][128] and their
+  // log-sum-exps [range][T][Hq] (log2 domain) and a merge kernel finishes the rows.
+  float* split_o;
+  float* split_lse;
 };
 
 // NQ = 16-row tiles per wave; a workgroup always covers 256 rows (16 / NQ waves).
@@ -599,7 +604,9 @@ constexpr int kPPTile = 64;   // keys per staged tile
 
 // FP8: the cache holds e4m3 bytes with one fp32 scale per (chunk, KV head); a piece is multiplied by
 // its chunk's scale and rounded to bf16 on its way into LDS, so both matrix phases are the bf16 ones.
-template <bool STAGGER, bool FP8>
+// SPLIT: the keys of a request are cut into gridDim.y ranges (a separate instantiation, so that the
+// ordinary kernel carries no tile offsets).
+template <bool STAGGER, bool FP8, bool SPLIT = false>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
   constexpr int HD = 128, KS = 4, DV = 8, NQ = 2, NT = 4, WAVES = 8;
   constexpr int ESZ = FP8 ? 1 : 2;       // bytes per cache element
@@ -618,7 +625,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   const int BQ = (16 * NQ) >> p.g_shift;
   const int SBQ = WAVES * BQ;
 
-  if (rank == 0) {
+  if (rank == 0 && (!SPLIT || blockIdx.y == 0)) {
     const int tq = p.cu_q[p.R];
     const int per_row = G * HD;
     for (int64_t i = (int64_t)tid * 8; i < (int64_t)(p.T - tq) * per_row; i += 512 * 8) {
@@ -643,7 +650,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   const int shift = Lk - Lq;
   const int last = Lk - 1;
   const int kend_wg = min(Lk, shift + min(q0_wg + SBQ, Lq));
-  const int ntl = (kend_wg + kPPTile - 1) / kPPTile;  // staged tiles of this workgroup
+  const int ntl_all = (kend_wg + kPPTile - 1) / kPPTile;  // staged tiles the rows of this workgroup can see
+  // this workgroup's share of them: tiles [tb, tb + ntl)
+  const int n_split = SPLIT ? (int)gridDim.y : 1, split = SPLIT ? (int)blockIdx.y : 0;
+  const int tb = SPLIT ? (int)((int64_t)ntl_all * split / n_split) : 0;
+  const int te = SPLIT ? (int)((int64_t)ntl_all * (split + 1) / n_split) : ntl_all;
+  const int ntl = te - tb;
 
   const int q0 = q0_wg + wave * BQ;
   const int nq = max(0, min(BQ, Lq - q0));
@@ -703,14 +715,14 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     };
     auto cursor_at = [&](int t) {
       Cursor c;
-      c.tile = min(t, ntl - 1);
+      c.tile = min(t, te - 1);
       c.ci = c.tile / tiles_per_chunk;
       c.tin = c.tile - c.ci * tiles_per_chunk;
       c.room = (last - c.tile * kPPTile) * tok_bytes;
       return c;
     };
     auto cursor_next = [&](Cursor& c) {  // one tile forward, sticking to the last tile
-      const bool adv = c.tile + 1 < ntl;
+      const bool adv = c.tile + 1 < te;
       const bool wrap = adv && (c.tin + 1 == tiles_per_chunk);
       c.tile += adv ? 1 : 0;
       c.room -= adv ? tile_bytes : 0;
@@ -823,7 +835,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // LDS, then fetch K(it+2) and V(it+2).  (Reading fragments ahead during the vector phase, or
     // moving score groups there, was measured slower: a wave sustains only ~32 B/clk of LDS reads
     // and the vector phase has no issue slots to spare.)
-    Cursor cur = cursor_at(2);  // the tile fetched during iteration 0
+    Cursor cur = cursor_at(tb + 2);  // the tile fetched during iteration 0
     int pc_cur = 0;             // its block-table entry (a per-lane copy, made scalar at its use)
     auto matrix_phase = [&](int it) {
       uint2 a0[4][2], a1[4][2];
@@ -859,8 +871,8 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       sc_mma(3, k1);
     };
     // ---- online softmax of tile t: s -> pf, rescale of the accumulators when a maximum moved ----
-    auto softmax = [&](int t) {
-      const int T = t * kPPTile;
+    auto softmax = [&](int t) {  // t counts from this workgroup's first tile
+      const int T = (tb + t) * kPPTile;
       const bool need_mask = T + kPPTile - 1 > full_until;
 #pragma unroll
       for (int nt = 0; nt < NQ; ++nt) {
@@ -918,7 +930,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     for (int i = tid * 16; i < kPPTile * kVPitch; i += 512 * 16)
       *reinterpret_cast<uint4*>(&Vs[2][i]) = make_uint4(0u, 0u, 0u, 0u);  // "tile -1"
     {
-      const Cursor c0 = cursor_at(0), c1 = cursor_at(1);
+      const Cursor c0 = cursor_at(tb), c1 = cursor_at(tb + 1);
       const int64_t off0 = tile_offset(c0, bt_row[c0.ci]);
       tile_loads(kbase, off0, c0.room, kreg);
       tile_loads(vbase, off0, c0.room, vreg);
@@ -962,27 +974,95 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     const int n = 16 * nt + m16;
     const int qi = n >> p.g_shift, u = n & (G - 1);
     if (qi < nq) {
-      uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * g;
+      if (!SPLIT) {
+        uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * g;
 #pragma unroll
-      for (int e = 0; e < DV; ++e)
-        st8(o + 16 * e, make_uint2(pack_bf16x2(acc[nt][e][0] * inv, acc[nt][e][1] * inv),
-                                   pack_bf16x2(acc[nt][e][2] * inv, acc[nt][e][3] * inv)));
+        for (int e = 0; e < DV; ++e)
+          st8(o + 16 * e, make_uint2(pack_bf16x2(acc[nt][e][0] * inv, acc[nt][e][1] * inv),
+                                     pack_bf16x2(acc[nt][e][2] * inv, acc[nt][e][3] * inv)));
+      } else {  // a range without visible keys (none for short requests) leaves zeros and -inf
+        const int64_t prow = ((int64_t)split * p.T + (q_begin + q0 + qi)) * p.Hq + (h * G + u);
+        float* o = p.split_o + prow * HD + 4 * g;
+#pragma unroll
+        for (int e = 0; e < DV; ++e)
+          *reinterpret_cast<float4*>(o + 16 * e) =
+              make_float4(acc[nt][e][0] * inv, acc[nt][e][1] * inv, acc[nt][e][2] * inv, acc[nt][e][3] * inv);
+        if (g == 0) p.split_lse[prow] = l_tot > 0.f ? m_run[nt] * p.scale_log2 + fast_log2(l_tot) : -INFINITY;
+      }
     }
   }
 }
 
+// Rows whose keys were split over several workgroups: o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max).
+// Grid (T, Hq), 128 threads = the output values of one (row, head).
+__global__ __launch_bounds__(128) void prefill_split_merge_kernel(PrefillParams p, int n_split) {
+  const int row = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
+  if (row >= p.cu_q[p.R]) return;  // padding rows: zeroed by the tile kernel
+  if (p.skip_single) {             // one-row requests were left to the decode kernels
+    int lo = 0, hi = p.R - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (p.cu_q[mid] <= row) lo = mid; else hi = mid - 1;
+    }
+    if (p.cu_q[lo + 1] - p.cu_q[lo] == 1) return;
+  }
+  float mx = -INFINITY, num = 0.f, den = 0.f;
+  for (int s0 = 0; s0 < n_split; s0 += 8) {
+    float lse[8], po[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int64_t prow = ((int64_t)min(s0 + j, n_split - 1) * p.T + row) * p.Hq + head;
+      lse[j] = p.split_lse[prow];
+      po[j] = p.split_o[prow * 128 + d];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (s0 + j < n_split && lse[j] != -INFINITY) {
+        const float m_new = fmaxf(mx, lse[j]);
+        const float a = fast_exp2(mx - m_new), wt = fast_exp2(lse[j] - m_new);
+        num = num * a + wt * po[j];
+        den = den * a + wt;
+        mx = m_new;
+      }
+    }
+  }
+  p.out[(int64_t)row * p.o_st + (int64_t)head * p.o_sh + d] = f32_to_bf16(den > 0.f ? num / den : 0.f);
+}
 
 }  // namespace mi
 
 using namespace mi;
 
+// Ranges the keys of every request are cut into by the two-phase tile kernel.  Few query rows over a
+// long context (a chunk of a prompt, a short turn after a long history) give few workgroups, each
+// with thousands of keys to walk: then the keys are split so that about one workgroup per CU exists,
+// every one keeping at least sixteen 64-key tiles (a 512-token prompt is not worth the merge).  Host-side quantities only (the lengths live on the GPU).
+static int prefill_kv_splits(int T, int Hq, int Hkv, int head_dim, int max_kv_len) {
+  if (head_dim != 128 || max_kv_len <= 0) return 1;
+  const int G = Hq / Hkv;
+  const int sbq = 256 / G;                               // query tokens per workgroup
+  const int64_t useful = (int64_t)Hkv * ((T + sbq - 1) / sbq);
+  const int cus = 256;
+  if (useful >= cus) return 1;
+  int64_t s = (cus + useful - 1) / useful;
+  const int64_t by_tiles = ((int64_t)max_kv_len + 63) / 64 / 16;
+  if (s > by_tiles) s = by_tiles;
+  if (s > 32) s = 32;  // (more ranges cost more in partials than they win: 64 rows over 131 072 keys, 16-32 is best)
+  return s < 2 ? 1 : (int)s;
+}
+
 extern "C" int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
                                               int32_t head_dim, int32_t max_kv_len,
                                               int32_t split_tokens) {
-  (void)T;
-  // Only the one-row (decode) requests of a mixed batch need scratch: they are streamed by the
-  // decode kernels, whose partials live here.
-  return mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens);
+  // The one-row (decode) requests of a mixed batch are streamed by the decode kernels, whose partials
+  // live here; behind them the partials of the tile kernel when it splits the keys.
+  int64_t bytes = mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens);
+  bytes = (bytes + 255) & ~(int64_t)255;
+  if (T > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0) {
+    const int s = prefill_kv_splits(T, Hq, Hkv, head_dim, max_kv_len);
+    if (s > 1) bytes += (int64_t)s * T * Hq * (head_dim + 1) * (int64_t)sizeof(float);
+  }
+  return bytes;
 }
 
 static int launch_paged_prefill(
@@ -991,7 +1071,7 @@ static int launch_paged_prefill(
     const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seqlens_q,
     const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head,
     void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
-    int32_t head_dim, int32_t chunk_tokens, int32_t split_tokens, float softmax_scale,
+    int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens, float softmax_scale,
     int32_t kv_dtype, const float* k_scales, const float* v_scales, void* stream) {
   const bool fp8 = kv_dtype == MI_KV_FP8_E4M3;
   if (T == 0 || R == 0) return MI_OK;
@@ -1038,6 +1118,7 @@ static int launch_paged_prefill(
   // With a workspace, one-row requests go through the bandwidth-optimised decode kernels.
   p.skip_single = workspace != nullptr;
   p.k_scale = k_scales; p.v_scale = v_scales;
+  p.split_o = nullptr; p.split_lse = nullptr;
 
   hipStream_t st = (hipStream_t)stream;
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
@@ -1051,7 +1132,27 @@ static int launch_paged_prefill(
     const bool timed = mi_profile_next(&ev_a, &ev_b);
     if (timed) (void)hipEventRecord(ev_a, st);
     const int pp = (chunk_tokens % 64 == 0) ? mi_tuning().prefill_pingpong : 0;  // staged tiles must not straddle chunks
-    if (fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true>), lgrid, dim3(512), 0, st, p);
+    // key ranges per request (two-phase kernel with a workspace only): partials behind the decode part's scratch
+    int n_split = 1;
+    if (pp != 0 && workspace && mi_tuning().prefill_kv_split != 0) {
+      n_split = mi_tuning().prefill_kv_split > 1 ? mi_tuning().prefill_kv_split
+                                                 : prefill_kv_splits(T, Hq, Hkv, head_dim, max_kv_len);
+      const int64_t dec_bytes = (mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens) + 255) &
+                                ~(int64_t)255;
+      const int64_t sp_bytes = (int64_t)n_split * T * Hq * (head_dim + 1) * (int64_t)sizeof(float);
+      if (n_split > 1 && workspace_bytes < dec_bytes + sp_bytes) n_split = 1;  // (a caller-sized workspace of the older layout)
+      if (n_split > 1) {
+        p.split_o = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + dec_bytes);
+        p.split_lse = p.split_o + (int64_t)n_split * T * Hq * head_dim;
+        lgrid.y = n_split;
+        workspace_bytes = dec_bytes;
+      }
+    }
+    if (n_split > 1 && fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true, true>), lgrid, dim3(512), 0, st, p);
+    else if (n_split > 1 && fp8) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, true, true>), lgrid, dim3(512), 0, st, p);
+    else if (n_split > 1 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, true>), lgrid, dim3(512), 0, st, p);
+    else if (n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, true>), lgrid, dim3(512), 0, st, p);
+    else if (fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true>), lgrid, dim3(512), 0, st, p);
     else if (fp8) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, true>), lgrid, dim3(512), 0, st, p);
     else if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false>), lgrid, dim3(512), 0, st, p);
     else if (pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false>), lgrid, dim3(512), 0, st, p);
@@ -1059,6 +1160,7 @@ static int launch_paged_prefill(
     else if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 2>), lgrid, dim3(512), 0, st, p);
     else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);  // (48 rows: 32-key tiles only)
     if (timed) (void)hipEventRecord(ev_b, st);
+    if (n_split > 1) hipLaunchKernelGGL(prefill_split_merge_kernel, dim3(T, Hq), dim3(128), 0, st, p, n_split);
     int rc0 = mi_check_launch("mi_paged_prefill_attention");
     if (rc0 != MI_OK || !p.skip_single) return rc0;
     return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
@@ -1100,11 +1202,10 @@ extern "C" int mi_paged_prefill_attention(
     void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
     int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
     float softmax_scale, void* stream) {
-  (void)max_kv_len;
   return launch_paged_prefill(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
                               kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out, o_stride_tok,
                               o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim, chunk_tokens,
-                              split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
+                              max_kv_len, split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
 }
 
 extern "C" int mi_paged_prefill_attention_fp8(
@@ -1115,11 +1216,11 @@ extern "C" int mi_paged_prefill_attention_fp8(
     int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq,
     int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
     float softmax_scale, void* stream) {
-  (void)max_kv_len;
   return launch_paged_prefill(q, q_stride_tok, q_stride_head, k_cache_fp8, v_cache_fp8, kv_stride_chunk,
                               kv_stride_tok, kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out,
                               o_stride_tok, o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim,
-                              chunk_tokens, split_tokens, softmax_scale, MI_KV_FP8_E4M3, k_scales, v_scales, stream);
+                              chunk_tokens, max_kv_len, split_tokens, softmax_scale, MI_KV_FP8_E4M3, k_scales, v_scales,
+                              stream);
 }
 
 extern "C" int mi_paged_prefill_attention_mla(

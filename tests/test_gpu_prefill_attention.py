@@ -149,3 +149,65 @@ def test_chunked_prefill_is_consistent_at_full_size(mi, dev):
     moved = mi.ops.paged_prefill_attention(q, kc_p, vc_p, cu_q, lens, bt_p, max_kv_len=int(lens.max()))
     torch.cuda.synchronize()
     assert torch.equal(moved, full)
+
+
+@pytest.mark.parametrize("forced", [1, 2, 7, 64])
+def test_few_rows_over_long_contexts_split_the_keys(mi, dev, forced):
+    """A chunk of a prompt (or a short turn) over a long cached context: the tile kernel cuts the keys of
+    every request into ranges (automatic = knob 1, or a forced count), writes partials and merges them.
+    Requests shorter than the number of ranges get empty ranges; one-token requests go the decode way."""
+    q_lens = [96, 1, 40, 1, 7]
+    ctx = [9000, 4000, 130, 0, 63]
+    Hq, Hkv, d, chunk = 32, 8, 128, 64
+    kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    gen = torch.Generator().manual_seed(31)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, gen)
+    q = torch.randn(int(cu_q[-1]), Hq, d, generator=gen).bfloat16().to(dev)
+    kc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
+    vc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
+    mi.ops.set_tuning("prefill_kv_split", forced)
+    try:
+        _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
+        split = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev),
+                                               max_kv_len=int(kv_lens.max()))
+        mi.ops.set_tuning("prefill_kv_split", 0)
+        whole = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev),
+                                               max_kv_len=int(kv_lens.max()))
+        torch.cuda.synchronize()
+        assert (split.float() - whole.float()).abs().max().item() <= 1e-2   # same arithmetic, another summation order
+    finally:
+        mi.ops.set_tuning("prefill_kv_split", 1)
+
+
+def test_split_keys_with_padding_rows_and_fp8(mi, dev):
+    """Padding rows behind the last request stay zero; the fp8 cache takes the same split path."""
+    q_lens, ctx = [50, 3], [5000, 2000]
+    Hq, Hkv, d, chunk = 16, 2, 128, 128
+    kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.tensor([0, 50, 53], dtype=torch.int32)
+    gen = torch.Generator().manual_seed(32)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, gen)
+    T = 53 + 11                                                   # 11 padding rows
+    q = torch.randn(T, Hq, d, generator=gen).bfloat16().to(dev)
+    kc = (torch.randn(N, chunk, Hkv, d, generator=gen) * 0.7).bfloat16().to(dev)
+    vc = (torch.randn(N, chunk, Hkv, d, generator=gen) * 0.7).bfloat16().to(dev)
+    out = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev), max_kv_len=int(kv_lens.max()))
+    torch.cuda.synchronize()
+    assert (out[53:] == 0).all()
+    ref = oa.paged_varlen_attention(q[:53].cpu(), kc.cpu(), vc.cpu(), cu_q, kv_lens, bt)
+    err = (out[:53].float().cpu() - ref).abs()
+    assert (err <= 2e-2 + 2e-2 * ref.abs()).all()
+    k8 = torch.empty(kc.shape, dtype=torch.uint8, device=dev)
+    v8 = torch.empty_like(k8)
+    ks = torch.empty(N, Hkv, dtype=torch.float32, device=dev)
+    vs = torch.empty_like(ks)
+    mi.ops.quantize_chunks_fp8(kc, k8, ks)
+    mi.ops.quantize_chunks_fp8(vc, v8, vs)
+    out8 = mi.ops.paged_prefill_attention(q, k8, v8, cu_q.to(dev), kv_lens.to(dev), bt.to(dev), max_kv_len=int(kv_lens.max()),
+                                          k_scales=ks, v_scales=vs)
+    torch.cuda.synchronize()
+    ref8 = oa.paged_varlen_attention(q[:53].cpu(), k8.cpu(), v8.cpu(), cu_q, kv_lens, bt, k_scales=ks.cpu(), v_scales=vs.cpu())
+    err8 = (out8[:53].float().cpu() - ref8).abs()
+    assert (err8 <= 2.5e-2 + 2.5e-2 * ref8.abs()).all() and (out8[53:] == 0).all()
