@@ -1059,7 +1059,8 @@ extern "C" int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, 
   int64_t bytes = mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens);
   bytes = (bytes + 255) & ~(int64_t)255;
   if (T > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0) {
-    const int s = prefill_kv_splits(T, Hq, Hkv, head_dim, max_kv_len);
+    const int knob = mi_tuning().prefill_kv_split;  // (a forced count is honoured here too)
+    const int s = knob > 1 ? knob : knob == 1 ? prefill_kv_splits(T, Hq, Hkv, head_dim, max_kv_len) : 1;
     if (s > 1) bytes += (int64_t)s * T * Hq * (head_dim + 1) * (int64_t)sizeof(float);
   }
   return bytes;

@@ -146,7 +146,9 @@ def case_prefill(mi, dev, rng, seed, fp8):
     if sum(q_lens) == 0:
         q_lens[0] = 3
     pp = rng.choice([1, 1, 2, 0])
-    _note(f"prefill fp8={fp8} seed={seed} d={d} Hq={Hq} Hkv={Hkv} chunk={chunk} q_lens={q_lens} ctx={ctx} pingpong={pp}")
+    ksplit = rng.choice([1, 1, 0, 3, 8])  # key ranges per request in the tile kernel (1 = automatic)
+    _note(f"prefill fp8={fp8} seed={seed} d={d} Hq={Hq} Hkv={Hkv} chunk={chunk} q_lens={q_lens} ctx={ctx} pingpong={pp} "
+          f"kv_split={ksplit}")
     kv_lens = torch.tensor([a + b if a else 0 for a, b in zip(q_lens, ctx)], dtype=torch.int32)
     cu_q = torch.zeros(R + 1, dtype=torch.int32)
     cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
@@ -156,6 +158,7 @@ def case_prefill(mi, dev, rng, seed, fp8):
     kc = (torch.randn(N + 1, chunk, Hkv, d, generator=gen) * 0.7).bfloat16()
     vc = (torch.randn(N + 1, chunk, Hkv, d, generator=gen) * 0.7).bfloat16()
     mi.ops.set_tuning("prefill_pingpong", pp)
+    mi.ops.set_tuning("prefill_kv_split", ksplit)
     try:
         if fp8:
             k8 = torch.empty(kc.shape, dtype=torch.uint8, device=dev)
@@ -180,6 +183,7 @@ def case_prefill(mi, dev, rng, seed, fp8):
             close(out, ref, 2e-2, "prefill")
     finally:
         mi.ops.set_tuning("prefill_pingpong", 1)
+        mi.ops.set_tuning("prefill_kv_split", 1)
 
 
 def case_mla_decode(mi, dev, rng, seed):
