@@ -54,7 +54,7 @@ const char* mi_last_error(void);
  * "prefill_tile_subtiles", "prefill_lds_row_tiles", "prefill_row_tiles" (the older kernels),
  * "norm_rope_vectorised" (16-byte-per-lane norm / rotary kernel: 1 = wherever alignment and the rotary
  * width allow it, 2 = the same but only from 256 tokens up (default), 0 = element-wise kernel always),
- * "prefill_kv_split" (key ranges per request in the head_dim-128 tile kernel: 1 = chosen from T and
+ * "prefill_kv_split" (key ranges per request in the two-phase tile kernel: 1 = chosen from T and
  * max_kv_len (default), 0 = never, 2..64 = forced where the workspace allows it),
  * "mla_decode_lds" (multi-latent decode: 1 = latent tiles shared through LDS by the wavefronts of a
  * workgroup when the chunk size is a multiple of 64 and at most 768 requests are in the call (default),
@@ -63,7 +63,7 @@ int mi_set_tuning(const char* name, int32_t value);
 
 /*
  * Kernel timing.  mi_profile_enable(1) makes the attention entry points bracket their main
- * kernel (decode: the KV-streaming kernel; prefill, head_dim 128: the tile kernel, followed by
+ * kernel (decode: the KV-streaming kernel; prefill, head_dim 128 or 64 with a chunk size that is a multiple of 64: the tile kernel, followed by
  * a second pair for the decode kernel of a mixed batch) with HIP events on the caller's
  * stream; mi_profile_collect waits for
  * the recorded pairs, writes their durations (milliseconds, HOST pointer) and returns how
@@ -199,7 +199,7 @@ int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q
  * padding) are zeroed.  With a workspace of mi_prefill_workspace_bytes() bytes, requests that
  * have exactly one query row (the decode requests of a mixed batch) are streamed by the
  * decode kernels at full bandwidth; with workspace == NULL one kernel handles every request.
- * The same workspace lets the head_dim-128 tile kernel cut the keys of every request into ranges when
+ * The same workspace lets the two-phase tile kernel (head_dim 128 or 64, chunk size a multiple of 64) cut the keys of every request into ranges when
  * the batch has few query rows over long contexts (a chunk of a prompt, a short turn after a long
  * history: without it a handful of workgroups would walk thousands of keys each): the ranges are
  * computed by separate workgroups and merged by log-sum-exp, as in the decode path.  `max_kv_len` (an

@@ -598,17 +598,25 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
 // accumulated by the matrix cores (an all-ones A fragment), and the cross-lane maximum uses the
 // lane-swap instructions instead of LDS permutes.
 // ---------------------------------------------------------------------------------------------
-constexpr int kKPitch = 288;  // bytes per staged K row: measured conflict-free for the 16-row x 64-byte fragment reads (272 is not)
-constexpr int kVPitch = 288;  // bytes per staged V row: 16 rows x 32 B tile the banks twice
+// bytes per staged K / V row.  head_dim 128: 288, measured conflict-free for the 16-row x 64-byte fragment
+// reads (272 is not), and 16 rows x 32 B of the transposing reads tile the banks twice; head_dim 64: 144
+// (36 dwords: the 16 rows of a fragment read start at 16 different multiples of four banks).
+template <int HD> constexpr int pp_pitch() { return HD == 128 ? 288 : 144; }
 constexpr int kPPTile = 64;   // keys per staged tile
 
 // FP8: the cache holds e4m3 bytes with one fp32 scale per (chunk, KV head); a piece is multiplied by
 // its chunk's scale and rounded to bf16 on its way into LDS, so both matrix phases are the bf16 ones.
 // SPLIT: the keys of a request are cut into gridDim.y ranges (a separate instantiation, so that the
 // ordinary kernel carries no tile offsets).
-template <bool STAGGER, bool FP8, bool SPLIT = false>
+template <bool STAGGER, bool FP8, bool SPLIT = false, int HD = 128>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
-  constexpr int HD = 128, KS = 4, DV = 8, NQ = 2, NT = 4, WAVES = 8;
+  static_assert(HD == 128 || (HD == 64 && !FP8), "head_dim 128, or 64 with a bf16 cache");
+  constexpr int KS = HD / 32, DV = HD / 16, NQ = 2, NT = 4, WAVES = 8;
+  constexpr int kKPitch = pp_pitch<HD>(), kVPitch = pp_pitch<HD>();
+  constexpr int PPR = HD * 2 / 16;       // 16-byte pieces (8 elements) per key row: 16 | 8
+  constexpr int RPP = 512 / PPR;         // key rows the 512 loader threads cover in one pass: 32 | 64
+  constexpr int NPASS = kPPTile / RPP;   // passes (rows per thread) per tile: 2 | 1
+  constexpr int NH = HD / 64;            // 64-column halves of the output
   constexpr int ESZ = FP8 ? 1 : 2;       // bytes per cache element
   constexpr int PIECE = FP8 ? 8 : 16;    // bytes one loader thread fetches of a row (8 elements)
   __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kPPTile * kKPitch];
@@ -691,10 +699,10 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     const int64_t chunk_bytes = p.kv_sc * ESZ;
     const int tok_bytes = p.kv_st * ESZ;
     // loader role: piece `lpiece` (8 elements) of key rows `lkey` and `lkey + 32` of a tile
-    const int lkey = tid >> 4, lpiece = tid & 15;
+    const int lkey = tid / PPR, lpiece = tid % PPR;
     const int k_off = lkey * kKPitch + lpiece * 16;
     const int v_off = lkey * kVPitch + lpiece * 16;
-    uint4 kreg[2], vreg[2];
+    uint4 kreg[NPASS], vreg[NPASS];
     // Staged tiles never straddle a chunk (the launcher only picks this kernel when the chunk size
     // is a multiple of 64), so a tile is addressed by scalars only -- physical chunk, tile index
     // inside the chunk -- plus a per-lane row offset that is fixed for the whole kernel.  The
@@ -704,7 +712,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     const int tiles_per_chunk = p.chunk / kPPTile;
     const int tile_bytes = kPPTile * tok_bytes;
     const uint32_t row_off0 = (uint32_t)(lkey * tok_bytes + lpiece * PIECE);
-    const uint32_t row_off1 = row_off0 + (uint32_t)(32 * tok_bytes);
+    const uint32_t row_off1 = row_off0 + (uint32_t)(RPP * tok_bytes);  // (second pass, head_dim 128 only)
     const uint32_t piece_off = (uint32_t)(lpiece * PIECE);
     float ksc_staged = 1.f, vsc_staged = 1.f;  // fp8: scales of the tile held in kreg / vreg (per-lane copies)
     const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
@@ -744,16 +752,16 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     };
     // this thread's two pieces of a tile (rows past the request's last key re-read the last row,
     // which every query row masks)
-    auto tile_loads = [&](const uint8_t* base, int64_t off, int room, uint4 (&reg)[2]) {
+    auto tile_loads = [&](const uint8_t* base, int64_t off, int room, uint4 (&reg)[NPASS]) {
       const uint8_t* tb = base + off;
       const uint32_t lim = (uint32_t)room + piece_off;
-      if (FP8) {
+      if constexpr (FP8) {
         const uint2 a = ld8(tb + min(row_off0, lim)), b = ld8(tb + min(row_off1, lim));
         reg[0] = make_uint4(a.x, a.y, 0u, 0u);
         reg[1] = make_uint4(b.x, b.y, 0u, 0u);
       } else {
         reg[0] = ld16(tb + min(row_off0, lim));
-        reg[1] = ld16(tb + min(row_off1, lim));
+        if constexpr (NPASS == 2) reg[1] = ld16(tb + min(row_off1, lim));
       }
     };
     // what goes into LDS for one staged piece: the bf16 bits, or (fp8) 8 bytes -> 8 bf16 of byte * scale
@@ -767,13 +775,13 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     auto store_k = [&](int t) {
       uint8_t* dst = &Ks[t & 1][k_off];
       *reinterpret_cast<uint4*>(dst) = lds_piece(kreg[0], ksc_staged);
-      *reinterpret_cast<uint4*>(dst + 32 * kKPitch) = lds_piece(kreg[1], ksc_staged);
+      if constexpr (NPASS == 2) *reinterpret_cast<uint4*>(dst + RPP * kKPitch) = lds_piece(kreg[1], ksc_staged);
     };
     auto vbuf = [](int t) { return (unsigned)(t + 3) % 3u; };  // tile -1 lives in buffer 2
     auto store_v = [&](int t) {
       uint8_t* dst = &Vs[vbuf(t)][v_off];
       *reinterpret_cast<uint4*>(dst) = lds_piece(vreg[0], vsc_staged);
-      *reinterpret_cast<uint4*>(dst + 32 * kVPitch) = lds_piece(vreg[1], vsc_staged);
+      if constexpr (NPASS == 2) *reinterpret_cast<uint4*>(dst + RPP * kVPitch) = lds_piece(vreg[1], vsc_staged);
     };
 
     const float scale = p.scale_log2;
@@ -788,7 +796,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // group are issued before the MFMAs of the previous group (scheduling barriers keep that
     // order), so a read has ~130 cycles of matrix work to hide behind and only two groups of
     // fragments are live at a time.
-    // S^T = K Q^T: group u = 16-key sub-tile u (4 K fragments, 8 MFMAs)
+    // S^T = K Q^T: group u = 16-key sub-tile u (KS K fragments, 2 KS MFMAs)
     auto sc_load = [&](int t, int u, uint4 (&kf)[KS]) {
       const uint8_t* ks = Ks[t & 1] + kfrag_off + 16 * u * kKPitch;
 #pragma unroll
@@ -806,7 +814,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // O^T += V^T P^T: group grp = (32-key step grp / 2, output columns 64 * (grp % 2) ..+63):
     // 8 transposed reads, 8 MFMAs (+2 for the denominators in the odd groups)
     auto pv_load = [&](int t, int grp, uint2 (&af)[4][2]) {
-      const uint8_t* vs = Vs[vbuf(t)] + vfrag_off + 32 * (grp >> 1) * kVPitch + 128 * (grp & 1);
+      const uint8_t* vs = Vs[vbuf(t)] + vfrag_off + 32 * (grp / NH) * kVPitch + 128 * (grp % NH);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         af[e][0] = lds_ld8_tr(vs + 32 * e);
@@ -814,7 +822,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       }
     };
     auto pv_mma = [&](int grp, const uint2 (&af)[4][2]) {
-      const int up = 2 * (grp >> 1), e0 = 4 * (grp & 1);
+      const int up = 2 * (grp / NH), e0 = 4 * (grp % NH);
       const uint4 pp0 = make_uint4(pf[0][up].x, pf[0][up].y, pf[0][up + 1].x, pf[0][up + 1].y);
       const uint4 pp1 = make_uint4(pf[1][up].x, pf[1][up].y, pf[1][up + 1].x, pf[1][up + 1].y);
 #pragma unroll
@@ -823,7 +831,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         acc[0][e0 + e] = mfma_16x16x32(a, pp0, acc[0][e0 + e]);
         acc[1][e0 + e] = mfma_16x16x32(a, pp1, acc[1][e0 + e]);
       }
-      if (grp & 1) {
+      if (grp % NH == NH - 1) {  // once per 32-key step
         accl[0] = mfma_16x16x32(ones, pp0, accl[0]);
         accl[1] = mfma_16x16x32(ones, pp1, accl[1]);
       }
@@ -841,6 +849,32 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       uint2 a0[4][2], a1[4][2];
       uint4 k0[KS], k1[KS];
       const int ta = it - 1, ts = it;
+      if constexpr (HD == 64) {  // half the matrix work per tile: two value groups, four 4-MFMA score groups
+        pv_load(ta, 0, a0);
+        pv_load(ta, 1, a1); MI_SB();
+        pv_mma(0, a0);
+        store_k(it + 1);
+        store_v(it + 1); MI_SB();
+        const int64_t off = tile_offset(cur, pc_cur);
+        const int room = cur.room;
+        tile_loads(kbase, off, room, kreg);
+        cursor_next(cur);
+        pc_cur = bt_row[cur.ci];  // block-table entry of tile it+3, consumed one iteration from now
+#pragma unroll
+        for (int i = 0; i < 10; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x006, 3, 0);  // up to three scalar / vector ALU instructions
+        }
+        MI_SB();
+        sc_load(ts, 0, k0); MI_SB();
+        pv_mma(1, a1);
+        tile_loads(vbase, off, room, vreg); MI_SB();
+        sc_load(ts, 1, k1); MI_SB(); sc_mma(0, k0); MI_SB();
+        sc_load(ts, 2, k0); MI_SB(); sc_mma(1, k1); MI_SB();
+        sc_load(ts, 3, k1); MI_SB(); sc_mma(2, k0); MI_SB();
+        sc_mma(3, k1);
+        return;
+      }
       pv_load(ta, 0, a0);
       pv_load(ta, 1, a1); MI_SB();
       pv_mma(0, a0);
@@ -994,8 +1028,8 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 }
 
 // Rows whose keys were split over several workgroups: o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max).
-// Grid (T, Hq), 128 threads = the output values of one (row, head).
-__global__ __launch_bounds__(128) void prefill_split_merge_kernel(PrefillParams p, int n_split) {
+// Grid (T, Hq), head_dim threads = the output values of one (row, head).
+__global__ __launch_bounds__(128) void prefill_split_merge_kernel(PrefillParams p, int n_split, int head_dim) {
   const int row = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   if (row >= p.cu_q[p.R]) return;  // padding rows: zeroed by the tile kernel
   if (p.skip_single) {             // one-row requests were left to the decode kernels
@@ -1013,7 +1047,7 @@ __global__ __launch_bounds__(128) void prefill_split_merge_kernel(PrefillParams 
     for (int j = 0; j < 8; ++j) {
       const int64_t prow = ((int64_t)min(s0 + j, n_split - 1) * p.T + row) * p.Hq + head;
       lse[j] = p.split_lse[prow];
-      po[j] = p.split_o[prow * 128 + d];
+      po[j] = p.split_o[prow * head_dim + d];
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -1038,7 +1072,7 @@ using namespace mi;
 // with thousands of keys to walk: then the keys are split so that about one workgroup per CU exists,
 // every one keeping at least sixteen 64-key tiles (a 512-token prompt is not worth the merge).  Host-side quantities only (the lengths live on the GPU).
 static int prefill_kv_splits(int T, int Hq, int Hkv, int head_dim, int max_kv_len) {
-  if (head_dim != 128 || max_kv_len <= 0) return 1;
+  if ((head_dim != 128 && head_dim != 64) || max_kv_len <= 0) return 1;
   const int G = Hq / Hkv;
   const int sbq = 256 / G;                               // query tokens per workgroup
   const int64_t useful = (int64_t)Hkv * ((T + sbq - 1) / sbq);
@@ -1124,7 +1158,8 @@ static int launch_paged_prefill(
   hipStream_t st = (hipStream_t)stream;
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
   const int lds_tiles = mi_tuning().prefill_lds_row_tiles;  // 0 = register-only kernel
-  if (head_dim == 128 && lds_tiles > 0) {
+  const bool pp64 = head_dim == 64 && lds_tiles > 0 && chunk_tokens % 64 == 0 && mi_tuning().prefill_pingpong != 0 && !fp8;
+  if ((head_dim == 128 && lds_tiles > 0) || pp64) {
     const int rows = 8 * 16 * ((lds_tiles == 2 || (mi_tuning().prefill_pingpong && chunk_tokens % 64 == 0)) ? 2 : 3);
     const int sbq_lds = rows / G;
     dim3 lgrid(((T + sbq_lds - 1) / sbq_lds + R) * Hkv);
@@ -1149,7 +1184,11 @@ static int launch_paged_prefill(
         workspace_bytes = dec_bytes;
       }
     }
-    if (n_split > 1 && fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true, true>), lgrid, dim3(512), 0, st, p);
+    if (pp64 && n_split > 1 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, true, 64>), lgrid, dim3(512), 0, st, p);
+    else if (pp64 && n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, true, 64>), lgrid, dim3(512), 0, st, p);
+    else if (pp64 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, false, 64>), lgrid, dim3(512), 0, st, p);
+    else if (pp64) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, false, 64>), lgrid, dim3(512), 0, st, p);
+    else if (n_split > 1 && fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true, true>), lgrid, dim3(512), 0, st, p);
     else if (n_split > 1 && fp8) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, true, true>), lgrid, dim3(512), 0, st, p);
     else if (n_split > 1 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, true>), lgrid, dim3(512), 0, st, p);
     else if (n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, true>), lgrid, dim3(512), 0, st, p);
@@ -1161,7 +1200,7 @@ static int launch_paged_prefill(
     else if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 2>), lgrid, dim3(512), 0, st, p);
     else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);  // (48 rows: 32-key tiles only)
     if (timed) (void)hipEventRecord(ev_b, st);
-    if (n_split > 1) hipLaunchKernelGGL(prefill_split_merge_kernel, dim3(T, Hq), dim3(128), 0, st, p, n_split);
+    if (n_split > 1) hipLaunchKernelGGL(prefill_split_merge_kernel, dim3(T, Hq), dim3(head_dim), 0, st, p, n_split, head_dim);
     int rc0 = mi_check_launch("mi_paged_prefill_attention");
     if (rc0 != MI_OK || !p.skip_single) return rc0;
     return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,

@@ -54,6 +54,11 @@ class DecodeLayerGraphs:
         hkv, d = ctx.num_kv_heads_per_partition, ctx.kv_channels
         need = ops.decode_workspace_bytes(ctx.max_requests, num_query_heads, hkv, d, ctx.chunk_size_tokens,
                                           ctx.max_sequence_length, 0)
+        if ctx.non_decode_cuda_graphs:  # prefill / mixed steps may split the keys of a request: more scratch
+            table_tokens = ctx.request_to_kv_chunk_ids.size(1) * ctx.chunk_size_tokens
+            for n in ctx.cuda_graph_token_counts:
+                for max_kv in (ctx.max_sequence_length, table_tokens):
+                    need = max(need, ops.prefill_workspace_bytes(n, ctx.max_requests, num_query_heads, hkv, d, max_kv, 0))
         self.workspace = torch.empty(max(need, 1), dtype=torch.uint8, device=ctx.device)
 
     @property

@@ -225,6 +225,13 @@ def decode_workspace_bytes(R: int, Hq: int, Hkv: int, head_dim: int, chunk: int,
     return int(_lib.load().mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, chunk, max_kv_len, split_tokens))
 
 
+def prefill_workspace_bytes(T: int, R: int, Hq: int, Hkv: int, head_dim: int, max_kv_len: int,
+                            split_tokens: int = 0) -> int:
+    """Scratch of one varlen attention call over ``T`` query rows of ``R`` requests: the decode part's
+    partials and, when the tile kernel splits the keys, its partials behind them."""
+    return int(_lib.load().mi_prefill_workspace_bytes(T, R, Hq, Hkv, head_dim, max_kv_len, split_tokens))
+
+
 def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens: Tensor, block_table: Tensor,
                            *, softmax_scale: Optional[float] = None, max_kv_len: Optional[int] = None,
                            split_tokens: int = 0, out: Optional[Tensor] = None,

@@ -79,13 +79,13 @@ def test_padded_requests_with_zero_lengths(mi, dev):
 @pytest.mark.parametrize("pingpong", [1, 2])
 @pytest.mark.parametrize("chunk", [64, 128, 256])
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 1), (16, 2)])
-def test_two_phase_kernel_ragged_lengths(mi, dev, pingpong, chunk, Hq, Hkv):
-    """The two-phase tile kernel (head_dim 128, chunk a multiple of 64): new-token counts and cached
+@pytest.mark.parametrize("d", [128, 64])
+def test_two_phase_kernel_ragged_lengths(mi, dev, pingpong, chunk, Hq, Hkv, d):
+    """The two-phase tile kernel (head_dim 128 or 64, chunk a multiple of 64): new-token counts and cached
     contexts around every tile (64 keys), workgroup (256 rows) and chunk boundary, for 1, 2, 4, 8
     and 16 query heads per KV head, staggered and lock-step."""
     q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 500, 256, 257, 3]
     ctx = [0, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0, 40, 7, 64, 63, 1020]
-    d = 128
     kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
     cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
     cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
@@ -151,14 +151,15 @@ def test_chunked_prefill_is_consistent_at_full_size(mi, dev):
     assert torch.equal(moved, full)
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("forced", [1, 2, 7, 64])
-def test_few_rows_over_long_contexts_split_the_keys(mi, dev, forced):
+def test_few_rows_over_long_contexts_split_the_keys(mi, dev, forced, d):
     """A chunk of a prompt (or a short turn) over a long cached context: the tile kernel cuts the keys of
     every request into ranges (automatic = knob 1, or a forced count), writes partials and merges them.
     Requests shorter than the number of ranges get empty ranges; one-token requests go the decode way."""
     q_lens = [96, 1, 40, 1, 7]
     ctx = [9000, 4000, 130, 0, 63]
-    Hq, Hkv, d, chunk = 32, 8, 128, 64
+    Hq, Hkv, chunk = 32, 8, 64
     kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
     cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
     cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
