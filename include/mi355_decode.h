@@ -246,7 +246,9 @@ int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t 
  * megatron/core/transformer/multi_latent_attention.py:801-825, called from
  * attention.py:406-411) and hands them to flash_attn_varlen_func (attention.py:546-557).
  * Same mask and padding rules as mi_paged_prefill_attention; each cache has its own strides
- * (elements); q `[T, Hq, 192]`, out `[T, Hq, 128]`.  One kernel serves every request.
+ * (elements); q `[T, Hq, 192]`, out `[T, Hq, 128]`.  One kernel serves every request: the
+ * two-phase LDS-tiled kernel when chunk_tokens is a multiple of 64 (and the knob prefill_pingpong
+ * is not 0), a register-only kernel otherwise.
  */
 int mi_paged_prefill_attention_mla(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
                                    const void* k_cache, int64_t k_stride_chunk, int64_t k_stride_tok,

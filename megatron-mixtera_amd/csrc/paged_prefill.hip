@@ -601,18 +601,25 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
 // bytes per staged K / V row.  head_dim 128: 288, measured conflict-free for the 16-row x 64-byte fragment
 // reads (272 is not), and 16 rows x 32 B of the transposing reads tile the banks twice; head_dim 64: 144
 // (36 dwords: the 16 rows of a fragment read start at 16 different multiples of four banks).
-template <int HD> constexpr int pp_pitch() { return HD == 128 ? 288 : 144; }
+// 192-wide keys (multi-latent attention): 416 (104 dwords = 8 x 13: the same bank pattern as 288).
+template <int HD> constexpr int pp_pitch() { return HD == 192 ? 416 : HD == 128 ? 288 : 144; }
 constexpr int kPPTile = 64;   // keys per staged tile
 
 // FP8: the cache holds e4m3 bytes with one fp32 scale per (chunk, KV head); a piece is multiplied by
 // its chunk's scale and rounded to bf16 on its way into LDS, so both matrix phases are the bf16 ones.
 // SPLIT: the keys of a request are cut into gridDim.y ranges (a separate instantiation, so that the
 // ordinary kernel carries no tile offsets).
-template <bool STAGGER, bool FP8, bool SPLIT = false, int HD = 128>
+// HD = width of values and output, HDK = width of queries and keys: equal, or 192 / 128 for the decompressed
+// caches of multi-latent attention, whose value cache has its own strides.
+template <bool STAGGER, bool FP8, bool SPLIT = false, int HD = 128, int HDK = HD>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
-  static_assert(HD == 128 || (HD == 64 && !FP8), "head_dim 128, or 64 with a bf16 cache");
-  constexpr int KS = HD / 32, DV = HD / 16, NQ = 2, NT = 4, WAVES = 8;
-  constexpr int kKPitch = pp_pitch<HD>(), kVPitch = pp_pitch<HD>();
+  static_assert((HD == 128 && HDK == 128) || (HD == 64 && HDK == 64 && !FP8) || (HD == 128 && HDK == 192 && !FP8 && !SPLIT),
+                "head_dim 128, or 64 with a bf16 cache, or 192 / 128 with bf16 caches");
+  constexpr bool MLA = HDK != HD;
+  constexpr int KS = HDK / 32, DV = HD / 16, NQ = 2, NT = 4, WAVES = 8;
+  constexpr int kKPitch = pp_pitch<HDK>(), kVPitch = pp_pitch<HD>();
+  constexpr int PPRK = HDK * 2 / 16;                 // 16-byte pieces per key row when it differs from a value row: 24
+  constexpr int NPK = kPPTile * PPRK / 512;          // key pieces per loader thread and tile: 3 | 2 | 1
   constexpr int PPR = HD * 2 / 16;       // 16-byte pieces (8 elements) per key row: 16 | 8
   constexpr int RPP = 512 / PPR;         // key rows the 512 loader threads cover in one pass: 32 | 64
   constexpr int NPASS = kPPTile / RPP;   // passes (rows per thread) per tile: 2 | 1
@@ -695,14 +702,16 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 
   if (ntl > 0) {
     const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * ESZ;
-    const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * ESZ;
+    const uint8_t* vbase = p.vc + (int64_t)h * (MLA ? p.v_sh : p.kv_sh) * ESZ;
     const int64_t chunk_bytes = p.kv_sc * ESZ;
     const int tok_bytes = p.kv_st * ESZ;
+    const int64_t v_chunk_bytes = MLA ? p.v_sc * ESZ : chunk_bytes;  // (value cache of its own: multi-latent only)
+    const int v_tok_bytes = MLA ? p.v_st * ESZ : tok_bytes;
     // loader role: piece `lpiece` (8 elements) of key rows `lkey` and `lkey + 32` of a tile
     const int lkey = tid / PPR, lpiece = tid % PPR;
     const int k_off = lkey * kKPitch + lpiece * 16;
     const int v_off = lkey * kVPitch + lpiece * 16;
-    uint4 kreg[NPASS], vreg[NPASS];
+    uint4 kreg[NPK], vreg[NPASS];
     // Staged tiles never straddle a chunk (the launcher only picks this kernel when the chunk size
     // is a multiple of 64), so a tile is addressed by scalars only -- physical chunk, tile index
     // inside the chunk -- plus a per-lane row offset that is fixed for the whole kernel.  The
@@ -711,15 +720,30 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // tile into a buffer nobody reads any more, which keeps the loop free of branches.
     const int tiles_per_chunk = p.chunk / kPPTile;
     const int tile_bytes = kPPTile * tok_bytes;
-    const uint32_t row_off0 = (uint32_t)(lkey * tok_bytes + lpiece * PIECE);
-    const uint32_t row_off1 = row_off0 + (uint32_t)(RPP * tok_bytes);  // (second pass, head_dim 128 only)
+    const int v_tile_bytes = kPPTile * v_tok_bytes;
+    const uint32_t row_off0 = (uint32_t)(lkey * v_tok_bytes + lpiece * PIECE);
+    const uint32_t row_off1 = row_off0 + (uint32_t)(RPP * v_tok_bytes);  // (second pass, head_dim 128 only)
     const uint32_t piece_off = (uint32_t)(lpiece * PIECE);
+    // 192-wide keys: 24 pieces per row do not divide the 512 loader threads into whole rows, so a thread
+    // takes pieces tid, tid + 512 and tid + 1024 of the tile's 1536
+    uint32_t mk_row_off[NPK], mk_piece_off[NPK];
+    int mk_lds[NPK];
+    if constexpr (MLA) {
+#pragma unroll
+      for (int i = 0; i < NPK; ++i) {
+        const int idx = tid + 512 * i, row = idx / PPRK, piece = idx - row * PPRK;
+        mk_row_off[i] = (uint32_t)(row * tok_bytes + piece * 16);
+        mk_piece_off[i] = (uint32_t)(piece * 16);
+        mk_lds[i] = row * kKPitch + piece * 16;
+      }
+    }
     float ksc_staged = 1.f, vsc_staged = 1.f;  // fp8: scales of the tile held in kreg / vreg (per-lane copies)
     const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
     struct Cursor {   // all members are wave-uniform
       int tile;       // tile index
       int ci, tin;    // logical chunk of the tile and tile index inside the chunk
       int room;       // bytes from the tile's first row to the request's last row (>= 0)
+      int room_v;     // the same in the value cache (multi-latent only)
     };
     auto cursor_at = [&](int t) {
       Cursor c;
@@ -727,6 +751,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       c.ci = c.tile / tiles_per_chunk;
       c.tin = c.tile - c.ci * tiles_per_chunk;
       c.room = (last - c.tile * kPPTile) * tok_bytes;
+      c.room_v = MLA ? (last - c.tile * kPPTile) * v_tok_bytes : 0;
       return c;
     };
     auto cursor_next = [&](Cursor& c) {  // one tile forward, sticking to the last tile
@@ -734,6 +759,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       const bool wrap = adv && (c.tin + 1 == tiles_per_chunk);
       c.tile += adv ? 1 : 0;
       c.room -= adv ? tile_bytes : 0;
+      if constexpr (MLA) c.room_v -= adv ? v_tile_bytes : 0;
       c.tin = wrap ? 0 : c.tin + (adv ? 1 : 0);
       c.ci += wrap ? 1 : 0;
     };
@@ -750,6 +776,10 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       tile_scales(pc);
       return (int64_t)pc * chunk_bytes + (int64_t)c.tin * tile_bytes;
     };
+    auto tile_offset_v = [&](const Cursor& c, int pc_lane) -> int64_t {
+      const int pc = __builtin_amdgcn_readfirstlane(pc_lane);
+      return (int64_t)pc * v_chunk_bytes + (int64_t)c.tin * v_tile_bytes;
+    };
     // this thread's two pieces of a tile (rows past the request's last key re-read the last row,
     // which every query row masks)
     auto tile_loads = [&](const uint8_t* base, int64_t off, int room, uint4 (&reg)[NPASS]) {
@@ -764,6 +794,15 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         if constexpr (NPASS == 2) reg[1] = ld16(tb + min(row_off1, lim));
       }
     };
+    auto tile_loads_k = [&](int64_t off, int room) {
+      if constexpr (MLA) {
+        const uint8_t* tb = kbase + off;
+#pragma unroll
+        for (int i = 0; i < NPK; ++i) kreg[i] = ld16(tb + min(mk_row_off[i], (uint32_t)room + mk_piece_off[i]));
+      } else {
+        tile_loads(kbase, off, room, kreg);
+      }
+    };
     // what goes into LDS for one staged piece: the bf16 bits, or (fp8) 8 bytes -> 8 bf16 of byte * scale
     auto lds_piece = [&](uint4 raw, float scale) {
       if (!FP8) return raw;
@@ -773,6 +812,11 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
                         pack_bf16x2(c.x * scale, c.y * scale), pack_bf16x2(d.x * scale, d.y * scale));
     };
     auto store_k = [&](int t) {
+      if constexpr (MLA) {
+#pragma unroll
+        for (int i = 0; i < NPK; ++i) *reinterpret_cast<uint4*>(&Ks[t & 1][mk_lds[i]]) = kreg[i];
+        return;
+      }
       uint8_t* dst = &Ks[t & 1][k_off];
       *reinterpret_cast<uint4*>(dst) = lds_piece(kreg[0], ksc_staged);
       if constexpr (NPASS == 2) *reinterpret_cast<uint4*>(dst + RPP * kKPitch) = lds_piece(kreg[1], ksc_staged);
@@ -809,6 +853,20 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       for (int kk = 1; kk < KS; ++kk) {
         s[0][u] = mfma_16x16x32(kf[kk], qf[0][kk], s[0][u]);
         s[1][u] = mfma_16x16x32(kf[kk], qf[1][kk], s[1][u]);
+      }
+    };
+    // 192-wide keys: a sub-tile's product in two halves of three fragments (half the fragment registers)
+    auto sc_load_half = [&](int t, int u, int half, uint4 (&kf)[3]) {
+      const uint8_t* ks = Ks[t & 1] + kfrag_off + 16 * u * kKPitch + 192 * half;
+#pragma unroll
+      for (int j = 0; j < 3; ++j) kf[j] = *reinterpret_cast<const uint4*>(ks + 64 * j);
+    };
+    auto sc_mma_half = [&](int u, int half, const uint4 (&kf)[3]) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        const int kk = 3 * half + j;
+        s[0][u] = mfma_16x16x32(kf[j], qf[0][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[0][u]);
+        s[1][u] = mfma_16x16x32(kf[j], qf[1][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[1][u]);
       }
     };
     // O^T += V^T P^T: group grp = (32-key step grp / 2, output columns 64 * (grp % 2) ..+63):
@@ -884,7 +942,9 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       pv_mma(1, a1);
       const int64_t off = tile_offset(cur, pc_cur);
       const int room = cur.room;
-      tile_loads(kbase, off, room, kreg);
+      const int64_t off_v = MLA ? tile_offset_v(cur, pc_cur) : off;
+      const int room_v = MLA ? cur.room_v : room;
+      tile_loads_k(off, room);
       cursor_next(cur);
       pc_cur = bt_row[cur.ci];  // block-table entry of tile it+3, consumed one iteration from now
       // spread the address arithmetic through the shadow of this group's MFMAs
@@ -896,7 +956,21 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       MI_SB();
       pv_load(ta, 3, a1); MI_SB();
       pv_mma(2, a0);
-      tile_loads(vbase, off, room, vreg); MI_SB();
+      tile_loads(vbase, off_v, room_v, vreg); MI_SB();
+      if constexpr (MLA) {
+        uint4 h0[3], h1[3];
+        sc_load_half(ts, 0, 0, h0); MI_SB();
+        pv_mma(3, a1); MI_SB();
+        sc_load_half(ts, 0, 1, h1); MI_SB(); sc_mma_half(0, 0, h0); MI_SB();
+        sc_load_half(ts, 1, 0, h0); MI_SB(); sc_mma_half(0, 1, h1); MI_SB();
+        sc_load_half(ts, 1, 1, h1); MI_SB(); sc_mma_half(1, 0, h0); MI_SB();
+        sc_load_half(ts, 2, 0, h0); MI_SB(); sc_mma_half(1, 1, h1); MI_SB();
+        sc_load_half(ts, 2, 1, h1); MI_SB(); sc_mma_half(2, 0, h0); MI_SB();
+        sc_load_half(ts, 3, 0, h0); MI_SB(); sc_mma_half(2, 1, h1); MI_SB();
+        sc_load_half(ts, 3, 1, h1); MI_SB(); sc_mma_half(3, 0, h0); MI_SB();
+        sc_mma_half(3, 1, h1);
+        return;
+      }
       sc_load(ts, 0, k0); MI_SB();
       pv_mma(3, a1); MI_SB();
       sc_load(ts, 1, k1); MI_SB(); sc_mma(0, k0); MI_SB();
@@ -965,15 +1039,16 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       *reinterpret_cast<uint4*>(&Vs[2][i]) = make_uint4(0u, 0u, 0u, 0u);  // "tile -1"
     {
       const Cursor c0 = cursor_at(tb), c1 = cursor_at(tb + 1);
-      const int64_t off0 = tile_offset(c0, bt_row[c0.ci]);
-      tile_loads(kbase, off0, c0.room, kreg);
-      tile_loads(vbase, off0, c0.room, vreg);
+      const int pc0 = bt_row[c0.ci], pc1 = bt_row[c1.ci];
+      const int64_t off0 = tile_offset(c0, pc0);
+      tile_loads_k(off0, c0.room);
+      tile_loads(vbase, MLA ? tile_offset_v(c0, pc0) : off0, MLA ? c0.room_v : c0.room, vreg);
       store_k(0);
       store_v(0);
       __syncthreads();  // K(0), V(0) and the zero-filled buffer are visible; the staging registers are free
-      const int64_t off1 = tile_offset(c1, bt_row[c1.ci]);
-      tile_loads(kbase, off1, c1.room, kreg);  // K(1), V(1): stored by matrix(0)
-      tile_loads(vbase, off1, c1.room, vreg);
+      const int64_t off1 = tile_offset(c1, pc1);
+      tile_loads_k(off1, c1.room);  // K(1), V(1): stored by matrix(0)
+      tile_loads(vbase, MLA ? tile_offset_v(c1, pc1) : off1, MLA ? c1.room_v : c1.room, vreg);
       pc_cur = bt_row[cur.ci];
     }
     if (lead) __syncthreads();  // second group idles through phase 0
@@ -1306,8 +1381,20 @@ extern "C" int mi_paged_prefill_attention_mla(
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.skip_single = 0;  // one kernel serves every request, one-row requests included
   p.k_scale = nullptr; p.v_scale = nullptr;
+  p.split_o = nullptr; p.split_lse = nullptr;
   const int sbq = 256 / G;  // query tokens per workgroup (256 rows)
-  dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * 8);
-  hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2>), grid, block, 0, (hipStream_t)stream, p);
+  const int pp = (chunk_tokens % 64 == 0 && mi_tuning().prefill_lds_row_tiles > 0) ? mi_tuning().prefill_pingpong : 0;
+  hipEvent_t ev_a, ev_b;
+  const bool timed = mi_profile_next(&ev_a, &ev_b);
+  if (timed) (void)hipEventRecord(ev_a, (hipStream_t)stream);
+  if (pp != 0) {  // two-phase tile kernel (staged tiles must not straddle chunks)
+    dim3 lgrid(((T + sbq - 1) / sbq + R) * Hkv);
+    if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, false, 128, 192>), lgrid, dim3(512), 0, (hipStream_t)stream, p);
+    else hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, false, 128, 192>), lgrid, dim3(512), 0, (hipStream_t)stream, p);
+  } else {
+    dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * 8);
+    hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2>), grid, block, 0, (hipStream_t)stream, p);
+  }
+  if (timed) (void)hipEventRecord(ev_b, (hipStream_t)stream);
   return mi_check_launch("mi_paged_prefill_attention_mla");
 }

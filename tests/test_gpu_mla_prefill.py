@@ -37,6 +37,35 @@ def test_mla_prefill_matches_checker(mi, dev, H, chunk):
     assert (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
 
 
+@pytest.mark.parametrize("pingpong", [0, 1, 2])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (8, 2), (16, 1)])
+def test_mla_prefill_kernel_choice_and_grouped_heads(mi, dev, pingpong, Hq, Hkv):
+    """The two-phase tile kernel (both wave schedules) and the register kernel, with several query heads
+    per key head, over lengths either side of the 64-key tiles and the chunk size."""
+    chunk = 128
+    q_lens = [1, 64, 65, 300, 2, 127, 1, 513]
+    ctx = [700, 0, 63, 129, 1000, 1, 0, 256]
+    kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    g = torch.Generator().manual_seed(100 + Hq + Hkv)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, g)
+    q = torch.randn(int(cu_q[-1]), Hq, 192, generator=g).bfloat16()
+    kc = torch.randn(N, chunk, Hkv, 192, generator=g).bfloat16()
+    vc = torch.randn(N, chunk, Hkv, 128, generator=g).bfloat16()
+    mi.ops.set_tuning("prefill_pingpong", pingpong)
+    try:
+        out = mi.ops.paged_prefill_attention_mla(q.to(dev), kc.to(dev), vc.to(dev), cu_q.to(dev), kv_lens.to(dev),
+                                                 bt.to(dev), softmax_scale=0.07)
+        torch.cuda.synchronize()
+    finally:
+        mi.ops.set_tuning("prefill_pingpong", 1)
+    ref = oa.paged_varlen_attention(q, kc, vc, cu_q, kv_lens, bt, softmax_scale=0.07)
+    got = out.float().cpu()
+    err = (got - ref).abs()
+    assert torch.isfinite(got).all() and (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
+
+
 def test_mla_prefill_strided_caches_and_padding_rows(mi, dev):
     """Key and value caches as views of one wider buffer (as a split of the up-projection output gives
     them), token padding after the last request, trailing zero-length requests."""

@@ -213,7 +213,56 @@ def case_mla_decode(mi, dev, rng, seed):
     close(out.squeeze(1), ref, 2e-2, "mla decode")
 
 
-KINDS = ["decode", "decode", "decode_fp8", "prefill", "prefill", "prefill_fp8", "mla"]
+def case_mla_prefill(mi, dev, rng, seed):
+    """Varlen attention over decompressed multi-latent caches: keys 192 wide, values 128, caches of their own
+    or two views of one buffer."""
+    gen = torch.Generator().manual_seed(seed)
+    Hkv = rng.choice([1, 2, 4, 16])
+    G = rng.choice([1, 1, 2, 4])
+    chunk = rng.choice([16, 64, 128, 256])
+    R = rng.randint(1, 8)
+    q_lens, ctx = [], []
+    for _ in range(R):
+        k = rng.random()
+        if k < 0.25:
+            q_lens.append(1)
+            ctx.append(rng.choice([0, rng.randint(0, 600)]))
+        elif k < 0.35:
+            q_lens.append(0)
+            ctx.append(0)
+        else:
+            q_lens.append(rng.choice([2, 16, 17, 63, 64, 65, 128, 257, rng.randint(1, 400)]))
+            ctx.append(rng.choice([0, 0, 5, chunk - 1, chunk, rng.randint(0, 700)]))
+    if sum(q_lens) == 0:
+        q_lens[0] = 5
+    pp = rng.choice([1, 1, 2, 0])
+    joint = rng.random() < 0.4
+    _note(f"mla_prefill seed={seed} Hq={Hkv * G} Hkv={Hkv} chunk={chunk} q_lens={q_lens} ctx={ctx} pingpong={pp} joint={joint}")
+    kv_lens = torch.tensor([a + b if a else 0 for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.zeros(R + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, gen)
+    q = torch.randn(int(cu_q[-1]), Hkv * G, 192, generator=gen).bfloat16()
+    kc = (torch.randn(N + 1, chunk, Hkv, 192, generator=gen) * 0.7).bfloat16()
+    vc = (torch.randn(N + 1, chunk, Hkv, 128, generator=gen) * 0.7).bfloat16()
+    if joint:
+        both = torch.cat([kc, vc], dim=-1).to(dev)
+        kd_, vd_ = both[..., :192], both[..., 192:]
+    else:
+        kd_, vd_ = kc.to(dev), vc.to(dev)
+    mi.ops.set_tuning("prefill_pingpong", pp)
+    try:
+        qd_ = q.to(dev)
+        poison(dev)
+        out = mi.ops.paged_prefill_attention_mla(qd_, kd_, vd_, cu_q.to(dev), kv_lens.to(dev), bt.to(dev), softmax_scale=0.08)
+        torch.cuda.synchronize()
+    finally:
+        mi.ops.set_tuning("prefill_pingpong", 1)
+    ref = oa.paged_varlen_attention(q, kc, vc, cu_q, kv_lens, bt, softmax_scale=0.08)
+    close(out, ref, 2e-2, "mla prefill")
+
+
+KINDS = ["decode", "decode", "decode_fp8", "prefill", "prefill", "prefill_fp8", "mla", "mla_prefill"]
 
 
 @pytest.mark.parametrize("block", range(8))
@@ -231,6 +280,8 @@ def test_random_cases_match_the_checker(mi, dev, block):
                 case_prefill(mi, dev, rng, seed, False)
             elif kind == "prefill_fp8":
                 case_prefill(mi, dev, rng, seed, True)
+            elif kind == "mla_prefill":
+                case_mla_prefill(mi, dev, rng, seed)
             else:
                 case_mla_decode(mi, dev, rng, seed)
         except mi._lib.KernelError as e:
