@@ -45,6 +45,9 @@ SECONDARY_WORKLOADS = {
     "mla_decode_h128": ("mla", dict(Hq=128, B=64, lo=512, hi=8192)),
     "mla_decode_h16_long": ("mla", dict(Hq=16, B=16, lo=65536, hi=65536)),
     "mla_decode_h128_long": ("mla", dict(Hq=128, B=16, lo=65536, hi=65536)),
+    "mla_prefill_h16": ("mla_prefill", dict(H=16, n=8, new=2048, ctx=2048)),
+    "mla_prefill_h128": ("mla_prefill", dict(H=128, n=2, new=2048, ctx=2048)),
+    "prefill_d64": ("prefill", dict(Hq=32, Hkv=8, d=64, n=8, new=2048, ctx=2048)),
     "sampling_top_k": ("sampling", dict(R=64, V=128256, top_k=50, top_p=0.0)),
     "sampling_top_p": ("sampling", dict(R=64, V=128256, top_k=0, top_p=0.9)),
     "sampling_greedy": ("sampling", dict(R=64, V=128256, top_k=1, top_p=0.0)),
@@ -72,6 +75,31 @@ def run_secondary(args, mi, lib, torch, dev):
         kernel = "paged_mla_decode_lds_kernel"
         what = (f"absorbed multi-latent decode attention, {Hq} query heads, batch {B}, latent rows of 576 bf16, "
                 f"context U[{prm['lo']},{prm['hi']}], chunk 256")
+        dtype = "bf16 (fp32 accumulate)"
+        timed_by_library = True
+    elif kind in ("mla_prefill", "prefill"):
+        mla = kind == "mla_prefill"
+        Hq, Hkv = (prm["H"], prm["H"]) if mla else (prm["Hq"], prm["Hkv"])
+        dk, dv = (192, 128) if mla else (prm["d"], prm["d"])
+        n, new, ctx = prm["n"], prm["new"], prm["ctx"]
+        lens = torch.full((n,), new + ctx, dtype=torch.int32)
+        cu_q = torch.arange(n + 1, dtype=torch.int32) * new
+        bt, N = mi.synthetic.build_block_table(lens, 256, gen)
+        kc = torch.empty(N + 1, 256, Hkv, dk, dtype=torch.bfloat16, device=dev).normal_(0, 0.5)
+        vc = torch.empty(N + 1, 256, Hkv, dv, dtype=torch.bfloat16, device=dev).normal_(0, 0.5)
+        q = torch.randn(n * new, Hq, dk, device=dev).bfloat16()
+        out = torch.empty(n * new, Hq, dv, dtype=torch.bfloat16, device=dev)
+        cu_d, lens_d, bt_d = cu_q.to(dev), lens.to(dev), bt.to(dev)
+        if mla:
+            step = lambda: mi.ops.paged_prefill_attention_mla(q, kc, vc, cu_d, lens_d, bt_d, softmax_scale=0.072, out=out)
+        else:
+            step = lambda: mi.ops.paged_prefill_attention(q, kc, vc, cu_d, lens_d, bt_d, max_kv_len=new + ctx, out=out)
+        pairs = n * (new * ctx + new * (new + 1) // 2)          # (query row, visible key) pairs per head
+        flops = 2 * Hq * (dk + dv) * pairs
+        nbytes = n * (new + ctx) * Hkv * (dk + dv) * 2 + n * new * Hq * (dk + dv) * 2
+        kernel = "paged_prefill_pp_kernel"
+        what = (f"paged varlen causal attention, {n} x {new} new tokens over {ctx} cached, {Hq}/{Hkv} heads, "
+                f"keys {dk} / values {dv} wide, chunk 256")
         dtype = "bf16 (fp32 accumulate)"
         timed_by_library = True
     elif kind == "sampling":
@@ -112,12 +140,16 @@ def run_secondary(args, mi, lib, torch, dev):
     call_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
     kernel_ms = call_ms
     if timed_by_library:
-        buf = (ctypes.c_float * args.steps)()
-        n_ev = lib.mi_profile_collect(buf, args.steps)
+        # (the two-width-equal prefill call times two launches per step: the tile kernel, then the decode
+        # kernel that serves one-row requests -- none here; the first of each pair is the tile kernel)
+        per_step = 2 if kind == "prefill" else 1
+        buf = (ctypes.c_float * (args.steps * per_step))()
+        n_ev = lib.mi_profile_collect(buf, args.steps * per_step)
         lib.mi_profile_enable(0)
-        kernel_ms = sum(buf[i] for i in range(min(n_ev, args.steps))) / max(1, min(n_ev, args.steps))
+        mine = [buf[i] for i in range(0, n_ev, per_step)]
+        kernel_ms = sum(mine) / max(1, len(mine))
     ms_per_step = elapsed * 1e3 / args.steps
-    mfma_bound = kind == "mla" and prm["Hq"] >= 64
+    mfma_bound = (kind == "mla" and prm["Hq"] >= 64) or kind in ("mla_prefill", "prefill")
     roofline = ({"bound": "mfma", "kernel": kernel, "achieved": round(flops / kernel_ms / 1e9, 1),
                  "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                  "frac": round(flops / kernel_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)} if mfma_bound else
@@ -141,7 +173,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2",
                     choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", *SECONDARY_WORKLOADS],
                     help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch; the "
-                         "mla_* / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
+                         "mla_* / prefill_d64 / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
     ap.add_argument("--split-tokens", type=int, default=0)
     ap.add_argument("--subtiles", type=int, default=0, help="16-token sub-tiles per loop iteration (1, 2 or 4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
