@@ -58,6 +58,7 @@ extern "C" int mi_set_tuning(const char* name, int32_t value) {
     return MI_OK;
   }
   if (!strcmp(name, "prefill_tile_subtiles")) {
+    if (value != 1 && value != 2 && value != 4) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_tile_subtiles must be 1, 2 or 4");
     mi_tuning().prefill_tile_subtiles = value;
     return MI_OK;
   }
@@ -105,9 +106,10 @@ extern "C" int mi_set_tuning(const char* name, int32_t value) {
 }
 
 // ---- kernel timing with HIP events --------------------------------------------------
-// When enabled, mi_paged_decode_attention brackets its split kernel (the kernel that
-// streams the KV cache) with a start/stop event pair on the caller's stream; the pairs are
-// read back with mi_profile_collect.  Host objects only: nothing is allocated on the
+// When enabled, the attention entry points bracket their main kernel (decode: the kernel that
+// streams the KV cache; prefill: the tile kernel, and after it the streaming kernel of the one-row
+// requests) with a start/stop event pair on the caller's stream; the pairs are read back, in
+// launch order, with mi_profile_collect.  Host objects only: nothing is allocated on the
 // device, and profiling must stay off while a stream is being captured into a graph.
 #include <mutex>
 #include <vector>

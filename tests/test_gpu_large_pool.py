@@ -20,7 +20,7 @@ N_POOL = 5 * 2048 + 3                    # 5 GiB and a bit
 
 
 def _chunk_ids(need, gen):
-    """`need` chunk ids: the last ones of the pool, the ones around 2 GiB and 4 GiB, the rest random."""
+    """`need` chunk ids: the last ones of the pool, the ones either side of the 2 GiB and 4 GiB marks, the rest random."""
     special = [N_POOL - 2, N_POOL - 3, 0, 4095, 4096, 4097, 8191, 8192, 8193, N_POOL - 4]
     rest = torch.randperm(N_POOL - 1, generator=gen).tolist()
     ids = []
