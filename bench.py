@@ -229,8 +229,6 @@ def run_mixed_batch(args, mi, lib, torch, dev):
     with U[512,8192] tokens, one varlen call.  Step = fused RMSNorm+RoPE+append of all new tokens,
     then paged varlen attention (tile kernel for the prefill requests, streaming + merge kernels for
     the one-token requests).  Two roofline objects: MFMA for the tile kernel, HBM for the stream."""
-    from oracle import rope_norm as orn
-
     Hq, Hkv, d, chunk = 32, 8, 128, 256
     q, kc, vc, cu_q, lens, bt = mi.synthetic.make_prefill_case(
         dev, n_prefill=8, new_tokens=2048, ctx_lo=0, ctx_hi=4096, n_decode=120, dec_lo=512, dec_hi=8192,
@@ -243,7 +241,7 @@ def run_mixed_batch(args, mi, lib, torch, dev):
     kw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16().to(dev)
     pos, tok_chunk, tok_local = mi.synthetic.prefill_token_rows(cu_q, lens, bt, chunk)
     max_len = int(lens.max())
-    table = orn.rotary_table(max_len + 1, d, base=500000.0).to(dev)
+    table = mi.synthetic.rotary_angle_table(max_len + 1, d, base=500000.0).to(dev)
     q_rot = torch.empty_like(q)
     out = torch.empty_like(q)
     ks = vs = None
@@ -294,9 +292,8 @@ def run_mixed_batch(args, mi, lib, torch, dev):
     lk = lens.cpu().long()
     pre = lq > 1
     flops = 4 * Hq * d * int((lq[pre] * (lk - lq)[pre] + lq[pre] * (lq[pre] + 1) // 2).sum())
-    from oracle import paged_attention as oa
     kvb = 1 if args.fp8_kv else 2
-    dec_bytes = oa.decode_attention_bytes(lk[~pre].tolist(), Hq, Hkv, d, chunk, kv_bytes=kvb, fp8_scales=args.fp8_kv)
+    dec_bytes = mi.synthetic.decode_attention_bytes(lk[~pre].tolist(), Hq, Hkv, d, chunk, kv_bytes=kvb, fp8_scales=args.fp8_kv)
     pre_kv_bytes = int(lk[pre].sum()) * Hkv * d * 2 * kvb + int(lq[pre].sum()) * Hq * d * 4
     ms_per_step = elapsed * 1e3 / args.steps
     total_bytes = dec_bytes + pre_kv_bytes
@@ -335,8 +332,6 @@ def main():
     import torch
 
     from __graft_entry__ import load_package
-    from oracle import paged_attention as oa
-    from oracle import rope_norm as orn
 
     mi = load_package()
     lib = mi._lib.load()  # raises if the HIP library is missing: there is no fallback to measure
@@ -374,7 +369,7 @@ def main():
     qw = (1 + 0.02 * torch.randn(cfg.d, generator=gen)).bfloat16().to(dev)
     kw = (1 + 0.02 * torch.randn(cfg.d, generator=gen)).bfloat16().to(dev)
     theta = cfg.rope_theta or 500000.0
-    table = orn.rotary_table(max_len + 1, cfg.d, base=theta).to(dev)
+    table = mi.synthetic.rotary_angle_table(max_len + 1, cfg.d, base=theta).to(dev)
     pos = (case.kv_lens.long() - 1).contiguous()
     q_in = case.q.clone()
     out = torch.empty_like(case.q)
@@ -441,7 +436,7 @@ def main():
     kernel_ms = sum(buf[i] for i in range(min(n_ev, args.steps))) / max(1, min(n_ev, args.steps))
 
     ms_per_step = elapsed * 1e3 / args.steps
-    nbytes = oa.decode_attention_bytes(lens_host.tolist(), cfg.Hq, cfg.Hkv, cfg.d, cfg.chunk,
+    nbytes = mi.synthetic.decode_attention_bytes(lens_host.tolist(), cfg.Hq, cfg.Hkv, cfg.d, cfg.chunk,
                                        kv_bytes=1 if cfg.fp8 else 2, fp8_scales=cfg.fp8)
     value = nbytes / (ms_per_step * 1e-3) / 1e9
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9

@@ -164,3 +164,24 @@ def prefill_token_rows(cu_seqlens_q: Tensor, kv_lens: Tensor, block_table: Tenso
     pos = torch.arange(T, device=cu.device) - cu[req] + (kv_lens.long() - lq)[req]
     chunk_idx = block_table.long()[req, pos // chunk]
     return pos.contiguous(), chunk_idx.contiguous(), (pos % chunk).contiguous()
+
+
+def rotary_angle_table(max_seq_len: int, dim: int, base: float = 10000.0) -> Tensor:
+    """fp32 ``[max_seq_len, 1, 1, dim]`` table of rotary angles in the layout the model hands to the
+    context (``emb = cat(freqs, freqs)`` with ``freqs = outer(positions, 1 / base^(2i/dim))``,
+    rotary_pos_embedding.py:79-81,151-181) -- a synthetic input for benchmarks and examples."""
+    inv_freq = 1.0 / (base ** (torch.arange(0, dim, 2, dtype=torch.float32) / dim))
+    freqs = torch.outer(torch.arange(max_seq_len, dtype=torch.float32), inv_freq)
+    return torch.cat((freqs, freqs), dim=-1)[:, None, None, :]
+
+
+def decode_attention_bytes(kv_lens, Hq: int, Hkv: int, d: int, chunk: int, kv_bytes: int = 2,
+                           fp8_scales: bool = False) -> int:
+    """Bytes one decode-attention call has to move: every cached K and V row once, q in, out back,
+    the block-table entries and lengths in use (and the per-chunk scales of an fp8 cache)."""
+    lens = [int(x) for x in kv_lens]
+    chunks = sum((l + chunk - 1) // chunk for l in lens)
+    total = sum(lens) * Hkv * d * 2 * kv_bytes + len(lens) * Hq * d * (2 + 2) + chunks * 4 + len(lens) * 4
+    if fp8_scales:
+        total += chunks * Hkv * 2 * 4
+    return total

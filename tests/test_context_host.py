@@ -562,3 +562,19 @@ def test_mla_latent_cache_sizing_and_views(mi):
         Ctx(params_dtype=torch.bfloat16, num_layers=1, kv_channels=128, num_attention_heads=16,
             max_sequence_length=256, buffer_size_gb=0.001, buffer_guaranteed_fraction=0.1, chunk_size_tokens=64,
             cache_mla_latent=True, device="cpu")
+
+
+def test_synthetic_input_helpers_agree_with_the_checker(mi):
+    """The benchmark builds its rotary table and counts its algorithmic bytes with helpers of the package
+    (so that its measured leg touches nothing of the checker); both must say what the checker says."""
+    from oracle import paged_attention as oa
+    from oracle import rope_norm as orn
+
+    for dim, base in ((128, 500000.0), (64, 10000.0)):
+        assert torch.equal(mi.synthetic.rotary_angle_table(300, dim, base), orn.rotary_table(300, dim, base=base))
+    lens = [5, 700, 0, 256, 257, 8192]
+    for kvb, sc in ((2, False), (1, True)):
+        assert mi.synthetic.decode_attention_bytes(lens, 32, 8, 128, 256, kv_bytes=kvb, fp8_scales=sc) == \
+            oa.decode_attention_bytes(lens, 32, 8, 128, 256, kv_bytes=kvb, fp8_scales=sc)
+    # by hand: one request of 3 tokens, 2/1 heads of 8 values, chunk 2 -> 2 chunks
+    assert mi.synthetic.decode_attention_bytes([3], 2, 1, 8, 2) == 3 * 1 * 8 * 2 * 2 + 2 * 8 * 4 + 2 * 4 + 4
