@@ -38,7 +38,7 @@ struct PrefillParams {
   uint16_t* out;
   int64_t o_st, o_sh;
   uint64_t chunk_magic;  // ceil(2^40 / chunk)
-  int32_t T, R, Hq, Hkv, G, g_shift, chunk;
+  int32_t T, R, Hq, Hkv, G, g_magic, chunk;  // g_magic = 65536 / G + 1: (n * g_magic) >> 16 == n / G for n <= 64, G <= 16
   int32_t skip_single;  // requests with exactly one query row are handled by the decode kernels
   float scale_log2;
   const float* k_scale;  // fp8 KV only: [n_chunks][Hkv]
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
   const int m16 = lane & 15, g = lane >> 4;
   const int h = blockIdx.y;
   const int G = p.G;
-  const int BQ = (16 * NQ) >> p.g_shift;  // query tokens per wave
+  const int BQ = ((16 * NQ) * p.g_magic) >> 16;  // query tokens per wave
   const int SBQ = WAVES * BQ;             // query tokens per workgroup
 
   // Rows beyond the last request (token padding of the batch) are defined as zeros; the first
@@ -105,7 +105,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 #pragma unroll
   for (int nt = 0; nt < NQ; ++nt) {
     const int n = 16 * nt + m16;
-    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     const bool valid = qi < nq;
     qpos[nt] = valid ? shift + q0 + qi : last;
     const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 #pragma unroll
     for (int nt = 0; nt < NQ; ++nt) {
       const int n = 16 * nt + m16;
-      const int qi = n >> p.g_shift, u = n & (G - 1);
+      const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
       if (qi < nq) {
         uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
         for (int i = 0; i < 4 * DV; i += 4) st8(o + i, make_uint2(0, 0));
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
     l_tot += xor32(l_tot);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int n = 16 * nt + m16;
-    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     if (qi < nq) {
       uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
 #pragma unroll
@@ -364,7 +364,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
   const int h = blockIdx.x % p.Hkv;
   const int rank = blockIdx.x / p.Hkv;
   const int G = p.G;
-  const int BQ = (16 * NQ) >> p.g_shift;  // query tokens per wave
+  const int BQ = ((16 * NQ) * p.g_magic) >> 16;  // query tokens per wave
   const int SBQ = WAVES * BQ;             // query tokens per workgroup
 
   if (rank == 0) {
@@ -404,7 +404,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
 #pragma unroll
   for (int nt = 0; nt < NQ; ++nt) {
     const int n = 16 * nt + m16;
-    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     const bool valid = qi < nq;
     qpos[nt] = valid ? shift + q0 + qi : last;
     const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
@@ -568,7 +568,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
     l_tot += xor32(l_tot);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int n = 16 * nt + m16;
-    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     if (qi < nq) {
       uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
 #pragma unroll
@@ -637,7 +637,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   const int h = blockIdx.x % p.Hkv;
   const int rank = blockIdx.x / p.Hkv;
   const int G = p.G;
-  const int BQ = (16 * NQ) >> p.g_shift;
+  const int BQ = ((16 * NQ) * p.g_magic) >> 16;
   const int SBQ = WAVES * BQ;
 
   if (rank == 0 && (!SPLIT || blockIdx.y == 0)) {
@@ -681,7 +681,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 #pragma unroll
   for (int nt = 0; nt < NQ; ++nt) {
     const int n = 16 * nt + m16;
-    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     const bool valid = qi < nq;
     qpos[nt] = valid ? shift + q0 + qi : last;
     const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
@@ -1081,7 +1081,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     const float l_tot = accl[nt][0];
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int n = 16 * nt + m16;
-    const int qi = n >> p.g_shift, u = n & (G - 1);
+    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     if (qi < nq) {
       if (!SPLIT) {
         uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * g;
@@ -1149,7 +1149,7 @@ using namespace mi;
 static int prefill_kv_splits(int T, int Hq, int Hkv, int head_dim, int max_kv_len) {
   if ((head_dim != 128 && head_dim != 64) || max_kv_len <= 0) return 1;
   const int G = Hq / Hkv;
-  const int sbq = 256 / G;                               // query tokens per workgroup
+  const int sbq = 8 * (32 / G);                          // query tokens per workgroup (8 wavefronts x 32 rows)
   const int64_t useful = (int64_t)Hkv * ((T + sbq - 1) / sbq);
   const int cus = 256;
   if (useful >= cus) return 1;
@@ -1190,8 +1190,8 @@ static int launch_paged_prefill(
   if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: need T, R >= 0 and Hq a multiple of Hkv");
   const int G = Hq / Hkv;
-  if (G > 16 || (G & (G - 1)))
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: query heads per KV head must be 1, 2, 4, 8 or 16");
+  if (G > 16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: at most 16 query heads per KV head");
   if (head_dim != 64 && head_dim != 128)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: head_dim must be 64 or 128");
   if (chunk_tokens <= 0 || chunk_tokens % 16)
@@ -1220,8 +1220,7 @@ static int launch_paged_prefill(
   p.bt = block_table; p.bt_stride = bt_stride; p.cu_q = cu_seqlens_q; p.lens = kv_lens;
   p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
   p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G;
-  p.g_shift = 0;
-  while ((1 << p.g_shift) < G) ++p.g_shift;
+  p.g_magic = 65536 / G + 1;
   p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
@@ -1236,7 +1235,7 @@ static int launch_paged_prefill(
   const bool pp64 = head_dim == 64 && lds_tiles > 0 && chunk_tokens % 64 == 0 && mi_tuning().prefill_pingpong != 0 && !fp8;
   if ((head_dim == 128 && lds_tiles > 0) || pp64) {
     const int rows = 8 * 16 * ((lds_tiles == 2 || (mi_tuning().prefill_pingpong && chunk_tokens % 64 == 0)) ? 2 : 3);
-    const int sbq_lds = rows / G;
+    const int sbq_lds = 8 * ((rows / 8) / G);  // 8 wavefronts x whole tokens in a wavefront's rows
     dim3 lgrid(((T + sbq_lds - 1) / sbq_lds + R) * Hkv);
     const bool wide = mi_tuning().prefill_tile_subtiles == 4;  // 64-key staged tiles
     hipEvent_t ev_a, ev_b;
@@ -1284,7 +1283,7 @@ static int launch_paged_prefill(
                                split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
   }
   const int nq = mi_tuning().prefill_row_tiles == 4 ? 4 : 2;
-  const int sbq = 256 / G;  // query tokens per workgroup (256 rows)
+  const int sbq = (16 / nq) * ((16 * nq) / G);  // query tokens per workgroup: whole tokens in each wavefront's rows
   dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * (16 / nq));
   // register-only kernel (head_dim 64, or LDS variant switched off): 16 or 32 keys per iteration
   const int nt = mi_tuning().prefill_tile_subtiles == 1 ? 1 : 2;
@@ -1351,8 +1350,8 @@ extern "C" int mi_paged_prefill_attention_mla(
   if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention_mla: need T, R >= 0 and Hq a multiple of Hkv");
   const int G = Hq / Hkv;
-  if (G > 16 || (G & (G - 1)))
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: query heads per KV head must be 1, 2, 4, 8 or 16");
+  if (G > 16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: at most 16 query heads per KV head");
   if (head_dim_k != 192 || head_dim_v != 128)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: key width 192 (128 + 64) and value width 128 only");
   if (chunk_tokens <= 0 || chunk_tokens % 16)
@@ -1374,15 +1373,14 @@ extern "C" int mi_paged_prefill_attention_mla(
   p.bt = block_table; p.bt_stride = bt_stride; p.cu_q = cu_seqlens_q; p.lens = kv_lens;
   p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
   p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G;
-  p.g_shift = 0;
-  while ((1 << p.g_shift) < G) ++p.g_shift;
+  p.g_magic = 65536 / G + 1;
   p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.skip_single = 0;  // one kernel serves every request, one-row requests included
   p.k_scale = nullptr; p.v_scale = nullptr;
   p.split_o = nullptr; p.split_lse = nullptr;
-  const int sbq = 256 / G;  // query tokens per workgroup (256 rows)
+  const int sbq = 8 * (32 / G);  // query tokens per workgroup (8 wavefronts x 32 rows)
   const int pp = (chunk_tokens % 64 == 0 && mi_tuning().prefill_lds_row_tiles > 0) ? mi_tuning().prefill_pingpong : 0;
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);

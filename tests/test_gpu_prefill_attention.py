@@ -212,3 +212,43 @@ def test_split_keys_with_padding_rows_and_fp8(mi, dev):
     ref8 = oa.paged_varlen_attention(q[:53].cpu(), k8.cpu(), v8.cpu(), cu_q, kv_lens, bt, k_scales=ks.cpu(), v_scales=vs.cpu())
     err8 = (out8[:53].float().cpu() - ref8).abs()
     assert (err8 <= 2.5e-2 + 2.5e-2 * ref8.abs()).all() and (out8[53:] == 0).all()
+
+
+@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_no_offset", "lock_step", "lock_step_48_rows", "registers", "split_keys"])
+@pytest.mark.parametrize("Hq,Hkv", [(12, 4), (10, 2), (28, 4), (6, 1), (12, 1), (15, 1)])
+@pytest.mark.parametrize("d", [128, 64])
+def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, d):
+    """3, 5, 6, 7, 12 or 15 query heads per KV head (Llama-3.2-3B, Qwen2.5-14B, Qwen2-7B ... have such groups):
+    a wavefront's 32 (48) rows then hold as many whole tokens as fit, the rest are padding rows.  Every
+    prefill kernel, lengths either side of the per-workgroup token counts (48 tokens at a group of 5)."""
+    knobs = {"two_phase": {}, "two_phase_no_offset": {"prefill_pingpong": 2}, "lock_step": {"prefill_pingpong": 0},
+             "lock_step_48_rows": {"prefill_pingpong": 0, "prefill_lds_row_tiles": 3},
+             "registers": {"prefill_lds_row_tiles": 0}, "split_keys": {"prefill_kv_split": 3}}[kernel]
+    if d == 64 and kernel.startswith("lock_step"):
+        pytest.skip("the lock-step LDS kernel is head_dim 128 only")
+    G = Hq // Hkv
+    per_wg = 8 * (32 // G)
+    q_lens = [1, per_wg - 1, per_wg, per_wg + 1, 2 * per_wg + 3, 1, 301, 5]
+    ctx = [300, 0, 64, 7, 500, 0, 129, 1000]
+    kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    gen = torch.Generator().manual_seed(Hq * 100 + Hkv + d)
+    bt, N = mi.synthetic.build_block_table(kv_lens, 64, gen)
+    q = torch.randn(int(cu_q[-1]) + 3, Hq, d, generator=gen).bfloat16().to(dev)   # three padding rows
+    kc = torch.randn(N, 64, Hkv, d, generator=gen).bfloat16().to(dev)
+    vc = torch.randn(N, 64, Hkv, d, generator=gen).bfloat16().to(dev)
+    for name, value in knobs.items():
+        mi.ops.set_tuning(name, value)
+    try:
+        out = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev), max_kv_len=int(kv_lens.max()))
+        torch.cuda.synchronize()
+    finally:
+        for name, value in {"prefill_pingpong": 1, "prefill_lds_row_tiles": 2, "prefill_kv_split": 1}.items():
+            mi.ops.set_tuning(name, value)
+    T = int(cu_q[-1])
+    ref = oa.paged_varlen_attention(q[:T].cpu(), kc.cpu(), vc.cpu(), cu_q, kv_lens, bt)
+    got = out.float().cpu()
+    assert torch.isfinite(got).all() and (got[T:] == 0).all()
+    err = (got[:T] - ref).abs()
+    assert (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"

@@ -127,7 +127,7 @@ def case_prefill(mi, dev, rng, seed, fp8):
     gen = torch.Generator().manual_seed(seed)
     d = rng.choice([64, 128]) if not fp8 else 128
     Hkv = rng.choice([1, 2, 4, 8])
-    G = rng.choice([1, 2, 4, 8])
+    G = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16])
     Hq = Hkv * G
     chunk = rng.choice([16, 32, 64, 128, 256])
     R = rng.randint(1, 10)
@@ -218,7 +218,7 @@ def case_mla_prefill(mi, dev, rng, seed):
     or two views of one buffer."""
     gen = torch.Generator().manual_seed(seed)
     Hkv = rng.choice([1, 2, 4, 16])
-    G = rng.choice([1, 1, 2, 4])
+    G = rng.choice([1, 1, 2, 3, 4, 5])
     chunk = rng.choice([16, 64, 128, 256])
     R = rng.randint(1, 8)
     q_lens, ctx = [], []
