@@ -69,7 +69,7 @@ def case_decode(mi, dev, rng, seed, fp8):
     gen = torch.Generator().manual_seed(seed)
     d = rng.choice([64, 128])
     Hkv = rng.choice([1, 2, 3, 4, 8, 16])
-    G = rng.choice([1, 2, 4, 5, 8, 16] if not fp8 else [1, 2, 4, 8])
+    G = rng.choice([1, 2, 3, 4, 5, 7, 8, 16])
     Hq = Hkv * G
     chunk = rng.choice([16, 32, 48, 64, 80, 128, 256])
     R = rng.randint(1, 24)
@@ -370,7 +370,7 @@ def case_norm_rope(mi, dev, rng, seed):
     d = rng.choice([64, 128])
     rot = rng.choice([d, d // 2, d, 32])
     Hkv = rng.choice([1, 2, 4, 8])
-    Hq = Hkv * rng.choice([1, 2, 4])
+    Hq = Hkv * rng.choice([1, 2, 3, 4, 5, 7])
     norm = rng.choice([None, "rms", "l2"])
     interleaved = rng.random() < 0.3
     vec = rng.choice([0, 1, 2])
