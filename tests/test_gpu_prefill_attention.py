@@ -214,7 +214,8 @@ def test_split_keys_with_padding_rows_and_fp8(mi, dev):
     assert (err8 <= 2.5e-2 + 2.5e-2 * ref8.abs()).all() and (out8[53:] == 0).all()
 
 
-@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_no_offset", "lock_step", "lock_step_48_rows", "registers", "split_keys"])
+@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_no_offset", "lock_step", "lock_step_48_rows", "registers",
+                                    "registers_64_rows", "split_keys"])
 @pytest.mark.parametrize("Hq,Hkv", [(12, 4), (10, 2), (28, 4), (6, 1), (12, 1), (15, 1)])
 @pytest.mark.parametrize("d", [128, 64])
 def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, d):
@@ -223,7 +224,9 @@ def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, 
     prefill kernel, lengths either side of the per-workgroup token counts (48 tokens at a group of 5)."""
     knobs = {"two_phase": {}, "two_phase_no_offset": {"prefill_pingpong": 2}, "lock_step": {"prefill_pingpong": 0},
              "lock_step_48_rows": {"prefill_pingpong": 0, "prefill_lds_row_tiles": 3},
-             "registers": {"prefill_lds_row_tiles": 0}, "split_keys": {"prefill_kv_split": 3}}[kernel]
+             "registers": {"prefill_lds_row_tiles": 0},
+             "registers_64_rows": {"prefill_lds_row_tiles": 0, "prefill_row_tiles": 4},
+             "split_keys": {"prefill_kv_split": 3}}[kernel]
     if d == 64 and kernel.startswith("lock_step"):
         pytest.skip("the lock-step LDS kernel is head_dim 128 only")
     G = Hq // Hkv
@@ -244,7 +247,8 @@ def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, 
         out = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev), max_kv_len=int(kv_lens.max()))
         torch.cuda.synchronize()
     finally:
-        for name, value in {"prefill_pingpong": 1, "prefill_lds_row_tiles": 2, "prefill_kv_split": 1}.items():
+        for name, value in {"prefill_pingpong": 1, "prefill_lds_row_tiles": 2, "prefill_kv_split": 1,
+                            "prefill_row_tiles": 2}.items():
             mi.ops.set_tuning(name, value)
     T = int(cu_q[-1])
     ref = oa.paged_varlen_attention(q[:T].cpu(), kc.cpu(), vc.cpu(), cu_q, kv_lens, bt)
