@@ -249,7 +249,11 @@ int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t 
  * Same mask and padding rules as mi_paged_prefill_attention; each cache has its own strides
  * (elements); q `[T, Hq, 192]`, out `[T, Hq, 128]`.  One kernel serves every request: the
  * two-phase LDS-tiled kernel when chunk_tokens is a multiple of 64 (and the knob prefill_pingpong
- * is not 0), a register-only kernel otherwise.
+ * is not 0), a register-only kernel otherwise.  `workspace` may be NULL; one of
+ * mi_prefill_workspace_bytes(T, R, Hq, Hkv, head_dim_v, max_kv_len, 0) bytes (256-byte aligned) lets
+ * the two-phase kernel cut the keys of every request into ranges when few query rows meet long
+ * contexts, as in mi_paged_prefill_attention (`max_kv_len` bounds every kv_lens[r]; it only sizes
+ * that split).
  */
 int mi_paged_prefill_attention_mla(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
                                    const void* k_cache, int64_t k_stride_chunk, int64_t k_stride_tok,
@@ -257,9 +261,10 @@ int mi_paged_prefill_attention_mla(const void* q, int64_t q_stride_tok, int64_t 
                                    int64_t v_stride_tok, int64_t v_stride_head,
                                    const int32_t* block_table, int64_t bt_stride,
                                    const int32_t* cu_seqlens_q, const int32_t* kv_lens, void* out,
-                                   int64_t o_stride_tok, int64_t o_stride_head, int32_t T, int32_t R,
-                                   int32_t Hq, int32_t Hkv, int32_t head_dim_k, int32_t head_dim_v,
-                                   int32_t chunk_tokens, float softmax_scale, void* stream);
+                                   int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
+                                   int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
+                                   int32_t head_dim_k, int32_t head_dim_v, int32_t chunk_tokens,
+                                   int32_t max_kv_len, float softmax_scale, void* stream);
 
 /*
  * Fused q/k head norm + rotary embedding (+ KV-append when k_cache is given).

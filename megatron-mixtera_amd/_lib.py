@@ -54,7 +54,7 @@ SIGNATURES = {
     "mi_paged_prefill_attention_mla": (
         c_int,
         [_P, _I64, _I64, _P, _I64, _I64, _I64, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _I64, _I64,
-         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
+         _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
     "mi_update_requests": (
         c_int, [_P] * 8 + [_I64, _I32] + [_P] * 14 + [_I32] * 7 + [_P]),
     "mi_decode_attention_state": (

@@ -613,7 +613,7 @@ constexpr int kPPTile = 64;   // keys per staged tile
 // caches of multi-latent attention, whose value cache has its own strides.
 template <bool STAGGER, bool FP8, bool SPLIT = false, int HD = 128, int HDK = HD>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
-  static_assert((HD == 128 && HDK == 128) || (HD == 64 && HDK == 64 && !FP8) || (HD == 128 && HDK == 192 && !FP8 && !SPLIT),
+  static_assert((HD == 128 && HDK == 128) || (HD == 64 && HDK == 64 && !FP8) || (HD == 128 && HDK == 192 && !FP8),
                 "head_dim 128, or 64 with a bf16 cache, or 192 / 128 with bf16 caches");
   constexpr bool MLA = HDK != HD;
   constexpr int KS = HDK / 32, DV = HD / 16, NQ = 2, NT = 4, WAVES = 8;
@@ -1341,12 +1341,14 @@ extern "C" int mi_paged_prefill_attention_mla(
     const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache, int64_t k_stride_chunk,
     int64_t k_stride_tok, int64_t k_stride_head, const void* v_cache, int64_t v_stride_chunk, int64_t v_stride_tok,
     int64_t v_stride_head, const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seqlens_q,
-    const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head, int32_t T, int32_t R,
-    int32_t Hq, int32_t Hkv, int32_t head_dim_k, int32_t head_dim_v, int32_t chunk_tokens, float softmax_scale,
-    void* stream) {
+    const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
+    int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim_k, int32_t head_dim_v,
+    int32_t chunk_tokens, int32_t max_kv_len, float softmax_scale, void* stream) {
   if (T == 0 || R == 0) return MI_OK;
   if (!q || !k_cache || !v_cache || !block_table || !cu_seqlens_q || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_mla: null pointer argument");
+  if (workspace && ((uintptr_t)workspace & 255))
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention_mla: the workspace must be 256-byte aligned");
   if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention_mla: need T, R >= 0 and Hq a multiple of Hkv");
   const int G = Hq / Hkv;
@@ -1385,14 +1387,33 @@ extern "C" int mi_paged_prefill_attention_mla(
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
   if (timed) (void)hipEventRecord(ev_a, (hipStream_t)stream);
+  int n_split = 1;
   if (pp != 0) {  // two-phase tile kernel (staged tiles must not straddle chunks)
     dim3 lgrid(((T + sbq - 1) / sbq + R) * Hkv);
-    if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, false, 128, 192>), lgrid, dim3(512), 0, (hipStream_t)stream, p);
-    else hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, false, 128, 192>), lgrid, dim3(512), 0, (hipStream_t)stream, p);
+    // few query rows over long contexts: key ranges per request, partials in the workspace (which holds
+    // nothing else here: one-row requests stay in the tile kernel)
+    if (workspace && mi_tuning().prefill_kv_split != 0) {
+      n_split = mi_tuning().prefill_kv_split > 1 ? mi_tuning().prefill_kv_split
+                                                 : prefill_kv_splits(T, Hq, Hkv, head_dim_v, max_kv_len);
+      const int64_t sp_bytes = (int64_t)n_split * T * Hq * (head_dim_v + 1) * (int64_t)sizeof(float);
+      if (n_split > 1 && workspace_bytes < sp_bytes) n_split = 1;
+      if (n_split > 1) {
+        p.split_o = reinterpret_cast<float*>(workspace);
+        p.split_lse = p.split_o + (int64_t)n_split * T * Hq * head_dim_v;
+        lgrid.y = n_split;
+      }
+    }
+    hipStream_t st = (hipStream_t)stream;
+    if (n_split > 1 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, true, 128, 192>), lgrid, dim3(512), 0, st, p);
+    else if (n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, true, 128, 192>), lgrid, dim3(512), 0, st, p);
+    else if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, false, 128, 192>), lgrid, dim3(512), 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, false, 128, 192>), lgrid, dim3(512), 0, st, p);
   } else {
     dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * 8);
     hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2>), grid, block, 0, (hipStream_t)stream, p);
   }
   if (timed) (void)hipEventRecord(ev_b, (hipStream_t)stream);
+  if (n_split > 1)
+    hipLaunchKernelGGL(prefill_split_merge_kernel, dim3(T, Hq), dim3(head_dim_v), 0, (hipStream_t)stream, p, n_split, head_dim_v);
   return mi_check_launch("mi_paged_prefill_attention_mla");
 }

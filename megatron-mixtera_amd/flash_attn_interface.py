@@ -79,7 +79,7 @@ def flash_attn_varlen_func(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor
         if k_scales is not None or v_scales is not None:
             raise NotImplementedError("no fp8 variant for caches with different key / value widths")
         return ops.paged_prefill_attention_mla(
-            q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table,
+            q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table, max_kv_len=max_seqlen_k,
             softmax_scale=softmax_scale if softmax_scale is not None else q.shape[-1] ** -0.5)
     return ops.paged_prefill_attention(q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table,
                                        softmax_scale=softmax_scale, max_kv_len=max_seqlen_k,

@@ -311,9 +311,12 @@ def paged_mla_decode_attention(q: Tensor, kv_cache: Tensor, kv_lens: Tensor, blo
 
 
 def paged_prefill_attention_mla(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seqlens_q: Tensor, kv_lens: Tensor,
-                                block_table: Tensor, *, softmax_scale: float, out: Optional[Tensor] = None) -> Tensor:
+                                block_table: Tensor, *, softmax_scale: float, max_kv_len: Optional[int] = None,
+                                out: Optional[Tensor] = None) -> Tensor:
     """Varlen causal attention over the decompressed caches of multi-latent attention: ``q`` ``[T, Hq, 192]``,
-    ``k_cache`` ``[N, C, H, 192]``, ``v_cache`` ``[N, C, H, 128]`` (each with its own strides) -> ``[T, Hq, 128]``."""
+    ``k_cache`` ``[N, C, H, 192]``, ``v_cache`` ``[N, C, H, 128]`` (each with its own strides) -> ``[T, Hq, 128]``.
+    ``max_kv_len`` (an upper bound of ``kv_lens``; default: what the block table can hold) sizes the split of
+    the keys when few query rows meet long contexts."""
     lib = _lib.load()
     stream = _stream(q)
     q3 = _qo_view(q, "q")
@@ -335,10 +338,19 @@ def paged_prefill_attention_mla(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_
         out = torch.empty(q.shape[:-1] + (Dv,), dtype=q.dtype, device=q.device)
     o3 = _qo_view(out, "out")
     _require(tuple(o3.shape) == (T, Hq, Dv), "out shape mismatch")
+    if max_kv_len is None:
+        max_kv_len = block_table.size(1) * C
+    need = lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, Dv, int(max_kv_len), 0)
+    if _workspace_override and _workspace_override[-1].numel() < need:
+        workspace = None  # the split of the keys is optional here: a caller-sized workspace that is too small turns it off
+    else:
+        workspace = _workspace(q.device, need)
+    ws_bytes = 0 if workspace is None else workspace.numel()
     _lib.check(lib.mi_paged_prefill_attention_mla(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), ksc, kst, ksh, v_cache.data_ptr(), vsc, vst, vsh,
         block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),
-        o3.data_ptr(), o3.stride(0), o3.stride(1), T, R, Hq, Hkv, Dk, Dv, C, float(softmax_scale), stream),
+        o3.data_ptr(), o3.stride(0), o3.stride(1), _ptr(workspace), ws_bytes, T, R, Hq, Hkv, Dk, Dv, C,
+        int(max_kv_len), float(softmax_scale), stream),
         "mi_paged_prefill_attention_mla")
     return out
 

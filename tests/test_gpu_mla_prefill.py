@@ -66,6 +66,29 @@ def test_mla_prefill_kernel_choice_and_grouped_heads(mi, dev, pingpong, Hq, Hkv)
     assert torch.isfinite(got).all() and (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
 
 
+@pytest.mark.parametrize("forced", [1, 3, 16])
+def test_mla_prefill_few_rows_over_long_contexts_split_the_keys(mi, dev, forced):
+    """A chunk of a prompt over a long history: the keys of a request are cut into ranges (automatic count,
+    or forced ones -- also more ranges than short requests have tiles), partials merged by a second kernel."""
+    H, chunk = 4, 64
+    q_lens, ctx = [40, 1, 17, 3], [3000, 2500, 0, 70]
+    q, kc, vc, cu_q, lens, bt = _case(mi, q_lens, ctx, H, chunk, seed=40 + forced)
+    q_pad = torch.cat([q, torch.randn(2, H, 192).bfloat16()])
+    mi.ops.set_tuning("prefill_kv_split", forced)
+    try:
+        out = mi.ops.paged_prefill_attention_mla(q_pad.to(dev), kc.to(dev), vc.to(dev), cu_q.to(dev), lens.to(dev),
+                                                 bt.to(dev), softmax_scale=0.07, max_kv_len=int(lens.max()))
+        torch.cuda.synchronize()
+    finally:
+        mi.ops.set_tuning("prefill_kv_split", 1)
+    ref = oa.paged_varlen_attention(q, kc, vc, cu_q, lens, bt, softmax_scale=0.07)
+    got = out.float().cpu()
+    T = q.size(0)
+    assert torch.isfinite(got).all() and (got[T:] == 0).all()
+    err = (got[:T] - ref).abs()
+    assert (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
+
+
 def test_mla_prefill_strided_caches_and_padding_rows(mi, dev):
     """Key and value caches as views of one wider buffer (as a split of the up-projection output gives
     them), token padding after the last request, trailing zero-length requests."""

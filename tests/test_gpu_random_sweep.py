@@ -236,6 +236,7 @@ def case_mla_prefill(mi, dev, rng, seed):
     if sum(q_lens) == 0:
         q_lens[0] = 5
     pp = rng.choice([1, 1, 2, 0])
+    ksplit = rng.choice([1, 1, 0, 3, 8])
     joint = rng.random() < 0.4
     _note(f"mla_prefill seed={seed} Hq={Hkv * G} Hkv={Hkv} chunk={chunk} q_lens={q_lens} ctx={ctx} pingpong={pp} joint={joint}")
     kv_lens = torch.tensor([a + b if a else 0 for a, b in zip(q_lens, ctx)], dtype=torch.int32)
@@ -251,6 +252,7 @@ def case_mla_prefill(mi, dev, rng, seed):
     else:
         kd_, vd_ = kc.to(dev), vc.to(dev)
     mi.ops.set_tuning("prefill_pingpong", pp)
+    mi.ops.set_tuning("prefill_kv_split", ksplit)
     try:
         qd_ = q.to(dev)
         poison(dev)
@@ -258,6 +260,7 @@ def case_mla_prefill(mi, dev, rng, seed):
         torch.cuda.synchronize()
     finally:
         mi.ops.set_tuning("prefill_pingpong", 1)
+        mi.ops.set_tuning("prefill_kv_split", 1)
     ref = oa.paged_varlen_attention(q, kc, vc, cu_q, kv_lens, bt, softmax_scale=0.08)
     close(out, ref, 2e-2, "mla prefill")
 
