@@ -14,6 +14,7 @@ from pathlib import Path
 
 PKG_DIR = Path(__file__).resolve().parent
 CSRC = PKG_DIR / "csrc"
+INCLUDE = PKG_DIR.parent / "include"   # the public header: every entry point is compiled against it
 LIB_NAME = "libmi355_decode.so"
 LIB_PATH = PKG_DIR / LIB_NAME
 
@@ -43,7 +44,7 @@ def sources() -> list[Path]:
 
 def build_library(verbose: bool = False) -> Path:
     """Compile all kernels into ``libmi355_decode.so`` (always recompiles)."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(CSRC), *map(str, sources()), "-o", str(LIB_PATH)]
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(CSRC), "-I", str(INCLUDE), *map(str, sources()), "-o", str(LIB_PATH)]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

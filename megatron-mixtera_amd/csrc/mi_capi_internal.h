@@ -5,22 +5,10 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-// Return codes of every entry point (0 = enqueued, negative = rejected, nothing launched).
-enum {
-  MI_OK = 0,
-  MI_ERR_NULL = -1,         // a required pointer is null
-  MI_ERR_SHAPE = -2,        // sizes inconsistent with each other
-  MI_ERR_ALIGN = -3,        // pointer or stride breaks the 16-byte row alignment
-  MI_ERR_UNSUPPORTED = -4,  // valid request this build has no kernel for
-  MI_ERR_WORKSPACE = -5,    // caller-provided workspace too small
-  MI_ERR_LAUNCH = -6,       // the HIP runtime refused the launch
-};
-
-// KV storage formats.
-enum { MI_KV_BF16 = 0, MI_KV_FP8_E4M3 = 1 };
-
-// Norm applied to the head vectors before RoPE.
-enum { MI_NORM_NONE = 0, MI_NORM_RMS = 1, MI_NORM_L2 = 2 };
+// Return codes (MI_OK, MI_ERR_*), KV storage formats (MI_KV_*), norm kinds (MI_NORM_*) and the prototype
+// of every entry point come from the public header, so a definition that drifts from its declaration
+// does not compile.
+#include "mi355_decode.h"
 
 struct MiTuning {
   int decode_tile_subtiles;  // 16-token sub-tiles per loop iteration of the decode kernel: 0 = automatic, 1, 2, 4 (fp8)

@@ -18,8 +18,6 @@
 #include "mi_common.h"
 #include "mi_capi_internal.h"
 
-extern "C" int64_t mi_decode_workspace_bytes(int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t);
-
 namespace mi {
 
 struct PrefillParams {

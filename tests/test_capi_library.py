@@ -1,6 +1,14 @@
-"""The C-ABI library loads and exports exactly what include/mi355_decode.h declares (no compute calls)."""
+"""The C-ABI library loads and exports exactly what include/mi355_decode.h declares (no compute calls).
+
+Three copies of every prototype exist: the public header, the definitions in ``csrc/*.hip`` and the ctypes
+table ``_lib.SIGNATURES``.  The definitions are compiled against the header (every source includes it, and a
+definition with C linkage that differs from its declaration is a compile error); the tests below parse the
+header and compare it, type by type, with the ctypes table, and build a C99 consumer against header and library.
+"""
 import ctypes
 import re
+import shutil
+import subprocess
 from pathlib import Path
 
 import pytest
@@ -14,6 +22,64 @@ def declared_functions():
     text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
     text = text[text.index('extern "C"'):]
     return re.findall(r"\b(mi_[a-z0-9_]+)\s*\(", text)
+
+
+def declared_prototypes():
+    """name -> (return type, [argument types]) with the C types normalised to ctypes classes."""
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    text = text[text.index('extern "C"'):]
+
+    def ctype(decl: str, is_return: bool = False):
+        decl = decl.strip()
+        if "*" in decl:
+            return ctypes.c_char_p if re.match(r"const\s+char\s*\*", decl) else ctypes.c_void_p
+        base = decl.split()[0] if not is_return else decl
+        return {"int": ctypes.c_int, "int32_t": ctypes.c_int32, "int64_t": ctypes.c_int64,
+                "float": ctypes.c_float}[base]
+
+    protos = {}
+    for m in re.finditer(r"([A-Za-z_][A-Za-z0-9_ ]*?\**)\s*\b(mi_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        ret, name, args = m.group(1), m.group(2), m.group(3).strip()
+        argtypes = [] if args in ("", "void") else [ctype(a) for a in args.split(",")]
+        protos[name] = (ctype(ret, is_return=True), argtypes)
+    return protos
+
+
+def test_ctypes_table_matches_the_header_type_by_type(mi):
+    protos = declared_prototypes()
+    assert set(protos) == set(declared_functions())
+    for name, (ret, args) in protos.items():
+        res, argtypes = mi._lib.SIGNATURES[name]
+        assert res is ret, f"{name}: return type {res} in the ctypes table, {ret} in the header"
+        assert len(argtypes) == len(args), f"{name}: {len(argtypes)} arguments in the ctypes table, {len(args)} in the header"
+        for i, (a, b) in enumerate(zip(argtypes, args)):
+            assert a is b, f"{name}: argument {i} is {a} in the ctypes table, {b} in the header"
+
+
+def test_the_parser_sees_a_transposed_argument():
+    """The comparison above is only worth something if a swapped int32 / int64 pair changes the parse."""
+    protos = declared_prototypes()
+    ret, args = protos["mi_kv_append"]
+    assert ret is ctypes.c_int and args[2] is ctypes.c_int64 and args[9] is ctypes.c_int32
+    assert protos["mi_last_error"] == (ctypes.c_char_p, [])
+    assert protos["mi_decode_workspace_bytes"][0] is ctypes.c_int64
+    assert protos["mi_set_tuning"][1] == [ctypes.c_char_p, ctypes.c_int32]
+
+
+@pytest.mark.skipif(shutil.which("gcc") is None, reason="needs a C compiler")
+def test_c99_consumer_compiles_links_and_runs(mi, tmp_path):
+    """A plain C99 program includes the header (-Wall -Werror -pedantic), links the library and makes calls that
+    need no GPU: the version, a no-op append, a rejected append and its message."""
+    src = Path(__file__).with_name("capi_consumer.c")
+    exe = tmp_path / "capi_consumer"
+    lib_dir = mi._lib.LIB_PATH.parent
+    cmd = ["gcc", "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", str(HEADER.parent), str(src),
+           "-L", str(lib_dir), "-lmi355_decode", f"-Wl,-rpath,{lib_dir}", "-o", str(exe)]
+    built = subprocess.run(cmd, capture_output=True, text=True)
+    assert built.returncode == 0, built.stderr
+    ran = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert ran.returncode == 0, ran.stdout + ran.stderr
+    assert "capi_consumer ok" in ran.stdout
 
 
 def test_header_declares_the_expected_entry_points():
