@@ -168,6 +168,29 @@ int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_str
                               void* stream);
 
 /*
+ * mi_paged_decode_attention for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments and results as mi_paged_decode_attention, minus the workspace: the
+ * partials live in a device array of MI_NOALLOC_SCRATCH_BYTES that is part of the library image
+ * (one copy per GPU the library runs on, held until the process ends).  Sizes for which
+ * mi_decode_workspace_bytes() exceeds that are rejected with MI_ERR_WORKSPACE.  The call allocates
+ * and frees nothing (keep mi_profile_enable off: it creates events).  All calls on one GPU share the
+ * array: calls that overlap on one GPU (two streams, two host threads) race; calls on one stream
+ * are ordered and need no clearing in between.  The first call on a device looks the array's
+ * address up (hipGetSymbolAddress), so make it before a stream capture starts.
+ */
+#define MI_NOALLOC_SCRATCH_BYTES (16 * 1024 * 1024)
+int mi_paged_decode_attention_noalloc(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
+                                      const void* k_cache, const void* v_cache, int64_t kv_stride_chunk,
+                                      int64_t kv_stride_tok, int64_t kv_stride_head,
+                                      const int32_t* block_table, int64_t bt_stride,
+                                      const int32_t* kv_lens, void* out, int64_t o_stride_tok,
+                                      int64_t o_stride_head, int32_t R, int32_t Hq, int32_t Hkv,
+                                      int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len,
+                                      int32_t split_tokens, float softmax_scale, int32_t kv_dtype,
+                                      const float* k_scales, const float* v_scales, void* stream);
+
+/*
  * Decode attention over the latent cache of multi-latent attention (absorbed form).
  * Replaces flash_mla_with_kvcache(q, kv_cache.unsqueeze(-2), block_table, cache_seqlens, head_dim_v,
  * tile_scheduler_metadata, num_splits, softmax_scale=, causal=True) together with get_mla_metadata

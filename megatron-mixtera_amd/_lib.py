@@ -38,6 +38,10 @@ SIGNATURES = {
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _I64, _I64, _P, _I64,
          _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P, _P]),
+    "mi_paged_decode_attention_noalloc": (
+        c_int,
+        [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _I64, _I64,
+         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P, _P]),
     "mi_mla_decode_workspace_bytes": (_I64, [_I32, _I32, _I32]),
     "mi_paged_mla_decode_attention": (
         c_int, [_P, _I64, _I64, _P, _I64, _I64, _P, _I64, _P, _P, _I64, _I64, _P, _I64,

@@ -963,6 +963,62 @@ extern "C" int mi_paged_decode_attention(
 }
 
 // ---------------------------------------------------------------------------------------------
+// Decode attention for callers that cannot allocate (code under HIP graph capture, serving loops and
+// harnesses that forbid hipMalloc): the partials and the per-request segment records live in a
+// file-scope device array instead of a caller workspace.  Every GPU the library runs on holds its own
+// copy of the array until the process ends; `scratch` below is only the host-side stand-in of the
+// symbol, so its device address is looked up once per device and only that address is ever handed to
+// a kernel.
+// ---------------------------------------------------------------------------------------------
+namespace {
+constexpr int64_t kNoAllocScratchBytes = (int64_t)MI_NOALLOC_SCRATCH_BYTES;
+}
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+static std::atomic<void*> g_scratch_ptr[64];  // per device: address of that device's copy of `scratch`
+
+static int noalloc_scratch(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64)
+    return mi_fail(MI_ERR_LAUNCH, "mi_paged_decode_attention_noalloc: cannot identify the current device");
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {  // first call on this device (several host threads may race here: they all get the same address)
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      (void)hipGetLastError();
+      return mi_fail(MI_ERR_LAUNCH, "mi_paged_decode_attention_noalloc: hipGetSymbolAddress(scratch) failed");
+    }
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return MI_OK;
+}
+
+extern "C" int mi_paged_decode_attention_noalloc(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
+    const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
+    const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
+    int64_t o_stride_tok, int64_t o_stride_head, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
+    int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens, float softmax_scale, int32_t kv_dtype,
+    const float* k_scales, const float* v_scales, void* stream) {
+  (void)max_kv_len;
+  if (R > 0 && Hq > 0 && Hkv > 0 && head_dim > 0 &&
+      mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, chunk_tokens, max_kv_len, split_tokens) > kNoAllocScratchBytes)
+    return mi_fail(MI_ERR_WORKSPACE,
+                   "mi_paged_decode_attention_noalloc: these sizes need more than the 16 MiB of built-in scratch "
+                   "(see mi_decode_workspace_bytes); use mi_paged_decode_attention with a workspace");
+  void* ptr = nullptr;
+  const int rc = noalloc_scratch(&ptr);
+  if (rc != MI_OK) return rc;
+  // Nothing in the scratch has to start at zero: every partial, log-sum-exp and segment record the merge
+  // kernel reads was written by the streaming kernel of the same call, so the previous call's contents
+  // (a larger batch's, say) are never looked at.
+  return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
+                             kv_stride_head, block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok,
+                             o_stride_head, ptr, kNoAllocScratchBytes, R, Hq, Hkv, head_dim, chunk_tokens,
+                             split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
 // Multi-latent attention (absorbed decode): one shared latent row per token, every query head
 // attends to it.  The streaming kernel sees the 16-head query groups as "KV heads" whose cache
 // head stride is zero, and is handed the same buffer as key and value cache.

@@ -278,6 +278,48 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
     return out
 
 
+def paged_decode_attention_noalloc(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens: Tensor, block_table: Tensor,
+                                   out: Tensor, *, softmax_scale: Optional[float] = None,
+                                   max_kv_len: Optional[int] = None, split_tokens: int = 0,
+                                   k_scales: Optional[Tensor] = None, v_scales: Optional[Tensor] = None) -> Tensor:
+    """:func:`paged_decode_attention` through the entry point that allocates nothing: the caller brings
+    ``out``, the partials live in the library's built-in device scratch (16 MiB per GPU; larger problems are
+    rejected).  Calls that overlap on one GPU share that scratch and race."""
+    lib = _lib.load()
+    stream = _stream(q)
+    q3 = _qo_view(q, "q")
+    R, Hq, D = q3.shape
+    N, C, Hkv, Dk = k_cache.shape
+    _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
+    fp8 = k_cache.element_size() == 1
+    _require(fp8 or k_cache.dtype == torch.bfloat16, "KV cache must be bf16 or a one-byte fp8 type")
+    _require(v_cache.dtype == k_cache.dtype, "k_cache / v_cache dtypes differ")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
+    _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
+    _require(kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "kv_lens must be contiguous int32")
+    _require(block_table.size(0) >= R and kv_lens.numel() >= R, "block_table / kv_lens shorter than the batch")
+    if fp8:
+        _require(k_scales is not None and v_scales is not None, "fp8 cache needs k_scales and v_scales")
+        _require(k_scales.dtype == torch.float32 and v_scales.dtype == torch.float32
+                 and k_scales.is_contiguous() and v_scales.is_contiguous()
+                 and tuple(k_scales.shape) == (N, Hkv) and tuple(v_scales.shape) == (N, Hkv),
+                 "scales must be contiguous fp32 [N, Hkv]")
+    o3 = _qo_view(out, "out")
+    _require(tuple(o3.shape) == (R, Hq, D), "out shape mismatch")
+    if max_kv_len is None:
+        max_kv_len = block_table.size(1) * C
+    if softmax_scale is None:
+        softmax_scale = D ** -0.5
+    _lib.check(lib.mi_paged_decode_attention_noalloc(
+        q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
+        block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
+        R, Hq, Hkv, D, C, int(max_kv_len), int(split_tokens), float(softmax_scale),
+        MI_KV_FP8_E4M3 if fp8 else MI_KV_BF16, _ptr(k_scales), _ptr(v_scales), stream),
+        "mi_paged_decode_attention_noalloc")
+    return out
+
+
 def paged_mla_decode_attention(q: Tensor, kv_cache: Tensor, kv_lens: Tensor, block_table: Tensor, *,
                                softmax_scale: float, head_dim_v: int = 512, max_kv_len: Optional[int] = None,
                                out: Optional[Tensor] = None) -> Tensor:

@@ -19,6 +19,7 @@ int main(void) {
       (const void*)(size_t)mi_kv_append_decode, (const void*)(size_t)mi_kv_quantize_chunks_fp8,
       (const void*)(size_t)mi_kv_append_decode_fp8, (const void*)(size_t)mi_kv_append_fp8,
       (const void*)(size_t)mi_decode_workspace_bytes, (const void*)(size_t)mi_paged_decode_attention,
+      (const void*)(size_t)mi_paged_decode_attention_noalloc,
       (const void*)(size_t)mi_mla_decode_workspace_bytes, (const void*)(size_t)mi_paged_mla_decode_attention,
       (const void*)(size_t)mi_prefill_workspace_bytes, (const void*)(size_t)mi_paged_prefill_attention,
       (const void*)(size_t)mi_paged_prefill_attention_fp8, (const void*)(size_t)mi_paged_prefill_attention_mla,
@@ -39,6 +40,7 @@ int main(void) {
   if (rc != MI_ERR_NULL || !strstr(p_error(), "null")) return 3;
   if (mi_set_tuning("no_such_knob", 1) != MI_ERR_UNSUPPORTED) return 4;
   if (mi_decode_workspace_bytes(0, 8, 2, 128, 16, 16, 0) != 0) return 5;
+  if (MI_NOALLOC_SCRATCH_BYTES != 16 * 1024 * 1024) return 6;
   printf("capi_consumer ok (ABI revision %d)\n", p_version());
   return 0;
 }
