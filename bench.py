@@ -36,6 +36,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_226_800_000, "cfg4": 8_724_000_000, "cfg5": 9_070_100_000,
                               # the mixed step (profiles/paged_prefill_pp_kernel_cfg3_mfma.md): tile kernel, stream kernel
                               "cfg3_tile": 402_300_000, "cfg3_stream": 2_195_700_000}
+# Where each figure above was read, so that a reader of the JSON line can tell a stale constant from a fresh one:
+# the summary file and the last commit that touched the kernel when the counters were collected.
+TRAFFIC_SOURCE = {
+    "cfg2": "profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
+    "cfg4": "profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
+    "cfg5": "profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
+    "cfg3_tile": "profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
+    "cfg3_stream": "profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
+}
 
 
 # Single-kernel workloads for the rows built around the path (multi-latent decode, the tail of a step).
@@ -165,13 +174,65 @@ def run_secondary(args, mi, lib, torch, dev):
         "roofline": roofline}), flush=True)
 
 
+def run_stream_read(args, mi, torch, dev):
+    """Calibration leg: a plain read-only streaming kernel (csrc/bench/stream_read.hip, built into
+    libmi355_bench.so) over a buffer of ``--read-mib`` MiB -- what a kernel that does nothing but read reaches
+    on this box, i.e. the practical ceiling under the published 8 TB/s that the KV-streaming kernel is held against."""
+    path = mi._lib.PKG_DIR / "libmi355_bench.so"
+    if not path.exists():
+        print(f"{path} not found: build first (python megatron-mixtera_amd/build.py)", file=sys.stderr)
+        sys.exit(2)
+    blib = ctypes.CDLL(str(path))
+    blib.mi_bench_stream_read.restype = ctypes.c_int
+    blib.mi_bench_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_int32,
+                                          ctypes.c_int32, ctypes.c_void_p]
+    nbytes = args.read_mib << 20
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    wgs = cus * args.read_wgs_per_cu
+    sink = torch.zeros(wgs, dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    results = {}
+    for name, nt in (("nontemporal", 1), ("cacheable", 0)):
+        def step():
+            rc = blib.mi_bench_stream_read(src.data_ptr(), nbytes, sink.data_ptr(), wgs, nt, stream)
+            assert rc == 0
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        t0 = time.perf_counter()
+        for a, b in events:
+            a.record()
+            step()
+            b.record()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        ms = sorted(a.elapsed_time(b) for a, b in events)
+        results[name] = {"kernel_ms_mean": sum(ms) / len(ms), "kernel_ms_min": ms[0], "ms_per_step": elapsed * 1e3 / args.steps}
+    best = results["nontemporal"]
+    achieved = nbytes / best["kernel_ms_mean"] / 1e6
+    print(json.dumps({
+        "metric": "stream_read_GBps", "value": round(nbytes / (best["ms_per_step"] * 1e-3) / 1e9, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(best["ms_per_step"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
+        "config": {"workload": f"read-only streaming kernel over {args.read_mib} MiB, {wgs} workgroups of 512 threads, "
+                               f"four 16-byte loads per thread per iteration, non-temporal loads",
+                   "algorithmic_bytes_per_step": nbytes,
+                   "cacheable_loads_GBps": round(nbytes / results["cacheable"]["kernel_ms_mean"] / 1e6, 1),
+                   "best_launch_GBps": round(nbytes / best["kernel_ms_min"] / 1e6, 1)},
+        "roofline": {"bound": "hbm", "kernel": "stream_read_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "kernel_ms": round(best["kernel_ms_mean"], 5), "traffic": None}}), flush=True)
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", *SECONDARY_WORKLOADS],
+                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", *SECONDARY_WORKLOADS],
                     help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch; the "
                          "mla_* / prefill_d64 / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
     ap.add_argument("--split-tokens", type=int, default=0)
@@ -180,48 +241,124 @@ def parse_args():
     ap.add_argument("--hip-graph", action="store_true", help="replay the step as one captured HIP graph")
     ap.add_argument("--attention-only", action="store_true", help="time the attention call alone")
     ap.add_argument("--fp8-kv", action="store_true", help="cfg3 only: run the mixed batch over an fp8-e4m3 KV cache")
+    ap.add_argument("--read-mib", type=int, default=1146,
+                    help="stream_read only: buffer size (default: the 1.2 GB one cfg2 launch streams)")
+    ap.add_argument("--read-wgs-per-cu", type=int, default=2, help="stream_read only: workgroups per CU")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run a plain device copy of this many MiB (a known-size reference for "
                          "scaling hardware traffic counters collected by an external profiler)")
     return ap.parse_args()
 
 
-def cpu_baseline(case, cfg, sample_requests: int):
-    """Time the CPU checker on the first ``sample_requests`` requests of the same seeded batch."""
+def _compact_chunks(torch, table_rows, n_pool, *tensors):
+    """The chunks some block-table rows use, copied to the CPU and renumbered 0..n-1 (same logical contents)."""
+    rows = table_rows.cpu()
+    used = rows[rows >= 0].unique().long()
+    remap = torch.full((n_pool,), -1, dtype=torch.int32)
+    remap[used] = torch.arange(used.numel(), dtype=torch.int32)
+    new_rows = torch.where(rows >= 0, remap[rows.clamp(min=0).long()], rows)
+    return new_rows, [None if t is None else t[used.to(t.device)].cpu() for t in tensors]
+
+
+def _time_cpu(torch, one_pass, budget_s: float = 12.0):
+    """Median pass time after one warm-up: at least 3 timed passes, about ``budget_s`` seconds of CPU work."""
+    torch.set_num_threads(os.cpu_count() or 1)
+    times = []
+    budget = time.perf_counter() + budget_s
+    while len(times) < 4 or (time.perf_counter() < budget and len(times) < 200):
+        t0 = time.perf_counter()
+        one_pass()
+        times.append(time.perf_counter() - t0)
+    return sorted(times[1:])[len(times[1:]) // 2], len(times) - 1
+
+
+def cpu_baseline(case, cfg, sample_requests: int, qw, kw, table, attention_only: bool):
+    """Time the CPU checker on the first ``sample_requests`` requests of the same seeded batch, doing what the GPU
+    step does: unfused q/k RMSNorm + RoPE (op by op in bf16), the scatter append of the new key / value rows
+    (quantising for an fp8 cache), then gather through the block table + fp32 attention."""
     import torch
 
     from oracle import paged_attention as oa
+    from oracle import rope_norm as orn
 
     n = min(sample_requests, case.q.size(0))
     q = case.q[:n].cpu().squeeze(1)
-    rows = case.block_table[:n].cpu()
+    k_new = case.k_new[:n].cpu().squeeze(1)
+    v_new = case.v_new[:n].cpu().squeeze(1)
     lens = case.kv_lens[:n].cpu()
-    used = rows[rows >= 0].unique().long()
-    # compact the sample's chunks into a small CPU cache (same logical contents)
-    remap = torch.full((case.k_cache.size(0),), -1, dtype=torch.int32)
-    remap[used] = torch.arange(used.numel(), dtype=torch.int32)
-    kc = case.k_cache[used.to(case.k_cache.device)].cpu()
-    vc = case.v_cache[used.to(case.k_cache.device)].cpu()
-    if kc.dtype == torch.uint8:
-        ks = case.k_scales[used.to(case.k_cache.device)].cpu()
-        vs = case.v_scales[used.to(case.k_cache.device)].cpu()
-    else:
-        ks = vs = None
-    bt = torch.where(rows >= 0, remap[rows.clamp(min=0).long()], rows)
-    torch.set_num_threads(os.cpu_count() or 1)
-    times = []
-    budget = time.perf_counter() + 12.0  # about 12 s of CPU work, at least 3 timed passes
-    while len(times) < 4 or (time.perf_counter() < budget and len(times) < 200):
-        t0 = time.perf_counter()
-        oa.paged_decode_attention(q, kc, vc, lens, bt, k_scales=ks, v_scales=vs)
-        times.append(time.perf_counter() - t0)
-    t = sorted(times[1:])[len(times[1:]) // 2]
+    bt, (kc, vc, ks, vs) = _compact_chunks(torch, case.block_table[:n], case.k_cache.size(0), case.k_cache,
+                                           case.v_cache, case.k_scales, case.v_scales)
+    pos = lens.long() - 1
+    qw_c, kw_c, table_c = qw.cpu(), kw.cpu(), table.cpu()
+    rows, ids, loc = oa.decode_slots(bt, lens, cfg.chunk)
+
+    def one_pass():
+        qn = q
+        if not attention_only:
+            qn = orn.norm_rope(q, pos, table_c, norm="rms", weight=qw_c, eps=1e-5)
+            kn = orn.norm_rope(k_new, pos, table_c, norm="rms", weight=kw_c, eps=1e-5)
+            if cfg.fp8:
+                oa.kv_append_fp8(kc, ks, kn[rows], ids, loc)
+                oa.kv_append_fp8(vc, vs, v_new[rows], ids, loc)
+            else:
+                oa.kv_append(kc, vc, kn[rows], v_new[rows], ids, loc)
+        return oa.paged_decode_attention(qn, kc, vc, lens, bt, k_scales=ks, v_scales=vs)
+
+    t, passes = _time_cpu(torch, one_pass)
     nbytes = oa.decode_attention_bytes(lens.tolist(), cfg.Hq, cfg.Hkv, cfg.d, cfg.chunk,
                                        kv_bytes=1 if cfg.fp8 else 2, fp8_scales=cfg.fp8)
+    what = ("fp32 gather + softmax checker" if attention_only else
+            "unfused RMSNorm + RoPE, scatter append, then fp32 gather + softmax (oracle/rope_norm.py, oracle/paged_attention.py)")
     return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"first {n} of {case.q.size(0)} requests of the same seeded batch, fp32 gather + softmax "
-                      f"checker (oracle/paged_attention.py), median of {len(times) - 1} passes after 1 warm-up, "
-                      f"{t * 1e3:.1f} ms/pass"}
+            "sample": f"first {n} of {case.q.size(0)} requests of the same seeded batch: {what}; attention bytes of "
+                      f"the sample / pass time, median of {passes} passes after 1 warm-up, {t * 1e3:.1f} ms/pass"}
+
+
+def cpu_baseline_mixed(q, k_new, v_new, kc, vc, cu_q, lens, bt, qw, kw, table, n_prefill: int, n_decode: int,
+                       Hq: int, Hkv: int, d: int, chunk: int):
+    """The mixed step on the CPU checker for a bounded sample of the batch: the first ``n_prefill`` prefill
+    requests and the first ``n_decode`` one-token requests -- unfused RMSNorm + RoPE of their new tokens, scatter
+    append, varlen causal attention through the block table."""
+    import torch
+
+    from oracle import paged_attention as oa
+    from oracle import rope_norm as orn
+
+    lq_all = (cu_q[1:] - cu_q[:-1]).cpu()
+    pre = [r for r in range(lens.numel()) if int(lq_all[r]) > 1][:n_prefill]
+    dec = [r for r in range(lens.numel()) if int(lq_all[r]) == 1][:n_decode]
+    reqs = pre + dec
+    cu = cu_q.cpu()
+    tok = torch.cat([torch.arange(int(cu[r]), int(cu[r + 1])) for r in reqs])
+    qs, ks_new, vs_new = q[tok.to(q.device)].cpu(), k_new[tok.to(q.device)].cpu(), v_new[tok.to(q.device)].cpu()
+    lens_s = lens.cpu()[reqs]
+    lq = lq_all[reqs]
+    cu_s = torch.zeros(len(reqs) + 1, dtype=torch.int32)
+    cu_s[1:] = torch.cumsum(lq, 0)
+    bt_s, (kcc, vcc) = _compact_chunks(torch, bt[reqs], kc.size(0), kc, vc)
+    # per-token position, chunk and slot, as the context lays them out
+    req_of = torch.repeat_interleave(torch.arange(len(reqs)), lq.long())
+    pos = torch.arange(tok.numel()) - cu_s[req_of].long() + (lens_s.long() - lq.long())[req_of]
+    ids = bt_s.long()[req_of, pos // chunk]
+    loc = pos % chunk
+    qw_c, kw_c, table_c = qw.cpu(), kw.cpu(), table.cpu()
+
+    def one_pass():
+        qn = orn.norm_rope(qs, pos, table_c, norm="rms", weight=qw_c, eps=1e-5)
+        kn = orn.norm_rope(ks_new, pos, table_c, norm="rms", weight=kw_c, eps=1e-5)
+        oa.kv_append(kcc, vcc, kn, vs_new, ids, loc)
+        return oa.paged_varlen_attention(qn, kcc, vcc, cu_s, lens_s, bt_s)
+
+    t, passes = _time_cpu(torch, one_pass)
+    lk = lens_s.long()
+    is_pre = lq > 1
+    dec_bytes = oa.decode_attention_bytes(lk[~is_pre].tolist(), Hq, Hkv, d, chunk)
+    pre_bytes = int(lk[is_pre].sum()) * Hkv * d * 2 * 2 + int(lq[is_pre].sum()) * Hq * d * 4
+    return {"value": (dec_bytes + pre_bytes) / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{len(pre)} of the prefill requests ({int(lq[is_pre].sum())} new tokens) and {len(dec)} of the "
+                      f"one-token requests of the same seeded batch: unfused RMSNorm + RoPE, scatter append, varlen "
+                      f"causal attention through the block table (oracle/); the sample's algorithmic bytes / pass time, "
+                      f"median of {passes} passes after 1 warm-up, {t * 1e3:.1f} ms/pass"}
 
 
 def run_mixed_batch(args, mi, lib, torch, dev):
@@ -312,13 +449,18 @@ def run_mixed_batch(args, mi, lib, torch, dev):
         "roofline": {"bound": "mfma", "kernel": "paged_prefill_pp_kernel", "achieved": round(flops / tile_ms / 1e9, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / tile_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "kernel_ms": round(tile_ms, 5),
-                     "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_tile"]},
+                     "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_tile"],
+                     "traffic_source": None if args.fp8_kv else TRAFFIC_SOURCE["cfg3_tile"]},
         "roofline_decode_part": {"bound": "hbm", "kernel": "paged_decode_stream_kernel",
                                  "achieved": round(dec_bytes / stream_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
                                  "unit": "GB/s", "frac": round(dec_bytes / stream_ms / 1e6 / HBM_PEAK_GBPS, 4),
                                  "kernel_ms": round(stream_ms, 5),
-                                 "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_stream"]},
+                                 "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_stream"],
+                                 "traffic_source": None if args.fp8_kv else TRAFFIC_SOURCE["cfg3_stream"]},
     }
+    if not args.no_cpu_baseline and not args.fp8_kv:
+        result["cpu_baseline"] = cpu_baseline_mixed(q, k_new, v_new, kc, vc, cu_q, lens, bt, qw, kw, table,
+                                                    n_prefill=1, n_decode=15, Hq=Hq, Hkv=Hkv, d=d, chunk=chunk)
     print(json.dumps(result), flush=True)
 
 
@@ -345,6 +487,9 @@ def main():
 
     if args.workload == "cfg3":
         run_mixed_batch(args, mi, lib, torch, dev)
+        return
+    if args.workload == "stream_read":
+        run_stream_read(args, mi, torch, dev)
         return
     if args.workload in SECONDARY_WORKLOADS:
         run_secondary(args, mi, lib, torch, dev)
@@ -473,11 +618,12 @@ def main():
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "kernel_ms": round(kernel_ms, 5),
             "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
+            "traffic_source": TRAFFIC_SOURCE.get(args.workload),
         },
     }
     if not args.no_cpu_baseline:
         sample = {"cfg1": 4, "cfg2": 64, "cfg3_decode": 64, "cfg4": 1, "cfg5": 16}[args.workload]
-        result["cpu_baseline"] = cpu_baseline(case, cfg, sample)
+        result["cpu_baseline"] = cpu_baseline(case, cfg, sample, qw, kw, table, args.attention_only)
     print(json.dumps(result), flush=True)
 
 

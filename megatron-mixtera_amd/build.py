@@ -17,6 +17,8 @@ CSRC = PKG_DIR / "csrc"
 INCLUDE = PKG_DIR.parent / "include"   # the public header: every entry point is compiled against it
 LIB_NAME = "libmi355_decode.so"
 LIB_PATH = PKG_DIR / LIB_NAME
+# measurement aids of bench.py (a streaming-read kernel); not part of the product library or its ABI
+BENCH_LIB_PATH = PKG_DIR / "libmi355_bench.so"
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -42,9 +44,8 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def build_library(verbose: bool = False) -> Path:
-    """Compile all kernels into ``libmi355_decode.so`` (always recompiles)."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(CSRC), "-I", str(INCLUDE), *map(str, sources()), "-o", str(LIB_PATH)]
+def _hipcc(inputs: list[Path], output: Path, verbose: bool) -> None:
+    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(CSRC), "-I", str(INCLUDE), *map(str, inputs), "-o", str(output)]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -54,6 +55,13 @@ def build_library(verbose: bool = False) -> Path:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
     if verbose and out.strip():
         print(out)
+
+
+def build_library(verbose: bool = False) -> Path:
+    """Compile all kernels into ``libmi355_decode.so`` and the benchmark's measurement kernels into
+    ``libmi355_bench.so`` (always recompiles)."""
+    _hipcc(sources(), LIB_PATH, verbose)
+    _hipcc(sorted((CSRC / "bench").glob("*.hip")), BENCH_LIB_PATH, verbose)
     return LIB_PATH
 
 
