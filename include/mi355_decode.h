@@ -351,11 +351,14 @@ int mi_qkv_norm_rope_append(const void* mixed_qkv, int64_t qkv_stride_tok, void*
  * `active_requests_mask` int32 [total - paused], `new_tokens` int64 [total - paused];
  * `paused_tokens` int64 [max_requests] holds the tokens of the paused rows on entry and on exit;
  * `next_tokens_scratch` int64 [max_requests], `scratch` int32 [4 * max_requests].
- * Results: `newly_paused_request_ids` int32 [max_requests] and `counters` int32 [8] =
+ * Results: `newly_paused_request_ids` int32 [max_requests], `finished_request_ids` int32
+ * [max_requests] (the ids of the requests whose mask entry is 0, in row order -- what
+ * TextGenerationController.async_generate_output_tokens_dynamic_batch reads with nonzero + index at
+ * text_generation_controller.py:527-530) and `counters` int32 [8] =
  * {total_request_count, paused_request_count, active_token_count, chunk_count_avail,
  *  number of newly paused ids (-1 = none), status (0 ok, 1 mask/count mismatch - nothing was
  *  changed, 2 no active request left, 3 resumed request not at a chunk start), 1 if the context
- *  was emptied, 0}; the caller copies `counters` to the host after the call.
+ *  was emptied, number of finished ids}; the caller copies `counters` to the host after the call.
  */
 int mi_update_requests(int32_t* request_ids, int32_t* request_query_lengths,
                        int32_t* request_output_lengths, int32_t* request_kv_length_offsets,
@@ -367,8 +370,8 @@ int mi_update_requests(int32_t* request_ids, int32_t* request_query_lengths,
                        int64_t* token_to_local_position_within_kv_chunk, int32_t* chunk_bag,
                        const int32_t* active_requests_mask, const int64_t* new_tokens,
                        int64_t* paused_tokens, int64_t* next_tokens_scratch, int32_t* scratch,
-                       int32_t* newly_paused_request_ids, int32_t* counters,
-                       int32_t total_request_count, int32_t paused_request_count,
+                       int32_t* newly_paused_request_ids, int32_t* finished_request_ids,
+                       int32_t* counters, int32_t total_request_count, int32_t paused_request_count,
                        int32_t chunk_count_avail, int32_t gtd_chunk_count, int32_t gtd_request_count,
                        int32_t chunk_size_tokens, int32_t max_requests, void* stream);
 
@@ -390,6 +393,27 @@ int mi_decode_attention_state(const int32_t* request_kv_length_offsets,
                               int32_t active_request_count, int32_t active_token_count,
                               int32_t padded_active_token_count, int32_t dummy_chunk_idx,
                               void* stream);
+
+/*
+ * The prefill / mixed-step part of DynamicInferenceContext.initialize_attention_state
+ * (dynamic_context.py:733-741, 752-775, 794-821) as one kernel: everything mi_decode_attention_state
+ * writes, plus cu_query_seq_lengths_out / cu_kv_seq_lengths_out int32 [padded_request_count + 1] (running
+ * sums of the query and kv lengths; padded requests add nothing) and max_lengths_out int32 [2] = {largest
+ * query length, largest kv length} -- the two values the reference fetches with `.max().item()`
+ * (:772, :808).  The mirrors' padded rows must already be zero.
+ */
+int mi_step_attention_state(const int32_t* request_kv_length_offsets,
+                            const int32_t* request_query_lengths,
+                            const int32_t* request_to_kv_chunk_ids, int64_t table_stride,
+                            int32_t max_kv_chunk_count, int32_t* query_seq_lengths_out,
+                            int32_t* kv_seq_lengths_out, int32_t* cu_query_seq_lengths_out,
+                            int32_t* cu_kv_seq_lengths_out, int32_t* block_table_out,
+                            int64_t block_table_out_stride, int64_t* token_to_chunk_idx,
+                            int64_t* token_to_local_position_within_kv_chunk,
+                            int64_t* token_to_position_in_request, int32_t* max_lengths_out,
+                            int32_t paused_request_count, int32_t active_request_count,
+                            int32_t padded_request_count, int32_t active_token_count,
+                            int32_t padded_active_token_count, int32_t dummy_chunk_idx, void* stream);
 
 /*
  * DynamicInferenceContext.last_token_logits (dynamic_context.py:890-918) as one launch:

@@ -142,8 +142,14 @@ class PagedSelfAttentionCore(torch.nn.Module):
 
     def _attend(self, query: Tensor, ctx) -> Tensor:
         k_cache, v_cache, block_table = ctx.key_value_cache(self.layer_number)
-        cu_q, max_q = ctx.cu_query_lengths()
-        cu_k, kv_lens, max_k = ctx.cu_kv_lengths()
+        if hasattr(ctx, "attention_length_bounds"):
+            # the host-side bounds decide which kernel runs and how the keys are split; taking the exact
+            # maxima (cu_query_lengths / cu_kv_lengths, as the reference does) would wait for the device
+            cu_q, cu_k, kv_lens = ctx.cu_query_seq_lengths, ctx.cu_kv_seq_lengths, ctx.kv_seq_lengths
+            max_q, max_k = ctx.attention_length_bounds()
+        else:
+            cu_q, max_q = ctx.cu_query_lengths()
+            cu_k, kv_lens, max_k = ctx.cu_kv_lengths()
         k_scales, v_scales = ctx.key_value_scales(self.layer_number) if hasattr(ctx, "key_value_scales") else (None, None)
         out = flash_decode_and_prefill(query, k_cache, v_cache, max_q, max_k, cu_q, cu_k, kv_lens, block_table,
                                        softmax_scale=self.softmax_scale, k_scales=k_scales, v_scales=v_scales)

@@ -26,6 +26,7 @@ import torch.nn.functional as F
 from torch import Tensor
 
 from .. import ops
+from ..flash_attn_interface import note_kv_lengths
 from .dynamic_chunk_allocator import ChunkAllocator
 
 
@@ -288,8 +289,21 @@ class DynamicInferenceContext:
             self._next_tokens_buf = torch.zeros(self.max_requests, dtype=torch.long, device=dev)
             self._update_scratch = torch.zeros(4 * self.max_requests, dtype=torch.int32, device=dev)
             self._newly_paused_buf = torch.zeros(self.max_requests, dtype=torch.int32, device=dev)
+            self._finished_ids_buf = torch.zeros(self.max_requests, dtype=torch.int32, device=dev)
             self._counters = torch.zeros(8, dtype=torch.int32, device=dev)
             self._counters_host = torch.zeros(8, dtype=torch.int32, pin_memory=True)
+            # largest query / kv length of a prefill or mixed step: written by the attention-state kernel,
+            # copied to pinned memory behind an event and only waited for when somebody reads the value
+            self._max_lengths = torch.zeros(2, dtype=torch.int32, device=dev)
+            self._max_lengths_host = torch.zeros(2, dtype=torch.int32, pin_memory=True)
+            self._max_lengths_event = torch.cuda.Event()
+        self._max_lengths_pending = False
+        # what the host knows without asking the device: the longest prompt admitted since the last
+        # update_requests (every other active request has one query token) and a bound on the kv lengths
+        self._host_max_query_len = 1
+        self._host_kv_len_bound = 0
+        # ids of the requests that finished in the last update_requests (fused bookkeeping), else None
+        self.last_finished_request_ids = None
 
         self.reset_attention_state()
 
@@ -337,6 +351,48 @@ class DynamicInferenceContext:
 
     def has_unfinished_requests(self) -> bool:
         return self.total_request_count > 0
+
+    # max_seqlen_q / max_seqlen_k keep the reference's meaning (exact maxima on prefill / mixed steps).  With the
+    # fused bookkeeping they are produced on the GPU and fetched lazily: reading one of them waits for the small
+    # copy issued by initialize_attention_state; a step that never reads them never waits.
+    def _resolve_max_lengths(self) -> None:
+        if self._max_lengths_pending:
+            self._max_lengths_event.synchronize()
+            self._max_seqlen_q, self._max_seqlen_k = self._max_lengths_host.tolist()
+            self._max_lengths_pending = False
+
+    @property
+    def max_seqlen_q(self):
+        self._resolve_max_lengths()
+        return self._max_seqlen_q
+
+    @max_seqlen_q.setter
+    def max_seqlen_q(self, value) -> None:
+        self._max_seqlen_q = value
+
+    @property
+    def max_seqlen_k(self):
+        self._resolve_max_lengths()
+        return self._max_seqlen_k
+
+    @max_seqlen_k.setter
+    def max_seqlen_k(self, value) -> None:
+        self._max_seqlen_k = value
+
+    def attention_length_bounds(self) -> Tuple[int, int]:
+        """``(max query length, upper bound of the kv lengths)`` of this step from what the host already knows,
+        without waiting for the device: 1 on decode steps (the padded token count on graph steps), else the
+        longest prompt admitted since the last ``update_requests``; kv lengths are bounded by the longest
+        prompt so far plus the steps taken, and by ``max_sequence_length``.  The attention kernels only need
+        bounds (which kernel, how to split the keys), not the exact maxima."""
+        if self.is_decode_only():
+            q_max = 1
+        elif self.using_cuda_graph_this_step():
+            q_max = self.padded_active_token_count
+        else:
+            q_max = max(1, self._host_max_query_len)
+        k_bound = min(self.max_sequence_length, max(1, self._host_kv_len_bound))
+        return q_max, k_bound
 
     def cu_query_lengths(self) -> Tuple[Optional[Tensor], int]:
         return self.cu_query_seq_lengths, self.max_seqlen_q
@@ -508,6 +564,8 @@ class DynamicInferenceContext:
     # ------------------------------------------------------------------ per-step attention state
     def reset_attention_state(self) -> None:
         """Forget the per-step attention metadata (the fixed-address mirrors are zeroed)."""
+        self._max_lengths_pending = False
+        note_kv_lengths(None, None)
         self.max_seqlen_q = None
         self.max_seqlen_k = None
         self.cu_query_seq_lengths = None
@@ -568,6 +626,26 @@ class DynamicInferenceContext:
         self.padded_active_request_count = padded if (graph_step or decode_only) else n_active_req
 
         act = self._active()
+        if self.fused_bookkeeping and not decode_only:
+            # Prefill / mixed step, one kernel and no wait: lengths, their running sums and the block table
+            # go into the fixed-address mirrors (as on graph steps; same values as the reference's fresh
+            # tensors), the padded token rows are pointed at the dummy chunk, and the two maxima follow
+            # through pinned memory for whoever reads max_seqlen_q / max_seqlen_k.
+            R = self.padded_active_request_count
+            ops.step_attention_state(self, n_active_req, R, padded)
+            self.kv_seq_lengths = self.kv_seq_lengths_cudagraph_only[:R]
+            self.block_table = self.request_to_kv_chunk_ids_cudagraph_only[:R]
+            self.cu_query_seq_lengths = self.cu_query_seq_lengths_cudagraph_only[: R + 1]
+            self.cu_kv_seq_lengths = self.cu_kv_seq_lengths_cudagraph_only[: R + 1]
+            if graph_step:
+                self.max_seqlen_q = padded
+                self.max_seqlen_k = self.max_sequence_length
+            else:
+                self._max_lengths_host.copy_(self._max_lengths, non_blocking=True)
+                self._max_lengths_event.record(torch.cuda.current_stream(self.device))
+                self._max_lengths_pending = True
+            note_kv_lengths(self.cu_kv_seq_lengths, self.kv_seq_lengths)
+            return
         if self.fused_bookkeeping and (graph_step or decode_only):
             # one kernel: padded token rows + fixed-address mirrors of lengths and block table
             ops.decode_attention_state(self, n_active_req, padded)
@@ -614,6 +692,7 @@ class DynamicInferenceContext:
             self.cu_kv_seq_lengths[1:] = torch.cumsum(kv_lens, dim=0)
             self.max_seqlen_k = kv_lens.max().item()
             self.block_table = self.request_to_kv_chunk_ids[act]
+        note_kv_lengths(self.cu_kv_seq_lengths, self.kv_seq_lengths)
 
     def reset(self) -> None:
         """Return to the empty state without reallocating anything (graphs keep the addresses)."""
@@ -642,6 +721,9 @@ class DynamicInferenceContext:
 
         self.reset_attention_state()
         self.chunk_allocator.reset()
+        self._host_max_query_len = 1
+        self._host_kv_len_bound = 0
+        self.last_finished_request_ids = None
 
     def current_input_and_position_ids(self, *, num_warmup_tokens: Optional[int] = None) -> Tuple[Tensor, Tensor]:
         """``[1, T]`` views of this step's input ids and position ids."""
@@ -706,6 +788,8 @@ class DynamicInferenceContext:
 
         self.total_request_count += 1
         self.active_token_count += length
+        self._host_max_query_len = max(self._host_max_query_len, length)
+        self._host_kv_len_bound = max(self._host_kv_len_bound, length)
 
     def _move_book_keeping_tensors(self, src_idxs, dst_idxs, next_tokens):
         """``row[dst] = row[src]`` for every per-request row (right-hand sides gathered first)."""
@@ -731,8 +815,12 @@ class DynamicInferenceContext:
         rows are rewritten for a one-token-per-request decode step.  Returns the ids of
         requests that were newly paused and stay paused, or ``None``.
         """
+        # after this call every active request has one query token and one more key
+        self._host_max_query_len = 1
+        self._host_kv_len_bound = min(self._host_kv_len_bound + 1, self.max_sequence_length)
         if self.fused_bookkeeping:
             return self._update_requests_fused(active_requests_mask, new_tokens)
+        self.last_finished_request_ids = None
         n_continue = (active_requests_mask == 1).sum().item()
         n_finished = (active_requests_mask == 0).sum().item()
         assert n_continue + n_finished + self.paused_request_count == self.total_request_count
@@ -842,8 +930,9 @@ class DynamicInferenceContext:
         ops.update_requests(self, mask, tokens)
         self._counters_host.copy_(self._counters, non_blocking=True)
         torch.cuda.current_stream(dev).synchronize()
-        total, paused, active, avail, n_newly, status, was_reset, _ = self._counters_host.tolist()
+        total, paused, active, avail, n_newly, status, was_reset, n_finished = self._counters_host.tolist()
         assert status != 1, "active + finished + paused requests != total_request_count"
+        self.last_finished_request_ids = self._finished_ids_buf[:n_finished].clone()
         self.reset_attention_state()
         assert status != 2, "active_request_count == 0."
         assert status != 3, (

@@ -30,6 +30,7 @@ struct UpdateParams {
   int64_t* next_tokens;      // scratch [max_requests]
   int32_t* scratch;          // scratch [4 * max_requests]
   int32_t* newly_paused;     // out [max_requests]
+  int32_t* finished;         // out [max_requests]: ids of the requests that finished, in row order
   int32_t* counters;         // out [8]
   int32_t total, paused, avail, gtd_chunks, gtd_requests, chunk, max_requests;
 };
@@ -143,13 +144,14 @@ __global__ __launch_bounds__(kThreads) void update_requests_kernel(UpdateParams 
   if (n_cont + P0 == 0) {
     if (n_fin > 0) {
       const int nf = compact(n, P0, list_a, [&](int i) { return p.mask[i] == 0; }, sh);
+      for (int k = t; k < nf; k += kThreads) p.finished[k] = p.ids[list_a[k]];
       avail = release_rows(p, list_a, nf, avail, counts, sh);
     }
     for (int64_t i = t; i < (int64_t)p.max_requests * p.M; i += kThreads)
       p.table[(i / p.M) * p.table_stride + (i % p.M)] = -1;
     if (t == 0) {
       p.counters[0] = 0; p.counters[1] = P0; p.counters[2] = 0; p.counters[3] = avail;
-      p.counters[4] = -1; p.counters[5] = 0; p.counters[6] = 1;
+      p.counters[4] = -1; p.counters[5] = 0; p.counters[6] = 1; p.counters[7] = n_fin;
     }
     return;
   }
@@ -162,6 +164,8 @@ __global__ __launch_bounds__(kThreads) void update_requests_kernel(UpdateParams 
   // ---- 4. finished requests: release chunks, fill their holes from the right ---------------
   if (n_fin > 0) {
     const int nf = compact(n, P0, list_a, [&](int i) { return p.mask[i] == 0; }, sh);
+    // their ids, in row order (what the caller of the step reports as finished), before any row moves
+    for (int k = t; k < nf; k += kThreads) p.finished[k] = p.ids[list_a[k]];
     avail = release_rows(p, list_a, nf, avail, counts, sh);
     for (int64_t i = t; i < (int64_t)nf * p.M; i += kThreads)
       p.table[(int64_t)list_a[i / p.M] * p.table_stride + (i % p.M)] = -1;
@@ -220,7 +224,7 @@ __global__ __launch_bounds__(kThreads) void update_requests_kernel(UpdateParams 
   paused -= n_resume;
   n_cont += n_resume;
   if (n_cont <= 0) {
-    if (t == 0) p.counters[5] = 2;
+    if (t == 0) { p.counters[5] = 2; p.counters[7] = n_fin; }
     return;
   }
   if (n_newly >= 0 && n_resume > 0) n_newly = max(0, n_newly - n_resume);
@@ -257,7 +261,7 @@ __global__ __launch_bounds__(kThreads) void update_requests_kernel(UpdateParams 
   avail -= n_resume;
   if (t == 0) {
     p.counters[0] = total; p.counters[1] = paused; p.counters[2] = n_cont; p.counters[3] = avail;
-    p.counters[4] = n_newly; p.counters[5] = (red[0] >> 30) ? 3 : 0; p.counters[6] = 0;
+    p.counters[4] = n_newly; p.counters[5] = (red[0] >> 30) ? 3 : 0; p.counters[6] = 0; p.counters[7] = n_fin;
   }
 }
 
@@ -290,6 +294,74 @@ __global__ __launch_bounds__(256) void decode_attention_state_kernel(DecodeState
   }
 }
 
+
+struct StepStateParams {
+  const int32_t* kv_off; const int32_t* q_len; const int32_t* table; int64_t table_stride; int32_t M;
+  int32_t* q_lens_out; int32_t* kv_lens_out; int32_t* cu_q_out; int32_t* cu_kv_out;
+  int32_t* table_out; int64_t table_out_stride;
+  int64_t* tok_chunk; int64_t* tok_local; int64_t* tok_in_req;
+  int32_t* maxes;  // out [2]: largest query length, largest kv length
+  int32_t paused, n_active, R, padded, active_tokens, dummy_chunk;
+};
+
+// initialize_attention_state of a prefill / mixed step: what decode_attention_state_kernel does, plus the
+// running sums of query and kv lengths over the R (padded) requests and the two maxima.
+// Workgroup 0 (1024 threads) owns the length rows: a block-wide scan over R entries; the other
+// workgroups copy the block-table rows of the active requests.
+__global__ __launch_bounds__(1024) void step_attention_state_kernel(StepStateParams p) {
+  const int t = threadIdx.x;
+  if (blockIdx.x > 0) {
+    for (int i = blockIdx.x - 1; i < p.n_active; i += gridDim.x - 1) {
+      const int r = p.paused + i;
+      for (int j = t; j < p.M; j += 1024)
+        p.table_out[(int64_t)i * p.table_out_stride + j] = p.table[(int64_t)r * p.table_stride + j];
+    }
+    return;
+  }
+  __shared__ int sh_q[1024], sh_k[1024];
+  __shared__ int red[2];
+  if (t < 2) red[t] = 0;
+  const int seg = (p.R + 1023) / 1024;
+  const int a = min(t * seg, p.R), b = min(a + seg, p.R);
+  int sq = 0, sk = 0, mq = 0, mk = 0;
+  for (int i = a; i < b; ++i) {
+    const int q = i < p.n_active ? p.q_len[p.paused + i] : 0;
+    const int k = i < p.n_active ? p.kv_off[p.paused + i] + q : 0;
+    if (i < p.n_active) {
+      p.q_lens_out[i] = q;
+      p.kv_lens_out[i] = k;
+    }
+    sq += q; sk += k;
+    mq = max(mq, q); mk = max(mk, k);
+  }
+  sh_q[t] = sq; sh_k[t] = sk;
+  __syncthreads();
+  for (int o = 1; o < 1024; o <<= 1) {
+    const int vq = t >= o ? sh_q[t - o] : 0, vk = t >= o ? sh_k[t - o] : 0;
+    __syncthreads();
+    sh_q[t] += vq; sh_k[t] += vk;
+    __syncthreads();
+  }
+  int cq = sh_q[t] - sq, ck = sh_k[t] - sk;  // sums before this thread's rows
+  if (t == 0) { p.cu_q_out[0] = 0; p.cu_kv_out[0] = 0; }
+  for (int i = a; i < b; ++i) {
+    const int q = i < p.n_active ? p.q_len[p.paused + i] : 0;
+    const int k = i < p.n_active ? p.kv_off[p.paused + i] + q : 0;
+    cq += q; ck += k;
+    p.cu_q_out[i + 1] = cq;
+    p.cu_kv_out[i + 1] = ck;
+  }
+  atomicMax(&red[0], mq);
+  atomicMax(&red[1], mk);
+  for (int tk = p.active_tokens + t; tk < p.padded; tk += 1024) {
+    p.tok_chunk[tk] = p.dummy_chunk;
+    p.tok_local[tk] = 0;
+    p.tok_in_req[tk] = 0;
+  }
+  __syncthreads();
+  if (t < 2) p.maxes[t] = red[t];
+}
+
 }  // namespace mi
 
 using namespace mi;
@@ -302,7 +374,7 @@ extern "C" int mi_update_requests(
     int64_t* token_to_request_idx, int64_t* token_to_position_in_request, int64_t* token_to_chunk_idx,
     int64_t* token_to_local_position_within_kv_chunk, int32_t* chunk_bag, const int32_t* active_requests_mask,
     const int64_t* new_tokens, int64_t* paused_tokens, int64_t* next_tokens_scratch, int32_t* scratch,
-    int32_t* newly_paused_request_ids, int32_t* counters, int32_t total_request_count,
+    int32_t* newly_paused_request_ids, int32_t* finished_request_ids, int32_t* counters, int32_t total_request_count,
     int32_t paused_request_count, int32_t chunk_count_avail, int32_t gtd_chunk_count,
     int32_t gtd_request_count, int32_t chunk_size_tokens, int32_t max_requests, void* stream) {
   if (!request_ids || !request_query_lengths || !request_output_lengths || !request_kv_length_offsets ||
@@ -310,7 +382,7 @@ extern "C" int mi_update_requests(
       !request_to_kv_chunk_ids || !token_to_input_ids || !token_to_pos_ids || !token_to_request_idx ||
       !token_to_position_in_request || !token_to_chunk_idx || !token_to_local_position_within_kv_chunk ||
       !chunk_bag || !active_requests_mask || !new_tokens || !paused_tokens || !next_tokens_scratch || !scratch ||
-      !newly_paused_request_ids || !counters)
+      !newly_paused_request_ids || !finished_request_ids || !counters)
     return mi_fail(MI_ERR_NULL, "mi_update_requests: null pointer argument");
   if (total_request_count < 0 || paused_request_count < 0 || paused_request_count > total_request_count ||
       total_request_count > max_requests || max_kv_chunk_count <= 0 || chunk_size_tokens <= 0)
@@ -325,7 +397,7 @@ extern "C" int mi_update_requests(
   p.tok_local = token_to_local_position_within_kv_chunk;
   p.bag = chunk_bag; p.mask = active_requests_mask; p.new_tokens = new_tokens;
   p.paused_tokens = paused_tokens; p.next_tokens = next_tokens_scratch; p.scratch = scratch;
-  p.newly_paused = newly_paused_request_ids; p.counters = counters;
+  p.newly_paused = newly_paused_request_ids; p.finished = finished_request_ids; p.counters = counters;
   p.total = total_request_count; p.paused = paused_request_count; p.avail = chunk_count_avail;
   p.gtd_chunks = gtd_chunk_count; p.gtd_requests = gtd_request_count; p.chunk = chunk_size_tokens;
   p.max_requests = max_requests;
@@ -360,4 +432,36 @@ extern "C" int mi_decode_attention_state(
   const int blocks = active_request_count > 0 ? active_request_count : 1;
   hipLaunchKernelGGL(decode_attention_state_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, p);
   return mi_check_launch("mi_decode_attention_state");
+}
+
+extern "C" int mi_step_attention_state(
+    const int32_t* request_kv_length_offsets, const int32_t* request_query_lengths,
+    const int32_t* request_to_kv_chunk_ids, int64_t table_stride, int32_t max_kv_chunk_count,
+    int32_t* query_seq_lengths_out, int32_t* kv_seq_lengths_out, int32_t* cu_query_seq_lengths_out,
+    int32_t* cu_kv_seq_lengths_out, int32_t* block_table_out, int64_t block_table_out_stride,
+    int64_t* token_to_chunk_idx, int64_t* token_to_local_position_within_kv_chunk,
+    int64_t* token_to_position_in_request, int32_t* max_lengths_out, int32_t paused_request_count,
+    int32_t active_request_count, int32_t padded_request_count, int32_t active_token_count,
+    int32_t padded_active_token_count, int32_t dummy_chunk_idx, void* stream) {
+  if (!request_kv_length_offsets || !request_query_lengths || !request_to_kv_chunk_ids || !query_seq_lengths_out ||
+      !kv_seq_lengths_out || !cu_query_seq_lengths_out || !cu_kv_seq_lengths_out || !block_table_out ||
+      !token_to_chunk_idx || !token_to_local_position_within_kv_chunk || !token_to_position_in_request ||
+      !max_lengths_out)
+    return mi_fail(MI_ERR_NULL, "mi_step_attention_state: null pointer argument");
+  if (paused_request_count < 0 || active_request_count < 0 || padded_request_count < active_request_count ||
+      active_token_count < 0 || padded_active_token_count < active_token_count || max_kv_chunk_count <= 0)
+    return mi_fail(MI_ERR_SHAPE, "mi_step_attention_state: inconsistent counts");
+  StepStateParams p;
+  p.kv_off = request_kv_length_offsets; p.q_len = request_query_lengths; p.table = request_to_kv_chunk_ids;
+  p.table_stride = table_stride; p.M = max_kv_chunk_count;
+  p.q_lens_out = query_seq_lengths_out; p.kv_lens_out = kv_seq_lengths_out;
+  p.cu_q_out = cu_query_seq_lengths_out; p.cu_kv_out = cu_kv_seq_lengths_out;
+  p.table_out = block_table_out; p.table_out_stride = block_table_out_stride;
+  p.tok_chunk = token_to_chunk_idx; p.tok_local = token_to_local_position_within_kv_chunk;
+  p.tok_in_req = token_to_position_in_request; p.maxes = max_lengths_out;
+  p.paused = paused_request_count; p.n_active = active_request_count; p.R = padded_request_count;
+  p.padded = padded_active_token_count; p.active_tokens = active_token_count; p.dummy_chunk = dummy_chunk_idx;
+  int copy_blocks = active_request_count < 255 ? active_request_count : 255;
+  hipLaunchKernelGGL(step_attention_state_kernel, dim3(1 + copy_blocks), dim3(1024), 0, (hipStream_t)stream, p);
+  return mi_check_launch("mi_step_attention_state");
 }

@@ -17,6 +17,29 @@ from torch import Tensor
 from . import ops
 
 
+# Per-request kv lengths that belong to a cu_seqlens_k tensor, published by the context that built both
+# (DynamicInferenceContext.initialize_attention_state).  The reference's call site hands flash_attn_varlen_func only
+# the running sums (attention.py:546-557); with this note the lengths need not be recomputed by a
+# subtraction + copy in every layer.  One entry: (data_ptr, numel, version) of the sums -> lengths.
+_kv_lengths_note = None
+
+
+def note_kv_lengths(cu_seqlens_k: Optional[Tensor], kv_lens: Optional[Tensor]) -> None:
+    """Remember that ``kv_lens`` are the differences of ``cu_seqlens_k`` (``None`` forgets)."""
+    global _kv_lengths_note
+    if cu_seqlens_k is None or kv_lens is None:
+        _kv_lengths_note = None
+    else:
+        _kv_lengths_note = ((cu_seqlens_k.data_ptr(), cu_seqlens_k.numel(), cu_seqlens_k._version), kv_lens)
+
+
+def _lengths_of(cu_seqlens_k: Tensor) -> Tensor:
+    note = _kv_lengths_note
+    if note is not None and note[0] == (cu_seqlens_k.data_ptr(), cu_seqlens_k.numel(), cu_seqlens_k._version):
+        return note[1]
+    return (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).contiguous()
+
+
 def _reject(**unsupported) -> None:
     bad = [k for k, v in unsupported.items() if v not in (None, False, 0, 0.0, (-1, -1))]
     if bad:
@@ -71,7 +94,7 @@ def flash_attn_varlen_func(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor
     if seqused_k is not None:
         kv_lens = seqused_k
     elif cu_seqlens_k is not None:
-        kv_lens = (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).contiguous()
+        kv_lens = _lengths_of(cu_seqlens_k)
     else:
         raise ValueError("need cu_seqlens_k or seqused_k")
     if k.size(-1) != v.size(-1):

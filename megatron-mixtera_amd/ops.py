@@ -588,7 +588,7 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
 # ---------------------------------------------------------------------------------------------
 def update_requests(ctx, mask_i32: Tensor, new_tokens_i64: Tensor) -> None:
     """Enqueue the single-kernel ``update_requests`` on the state tensors of ``ctx`` (results land in
-    ``ctx._counters`` / ``ctx._newly_paused_buf`` / ``ctx._paused_tokens_buf``)."""
+    ``ctx._counters`` / ``ctx._newly_paused_buf`` / ``ctx._finished_ids_buf`` / ``ctx._paused_tokens_buf``)."""
     lib = _lib.load()
     table = ctx.request_to_kv_chunk_ids
     _require(table.stride(1) == 1, "request_to_kv_chunk_ids rows must be contiguous")
@@ -602,7 +602,7 @@ def update_requests(ctx, mask_i32: Tensor, new_tokens_i64: Tensor) -> None:
         ctx.token_to_local_position_within_kv_chunk.data_ptr(), ctx.chunk_allocator.chunk_bag.data_ptr(),
         mask_i32.data_ptr(), new_tokens_i64.data_ptr(), ctx._paused_tokens_buf.data_ptr(),
         ctx._next_tokens_buf.data_ptr(), ctx._update_scratch.data_ptr(), ctx._newly_paused_buf.data_ptr(),
-        ctx._counters.data_ptr(), ctx.total_request_count, ctx.paused_request_count,
+        ctx._finished_ids_buf.data_ptr(), ctx._counters.data_ptr(), ctx.total_request_count, ctx.paused_request_count,
         ctx.chunk_allocator.chunk_count_avail, ctx.gtd_chunk_count, ctx.gtd_request_count,
         ctx.chunk_size_tokens, ctx.max_requests, _stream(table)), "mi_update_requests")
 
@@ -619,6 +619,23 @@ def decode_attention_state(ctx, n_active_requests: int, padded_tokens: int) -> N
         ctx.token_to_chunk_idx.data_ptr(), ctx.token_to_local_position_within_kv_chunk.data_ptr(),
         ctx.token_to_position_in_request.data_ptr(), ctx.paused_request_count, n_active_requests,
         ctx.active_token_count, padded_tokens, ctx.dummy_chunk_idx, _stream(table)), "mi_decode_attention_state")
+
+
+def step_attention_state(ctx, n_active_requests: int, padded_requests: int, padded_tokens: int) -> None:
+    """Prefill / mixed steps: the fixed-address mirrors of lengths, their running sums and the block table, the
+    padded token rows and the two maxima (into ``ctx._max_lengths``) in one launch."""
+    lib = _lib.load()
+    table = ctx.request_to_kv_chunk_ids
+    mirror = ctx.request_to_kv_chunk_ids_cudagraph_only
+    _lib.check(lib.mi_step_attention_state(
+        ctx.request_kv_length_offsets.data_ptr(), ctx.request_query_lengths.data_ptr(), table.data_ptr(),
+        table.stride(0), table.size(1), ctx.query_seq_lengths_cudagraph_only.data_ptr(),
+        ctx.kv_seq_lengths_cudagraph_only.data_ptr(), ctx.cu_query_seq_lengths_cudagraph_only.data_ptr(),
+        ctx.cu_kv_seq_lengths_cudagraph_only.data_ptr(), mirror.data_ptr(), mirror.stride(0),
+        ctx.token_to_chunk_idx.data_ptr(), ctx.token_to_local_position_within_kv_chunk.data_ptr(),
+        ctx.token_to_position_in_request.data_ptr(), ctx._max_lengths.data_ptr(), ctx.paused_request_count,
+        n_active_requests, padded_requests, ctx.active_token_count, padded_tokens, ctx.dummy_chunk_idx,
+        _stream(table)), "mi_step_attention_state")
 
 
 # ---------------------------------------------------------------------------------------------

@@ -25,6 +25,7 @@ int main(void) {
       (const void*)(size_t)mi_paged_prefill_attention_fp8, (const void*)(size_t)mi_paged_prefill_attention_mla,
       (const void*)(size_t)mi_norm_rope_append, (const void*)(size_t)mi_qkv_norm_rope_append,
       (const void*)(size_t)mi_update_requests, (const void*)(size_t)mi_decode_attention_state,
+      (const void*)(size_t)mi_step_attention_state,
       (const void*)(size_t)mi_last_token_gather, (const void*)(size_t)mi_selected_log_probs,
       (const void*)(size_t)mi_sample_from_logits};
   size_t i;

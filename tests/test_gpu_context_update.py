@@ -185,7 +185,7 @@ def test_kernel_and_torch_op_sequence_agree_on_a_wide_batch(mi, Ctx, dev):
     b = Ctx(fused_bookkeeping=False, **kw)
     rng = random.Random(11)
     next_id = 0
-    saw_pause = False
+    saw_pause = saw_mixed = saw_finished = False
     widest = 0
     for step in range(40):
         for _ in range(rng.randint(0, 100)):
@@ -206,13 +206,34 @@ def test_kernel_and_torch_op_sequence_agree_on_a_wide_batch(mi, Ctx, dev):
             c.initialize_attention_state()
         if a.is_decode_only():
             assert torch.equal(a.kv_seq_lengths, b.kv_seq_lengths) and torch.equal(a.block_table, b.block_table)
+        else:
+            # prefill / mixed step: one launch and no wait on the kernel side, the torch ops and two .item()
+            # calls on the other; every published value must be the same
+            saw_mixed = True
+            assert a._max_lengths_pending, "the kernel path must not have waited for the maxima yet"
+            q_bound, k_bound = a.attention_length_bounds()
+            for name in ("cu_query_seq_lengths", "cu_kv_seq_lengths", "kv_seq_lengths", "block_table"):
+                assert torch.equal(getattr(a, name), getattr(b, name)), name
+            pad = slice(a.active_token_count, a.padded_active_token_count)
+            for name in ("token_to_chunk_idx", "token_to_local_position_within_kv_chunk", "token_to_position_in_request"):
+                assert torch.equal(getattr(a, name)[pad], getattr(b, name)[pad]), name
+            assert a.cu_query_lengths()[1] == b.max_seqlen_q and a.cu_kv_lengths()[2] == b.max_seqlen_k
+            assert not a._max_lengths_pending
+            assert q_bound == b.max_seqlen_q, "the host knows the longest query exactly"
+            assert b.max_seqlen_k <= k_bound <= a.max_sequence_length
         seq = (a.request_kv_length_offsets + a.request_query_lengths)[a.paused_request_count:a.total_request_count]
         budget = a.request_output_lengths[a.paused_request_count:a.total_request_count]
         mask = torch.tensor([(0 if (x + 1 >= y or rng.random() < 0.05) else 1)
                              for x, y in zip(seq.tolist(), budget.tolist())], dtype=torch.int32, device=dev)
         new = torch.randint(0, 100, (n_act,), device=dev)
+        ids_before = a.request_ids[a.paused_request_count:a.total_request_count].clone()
         ga = a.update_requests(mask, new)
         gb = b.update_requests(mask, new)
+        # ids of the finished requests, listed by the kernel in row order; the torch path lists nothing
+        assert b.last_finished_request_ids is None
+        assert a.last_finished_request_ids.dtype == torch.int32
+        assert a.last_finished_request_ids.tolist() == ids_before[mask == 0].tolist()
+        saw_finished |= bool((mask == 0).any())
         assert (ga is None) == (gb is None)
         if ga is not None:
             assert ga.tolist() == gb.tolist()
@@ -221,4 +242,4 @@ def test_kernel_and_torch_op_sequence_agree_on_a_wide_batch(mi, Ctx, dev):
         assert _snapshot_product(a) == _snapshot_product(b), f"step {step}"
         if a.paused_request_count:
             assert a.paused_tokens.tolist() == b.paused_tokens.tolist()
-    assert widest > 256 and saw_pause
+    assert widest > 256 and saw_pause and saw_mixed and saw_finished

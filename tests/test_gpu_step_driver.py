@@ -116,7 +116,8 @@ def test_steps_follow_the_dense_model_and_the_bookkeeping_rules(mi, dev):
                 history[rid].append(tok)
                 if tok == TERM or len(history[rid]) >= len(prompts[rid]) + budget[rid]:
                     finished.append(rid)
-            assert sorted(result["finished_request_ids"].tolist()) == sorted(finished)
+            # (listed by the bookkeeping kernel, in the row order the reference's nonzero + index gives)
+            assert result["finished_request_ids"].tolist() == finished
             live -= set(finished)
             finished_all += finished
             assert ctx.total_request_count == len(live)
