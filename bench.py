@@ -226,13 +226,70 @@ def run_stream_read(args, mi, torch, dev):
                      "kernel_ms": round(best["kernel_ms_mean"], 5), "traffic": None}}), flush=True)
 
 
+def run_cu_probes(args, mi, torch, dev):
+    """Calibration leg: what one compute unit delivers to the prefill tile kernel (csrc/bench/cu_probes.hip) --
+    LDS fragment reads per wavefront and per CU, the same fragments through the vector L1, how matrix and vector
+    instructions of two wavefronts of a SIMD overlap, and the core clock a matrix-bound kernel really runs at."""
+    path = mi._lib.PKG_DIR / "libmi355_bench.so"
+    if not path.exists():
+        print(f"{path} not found: build first (python megatron-mixtera_amd/build.py)", file=sys.stderr)
+        sys.exit(2)
+    blib = ctypes.CDLL(str(path))
+    P, I = ctypes.c_void_p, ctypes.c_int32
+    blib.mi_bench_read_probe.restype = ctypes.c_int
+    blib.mi_bench_read_probe.argtypes = [I, I, I, I, P, P, P, P]
+    blib.mi_bench_coexec_probe.restype = ctypes.c_int
+    blib.mi_bench_coexec_probe.argtypes = [I, I, I, I, P, P, P]
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    cyc = torch.zeros(16, dtype=torch.int64, device=dev)
+    sink = torch.zeros(cus * 1024, dtype=torch.int32, device=dev)
+    gsrc = torch.ones(cus * 64 * 2048, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    t0 = time.perf_counter()
+    reads = {}
+    iters = 2000
+    for mode, name in ((0, "lds_b128"), (1, "lds_tr_b64"), (2, "global_b128_l1_resident")):
+        for waves in (1, 4, 8, 16):
+            for _ in range(2):
+                assert blib.mi_bench_read_probe(mode, waves, cus, iters, cyc.data_ptr(), sink.data_ptr(), gsrc.data_ptr(), stream) == 0
+            torch.cuda.synchronize()
+            worst = int(cyc[:waves].max())
+            nbytes = iters * 16 * 1024 * waves
+            reads[f"{name}_{waves}_waves"] = {"bytes_per_clk_per_cu": round(nbytes / worst, 1),
+                                              "bytes_per_clk_per_wave": round(nbytes / worst / waves, 2)}
+    names = {0: "idle", 1: "mfma_16x16x32", 2: "mfma_32x32x16", 3: "fma", 4: "exp2"}
+    per_iter = {1: 32, 2: 16, 3: 32, 4: 32}
+    coexec = {}
+    iters = 20000
+    for a, b in ((1, 0), (2, 0), (3, 0), (4, 0), (3, 3), (1, 3), (1, 4), (2, 3), (2, 4), (1, 1)):
+        for wgs in (1, cus):   # one workgroup alone; every CU busy (the clock a loaded chip runs at)
+            for _ in range(2):
+                assert blib.mi_bench_coexec_probe(a, b, wgs, iters, cyc.data_ptr(), sink.data_ptr(), stream) == 0
+            torch.cuda.synchronize()
+            c = cyc.tolist()
+            entry = {"a_clk_per_instr": round(c[0] / (iters * per_iter[a]), 2)}
+            if b:
+                entry["b_clk_per_instr"] = round(c[4] / (iters * per_iter[b]), 2)
+            entry["core_clock_mhz"] = round(c[0] / max(c[8], 1) * 100)
+            coexec[f"{names[a]}+{names[b]}" + ("_all_cus" if wgs > 1 else "_one_cu")] = entry
+    elapsed = time.perf_counter() - t0
+    print(json.dumps({
+        "metric": "cu_probes", "value": reads["lds_b128_16_waves"]["bytes_per_clk_per_cu"], "unit": "LDS B/clk/CU",
+        "n_gpus": 1, "steps": 1, "warmup": 0, "ms_per_step": round(elapsed * 1e3, 1), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u8 / bf16 / f32", "data": "synthetic",
+        "config": {"workload": "probes of one compute unit: fragment reads from LDS and through the vector L1 "
+                               "(bytes per core clock), matrix / vector co-execution of two wavefronts of a SIMD "
+                               "(core clocks per instruction; a = wavefronts 0-3, b = wavefronts 4-7), core clock"},
+        "reads": reads, "coexec": coexec}), flush=True)
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", *SECONDARY_WORKLOADS],
+                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", "cu_probes", *SECONDARY_WORKLOADS],
                     help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch; the "
                          "mla_* / prefill_d64 / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
     ap.add_argument("--split-tokens", type=int, default=0)
@@ -490,6 +547,9 @@ def main():
         return
     if args.workload == "stream_read":
         run_stream_read(args, mi, torch, dev)
+        return
+    if args.workload == "cu_probes":
+        run_cu_probes(args, mi, torch, dev)
         return
     if args.workload in SECONDARY_WORKLOADS:
         run_secondary(args, mi, lib, torch, dev)
