@@ -540,7 +540,7 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     if args.subtiles:
-        mi.ops.set_tuning("decode_tile_subtiles", args.subtiles)
+        mi.ops.set_tuning("decode_tile_subtiles", args.subtiles)  # (passed with every call of the ops module)
 
     if args.workload == "cfg3":
         run_mixed_batch(args, mi, lib, torch, dev)

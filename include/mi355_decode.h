@@ -15,6 +15,12 @@
  *  - Return value: 0 = enqueued; negative = rejected, nothing was launched
  *    (MI_ERR_*); mi_last_error() gives the message of the calling thread's last
  *    rejection.
+ *  - The library keeps no state between calls: what a call does depends on its
+ *    arguments only (kernel timing, mi_profile_enable, is the one exception and is a
+ *    measurement aid).  Experiment knobs travel with the call (MiTuning).
+ *  - `dtype` is the 16-bit element type of q / k / v / out, of a cache that is not
+ *    fp8 and of norm weights: MI_DTYPE_BF16 or MI_DTYPE_FP16 (the reference's
+ *    params_dtype, dynamic_context.py:195,287-308).
  *  - KV cache layout is the reference's: key cache = memory_buffer[0, layer],
  *    value cache = memory_buffer[1, layer], each `[n_chunks, chunk_tokens, Hkv, d]`
  *    (megatron/core/inference/contexts/dynamic_context.py:296-308,547-564).
@@ -38,7 +44,9 @@ enum {
   MI_ERR_LAUNCH = -6
 };
 
-enum { MI_KV_BF16 = 0, MI_KV_FP8_E4M3 = 1 };
+enum { MI_DTYPE_BF16 = 0, MI_DTYPE_FP16 = 1 };
+/* KV storage: the 16-bit type given by `dtype`, or fp8-e4m3 bytes with scales (needs MI_DTYPE_BF16). */
+enum { MI_KV_16BIT = 0, MI_KV_BF16 = 0, MI_KV_FP8_E4M3 = 1 };
 enum { MI_NORM_NONE = 0, MI_NORM_RMS = 1, MI_NORM_L2 = 2 };
 
 /* ABI revision of the loaded library. */
@@ -47,19 +55,30 @@ int mi_version(void);
 /* Message of the calling thread's most recent rejected call ("" if none). */
 const char* mi_last_error(void);
 
-/* Experiment knobs (defaults are the measured best; out-of-range values are rejected):
- * "decode_tile_subtiles" (0 = automatic, 1, 2, 4), "decode_min_waves" (2..4), "decode_wgs_per_cu",
- * "decode_grid" (0 = automatic), "decode_waves_per_block" (1..8), "prefill_pingpong" (1 = two-phase
- * tile kernel, 2 = the same kernel with its wave groups in lock-step, 0 = older LDS kernel),
- * "prefill_tile_subtiles", "prefill_lds_row_tiles", "prefill_row_tiles" (the older kernels),
- * "norm_rope_vectorised" (16-byte-per-lane norm / rotary kernel: 1 = wherever alignment and the rotary
- * width allow it, 2 = the same but only from 256 tokens up (default), 0 = element-wise kernel always),
- * "prefill_kv_split" (key ranges per request in the two-phase tile kernel: 1 = chosen from T and
- * max_kv_len (default), 0 = never, 2..64 = forced where the workspace allows it),
- * "mla_decode_lds" (multi-latent decode: 1 = latent tiles shared through LDS by the wavefronts of a
- * workgroup when the chunk size is a multiple of 64 and at most 768 requests are in the call (default),
- * 0 = one streaming wavefront per 16-head group always). */
-int mi_set_tuning(const char* name, int32_t value);
+/*
+ * Experiment knobs, passed per call.  NULL, or a field left 0, selects the default (the measured best
+ * on MI355X); they exist for sweeps and tests.  Out-of-range values are rejected (MI_ERR_UNSUPPORTED).
+ * Pass the same knobs to a *_workspace_bytes function and to the attention call it sizes.
+ */
+typedef struct MiTuning {
+  int32_t decode_tile_subtiles;   /* decode kernel, 16-token sub-tiles per loop iteration: 0 = automatic, 1, 2, 4 */
+  int32_t decode_min_waves;       /* decode kernel, wavefronts per SIMD to compile for: 0 = default (3), 2..4 */
+  int32_t decode_wgs_per_cu;      /* decode kernel, workgroups of 8 wavefronts per CU: 0 = default (1), 1..8 */
+  int32_t decode_grid;            /* decode kernels, spans the tile sequence is cut into: 0 = automatic, 1..65535 */
+  int32_t decode_waves_per_block; /* decode kernel, KV heads per workgroup: 0 = default (8), 1..8 */
+  int32_t prefill_two_phase;      /* prefill: 0 = default (1), 1 = two-phase tile kernel, 2 = the same with its
+                                     wave groups in lock-step, -1 = register-only kernel */
+  int32_t prefill_tile_subtiles;  /* register-only prefill kernel, 16-key sub-tiles per iteration: 0 = default (2), 1, 2 */
+  int32_t prefill_row_tiles;      /* register-only prefill kernel, 16-row tiles per wavefront: 0 = default (2), 2, 4 */
+  int32_t prefill_kv_split;       /* two-phase kernel, key ranges per request: 0 = from T and max_kv_len, -1 = never,
+                                     2..64 = forced where the workspace allows it */
+  int32_t norm_rope_vectorised;   /* 16-byte-per-lane norm / rotary kernel: 0 = default (from 256 tokens up, where
+                                     alignment and rotary width allow), 1 = wherever they allow, -1 = never */
+  int32_t mla_decode_lds;         /* multi-latent decode: 0 = default (latent tiles shared through LDS when the chunk
+                                     size is a multiple of 64 and the call has at most 768 requests), -1 = one
+                                     streaming wavefront per 16-head group always */
+  int32_t reserved[5];            /* must be 0 */
+} MiTuning;
 
 /*
  * Kernel timing.  mi_profile_enable(1) makes the attention entry points bracket their main
@@ -141,7 +160,8 @@ int mi_kv_append_fp8(const void* key_bf16, const void* value_bf16, int64_t src_s
  * device (partials of the workgroups that share a request + per-request bookkeeping).
  */
 int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
-                                  int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens);
+                                  int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
+                                  const MiTuning* tuning);
 
 /*
  * Paged GQA decode attention (one query token per request).
@@ -165,7 +185,7 @@ int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_str
                               int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
                               int32_t max_kv_len, int32_t split_tokens, float softmax_scale,
                               int32_t kv_dtype, const float* k_scales, const float* v_scales,
-                              void* stream);
+                              int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * mi_paged_decode_attention for callers that cannot allocate device memory: code under HIP graph
@@ -188,7 +208,7 @@ int mi_paged_decode_attention_noalloc(const void* q, int64_t q_stride_tok, int64
                                       int64_t o_stride_head, int32_t R, int32_t Hq, int32_t Hkv,
                                       int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len,
                                       int32_t split_tokens, float softmax_scale, int32_t kv_dtype,
-                                      const float* k_scales, const float* v_scales, void* stream);
+                                      const float* k_scales, const float* v_scales, int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * Decode attention over the latent cache of multi-latent attention (absorbed form).
@@ -202,7 +222,7 @@ int mi_paged_decode_attention_noalloc(const void* q, int64_t q_stride_tok, int64
  * q bf16 `[R, Hq, 576]`, out bf16 `[R, Hq, 512]`, kv_cache bf16 `[n_chunks, chunk_tokens, 576]` with
  * the given chunk / token strides (elements).  Hq: 1, 2, 4, 8 or a multiple of 16.
  */
-int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v);
+int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v, const MiTuning* tuning);
 
 int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
                                   const void* kv_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok,
@@ -210,7 +230,7 @@ int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q
                                   void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
                                   int64_t workspace_bytes, int32_t R, int32_t Hq, int32_t head_dim_k,
                                   int32_t head_dim_v, int32_t chunk_tokens, int32_t max_kv_len,
-                                  float softmax_scale, void* stream);
+                                  float softmax_scale, int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * Paged varlen causal attention for prefill / mixed prefill+decode batches.
@@ -231,7 +251,7 @@ int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q
  * values to mi_prefill_workspace_bytes and to the attention call.
  */
 int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
-                                   int32_t max_kv_len, int32_t split_tokens);
+                                   int32_t max_kv_len, int32_t split_tokens, const MiTuning* tuning);
 
 int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
                                const void* k_cache, const void* v_cache, int64_t kv_stride_chunk,
@@ -242,7 +262,7 @@ int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_st
                                int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq,
                                int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
                                int32_t max_kv_len, int32_t split_tokens, float softmax_scale,
-                               void* stream);
+                               int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * The same call over an fp8-e4m3 cache (byte caches `[n_chunks, chunk_tokens, Hkv, d]`, strides in
@@ -260,7 +280,7 @@ int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t 
                                    int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
                                    int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                    int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
-                                   float softmax_scale, void* stream);
+                                   float softmax_scale, const MiTuning* tuning, void* stream);
 
 /*
  * Paged varlen causal attention with keys wider than values: the prefill / mixed step of
@@ -287,7 +307,7 @@ int mi_paged_prefill_attention_mla(const void* q, int64_t q_stride_tok, int64_t 
                                    int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
                                    int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
                                    int32_t head_dim_k, int32_t head_dim_v, int32_t chunk_tokens,
-                                   int32_t max_kv_len, float softmax_scale, void* stream);
+                                   int32_t max_kv_len, float softmax_scale, int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * Fused q/k head norm + rotary embedding (+ KV-append when k_cache is given).
@@ -317,7 +337,7 @@ int mi_norm_rope_append(const void* q, int64_t q_stride_tok, void* q_out, int64_
                         const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos,
                         const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
                         int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv, int32_t head_dim,
-                        int32_t faithful_rounding, void* stream);
+                        int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * The same launch reading the QKV projection's output directly: replaces the split of
@@ -339,7 +359,7 @@ int mi_qkv_norm_rope_append(const void* mixed_qkv, int64_t qkv_stride_tok, void*
                             const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos,
                             const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
                             int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv, int32_t head_dim,
-                            int32_t faithful_rounding, void* stream);
+                            int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * DynamicInferenceContext.update_requests as one kernel
@@ -430,7 +450,7 @@ int mi_last_token_gather(const void* src, int64_t src_stride_row, void* dst, int
  * The arithmetic of DynamicInferenceContext.calculate_log_probs (dynamic_context.py:1300-1365):
  *   log_probs[t] = log_softmax(float(logits[t, :]))[token_ids[t]],  t < T
  * without materialising the `[T, vocab]` fp32 log-softmax matrix: one read of each row.  logits
- * `[T, vocab]` fp32 (0) or bf16 (1), row stride in elements; token_ids int64 `[T]` (the caller builds
+ * `[T, vocab]` fp32 (0), bf16 (1) or fp16 (2), row stride in elements; token_ids int64 `[T]` (the caller builds
  * them as the reference does: the prompt token that follows each position, the newly sampled token at
  * the last position of each request); an id outside [0, vocab) yields NaN.  fp32 results.
  */
@@ -441,9 +461,9 @@ int mi_selected_log_probs(const void* logits, int64_t stride_row, int32_t logits
  * TextGenerationController.sample_from_logits and the finished-request test that follows it
  * (megatron/core/inference/text_generation_controllers/text_generation_controller.py:172-315,
  * 519-530) as one launch, one workgroup per row of `logits` `[R, vocab]` (logits_dtype 0 = fp32,
- * 1 = bf16; row stride in elements):
+ * 1 = bf16, 2 = fp16; row stride in elements):
  *   top_k == 1             : samples[r] = argmax (lowest index among equal maxima);
- *   otherwise              : x = logits * (1 / temperature) (rounded to bf16 for bf16 logits, as the
+ *   otherwise              : x = logits * (1 / temperature) (rounded to the logits' type for 16-bit logits, as the
  *                            reference's in-place division rounds), then
  *     top_k > 1            : keep x >= the top_k-th largest value (ties kept, as `logits < kth`),
  *     top_p > 0 (top_k 0)  : order by value, keep the shortest prefix whose softmax mass exceeds

@@ -12,8 +12,18 @@ from pathlib import Path
 PKG_DIR = Path(__file__).resolve().parent
 LIB_PATH = PKG_DIR / "libmi355_decode.so"
 
-MI_KV_BF16, MI_KV_FP8_E4M3 = 0, 1
+MI_DTYPE_BF16, MI_DTYPE_FP16 = 0, 1
+MI_KV_16BIT, MI_KV_BF16, MI_KV_FP8_E4M3 = 0, 0, 1
 MI_NORM_NONE, MI_NORM_RMS, MI_NORM_L2 = 0, 1, 2
+
+
+class MiTuning(ctypes.Structure):
+    """Per-call experiment knobs (``MiTuning`` of the header); all zero = the defaults."""
+    _fields_ = [(name, c_int32) for name in (
+        "decode_tile_subtiles", "decode_min_waves", "decode_wgs_per_cu", "decode_grid", "decode_waves_per_block",
+        "prefill_two_phase", "prefill_tile_subtiles", "prefill_row_tiles", "prefill_kv_split",
+        "norm_rope_vectorised", "mla_decode_lds")] + [("reserved", c_int32 * 5)]
+
 
 _P, _I32, _I64, _F = c_void_p, c_int32, c_int64, c_float
 
@@ -21,7 +31,6 @@ _P, _I32, _I64, _F = c_void_p, c_int32, c_int64, c_float
 SIGNATURES = {
     "mi_version": (c_int, []),
     "mi_last_error": (c_char_p, []),
-    "mi_set_tuning": (c_int, [c_char_p, _I32]),
     "mi_profile_enable": (c_int, [_I32]),
     "mi_profile_collect": (_I32, [_P, _I32]),
     "mi_kv_append": (c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _I32, _I32, _I32, _P]),
@@ -33,32 +42,32 @@ SIGNATURES = {
         c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _F, _P]),
     "mi_kv_append_fp8": (
         c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _F, _P]),
-    "mi_decode_workspace_bytes": (_I64, [_I32, _I32, _I32, _I32, _I32, _I32, _I32]),
+    "mi_decode_workspace_bytes": (_I64, [_I32, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
     "mi_paged_decode_attention": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _I64, _I64, _P, _I64,
-         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P, _P]),
+         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P, _I32, _P, _P]),
     "mi_paged_decode_attention_noalloc": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _I64, _I64,
-         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P, _P]),
-    "mi_mla_decode_workspace_bytes": (_I64, [_I32, _I32, _I32]),
+         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P, _I32, _P, _P]),
+    "mi_mla_decode_workspace_bytes": (_I64, [_I32, _I32, _I32, _P]),
     "mi_paged_mla_decode_attention": (
         c_int, [_P, _I64, _I64, _P, _I64, _I64, _P, _I64, _P, _P, _I64, _I64, _P, _I64,
-                _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
-    "mi_prefill_workspace_bytes": (_I64, [_I32, _I32, _I32, _I32, _I32, _I32, _I32]),
+                _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P]),
+    "mi_prefill_workspace_bytes": (_I64, [_I32, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
     "mi_paged_prefill_attention": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _I64, _I64, _P, _I64,
-         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
+         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P]),
     "mi_paged_prefill_attention_fp8": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _P, _P, _I64, _P, _P, _P, _I64, _I64, _P, _I64,
-         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
+         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P, _P]),
     "mi_paged_prefill_attention_mla": (
         c_int,
         [_P, _I64, _I64, _P, _I64, _I64, _I64, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _I64, _I64,
-         _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P]),
+         _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P]),
     "mi_update_requests": (
         c_int, [_P] * 8 + [_I64, _I32] + [_P] * 15 + [_I32] * 7 + [_P]),
     "mi_step_attention_state": (
@@ -72,11 +81,11 @@ SIGNATURES = {
     "mi_norm_rope_append": (
         c_int,
         [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F,
-         _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
+         _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _P, _P]),
     "mi_qkv_norm_rope_append": (
         c_int,
         [_P, _I64, _P, _I64, _P, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F,
-         _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
+         _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _P, _P]),
 }
 
 

@@ -10,6 +10,8 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 PKG_DIR = Path(__file__).resolve().parent
@@ -29,7 +31,6 @@ HIPCC_FLAGS = [
     # packed fp32 VALU forms are kept out of the generated code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-    "-DMI_NT_LOADS",
 ]
 
 
@@ -44,8 +45,7 @@ def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
 
-def _hipcc(inputs: list[Path], output: Path, verbose: bool) -> None:
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-I", str(CSRC), "-I", str(INCLUDE), *map(str, inputs), "-o", str(output)]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -55,6 +55,18 @@ def _hipcc(inputs: list[Path], output: Path, verbose: bool) -> None:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
     if verbose and out.strip():
         print(out)
+
+
+def _hipcc(inputs: list[Path], output: Path, verbose: bool) -> None:
+    """Compile every source to an object (in parallel: one hipcc per file), then link the shared object."""
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    with tempfile.TemporaryDirectory(prefix="mi355_build_") as tmp:
+        objects = [Path(tmp) / (src.stem + ".o") for src in inputs]
+        jobs = [[hipcc_path(), *flags, "-I", str(CSRC), "-I", str(INCLUDE), "-c", str(src), "-o", str(obj)]
+                for src, obj in zip(inputs, objects)]
+        with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1, 16)) as pool:
+            list(pool.map(lambda cmd: _run(cmd, verbose), jobs))
+        _run([hipcc_path(), "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objects), "-o", str(output)], verbose)
 
 
 def build_library(verbose: bool = False) -> Path:

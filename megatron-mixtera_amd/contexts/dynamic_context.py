@@ -955,8 +955,8 @@ class DynamicInferenceContext:
         p is the prompt token at p+1; the last position of each request takes ``new_tokens``.
         """
         rows = logits.squeeze(0)
-        if rows.is_cuda:
-            # one read of every row, no [T, V] fp32 intermediate
+        if rows.is_cuda and rows.dtype in (torch.float32, torch.bfloat16, torch.float16) and rows.stride(-1) == 1:
+            # one read of every row, no [T, V] fp32 intermediate (other dtypes / layouts: the torch ops below)
             def pick(ids):
                 return ops.selected_log_probs(rows[: ids.numel()], ids.to(torch.int64).contiguous())
         else:

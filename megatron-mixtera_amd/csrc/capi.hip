@@ -19,90 +19,46 @@ int mi_check_launch(const char* where) {
   return MI_ERR_LAUNCH;
 }
 
-static int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return (v && *v) ? atoi(v) : dflt;
-}
-
-MiTuning& mi_tuning() {
-  static MiTuning t = {env_int("MI355_DECODE_SUBTILES", 0), env_int("MI355_PREFILL_SUBTILES", 4),
-                      env_int("MI355_PREFILL_LDS_ROW_TILES", 2), env_int("MI355_PREFILL_ROW_TILES", 2),
-                      env_int("MI355_DECODE_MIN_WAVES", 3),
-                      env_int("MI355_DECODE_WGS_PER_CU", 1), env_int("MI355_DECODE_GRID", 0),
-                      env_int("MI355_DECODE_WAVES_PER_BLOCK", 8), env_int("MI355_NORM_ROPE_VECTORISED", 2),
-                      env_int("MI355_MLA_DECODE_LDS", 1), env_int("MI355_PREFILL_KV_SPLIT", 1),
-                      env_int("MI355_PREFILL_PINGPONG", 1)};
-  return t;
-}
-
-extern "C" int mi_version(void) { return 1; }
+extern "C" int mi_version(void) { return 2; }
 
 extern "C" const char* mi_last_error(void) { return g_err; }
 
-extern "C" int mi_set_tuning(const char* name, int32_t value) {
-  if (!name) return mi_fail(MI_ERR_NULL, "mi_set_tuning: null name");
-  if (!strcmp(name, "decode_tile_subtiles")) {
-    if (value != 0 && value != 1 && value != 2 && value != 4)
-      return mi_fail(MI_ERR_UNSUPPORTED, "decode_tile_subtiles must be 0 (automatic), 1, 2 or 4");
-    mi_tuning().decode_tile_subtiles = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "prefill_lds_row_tiles")) {
-    if (value != 0 && value != 2 && value != 3) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_lds_row_tiles must be 0, 2 or 3");
-    mi_tuning().prefill_lds_row_tiles = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "prefill_row_tiles")) {
-    if (value != 2 && value != 4) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_row_tiles must be 2 or 4");
-    mi_tuning().prefill_row_tiles = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "prefill_tile_subtiles")) {
-    if (value != 1 && value != 2 && value != 4) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_tile_subtiles must be 1, 2 or 4");
-    mi_tuning().prefill_tile_subtiles = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "decode_min_waves")) {
-    if (value < 2 || value > 4) return mi_fail(MI_ERR_UNSUPPORTED, "decode_min_waves must be 2, 3 or 4");
-    mi_tuning().decode_min_waves = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "decode_wgs_per_cu")) {
-    if (value < 1 || value > 8) return mi_fail(MI_ERR_UNSUPPORTED, "decode_wgs_per_cu must be 1..8");
-    mi_tuning().decode_wgs_per_cu = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "decode_grid")) {
-    if (value < 0 || value > 65535) return mi_fail(MI_ERR_UNSUPPORTED, "decode_grid must be 0..65535");
-    mi_tuning().decode_grid = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "norm_rope_vectorised")) {
-    if (value < 0 || value > 2) return mi_fail(MI_ERR_UNSUPPORTED, "norm_rope_vectorised must be 0, 1 or 2");
-    mi_tuning().norm_rope_vectorised = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "prefill_pingpong")) {
-    if (value < 0 || value > 2) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_pingpong must be 0, 1 or 2");
-    mi_tuning().prefill_pingpong = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "prefill_kv_split")) {
-    if (value < 0 || value > 64) return mi_fail(MI_ERR_UNSUPPORTED, "prefill_kv_split must be 0 (never), 1 (automatic) or 2..64");
-    mi_tuning().prefill_kv_split = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "mla_decode_lds")) {
-    if (value != 0 && value != 1) return mi_fail(MI_ERR_UNSUPPORTED, "mla_decode_lds must be 0 or 1");
-    mi_tuning().mla_decode_lds = value;
-    return MI_OK;
-  }
-  if (!strcmp(name, "decode_waves_per_block")) {
-    if (value < 1 || value > 8) return mi_fail(MI_ERR_UNSUPPORTED, "decode_waves_per_block must be 1..8");
-    mi_tuning().decode_waves_per_block = value;
-    return MI_OK;
-  }
-  return mi_fail(MI_ERR_UNSUPPORTED, "mi_set_tuning: unknown knob");
+int mi_resolve_tuning(const MiTuning* given, MiTuning* out, const char* who) {
+  MiTuning t = {};
+  if (given) t = *given;
+  char msg[200];
+  auto bad = [&](const char* what) {
+    snprintf(msg, sizeof msg, "%s: tuning: %s", who, what);
+    return mi_fail(MI_ERR_UNSUPPORTED, msg);
+  };
+  for (int r : t.reserved)
+    if (r != 0) return bad("reserved fields must be 0");
+  if (t.decode_tile_subtiles != 0 && t.decode_tile_subtiles != 1 && t.decode_tile_subtiles != 2 && t.decode_tile_subtiles != 4)
+    return bad("decode_tile_subtiles must be 0 (automatic), 1, 2 or 4");
+  if (t.decode_min_waves == 0) t.decode_min_waves = 3;
+  if (t.decode_min_waves < 2 || t.decode_min_waves > 4) return bad("decode_min_waves must be 0 (default), 2, 3 or 4");
+  if (t.decode_wgs_per_cu == 0) t.decode_wgs_per_cu = 1;
+  if (t.decode_wgs_per_cu < 1 || t.decode_wgs_per_cu > 8) return bad("decode_wgs_per_cu must be 0 (default) or 1..8");
+  if (t.decode_grid < 0 || t.decode_grid > 65535) return bad("decode_grid must be 0 (automatic) or 1..65535");
+  if (t.decode_waves_per_block == 0) t.decode_waves_per_block = 8;
+  if (t.decode_waves_per_block < 1 || t.decode_waves_per_block > 8) return bad("decode_waves_per_block must be 0 (default) or 1..8");
+  if (t.prefill_two_phase == 0) t.prefill_two_phase = 1;
+  if (t.prefill_two_phase != 1 && t.prefill_two_phase != 2 && t.prefill_two_phase != -1)
+    return bad("prefill_two_phase must be 0 (default), 1, 2 or -1 (register-only kernel)");
+  if (t.prefill_tile_subtiles == 0) t.prefill_tile_subtiles = 2;
+  if (t.prefill_tile_subtiles != 1 && t.prefill_tile_subtiles != 2) return bad("prefill_tile_subtiles must be 0 (default), 1 or 2");
+  if (t.prefill_row_tiles == 0) t.prefill_row_tiles = 2;
+  if (t.prefill_row_tiles != 2 && t.prefill_row_tiles != 4) return bad("prefill_row_tiles must be 0 (default), 2 or 4");
+  if (t.prefill_kv_split == 0) t.prefill_kv_split = 1;  // 1 = automatic from here on
+  if (t.prefill_kv_split != -1 && (t.prefill_kv_split < 1 || t.prefill_kv_split > 64))
+    return bad("prefill_kv_split must be 0 (automatic), -1 (never) or 2..64");
+  if (t.norm_rope_vectorised == 0) t.norm_rope_vectorised = 2;  // 2 = from 256 tokens up
+  if (t.norm_rope_vectorised != 1 && t.norm_rope_vectorised != 2 && t.norm_rope_vectorised != -1)
+    return bad("norm_rope_vectorised must be 0 (default), 1 or -1 (never)");
+  if (t.mla_decode_lds == 0) t.mla_decode_lds = 1;
+  if (t.mla_decode_lds != 1 && t.mla_decode_lds != -1) return bad("mla_decode_lds must be 0 (default) or -1 (streaming kernel)");
+  *out = t;
+  return MI_OK;
 }
 
 // ---- kernel timing with HIP events --------------------------------------------------

@@ -3,8 +3,8 @@
 // Conventions used by every kernel in this directory:
 //  * a wavefront is 64 lanes; `m16 = lane & 15` and `g = lane >> 4` are the two
 //    coordinates every MFMA operand layout is expressed in;
-//  * bf16 values travel as raw uint16_t / packed uint32_t pairs and are only
-//    reinterpreted at the MFMA call sites;
+//  * bf16 / fp16 values travel as raw uint16_t / packed uint32_t pairs and are only
+//    reinterpreted by the helpers below (template parameter F16);
 //  * all kernels are enqueue-only: no host synchronisation, no device-side
 //    allocation, every buffer is owned by the caller.
 #pragma once
@@ -22,21 +22,34 @@ typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 
 constexpr int kWave = 64;
 
-// D(16x16) += A(16x32) * B(32x16), bf16 inputs, fp32 accumulate.
+// 16-bit element types.  Every kernel that touches q / k / v / out elements is compiled twice, for bf16
+// (F16 = false) and for IEEE fp16 (F16 = true); values travel as raw uint16_t / packed uint32_t pairs and the
+// helpers below are the only places that know which of the two they are.
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+
+// D(16x16) += A(16x32) * B(32x16), 16-bit inputs, fp32 accumulate.
 // Lane (m16, g) supplies A[m16][8g..8g+7] and B[8g..8g+7][m16]; it receives
 // D[4g+i][m16] in slot i.  Only the pairing "A slot j of group g meets B slot j
 // of group g" is relied upon, so any consistent assignment of contraction
 // indices to (g, j) gives the same dot products.
+template <bool F16 = false>
 static __device__ __forceinline__ f32x4_t mfma_16x16x32(uint4 a, uint4 b, f32x4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a),
-                                                 __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
 }
 
-// D(16x16) += A(16x16) * B(16x16), bf16 inputs, fp32 accumulate.
+// D(16x16) += A(16x16) * B(16x16), 16-bit inputs, fp32 accumulate.
 // Lane (m16, g) supplies A[m16][4g..4g+3] and B[4g..4g+3][m16]; D as above.
+template <bool F16 = false>
 static __device__ __forceinline__ f32x4_t mfma_16x16x16(uint2 a, uint2 b, f32x4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a),
-                                                   __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
+  if constexpr (F16)
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, a), __builtin_bit_cast(f16x4_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, a), __builtin_bit_cast(s16x4_t, b), c, 0, 0, 0);
 }
 
 // Two fp32 -> packed bf16 pair (round to nearest even), `lo` in bits 0..15.
@@ -45,9 +58,25 @@ static __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
   return __builtin_bit_cast(uint32_t, r);
 }
+// Two fp32 -> packed pair of the kernel's 16-bit type (round to nearest even), `lo` in bits 0..15.
+template <bool F16>
+static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  if constexpr (F16) {
+    f32x2_t v = {lo, hi};
+    f16x2_t r = __builtin_convertvector(v, f16x2_t);
+    return __builtin_bit_cast(uint32_t, r);
+  } else {
+    return pack_bf16x2(lo, hi);
+  }
+}
 
 static __device__ __forceinline__ uint16_t f32_to_bf16(float x) {
   return (uint16_t)(pack_bf16x2(x, 0.f) & 0xffffu);
+}
+template <bool F16>
+static __device__ __forceinline__ uint16_t f32_to_16(float x) {
+  if constexpr (F16) return __builtin_bit_cast(uint16_t, (_Float16)x);
+  else return f32_to_bf16(x);
 }
 
 static __device__ __forceinline__ float bf16_to_f32(uint16_t x) {
@@ -59,6 +88,24 @@ static __device__ __forceinline__ float bf16lo_to_f32(uint32_t pair) {
 static __device__ __forceinline__ float bf16hi_to_f32(uint32_t pair) {
   return __builtin_bit_cast(float, pair & 0xffff0000u);
 }
+template <bool F16>
+static __device__ __forceinline__ float to_f32(uint16_t x) {
+  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, x);
+  else return bf16_to_f32(x);
+}
+template <bool F16>
+static __device__ __forceinline__ float lo_to_f32(uint32_t pair) {
+  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)(pair & 0xffffu));
+  else return bf16lo_to_f32(pair);
+}
+template <bool F16>
+static __device__ __forceinline__ float hi_to_f32(uint32_t pair) {
+  if constexpr (F16) return (float)__builtin_bit_cast(_Float16, (uint16_t)(pair >> 16));
+  else return bf16hi_to_f32(pair);
+}
+// 1.0 twice, as a packed pair of the kernel's 16-bit type
+template <bool F16>
+static __device__ __forceinline__ constexpr uint32_t ones2() { return F16 ? 0x3c003c00u : 0x3f803f80u; }
 
 // (hi16 of a | lo16 ... ) helpers for the in-register 4x4 bf16 transposes.
 // low_halves(a, b)  = (a.lo16 << 16) | b.lo16
@@ -84,20 +131,12 @@ static __device__ __forceinline__ uint2 ld8(const void* p) { return *reinterpret
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 static __device__ __forceinline__ uint4 ld16_stream(const void* p) {
-#ifdef MI_NT_LOADS
   const u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
   return make_uint4(v.x, v.y, v.z, v.w);
-#else
-  return ld16(p);
-#endif
 }
 static __device__ __forceinline__ uint2 ld8_stream(const void* p) {
-#ifdef MI_NT_LOADS
   const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
   return make_uint2(v.x, v.y);
-#else
-  return ld8(p);
-#endif
 }
 static __device__ __forceinline__ void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
 static __device__ __forceinline__ void st8(void* p, uint2 v) { *reinterpret_cast<uint2*>(p) = v; }

@@ -12,9 +12,9 @@
 //        megatron/core/models/common/embeddings/rope_utils.py:73-126),
 //   append_key_value_cache (dynamic_context.py:511-545) when a cache is given.
 //
-// Rounding: with `faithful != 0` every point where the unfused bf16 chain rounds
+// Rounding: with `faithful != 0` every point where the unfused 16-bit (bf16 or fp16) chain rounds
 // is rounded here too -- norm output, cos and sin, both products and their sum --
-// so the result equals the op-by-op bf16 evaluation; with `faithful == 0` the
+// so the result equals the op-by-op evaluation in that type; with `faithful == 0` the
 // whole expression is evaluated in fp32 and rounded once.
 //
 // grid = (tokens, groups of head vectors); a workgroup of 4 waves handles 4 (d = 128) or 8
@@ -57,7 +57,9 @@ struct NormRopeParams {
   float eps, mscale;
 };
 
-static __device__ __forceinline__ float round_bf16(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+// one rounding to the tensors' 16-bit type and back
+template <bool F16>
+static __device__ __forceinline__ float round16(float x) { return to_f32<F16>(f32_to_16<F16>(x)); }
 
 // First element of head vector `vec` (query heads first, then key heads) of token t.
 static __device__ __forceinline__ const uint16_t* head_vector(const NormRopeParams& p, int t, int vec) {
@@ -69,7 +71,7 @@ static __device__ __forceinline__ const uint16_t* head_vector(const NormRopePara
   return p.k + (int64_t)t * p.k_st + (int64_t)(vec - p.Hq) * p.k_hst;
 }
 
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p) {
   constexpr int LPV = D / 2;        // lanes per head vector
   constexpr int VPW = 64 / LPV;     // head vectors per wave
@@ -131,8 +133,8 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
           const float a = p.emb[(which ? kp : qp) * p.emb_stride + e];
           float c = cosf(a) * p.mscale, sn = sinf(a) * p.mscale;
           if (faithful) {
-            c = round_bf16(c);
-            sn = round_bf16(sn);
+            c = round16<F16>(c);
+            sn = round16<F16>(sn);
           }
           cs[which][w][0] = c;
           cs[which][w][1] = sn;
@@ -149,8 +151,8 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
     float x0 = 0.f, x1 = 0.f;
     if (active) {
       const uint16_t* src = head_vector(p, t, vec);
-      x0 = bf16_to_f32(src[i]);
-      x1 = bf16_to_f32(src[i + LPV]);
+      x0 = to_f32<F16>(src[i]);
+      x1 = to_f32<F16>(src[i + LPV]);
     }
     float y0 = x0, y1 = x1;
     if (p.norm != MI_NORM_NONE) {
@@ -162,12 +164,12 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
       y1 = x1 * rstd;
       const uint16_t* w = is_q ? p.q_w : p.k_w;
       if (p.norm == MI_NORM_RMS && w) {
-        y0 *= bf16_to_f32(w[i]);
-        y1 *= bf16_to_f32(w[i + LPV]);
+        y0 *= to_f32<F16>(w[i]);
+        y1 *= to_f32<F16>(w[i + LPV]);
       }
       if (faithful) {
-        y0 = round_bf16(y0);
-        y1 = round_bf16(y1);
+        y0 = round16<F16>(y0);
+        y1 = round16<F16>(y1);
       }
     }
     float o0 = y0, o1 = y1;
@@ -181,14 +183,14 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
           const float y = w ? y1 : y0;
           const float c = cs[is_q ? 0 : 1][w][0], sn = cs[is_q ? 0 : 1][w][1];
           const float yp = lds[slot][partner[w]] * sign[w];
-          const float out = faithful ? round_bf16(y * c) + round_bf16(yp * sn) : y * c + yp * sn;
+          const float out = faithful ? round16<F16>(y * c) + round16<F16>(yp * sn) : y * c + yp * sn;
           if (w) o1 = out; else o0 = out;
         }
       }
       __syncthreads();
     }
     if (active) {
-      const uint16_t b0 = f32_to_bf16(o0), b1 = f32_to_bf16(o1);
+      const uint16_t b0 = f32_to_16<F16>(o0), b1 = f32_to_16<F16>(o1);
       if (is_q) {
         uint16_t* dst = p.q_out + (int64_t)t * p.qo_st + (int64_t)head * D;
         dst[i] = b0;
@@ -229,7 +231,7 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
 // flight meanwhile: the first pass's head vector and the value row are requested before the chain,
 // and cos / sin / norm weights live in LDS or packed registers to stay within 64 VGPRs (8 waves per
 // SIMD).  Each angle's cos or sin is evaluated by exactly one thread of the workgroup.
-template <int D>
+template <int D, bool F16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void norm_rope_append_vec_kernel(NormRopeParams p) {
   constexpr int LPV = D / 8;        // lanes per head vector
   constexpr int VPW = 64 / LPV;     // head vectors per wave
@@ -292,7 +294,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
       if (e < p.rot) {
         const float a = p.emb[(which ? kp : qp) * p.emb_stride + e];
         r = (fn ? sinf(a) : cosf(a)) * p.mscale;
-        if (faithful) r = round_bf16(r);
+        if (faithful) r = round16<F16>(r);
       }
       cs_lds[which][fn][e] = r;
     }
@@ -303,7 +305,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
     }
   }
   // norm weights of this lane's elements, kept packed
-  uint4 wq_raw = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u), wk_raw = wq_raw;
+  uint4 wq_raw = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>()), wk_raw = wq_raw;
   if (p.norm == MI_NORM_RMS) {
     if (p.q_w) wq_raw = ld16(p.q_w + e0);
     if (p.k_w) wk_raw = ld16(p.k_w + e0);
@@ -327,7 +329,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
     {
       const uint32_t w4[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) { y[2 * j] = bf16lo_to_f32(w4[j]); y[2 * j + 1] = bf16hi_to_f32(w4[j]); }
+      for (int j = 0; j < 4; ++j) { y[2 * j] = lo_to_f32<F16>(w4[j]); y[2 * j + 1] = hi_to_f32<F16>(w4[j]); }
     }
     raw = load_vec(vec + gridDim.y * VPB);  // next pass, in flight during this one
     if (p.norm != MI_NORM_NONE) {
@@ -342,8 +344,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         float v = y[j] * rstd;
-        if (p.norm == MI_NORM_RMS) v *= (j & 1) ? bf16hi_to_f32(w4[j >> 1]) : bf16lo_to_f32(w4[j >> 1]);
-        y[j] = faithful ? round_bf16(v) : v;
+        if (p.norm == MI_NORM_RMS) v *= (j & 1) ? hi_to_f32<F16>(w4[j >> 1]) : lo_to_f32<F16>(w4[j >> 1]);
+        y[j] = faithful ? round16<F16>(v) : v;
       }
     }
     float o[8];
@@ -365,12 +367,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
         if (p.interleaved) yp = (j & 1) ? y[j ^ 1] : -y[j ^ 1];
         else yp = __shfl(y[j], src_lane, 64) * psign;
         // elements past the rotary width carry cos = 1, sin = 0 in the table
-        if (e0 + j < p.rot) o[j] = faithful ? round_bf16(y[j] * c[j]) + round_bf16(yp * sn[j]) : y[j] * c[j] + yp * sn[j];
+        if (e0 + j < p.rot) o[j] = faithful ? round16<F16>(y[j] * c[j]) + round16<F16>(yp * sn[j]) : y[j] * c[j] + yp * sn[j];
       }
     }
     if (active) {
-      const uint4 packed = make_uint4(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]),
-                                      pack_bf16x2(o[4], o[5]), pack_bf16x2(o[6], o[7]));
+      const uint4 packed = make_uint4(pack2<F16>(o[0], o[1]), pack2<F16>(o[2], o[3]),
+                                      pack2<F16>(o[4], o[5]), pack2<F16>(o[6], o[7]));
       if (is_q) {
         st16(p.q_out + (int64_t)t * p.qo_st + (int64_t)head * D + e0, packed);
       } else {
@@ -389,13 +391,18 @@ namespace {
 
 // Argument checks shared by both entry points, kernel choice and launch.  `p` carries every pointer,
 // stride and size; `name` prefixes error messages.
-int norm_rope_launch(NormRopeParams& p, hipStream_t st, const char* name) {
+int norm_rope_launch(NormRopeParams& p, int32_t dtype, const MiTuning* tuning, hipStream_t st, const char* name) {
   char msg[160];
   auto fail = [&](int code, const char* what) {
     snprintf(msg, sizeof msg, "%s: %s", name, what);
     return mi_fail(code, msg);
   };
   if (p.T == 0) return MI_OK;
+  MiTuning tune;
+  const int rc_t = mi_resolve_tuning(tuning, &tune, name);
+  if (rc_t != MI_OK) return rc_t;
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16) return fail(MI_ERR_UNSUPPORTED, "dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  const bool f16 = dtype == MI_DTYPE_FP16;
   if (p.T < 0 || p.Hq < 0 || p.Hkv < 0 || p.Hq + p.Hkv == 0) return fail(MI_ERR_SHAPE, "bad sizes");
   if ((p.Hq > 0 && (!p.q || !p.q_out)) || (p.Hkv > 0 && !p.k)) return fail(MI_ERR_NULL, "q / q_out / k missing");
   if (p.d != 64 && p.d != 128) return fail(MI_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
@@ -427,20 +434,23 @@ int norm_rope_launch(NormRopeParams& p, hipStream_t st, const char* name) {
                           (to_cache ? (p.chunk_elems | p.tok_elems | p.v_st | p.v_hst) : 0);
   // The 16-byte-per-lane kernel wins on many tokens; on a decode batch (a few hundred rows at most) the
   // element-wise kernel's shorter dependent chain does (4.8 against 5.7 us at 64 tokens).
-  const int mode = mi_tuning().norm_rope_vectorised;  // 0 never, 1 whenever the shapes allow, 2 automatic
+  const int mode = tune.norm_rope_vectorised;  // -1 never, 1 whenever the shapes allow, 2 automatic
   const bool vec = rot_ok && (ptrs & 15) == 0 && (strides & 7) == 0 && (mode == 1 || (mode == 2 && p.T >= 256));
   const int vpb = vec ? (p.d == 128 ? 16 : 32) : (p.d == 128 ? 4 : 8);
   const int passes = (p.Hq + p.Hkv + vpb - 1) / vpb;
   int gy = (2048 + p.T - 1) / p.T;
   gy = gy < 1 ? 1 : (gy > passes ? passes : gy);
   dim3 grid(p.T, gy);
-  if (vec) {
-    if (p.d == 128) hipLaunchKernelGGL((norm_rope_append_vec_kernel<128>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((norm_rope_append_vec_kernel<64>), grid, dim3(256), 0, st, p);
-  } else {
-    if (p.d == 128) hipLaunchKernelGGL((norm_rope_append_kernel<128>), grid, dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((norm_rope_append_kernel<64>), grid, dim3(256), 0, st, p);
-  }
+#define MI_NR_LAUNCH(KERNEL_)                                                                   \
+  do {                                                                                          \
+    if (p.d == 128 && f16) hipLaunchKernelGGL((KERNEL_<128, true>), grid, dim3(256), 0, st, p);   \
+    else if (p.d == 128) hipLaunchKernelGGL((KERNEL_<128, false>), grid, dim3(256), 0, st, p);    \
+    else if (f16) hipLaunchKernelGGL((KERNEL_<64, true>), grid, dim3(256), 0, st, p);             \
+    else hipLaunchKernelGGL((KERNEL_<64, false>), grid, dim3(256), 0, st, p);                     \
+  } while (0)
+  if (vec) MI_NR_LAUNCH(norm_rope_append_vec_kernel);
+  else MI_NR_LAUNCH(norm_rope_append_kernel);
+#undef MI_NR_LAUNCH
   return mi_check_launch(name);
 }
 
@@ -456,7 +466,7 @@ extern "C" int mi_norm_rope_append(
     int64_t kv_stride_chunk, int64_t kv_stride_tok, const int64_t* token_to_chunk_idx,
     const int64_t* token_to_local_pos, const int32_t* block_table, int64_t bt_stride,
     const int32_t* kv_lens, int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv,
-    int32_t head_dim, int32_t faithful_rounding, void* stream) {
+    int32_t head_dim, int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning, void* stream) {
   NormRopeParams p = {};
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_gst = 0; p.q_group = Hq > 0 ? Hq : 1;
   p.q_out = (uint16_t*)q_out; p.qo_st = q_out_stride_tok;
@@ -473,7 +483,7 @@ extern "C" int mi_norm_rope_append(
   p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.d = head_dim; p.rot = rot_dim; p.chunk = chunk_tokens;
   p.norm = norm_kind; p.interleaved = rotary_interleaved; p.faithful = faithful_rounding;
   p.eps = eps; p.mscale = mscale;
-  return norm_rope_launch(p, (hipStream_t)stream, "mi_norm_rope_append");
+  return norm_rope_launch(p, dtype, tuning, (hipStream_t)stream, "mi_norm_rope_append");
 }
 
 extern "C" int mi_qkv_norm_rope_append(
@@ -484,7 +494,7 @@ extern "C" int mi_qkv_norm_rope_append(
     int64_t kv_stride_chunk, int64_t kv_stride_tok, const int64_t* token_to_chunk_idx,
     const int64_t* token_to_local_pos, const int32_t* block_table, int64_t bt_stride,
     const int32_t* kv_lens, int32_t chunk_tokens, int32_t T, int32_t Hq, int32_t Hkv,
-    int32_t head_dim, int32_t faithful_rounding, void* stream) {
+    int32_t head_dim, int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning, void* stream) {
   if (T == 0) return MI_OK;
   if (!mixed_qkv) return mi_fail(MI_ERR_NULL, "mi_qkv_norm_rope_append: mixed_qkv missing");
   if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0)
@@ -512,5 +522,5 @@ extern "C" int mi_qkv_norm_rope_append(
   p.T = T; p.Hq = Hq; p.Hkv = Hkv; p.d = head_dim; p.rot = rot_dim; p.chunk = chunk_tokens;
   p.norm = norm_kind; p.interleaved = rotary_interleaved; p.faithful = faithful_rounding;
   p.eps = eps; p.mscale = mscale;
-  return norm_rope_launch(p, (hipStream_t)stream, "mi_qkv_norm_rope_append");
+  return norm_rope_launch(p, dtype, tuning, (hipStream_t)stream, "mi_qkv_norm_rope_append");
 }

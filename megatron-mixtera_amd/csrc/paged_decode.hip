@@ -76,7 +76,7 @@ static __device__ __forceinline__ int chunk_of(int tok, uint64_t magic) {
 // HDK = width of the keys (and queries), HDV = width of the values (and of the output).  They differ
 // only for the latent cache of multi-latent attention (576 / 512: the value is the first 512 of the
 // shared 576-wide row, the caller points both cache arguments at the same buffer).
-template <int HDK, int HDV, int NT, bool FP8>
+template <int HDK, int HDV, int NT, bool FP8, bool F16>
 static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int row, int h, int len,
                                                       int start, int end, bool whole, int slot, int lane,
                                                       uint8_t* q_lds) {
@@ -92,7 +92,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   constexpr int DV = HDV / 16;
   constexpr int VW = DV * (FP8 ? 1 : 2) / 16;  // 16-byte loads per token and lane of the value operand (0: 8 bytes)
   static_assert((HDK == 64 || HDK == 128 || HDK == 576) && (HDV == 64 || HDV == 128 || HDV == 512), "head widths");
-  static_assert(!FP8 || (HDK == 128 && HDV == 128), "fp8 KV: head_dim 128");
+  static_assert(!FP8 || (HDK == 128 && HDV == 128 && !F16), "fp8 KV: head_dim 128, bf16 queries");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
   // tile base addresses below run on the scalar unit instead of costing vector instructions.
@@ -268,7 +268,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     kcur.sc = ksc_tile = uniform_f(ksc_first);
     vcur.sc = vsc_tile = uniform_f(vsc_first);
   }
-  const uint2 ones = make_uint2(0x3f803f80u, 0x3f803f80u);  // four bf16 1.0
+  const uint2 ones = make_uint2(ones2<F16>(), ones2<F16>());  // four times 1.0
   for (int T = start; T < end; T += 16 * NT) {
     // ---- S^T = K Q^T ---------------------------------------------------------
     // The tile lies in one chunk, so one K scale and one V scale hold for all of it; the score
@@ -285,13 +285,13 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
         for (int kk = 0; kk < KS / 2; ++kk) {
           const uint2 a0 = fp8x4_to_bf16x4(kf[u][kk].x), a1 = fp8x4_to_bf16x4(kf[u][kk].y);
           const uint2 b0 = fp8x4_to_bf16x4(kf[u][kk].z), b1 = fp8x4_to_bf16x4(kf[u][kk].w);
-          sacc = mfma_16x16x32(make_uint4(a0.x, a0.y, a1.x, a1.y), qf[2 * kk], sacc);
-          sacc = mfma_16x16x32(make_uint4(b0.x, b0.y, b1.x, b1.y), qf[2 * kk + 1], sacc);
+          sacc = mfma_16x16x32<F16>(make_uint4(a0.x, a0.y, a1.x, a1.y), qf[2 * kk], sacc);
+          sacc = mfma_16x16x32<F16>(make_uint4(b0.x, b0.y, b1.x, b1.y), qf[2 * kk + 1], sacc);
         }
       } else {
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk)
-          sacc = mfma_16x16x32(kf[u][kk], Q_IN_LDS ? lds_ld16(q_frag + 64 * kk) : qf[Q_IN_LDS ? 0 : kk], sacc);
+          sacc = mfma_16x16x32<F16>(kf[u][kk], Q_IN_LDS ? lds_ld16(q_frag + 64 * kk) : qf[Q_IN_LDS ? 0 : kk], sacc);
       }
       if (ragged) {
         const int tok0 = T + 16 * u + 4 * g;
@@ -327,8 +327,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       const float p1 = fast_exp2(__builtin_fmaf(sc[u][1], mul, neg));
       const float p2 = fast_exp2(__builtin_fmaf(sc[u][2], mul, neg));
       const float p3 = fast_exp2(__builtin_fmaf(sc[u][3], mul, neg));
-      pf[u] = make_uint2(pack_bf16x2(p0, p1), pack_bf16x2(p2, p3));
-      psum4 = mfma_16x16x16(ones, pf[u], psum4);
+      pf[u] = make_uint2(pack2<F16>(p0, p1), pack2<F16>(p2, p3));
+      psum4 = mfma_16x16x16<F16>(ones, pf[u], psum4);
     }
     // (every slot of psum4 holds the row sum of this lane's query row)
     l_run = l_run * alpha + (FP8 ? psum4[0] * __builtin_amdgcn_rcpf(vscale) : psum4[0]);
@@ -351,18 +351,18 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
           const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3][w]);
 #pragma unroll
           for (int pr = 0; pr < 4; ++pr) {
-            acc[8 * w + 2 * pr] = mfma_16x16x16(
+            acc[8 * w + 2 * pr] = mfma_16x16x16<F16>(
                 make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr])), pf[u], acc[8 * w + 2 * pr]);
-            acc[8 * w + 2 * pr + 1] = mfma_16x16x16(
+            acc[8 * w + 2 * pr + 1] = mfma_16x16x16<F16>(
                 make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr])), pf[u], acc[8 * w + 2 * pr + 1]);
           }
         }
       } else if (!FP8) {  // bf16, value width 64: four values per token per lane
         const uint2 a = vf8[u][0], b = vf8[u][1], c = vf8[u][2], d = vf8[u][3];
-        acc[0] = mfma_16x16x16(make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x)), pf[u], acc[0]);
-        acc[1] = mfma_16x16x16(make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x)), pf[u], acc[1]);
-        acc[2] = mfma_16x16x16(make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y)), pf[u], acc[2]);
-        acc[3] = mfma_16x16x16(make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y)), pf[u], acc[3]);
+        acc[0] = mfma_16x16x16<F16>(make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x)), pf[u], acc[0]);
+        acc[1] = mfma_16x16x16<F16>(make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x)), pf[u], acc[1]);
+        acc[2] = mfma_16x16x16<F16>(make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y)), pf[u], acc[2]);
+        acc[3] = mfma_16x16x16<F16>(make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y)), pf[u], acc[3]);
       } else {  // fp8, width 128: eight bytes per token per lane
         uint2 w[4][2];  // [token j][half] -> two packed bf16 pairs (4 d values)
 #pragma unroll
@@ -372,13 +372,13 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
         }
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-          acc[4 * hf + 0] = mfma_16x16x16(
+          acc[4 * hf + 0] = mfma_16x16x16<F16>(
               make_uint2(low_halves(w[1][hf].x, w[0][hf].x), low_halves(w[3][hf].x, w[2][hf].x)), pf[u], acc[4 * hf + 0]);
-          acc[4 * hf + 1] = mfma_16x16x16(
+          acc[4 * hf + 1] = mfma_16x16x16<F16>(
               make_uint2(high_halves(w[1][hf].x, w[0][hf].x), high_halves(w[3][hf].x, w[2][hf].x)), pf[u], acc[4 * hf + 1]);
-          acc[4 * hf + 2] = mfma_16x16x16(
+          acc[4 * hf + 2] = mfma_16x16x16<F16>(
               make_uint2(low_halves(w[1][hf].y, w[0][hf].y), low_halves(w[3][hf].y, w[2][hf].y)), pf[u], acc[4 * hf + 2]);
-          acc[4 * hf + 3] = mfma_16x16x16(
+          acc[4 * hf + 3] = mfma_16x16x16<F16>(
               make_uint2(high_halves(w[1][hf].y, w[0][hf].y), high_halves(w[3][hf].y, w[2][hf].y)), pf[u], acc[4 * hf + 3]);
         }
       }
@@ -401,13 +401,13 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
 #pragma unroll
         for (int w = 0; w < DV / 8; ++w)
           st16(o + DV * i + 8 * w,
-               make_uint4(pack_bf16x2(acc[8 * w + 0][i] * inv, acc[8 * w + 1][i] * inv),
-                          pack_bf16x2(acc[8 * w + 2][i] * inv, acc[8 * w + 3][i] * inv),
-                          pack_bf16x2(acc[8 * w + 4][i] * inv, acc[8 * w + 5][i] * inv),
-                          pack_bf16x2(acc[8 * w + 6][i] * inv, acc[8 * w + 7][i] * inv)));
+               make_uint4(pack2<F16>(acc[8 * w + 0][i] * inv, acc[8 * w + 1][i] * inv),
+                          pack2<F16>(acc[8 * w + 2][i] * inv, acc[8 * w + 3][i] * inv),
+                          pack2<F16>(acc[8 * w + 4][i] * inv, acc[8 * w + 5][i] * inv),
+                          pack2<F16>(acc[8 * w + 6][i] * inv, acc[8 * w + 7][i] * inv)));
       } else {
-        st8(o + 4 * i, make_uint2(pack_bf16x2(acc[0][i] * inv, acc[1][i] * inv),
-                                  pack_bf16x2(acc[2][i] * inv, acc[3][i] * inv)));
+        st8(o + 4 * i, make_uint2(pack2<F16>(acc[0][i] * inv, acc[1][i] * inv),
+                                  pack2<F16>(acc[2][i] * inv, acc[3][i] * inv)));
       }
     }
   } else {
@@ -513,7 +513,7 @@ static __device__ __forceinline__ void walk_segments(const DecodeParams& p, Seg 
 }
 
 // The body of the register-streaming kernels: one wavefront per (virtual) KV head.
-template <int HDK, int HDV, int NT, bool FP8>
+template <int HDK, int HDV, int NT, bool FP8, bool F16>
 static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p) {
   extern __shared__ int cum[];
   const int lane = threadIdx.x & 63;
@@ -523,21 +523,22 @@ static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p)
   uint8_t* const q_lds = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15) +
                          (size_t)wave * 16 * (HDK * 2 + 16);
   walk_segments<16 * NT>(p, [&](int r, int row, int len, int start, int end, bool whole, int slot) {
-    decode_segment<HDK, HDV, NT, FP8>(p, r, row, h, len, start, end, whole, slot, lane, q_lds);
+    decode_segment<HDK, HDV, NT, FP8, F16>(p, r, row, h, len, start, end, whole, slot, lane, q_lds);
   });
 }
 
-template <int HD, int NT, bool FP8, int MINW>
+template <int HD, int NT, bool FP8, int MINW, bool F16>
 __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
-  decode_stream_body<HD, HD, NT, FP8>(p);
+  decode_stream_body<HD, HD, NT, FP8, F16>(p);
 }
 
 // Multi-latent attention, absorbed form: every query head attends to the same 576-wide latent rows
 // (scores over all 576 values, output = weighted sum of the first 512).  A wavefront takes 16 query
 // heads; with 128 accumulator registers per lane a SIMD holds one wavefront, hence at most four per
 // workgroup.
+template <bool F16>
 __global__ __launch_bounds__(256, 1) void paged_mla_decode_stream_kernel(DecodeParams p) {
-  decode_stream_body<576, 512, 1, false>(p);
+  decode_stream_body<576, 512, 1, false, F16>(p);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -556,7 +557,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_stream_kernel(DecodeP
 constexpr int kMlaTile = 64;                 // tokens per staged tile
 constexpr int kMlaPitch = 576 * 2 + 16;      // LDS bytes per staged row: 16 rows of a fragment read cover all banks
 
-template <int PARTS>
+template <int PARTS, bool F16>
 __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodeParams p) {
   constexpr int HDK = 576, HDV = 512, KS = HDK / 32;
   constexpr int NG = 8 / PARTS;               // head groups per workgroup
@@ -587,7 +588,7 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
   // fragment reads: keys as the A operand of the scores, values transposed as the A operand of P.V
   const int kfrag_off = m16 * kMlaPitch + 16 * g;
   const int vfrag_off = (4 * g + (m16 >> 2)) * kMlaPitch + 2 * c0 + 8 * (m16 & 3);
-  const uint4 ones = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+  const uint4 ones = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
 
   walk_segments<kMlaTile>(p, [&](int r, int row, int len, int start, int end, bool whole, int slot) {
     r = __builtin_amdgcn_readfirstlane(r);
@@ -642,7 +643,7 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
         const uint8_t* ks = buf + kfrag_off + 16 * su * kMlaPitch + 64 * k0;
         f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kk = 0; kk < KSW; ++kk) sacc = mfma_16x16x32(lds_ld16(ks + 64 * kk), qf[kk], sacc);
+        for (int kk = 0; kk < KSW; ++kk) sacc = mfma_16x16x32<F16>(lds_ld16(ks + 64 * kk), qf[kk], sacc);
         sbuf[((k0 ? 1 : 0) * 4 + su) * 64 + lane] = make_float4(sacc[0], sacc[1], sacc[2], sacc[3]);
       }
       __syncthreads();
@@ -681,7 +682,7 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
         const float p1 = fast_exp2(__builtin_fmaf(sc[u][1], mul, -m_new));
         const float p2 = fast_exp2(__builtin_fmaf(sc[u][2], mul, -m_new));
         const float p3 = fast_exp2(__builtin_fmaf(sc[u][3], mul, -m_new));
-        pf[u] = make_uint2(pack_bf16x2(p0, p1), pack_bf16x2(p2, p3));
+        pf[u] = make_uint2(pack2<F16>(p0, p1), pack2<F16>(p2, p3));
       }
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
@@ -698,9 +699,9 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
 #pragma unroll
         for (int e = 0; e < DVW; ++e) {
           const uint2 a0 = lds_ld8_tr(vs + 32 * e), a1 = lds_ld8_tr(vs + 16 * kMlaPitch + 32 * e);
-          acc[e] = mfma_16x16x32(make_uint4(a0.x, a0.y, a1.x, a1.y), pp, acc[e]);
+          acc[e] = mfma_16x16x32<F16>(make_uint4(a0.x, a0.y, a1.x, a1.y), pp, acc[e]);
         }
-        psum4 = mfma_16x16x32(ones, pp, psum4);
+        psum4 = mfma_16x16x32<F16>(ones, pp, psum4);
       }
       l_run = l_run * alpha + psum4[0];
       if (t + 1 < ntile) store(t + 1);
@@ -714,8 +715,8 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
         uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + c0 + 4 * g;
 #pragma unroll
         for (int e = 0; e < DVW; ++e)
-          st8(o + 16 * e, make_uint2(pack_bf16x2(acc[e][0] * inv, acc[e][1] * inv),
-                                     pack_bf16x2(acc[e][2] * inv, acc[e][3] * inv)));
+          st8(o + 16 * e, make_uint2(pack2<F16>(acc[e][0] * inv, acc[e][1] * inv),
+                                     pack2<F16>(acc[e][2] * inv, acc[e][3] * inv)));
       } else {
         const int64_t prow = (int64_t)slot * p.Hq + hq;
         float* o = p.part_o + prow * HDV + c0 + 4 * g;
@@ -733,7 +734,7 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
 // shared the request; zero-length rows get zeros.  blockDim.x = HD * S: S groups of HD threads take the
 // segments round-robin in batches of 8 (a request cut over hundreds of workgroups is a chain of dependent
 // memory round trips otherwise) and group 0 folds the S running (maximum, numerator, denominator) triples.
-template <int HD>
+template <int HD, bool F16>
 __global__ __launch_bounds__(1024) void paged_decode_merge_kernel(DecodeParams p) {
   constexpr int kMaxGroups = 1024 / HD;
   __shared__ float red[3][kMaxGroups > 1 ? 1024 : 1];
@@ -786,7 +787,7 @@ __global__ __launch_bounds__(1024) void paged_decode_merge_kernel(DecodeParams p
       mx = m_new;
     }
   }
-  *o = f32_to_bf16(num / den);
+  *o = f32_to_16<F16>(num / den);
 }
 
 // Thread groups per merge workgroup: one per 8 segments a request is expected to be cut into.
@@ -799,8 +800,8 @@ static int merge_groups(int grid_x, int R, int head_dim) {
   return g < 1 ? 1 : g;
 }
 
-static int pick_waves_per_block(int Hkv) {
-  int cap = mi_tuning().decode_waves_per_block;
+static int pick_waves_per_block(int Hkv, const MiTuning& tune) {
+  int cap = tune.decode_waves_per_block;
   if (cap < 1 || cap > 8) cap = 8;
   for (int w = cap; w >= 1; --w)
     if (Hkv % w == 0) return w;
@@ -821,12 +822,12 @@ static int device_cu_count() {
 
 // Workgroups along the flattened tile sequence: enough to put `decode_wgs_per_cu`
 // workgroups of 8 waves (or the equivalent in smaller workgroups) on every CU.
-int decode_grid_size(int Hkv) {
-  const int forced = mi_tuning().decode_grid;
+int decode_grid_size(int Hkv, const MiTuning& tune) {
+  const int forced = tune.decode_grid;
   if (forced > 0) return forced;
-  const int wpb = pick_waves_per_block(Hkv);
+  const int wpb = pick_waves_per_block(Hkv, tune);
   const int head_groups = Hkv / wpb;
-  int per_cu = mi_tuning().decode_wgs_per_cu * (8 / wpb);
+  int per_cu = tune.decode_wgs_per_cu * (8 / wpb);
   int grid = device_cu_count() * per_cu / head_groups;
   return grid < 1 ? 1 : grid;
 }
@@ -837,10 +838,12 @@ using namespace mi;
 
 extern "C" int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                              int32_t chunk_tokens, int32_t max_kv_len,
-                                             int32_t split_tokens) {
-  (void)chunk_tokens; (void)max_kv_len; (void)split_tokens;
+                                             int32_t split_tokens, const MiTuning* tuning) {
+  (void)chunk_tokens; (void)max_kv_len; (void)split_tokens;  // (the size depends on R, the head counts and the grid only)
   if (R <= 0 || Hq <= 0 || Hkv <= 0 || head_dim <= 0) return 0;
-  const int64_t slots = (int64_t)decode_grid_size(Hkv) + R;
+  MiTuning tune;
+  if (mi_resolve_tuning(tuning, &tune, "mi_decode_workspace_bytes") != MI_OK) return -1;
+  const int64_t slots = (int64_t)decode_grid_size(Hkv, tune) + R;
   return slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
 
@@ -851,8 +854,13 @@ int mi::launch_paged_decode(
     void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
     int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
     int32_t split_tokens, float softmax_scale, int32_t kv_dtype, const float* k_scales,
-    const float* v_scales, void* stream) {
+    const float* v_scales, int32_t dtype, const MiTuning& tune, void* stream) {
   if (R == 0) return MI_OK;
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  const bool f16 = dtype == MI_DTYPE_FP16;
+  if (f16 && kv_dtype == MI_KV_FP8_E4M3)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: an fp8 cache needs bf16 queries");
   if (!q || !k_cache || !v_cache || !block_table || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_decode_attention: null pointer argument");
   if (R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv)
@@ -880,7 +888,7 @@ int mi::launch_paged_decode(
   if ((int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: batch too large for the in-LDS prefix sum (7680 requests)");
 
-  const int grid_x = decode_grid_size(Hkv);
+  const int grid_x = decode_grid_size(Hkv, tune);
   const int64_t slots = (int64_t)grid_x + R;
   const int64_t need = slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
   if (!workspace || workspace_bytes < need)
@@ -889,10 +897,10 @@ int mi::launch_paged_decode(
     return mi_fail(MI_ERR_ALIGN, "mi_paged_decode_attention: workspace must be 16-byte aligned");
 
   // 16-token sub-tiles per loop iteration (0 = automatic).
-  int nt = mi_tuning().decode_tile_subtiles;
+  int nt = tune.decode_tile_subtiles;
   if (nt != 1 && nt != 2 && nt != 4) nt = kv_dtype == MI_KV_FP8_E4M3 ? 4 : 2;
   while (chunk_tokens % (16 * nt)) nt >>= 1;  // a tile must not straddle two chunks
-  const int minw = mi_tuning().decode_min_waves;
+  const int minw = tune.decode_min_waves;
   const int tk = 16 * nt;
   // a small batch is cut finer than a large one needs: 64 tokens per workgroup put a single 8 192-token
   // request on 128 CUs (17.8 us against 33 us with 256-token spans); large batches get equal spans anyway
@@ -914,36 +922,35 @@ int mi::launch_paged_decode(
   p.grid = grid_x;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
 
-  const int wpb = pick_waves_per_block(Hkv);
+  const int wpb = pick_waves_per_block(Hkv, tune);
   dim3 grid(grid_x, Hkv / wpb), block(64 * wpb);
   const size_t lds = (size_t)R * 2 * sizeof(int32_t);
   hipStream_t st = (hipStream_t)stream;
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
   if (timed) (void)hipEventRecord(ev_a, st);
-#define MI_LAUNCH_DECODE(HD_, FP8_)                                                                             \
-  do {                                                                                                          \
-    if (nt == 1 && minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 4>), grid, block, lds, st, p); \
-    else if (nt == 1) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 3>), grid, block, lds, st, p);       \
-    else if (minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 4>), grid, block, lds, st, p);     \
-    else if (minw == 3) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 3>), grid, block, lds, st, p);     \
-    else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 2>), grid, block, lds, st, p);                    \
+#define MI_LAUNCH_DECODE(HD_, FP8_, F16_)                                                                              \
+  do {                                                                                                                 \
+    if (nt == 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 4, FP8_, 2, F16_>), grid, block, lds, st, p);          \
+    else if (nt == 1 && minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 4, F16_>), grid, block, lds, st, p); \
+    else if (nt == 1) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, FP8_, 3, F16_>), grid, block, lds, st, p);     \
+    else if (minw >= 4) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 4, F16_>), grid, block, lds, st, p);   \
+    else if (minw == 3) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 3, F16_>), grid, block, lds, st, p);   \
+    else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 2, F16_>), grid, block, lds, st, p);                  \
   } while (0)
-  if (kv_dtype == MI_KV_FP8_E4M3 && nt == 4)
-    hipLaunchKernelGGL((paged_decode_stream_kernel<128, 4, true, 2>), grid, block, lds, st, p);
-  else if (head_dim == 128 && nt == 4)
-    hipLaunchKernelGGL((paged_decode_stream_kernel<128, 4, false, 2>), grid, block, lds, st, p);
-  else if (nt == 4)
-    hipLaunchKernelGGL((paged_decode_stream_kernel<64, 4, false, 2>), grid, block, lds, st, p);
-  else if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true);
-  else if (head_dim == 128) MI_LAUNCH_DECODE(128, false);
-  else MI_LAUNCH_DECODE(64, false);
+  if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true, false);
+  else if (head_dim == 128 && f16) MI_LAUNCH_DECODE(128, false, true);
+  else if (head_dim == 128) MI_LAUNCH_DECODE(128, false, false);
+  else if (f16) MI_LAUNCH_DECODE(64, false, true);
+  else MI_LAUNCH_DECODE(64, false, false);
 #undef MI_LAUNCH_DECODE
   if (timed) (void)hipEventRecord(ev_b, st);
   dim3 mgrid(Hq, R);
   const dim3 mblock(head_dim * merge_groups(p.grid, R, head_dim));
-  if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128>), mgrid, mblock, 0, st, p);
-  else hipLaunchKernelGGL((paged_decode_merge_kernel<64>), mgrid, mblock, 0, st, p);
+  if (head_dim == 128 && f16) hipLaunchKernelGGL((paged_decode_merge_kernel<128, true>), mgrid, mblock, 0, st, p);
+  else if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128, false>), mgrid, mblock, 0, st, p);
+  else if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<64, true>), mgrid, mblock, 0, st, p);
+  else hipLaunchKernelGGL((paged_decode_merge_kernel<64, false>), mgrid, mblock, 0, st, p);
   return mi_check_launch("mi_paged_decode_attention");
 }
 
@@ -954,12 +961,15 @@ extern "C" int mi_paged_decode_attention(
     int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
     int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len,
     int32_t split_tokens, float softmax_scale, int32_t kv_dtype, const float* k_scales,
-    const float* v_scales, void* stream) {
+    const float* v_scales, int32_t dtype, const MiTuning* tuning, void* stream) {
   (void)max_kv_len;
+  MiTuning tune;
+  const int rc = mi_resolve_tuning(tuning, &tune, "mi_paged_decode_attention");
+  if (rc != MI_OK) return rc;
   return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
                              kv_stride_head, block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok,
                              o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
-                             split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
+                             split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, dtype, tune, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -999,10 +1009,13 @@ extern "C" int mi_paged_decode_attention_noalloc(
     const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
     int64_t o_stride_tok, int64_t o_stride_head, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
     int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens, float softmax_scale, int32_t kv_dtype,
-    const float* k_scales, const float* v_scales, void* stream) {
+    const float* k_scales, const float* v_scales, int32_t dtype, const MiTuning* tuning, void* stream) {
   (void)max_kv_len;
+  MiTuning tune;
+  const int rc_t = mi_resolve_tuning(tuning, &tune, "mi_paged_decode_attention_noalloc");
+  if (rc_t != MI_OK) return rc_t;
   if (R > 0 && Hq > 0 && Hkv > 0 && head_dim > 0 &&
-      mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, chunk_tokens, max_kv_len, split_tokens) > kNoAllocScratchBytes)
+      mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, chunk_tokens, max_kv_len, split_tokens, tuning) > kNoAllocScratchBytes)
     return mi_fail(MI_ERR_WORKSPACE,
                    "mi_paged_decode_attention_noalloc: these sizes need more than the 16 MiB of built-in scratch "
                    "(see mi_decode_workspace_bytes); use mi_paged_decode_attention with a workspace");
@@ -1015,7 +1028,7 @@ extern "C" int mi_paged_decode_attention_noalloc(
   return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
                              kv_stride_head, block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok,
                              o_stride_head, ptr, kNoAllocScratchBytes, R, Hq, Hkv, head_dim, chunk_tokens,
-                             split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
+                             split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, dtype, tune, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1031,8 +1044,8 @@ static int mla_waves_per_block(int groups) {
   return 1;
 }
 // spans along the flattened tile sequence: four wavefronts on every CU in total
-static int mla_grid_size(int groups) {
-  const int forced = mi_tuning().decode_grid;
+static int mla_grid_size(int groups, const MiTuning& tune) {
+  const int forced = tune.decode_grid;
   if (forced > 0) return forced;
   const int grid = device_cu_count() * 4 / groups;
   return grid < 1 ? 1 : grid;
@@ -1040,10 +1053,12 @@ static int mla_grid_size(int groups) {
 static int mla_groups(int Hq) { return Hq <= 16 ? 1 : Hq / 16; }
 }  // namespace mi
 
-extern "C" int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v) {
+extern "C" int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v, const MiTuning* tuning) {
   if (R <= 0 || Hq <= 0 || head_dim_v <= 0) return 0;
+  MiTuning tune;
+  if (mi_resolve_tuning(tuning, &tune, "mi_mla_decode_workspace_bytes") != MI_OK) return -1;
   // (the per-wavefront kernel uses the larger grid of the two: enough for either)
-  const int64_t slots = (int64_t)mla_grid_size(mla_groups(Hq)) + R;
+  const int64_t slots = (int64_t)mla_grid_size(mla_groups(Hq), tune) + R;
   return slots * Hq * (head_dim_v + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
 
@@ -1052,9 +1067,15 @@ extern "C" int mi_paged_mla_decode_attention(
     int64_t kv_stride_tok, const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
     int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq,
     int32_t head_dim_k, int32_t head_dim_v, int32_t chunk_tokens, int32_t max_kv_len, float softmax_scale,
-    void* stream) {
+    int32_t dtype, const MiTuning* tuning, void* stream) {
   (void)max_kv_len;
   if (R == 0) return MI_OK;
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  const bool f16 = dtype == MI_DTYPE_FP16;
+  MiTuning tune;
+  const int rc_t = mi_resolve_tuning(tuning, &tune, "mi_paged_mla_decode_attention");
+  if (rc_t != MI_OK) return rc_t;
   if (!q || !kv_cache || !block_table || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_mla_decode_attention: null pointer argument");
   if (R < 0 || Hq <= 0) return mi_fail(MI_ERR_SHAPE, "mi_paged_mla_decode_attention: need R >= 0 and Hq > 0");
@@ -1079,11 +1100,11 @@ extern "C" int mi_paged_mla_decode_attention(
   // of 64 tokens that do not straddle chunks), or one wavefront per head group streaming on its own.
   const size_t lds_head = ((size_t)R * 2 * sizeof(int32_t) + 15) & ~(size_t)15;
   const size_t lds_shared = lds_head + (size_t)2 * kMlaTile * kMlaPitch + 8 * 1024;  // tiles + partial scores
-  const bool shared_tile = chunk_tokens % kMlaTile == 0 && mi_tuning().mla_decode_lds != 0 && lds_shared <= 160 * 1024;
+  const bool shared_tile = chunk_tokens % kMlaTile == 0 && tune.mla_decode_lds > 0 && lds_shared <= 160 * 1024;
   const int parts = (groups % 2 == 0) ? 4 : 8;            // output-column parts per head group
   const int wg_y = shared_tile ? groups / (8 / parts) : 0;  // workgroups per span (shared-tile kernel)
-  int grid_x = mla_grid_size(groups);
-  if (shared_tile && mi_tuning().decode_grid <= 0) {
+  int grid_x = mla_grid_size(groups, tune);
+  if (shared_tile && tune.decode_grid <= 0) {
     grid_x = device_cu_count() / wg_y;
     if (grid_x < 1) grid_x = 1;
   }
@@ -1120,22 +1141,32 @@ extern "C" int mi_paged_mla_decode_attention(
   if (hipGetDevice(&dev_id) != hipSuccess || dev_id < 0 || dev_id >= 64) dev_id = 0;
   if (!lds_limit_raised[dev_id].load(std::memory_order_acquire)) {
     const hipFuncAttribute attr = hipFuncAttributeMaxDynamicSharedMemorySize;
-    if (hipFuncSetAttribute((const void*)paged_mla_decode_stream_kernel, attr, 160 * 1024) != hipSuccess ||
-        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<4>, attr, 160 * 1024) != hipSuccess ||
-        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8>, attr, 160 * 1024) != hipSuccess)
+    if (hipFuncSetAttribute((const void*)paged_mla_decode_stream_kernel<false>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_stream_kernel<true>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<4, false>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<4, true>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8, false>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8, true>, attr, 160 * 1024) != hipSuccess)
       return mi_fail(MI_ERR_LAUNCH, "mi_paged_mla_decode_attention: cannot raise the dynamic LDS limit");
     lds_limit_raised[dev_id].store(true, std::memory_order_release);
   }
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
   if (timed) (void)hipEventRecord(ev_a, st);
-  if (shared_tile && parts == 4)
-    hipLaunchKernelGGL(paged_mla_decode_lds_kernel<4>, dim3(grid_x, wg_y), dim3(512), lds, st, p);
-  else if (shared_tile)
-    hipLaunchKernelGGL(paged_mla_decode_lds_kernel<8>, dim3(grid_x, wg_y), dim3(512), lds, st, p);
-  else
-    hipLaunchKernelGGL(paged_mla_decode_stream_kernel, dim3(grid_x, groups / wpb), dim3(64 * wpb), lds, st, p);
+#define MI_LAUNCH_MLA(F16_)                                                                                       \
+  do {                                                                                                            \
+    if (shared_tile && parts == 4)                                                                                \
+      hipLaunchKernelGGL((paged_mla_decode_lds_kernel<4, F16_>), dim3(grid_x, wg_y), dim3(512), lds, st, p);       \
+    else if (shared_tile)                                                                                         \
+      hipLaunchKernelGGL((paged_mla_decode_lds_kernel<8, F16_>), dim3(grid_x, wg_y), dim3(512), lds, st, p);       \
+    else                                                                                                          \
+      hipLaunchKernelGGL((paged_mla_decode_stream_kernel<F16_>), dim3(grid_x, groups / wpb), dim3(64 * wpb), lds, st, p); \
+  } while (0)
+  if (f16) MI_LAUNCH_MLA(true); else MI_LAUNCH_MLA(false);
+#undef MI_LAUNCH_MLA
   if (timed) (void)hipEventRecord(ev_b, st);
-  hipLaunchKernelGGL((paged_decode_merge_kernel<512>), dim3(Hq, R), dim3(512 * merge_groups(grid_x, R, 512)), 0, st, p);
+  const dim3 mgrid(Hq, R), mblock(512 * merge_groups(grid_x, R, 512));
+  if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<512, true>), mgrid, mblock, 0, st, p);
+  else hipLaunchKernelGGL((paged_decode_merge_kernel<512, false>), mgrid, mblock, 0, st, p);
   return mi_check_launch("mi_paged_mla_decode_attention");
 }

@@ -51,7 +51,7 @@ struct PrefillParams {
 // NQ = 16-row tiles per wave; a workgroup always covers 256 rows (16 / NQ waves).
 // HDK = width of queries and keys, HDV = width of values and of the output (they differ for the
 // decompressed caches of multi-latent attention: 192 / 128); the value cache has its own strides.
-template <int HDK, int HDV, int NT, int NQ>
+template <int HDK, int HDV, int NT, int NQ, bool F16>
 __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillParams p) {
   constexpr int KS = HDK / 32;
   constexpr int DV = HDV / 16;
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
       for (int u = 0; u < NT; ++u) {
         f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32(kf[u][kk], qf[nt][kk], sacc);
+        for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32<F16>(kf[u][kk], qf[nt][kk], sacc);
         s[nt][u] = sacc;
       }
     }
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
           pv[i] = fast_exp2(__builtin_fmaf(s[nt][u][i], scale, neg));
           psum += pv[i];
         }
-        pf[nt][u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
+        pf[nt][u] = make_uint2(pack2<F16>(pv[0], pv[1]), pack2<F16>(pv[2], pv[3]));
       }
       l_run[nt] = l_run[nt] * alpha + psum;
       // The running max rarely moves once a few tiles have been seen: skip the rescale of the
@@ -286,7 +286,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
           const uint4 pp = make_uint4(pf[nt][u].x, pf[nt][u].y, pf[nt][u + 1].x, pf[nt][u + 1].y);
 #pragma unroll
           for (int e = 0; e < DV; ++e)
-            acc[nt][e] = mfma_16x16x32(make_uint4(va[e].x, va[e].y, vb[e].x, vb[e].y), pp, acc[nt][e]);
+            acc[nt][e] = mfma_16x16x32<F16>(make_uint4(va[e].x, va[e].y, vb[e].x, vb[e].y), pp, acc[nt][e]);
         }
       }
     } else {
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
         for (int nt = 0; nt < NQ; ++nt) {
           if (nt >= ntiles) break;
 #pragma unroll
-          for (int e = 0; e < DV; ++e) acc[nt][e] = mfma_16x16x16(vt[e], pf[nt][u], acc[nt][e]);
+          for (int e = 0; e < DV; ++e) acc[nt][e] = mfma_16x16x16<F16>(vt[e], pf[nt][u], acc[nt][e]);
         }
       }
     }
@@ -319,13 +319,13 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if constexpr (DV == 8) {
-          st16(o + 8 * i, make_uint4(pack_bf16x2(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
-                                     pack_bf16x2(acc[nt][2][i] * inv, acc[nt][3][i] * inv),
-                                     pack_bf16x2(acc[nt][4][i] * inv, acc[nt][5][i] * inv),
-                                     pack_bf16x2(acc[nt][6][i] * inv, acc[nt][7][i] * inv)));
+          st16(o + 8 * i, make_uint4(pack2<F16>(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
+                                     pack2<F16>(acc[nt][2][i] * inv, acc[nt][3][i] * inv),
+                                     pack2<F16>(acc[nt][4][i] * inv, acc[nt][5][i] * inv),
+                                     pack2<F16>(acc[nt][6][i] * inv, acc[nt][7][i] * inv)));
         } else {
-          st8(o + 4 * i, make_uint2(pack_bf16x2(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
-                                    pack_bf16x2(acc[nt][2][i] * inv, acc[nt][3][i] * inv)));
+          st8(o + 4 * i, make_uint2(pack2<F16>(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
+                                    pack2<F16>(acc[nt][2][i] * inv, acc[nt][3][i] * inv)));
         }
       }
     }
@@ -334,255 +334,11 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 
 
 // ---------------------------------------------------------------------------------------------
-// LDS-shared variant (head_dim 128): 8 waves x 48 rows = 384 rows per workgroup.  Each 32-key
-// K tile and V tile is fetched from HBM/L2 once per workgroup (one 16-byte piece per thread),
-// staged row-major in LDS with a 272-byte pitch (conflict-free for both read patterns), double
-// buffered with one barrier per tile; the waves read their MFMA operands from LDS.  The tile for
-// step t+1 is in flight in registers while step t computes.
-// ---------------------------------------------------------------------------------------------
-constexpr int kLdsPitch = 272;   // bytes per staged row (256 + 16 padding)
-
-// NQ = 16-row tiles per wave, NT = 16-key sub-tiles per staged tile (2 or 4).
-template <int NQ, int NT>
-__global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams p) {
-  constexpr int HD = 128, KS = 4, DV = 8, WAVES = 8;
-  constexpr int kLdsTile = 16 * NT;  // keys per staged tile
-  constexpr int LP = NT / 2;         // loader passes (512 threads fetch 32 rows per pass)
-  static_assert(NT == 2 || NT == 4, "staged tile of 32 or 64 keys");
-  __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kLdsTile * kLdsPitch];
-  __shared__ __attribute__((aligned(16))) uint8_t Vs[2][kLdsTile * kLdsPitch];
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int m16 = lane & 15, g = lane >> 4;
-  // Heaviest workgroups first: within a request the visible keys grow with the query position, so
-  // the linear index walks the query blocks backwards; consecutive indices are the KV heads of
-  // one block (they land on different XCDs, each of which then keeps one head's K/V in its L2).
-  const int h = blockIdx.x % p.Hkv;
-  const int rank = blockIdx.x / p.Hkv;
-  const int G = p.G;
-  const int BQ = ((16 * NQ) * p.g_magic) >> 16;  // query tokens per wave
-  const int SBQ = WAVES * BQ;             // query tokens per workgroup
-
-  if (rank == 0) {
-    const int tq = p.cu_q[p.R];
-    const int per_row = G * HD;
-    for (int64_t i = (int64_t)tid * 8; i < (int64_t)(p.T - tq) * per_row; i += 512 * 8) {
-      const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
-      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
-    }
-  }
-
-  const int sb = (int)(gridDim.x / p.Hkv) - 1 - rank;
-  int lo = 0, hi = p.R - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (p.cu_q[mid] / SBQ + mid <= sb) lo = mid; else hi = mid - 1;
-  }
-  const int r = lo;
-  const int q_begin = p.cu_q[r];
-  const int Lq = p.cu_q[r + 1] - q_begin;
-  const int q0_wg = (sb - (q_begin / SBQ + r)) * SBQ;
-  // Everything up to here is uniform over the workgroup: nobody is left behind at a barrier.
-  if (q0_wg >= Lq) return;
-  if (p.skip_single && Lq == 1) return;
-  const int Lk = p.lens[r];
-  const int shift = Lk - Lq;
-  const int last = Lk - 1;
-  const int kend_wg = min(Lk, shift + min(q0_wg + SBQ, Lq));  // keys some row of the workgroup sees
-
-  const int q0 = q0_wg + wave * BQ;
-  const int nq = max(0, min(BQ, Lq - q0));      // valid query tokens of this wave (may be 0)
-  const int kend = nq > 0 ? min(Lk, shift + q0 + nq) : 0;
-  const int ntiles = (nq * G + 15) >> 4;
-
-  uint4 qf[NQ][KS];
-  int qpos[NQ];
-#pragma unroll
-  for (int nt = 0; nt < NQ; ++nt) {
-    const int n = 16 * nt + m16;
-    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
-    const bool valid = qi < nq;
-    qpos[nt] = valid ? shift + q0 + qi : last;
-    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk)
-      qf[nt][kk] = valid ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
-  }
-
-  float m_run[NQ], l_run[NQ];
-  f32x4_t acc[NQ][DV];
-#pragma unroll
-  for (int nt = 0; nt < NQ; ++nt) {
-    m_run[nt] = -INFINITY;
-    l_run[nt] = 0.f;
-#pragma unroll
-    for (int e = 0; e < DV; ++e) acc[nt][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  }
-
-  if (kend_wg > 0) {
-    const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * 2;
-    const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * 2;
-    const int64_t chunk_bytes = p.kv_sc * 2;
-    const int tok_bytes = p.kv_st * 2;
-    // loader role of this thread: one 16-byte piece of one key row, for K and for V
-    const int lkey = tid >> 4, lpiece = tid & 15;
-    const int lds_off = lkey * kLdsPitch + lpiece * 16;
-    uint4 kreg[LP], vreg[LP];
-    auto gload = [&](int T) {
-#pragma unroll
-      for (int lp = 0; lp < LP; ++lp) {
-        const int tok = min(T + 32 * lp + lkey, last);
-        const int ci = (int)(((uint64_t)(uint32_t)tok * p.chunk_magic) >> 40);
-        const int pc = p.bt[(int64_t)r * p.bt_stride + ci];
-        const int64_t off = (int64_t)pc * chunk_bytes + (int64_t)(tok - ci * p.chunk) * tok_bytes + lpiece * 16;
-        kreg[lp] = ld16(kbase + off);
-        vreg[lp] = ld16(vbase + off);
-      }
-    };
-    auto lstore = [&](int buf) {
-#pragma unroll
-      for (int lp = 0; lp < LP; ++lp) {
-        *reinterpret_cast<uint4*>(&Ks[buf][lds_off + 32 * lp * kLdsPitch]) = kreg[lp];
-        *reinterpret_cast<uint4*>(&Vs[buf][lds_off + 32 * lp * kLdsPitch]) = vreg[lp];
-      }
-    };
-    const int full_until = shift + q0;
-    const float scale = p.scale_log2;
-
-    gload(0);
-    lstore(0);
-    __syncthreads();
-    int buf = 0;
-    for (int T = 0; T < kend_wg; T += kLdsTile, buf ^= 1) {
-      const bool more = T + kLdsTile < kend_wg;  // workgroup-uniform
-      if (more) gload(T + kLdsTile);
-      if (T < kend) {  // wave-uniform: this wave still has visible keys in the tile
-        const uint8_t* ks = Ks[buf];
-        const uint8_t* vs = Vs[buf];
-        // ---- S^T = K Q^T ---------------------------------------------------------------
-        f32x4_t s[NQ][NT];
-#pragma unroll
-        for (int u = 0; u < NT; ++u) {
-          uint4 kf[KS];
-#pragma unroll
-          for (int kk = 0; kk < KS; ++kk)
-            kf[kk] = lds_ld16(ks + (16 * u + m16) * kLdsPitch + (32 * kk + 8 * g) * 2);
-#pragma unroll
-          for (int nt = 0; nt < NQ; ++nt) {
-            if (nt >= ntiles) break;
-            f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int kk = 0; kk < KS; ++kk) sacc = mfma_16x16x32(kf[kk], qf[nt][kk], sacc);
-            s[nt][u] = sacc;
-          }
-        }
-        // ---- online softmax ---------------------------------------------------------------
-        const bool need_mask = T + kLdsTile - 1 > full_until;
-        uint2 pf[NQ][NT];
-#pragma unroll
-        for (int nt = 0; nt < NQ; ++nt) {
-          if (nt >= ntiles) break;
-          float tmax = -INFINITY;
-#pragma unroll
-          for (int u = 0; u < NT; ++u) {
-            if (need_mask) {
-              const int tok0 = T + 16 * u + 4 * g;
-#pragma unroll
-              for (int i = 0; i < 4; ++i)
-                if (tok0 + i > qpos[nt]) s[nt][u][i] = -INFINITY;
-            }
-            tmax = fmaxf(fmaxf(fmaxf(s[nt][u][0], s[nt][u][1]), fmaxf(s[nt][u][2], s[nt][u][3])), tmax);
-          }
-          tmax = fmaxf(tmax, xor16(tmax));
-          tmax = fmaxf(tmax, xor32(tmax));
-          const float m_raw = fmaxf(m_run[nt], tmax);
-          const float m_use = m_raw == -INFINITY ? 0.f : m_raw;
-          const float alpha = fast_exp2((m_run[nt] - m_use) * scale);
-          const float neg = -m_use * scale;
-          m_run[nt] = m_raw;
-          float psum = 0.f;
-#pragma unroll
-          for (int u = 0; u < NT; ++u) {
-            float pv[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              pv[i] = fast_exp2(__builtin_fmaf(s[nt][u][i], scale, neg));
-              psum += pv[i];
-            }
-            pf[nt][u] = make_uint2(pack_bf16x2(pv[0], pv[1]), pack_bf16x2(pv[2], pv[3]));
-          }
-          l_run[nt] = l_run[nt] * alpha + psum;
-          if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
-#pragma unroll
-            for (int e = 0; e < DV; ++e) {
-              acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
-            }
-          }
-        }
-        // ---- O^T += V^T P^T (k = 32: two 16-key sub-tiles per mfma) ------------------------
-#pragma unroll
-        for (int up = 0; up < NT; up += 2) {
-          uint4 va[4], vb[4];
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            va[j] = lds_ld16(vs + (16 * up + 4 * g + j) * kLdsPitch + 16 * m16);
-            vb[j] = lds_ld16(vs + (16 * up + 16 + 4 * g + j) * kLdsPitch + 16 * m16);
-          }
-          const uint32_t* a0 = reinterpret_cast<const uint32_t*>(&va[0]);
-          const uint32_t* a1 = reinterpret_cast<const uint32_t*>(&va[1]);
-          const uint32_t* a2 = reinterpret_cast<const uint32_t*>(&va[2]);
-          const uint32_t* a3 = reinterpret_cast<const uint32_t*>(&va[3]);
-          const uint32_t* b0 = reinterpret_cast<const uint32_t*>(&vb[0]);
-          const uint32_t* b1 = reinterpret_cast<const uint32_t*>(&vb[1]);
-          const uint32_t* b2 = reinterpret_cast<const uint32_t*>(&vb[2]);
-          const uint32_t* b3 = reinterpret_cast<const uint32_t*>(&vb[3]);
-#pragma unroll
-          for (int pr = 0; pr < 4; ++pr) {
-            const uint4 lo4 = make_uint4(low_halves(a1[pr], a0[pr]), low_halves(a3[pr], a2[pr]),
-                                         low_halves(b1[pr], b0[pr]), low_halves(b3[pr], b2[pr]));
-            const uint4 hi4 = make_uint4(high_halves(a1[pr], a0[pr]), high_halves(a3[pr], a2[pr]),
-                                         high_halves(b1[pr], b0[pr]), high_halves(b3[pr], b2[pr]));
-#pragma unroll
-            for (int nt = 0; nt < NQ; ++nt) {
-              if (nt >= ntiles) break;
-              const uint4 pp = make_uint4(pf[nt][up].x, pf[nt][up].y, pf[nt][up + 1].x, pf[nt][up + 1].y);
-              acc[nt][2 * pr] = mfma_16x16x32(lo4, pp, acc[nt][2 * pr]);
-              acc[nt][2 * pr + 1] = mfma_16x16x32(hi4, pp, acc[nt][2 * pr + 1]);
-            }
-          }
-        }
-      }
-      if (more) lstore(buf ^ 1);
-      __syncthreads();
-    }
-  }
-
-  // ---- epilogue (rows of a request without keys get zeros: l_tot == 0) -------------------
-#pragma unroll
-  for (int nt = 0; nt < NQ; ++nt) {
-    float l_tot = l_run[nt] + xor16(l_run[nt]);
-    l_tot += xor32(l_tot);
-    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-    const int n = 16 * nt + m16;
-    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
-    if (qi < nq) {
-      uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        st16(o + 8 * i, make_uint4(pack_bf16x2(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
-                                   pack_bf16x2(acc[nt][2][i] * inv, acc[nt][3][i] * inv),
-                                   pack_bf16x2(acc[nt][4][i] * inv, acc[nt][5][i] * inv),
-                                   pack_bf16x2(acc[nt][6][i] * inv, acc[nt][7][i] * inv)));
-    }
-  }
-}
-
-
-// ---------------------------------------------------------------------------------------------
-// Two-phase ("ping-pong") variant of the LDS kernel, head_dim 128.
+// Two-phase ("ping-pong") LDS-tiled kernel.
 //
+// A workgroup of 8 wavefronts takes 256 consecutive (query token, head-in-group) rows of one (request, KV head),
+// 32 rows per wavefront; each 64-key K tile and V tile is fetched from memory once per workgroup (16 bytes per
+// loader thread), staged row-major in LDS, and the wavefronts read their matrix operands from there.
 // The per-tile work of a wave is split into a matrix phase  { O^T += V^T P^T of the previous tile,
 // S^T = K Q^T of this tile }  and a vector phase  { online softmax of this tile, staging of the
 // next tiles into LDS }.  The 8 waves form two groups of four (waves w and w+4 share a SIMD);
@@ -591,10 +347,9 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_lds_kernel(PrefillParams
 // convert chain.  Because the groups read a staged tile one phase apart, the first group stages
 // one tile ahead of its own use and the second group two (see the table in the loop).
 //
-// Other differences to paged_prefill_lds_kernel: V fragments come out of LDS already transposed
-// (ds_read_b64_tr_b16, 288-byte V pitch), so there is no permute work; the softmax denominator is
-// accumulated by the matrix cores (an all-ones A fragment), and the cross-lane maximum uses the
-// lane-swap instructions instead of LDS permutes.
+// V fragments come out of LDS already transposed (ds_read_b64_tr_b16, 288-byte V pitch), so there is no
+// permute work; the softmax denominator is accumulated by the matrix cores (an all-ones A fragment), and
+// the cross-lane maximum uses the lane-swap instructions instead of LDS permutes.
 // ---------------------------------------------------------------------------------------------
 // bytes per staged K / V row.  head_dim 128: 288, measured conflict-free for the 16-row x 64-byte fragment
 // reads (272 is not), and 16 rows x 32 B of the transposing reads tile the banks twice; head_dim 64: 144
@@ -609,10 +364,11 @@ constexpr int kPPTile = 64;   // keys per staged tile
 // ordinary kernel carries no tile offsets).
 // HD = width of values and output, HDK = width of queries and keys: equal, or 192 / 128 for the decompressed
 // caches of multi-latent attention, whose value cache has its own strides.
-template <bool STAGGER, bool FP8, bool SPLIT = false, int HD = 128, int HDK = HD>
+template <bool STAGGER, bool FP8, bool SPLIT, int HD, int HDK, bool F16>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
   static_assert((HD == 128 && HDK == 128) || (HD == 64 && HDK == 64 && !FP8) || (HD == 128 && HDK == 192 && !FP8),
-                "head_dim 128, or 64 with a bf16 cache, or 192 / 128 with bf16 caches");
+                "head_dim 128, or 64 with a 16-bit cache, or 192 / 128 with 16-bit caches");
+  static_assert(!(FP8 && F16), "an fp8 cache is staged as bf16: bf16 queries only");
   constexpr bool MLA = HDK != HD;
   constexpr int KS = HDK / 32, DV = HD / 16, NQ = 2, NT = 4, WAVES = 8;
   constexpr int kKPitch = pp_pitch<HDK>(), kVPitch = pp_pitch<HD>();
@@ -806,8 +562,8 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       if (!FP8) return raw;
       const f32x2_t a = fp8x2_lo_to_f32(raw.x), b = fp8x2_hi_to_f32(raw.x);
       const f32x2_t c = fp8x2_lo_to_f32(raw.y), d = fp8x2_hi_to_f32(raw.y);
-      return make_uint4(pack_bf16x2(a.x * scale, a.y * scale), pack_bf16x2(b.x * scale, b.y * scale),
-                        pack_bf16x2(c.x * scale, c.y * scale), pack_bf16x2(d.x * scale, d.y * scale));
+      return make_uint4(pack2<F16>(a.x * scale, a.y * scale), pack2<F16>(b.x * scale, b.y * scale),
+                        pack2<F16>(c.x * scale, c.y * scale), pack2<F16>(d.x * scale, d.y * scale));
     };
     auto store_k = [&](int t) {
       if constexpr (MLA) {
@@ -827,7 +583,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     };
 
     const float scale = p.scale_log2;
-    const uint4 ones = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+    const uint4 ones = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
     f32x4_t s[NQ][NT];
     uint2 pf[NQ][NT];
     // fixed per-lane offsets of the fragment reads
@@ -845,12 +601,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       for (int kk = 0; kk < KS; ++kk) kf[kk] = *reinterpret_cast<const uint4*>(ks + 64 * kk);
     };
     auto sc_mma = [&](int u, const uint4 (&kf)[KS]) {
-      s[0][u] = mfma_16x16x32(kf[0], qf[0][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
-      s[1][u] = mfma_16x16x32(kf[0], qf[1][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
+      s[0][u] = mfma_16x16x32<F16>(kf[0], qf[0][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
+      s[1][u] = mfma_16x16x32<F16>(kf[0], qf[1][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
       for (int kk = 1; kk < KS; ++kk) {
-        s[0][u] = mfma_16x16x32(kf[kk], qf[0][kk], s[0][u]);
-        s[1][u] = mfma_16x16x32(kf[kk], qf[1][kk], s[1][u]);
+        s[0][u] = mfma_16x16x32<F16>(kf[kk], qf[0][kk], s[0][u]);
+        s[1][u] = mfma_16x16x32<F16>(kf[kk], qf[1][kk], s[1][u]);
       }
     };
     // 192-wide keys: a sub-tile's product in two halves of three fragments (half the fragment registers)
@@ -863,8 +619,8 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
         const int kk = 3 * half + j;
-        s[0][u] = mfma_16x16x32(kf[j], qf[0][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[0][u]);
-        s[1][u] = mfma_16x16x32(kf[j], qf[1][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[1][u]);
+        s[0][u] = mfma_16x16x32<F16>(kf[j], qf[0][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[0][u]);
+        s[1][u] = mfma_16x16x32<F16>(kf[j], qf[1][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[1][u]);
       }
     };
     // O^T += V^T P^T: group grp = (32-key step grp / 2, output columns 64 * (grp % 2) ..+63):
@@ -884,12 +640,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const uint4 a = make_uint4(af[e][0].x, af[e][0].y, af[e][1].x, af[e][1].y);
-        acc[0][e0 + e] = mfma_16x16x32(a, pp0, acc[0][e0 + e]);
-        acc[1][e0 + e] = mfma_16x16x32(a, pp1, acc[1][e0 + e]);
+        acc[0][e0 + e] = mfma_16x16x32<F16>(a, pp0, acc[0][e0 + e]);
+        acc[1][e0 + e] = mfma_16x16x32<F16>(a, pp1, acc[1][e0 + e]);
       }
       if (grp % NH == NH - 1) {  // once per 32-key step
-        accl[0] = mfma_16x16x32(ones, pp0, accl[0]);
-        accl[1] = mfma_16x16x32(ones, pp1, accl[1]);
+        accl[0] = mfma_16x16x32<F16>(ones, pp0, accl[0]);
+        accl[1] = mfma_16x16x32<F16>(ones, pp1, accl[1]);
       }
     };
 #define MI_SB() __builtin_amdgcn_sched_barrier(0)
@@ -1011,7 +767,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
           const float p1 = fast_exp2(__builtin_fmaf(s[nt][u][1], scale, neg));
           const float p2 = fast_exp2(__builtin_fmaf(s[nt][u][2], scale, neg));
           const float p3 = fast_exp2(__builtin_fmaf(s[nt][u][3], scale, neg));
-          pf[nt][u] = make_uint2(pack_bf16x2(p0, p1), pack_bf16x2(p2, p3));
+          pf[nt][u] = make_uint2(pack2<F16>(p0, p1), pack2<F16>(p2, p3));
         }
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
@@ -1085,8 +841,8 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * g;
 #pragma unroll
         for (int e = 0; e < DV; ++e)
-          st8(o + 16 * e, make_uint2(pack_bf16x2(acc[nt][e][0] * inv, acc[nt][e][1] * inv),
-                                     pack_bf16x2(acc[nt][e][2] * inv, acc[nt][e][3] * inv)));
+          st8(o + 16 * e, make_uint2(pack2<F16>(acc[nt][e][0] * inv, acc[nt][e][1] * inv),
+                                     pack2<F16>(acc[nt][e][2] * inv, acc[nt][e][3] * inv)));
       } else {  // a range without visible keys (none for short requests) leaves zeros and -inf
         const int64_t prow = ((int64_t)split * p.T + (q_begin + q0 + qi)) * p.Hq + (h * G + u);
         float* o = p.split_o + prow * HD + 4 * g;
@@ -1102,6 +858,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 
 // Rows whose keys were split over several workgroups: o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max).
 // Grid (T, Hq), head_dim threads = the output values of one (row, head).
+template <bool F16>
 __global__ __launch_bounds__(128) void prefill_split_merge_kernel(PrefillParams p, int n_split, int head_dim) {
   const int row = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   if (row >= p.cu_q[p.R]) return;  // padding rows: zeroed by the tile kernel
@@ -1133,7 +890,7 @@ __global__ __launch_bounds__(128) void prefill_split_merge_kernel(PrefillParams 
       }
     }
   }
-  p.out[(int64_t)row * p.o_st + (int64_t)head * p.o_sh + d] = f32_to_bf16(den > 0.f ? num / den : 0.f);
+  p.out[(int64_t)row * p.o_st + (int64_t)head * p.o_sh + d] = f32_to_16<F16>(den > 0.f ? num / den : 0.f);
 }
 
 }  // namespace mi
@@ -1158,20 +915,36 @@ static int prefill_kv_splits(int T, int Hq, int Hkv, int head_dim, int max_kv_le
   return s < 2 ? 1 : (int)s;
 }
 
+// key ranges for these sizes under the caller's knob (1 = automatic, -1 = never, n > 1 = forced)
+static int kv_split_count(const MiTuning& tune, int T, int Hq, int Hkv, int head_dim, int max_kv_len) {
+  if (tune.prefill_kv_split < 0) return 1;
+  return tune.prefill_kv_split > 1 ? tune.prefill_kv_split : prefill_kv_splits(T, Hq, Hkv, head_dim, max_kv_len);
+}
+
 extern "C" int64_t mi_prefill_workspace_bytes(int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
                                               int32_t head_dim, int32_t max_kv_len,
-                                              int32_t split_tokens) {
+                                              int32_t split_tokens, const MiTuning* tuning) {
+  MiTuning tune;
+  if (mi_resolve_tuning(tuning, &tune, "mi_prefill_workspace_bytes") != MI_OK) return -1;
   // The one-row (decode) requests of a mixed batch are streamed by the decode kernels, whose partials
   // live here; behind them the partials of the tile kernel when it splits the keys.
-  int64_t bytes = mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens);
+  int64_t bytes = mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens, tuning);
   bytes = (bytes + 255) & ~(int64_t)255;
   if (T > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0) {
-    const int knob = mi_tuning().prefill_kv_split;  // (a forced count is honoured here too)
-    const int s = knob > 1 ? knob : knob == 1 ? prefill_kv_splits(T, Hq, Hkv, head_dim, max_kv_len) : 1;
+    const int s = kv_split_count(tune, T, Hq, Hkv, head_dim, max_kv_len);  // (a forced count is honoured here too)
     if (s > 1) bytes += (int64_t)s * T * Hq * (head_dim + 1) * (int64_t)sizeof(float);
   }
   return bytes;
 }
+
+// The two-phase tile kernel for one combination of (wave groups staggered?, fp8 cache?, keys split?, widths, type).
+#define MI_PP_LAUNCH(FP8_, HD_, HDK_, F16_)                                                                         \
+  do {                                                                                                              \
+    if (n_split > 1 && stagger) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, FP8_, true, HD_, HDK_, F16_>), lgrid, dim3(512), 0, st, p);   \
+    else if (n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, FP8_, true, HD_, HDK_, F16_>), lgrid, dim3(512), 0, st, p);      \
+    else if (stagger) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, FP8_, false, HD_, HDK_, F16_>), lgrid, dim3(512), 0, st, p);          \
+    else hipLaunchKernelGGL((paged_prefill_pp_kernel<false, FP8_, false, HD_, HDK_, F16_>), lgrid, dim3(512), 0, st, p);                      \
+  } while (0)
 
 static int launch_paged_prefill(
     const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
@@ -1180,9 +953,16 @@ static int launch_paged_prefill(
     const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head,
     void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
     int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens, float softmax_scale,
-    int32_t kv_dtype, const float* k_scales, const float* v_scales, void* stream) {
+    int32_t kv_dtype, const float* k_scales, const float* v_scales, int32_t dtype, const MiTuning* tuning,
+    void* stream) {
   const bool fp8 = kv_dtype == MI_KV_FP8_E4M3;
   if (T == 0 || R == 0) return MI_OK;
+  MiTuning tune;
+  const int rc_t = mi_resolve_tuning(tuning, &tune, "mi_paged_prefill_attention");
+  if (rc_t != MI_OK) return rc_t;
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  const bool f16 = dtype == MI_DTYPE_FP16;
   if (!q || !k_cache || !v_cache || !block_table || !cu_seqlens_q || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention: null pointer argument");
   if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
@@ -1200,15 +980,22 @@ static int launch_paged_prefill(
     return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention: strides must keep rows 16-byte aligned");
   if (kv_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: one chunk must span less than 2 GiB");
-  if (kv_dtype != MI_KV_BF16 && !fp8)
+  if (kv_dtype != MI_KV_16BIT && !fp8)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: unknown kv_dtype");
   if (fp8 && (!k_scales || !v_scales))
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_fp8: both scale arrays are required");
-  if (fp8 && (head_dim != 128 || chunk_tokens % 64 || mi_tuning().prefill_pingpong == 0 ||
-              mi_tuning().prefill_lds_row_tiles == 0))
+  // the two-phase tile kernel stages 64-key tiles that must not straddle chunks; other chunk sizes (and the
+  // knob) select the register-only kernel
+  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0;
+  if (fp8 && (head_dim != 128 || !two_phase || f16))
     return mi_fail(MI_ERR_UNSUPPORTED,
-                   "mi_paged_prefill_attention_fp8: fp8 KV needs head_dim 128, a chunk size that is a multiple "
-                   "of 64 and the two-phase tile kernel");
+                   "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 128, a chunk size that is a "
+                   "multiple of 64 and the two-phase tile kernel");
+  if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
+  // Everything is checked before the first launch: the decode part of a mixed batch must not be rejected after
+  // the tile kernel has written its rows.
+  if (workspace && (int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: batch too large for the in-LDS prefix sum (7680 requests)");
 
   PrefillParams p;
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;
@@ -1228,27 +1015,21 @@ static int launch_paged_prefill(
   p.split_o = nullptr; p.split_lse = nullptr;
 
   hipStream_t st = (hipStream_t)stream;
-  if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
-  const int lds_tiles = mi_tuning().prefill_lds_row_tiles;  // 0 = register-only kernel
-  const bool pp64 = head_dim == 64 && lds_tiles > 0 && chunk_tokens % 64 == 0 && mi_tuning().prefill_pingpong != 0 && !fp8;
-  if ((head_dim == 128 && lds_tiles > 0) || pp64) {
-    const int rows = 8 * 16 * ((lds_tiles == 2 || (mi_tuning().prefill_pingpong && chunk_tokens % 64 == 0)) ? 2 : 3);
-    const int sbq_lds = 8 * ((rows / 8) / G);  // 8 wavefronts x whole tokens in a wavefront's rows
+  if (two_phase) {
+    const int sbq_lds = 8 * (32 / G);  // 8 wavefronts x whole tokens in a wavefront's 32 rows
     dim3 lgrid(((T + sbq_lds - 1) / sbq_lds + R) * Hkv);
-    const bool wide = mi_tuning().prefill_tile_subtiles == 4;  // 64-key staged tiles
     hipEvent_t ev_a, ev_b;
     const bool timed = mi_profile_next(&ev_a, &ev_b);
     if (timed) (void)hipEventRecord(ev_a, st);
-    const int pp = (chunk_tokens % 64 == 0) ? mi_tuning().prefill_pingpong : 0;  // staged tiles must not straddle chunks
-    // key ranges per request (two-phase kernel with a workspace only): partials behind the decode part's scratch
+    const bool stagger = tune.prefill_two_phase == 1;
+    // key ranges per request (with a workspace only): partials behind the decode part's scratch
     int n_split = 1;
-    if (pp != 0 && workspace && mi_tuning().prefill_kv_split != 0) {
-      n_split = mi_tuning().prefill_kv_split > 1 ? mi_tuning().prefill_kv_split
-                                                 : prefill_kv_splits(T, Hq, Hkv, head_dim, max_kv_len);
-      const int64_t dec_bytes = (mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens) + 255) &
+    if (workspace) {
+      n_split = kv_split_count(tune, T, Hq, Hkv, head_dim, max_kv_len);
+      const int64_t dec_bytes = (mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, 16, max_kv_len, split_tokens, tuning) + 255) &
                                 ~(int64_t)255;
       const int64_t sp_bytes = (int64_t)n_split * T * Hq * (head_dim + 1) * (int64_t)sizeof(float);
-      if (n_split > 1 && workspace_bytes < dec_bytes + sp_bytes) n_split = 1;  // (a caller-sized workspace of the older layout)
+      if (n_split > 1 && workspace_bytes < dec_bytes + sp_bytes) n_split = 1;  // (a caller-sized workspace without room for them)
       if (n_split > 1) {
         p.split_o = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(workspace) + dec_bytes);
         p.split_lse = p.split_o + (int64_t)n_split * T * Hq * head_dim;
@@ -1256,54 +1037,41 @@ static int launch_paged_prefill(
         workspace_bytes = dec_bytes;
       }
     }
-    if (pp64 && n_split > 1 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, true, 64>), lgrid, dim3(512), 0, st, p);
-    else if (pp64 && n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, true, 64>), lgrid, dim3(512), 0, st, p);
-    else if (pp64 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, false, 64>), lgrid, dim3(512), 0, st, p);
-    else if (pp64) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, false, 64>), lgrid, dim3(512), 0, st, p);
-    else if (n_split > 1 && fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true, true>), lgrid, dim3(512), 0, st, p);
-    else if (n_split > 1 && fp8) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, true, true>), lgrid, dim3(512), 0, st, p);
-    else if (n_split > 1 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, true>), lgrid, dim3(512), 0, st, p);
-    else if (n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, true>), lgrid, dim3(512), 0, st, p);
-    else if (fp8 && pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, true>), lgrid, dim3(512), 0, st, p);
-    else if (fp8) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, true>), lgrid, dim3(512), 0, st, p);
-    else if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false>), lgrid, dim3(512), 0, st, p);
-    else if (pp == 2) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false>), lgrid, dim3(512), 0, st, p);
-    else if (lds_tiles == 2 && wide) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 4>), lgrid, dim3(512), 0, st, p);
-    else if (lds_tiles == 2) hipLaunchKernelGGL((paged_prefill_lds_kernel<2, 2>), lgrid, dim3(512), 0, st, p);
-    else hipLaunchKernelGGL((paged_prefill_lds_kernel<3, 2>), lgrid, dim3(512), 0, st, p);  // (48 rows: 32-key tiles only)
+    if (fp8) MI_PP_LAUNCH(true, 128, 128, false);
+    else if (head_dim == 128 && f16) MI_PP_LAUNCH(false, 128, 128, true);
+    else if (head_dim == 128) MI_PP_LAUNCH(false, 128, 128, false);
+    else if (f16) MI_PP_LAUNCH(false, 64, 64, true);
+    else MI_PP_LAUNCH(false, 64, 64, false);
     if (timed) (void)hipEventRecord(ev_b, st);
-    if (n_split > 1) hipLaunchKernelGGL(prefill_split_merge_kernel, dim3(T, Hq), dim3(head_dim), 0, st, p, n_split, head_dim);
-    int rc0 = mi_check_launch("mi_paged_prefill_attention");
-    if (rc0 != MI_OK || !p.skip_single) return rc0;
-    return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
-                               kv_stride_head, block_table, bt_stride, kv_lens, cu_seqlens_q, out, o_stride_tok,
-                               o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
-                               split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, stream);
-  }
-  const int nq = mi_tuning().prefill_row_tiles == 4 ? 4 : 2;
-  const int sbq = (16 / nq) * ((16 * nq) / G);  // query tokens per workgroup: whole tokens in each wavefront's rows
-  dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * (16 / nq));
-  // register-only kernel (head_dim 64, or LDS variant switched off): 16 or 32 keys per iteration
-  const int nt = mi_tuning().prefill_tile_subtiles == 1 ? 1 : 2;
-#define MI_LAUNCH_PREFILL(HD_, NT_)                                                                        \
-  do {                                                                                                     \
-    if (nq == 4) hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, NT_, 4>), grid, block, 0, st, p);      \
-    else hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, NT_, 2>), grid, block, 0, st, p);              \
-  } while (0)
-  if (head_dim == 128) {
-    if (nt == 1) MI_LAUNCH_PREFILL(128, 1);
-    else MI_LAUNCH_PREFILL(128, 2);
+    if (n_split > 1) {
+      if (f16) hipLaunchKernelGGL(prefill_split_merge_kernel<true>, dim3(T, Hq), dim3(head_dim), 0, st, p, n_split, head_dim);
+      else hipLaunchKernelGGL(prefill_split_merge_kernel<false>, dim3(T, Hq), dim3(head_dim), 0, st, p, n_split, head_dim);
+    }
   } else {
-    if (nt == 1) MI_LAUNCH_PREFILL(64, 1);
-    else MI_LAUNCH_PREFILL(64, 2);
-  }
+    // register-only kernel: any chunk size that is a multiple of 16; 16 or 32 keys per iteration
+    const int nq = tune.prefill_row_tiles == 4 ? 4 : 2;
+    const int sbq = (16 / nq) * ((16 * nq) / G);  // query tokens per workgroup: whole tokens in each wavefront's rows
+    dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * (16 / nq));
+    const int nt = tune.prefill_tile_subtiles == 1 ? 1 : 2;
+#define MI_LAUNCH_PREFILL(HD_, F16_)                                                                           \
+  do {                                                                                                         \
+    if (nq == 4 && nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, 1, 4, F16_>), grid, block, 0, st, p);  \
+    else if (nq == 4) hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, 2, 4, F16_>), grid, block, 0, st, p);        \
+    else if (nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, 1, 2, F16_>), grid, block, 0, st, p);        \
+    else hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, 2, 2, F16_>), grid, block, 0, st, p);                     \
+  } while (0)
+    if (head_dim == 128 && f16) MI_LAUNCH_PREFILL(128, true);
+    else if (head_dim == 128) MI_LAUNCH_PREFILL(128, false);
+    else if (f16) MI_LAUNCH_PREFILL(64, true);
+    else MI_LAUNCH_PREFILL(64, false);
 #undef MI_LAUNCH_PREFILL
-  int rc = mi_check_launch("mi_paged_prefill_attention");
+  }
+  const int rc = mi_check_launch("mi_paged_prefill_attention");
   if (rc != MI_OK || !p.skip_single) return rc;
   return launch_paged_decode(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
                              kv_stride_head, block_table, bt_stride, kv_lens, cu_seqlens_q, out, o_stride_tok,
                              o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
-                             split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
+                             split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, dtype, tune, stream);
 }
 
 extern "C" int mi_paged_prefill_attention(
@@ -1313,11 +1081,12 @@ extern "C" int mi_paged_prefill_attention(
     const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head,
     void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv,
     int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
-    float softmax_scale, void* stream) {
+    float softmax_scale, int32_t dtype, const MiTuning* tuning, void* stream) {
   return launch_paged_prefill(q, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk, kv_stride_tok,
                               kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out, o_stride_tok,
                               o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim, chunk_tokens,
-                              max_kv_len, split_tokens, softmax_scale, MI_KV_BF16, nullptr, nullptr, stream);
+                              max_kv_len, split_tokens, softmax_scale, MI_KV_16BIT, nullptr, nullptr, dtype, tuning,
+                              stream);
 }
 
 extern "C" int mi_paged_prefill_attention_fp8(
@@ -1327,12 +1096,12 @@ extern "C" int mi_paged_prefill_attention_fp8(
     const int32_t* cu_seqlens_q, const int32_t* kv_lens, void* out, int64_t o_stride_tok,
     int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq,
     int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
-    float softmax_scale, void* stream) {
+    float softmax_scale, const MiTuning* tuning, void* stream) {
   return launch_paged_prefill(q, q_stride_tok, q_stride_head, k_cache_fp8, v_cache_fp8, kv_stride_chunk,
                               kv_stride_tok, kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out,
                               o_stride_tok, o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim,
                               chunk_tokens, max_kv_len, split_tokens, softmax_scale, MI_KV_FP8_E4M3, k_scales, v_scales,
-                              stream);
+                              MI_DTYPE_BF16, tuning, stream);
 }
 
 extern "C" int mi_paged_prefill_attention_mla(
@@ -1341,8 +1110,15 @@ extern "C" int mi_paged_prefill_attention_mla(
     int64_t v_stride_head, const int32_t* block_table, int64_t bt_stride, const int32_t* cu_seqlens_q,
     const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
     int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim_k, int32_t head_dim_v,
-    int32_t chunk_tokens, int32_t max_kv_len, float softmax_scale, void* stream) {
+    int32_t chunk_tokens, int32_t max_kv_len, float softmax_scale, int32_t dtype, const MiTuning* tuning,
+    void* stream) {
   if (T == 0 || R == 0) return MI_OK;
+  MiTuning tune;
+  const int rc_t = mi_resolve_tuning(tuning, &tune, "mi_paged_prefill_attention_mla");
+  if (rc_t != MI_OK) return rc_t;
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  const bool f16 = dtype == MI_DTYPE_FP16;
   if (!q || !k_cache || !v_cache || !block_table || !cu_seqlens_q || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_mla: null pointer argument");
   if (workspace && ((uintptr_t)workspace & 255))
@@ -1381,18 +1157,19 @@ extern "C" int mi_paged_prefill_attention_mla(
   p.k_scale = nullptr; p.v_scale = nullptr;
   p.split_o = nullptr; p.split_lse = nullptr;
   const int sbq = 8 * (32 / G);  // query tokens per workgroup (8 wavefronts x 32 rows)
-  const int pp = (chunk_tokens % 64 == 0 && mi_tuning().prefill_lds_row_tiles > 0) ? mi_tuning().prefill_pingpong : 0;
+  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0;  // staged tiles must not straddle chunks
+  hipStream_t st = (hipStream_t)stream;
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
-  if (timed) (void)hipEventRecord(ev_a, (hipStream_t)stream);
+  if (timed) (void)hipEventRecord(ev_a, st);
   int n_split = 1;
-  if (pp != 0) {  // two-phase tile kernel (staged tiles must not straddle chunks)
+  if (two_phase) {
     dim3 lgrid(((T + sbq - 1) / sbq + R) * Hkv);
+    const bool stagger = tune.prefill_two_phase == 1;
     // few query rows over long contexts: key ranges per request, partials in the workspace (which holds
     // nothing else here: one-row requests stay in the tile kernel)
-    if (workspace && mi_tuning().prefill_kv_split != 0) {
-      n_split = mi_tuning().prefill_kv_split > 1 ? mi_tuning().prefill_kv_split
-                                                 : prefill_kv_splits(T, Hq, Hkv, head_dim_v, max_kv_len);
+    if (workspace) {
+      n_split = kv_split_count(tune, T, Hq, Hkv, head_dim_v, max_kv_len);
       const int64_t sp_bytes = (int64_t)n_split * T * Hq * (head_dim_v + 1) * (int64_t)sizeof(float);
       if (n_split > 1 && workspace_bytes < sp_bytes) n_split = 1;
       if (n_split > 1) {
@@ -1401,17 +1178,18 @@ extern "C" int mi_paged_prefill_attention_mla(
         lgrid.y = n_split;
       }
     }
-    hipStream_t st = (hipStream_t)stream;
-    if (n_split > 1 && pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, true, 128, 192>), lgrid, dim3(512), 0, st, p);
-    else if (n_split > 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, true, 128, 192>), lgrid, dim3(512), 0, st, p);
-    else if (pp == 1) hipLaunchKernelGGL((paged_prefill_pp_kernel<true, false, false, 128, 192>), lgrid, dim3(512), 0, st, p);
-    else hipLaunchKernelGGL((paged_prefill_pp_kernel<false, false, false, 128, 192>), lgrid, dim3(512), 0, st, p);
+    if (f16) MI_PP_LAUNCH(false, 128, 192, true);
+    else MI_PP_LAUNCH(false, 128, 192, false);
   } else {
     dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * 8);
-    hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2>), grid, block, 0, (hipStream_t)stream, p);
+    if (f16) hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2, true>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2, false>), grid, block, 0, st, p);
   }
-  if (timed) (void)hipEventRecord(ev_b, (hipStream_t)stream);
-  if (n_split > 1)
-    hipLaunchKernelGGL(prefill_split_merge_kernel, dim3(T, Hq), dim3(head_dim_v), 0, (hipStream_t)stream, p, n_split, head_dim_v);
+  if (timed) (void)hipEventRecord(ev_b, st);
+  if (n_split > 1) {
+    if (f16) hipLaunchKernelGGL(prefill_split_merge_kernel<true>, dim3(T, Hq), dim3(head_dim_v), 0, st, p, n_split, head_dim_v);
+    else hipLaunchKernelGGL(prefill_split_merge_kernel<false>, dim3(T, Hq), dim3(head_dim_v), 0, st, p, n_split, head_dim_v);
+  }
   return mi_check_launch("mi_paged_prefill_attention_mla");
 }
+#undef MI_PP_LAUNCH

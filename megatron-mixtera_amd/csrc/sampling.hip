@@ -69,9 +69,9 @@ static __device__ __forceinline__ uint64_t wave_scan_incl_u64(uint64_t v, int la
   return v;
 }
 
-// One row of logits.  VEC = elements per 16-byte load (4 fp32, 8 bf16) when the row is 16-byte
-// aligned, 1 otherwise.
-template <bool BF16, int VEC>
+// One row of logits.  DT = element type (0 fp32, 1 bf16, 2 fp16); VEC = elements per 16-byte load (4 fp32,
+// 8 of a 16-bit type) when the row is 16-byte aligned, 1 otherwise.
+template <int DT, int VEC>
 struct RowReader {
   const uint8_t* row; int V; float inv_t; bool scale;
   // the value the filters see: logit * (1 / temperature), rounded to the logits' dtype as the
@@ -79,22 +79,22 @@ struct RowReader {
   __device__ __forceinline__ float finish(float x) const {
     if (scale) {
       x *= inv_t;
-      if (BF16) x = bf16_to_f32(f32_to_bf16(x));
+      if (DT != 0) x = to_f32<DT == 2>(f32_to_16<DT == 2>(x));
     }
     return x + 0.0f;
   }
   __device__ __forceinline__ float at(int i) const {
-    return finish(BF16 ? bf16_to_f32(reinterpret_cast<const uint16_t*>(row)[i]) : reinterpret_cast<const float*>(row)[i]);
+    return finish(DT != 0 ? to_f32<DT == 2>(reinterpret_cast<const uint16_t*>(row)[i]) : reinterpret_cast<const float*>(row)[i]);
   }
   // elements i0 .. i0+VEC-1 (i0 a multiple of VEC), all inside the row
   __device__ __forceinline__ void load_full(int i0, float (&x)[VEC]) const {
     if (VEC > 1) {
-      const uint4 w = ld16(row + (int64_t)i0 * (BF16 ? 2 : 4));
+      const uint4 w = ld16(row + (int64_t)i0 * (DT != 0 ? 2 : 4));
       const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         float v;
-        if (BF16) v = (j & 1) ? bf16hi_to_f32(u[(j >> 1) & 3]) : bf16lo_to_f32(u[(j >> 1) & 3]);
+        if (DT != 0) v = (j & 1) ? hi_to_f32<DT == 2>(u[(j >> 1) & 3]) : lo_to_f32<DT == 2>(u[(j >> 1) & 3]);
         else v = __uint_as_float(u[j & 3]);
         x[j] = finish(v);
       }
@@ -105,12 +105,12 @@ struct RowReader {
   // the same with slots at or past V set to 0
   __device__ __forceinline__ void load(int i0, float (&x)[VEC]) const {
     if (VEC > 1 && i0 + VEC <= V) {
-      const uint4 w = ld16(row + (int64_t)i0 * (BF16 ? 2 : 4));
+      const uint4 w = ld16(row + (int64_t)i0 * (DT != 0 ? 2 : 4));
       const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
       for (int j = 0; j < VEC; ++j) {
         float v;
-        if (BF16) v = (j & 1) ? bf16hi_to_f32(u[(j >> 1) & 3]) : bf16lo_to_f32(u[(j >> 1) & 3]);
+        if (DT != 0) v = (j & 1) ? hi_to_f32<DT == 2>(u[(j >> 1) & 3]) : lo_to_f32<DT == 2>(u[(j >> 1) & 3]);
         else v = __uint_as_float(u[j & 3]);
         x[j] = finish(v);
       }
@@ -126,8 +126,8 @@ struct RowReader {
 // makes the same number of calls, so f may use wavefront-wide operations.  begin % VEC == 0.
 // Whole blocks of U strides run without any bounds test (the flag is the constant true there);
 // only the rest of the range pays for guards.
-template <int U, bool BF16, int VEC, typename F>
-static __device__ __forceinline__ void sweep(const RowReader<BF16, VEC>& rd, int begin, int end, int t, int nthreads, F f) {
+template <int U, int DT, int VEC, typename F>
+static __device__ __forceinline__ void sweep(const RowReader<DT, VEC>& rd, int begin, int end, int t, int nthreads, F f) {
   const int stride = nthreads * VEC;
   const int row_end = rd.V - (rd.V % VEC);  // whole 16-byte groups of the row end here
   int base = begin;
@@ -220,7 +220,7 @@ static __device__ void find_crossing(const uint64_t* hist, uint64_t above, uint6
 
 constexpr int kMemberCap = 4096;  // members of the chosen value bin that fit the LDS list
 
-template <bool BF16, int VEC>
+template <int DT, int VEC>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) {
   __shared__ uint64_t hist[256];
   __shared__ uint64_t res[2];
@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int V = p.V;
   const bool greedy = p.top_k == 1;
-  const RowReader<BF16, VEC> rd{reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)r * p.stride * (BF16 ? 2 : 4), V,
+  const RowReader<DT, VEC> rd{reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)r * p.stride * (DT != 0 ? 2 : 4), V,
                                 p.inv_temperature, !greedy && p.inv_temperature != 1.0f};
   constexpr int U = 8;  // loads in flight per thread
 
@@ -484,12 +484,12 @@ constexpr int kLogProbThreads = 512;
 
 // out[t] = log_softmax(logits[t])[token_ids[t]] in fp32: one pass over the row with a running
 // (maximum, sum of exp(x - maximum)) pair per thread, merged over the workgroup.  One workgroup per row.
-template <bool BF16, int VEC>
+template <int DT, int VEC>
 __global__ __launch_bounds__(kLogProbThreads) void selected_log_probs_kernel(LogProbParams p) {
   __shared__ float red_m[kLogProbThreads / 64], red_s[kLogProbThreads / 64];
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  RowReader<BF16, VEC> rd;
-  rd.row = reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)t * p.stride * (BF16 ? 2 : 4);
+  RowReader<DT, VEC> rd;
+  rd.row = reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)t * p.stride * (DT != 0 ? 2 : 4);
   rd.V = p.V; rd.inv_t = 1.f; rd.scale = false;
   constexpr float kLog2e = 1.4426950408889634f;
   // a finite start keeps exp(-inf - m) = 0 for masked (-inf) logits
@@ -506,11 +506,11 @@ __global__ __launch_bounds__(kLogProbThreads) void selected_log_probs_kernel(Log
       float x[U * VEC];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const uint4 w = ld16(rd.row + (int64_t)(base + u * stride + tid * VEC) * (BF16 ? 2 : 4));
+        const uint4 w = ld16(rd.row + (int64_t)(base + u * stride + tid * VEC) * (DT != 0 ? 2 : 4));
         const uint32_t q[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int j = 0; j < VEC; ++j)
-          x[u * VEC + j] = BF16 ? ((j & 1) ? bf16hi_to_f32(q[(j >> 1) & 3]) : bf16lo_to_f32(q[(j >> 1) & 3]))
+          x[u * VEC + j] = DT != 0 ? ((j & 1) ? hi_to_f32<DT == 2>(q[(j >> 1) & 3]) : lo_to_f32<DT == 2>(q[(j >> 1) & 3]))
                                 : __uint_as_float(q[j & 3]);
       }
       float bm = x[0];
@@ -597,8 +597,8 @@ extern "C" int mi_sample_from_logits(const void* logits, int64_t stride_row, int
   if (!logits || !samples) return mi_fail(MI_ERR_NULL, "mi_sample_from_logits: null pointer argument");
   if (R < 0 || vocab <= 0 || stride_row < vocab)
     return mi_fail(MI_ERR_SHAPE, "mi_sample_from_logits: need R >= 0, vocab > 0 and a row stride of at least vocab");
-  if (logits_dtype != 0 && logits_dtype != 1)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_sample_from_logits: logits must be fp32 (0) or bf16 (1)");
+  if (logits_dtype < 0 || logits_dtype > 2)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_sample_from_logits: logits must be fp32 (0), bf16 (1) or fp16 (2)");
   if (top_k < 0 || !(top_p >= 0.f && top_p <= 1.f))
     return mi_fail(MI_ERR_SHAPE, "mi_sample_from_logits: need top_k >= 0 and top_p in [0, 1]");
   if (top_k > 0 && top_p > 0.f)
@@ -619,16 +619,19 @@ extern "C" int mi_sample_from_logits(const void* logits, int64_t stride_row, int
   p.uniform = uniform; p.vocab_clamp = vocab_clamp; p.samples = samples; p.cut_out = cut_values;
   p.kv_off = request_kv_length_offsets; p.q_len = request_query_lengths; p.out_len = request_output_lengths;
   p.termination_id = termination_id; p.active_mask = active_request_mask;
-  const int esize = logits_dtype == 1 ? 2 : 4;
+  const int esize = logits_dtype != 0 ? 2 : 4;
   const bool wide = !(((uintptr_t)logits | (uintptr_t)(stride_row * esize)) & 15);  // 16-byte loads
   const dim3 grid(R), block(kSampleThreads);
   hipStream_t st = (hipStream_t)stream;
-  if (logits_dtype == 1) {
-    if (wide) hipLaunchKernelGGL((sample_kernel<true, 8>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((sample_kernel<true, 1>), grid, block, 0, st, p);
+  if (logits_dtype == 2) {
+    if (wide) hipLaunchKernelGGL((sample_kernel<2, 8>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((sample_kernel<2, 1>), grid, block, 0, st, p);
+  } else if (logits_dtype == 1) {
+    if (wide) hipLaunchKernelGGL((sample_kernel<1, 8>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((sample_kernel<1, 1>), grid, block, 0, st, p);
   } else {
-    if (wide) hipLaunchKernelGGL((sample_kernel<false, 4>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((sample_kernel<false, 1>), grid, block, 0, st, p);
+    if (wide) hipLaunchKernelGGL((sample_kernel<0, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((sample_kernel<0, 1>), grid, block, 0, st, p);
   }
   return mi_check_launch("mi_sample_from_logits");
 }
@@ -639,20 +642,23 @@ extern "C" int mi_selected_log_probs(const void* logits, int64_t stride_row, int
   if (!logits || !token_ids || !log_probs) return mi_fail(MI_ERR_NULL, "mi_selected_log_probs: null pointer argument");
   if (T < 0 || vocab <= 0 || stride_row < vocab)
     return mi_fail(MI_ERR_SHAPE, "mi_selected_log_probs: need T >= 0, vocab > 0 and a row stride of at least vocab");
-  if (logits_dtype != 0 && logits_dtype != 1)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_selected_log_probs: logits must be fp32 (0) or bf16 (1)");
+  if (logits_dtype < 0 || logits_dtype > 2)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_selected_log_probs: logits must be fp32 (0), bf16 (1) or fp16 (2)");
   LogProbParams p;
   p.logits = logits; p.stride = stride_row; p.T = T; p.V = vocab; p.token_ids = token_ids; p.out = log_probs;
-  const int esize = logits_dtype == 1 ? 2 : 4;
+  const int esize = logits_dtype != 0 ? 2 : 4;
   const bool wide = !(((uintptr_t)logits | (uintptr_t)(stride_row * esize)) & 15);  // 16-byte loads
   const dim3 grid(T), block(kLogProbThreads);
   hipStream_t st = (hipStream_t)stream;
-  if (logits_dtype == 1) {
-    if (wide) hipLaunchKernelGGL((selected_log_probs_kernel<true, 8>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((selected_log_probs_kernel<true, 1>), grid, block, 0, st, p);
+  if (logits_dtype == 2) {
+    if (wide) hipLaunchKernelGGL((selected_log_probs_kernel<2, 8>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((selected_log_probs_kernel<2, 1>), grid, block, 0, st, p);
+  } else if (logits_dtype == 1) {
+    if (wide) hipLaunchKernelGGL((selected_log_probs_kernel<1, 8>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((selected_log_probs_kernel<1, 1>), grid, block, 0, st, p);
   } else {
-    if (wide) hipLaunchKernelGGL((selected_log_probs_kernel<false, 4>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((selected_log_probs_kernel<false, 1>), grid, block, 0, st, p);
+    if (wide) hipLaunchKernelGGL((selected_log_probs_kernel<0, 4>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((selected_log_probs_kernel<0, 1>), grid, block, 0, st, p);
   }
   return mi_check_launch("mi_selected_log_probs");
 }

@@ -11,8 +11,12 @@ from typing import Optional, Tuple
 import torch
 from torch import Tensor
 
+import ctypes
+import threading
+
 from . import _lib
-from ._lib import MI_KV_BF16, MI_KV_FP8_E4M3, MI_NORM_L2, MI_NORM_NONE, MI_NORM_RMS  # noqa: F401
+from ._lib import (MI_DTYPE_BF16, MI_DTYPE_FP16, MI_KV_16BIT, MI_KV_BF16, MI_KV_FP8_E4M3,  # noqa: F401
+                   MI_NORM_L2, MI_NORM_NONE, MI_NORM_RMS)
 
 _NORM_KINDS = {None: MI_NORM_NONE, "none": MI_NORM_NONE, "rms": MI_NORM_RMS, "l2": MI_NORM_L2}
 
@@ -39,7 +43,9 @@ def _cache_strides(cache: Tensor) -> Tuple[int, int, int]:
     return cache.stride(0), cache.stride(1), cache.stride(2)
 
 
-# per-device split-K workspace, grown on demand (owned here, handed to the C ABI as caller memory)
+# Split-K workspaces, one per (device, stream) and grown on demand (owned here, handed to the C ABI as caller
+# memory).  Calls on one stream are ordered and may share a buffer; calls on different streams of a device may
+# overlap, so each stream gets its own.
 _workspaces: dict = {}
 _retired_workspaces: list = []   # outgrown buffers stay alive: work already enqueued may still use them
 _workspace_override: list = []   # innermost ``use_workspace`` buffer
@@ -52,12 +58,13 @@ def _workspace(device: torch.device, nbytes: int) -> Optional[Tensor]:
         ws = _workspace_override[-1]
         _require(ws.device == device and ws.numel() >= nbytes, "the workspace given to use_workspace is too small")
         return ws
-    ws = _workspaces.get(device)
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
             _retired_workspaces.append(ws)
         ws = torch.empty(max(nbytes, 2 * (0 if ws is None else ws.numel())), dtype=torch.uint8, device=device)
-        _workspaces[device] = ws
+        _workspaces[key] = ws
     return ws
 
 
@@ -77,9 +84,68 @@ class use_workspace:
         return False
 
 
+# ---------------------------------------------------------------------------------------------
+# experiment knobs: the C ABI takes them per call (MiTuning); this module keeps the set that its own calls pass
+# ---------------------------------------------------------------------------------------------
+_TUNING_FIELDS = tuple(name for name, _ in _lib.MiTuning._fields_ if name != "reserved")
+_tuning_defaults: dict = {}          # set_tuning: every thread, until changed back
+_tuning_local = threading.local()    # tuning(...): this thread, inside the with block
+
+
 def set_tuning(name: str, value: int) -> None:
-    lib = _lib.load()
-    _lib.check(lib.mi_set_tuning(name.encode(), int(value)), "mi_set_tuning")
+    """Knob ``name`` (a field of ``MiTuning`` in the header) for every later call of this module; 0 = the default.
+    A sweep / test hook: the library itself keeps no such state."""
+    _require(name in _TUNING_FIELDS, f"unknown knob {name!r}; the knobs are {', '.join(_TUNING_FIELDS)}")
+    if int(value) == 0:
+        _tuning_defaults.pop(name, None)
+    else:
+        _tuning_defaults[name] = int(value)
+
+
+class tuning:
+    """``with ops.tuning(decode_grid=7, prefill_two_phase=-1): ...`` -- knobs for the calls this thread makes
+    inside the block (on top of :func:`set_tuning`)."""
+
+    def __init__(self, **knobs: int):
+        for name in knobs:
+            _require(name in _TUNING_FIELDS, f"unknown knob {name!r}")
+        self.knobs = {k: int(v) for k, v in knobs.items()}
+
+    def __enter__(self):
+        stack = getattr(_tuning_local, "stack", None)
+        if stack is None:
+            stack = _tuning_local.stack = []
+        stack.append(self.knobs)
+        return self
+
+    def __exit__(self, *exc):
+        _tuning_local.stack.pop()
+        return False
+
+
+def current_tuning() -> dict:
+    """The knobs a call made now would pass (name -> non-zero value)."""
+    merged = dict(_tuning_defaults)
+    for layer in getattr(_tuning_local, "stack", None) or ():
+        merged.update(layer)
+    return {k: v for k, v in merged.items() if v != 0}
+
+
+def _tuning_arg():
+    """``const MiTuning*`` for a C call: NULL when every knob is at its default."""
+    knobs = current_tuning()
+    return ctypes.byref(_lib.MiTuning(**knobs)) if knobs else None
+
+
+_DTYPE_CODES = {torch.bfloat16: MI_DTYPE_BF16, torch.float16: MI_DTYPE_FP16}
+
+
+_LOGIT_CODES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}
+
+
+def _dtype_code(t: Tensor, name: str) -> int:
+    _require(t.dtype in _DTYPE_CODES, f"{name} must be bf16 or fp16, got {t.dtype}")
+    return _DTYPE_CODES[t.dtype]
 
 
 # ---------------------------------------------------------------------------------------------
@@ -216,20 +282,22 @@ def _qo_view(x: Tensor, name: str) -> Tensor:
         _require(x.size(1) == 1, f"{name} must be [T, 1, Hq, d] or [T, Hq, d]")
         x = x.squeeze(1)
     _require(x.dim() == 3 and x.stride(2) == 1, f"{name} must be [T, Hq, d] with contiguous d")
-    _require(x.dtype == torch.bfloat16, f"{name} must be bf16")
+    _require(x.dtype in _DTYPE_CODES, f"{name} must be bf16 or fp16, got {x.dtype}")
     return x
 
 
 def decode_workspace_bytes(R: int, Hq: int, Hkv: int, head_dim: int, chunk: int, max_kv_len: int,
                            split_tokens: int = 0) -> int:
-    return int(_lib.load().mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, chunk, max_kv_len, split_tokens))
+    return int(_lib.load().mi_decode_workspace_bytes(R, Hq, Hkv, head_dim, chunk, max_kv_len, split_tokens,
+                                                     _tuning_arg()))
 
 
 def prefill_workspace_bytes(T: int, R: int, Hq: int, Hkv: int, head_dim: int, max_kv_len: int,
                             split_tokens: int = 0) -> int:
     """Scratch of one varlen attention call over ``T`` query rows of ``R`` requests: the decode part's
     partials and, when the tile kernel splits the keys, its partials behind them."""
-    return int(_lib.load().mi_prefill_workspace_bytes(T, R, Hq, Hkv, head_dim, max_kv_len, split_tokens))
+    return int(_lib.load().mi_prefill_workspace_bytes(T, R, Hq, Hkv, head_dim, max_kv_len, split_tokens,
+                                                      _tuning_arg()))
 
 
 def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens: Tensor, block_table: Tensor,
@@ -245,7 +313,8 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
     N, C, Hkv, Dk = k_cache.shape
     _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
     fp8 = k_cache.element_size() == 1
-    _require(fp8 or k_cache.dtype == torch.bfloat16, "KV cache must be bf16 or a one-byte fp8 type")
+    _require(fp8 or k_cache.dtype == q3.dtype, "the KV cache must have the queries' 16-bit type, or be a one-byte fp8 type")
+    _require(not fp8 or q3.dtype == torch.bfloat16, "an fp8 cache needs bf16 queries")
     _require(v_cache.dtype == k_cache.dtype, "k_cache / v_cache dtypes differ")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
@@ -264,8 +333,9 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
     if out is None:
         out = torch.empty_like(q)
     o3 = _qo_view(out, "out")
-    _require(tuple(o3.shape) == (R, Hq, D), "out shape mismatch")
-    need = lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, C, max_kv_len, split_tokens)
+    _require(tuple(o3.shape) == (R, Hq, D) and o3.dtype == q3.dtype, "out shape / dtype mismatch")
+    tune = _tuning_arg()
+    need = lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, C, max_kv_len, split_tokens, tune)
     if workspace is None:
         workspace = _workspace(q.device, need)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
@@ -273,8 +343,8 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
         block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
         _ptr(workspace), ws_bytes, R, Hq, Hkv, D, C, int(max_kv_len), int(split_tokens), float(softmax_scale),
-        MI_KV_FP8_E4M3 if fp8 else MI_KV_BF16, _ptr(k_scales), _ptr(v_scales), _stream(q)),
-        "mi_paged_decode_attention")
+        MI_KV_FP8_E4M3 if fp8 else MI_KV_16BIT, _ptr(k_scales), _ptr(v_scales), _dtype_code(q3, "q"), tune,
+        _stream(q)), "mi_paged_decode_attention")
     return out
 
 
@@ -292,7 +362,8 @@ def paged_decode_attention_noalloc(q: Tensor, k_cache: Tensor, v_cache: Tensor, 
     N, C, Hkv, Dk = k_cache.shape
     _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
     fp8 = k_cache.element_size() == 1
-    _require(fp8 or k_cache.dtype == torch.bfloat16, "KV cache must be bf16 or a one-byte fp8 type")
+    _require(fp8 or k_cache.dtype == q3.dtype, "the KV cache must have the queries' 16-bit type, or be a one-byte fp8 type")
+    _require(not fp8 or q3.dtype == torch.bfloat16, "an fp8 cache needs bf16 queries")
     _require(v_cache.dtype == k_cache.dtype, "k_cache / v_cache dtypes differ")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
@@ -306,7 +377,7 @@ def paged_decode_attention_noalloc(q: Tensor, k_cache: Tensor, v_cache: Tensor, 
                  and tuple(k_scales.shape) == (N, Hkv) and tuple(v_scales.shape) == (N, Hkv),
                  "scales must be contiguous fp32 [N, Hkv]")
     o3 = _qo_view(out, "out")
-    _require(tuple(o3.shape) == (R, Hq, D), "out shape mismatch")
+    _require(tuple(o3.shape) == (R, Hq, D) and o3.dtype == q3.dtype, "out shape / dtype mismatch")
     if max_kv_len is None:
         max_kv_len = block_table.size(1) * C
     if softmax_scale is None:
@@ -315,8 +386,8 @@ def paged_decode_attention_noalloc(q: Tensor, k_cache: Tensor, v_cache: Tensor, 
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
         block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
         R, Hq, Hkv, D, C, int(max_kv_len), int(split_tokens), float(softmax_scale),
-        MI_KV_FP8_E4M3 if fp8 else MI_KV_BF16, _ptr(k_scales), _ptr(v_scales), stream),
-        "mi_paged_decode_attention_noalloc")
+        MI_KV_FP8_E4M3 if fp8 else MI_KV_16BIT, _ptr(k_scales), _ptr(v_scales), _dtype_code(q3, "q"), _tuning_arg(),
+        stream), "mi_paged_decode_attention_noalloc")
     return out
 
 
@@ -333,7 +404,7 @@ def paged_mla_decode_attention(q: Tensor, kv_cache: Tensor, kv_lens: Tensor, blo
         _require(kv_cache.size(2) == 1, "the latent cache has one row per token")
         kv_cache = kv_cache.squeeze(2)
     _require(kv_cache.dim() == 3 and kv_cache.stride(2) == 1 and kv_cache.size(2) == Dk
-             and kv_cache.dtype == torch.bfloat16, "kv_cache must be bf16 [N, C, 576] with contiguous rows")
+             and kv_cache.dtype == q3.dtype, "kv_cache must be [N, C, 576] of the queries' type with contiguous rows")
     _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
     _require(kv_lens.dtype == torch.int32 and kv_lens.is_contiguous() and kv_lens.numel() >= R, "bad kv_lens")
     C = kv_cache.size(1)
@@ -343,12 +414,13 @@ def paged_mla_decode_attention(q: Tensor, kv_cache: Tensor, kv_lens: Tensor, blo
         out = torch.empty(q.shape[:-1] + (head_dim_v,), dtype=q.dtype, device=q.device)
     o3 = _qo_view(out, "out")
     _require(tuple(o3.shape) == (R, Hq, head_dim_v), "out shape mismatch")
-    workspace = _workspace(q.device, lib.mi_mla_decode_workspace_bytes(R, Hq, head_dim_v))
+    tune = _tuning_arg()
+    workspace = _workspace(q.device, lib.mi_mla_decode_workspace_bytes(R, Hq, head_dim_v, tune))
     _lib.check(lib.mi_paged_mla_decode_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), kv_cache.data_ptr(), kv_cache.stride(0), kv_cache.stride(1),
         block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
         _ptr(workspace), 0 if workspace is None else workspace.numel(), R, Hq, Dk, head_dim_v, C, int(max_kv_len),
-        float(softmax_scale), stream), "mi_paged_mla_decode_attention")
+        float(softmax_scale), _dtype_code(q3, "q"), tune, stream), "mi_paged_mla_decode_attention")
     return out
 
 
@@ -365,7 +437,7 @@ def paged_prefill_attention_mla(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_
     T, Hq, Dk = q3.shape
     _require(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[:3] == v_cache.shape[:3],
              "key / value caches must be [N, C, H, d] with equal leading dimensions")
-    _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16, "the caches must be bf16")
+    _require(k_cache.dtype == q3.dtype and v_cache.dtype == q3.dtype, "the caches must have the queries' 16-bit type")
     N, C, Hkv, _ = k_cache.shape
     Dv = v_cache.size(3)
     _require(k_cache.size(3) == Dk, "query and key widths differ")
@@ -379,10 +451,11 @@ def paged_prefill_attention_mla(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_
     if out is None:
         out = torch.empty(q.shape[:-1] + (Dv,), dtype=q.dtype, device=q.device)
     o3 = _qo_view(out, "out")
-    _require(tuple(o3.shape) == (T, Hq, Dv), "out shape mismatch")
+    _require(tuple(o3.shape) == (T, Hq, Dv) and o3.dtype == q3.dtype, "out shape / dtype mismatch")
     if max_kv_len is None:
         max_kv_len = block_table.size(1) * C
-    need = lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, Dv, int(max_kv_len), 0)
+    tune = _tuning_arg()
+    need = lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, Dv, int(max_kv_len), 0, tune)
     if _workspace_override and _workspace_override[-1].numel() < need:
         workspace = None  # the split of the keys is optional here: a caller-sized workspace that is too small turns it off
     else:
@@ -392,7 +465,7 @@ def paged_prefill_attention_mla(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), ksc, kst, ksh, v_cache.data_ptr(), vsc, vst, vsh,
         block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),
         o3.data_ptr(), o3.stride(0), o3.stride(1), _ptr(workspace), ws_bytes, T, R, Hq, Hkv, Dk, Dv, C,
-        int(max_kv_len), float(softmax_scale), stream),
+        int(max_kv_len), float(softmax_scale), _dtype_code(q3, "q"), tune, stream),
         "mi_paged_prefill_attention_mla")
     return out
 
@@ -416,8 +489,8 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
                  and k_scales.is_contiguous() and v_scales.is_contiguous() and tuple(k_scales.shape) == (N, Hkv)
                  and tuple(v_scales.shape) == (N, Hkv), "scales must be contiguous fp32 [N, Hkv]")
     else:
-        _require(k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16,
-                 "the cache must be bf16, or bytes with scales")
+        _require(k_cache.dtype == q3.dtype and v_cache.dtype == q3.dtype,
+                 "the cache must have the queries' 16-bit type, or be bytes with scales")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
     _require(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.is_contiguous(), "cu_seqlens_q must be contiguous int32")
@@ -432,23 +505,24 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
     if out is None:
         out = torch.empty_like(q)
     o3 = _qo_view(out, "out")
-    _require(tuple(o3.shape) == (T, Hq, D), "out shape mismatch")
-    workspace = _workspace(q.device, lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, D, int(max_kv_len), 0))
+    _require(tuple(o3.shape) == (T, Hq, D) and o3.dtype == q3.dtype, "out shape / dtype mismatch")
+    tune = _tuning_arg()
+    workspace = _workspace(q.device, lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, D, int(max_kv_len), 0, tune))
     ws_bytes = 0 if workspace is None else workspace.numel()
     if fp8:
         _lib.check(lib.mi_paged_prefill_attention_fp8(
             q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
             k_scales.data_ptr(), v_scales.data_ptr(), block_table.data_ptr(), block_table.stride(0),
             cu_seqlens_q.data_ptr(), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
-            _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C, int(max_kv_len), 0, float(softmax_scale), _stream(q)),
-            "mi_paged_prefill_attention_fp8")
+            _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C, int(max_kv_len), 0, float(softmax_scale), tune,
+            _stream(q)), "mi_paged_prefill_attention_fp8")
         return out
     _lib.check(lib.mi_paged_prefill_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
         block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),
         o3.data_ptr(), o3.stride(0), o3.stride(1), _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C,
         int(max_kv_len), 0,
-        float(softmax_scale), _stream(q)), "mi_paged_prefill_attention")
+        float(softmax_scale), _dtype_code(q3, "q"), tune, _stream(q)), "mi_paged_prefill_attention")
     return out
 
 
@@ -506,19 +580,23 @@ def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: O
         _require(tuple(v3.shape) == tuple(k3.shape) and v3.stride(1) == D, "value shape")
     ang, a_stride, rot = _angles(rotary_emb)
     for w in (q_weight, k_weight):
-        _require(w is None or (w.dtype == torch.bfloat16 and w.numel() == D and w.is_contiguous()), "norm weights must be bf16 [d]")
+        _require(w is None or (w.dtype == ref.dtype and w.numel() == D and w.is_contiguous()),
+                 "norm weights must be [d] of the tensors' 16-bit type")
     for pz in (q_positions, k_positions, token_to_chunk_idx, token_to_local_pos):
         _require(pz is None or (pz.dtype == torch.int64 and pz.is_contiguous() and pz.numel() >= T), "index rows must be int64 [>=T]")
     sc = st = 0
     chunk = 0
     if k_cache is not None:
-        _require(k_cache.dtype == torch.bfloat16 and v_cache is not None and v_cache.dtype == torch.bfloat16, "bf16 caches")
+        _require(k_cache.dtype == ref.dtype and v_cache is not None and v_cache.dtype == ref.dtype,
+                 "the caches must have the tensors' 16-bit type")
         sc, st, sh = _cache_strides(k_cache)
         _require(_cache_strides(v_cache) == (sc, st, sh) and sh == D, "cache layout")
         chunk = k_cache.size(1)
         if block_table is not None:
             _require(block_table.dtype == torch.int32 and block_table.stride(1) == 1, "bad block_table")
             _require(kv_lens is not None and kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "bad kv_lens")
+    for other in (q3, k3, qo3, ko3, v3):
+        _require(other is None or other.dtype == ref.dtype, "query / key / value / outputs must share one 16-bit type")
     _lib.check(lib.mi_norm_rope_append(
         _ptr(q3), 0 if q3 is None else q3.stride(0), _ptr(qo3), 0 if qo3 is None else qo3.stride(0),
         _ptr(k3), 0 if k3 is None else k3.stride(0),
@@ -527,7 +605,8 @@ def norm_rope_append(query: Optional[Tensor], key: Optional[Tensor], *, value: O
         int(bool(rotary_interleaved)), float(mscale), _ptr(q_positions), _ptr(k_positions),
         _ptr(k_cache), _ptr(v_cache), sc, st, _ptr(token_to_chunk_idx), _ptr(token_to_local_pos),
         _ptr(block_table), 0 if block_table is None else block_table.stride(0), _ptr(kv_lens), chunk,
-        T, Hq, Hkv, D, int(bool(faithful_rounding)), _stream(ref)), "mi_norm_rope_append")
+        T, Hq, Hkv, D, int(bool(faithful_rounding)), _dtype_code(ref, "query / key"), _tuning_arg(), _stream(ref)),
+        "mi_norm_rope_append")
 
 
 def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_heads: int, query_out: Tensor,
@@ -543,7 +622,7 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
     query group: its query heads, then its key head, then its value head -- the layout that
     ``get_query_key_value_tensors`` splits, attention.py:985-1030) without materialising the split."""
     lib = _lib.load()
-    _require(mixed_qkv.is_cuda and mixed_qkv.dtype == torch.bfloat16, "mixed_qkv must be a bf16 device tensor")
+    _require(mixed_qkv.is_cuda and mixed_qkv.dtype in _DTYPE_CODES, "mixed_qkv must be a bf16 or fp16 device tensor")
     if mixed_qkv.dim() == 3:
         _require(mixed_qkv.size(1) == 1, "mixed_qkv must be [T, 1, W]")
         mixed_qkv = mixed_qkv[:, 0]
@@ -553,7 +632,8 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
     _require(Hq > 0 and Hkv > 0 and Hq % Hkv == 0 and W % (Hq + 2 * Hkv) == 0, "mixed_qkv width / head counts")
     D = W // (Hq + 2 * Hkv)
     qo3 = _qo_view(query_out, "query_out")
-    _require(tuple(qo3.shape) == (T, Hq, D) and qo3.stride(1) == D, "query_out must be [T, Hq, d]")
+    _require(tuple(qo3.shape) == (T, Hq, D) and qo3.stride(1) == D and qo3.dtype == mixed_qkv.dtype,
+             "query_out must be [T, Hq, d] of the projection's type")
     ko3 = None
     if key_out is not None:
         ko3 = _qo_view(key_out, "key_out")
@@ -561,13 +641,15 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
     _require(ko3 is not None or k_cache is not None, "the key needs a destination: key_out and/or the cache")
     ang, a_stride, rot = _angles(rotary_emb)
     for w in (q_weight, k_weight):
-        _require(w is None or (w.dtype == torch.bfloat16 and w.numel() == D and w.is_contiguous()), "norm weights must be bf16 [d]")
+        _require(w is None or (w.dtype == mixed_qkv.dtype and w.numel() == D and w.is_contiguous()),
+                 "norm weights must be [d] of the tensors' 16-bit type")
     for pz in (q_positions, k_positions, token_to_chunk_idx, token_to_local_pos):
         _require(pz is None or (pz.dtype == torch.int64 and pz.is_contiguous() and pz.numel() >= T), "index rows must be int64 [>=T]")
     sc = st = 0
     chunk = 0
     if k_cache is not None:
-        _require(k_cache.dtype == torch.bfloat16 and v_cache is not None and v_cache.dtype == torch.bfloat16, "bf16 caches")
+        _require(k_cache.dtype == mixed_qkv.dtype and v_cache is not None and v_cache.dtype == mixed_qkv.dtype,
+                 "the caches must have the projection's 16-bit type")
         sc, st, sh = _cache_strides(k_cache)
         _require(_cache_strides(v_cache) == (sc, st, sh) and sh == D, "cache layout")
         chunk = k_cache.size(1)
@@ -580,7 +662,8 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
         int(bool(rotary_interleaved)), float(mscale), _ptr(q_positions), _ptr(k_positions),
         _ptr(k_cache), _ptr(v_cache), sc, st, _ptr(token_to_chunk_idx), _ptr(token_to_local_pos),
         _ptr(block_table), 0 if block_table is None else block_table.stride(0), _ptr(kv_lens), chunk,
-        T, Hq, Hkv, D, int(bool(faithful_rounding)), _stream(mixed_qkv)), "mi_qkv_norm_rope_append")
+        T, Hq, Hkv, D, int(bool(faithful_rounding)), _dtype_code(mixed_qkv, "mixed_qkv"), _tuning_arg(),
+        _stream(mixed_qkv)), "mi_qkv_norm_rope_append")
 
 
 # ---------------------------------------------------------------------------------------------
@@ -662,18 +745,18 @@ def last_token_gather(rows: Tensor, request_query_lengths: Tensor, out: Optional
 
 def selected_log_probs(logits: Tensor, token_ids: Tensor) -> Tensor:
     """``log_softmax(logits.float(), -1)[arange(T), token_ids]`` (fp32 ``[T]``) with one read of each row of
-    ``logits`` ``[T, V]`` (fp32 or bf16) and no ``[T, V]`` intermediate."""
+    ``logits`` ``[T, V]`` (fp32, bf16 or fp16) and no ``[T, V]`` intermediate."""
     lib = _lib.load()
     stream = _stream(logits)
     _require(logits.dim() == 2 and logits.stride(1) == 1, "logits must be [T, V] with contiguous V")
-    _require(logits.dtype in (torch.float32, torch.bfloat16), "logits must be fp32 or bf16")
+    _require(logits.dtype in _LOGIT_CODES, "logits must be fp32, bf16 or fp16")
     T, V = logits.shape
     _require(token_ids.dtype == torch.int64 and token_ids.dim() == 1 and token_ids.numel() == T
              and token_ids.is_contiguous() and token_ids.device == logits.device,
              "token_ids must be a contiguous int64 row with one id per row of logits")
     out = torch.empty(T, dtype=torch.float32, device=logits.device)
     _lib.check(lib.mi_selected_log_probs(logits.data_ptr(), logits.stride(0),
-                                         1 if logits.dtype == torch.bfloat16 else 0, T, V,
+                                         _LOGIT_CODES[logits.dtype], T, V,
                                          token_ids.data_ptr(), out.data_ptr(), stream), "mi_selected_log_probs")
     return out
 
@@ -683,7 +766,7 @@ def sample_from_logits(logits: Tensor, *, top_k: int = 0, top_p: float = 0.0, te
                        termination_id: Optional[int] = None, kv_length_offsets: Optional[Tensor] = None,
                        query_lengths: Optional[Tensor] = None, output_lengths: Optional[Tensor] = None,
                        return_cut: bool = False):
-    """One launch: filter + draw per row of ``logits`` ``[R, V]`` (fp32 or bf16) and, when
+    """One launch: filter + draw per row of ``logits`` ``[R, V]`` (fp32, bf16 or fp16) and, when
     ``termination_id`` is given, the uint8 mask of requests that go on generating.
 
     Returns ``(samples int64 [R], mask uint8 [R] or None)`` and, with ``return_cut``, also the
@@ -691,7 +774,7 @@ def sample_from_logits(logits: Tensor, *, top_k: int = 0, top_p: float = 0.0, te
     lib = _lib.load()
     stream = _stream(logits)
     _require(logits.dim() == 2 and logits.stride(1) == 1, "logits must be [R, V] with contiguous V")
-    _require(logits.dtype in (torch.float32, torch.bfloat16), "logits must be fp32 or bf16")
+    _require(logits.dtype in _LOGIT_CODES, "logits must be fp32, bf16 or fp16")
     R, V = logits.shape
     dev = logits.device
     if top_k != 1:
@@ -712,7 +795,7 @@ def sample_from_logits(logits: Tensor, *, top_k: int = 0, top_p: float = 0.0, te
         _require(all(t is None for t in lens), "request lengths without a termination id")
     cut = torch.empty(R, dtype=torch.float32, device=dev) if return_cut else None
     _lib.check(lib.mi_sample_from_logits(
-        logits.data_ptr(), logits.stride(0), 1 if logits.dtype == torch.bfloat16 else 0, R, V, int(top_k),
+        logits.data_ptr(), logits.stride(0), _LOGIT_CODES[logits.dtype], R, V, int(top_k),
         float(top_p), float(temperature), _ptr(uniform), int(vocab_size or 0), samples.data_ptr(), _ptr(cut),
         _ptr(kv_length_offsets), _ptr(query_lengths), _ptr(output_lengths),
         int(termination_id) if termination_id is not None else -1, _ptr(mask), stream), "mi_sample_from_logits")

@@ -95,12 +95,12 @@ class DecodeCase:
 
 def make_decode_case(cfg: DecodeConfig, device, *, batch: Optional[int] = None, seed: Optional[int] = None,
                      on_device_rng: bool = False, pool_chunks: Optional[int] = None,
-                     lens: Optional[Tensor] = None) -> DecodeCase:
+                     lens: Optional[Tensor] = None, dtype: torch.dtype = torch.bfloat16) -> DecodeCase:
     """Build q, the new K/V rows, a bf16 cache filled with N(0,1), block table and lengths.
 
     ``on_device_rng=False`` draws values on the CPU and moves them (bit-identical inputs
     for a CPU checker); ``True`` draws the cache on ``device`` (for full-size runs).
-    The cache is always bf16 here; fp8 configurations quantise it afterwards with the
+    The cache has ``dtype`` (bf16 or fp16) here; fp8 configurations quantise a bf16 one afterwards with the
     library's own kernel or the checker's quantiser.
     """
     device = torch.device(device)
@@ -109,24 +109,24 @@ def make_decode_case(cfg: DecodeConfig, device, *, batch: Optional[int] = None, 
     if lens is None:
         lens = draw_lengths(B, cfg.len_lo, cfg.len_hi, cpu_gen)
     table, N = build_block_table(lens, cfg.chunk, cpu_gen, pool_chunks)
-    q = torch.randn(B, 1, cfg.Hq, cfg.d, generator=cpu_gen).bfloat16()
-    k_new = torch.randn(B, 1, cfg.Hkv, cfg.d, generator=cpu_gen).bfloat16()
-    v_new = torch.randn(B, 1, cfg.Hkv, cfg.d, generator=cpu_gen).bfloat16()
+    q = torch.randn(B, 1, cfg.Hq, cfg.d, generator=cpu_gen).to(dtype)
+    k_new = torch.randn(B, 1, cfg.Hkv, cfg.d, generator=cpu_gen).to(dtype)
+    v_new = torch.randn(B, 1, cfg.Hkv, cfg.d, generator=cpu_gen).to(dtype)
     shape = (N, cfg.chunk, cfg.Hkv, cfg.d)
     if on_device_rng and device.type != "cpu":
         dgen = torch.Generator(device=device).manual_seed((cfg.seed if seed is None else seed) + 7)
-        k_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16, device=device), dgen)
-        v_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16, device=device), dgen)
+        k_cache = randn_fill_(torch.empty(shape, dtype=dtype, device=device), dgen)
+        v_cache = randn_fill_(torch.empty(shape, dtype=dtype, device=device), dgen)
     else:
-        k_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16), cpu_gen).to(device)
-        v_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16), cpu_gen).to(device)
+        k_cache = randn_fill_(torch.empty(shape, dtype=dtype), cpu_gen).to(device)
+        v_cache = randn_fill_(torch.empty(shape, dtype=dtype), cpu_gen).to(device)
     return DecodeCase(cfg, q.to(device), k_new.to(device), v_new.to(device), k_cache, v_cache,
                       table.to(device), lens.to(device))
 
 
 def make_prefill_case(device, *, n_prefill: int, new_tokens: int, ctx_lo: int, ctx_hi: int, n_decode: int,
                       dec_lo: int, dec_hi: int, Hq: int, Hkv: int, d: int, chunk: int = 256, seed: int = 1003,
-                      on_device_rng: bool = False):
+                      on_device_rng: bool = False, dtype: torch.dtype = torch.bfloat16):
     """Mixed batch: ``n_prefill`` requests with ``new_tokens`` new tokens over an existing context
     of U[ctx_lo, ctx_hi] tokens, followed by ``n_decode`` one-token requests with total length
     U[dec_lo, dec_hi].  Returns (q [T,Hq,d], k_cache, v_cache, cu_seqlens_q, kv_lens, block_table)."""
@@ -141,15 +141,15 @@ def make_prefill_case(device, *, n_prefill: int, new_tokens: int, ctx_lo: int, c
     cu_q[1:] = torch.cumsum(q_lens, 0)
     table, N = build_block_table(kv_lens, chunk, gen)
     T = int(cu_q[-1])
-    q = torch.randn(T, Hq, d, generator=gen).bfloat16()
+    q = torch.randn(T, Hq, d, generator=gen).to(dtype)
     shape = (N, chunk, Hkv, d)
     if on_device_rng and device.type != "cpu":
         dgen = torch.Generator(device=device).manual_seed(seed + 7)
-        k_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16, device=device), dgen)
-        v_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16, device=device), dgen)
+        k_cache = randn_fill_(torch.empty(shape, dtype=dtype, device=device), dgen)
+        v_cache = randn_fill_(torch.empty(shape, dtype=dtype, device=device), dgen)
     else:
-        k_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16), gen).to(device)
-        v_cache = randn_fill_(torch.empty(shape, dtype=torch.bfloat16), gen).to(device)
+        k_cache = randn_fill_(torch.empty(shape, dtype=dtype), gen).to(device)
+        v_cache = randn_fill_(torch.empty(shape, dtype=dtype), gen).to(device)
     return q.to(device), k_cache, v_cache, cu_q.to(device), kv_lens.to(device), table.to(device)
 
 

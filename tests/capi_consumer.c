@@ -14,7 +14,7 @@ int main(void) {
   int (*p_version)(void) = mi_version;
   const char* (*p_error)(void) = mi_last_error;
   const void* table[] = {
-      (const void*)(size_t)mi_set_tuning, (const void*)(size_t)mi_profile_enable,
+      (const void*)(size_t)mi_profile_enable,
       (const void*)(size_t)mi_profile_collect, (const void*)(size_t)mi_kv_append,
       (const void*)(size_t)mi_kv_append_decode, (const void*)(size_t)mi_kv_quantize_chunks_fp8,
       (const void*)(size_t)mi_kv_append_decode_fp8, (const void*)(size_t)mi_kv_append_fp8,
@@ -39,8 +39,15 @@ int main(void) {
   /* null pointers with T > 0: rejected on the host, with a message */
   rc = mi_kv_append(NULL, NULL, 8, NULL, NULL, 8, 8, NULL, NULL, 4, 8, 2, NULL);
   if (rc != MI_ERR_NULL || !strstr(p_error(), "null")) return 3;
-  if (mi_set_tuning("no_such_knob", 1) != MI_ERR_UNSUPPORTED) return 4;
-  if (mi_decode_workspace_bytes(0, 8, 2, 128, 16, 16, 0) != 0) return 5;
+  {
+    MiTuning knobs = {0};
+    knobs.decode_grid = 7;
+    if (mi_decode_workspace_bytes(4, 8, 2, 128, 16, 16, 0, &knobs) != (7 + 4) * 8 * 129 * 4 + 4 * 8) return 4;
+    knobs.decode_min_waves = 9;  /* out of range */
+    if (mi_decode_workspace_bytes(4, 8, 2, 128, 16, 16, 0, &knobs) != -1) return 4;
+  }
+  if (mi_decode_workspace_bytes(0, 8, 2, 128, 16, 16, 0, NULL) != 0) return 5;
+  if (sizeof(MiTuning) != 64) return 7;
   if (MI_NOALLOC_SCRATCH_BYTES != 16 * 1024 * 1024) return 6;
   printf("capi_consumer ok (ABI revision %d)\n", p_version());
   return 0;

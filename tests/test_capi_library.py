@@ -63,7 +63,7 @@ def test_the_parser_sees_a_transposed_argument():
     assert ret is ctypes.c_int and args[2] is ctypes.c_int64 and args[9] is ctypes.c_int32
     assert protos["mi_last_error"] == (ctypes.c_char_p, [])
     assert protos["mi_decode_workspace_bytes"][0] is ctypes.c_int64
-    assert protos["mi_set_tuning"][1] == [ctypes.c_char_p, ctypes.c_int32]
+    assert protos["mi_decode_workspace_bytes"][1][-1] is ctypes.c_void_p  # const MiTuning*
 
 
 @pytest.mark.skipif(shutil.which("gcc") is None, reason="needs a C compiler")
@@ -107,10 +107,12 @@ def test_python_binding_covers_the_header(mi):
 def test_argument_validation_needs_no_gpu(mi):
     """Rejections happen on the host before anything is enqueued."""
     lib = mi._lib.load()
-    assert lib.mi_set_tuning(b"no_such_knob", 1) < 0
-    assert b"unknown knob" in lib.mi_last_error()
-    assert lib.mi_set_tuning(b"decode_tile_subtiles", 3) < 0
-    assert lib.mi_set_tuning(b"decode_tile_subtiles", 0) == 0
+    # knobs travel with the call; an out-of-range one is rejected before anything else is looked at
+    bad = mi._lib.MiTuning(decode_tile_subtiles=3)
+    assert lib.mi_decode_workspace_bytes(4, 8, 2, 128, 16, 16, 0, ctypes.byref(bad)) == -1
+    assert b"decode_tile_subtiles" in lib.mi_last_error()
+    assert lib.mi_decode_workspace_bytes(4, 8, 2, 128, 16, 16, 0, ctypes.byref(mi._lib.MiTuning(decode_grid=7))) == \
+        (7 + 4) * 8 * 129 * 4 + 4 * 8
     # null pointers
     rc = lib.mi_kv_append(None, None, 8, None, None, 8, 8, None, None, 4, 8, 2, None)
     assert rc == -1 and b"null" in lib.mi_last_error()
@@ -119,15 +121,19 @@ def test_argument_validation_needs_no_gpu(mi):
     # unsupported head_dim / grouping are refused with a message
     one = ctypes.c_void_p(16)
     rc = lib.mi_paged_decode_attention(one, 96, 96, one, one, 96, 96, 96, one, 1, one, one, 96, 96, one, 1 << 30,
-                                       1, 1, 1, 96, 16, 16, 0, 0.1, 0, None, None, None)
+                                       1, 1, 1, 96, 16, 16, 0, 0.1, 0, None, None, 0, None, None)
     assert rc == -4 and b"head_dim" in lib.mi_last_error()
     rc = lib.mi_paged_decode_attention(one, 128, 128, one, one, 128, 128, 128, one, 1, one, one, 128, 128, one,
-                                       1 << 30, 1, 34, 2, 128, 16, 16, 0, 0.1, 0, None, None, None)
+                                       1 << 30, 1, 34, 2, 128, 16, 16, 0, 0.1, 0, None, None, 0, None, None)
     assert rc == -4 and b"16 query heads" in lib.mi_last_error()
     rc = lib.mi_paged_decode_attention(one, 128, 128, one, one, 128, 128, 128, one, 1, one, one, 128, 128, one,
-                                       1 << 30, 1, 8, 2, 128, 24, 16, 0, 0.1, 0, None, None, None)
+                                       1 << 30, 1, 8, 2, 128, 24, 16, 0, 0.1, 0, None, None, 0, None, None)
     assert rc == -2 and b"multiple of 16" in lib.mi_last_error()
-    assert lib.mi_decode_workspace_bytes(0, 8, 2, 128, 16, 16, 0) == 0
+    # an element type the kernels do not have (fp32 parameters) is refused, not misread
+    rc = lib.mi_paged_decode_attention(one, 128, 128, one, one, 128, 128, 128, one, 1, one, one, 128, 128, one,
+                                       1 << 30, 1, 8, 2, 128, 16, 16, 0, 0.1, 0, None, None, 7, None, None)
+    assert rc == -4 and b"dtype" in lib.mi_last_error()
+    assert lib.mi_decode_workspace_bytes(0, 8, 2, 128, 16, 16, 0, None) == 0
 
 
 @pytest.mark.skipif(torch.cuda.is_available(), reason="this checks the behaviour on a machine without a GPU")

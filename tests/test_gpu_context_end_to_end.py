@@ -18,11 +18,11 @@ pytestmark = pytest.mark.gpu
 L, HQ, HKV, D, C = 2, 8, 2, 128, 16
 
 
-def _make_ctx(mi, dev):
+def _make_ctx(mi, dev, dtype=torch.bfloat16):
     mi.DynamicInferenceContext.TOKEN_ROUNDER = 4
     mi.DynamicInferenceContext.REQUEST_ROUNDER = 4
     return mi.DynamicInferenceContext(
-        params_dtype=torch.bfloat16, num_layers=L, kv_channels=D, num_attention_heads=HKV,
+        params_dtype=dtype, num_layers=L, kv_channels=D, num_attention_heads=HKV,
         max_sequence_length=96, buffer_size_gb=200 * (2 * 2 * L * C * HKV * D) / 1024**3,
         buffer_guaranteed_fraction=0.1, chunk_size_tokens=C, max_requests_override=16, max_tokens_override=256,
         device=dev)
@@ -53,11 +53,14 @@ class Shadow:
         return oa.paged_varlen_attention(qr[:act], self.k[l], self.v[l], ctx.cu_query_seq_lengths.cpu(), lens, bt)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("fused", [True, False])
-def test_prefill_then_decode_steps(mi, dev, fused):
+def test_prefill_then_decode_steps(mi, dev, fused, dtype):
+    """Both 16-bit parameter types of the reference (params_dtype, dynamic_context.py:195,287-308)."""
     saved = (mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER)
     try:
-        ctx = _make_ctx(mi, dev)
+        ctx = _make_ctx(mi, dev, dtype)
+        assert ctx.memory_buffer.dtype == dtype
         shadow = Shadow(ctx)
         gen = torch.Generator().manual_seed(5)
         table = orn.rotary_table(96, D, base=500000.0)
@@ -65,9 +68,9 @@ def test_prefill_then_decode_steps(mi, dev, fused):
         layers = []
         weights = []
         for l in range(L):
-            core = mi.PagedSelfAttentionCore(l + 1, D, qk_norm="rms", eps=1e-5, fused=fused, device=dev)
-            qw = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
-            kw = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+            core = mi.PagedSelfAttentionCore(l + 1, D, qk_norm="rms", eps=1e-5, fused=fused, dtype=dtype, device=dev)
+            qw = (1 + 0.02 * torch.randn(D, generator=gen)).to(dtype)
+            kw = (1 + 0.02 * torch.randn(D, generator=gen)).to(dtype)
             core.q_layernorm_weight.data.copy_(qw)
             core.k_layernorm_weight.data.copy_(kw)
             layers.append(core)
@@ -80,9 +83,9 @@ def test_prefill_then_decode_steps(mi, dev, fused):
             n = ctx.padded_active_token_count
             act = ctx.active_token_count
             for l in range(L):
-                q = torch.randn(n, 1, HQ, D, generator=gen).bfloat16()
-                k = torch.randn(n, 1, HKV, D, generator=gen).bfloat16()
-                v = torch.randn(n, 1, HKV, D, generator=gen).bfloat16()
+                q = torch.randn(n, 1, HQ, D, generator=gen).to(dtype)
+                k = torch.randn(n, 1, HKV, D, generator=gen).to(dtype)
+                v = torch.randn(n, 1, HKV, D, generator=gen).to(dtype)
                 ref = shadow.layer(l, ctx, q, k, v, table, weights[l])
                 out = layers[l](q.to(dev), k.to(dev), v.to(dev), ctx, (table_d, table_d))
                 torch.cuda.synchronize()

@@ -29,13 +29,13 @@ def test_fp8_mixed_prefill_and_decode(mi, dev, Hq, Hkv, chunk, pingpong):
     q, k8, v8, ks, vs, cu_q, lens, bt = _fp8_case(
         mi, dev, n_prefill=3, new_tokens=150, ctx_lo=0, ctx_hi=400, n_decode=5, dec_lo=1, dec_hi=700,
         Hq=Hq, Hkv=Hkv, d=128, chunk=chunk, seed=Hq + Hkv + chunk)
-    mi.ops.set_tuning("prefill_pingpong", pingpong)
+    mi.ops.set_tuning("prefill_two_phase", pingpong)
     try:
         out = mi.ops.paged_prefill_attention(q, k8, v8, cu_q, lens, bt, max_kv_len=int(lens.max()),
                                              k_scales=ks, v_scales=vs)
         torch.cuda.synchronize()
     finally:
-        mi.ops.set_tuning("prefill_pingpong", 1)
+        mi.ops.set_tuning("prefill_two_phase", 0)
     ref = oa.paged_varlen_attention(q.cpu(), k8.cpu(), v8.cpu(), cu_q.cpu(), lens.cpu(), bt.cpu(),
                                     k_scales=ks.cpu(), v_scales=vs.cpu())
     got = out.float().cpu()
@@ -81,7 +81,7 @@ def test_fp8_prefill_rejects_what_it_cannot_run(mi, dev):
         mi.ops.paged_prefill_attention(q, k8, v8, cu_q, lens, bt, k_scales=ks, v_scales=vs)
     with pytest.raises(ValueError, match="scales"):
         mi.ops.paged_prefill_attention(q, k8, v8, cu_q, lens, bt, k_scales=ks)
-    with pytest.raises(ValueError, match="bf16"):
+    with pytest.raises(ValueError, match="16-bit type"):
         mi.ops.paged_prefill_attention(q, k8, v8, cu_q, lens, bt)
 
 

@@ -30,19 +30,19 @@ def _check(mi, dev, q, cache, lens, bt, scale):
     return out
 
 
-@pytest.fixture(params=[1, 0], ids=["lds_tile", "streaming"])
+@pytest.fixture(params=[0, -1], ids=["lds_tile", "streaming"])
 def kernel_choice(request, mi):
     """Both decode kernels: latent tiles shared through LDS (chunk sizes that are multiples of 64 only;
     other sizes stream either way) and one streaming wavefront per head group."""
-    mi.ops.set_tuning("mla_decode_lds", request.param)
+    mi.ops.set_tuning("mla_decode_lds", request.param)  # 0 = default (the LDS-tile kernel), -1 = never
     yield request.param
-    mi.ops.set_tuning("mla_decode_lds", 1)
+    mi.ops.set_tuning("mla_decode_lds", 0)
 
 
 @pytest.mark.parametrize("Hq", [1, 8, 16, 32, 48, 128])
 @pytest.mark.parametrize("chunk", [16, 64, 256])
 def test_mla_decode_matches_checker(mi, dev, Hq, chunk, kernel_choice):
-    if chunk == 16 and kernel_choice == 0:
+    if chunk == 16 and kernel_choice == -1:
         pytest.skip("chunk 16 always streams")
     lens = [0, 1, 15, 16, 17, chunk - 1, chunk, chunk + 1, 3 * chunk + 5, 700, 0, 2049]
     q, cache, lens, bt = _case(mi, dev, lens, Hq, chunk, seed=Hq + chunk)

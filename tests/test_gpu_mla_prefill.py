@@ -37,7 +37,7 @@ def test_mla_prefill_matches_checker(mi, dev, H, chunk):
     assert (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
 
 
-@pytest.mark.parametrize("pingpong", [0, 1, 2])
+@pytest.mark.parametrize("pingpong", [-1, 1, 2])  # register-only kernel, two-phase, two-phase in lock-step
 @pytest.mark.parametrize("Hq,Hkv", [(8, 8), (8, 2), (16, 1)])
 def test_mla_prefill_kernel_choice_and_grouped_heads(mi, dev, pingpong, Hq, Hkv):
     """The two-phase tile kernel (both wave schedules) and the register kernel, with several query heads
@@ -53,20 +53,20 @@ def test_mla_prefill_kernel_choice_and_grouped_heads(mi, dev, pingpong, Hq, Hkv)
     q = torch.randn(int(cu_q[-1]), Hq, 192, generator=g).bfloat16()
     kc = torch.randn(N, chunk, Hkv, 192, generator=g).bfloat16()
     vc = torch.randn(N, chunk, Hkv, 128, generator=g).bfloat16()
-    mi.ops.set_tuning("prefill_pingpong", pingpong)
+    mi.ops.set_tuning("prefill_two_phase", pingpong)
     try:
         out = mi.ops.paged_prefill_attention_mla(q.to(dev), kc.to(dev), vc.to(dev), cu_q.to(dev), kv_lens.to(dev),
                                                  bt.to(dev), softmax_scale=0.07)
         torch.cuda.synchronize()
     finally:
-        mi.ops.set_tuning("prefill_pingpong", 1)
+        mi.ops.set_tuning("prefill_two_phase", 0)
     ref = oa.paged_varlen_attention(q, kc, vc, cu_q, kv_lens, bt, softmax_scale=0.07)
     got = out.float().cpu()
     err = (got - ref).abs()
     assert torch.isfinite(got).all() and (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
 
 
-@pytest.mark.parametrize("forced", [1, 3, 16])
+@pytest.mark.parametrize("forced", [0, 3, 16])
 def test_mla_prefill_few_rows_over_long_contexts_split_the_keys(mi, dev, forced):
     """A chunk of a prompt over a long history: the keys of a request are cut into ranges (automatic count,
     or forced ones -- also more ranges than short requests have tiles), partials merged by a second kernel."""
@@ -80,7 +80,7 @@ def test_mla_prefill_few_rows_over_long_contexts_split_the_keys(mi, dev, forced)
                                                  bt.to(dev), softmax_scale=0.07, max_kv_len=int(lens.max()))
         torch.cuda.synchronize()
     finally:
-        mi.ops.set_tuning("prefill_kv_split", 1)
+        mi.ops.set_tuning("prefill_kv_split", 0)
     ref = oa.paged_varlen_attention(q, kc, vc, cu_q, lens, bt, softmax_scale=0.07)
     got = out.float().cpu()
     T = q.size(0)

@@ -25,7 +25,7 @@ def _ulp_diff(a, b):
 @pytest.mark.parametrize("norm", [None, "rms", "l2"])
 @pytest.mark.parametrize("interleaved", [False, True])
 @pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64), (128, 96), (64, 32), (128, 40)])
-@pytest.mark.parametrize("vectorised", [1, 0])
+@pytest.mark.parametrize("vectorised", [1, -1])
 def test_norm_rope_matches_unfused_chain(mi, dev, norm, interleaved, d, rot, vectorised):
     """Both kernels: 16 bytes per lane (taken when every rotary partner is a whole number of lanes
     away; rot 40 falls back for half-split pairs by itself) and the element-wise one."""
@@ -33,7 +33,7 @@ def test_norm_rope_matches_unfused_chain(mi, dev, norm, interleaved, d, rot, vec
     try:
         _norm_rope_case(mi, dev, norm, interleaved, d, rot)
     finally:
-        mi.ops.set_tuning("norm_rope_vectorised", 2)
+        mi.ops.set_tuning("norm_rope_vectorised", 0)
 
 
 def _norm_rope_case(mi, dev, norm, interleaved, d, rot):
@@ -117,7 +117,7 @@ def test_fused_append_writes_rotated_key_and_raw_value(mi, dev, mode):
 
 
 @pytest.mark.parametrize("d,hq,hkv", [(128, 32, 8), (128, 8, 8), (64, 12, 4), (128, 5, 1)])
-@pytest.mark.parametrize("vectorised", [1, 0])
+@pytest.mark.parametrize("vectorised", [1, -1])
 @pytest.mark.parametrize("interleaved", [False, True])
 def test_mixed_qkv_input_equals_split_inputs(mi, dev, d, hq, hkv, vectorised, interleaved):
     """Reading the QKV projection's output directly gives the bits the same launch produces from the
@@ -176,7 +176,7 @@ def test_mixed_qkv_input_equals_split_inputs(mi, dev, d, hq, hkv, vectorised, in
             assert (err <= 2e-2 + 2e-2 * ref.float().abs()).all(), f"max err {err.max().item()}"
             assert (_ulp_diff(got, ref) > 0).float().mean().item() < 0.01
     finally:
-        mi.ops.set_tuning("norm_rope_vectorised", 2)
+        mi.ops.set_tuning("norm_rope_vectorised", 0)
 
 
 def test_mixed_qkv_argument_errors(mi, dev):

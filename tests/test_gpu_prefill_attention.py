@@ -25,9 +25,11 @@ def test_mixed_prefill_and_decode(mi, dev, Hq, Hkv, d):
     _check(mi, q, kc, vc, cu_q, lens, bt)
 
 
-@pytest.mark.parametrize("subtiles,lds_rows", [(1, 0), (2, 0), (2, 2), (2, 3), (4, 2), (4, 3)])
-def test_ragged_prefill_lengths(mi, dev, subtiles, lds_rows):
-    """New-token counts around every block boundary, with and without existing context."""
+@pytest.mark.parametrize("subtiles,row_tiles", [(1, 2), (2, 2), (1, 4), (2, 4)])
+def test_ragged_prefill_lengths(mi, dev, subtiles, row_tiles):
+    """New-token counts around every block boundary, with and without existing context, at a chunk size (32) that
+    is no multiple of the 64-key staged tiles: the register-only kernel, 16 or 32 keys per iteration, 32 or 64 rows
+    per wavefront."""
     torch.manual_seed(0)
     q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 500]
     ctx = [0, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0, 40, 7]
@@ -40,13 +42,8 @@ def test_ragged_prefill_lengths(mi, dev, subtiles, lds_rows):
     q = torch.randn(int(cu_q[-1]), Hq, d, generator=gen).bfloat16().to(dev)
     kc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
     vc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
-    mi.ops.set_tuning("prefill_tile_subtiles", subtiles)
-    mi.ops.set_tuning("prefill_lds_row_tiles", lds_rows)  # 0 = register-only kernel
-    try:
+    with mi.ops.tuning(prefill_tile_subtiles=subtiles, prefill_row_tiles=row_tiles):
         _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
-    finally:
-        mi.ops.set_tuning("prefill_tile_subtiles", 4)
-        mi.ops.set_tuning("prefill_lds_row_tiles", 2)
 
 
 def test_prefill_equals_decode_for_single_tokens(mi, dev):
@@ -94,11 +91,11 @@ def test_two_phase_kernel_ragged_lengths(mi, dev, pingpong, chunk, Hq, Hkv, d):
     q = torch.randn(int(cu_q[-1]), Hq, d, generator=gen).bfloat16().to(dev)
     kc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
     vc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
-    mi.ops.set_tuning("prefill_pingpong", pingpong)
+    mi.ops.set_tuning("prefill_two_phase", pingpong)
     try:
         _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
     finally:
-        mi.ops.set_tuning("prefill_pingpong", 1)
+        mi.ops.set_tuning("prefill_two_phase", 0)
 
 
 def test_stale_cache_rows_beyond_the_length_do_not_leak(mi, dev):
@@ -152,10 +149,10 @@ def test_chunked_prefill_is_consistent_at_full_size(mi, dev):
 
 
 @pytest.mark.parametrize("d", [128, 64])
-@pytest.mark.parametrize("forced", [1, 2, 7, 64])
+@pytest.mark.parametrize("forced", [0, 2, 7, 64])
 def test_few_rows_over_long_contexts_split_the_keys(mi, dev, forced, d):
     """A chunk of a prompt (or a short turn) over a long cached context: the tile kernel cuts the keys of
-    every request into ranges (automatic = knob 1, or a forced count), writes partials and merges them.
+    every request into ranges (automatic = knob 0, or a forced count), writes partials and merges them.
     Requests shorter than the number of ranges get empty ranges; one-token requests go the decode way."""
     q_lens = [96, 1, 40, 1, 7]
     ctx = [9000, 4000, 130, 0, 63]
@@ -173,13 +170,13 @@ def test_few_rows_over_long_contexts_split_the_keys(mi, dev, forced, d):
         _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
         split = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev),
                                                max_kv_len=int(kv_lens.max()))
-        mi.ops.set_tuning("prefill_kv_split", 0)
+        mi.ops.set_tuning("prefill_kv_split", -1)
         whole = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev),
                                                max_kv_len=int(kv_lens.max()))
         torch.cuda.synchronize()
         assert (split.float() - whole.float()).abs().max().item() <= 1e-2   # same arithmetic, another summation order
     finally:
-        mi.ops.set_tuning("prefill_kv_split", 1)
+        mi.ops.set_tuning("prefill_kv_split", 0)
 
 
 def test_split_keys_with_padding_rows_and_fp8(mi, dev):
@@ -214,21 +211,17 @@ def test_split_keys_with_padding_rows_and_fp8(mi, dev):
     assert (err8 <= 2.5e-2 + 2.5e-2 * ref8.abs()).all() and (out8[53:] == 0).all()
 
 
-@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_no_offset", "lock_step", "lock_step_48_rows", "registers",
-                                    "registers_64_rows", "split_keys"])
+@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_no_offset", "registers", "registers_64_rows", "split_keys"])
 @pytest.mark.parametrize("Hq,Hkv", [(12, 4), (10, 2), (28, 4), (6, 1), (12, 1), (15, 1)])
 @pytest.mark.parametrize("d", [128, 64])
 def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, d):
     """3, 5, 6, 7, 12 or 15 query heads per KV head (Llama-3.2-3B, Qwen2.5-14B, Qwen2-7B ... have such groups):
-    a wavefront's 32 (48) rows then hold as many whole tokens as fit, the rest are padding rows.  Every
+    a wavefront's 32 (64) rows then hold as many whole tokens as fit, the rest are padding rows.  Every
     prefill kernel, lengths either side of the per-workgroup token counts (48 tokens at a group of 5)."""
-    knobs = {"two_phase": {}, "two_phase_no_offset": {"prefill_pingpong": 2}, "lock_step": {"prefill_pingpong": 0},
-             "lock_step_48_rows": {"prefill_pingpong": 0, "prefill_lds_row_tiles": 3},
-             "registers": {"prefill_lds_row_tiles": 0},
-             "registers_64_rows": {"prefill_lds_row_tiles": 0, "prefill_row_tiles": 4},
+    knobs = {"two_phase": {}, "two_phase_no_offset": {"prefill_two_phase": 2},
+             "registers": {"prefill_two_phase": -1},
+             "registers_64_rows": {"prefill_two_phase": -1, "prefill_row_tiles": 4},
              "split_keys": {"prefill_kv_split": 3}}[kernel]
-    if d == 64 and kernel.startswith("lock_step"):
-        pytest.skip("the lock-step LDS kernel is head_dim 128 only")
     G = Hq // Hkv
     per_wg = 8 * (32 // G)
     q_lens = [1, per_wg - 1, per_wg, per_wg + 1, 2 * per_wg + 3, 1, 301, 5]
@@ -241,15 +234,9 @@ def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, 
     q = torch.randn(int(cu_q[-1]) + 3, Hq, d, generator=gen).bfloat16().to(dev)   # three padding rows
     kc = torch.randn(N, 64, Hkv, d, generator=gen).bfloat16().to(dev)
     vc = torch.randn(N, 64, Hkv, d, generator=gen).bfloat16().to(dev)
-    for name, value in knobs.items():
-        mi.ops.set_tuning(name, value)
-    try:
+    with mi.ops.tuning(**knobs):
         out = mi.ops.paged_prefill_attention(q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev), max_kv_len=int(kv_lens.max()))
         torch.cuda.synchronize()
-    finally:
-        for name, value in {"prefill_pingpong": 1, "prefill_lds_row_tiles": 2, "prefill_kv_split": 1,
-                            "prefill_row_tiles": 2}.items():
-            mi.ops.set_tuning(name, value)
     T = int(cu_q[-1])
     ref = oa.paged_varlen_attention(q[:T].cpu(), kc.cpu(), vc.cpu(), cu_q, kv_lens, bt)
     got = out.float().cpu()

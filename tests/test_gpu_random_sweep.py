@@ -120,7 +120,7 @@ def case_decode(mi, dev, rng, seed, fp8):
     finally:
         mi.ops.set_tuning("decode_grid", 0)
         mi.ops.set_tuning("decode_tile_subtiles", 0)
-        mi.ops.set_tuning("decode_waves_per_block", 8)
+        mi.ops.set_tuning("decode_waves_per_block", 0)
 
 
 def case_prefill(mi, dev, rng, seed, fp8):
@@ -145,8 +145,8 @@ def case_prefill(mi, dev, rng, seed, fp8):
             ctx.append(rng.choice([0, 0, 5, chunk - 1, chunk, rng.randint(0, 700)]))
     if sum(q_lens) == 0:
         q_lens[0] = 3
-    pp = rng.choice([1, 1, 2, 0])
-    ksplit = rng.choice([1, 1, 0, 3, 8])  # key ranges per request in the tile kernel (1 = automatic)
+    pp = rng.choice([0, 0, 2, -1])  # two-phase tile kernel (default), the same in lock-step, register-only kernel
+    ksplit = rng.choice([0, 0, -1, 3, 8])  # key ranges per request in the tile kernel (0 = automatic, -1 = never)
     _note(f"prefill fp8={fp8} seed={seed} d={d} Hq={Hq} Hkv={Hkv} chunk={chunk} q_lens={q_lens} ctx={ctx} pingpong={pp} "
           f"kv_split={ksplit}")
     kv_lens = torch.tensor([a + b if a else 0 for a, b in zip(q_lens, ctx)], dtype=torch.int32)
@@ -157,7 +157,7 @@ def case_prefill(mi, dev, rng, seed, fp8):
     q = (torch.randn(T, Hq, d, generator=gen)).bfloat16()
     kc = (torch.randn(N + 1, chunk, Hkv, d, generator=gen) * 0.7).bfloat16()
     vc = (torch.randn(N + 1, chunk, Hkv, d, generator=gen) * 0.7).bfloat16()
-    mi.ops.set_tuning("prefill_pingpong", pp)
+    mi.ops.set_tuning("prefill_two_phase", pp)
     mi.ops.set_tuning("prefill_kv_split", ksplit)
     try:
         if fp8:
@@ -182,8 +182,8 @@ def case_prefill(mi, dev, rng, seed, fp8):
             ref = oa.paged_varlen_attention(q, kc, vc, cu_q, kv_lens, bt)
             close(out, ref, 2e-2, "prefill")
     finally:
-        mi.ops.set_tuning("prefill_pingpong", 1)
-        mi.ops.set_tuning("prefill_kv_split", 1)
+        mi.ops.set_tuning("prefill_two_phase", 0)
+        mi.ops.set_tuning("prefill_kv_split", 0)
 
 
 def case_mla_decode(mi, dev, rng, seed):
@@ -193,7 +193,7 @@ def case_mla_decode(mi, dev, rng, seed):
     R = rng.randint(1, 12)
     lens = rand_lens(rng, R, chunk, 1200)
     grid = rng.choice([0, 0, 1, 5, 41])
-    lds = rng.choice([1, 1, 0])
+    lds = rng.choice([0, 0, -1])
     _note(f"mla_decode seed={seed} Hq={Hq} chunk={chunk} lens={lens} grid={grid} lds={lds}")
     lens_t = torch.tensor(lens, dtype=torch.int32)
     bt, N = mi.synthetic.build_block_table(lens_t, chunk, gen)
@@ -208,7 +208,7 @@ def case_mla_decode(mi, dev, rng, seed):
         torch.cuda.synchronize()
     finally:
         mi.ops.set_tuning("decode_grid", 0)
-        mi.ops.set_tuning("mla_decode_lds", 1)
+        mi.ops.set_tuning("mla_decode_lds", 0)
     ref = oa.mla_decode_attention(q.squeeze(1), cache, lens_t, bt, 0.07, 512)
     close(out.squeeze(1), ref, 2e-2, "mla decode")
 
@@ -235,8 +235,8 @@ def case_mla_prefill(mi, dev, rng, seed):
             ctx.append(rng.choice([0, 0, 5, chunk - 1, chunk, rng.randint(0, 700)]))
     if sum(q_lens) == 0:
         q_lens[0] = 5
-    pp = rng.choice([1, 1, 2, 0])
-    ksplit = rng.choice([1, 1, 0, 3, 8])
+    pp = rng.choice([0, 0, 2, -1])  # two-phase tile kernel (default), the same in lock-step, register-only kernel
+    ksplit = rng.choice([0, 0, -1, 3, 8])
     joint = rng.random() < 0.4
     _note(f"mla_prefill seed={seed} Hq={Hkv * G} Hkv={Hkv} chunk={chunk} q_lens={q_lens} ctx={ctx} pingpong={pp} joint={joint}")
     kv_lens = torch.tensor([a + b if a else 0 for a, b in zip(q_lens, ctx)], dtype=torch.int32)
@@ -251,7 +251,7 @@ def case_mla_prefill(mi, dev, rng, seed):
         kd_, vd_ = both[..., :192], both[..., 192:]
     else:
         kd_, vd_ = kc.to(dev), vc.to(dev)
-    mi.ops.set_tuning("prefill_pingpong", pp)
+    mi.ops.set_tuning("prefill_two_phase", pp)
     mi.ops.set_tuning("prefill_kv_split", ksplit)
     try:
         qd_ = q.to(dev)
@@ -259,8 +259,8 @@ def case_mla_prefill(mi, dev, rng, seed):
         out = mi.ops.paged_prefill_attention_mla(qd_, kd_, vd_, cu_q.to(dev), kv_lens.to(dev), bt.to(dev), softmax_scale=0.08)
         torch.cuda.synchronize()
     finally:
-        mi.ops.set_tuning("prefill_pingpong", 1)
-        mi.ops.set_tuning("prefill_kv_split", 1)
+        mi.ops.set_tuning("prefill_two_phase", 0)
+        mi.ops.set_tuning("prefill_kv_split", 0)
     ref = oa.paged_varlen_attention(q, kc, vc, cu_q, kv_lens, bt, softmax_scale=0.08)
     close(out, ref, 2e-2, "mla prefill")
 
@@ -376,7 +376,7 @@ def case_norm_rope(mi, dev, rng, seed):
     Hq = Hkv * rng.choice([1, 2, 3, 4, 5, 7])
     norm = rng.choice([None, "rms", "l2"])
     interleaved = rng.random() < 0.3
-    vec = rng.choice([0, 1, 2])
+    vec = rng.choice([-1, 1, 0])
     mixed = rng.random() < 0.5
     q_lens, ctx, cu_q, kv_lens, bt, N, pos, ci, lo = mixed_batch(mi, rng, gen, chunk)
     _note(f"norm_rope seed={seed} chunk={chunk} d={d} rot={rot} Hq={Hq} Hkv={Hkv} norm={norm} il={interleaved} "
@@ -414,7 +414,7 @@ def case_norm_rope(mi, dev, rng, seed):
                                     token_to_chunk_idx=ci.to(dev), token_to_local_pos=lo.to(dev))
         torch.cuda.synchronize()
     finally:
-        mi.ops.set_tuning("norm_rope_vectorised", 2)
+        mi.ops.set_tuning("norm_rope_vectorised", 0)
     got_q = q_out.cpu().view(T, Hq, d)
     err = (got_q.float() - q_ref.float()).abs()
     assert torch.isfinite(got_q.float()).all()

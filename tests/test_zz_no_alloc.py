@@ -29,6 +29,7 @@ def _args(case, out):
     tail = [R, Hq, kc.size(2), D, kc.size(1), case.block_table.size(1) * kc.size(1), 0, float(D) ** -0.5,
             1 if fp8 else 0,
             case.k_scales.data_ptr() if fp8 else None, case.v_scales.data_ptr() if fp8 else None,
+            1 if q3.dtype == torch.float16 else 0, None,   # element type, knobs (NULL = defaults)
             torch.cuda.current_stream().cuda_stream]
     return head, tail
 
@@ -36,7 +37,7 @@ def _args(case, out):
 def _with_workspace(lib, case):
     out = torch.full_like(case.q, float("nan"))
     head, tail = _args(case, out)
-    need = lib.mi_decode_workspace_bytes(*tail[:6], 0)
+    need = lib.mi_decode_workspace_bytes(*tail[:6], 0, None)
     ws = torch.empty(need, dtype=torch.uint8, device=case.q.device)
     rc = lib.mi_paged_decode_attention(*head, ws.data_ptr(), need, *tail)
     assert rc == 0, lib.mi_last_error()
@@ -106,8 +107,8 @@ def test_sizes_beyond_the_scratch_are_rejected(mi, dev):
     """A problem whose partials do not fit the built-in scratch is refused with a message, nothing is launched."""
     lib = mi._lib.load()
     R, Hq, Hkv, D = 2048, 64, 8, 128
-    assert lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, 256, 4096, 0) > SCRATCH_BYTES
+    assert lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, 256, 4096, 0, None) > SCRATCH_BYTES
     one = ctypes.c_void_p(256)
     rc = lib.mi_paged_decode_attention_noalloc(one, Hq * D, D, one, one, 256 * Hkv * D, Hkv * D, D, one, 16, one, one,
-                                               Hq * D, D, R, Hq, Hkv, D, 256, 4096, 0, 0.1, 0, None, None, None)
+                                               Hq * D, D, R, Hq, Hkv, D, 256, 4096, 0, 0.1, 0, None, None, 0, None, None)
     assert rc == -5 and b"16 MiB" in lib.mi_last_error()
