@@ -21,7 +21,7 @@ int mi_check_launch(const char* where);
 bool mi_profile_next(hipEvent_t* start, hipEvent_t* stop);
 
 namespace mi {
-int decode_grid_size(int Hkv, const MiTuning& tune);
+int decode_grid_size(int Hq, int Hkv, const MiTuning& tune);
 // Shared by the decode entry point and by the mixed-batch path of the prefill entry point
 // (cu_seqlens_q non-null: only requests with one query row take part, at row cu_seqlens_q[r]).
 int launch_paged_decode(const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,

@@ -138,6 +138,68 @@ static __device__ __forceinline__ uint2 ld8_stream(const void* p) {
   const u32x2_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
   return make_uint2(v.x, v.y);
 }
+// N consecutive dwords read once from global memory into registers.  The address is aligned to the largest
+// power of two that divides 4 N (at most 16): 12 bytes (N = 3) sit at any multiple of 4, so that load is declared
+// with 4-byte alignment and the compiler picks an encoding the alignment allows.
+typedef uint32_t u32x3a4_t __attribute__((ext_vector_type(3), aligned(4)));
+template <int N>
+static __device__ __forceinline__ void ld_dwords_stream(const void* p, uint32_t (&dst)[N]) {
+  static_assert(N == 3 || N % 2 == 0, "dword counts of the value fragments");
+  if constexpr (N % 4 == 0) {
+#pragma unroll
+    for (int w = 0; w < N / 4; ++w) {
+      const uint4 v = ld16_stream(reinterpret_cast<const uint8_t*>(p) + 16 * w);
+      dst[4 * w] = v.x; dst[4 * w + 1] = v.y; dst[4 * w + 2] = v.z; dst[4 * w + 3] = v.w;
+    }
+  } else if constexpr (N % 2 == 0) {
+#pragma unroll
+    for (int w = 0; w < N / 2; ++w) {
+      const uint2 v = ld8_stream(reinterpret_cast<const uint8_t*>(p) + 8 * w);
+      dst[2 * w] = v.x; dst[2 * w + 1] = v.y;
+    }
+  } else {
+    const u32x3a4_t v = __builtin_nontemporal_load(reinterpret_cast<const u32x3a4_t*>(p));
+    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z;
+  }
+}
+template <int N>
+static __device__ __forceinline__ void ld_dwords(const void* p, uint32_t (&dst)[N]) {  // the cacheable form
+  static_assert(N == 3 || N % 2 == 0, "dword counts of the value fragments");
+  if constexpr (N % 4 == 0) {
+#pragma unroll
+    for (int w = 0; w < N / 4; ++w) {
+      const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(p) + 16 * w);
+      dst[4 * w] = v.x; dst[4 * w + 1] = v.y; dst[4 * w + 2] = v.z; dst[4 * w + 3] = v.w;
+    }
+  } else if constexpr (N % 2 == 0) {
+#pragma unroll
+    for (int w = 0; w < N / 2; ++w) {
+      const uint2 v = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint8_t*>(p) + 8 * w);
+      dst[2 * w] = v.x; dst[2 * w + 1] = v.y;
+    }
+  } else {
+    const u32x3a4_t v = *reinterpret_cast<const u32x3a4_t*>(p);
+    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z;
+  }
+}
+// N consecutive dwords written from registers, same alignment rule.
+template <int N>
+static __device__ __forceinline__ void st_dwords(void* p, const uint32_t (&src)[N]) {
+  static_assert(N == 3 || N % 2 == 0, "dword counts of the output fragments");
+  if constexpr (N % 4 == 0) {
+#pragma unroll
+    for (int w = 0; w < N / 4; ++w)
+      *reinterpret_cast<uint4*>(reinterpret_cast<uint8_t*>(p) + 16 * w) =
+          make_uint4(src[4 * w], src[4 * w + 1], src[4 * w + 2], src[4 * w + 3]);
+  } else if constexpr (N % 2 == 0) {
+#pragma unroll
+    for (int w = 0; w < N / 2; ++w)
+      *reinterpret_cast<uint2*>(reinterpret_cast<uint8_t*>(p) + 8 * w) = make_uint2(src[2 * w], src[2 * w + 1]);
+  } else {
+    u32x3a4_t v = {src[0], src[1], src[2]};
+    *reinterpret_cast<u32x3a4_t*>(p) = v;
+  }
+}
 static __device__ __forceinline__ void st16(void* p, uint4 v) { *reinterpret_cast<uint4*>(p) = v; }
 static __device__ __forceinline__ void st8(void* p, uint2 v) { *reinterpret_cast<uint2*>(p) = v; }
 

@@ -17,10 +17,10 @@
 // so the result equals the op-by-op evaluation in that type; with `faithful == 0` the
 // whole expression is evaluated in fp32 and rounded once.
 //
-// grid = (tokens, groups of head vectors); a workgroup of 4 waves handles 4 (d = 128) or 8
-// (d = 64) head vectors of one token per pass, each by d/2 lanes, lane i owning elements i and
-// i + d/2.  The normalised vector goes through a few hundred bytes of LDS so that any rotary
-// pairing (half-split, interleaved, partial rotary width) reads its partner from there.
+// grid = (tokens, groups of head vectors); a workgroup of 4 waves handles 4 (d = 128, 192, 256) or 8
+// (d = 64, 96) head vectors of one token per pass, each by 64 or 32 lanes, lane i owning elements i,
+// i + lanes, ... (two, three or four of them).  The normalised vector goes through a few hundred bytes of
+// LDS so that any rotary pairing (half-split, interleaved, partial rotary width) reads its partner from there.
 #include <stdio.h>
 
 #include "mi_common.h"
@@ -73,9 +73,11 @@ static __device__ __forceinline__ const uint16_t* head_vector(const NormRopePara
 
 template <int D, bool F16>
 __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p) {
-  constexpr int LPV = D / 2;        // lanes per head vector
+  constexpr int LPV = D >= 128 ? 64 : 32;  // lanes per head vector
+  constexpr int EPL = D / LPV;             // elements per lane: i, i + LPV, ...
   constexpr int VPW = 64 / LPV;     // head vectors per wave
   constexpr int VPB = 4 * VPW;      // head vectors per workgroup pass
+  static_assert(EPL * LPV == D && EPL >= 2 && EPL <= 4, "head widths 64, 96, 128, 192, 256");
   __shared__ float lds[VPB][D];
 
   const int t = blockIdx.x;
@@ -100,17 +102,17 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
     }
   }
 
-  // cos / sin of this lane's two elements depend only on the token position, not on the head:
+  // cos / sin of this lane's elements depend only on the token position, not on the head:
   // evaluate them once (twice if query and key positions differ) and reuse them for every head.
-  float cs[2][2][2] = {};  // [q|k][element][cos|sin]
-  int partner[2] = {0, 0};
-  float sign[2] = {0.f, 0.f};
-  bool rotate[2] = {false, false};
+  float cs[2][EPL][2] = {};  // [q|k][element][cos|sin]
+  int partner[EPL] = {};
+  float sign[EPL] = {};
+  bool rotate[EPL] = {};
   if (p.emb) {
     const int64_t qp = p.q_pos ? p.q_pos[t] : 0;
     const int64_t kp = p.k_pos ? p.k_pos[t] : qp;
 #pragma unroll
-    for (int w = 0; w < 2; ++w) {
+    for (int w = 0; w < EPL; ++w) {
       const int e = i + w * LPV;
       rotate[w] = e < p.rot;
       if (p.interleaved) {
@@ -148,64 +150,54 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
     const bool active = vec < nvec;
     const bool is_q = vec < p.Hq;
     const int head = is_q ? vec : vec - p.Hq;
-    float x0 = 0.f, x1 = 0.f;
+    float y[EPL] = {};
     if (active) {
       const uint16_t* src = head_vector(p, t, vec);
-      x0 = to_f32<F16>(src[i]);
-      x1 = to_f32<F16>(src[i + LPV]);
+#pragma unroll
+      for (int w = 0; w < EPL; ++w) y[w] = to_f32<F16>(src[i + w * LPV]);
     }
-    float y0 = x0, y1 = x1;
     if (p.norm != MI_NORM_NONE) {
-      float ss = x0 * x0 + x1 * x1;
+      float ss = y[0] * y[0] + y[1] * y[1];
+#pragma unroll
+      for (int w = 2; w < EPL; ++w) ss += y[w] * y[w];
 #pragma unroll
       for (int o = LPV / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
       const float rstd = rsqrtf(ss * (1.f / D) + p.eps);
-      y0 = x0 * rstd;
-      y1 = x1 * rstd;
-      const uint16_t* w = is_q ? p.q_w : p.k_w;
-      if (p.norm == MI_NORM_RMS && w) {
-        y0 *= to_f32<F16>(w[i]);
-        y1 *= to_f32<F16>(w[i + LPV]);
-      }
-      if (faithful) {
-        y0 = round16<F16>(y0);
-        y1 = round16<F16>(y1);
+      const uint16_t* wt = is_q ? p.q_w : p.k_w;
+#pragma unroll
+      for (int w = 0; w < EPL; ++w) {
+        y[w] *= rstd;
+        if (p.norm == MI_NORM_RMS && wt) y[w] *= to_f32<F16>(wt[i + w * LPV]);
+        if (faithful) y[w] = round16<F16>(y[w]);
       }
     }
-    float o0 = y0, o1 = y1;
+    float o[EPL];
+#pragma unroll
+    for (int w = 0; w < EPL; ++w) o[w] = y[w];
     if (p.emb) {
-      lds[slot][i] = y0;
-      lds[slot][i + LPV] = y1;
+#pragma unroll
+      for (int w = 0; w < EPL; ++w) lds[slot][i + w * LPV] = y[w];
       __syncthreads();
 #pragma unroll
-      for (int w = 0; w < 2; ++w) {
+      for (int w = 0; w < EPL; ++w) {
         if (active && rotate[w]) {
-          const float y = w ? y1 : y0;
           const float c = cs[is_q ? 0 : 1][w][0], sn = cs[is_q ? 0 : 1][w][1];
           const float yp = lds[slot][partner[w]] * sign[w];
-          const float out = faithful ? round16<F16>(y * c) + round16<F16>(yp * sn) : y * c + yp * sn;
-          if (w) o1 = out; else o0 = out;
+          o[w] = faithful ? round16<F16>(y[w] * c) + round16<F16>(yp * sn) : y[w] * c + yp * sn;
         }
       }
       __syncthreads();
     }
     if (active) {
-      const uint16_t b0 = f32_to_16<F16>(o0), b1 = f32_to_16<F16>(o1);
-      if (is_q) {
-        uint16_t* dst = p.q_out + (int64_t)t * p.qo_st + (int64_t)head * D;
-        dst[i] = b0;
-        dst[i + LPV] = b1;
-      } else {
-        if (p.k_out) {
-          uint16_t* dst = p.k_out + (int64_t)t * p.ko_st + (int64_t)head * D;
-          dst[i] = b0;
-          dst[i + LPV] = b1;
-        }
-        if (cache_off >= 0) {
-          uint16_t* dst = p.kc + cache_off + (int64_t)head * D;
-          dst[i] = b0;
-          dst[i + LPV] = b1;
-        }
+      uint16_t* dst_q = is_q ? p.q_out + (int64_t)t * p.qo_st + (int64_t)head * D : nullptr;
+      uint16_t* dst_k = (!is_q && p.k_out) ? p.k_out + (int64_t)t * p.ko_st + (int64_t)head * D : nullptr;
+      uint16_t* dst_c = (!is_q && cache_off >= 0) ? p.kc + cache_off + (int64_t)head * D : nullptr;
+#pragma unroll
+      for (int w = 0; w < EPL; ++w) {
+        const uint16_t b = f32_to_16<F16>(o[w]);
+        if (dst_q) dst_q[i + w * LPV] = b;
+        if (dst_k) dst_k[i + w * LPV] = b;
+        if (dst_c) dst_c[i + w * LPV] = b;
       }
     }
   }
@@ -224,7 +216,8 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
 // load / store) each.  The rotary partner of an element is in the same lane (interleaved pairs) or
 // one lane shuffle away (half-split pairs, when rot/2 is a multiple of 8).  Same rounding points as
 // norm_rope_append_kernel; only the order of the sum of squares differs.  grid = (tokens, groups of
-// head vectors) as above, 16 (d = 128) or 32 (d = 64) head vectors per workgroup pass.
+// head vectors) as above, 16 (d = 128, 96), 32 (d = 64) or 8 (d = 192, 256) head vectors per workgroup pass;
+// at d = 96 and 192 a vector's 12 / 24 lanes sit in a group of 16 / 32 whose other lanes idle.
 //
 // A token's work starts with a chain of dependent loads (position -> angle row -> cos / sin), so
 // the kernel is latency-bound unless enough workgroups are resident and independent loads are in
@@ -233,19 +226,21 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
 // SIMD).  Each angle's cos or sin is evaluated by exactly one thread of the workgroup.
 template <int D, bool F16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void norm_rope_append_vec_kernel(NormRopeParams p) {
-  constexpr int LPV = D / 8;        // lanes per head vector
-  constexpr int VPW = 64 / LPV;     // head vectors per wave
+  constexpr int LPV = D / 8;        // lanes that hold a head vector
+  constexpr int LPG = LPV <= 8 ? 8 : LPV <= 16 ? 16 : 32;  // lane group of a head vector (a power of two)
+  constexpr int VPW = 64 / LPG;     // head vectors per wave
   constexpr int VPB = 4 * VPW;      // head vectors per workgroup pass
   const int t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int li = lane % LPV;
-  const int slot = wave * VPW + lane / LPV;
+  const int li = lane % LPG;
+  const bool lane_on = LPG == LPV || li < LPV;
+  const int slot = wave * VPW + lane / LPG;
   const int nvec = p.Hq + p.Hkv;
   const bool faithful = p.faithful != 0;
-  const int e0 = 8 * li;  // first element of this lane
+  const int e0 = lane_on ? 8 * li : 0;  // first element of this lane (idle lanes read what lane 0 reads)
 
   auto load_vec = [&](int vec) -> uint4 {
-    if (vec >= nvec) return make_uint4(0, 0, 0, 0);
+    if (vec >= nvec || !lane_on) return make_uint4(0, 0, 0, 0);
     return ld16(head_vector(p, t, vec) + e0);
   };
   // Independent of the position chain: first head vector, value row (first workgroup of the token).
@@ -337,7 +332,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
 #pragma unroll
       for (int j = 0; j < 8; ++j) ss += y[j] * y[j];
 #pragma unroll
-      for (int o = LPV / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      for (int o = LPG / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
       const float rstd = rsqrtf(ss * (1.f / D) + p.eps);
       const uint4 wr = is_q ? wq_raw : wk_raw;
       const uint32_t w4[4] = {wr.x, wr.y, wr.z, wr.w};
@@ -370,7 +365,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
         if (e0 + j < p.rot) o[j] = faithful ? round16<F16>(y[j] * c[j]) + round16<F16>(yp * sn[j]) : y[j] * c[j] + yp * sn[j];
       }
     }
-    if (active) {
+    if (active && lane_on) {
       const uint4 packed = make_uint4(pack2<F16>(o[0], o[1]), pack2<F16>(o[2], o[3]),
                                       pack2<F16>(o[4], o[5]), pack2<F16>(o[6], o[7]));
       if (is_q) {
@@ -405,7 +400,8 @@ int norm_rope_launch(NormRopeParams& p, int32_t dtype, const MiTuning* tuning, h
   const bool f16 = dtype == MI_DTYPE_FP16;
   if (p.T < 0 || p.Hq < 0 || p.Hkv < 0 || p.Hq + p.Hkv == 0) return fail(MI_ERR_SHAPE, "bad sizes");
   if ((p.Hq > 0 && (!p.q || !p.q_out)) || (p.Hkv > 0 && !p.k)) return fail(MI_ERR_NULL, "q / q_out / k missing");
-  if (p.d != 64 && p.d != 128) return fail(MI_ERR_UNSUPPORTED, "head_dim must be 64 or 128");
+  if (p.d != 64 && p.d != 96 && p.d != 128 && p.d != 192 && p.d != 256)
+    return fail(MI_ERR_UNSUPPORTED, "head_dim must be 64, 96, 128, 192 or 256");
   if (p.norm != MI_NORM_NONE && p.norm != MI_NORM_RMS && p.norm != MI_NORM_L2)
     return fail(MI_ERR_UNSUPPORTED, "unknown norm kind");
   if (p.emb) {
@@ -436,7 +432,8 @@ int norm_rope_launch(NormRopeParams& p, int32_t dtype, const MiTuning* tuning, h
   // element-wise kernel's shorter dependent chain does (4.8 against 5.7 us at 64 tokens).
   const int mode = tune.norm_rope_vectorised;  // -1 never, 1 whenever the shapes allow, 2 automatic
   const bool vec = rot_ok && (ptrs & 15) == 0 && (strides & 7) == 0 && (mode == 1 || (mode == 2 && p.T >= 256));
-  const int vpb = vec ? (p.d == 128 ? 16 : 32) : (p.d == 128 ? 4 : 8);
+  // head vectors per workgroup pass (see the kernels)
+  const int vpb = vec ? (p.d == 64 ? 32 : p.d <= 128 ? 16 : 8) : (p.d >= 128 ? 4 : 8);
   const int passes = (p.Hq + p.Hkv + vpb - 1) / vpb;
   int gy = (2048 + p.T - 1) / p.T;
   gy = gy < 1 ? 1 : (gy > passes ? passes : gy);
@@ -445,8 +442,14 @@ int norm_rope_launch(NormRopeParams& p, int32_t dtype, const MiTuning* tuning, h
   do {                                                                                          \
     if (p.d == 128 && f16) hipLaunchKernelGGL((KERNEL_<128, true>), grid, dim3(256), 0, st, p);   \
     else if (p.d == 128) hipLaunchKernelGGL((KERNEL_<128, false>), grid, dim3(256), 0, st, p);    \
-    else if (f16) hipLaunchKernelGGL((KERNEL_<64, true>), grid, dim3(256), 0, st, p);             \
-    else hipLaunchKernelGGL((KERNEL_<64, false>), grid, dim3(256), 0, st, p);                     \
+    else if (p.d == 64 && f16) hipLaunchKernelGGL((KERNEL_<64, true>), grid, dim3(256), 0, st, p);  \
+    else if (p.d == 64) hipLaunchKernelGGL((KERNEL_<64, false>), grid, dim3(256), 0, st, p);      \
+    else if (p.d == 96 && f16) hipLaunchKernelGGL((KERNEL_<96, true>), grid, dim3(256), 0, st, p);  \
+    else if (p.d == 96) hipLaunchKernelGGL((KERNEL_<96, false>), grid, dim3(256), 0, st, p);      \
+    else if (p.d == 192 && f16) hipLaunchKernelGGL((KERNEL_<192, true>), grid, dim3(256), 0, st, p); \
+    else if (p.d == 192) hipLaunchKernelGGL((KERNEL_<192, false>), grid, dim3(256), 0, st, p);    \
+    else if (f16) hipLaunchKernelGGL((KERNEL_<256, true>), grid, dim3(256), 0, st, p);            \
+    else hipLaunchKernelGGL((KERNEL_<256, false>), grid, dim3(256), 0, st, p);                    \
   } while (0)
   if (vec) MI_NR_LAUNCH(norm_rope_append_vec_kernel);
   else MI_NR_LAUNCH(norm_rope_append_kernel);

@@ -63,6 +63,7 @@ struct DecodeParams {
   const float* v_scale;
   uint64_t chunk_magic;  // ceil(2^40 / chunk)
   int32_t R, Hq, Hkv, G, chunk, min_span_tiles, grid;
+  int32_t parts;  // wavefronts per KV head: each takes up to 16 of the G query heads that share it
   float scale_log2;
 };
 
@@ -71,27 +72,28 @@ static __device__ __forceinline__ int chunk_of(int tok, uint64_t magic) {
   return (int)(((uint64_t)(uint32_t)tok * magic) >> 40);
 }
 
-// One segment: tokens [start, end) of request r for KV head h (one wavefront).
-// `whole` = the segment is the entire request (write bf16 output, no partial).
+// One segment: tokens [start, end) of request r for KV head h (one wavefront) and the `gq` <= 16 query heads
+// hq0 .. hq0 + gq - 1 that share it.  `whole` = the segment is the entire request (write the 16-bit output, no
+// partial).
 // HDK = width of the keys (and queries), HDV = width of the values (and of the output).  They differ
 // only for the latent cache of multi-latent attention (576 / 512: the value is the first 512 of the
 // shared 576-wide row, the caller points both cache arguments at the same buffer).
 template <int HDK, int HDV, int NT, bool FP8, bool F16>
-static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int row, int h, int len,
-                                                      int start, int end, bool whole, int slot, int lane,
+static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int row, int h, int hq0, int gq,
+                                                      int len, int start, int end, bool whole, int slot, int lane,
                                                       uint8_t* q_lds) {
   constexpr int KS = HDK / 32;
   // Wide keys (the 576-wide latent rows): the query fragments would take 72 registers per lane next
   // to 128 accumulator registers, so they live in this wavefront's piece of LDS instead (16 rows with
   // a pitch that spreads the 16 rows of a fragment read over all banks).
-  constexpr bool Q_IN_LDS = HDK > 128;
+  constexpr bool Q_IN_LDS = HDK > 256;
   // The latent rows are read twice (as keys, then their first part as values) and by every query
   // group: those loads stay cacheable; an ordinary KV cache is read exactly once and streams past.
   constexpr bool SHARED_KV = HDK != HDV;
   constexpr int kQPitch = HDK * 2 + 16;
   constexpr int DV = HDV / 16;
-  constexpr int VW = DV * (FP8 ? 1 : 2) / 16;  // 16-byte loads per token and lane of the value operand (0: 8 bytes)
-  static_assert((HDK == 64 || HDK == 128 || HDK == 576) && (HDV == 64 || HDV == 128 || HDV == 512), "head widths");
+  constexpr int VD = FP8 ? 2 : DV / 2;  // dwords per token and lane of the value operand
+  static_assert(HDK % 32 == 0 && HDV % 32 == 0 && HDK >= 64 && HDV >= 64, "head widths: multiples of 32");
   static_assert(!FP8 || (HDK == 128 && HDV == 128 && !F16), "fp8 KV: head_dim 128, bf16 queries");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
@@ -103,8 +105,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   end = __builtin_amdgcn_readfirstlane(end);
   slot = __builtin_amdgcn_readfirstlane(slot);
   const int m16 = lane & 15, g = lane >> 4;
-  const int G = p.G;
-  const int hq = h * G + m16;  // query head of this lane's row (valid when m16 < G)
+  const int G = gq;
+  const int hq = hq0 + m16;  // query head of this lane's row (valid when m16 < G)
   // Loads are clamped to the last token of this segment (not of the request): the software
   // pipeline requests one tile past the end, and that tile belongs to another workgroup's span --
   // clamped, the request degenerates to re-reading one row instead of streaming 2 tiles from HBM.
@@ -148,8 +150,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   // scores of the current one exist, V of the next tile as soon as the current P.V is done,
   // so every wave keeps loads in flight while it computes.
   uint4 kf[NT][FP8 ? KS / 2 : KS];
-  uint4 vf16[NT][4][VW > 0 ? VW : 1];  // bf16, value width 128 (512): 16 (64) bytes per token and lane
-  uint2 vf8[NT][4];                    // bf16 width 64 or fp8 width 128: 8 bytes per token and lane
+  uint32_t vf[NT][4][VD];  // 16-bit cache: HDV / 8 bytes per token and lane; fp8 (width 128): 8 bytes
   float ksc_tile = 1.f, vsc_tile = 1.f;  // fp8: scales of the chunk the staged K / V tile lies in
 
   // Addressing.  A tile of 16*NT tokens never straddles a chunk (the launcher picks NT so that the
@@ -251,12 +252,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint8_t* vrow = tile + min(v_lane[j], cap);
-        if (VW > 0) {
-#pragma unroll
-          for (int w = 0; w < VW; ++w) vf16[u][j][w] = SHARED_KV ? ld16(vrow + 16 * w) : ld16_stream(vrow + 16 * w);
-        } else {
-          vf8[u][j] = ld8_stream(vrow);
-        }
+        if constexpr (SHARED_KV) ld_dwords(vrow, vf[u][j]);
+        else ld_dwords_stream(vrow, vf[u][j]);
       }
     }
   };
@@ -342,33 +339,20 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     // ---- O^T += V^T P^T --------------------------------------------------------
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
-      if (VW > 0) {  // bf16, 8 * VW values per token per lane
+      if constexpr (!FP8) {  // 16-bit cache: dword dw of a token holds this lane's values 2 dw, 2 dw + 1
 #pragma unroll
-        for (int w = 0; w < VW; ++w) {
-          const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0][w]);
-          const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1][w]);
-          const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2][w]);
-          const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3][w]);
-#pragma unroll
-          for (int pr = 0; pr < 4; ++pr) {
-            acc[8 * w + 2 * pr] = mfma_16x16x16<F16>(
-                make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr])), pf[u], acc[8 * w + 2 * pr]);
-            acc[8 * w + 2 * pr + 1] = mfma_16x16x16<F16>(
-                make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr])), pf[u], acc[8 * w + 2 * pr + 1]);
-          }
+        for (int dw = 0; dw < VD; ++dw) {
+          const uint32_t r0 = vf[u][0][dw], r1 = vf[u][1][dw], r2 = vf[u][2][dw], r3 = vf[u][3][dw];
+          acc[2 * dw] = mfma_16x16x16<F16>(make_uint2(low_halves(r1, r0), low_halves(r3, r2)), pf[u], acc[2 * dw]);
+          acc[2 * dw + 1] =
+              mfma_16x16x16<F16>(make_uint2(high_halves(r1, r0), high_halves(r3, r2)), pf[u], acc[2 * dw + 1]);
         }
-      } else if (!FP8) {  // bf16, value width 64: four values per token per lane
-        const uint2 a = vf8[u][0], b = vf8[u][1], c = vf8[u][2], d = vf8[u][3];
-        acc[0] = mfma_16x16x16<F16>(make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x)), pf[u], acc[0]);
-        acc[1] = mfma_16x16x16<F16>(make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x)), pf[u], acc[1]);
-        acc[2] = mfma_16x16x16<F16>(make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y)), pf[u], acc[2]);
-        acc[3] = mfma_16x16x16<F16>(make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y)), pf[u], acc[3]);
       } else {  // fp8, width 128: eight bytes per token per lane
         uint2 w[4][2];  // [token j][half] -> two packed bf16 pairs (4 d values)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          w[j][0] = fp8x4_to_bf16x4(vf8[u][j].x);
-          w[j][1] = fp8x4_to_bf16x4(vf8[u][j].y);
+          w[j][0] = fp8x4_to_bf16x4(vf[u][j][0]);
+          w[j][1] = fp8x4_to_bf16x4(vf[u][j][1]);
         }
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
@@ -397,28 +381,26 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + 4 * DV * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      if constexpr (DV >= 8) {
+      uint32_t ow[DV / 2];
 #pragma unroll
-        for (int w = 0; w < DV / 8; ++w)
-          st16(o + DV * i + 8 * w,
-               make_uint4(pack2<F16>(acc[8 * w + 0][i] * inv, acc[8 * w + 1][i] * inv),
-                          pack2<F16>(acc[8 * w + 2][i] * inv, acc[8 * w + 3][i] * inv),
-                          pack2<F16>(acc[8 * w + 4][i] * inv, acc[8 * w + 5][i] * inv),
-                          pack2<F16>(acc[8 * w + 6][i] * inv, acc[8 * w + 7][i] * inv)));
-      } else {
-        st8(o + 4 * i, make_uint2(pack2<F16>(acc[0][i] * inv, acc[1][i] * inv),
-                                  pack2<F16>(acc[2][i] * inv, acc[3][i] * inv)));
-      }
+      for (int dw = 0; dw < DV / 2; ++dw) ow[dw] = pack2<F16>(acc[2 * dw][i] * inv, acc[2 * dw + 1][i] * inv);
+      st_dwords(o + DV * i, ow);
     }
   } else {
     const int64_t row = (int64_t)slot * p.Hq + hq;
     float* o = p.part_o + row * HDV + 4 * DV * g;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      if constexpr (DV % 4 == 0) {
 #pragma unroll
-      for (int e = 0; e < DV; e += 4) {
-        float4 v = make_float4(acc[e][i] * inv, acc[e + 1][i] * inv, acc[e + 2][i] * inv, acc[e + 3][i] * inv);
-        *reinterpret_cast<float4*>(o + DV * i + e) = v;
+        for (int e = 0; e < DV; e += 4) {
+          float4 v = make_float4(acc[e][i] * inv, acc[e + 1][i] * inv, acc[e + 2][i] * inv, acc[e + 3][i] * inv);
+          *reinterpret_cast<float4*>(o + DV * i + e) = v;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < DV; e += 2)
+          *reinterpret_cast<float2*>(o + DV * i + e) = make_float2(acc[e][i] * inv, acc[e + 1][i] * inv);
       }
     }
     if (g == 0) p.part_lse[row] = m_run + fast_log2(l_tot);
@@ -518,12 +500,17 @@ static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p)
   extern __shared__ int cum[];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  const int h = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x >> 6) + wave);
+  // wavefront index along the heads: `parts` consecutive ones share a KV head and split its query heads by 16
+  const int hv = __builtin_amdgcn_readfirstlane(blockIdx.y * (blockDim.x >> 6) + wave);
+  const int h = p.parts > 1 ? hv / p.parts : hv;
+  const int part = hv - h * p.parts;
+  const int hq0 = h * p.G + 16 * part;
+  const int gq = min(16, p.G - 16 * part);
   // wide keys: 16 query rows per wavefront behind the two integer arrays (see decode_segment)
   uint8_t* const q_lds = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15) +
                          (size_t)wave * 16 * (HDK * 2 + 16);
   walk_segments<16 * NT>(p, [&](int r, int row, int len, int start, int end, bool whole, int slot) {
-    decode_segment<HDK, HDV, NT, FP8, F16>(p, r, row, h, len, start, end, whole, slot, lane, q_lds);
+    decode_segment<HDK, HDV, NT, FP8, F16>(p, r, row, h, hq0, gq, len, start, end, whole, slot, lane, q_lds);
   });
 }
 
@@ -800,11 +787,14 @@ static int merge_groups(int grid_x, int R, int head_dim) {
   return g < 1 ? 1 : g;
 }
 
-static int pick_waves_per_block(int Hkv, const MiTuning& tune) {
+// Wavefronts along the heads: one per KV head and 16 query heads that share it.
+static int head_waves(int Hq, int Hkv) { return Hkv * ((Hq / Hkv + 15) / 16); }
+
+static int pick_waves_per_block(int waves, const MiTuning& tune) {
   int cap = tune.decode_waves_per_block;
   if (cap < 1 || cap > 8) cap = 8;
   for (int w = cap; w >= 1; --w)
-    if (Hkv % w == 0) return w;
+    if (waves % w == 0) return w;
   return 1;
 }
 
@@ -822,11 +812,12 @@ static int device_cu_count() {
 
 // Workgroups along the flattened tile sequence: enough to put `decode_wgs_per_cu`
 // workgroups of 8 waves (or the equivalent in smaller workgroups) on every CU.
-int decode_grid_size(int Hkv, const MiTuning& tune) {
+int decode_grid_size(int Hq, int Hkv, const MiTuning& tune) {
   const int forced = tune.decode_grid;
   if (forced > 0) return forced;
-  const int wpb = pick_waves_per_block(Hkv, tune);
-  const int head_groups = Hkv / wpb;
+  const int waves = head_waves(Hq, Hkv);
+  const int wpb = pick_waves_per_block(waves, tune);
+  const int head_groups = waves / wpb;
   int per_cu = tune.decode_wgs_per_cu * (8 / wpb);
   int grid = device_cu_count() * per_cu / head_groups;
   return grid < 1 ? 1 : grid;
@@ -840,10 +831,10 @@ extern "C" int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv,
                                              int32_t chunk_tokens, int32_t max_kv_len,
                                              int32_t split_tokens, const MiTuning* tuning) {
   (void)chunk_tokens; (void)max_kv_len; (void)split_tokens;  // (the size depends on R, the head counts and the grid only)
-  if (R <= 0 || Hq <= 0 || Hkv <= 0 || head_dim <= 0) return 0;
+  if (R <= 0 || Hq <= 0 || Hkv <= 0 || head_dim <= 0 || Hq % Hkv) return 0;
   MiTuning tune;
   if (mi_resolve_tuning(tuning, &tune, "mi_decode_workspace_bytes") != MI_OK) return -1;
-  const int64_t slots = (int64_t)decode_grid_size(Hkv, tune) + R;
+  const int64_t slots = (int64_t)decode_grid_size(Hq, Hkv, tune) + R;
   return slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
 
@@ -866,9 +857,9 @@ int mi::launch_paged_decode(
   if (R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: need R >= 0 and Hq a multiple of Hkv");
   const int G = Hq / Hkv;
-  if (G > 16) return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: more than 16 query heads per KV head");
-  if (head_dim != 64 && head_dim != 128)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: head_dim must be 64 or 128");
+  if (G > 64) return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: more than 64 query heads per KV head");
+  if (head_dim != 64 && head_dim != 96 && head_dim != 128 && head_dim != 192 && head_dim != 256)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: head_dim must be 64, 96, 128, 192 or 256");
   if (chunk_tokens <= 0 || chunk_tokens % 16)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: chunk size must be a positive multiple of 16");
   if (kv_dtype != MI_KV_BF16 && kv_dtype != MI_KV_FP8_E4M3)
@@ -888,7 +879,7 @@ int mi::launch_paged_decode(
   if ((int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: batch too large for the in-LDS prefix sum (7680 requests)");
 
-  const int grid_x = decode_grid_size(Hkv, tune);
+  const int grid_x = decode_grid_size(Hq, Hkv, tune);
   const int64_t slots = (int64_t)grid_x + R;
   const int64_t need = slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
   if (!workspace || workspace_bytes < need)
@@ -899,8 +890,10 @@ int mi::launch_paged_decode(
   // 16-token sub-tiles per loop iteration (0 = automatic).
   int nt = tune.decode_tile_subtiles;
   if (nt != 1 && nt != 2 && nt != 4) nt = kv_dtype == MI_KV_FP8_E4M3 ? 4 : 2;
+  if (head_dim == 256) nt = 1;                 // (registers: 64 accumulators + 32 each for queries, keys, values)
+  else if (head_dim == 192 && nt > 2) nt = 2;
   while (chunk_tokens % (16 * nt)) nt >>= 1;  // a tile must not straddle two chunks
-  const int minw = tune.decode_min_waves;
+  const int minw = head_dim > 128 ? 2 : tune.decode_min_waves;
   const int tk = 16 * nt;
   // a small batch is cut finer than a large one needs: 64 tokens per workgroup put a single 8 192-token
   // request on 128 CUs (17.8 us against 33 us with 256-token spans); large batches get equal spans anyway
@@ -917,13 +910,15 @@ int mi::launch_paged_decode(
   p.seg_info = (int32_t*)(p.part_lse + slots * Hq);
   p.k_scale = k_scales; p.v_scale = v_scales;
   p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G; p.chunk = chunk_tokens;
+  p.parts = (G + 15) / 16;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
   p.min_span_tiles = (min_span_tokens + tk - 1) / tk;
   p.grid = grid_x;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
 
-  const int wpb = pick_waves_per_block(Hkv, tune);
-  dim3 grid(grid_x, Hkv / wpb), block(64 * wpb);
+  const int waves = head_waves(Hq, Hkv);
+  const int wpb = pick_waves_per_block(waves, tune);
+  dim3 grid(grid_x, waves / wpb), block(64 * wpb);
   const size_t lds = (size_t)R * 2 * sizeof(int32_t);
   hipStream_t st = (hipStream_t)stream;
   hipEvent_t ev_a, ev_b;
@@ -938,19 +933,39 @@ int mi::launch_paged_decode(
     else if (minw == 3) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 3, F16_>), grid, block, lds, st, p);   \
     else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 2, FP8_, 2, F16_>), grid, block, lds, st, p);                  \
   } while (0)
+  // wide heads: two wavefronts per SIMD (256 registers each), tiles of 16 or 32 tokens
+#define MI_LAUNCH_DECODE_WIDE(HD_, F16_)                                                                               \
+  do {                                                                                                                 \
+    if (nt == 2 && HD_ < 256) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, (HD_ < 256 ? 2 : 1), false, 2, F16_>), grid, block, lds, st, p); \
+    else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, false, 2, F16_>), grid, block, lds, st, p);               \
+  } while (0)
   if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true, false);
   else if (head_dim == 128 && f16) MI_LAUNCH_DECODE(128, false, true);
   else if (head_dim == 128) MI_LAUNCH_DECODE(128, false, false);
-  else if (f16) MI_LAUNCH_DECODE(64, false, true);
-  else MI_LAUNCH_DECODE(64, false, false);
+  else if (head_dim == 64 && f16) MI_LAUNCH_DECODE(64, false, true);
+  else if (head_dim == 64) MI_LAUNCH_DECODE(64, false, false);
+  else if (head_dim == 96 && f16) MI_LAUNCH_DECODE(96, false, true);
+  else if (head_dim == 96) MI_LAUNCH_DECODE(96, false, false);
+  else if (head_dim == 192 && f16) MI_LAUNCH_DECODE_WIDE(192, true);
+  else if (head_dim == 192) MI_LAUNCH_DECODE_WIDE(192, false);
+  else if (f16) MI_LAUNCH_DECODE_WIDE(256, true);
+  else MI_LAUNCH_DECODE_WIDE(256, false);
 #undef MI_LAUNCH_DECODE
+#undef MI_LAUNCH_DECODE_WIDE
   if (timed) (void)hipEventRecord(ev_b, st);
   dim3 mgrid(Hq, R);
   const dim3 mblock(head_dim * merge_groups(p.grid, R, head_dim));
-  if (head_dim == 128 && f16) hipLaunchKernelGGL((paged_decode_merge_kernel<128, true>), mgrid, mblock, 0, st, p);
-  else if (head_dim == 128) hipLaunchKernelGGL((paged_decode_merge_kernel<128, false>), mgrid, mblock, 0, st, p);
-  else if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<64, true>), mgrid, mblock, 0, st, p);
-  else hipLaunchKernelGGL((paged_decode_merge_kernel<64, false>), mgrid, mblock, 0, st, p);
+#define MI_LAUNCH_MERGE(HD_)                                                                                          \
+  do {                                                                                                                 \
+    if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<HD_, true>), mgrid, mblock, 0, st, p);                      \
+    else hipLaunchKernelGGL((paged_decode_merge_kernel<HD_, false>), mgrid, mblock, 0, st, p);                         \
+  } while (0)
+  if (head_dim == 128) MI_LAUNCH_MERGE(128);
+  else if (head_dim == 64) MI_LAUNCH_MERGE(64);
+  else if (head_dim == 96) MI_LAUNCH_MERGE(96);
+  else if (head_dim == 192) MI_LAUNCH_MERGE(192);
+  else MI_LAUNCH_MERGE(256);
+#undef MI_LAUNCH_MERGE
   return mi_check_launch("mi_paged_decode_attention");
 }
 
@@ -1125,7 +1140,7 @@ extern "C" int mi_paged_mla_decode_attention(
   p.part_lse = p.part_o + slots * Hq * head_dim_v;
   p.seg_info = (int32_t*)(p.part_lse + slots * Hq);
   p.k_scale = nullptr; p.v_scale = nullptr;
-  p.R = R; p.Hq = Hq; p.Hkv = groups; p.G = Hq < 16 ? Hq : 16; p.chunk = chunk_tokens;
+  p.R = R; p.Hq = Hq; p.Hkv = groups; p.G = Hq < 16 ? Hq : 16; p.parts = 1; p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
   p.min_span_tiles = shared_tile ? 64 / kMlaTile : 64 / 16;
   p.grid = grid_x;

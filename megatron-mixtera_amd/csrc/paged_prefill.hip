@@ -37,6 +37,7 @@ struct PrefillParams {
   int64_t o_st, o_sh;
   uint64_t chunk_magic;  // ceil(2^40 / chunk)
   int32_t T, R, Hq, Hkv, G, g_magic, chunk;  // g_magic = 65536 / G + 1: (n * g_magic) >> 16 == n / G for n <= 64, G <= 16
+  int32_t parts;         // workgroups per KV head along the query heads: each takes up to 16 of the G that share it
   int32_t skip_single;  // requests with exactly one query row are handled by the decode kernels
   float scale_log2;
   const float* k_scale;  // fp8 KV only: [n_chunks][Hkv]
@@ -48,20 +49,43 @@ struct PrefillParams {
   float* split_lse;
 };
 
-// NQ = 16-row tiles per wave; a workgroup always covers 256 rows (16 / NQ waves).
+// The query heads one workgroup serves: with at most 16 query heads per KV head, all G of KV head `hv`; with more,
+// `parts` workgroups share a KV head and take 16 query heads each (the last one the rest).
+struct HeadSlice {
+  int h;        // KV head
+  int hq0;      // first query head
+  int G;        // query heads (1..16)
+  int g_magic;  // 65536 / G + 1
+};
+static __device__ __forceinline__ HeadSlice head_slice(const PrefillParams& p, int hv) {
+  HeadSlice s;
+  if (p.parts <= 1) {
+    s.h = hv; s.hq0 = hv * p.G; s.G = p.G; s.g_magic = p.g_magic;
+  } else {
+    s.h = hv / p.parts;
+    const int part = hv - s.h * p.parts;
+    s.hq0 = s.h * p.G + 16 * part;
+    s.G = min(16, p.G - 16 * part);
+    s.g_magic = 65536 / s.G + 1;
+  }
+  return s;
+}
+
+// NQ = 16-row tiles per wave, WAVES wavefronts per workgroup (256 rows for the narrow heads, 128 at width 256).
 // HDK = width of queries and keys, HDV = width of values and of the output (they differ for the
 // decompressed caches of multi-latent attention: 192 / 128); the value cache has its own strides.
-template <int HDK, int HDV, int NT, int NQ, bool F16>
-__global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillParams p) {
+template <int HDK, int HDV, int NT, int NQ, bool F16, int WAVES = 16 / NQ>
+__global__ __launch_bounds__(64 * WAVES) void paged_prefill_kernel(PrefillParams p) {
   constexpr int KS = HDK / 32;
   constexpr int DV = HDV / 16;
-  constexpr int WAVES = 16 / NQ;
+  constexpr int VD = DV / 2;  // dwords per token and lane of the value operand
 
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int m16 = lane & 15, g = lane >> 4;
-  const int h = blockIdx.y;
-  const int G = p.G;
+  const HeadSlice hs = head_slice(p, blockIdx.y);
+  const int h = hs.h, G = hs.G, g_magic = hs.g_magic, hq0 = hs.hq0;
+  // (the same for every head slice of a launch: the request -> workgroup map depends on it)
   const int BQ = ((16 * NQ) * p.g_magic) >> 16;  // query tokens per wave
   const int SBQ = WAVES * BQ;             // query tokens per workgroup
 
@@ -72,7 +96,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
     const int per_row = G * HDV;  // contiguous elements of this head group in one row
     for (int64_t i = (int64_t)threadIdx.x * 8; i < (int64_t)(p.T - tq) * per_row; i += 64 * WAVES * 8) {
       const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
-      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HDV) * p.o_sh + (e % HDV), make_uint4(0, 0, 0, 0));
+      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(hq0 + e / HDV) * p.o_sh + (e % HDV), make_uint4(0, 0, 0, 0));
     }
   }
 
@@ -103,10 +127,10 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 #pragma unroll
   for (int nt = 0; nt < NQ; ++nt) {
     const int n = 16 * nt + m16;
-    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
+    const int qi = (n * g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     const bool valid = qi < nq;
     qpos[nt] = valid ? shift + q0 + qi : last;
-    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
+    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(hq0 + u) * p.q_sh;
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk)
       qf[nt][kk] = valid ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
@@ -135,10 +159,10 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 #pragma unroll
     for (int nt = 0; nt < NQ; ++nt) {
       const int n = 16 * nt + m16;
-      const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
+      const int qi = (n * g_magic) >> 16, u = n - qi * G;  // n / G, n % G
       if (qi < nq) {
-        uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
-        for (int i = 0; i < 4 * DV; i += 4) st8(o + i, make_uint2(0, 0));
+        uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(hq0 + u) * p.o_sh + 4 * DV * g;
+        for (int i = 0; i < 4 * DV; i += 2) *reinterpret_cast<uint32_t*>(o + i) = 0u;
       }
     }
     return;
@@ -147,8 +171,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
   // K / V staging registers of one tile of 16*NT keys; the loop is software pipelined on them
   // (K of the next tile is requested once all scores of this one exist, V once P.V is done).
   uint4 kf[NT][KS];
-  uint4 vf16[NT][4];
-  uint2 vf8[NT][4];
+  uint32_t vf[NT][4][VD];
   auto load_k = [&](int T) {
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
@@ -172,8 +195,7 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const uint8_t* vrow = vc + (min(T0 + 4 * g + j, last) - ci * p.chunk) * v_tok_bytes + DV * m16 * 2;
-        if (HDV == 128) vf16[u][j] = ld16(vrow);
-        else vf8[u][j] = ld8(vrow);
+        ld_dwords(vrow, vf[u][j]);
       }
     }
   };
@@ -256,22 +278,11 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
     // Two 16-key sub-tiles are contracted by one mfma 16x16x32 (slots 0-3 = tokens 4g..4g+3 of
     // the first sub-tile, slots 4-7 = the same of the second; P is packed the same way).
     auto transpose_v = [&](int u, uint2 (&vt)[DV]) {
-      if constexpr (HDV == 128) {
-        const uint32_t* r0 = reinterpret_cast<const uint32_t*>(&vf16[u][0]);
-        const uint32_t* r1 = reinterpret_cast<const uint32_t*>(&vf16[u][1]);
-        const uint32_t* r2 = reinterpret_cast<const uint32_t*>(&vf16[u][2]);
-        const uint32_t* r3 = reinterpret_cast<const uint32_t*>(&vf16[u][3]);
 #pragma unroll
-        for (int pr = 0; pr < 4; ++pr) {
-          vt[2 * pr] = make_uint2(low_halves(r1[pr], r0[pr]), low_halves(r3[pr], r2[pr]));
-          vt[2 * pr + 1] = make_uint2(high_halves(r1[pr], r0[pr]), high_halves(r3[pr], r2[pr]));
-        }
-      } else {
-        const uint2 a = vf8[u][0], b = vf8[u][1], c = vf8[u][2], d = vf8[u][3];
-        vt[0] = make_uint2(low_halves(b.x, a.x), low_halves(d.x, c.x));
-        vt[1] = make_uint2(high_halves(b.x, a.x), high_halves(d.x, c.x));
-        vt[2] = make_uint2(low_halves(b.y, a.y), low_halves(d.y, c.y));
-        vt[3] = make_uint2(high_halves(b.y, a.y), high_halves(d.y, c.y));
+      for (int dw = 0; dw < VD; ++dw) {
+        const uint32_t r0 = vf[u][0][dw], r1 = vf[u][1][dw], r2 = vf[u][2][dw], r3 = vf[u][3][dw];
+        vt[2 * dw] = make_uint2(low_halves(r1, r0), low_halves(r3, r2));
+        vt[2 * dw + 1] = make_uint2(high_halves(r1, r0), high_halves(r3, r2));
       }
     };
     if constexpr (NT % 2 == 0) {
@@ -313,20 +324,15 @@ __global__ __launch_bounds__(64 * (16 / NQ)) void paged_prefill_kernel(PrefillPa
     l_tot += xor32(l_tot);
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int n = 16 * nt + m16;
-    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
+    const int qi = (n * g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     if (qi < nq) {
-      uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * DV * g;
+      uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(hq0 + u) * p.o_sh + 4 * DV * g;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        if constexpr (DV == 8) {
-          st16(o + 8 * i, make_uint4(pack2<F16>(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
-                                     pack2<F16>(acc[nt][2][i] * inv, acc[nt][3][i] * inv),
-                                     pack2<F16>(acc[nt][4][i] * inv, acc[nt][5][i] * inv),
-                                     pack2<F16>(acc[nt][6][i] * inv, acc[nt][7][i] * inv)));
-        } else {
-          st8(o + 4 * i, make_uint2(pack2<F16>(acc[nt][0][i] * inv, acc[nt][1][i] * inv),
-                                    pack2<F16>(acc[nt][2][i] * inv, acc[nt][3][i] * inv)));
-        }
+        uint32_t ow[VD];
+#pragma unroll
+        for (int dw = 0; dw < VD; ++dw) ow[dw] = pack2<F16>(acc[nt][2 * dw][i] * inv, acc[nt][2 * dw + 1][i] * inv);
+        st_dwords(o + DV * i, ow);
       }
     }
   }
@@ -388,9 +394,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform values stay in SGPRs
   const int m16 = lane & 15, g = lane >> 4;
   const int lead = STAGGER ? (wave >> 2) : 0;  // 0: first group, 1: second group (one phase behind)
-  const int h = blockIdx.x % p.Hkv;
-  const int rank = blockIdx.x / p.Hkv;
-  const int G = p.G;
+  const int HV = p.Hkv * p.parts;  // workgroups along the heads
+  const HeadSlice hs = head_slice(p, blockIdx.x % HV);
+  const int h = hs.h, G = hs.G, g_magic = hs.g_magic, hq0 = hs.hq0;
+  const int rank = blockIdx.x / HV;
+  // query tokens per workgroup: the same for every head slice of a launch (the request -> workgroup map
+  // depends on it), i.e. the count of the widest slice; a narrower last slice leaves rows unused
   const int BQ = ((16 * NQ) * p.g_magic) >> 16;
   const int SBQ = WAVES * BQ;
 
@@ -399,11 +408,11 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     const int per_row = G * HD;
     for (int64_t i = (int64_t)tid * 8; i < (int64_t)(p.T - tq) * per_row; i += 512 * 8) {
       const int row = (int)(i / per_row), e = (int)(i - (int64_t)row * per_row);
-      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(h * G + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
+      st16(p.out + (int64_t)(tq + row) * p.o_st + (int64_t)(hq0 + e / HD) * p.o_sh + (e % HD), make_uint4(0, 0, 0, 0));
     }
   }
 
-  const int sb = (int)(gridDim.x / p.Hkv) - 1 - rank;
+  const int sb = (int)(gridDim.x / HV) - 1 - rank;
   int lo = 0, hi = p.R - 1;
   while (lo < hi) {
     const int mid = (lo + hi + 1) >> 1;
@@ -435,10 +444,10 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 #pragma unroll
   for (int nt = 0; nt < NQ; ++nt) {
     const int n = 16 * nt + m16;
-    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
+    const int qi = (n * g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     const bool valid = qi < nq;
     qpos[nt] = valid ? shift + q0 + qi : last;
-    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(h * G + u) * p.q_sh;
+    const uint16_t* qrow = p.q + (int64_t)(q_begin + q0 + qi) * p.q_st + (int64_t)(hq0 + u) * p.q_sh;
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk)
       qf[nt][kk] = valid ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
@@ -835,16 +844,16 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     const float l_tot = accl[nt][0];
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int n = 16 * nt + m16;
-    const int qi = (n * p.g_magic) >> 16, u = n - qi * G;  // n / G, n % G
+    const int qi = (n * g_magic) >> 16, u = n - qi * G;  // n / G, n % G
     if (qi < nq) {
       if (!SPLIT) {
-        uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(h * G + u) * p.o_sh + 4 * g;
+        uint16_t* o = p.out + (int64_t)(q_begin + q0 + qi) * p.o_st + (int64_t)(hq0 + u) * p.o_sh + 4 * g;
 #pragma unroll
         for (int e = 0; e < DV; ++e)
           st8(o + 16 * e, make_uint2(pack2<F16>(acc[nt][e][0] * inv, acc[nt][e][1] * inv),
                                      pack2<F16>(acc[nt][e][2] * inv, acc[nt][e][3] * inv)));
       } else {  // a range without visible keys (none for short requests) leaves zeros and -inf
-        const int64_t prow = ((int64_t)split * p.T + (q_begin + q0 + qi)) * p.Hq + (h * G + u);
+        const int64_t prow = ((int64_t)split * p.T + (q_begin + q0 + qi)) * p.Hq + (hq0 + u);
         float* o = p.split_o + prow * HD + 4 * g;
 #pragma unroll
         for (int e = 0; e < DV; ++e)
@@ -903,9 +912,9 @@ using namespace mi;
 // every one keeping at least sixteen 64-key tiles (a 512-token prompt is not worth the merge).  Host-side quantities only (the lengths live on the GPU).
 static int prefill_kv_splits(int T, int Hq, int Hkv, int head_dim, int max_kv_len) {
   if ((head_dim != 128 && head_dim != 64) || max_kv_len <= 0) return 1;
-  const int G = Hq / Hkv;
-  const int sbq = 8 * (32 / G);                          // query tokens per workgroup (8 wavefronts x 32 rows)
-  const int64_t useful = (int64_t)Hkv * ((T + sbq - 1) / sbq);
+  const int G = Hq / Hkv, Gw = G < 16 ? G : 16, parts = (G + 15) / 16;
+  const int sbq = 8 * (32 / Gw);                         // query tokens per workgroup (8 wavefronts x 32 rows)
+  const int64_t useful = (int64_t)Hkv * parts * ((T + sbq - 1) / sbq);
   const int cus = 256;
   if (useful >= cus) return 1;
   int64_t s = (cus + useful - 1) / useful;
@@ -968,10 +977,11 @@ static int launch_paged_prefill(
   if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: need T, R >= 0 and Hq a multiple of Hkv");
   const int G = Hq / Hkv;
-  if (G > 16)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: at most 16 query heads per KV head");
-  if (head_dim != 64 && head_dim != 128)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: head_dim must be 64 or 128");
+  if (G > 64)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: at most 64 query heads per KV head");
+  if (head_dim != 64 && head_dim != 96 && head_dim != 128 && head_dim != 192 && head_dim != 256)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: head_dim must be 64, 96, 128, 192 or 256");
+  const int Gw = G < 16 ? G : 16, parts = (G + 15) / 16;  // query heads per workgroup, workgroups per KV head
   if (chunk_tokens <= 0 || chunk_tokens % 16)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: chunk size must be a positive multiple of 16");
   if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15)
@@ -984,9 +994,9 @@ static int launch_paged_prefill(
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: unknown kv_dtype");
   if (fp8 && (!k_scales || !v_scales))
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_fp8: both scale arrays are required");
-  // the two-phase tile kernel stages 64-key tiles that must not straddle chunks; other chunk sizes (and the
-  // knob) select the register-only kernel
-  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0;
+  // the two-phase tile kernel stages 64-key tiles that must not straddle chunks and exists for the common widths;
+  // other chunk sizes and widths (and the knob) select the register-only kernel
+  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0 && (head_dim == 64 || head_dim == 128);
   if (fp8 && (head_dim != 128 || !two_phase || f16))
     return mi_fail(MI_ERR_UNSUPPORTED,
                    "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 128, a chunk size that is a "
@@ -1004,8 +1014,8 @@ static int launch_paged_prefill(
   p.v_sc = p.kv_sc; p.v_st = p.kv_st; p.v_sh = p.kv_sh;
   p.bt = block_table; p.bt_stride = bt_stride; p.cu_q = cu_seqlens_q; p.lens = kv_lens;
   p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
-  p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G;
-  p.g_magic = 65536 / G + 1;
+  p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G; p.parts = parts;
+  p.g_magic = 65536 / Gw + 1;
   p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
@@ -1016,8 +1026,8 @@ static int launch_paged_prefill(
 
   hipStream_t st = (hipStream_t)stream;
   if (two_phase) {
-    const int sbq_lds = 8 * (32 / G);  // 8 wavefronts x whole tokens in a wavefront's 32 rows
-    dim3 lgrid(((T + sbq_lds - 1) / sbq_lds + R) * Hkv);
+    const int sbq_lds = 8 * (32 / Gw);  // 8 wavefronts x whole tokens in a wavefront's 32 rows
+    dim3 lgrid(((T + sbq_lds - 1) / sbq_lds + R) * Hkv * parts);
     hipEvent_t ev_a, ev_b;
     const bool timed = mi_profile_next(&ev_a, &ev_b);
     if (timed) (void)hipEventRecord(ev_a, st);
@@ -1049,10 +1059,12 @@ static int launch_paged_prefill(
     }
   } else {
     // register-only kernel: any chunk size that is a multiple of 16; 16 or 32 keys per iteration
-    const int nq = tune.prefill_row_tiles == 4 ? 4 : 2;
-    const int sbq = (16 / nq) * ((16 * nq) / G);  // query tokens per workgroup: whole tokens in each wavefront's rows
-    dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * (16 / nq));
-    const int nt = tune.prefill_tile_subtiles == 1 ? 1 : 2;
+    // (wide heads: fewer rows per wavefront and keys per iteration, so that accumulators and fragments fit)
+    const int nq = head_dim == 256 ? 1 : head_dim == 192 ? 2 : tune.prefill_row_tiles == 4 ? 4 : 2;
+    const int waves = head_dim == 256 ? 8 : 16 / nq;
+    const int sbq = waves * ((16 * nq) / Gw);  // query tokens per workgroup: whole tokens in each wavefront's rows
+    dim3 grid((T + sbq - 1) / sbq + R, Hkv * parts), block(64 * waves);
+    const int nt = (tune.prefill_tile_subtiles == 1 || head_dim >= 192) ? 1 : 2;
 #define MI_LAUNCH_PREFILL(HD_, F16_)                                                                           \
   do {                                                                                                         \
     if (nq == 4 && nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, 1, 4, F16_>), grid, block, 0, st, p);  \
@@ -1062,8 +1074,14 @@ static int launch_paged_prefill(
   } while (0)
     if (head_dim == 128 && f16) MI_LAUNCH_PREFILL(128, true);
     else if (head_dim == 128) MI_LAUNCH_PREFILL(128, false);
-    else if (f16) MI_LAUNCH_PREFILL(64, true);
-    else MI_LAUNCH_PREFILL(64, false);
+    else if (head_dim == 64 && f16) MI_LAUNCH_PREFILL(64, true);
+    else if (head_dim == 64) MI_LAUNCH_PREFILL(64, false);
+    else if (head_dim == 96 && f16) MI_LAUNCH_PREFILL(96, true);
+    else if (head_dim == 96) MI_LAUNCH_PREFILL(96, false);
+    else if (head_dim == 192 && f16) hipLaunchKernelGGL((paged_prefill_kernel<192, 192, 1, 2, true>), grid, block, 0, st, p);
+    else if (head_dim == 192) hipLaunchKernelGGL((paged_prefill_kernel<192, 192, 1, 2, false>), grid, block, 0, st, p);
+    else if (f16) hipLaunchKernelGGL((paged_prefill_kernel<256, 256, 1, 1, true, 8>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_kernel<256, 256, 1, 1, false, 8>), grid, block, 0, st, p);
 #undef MI_LAUNCH_PREFILL
   }
   const int rc = mi_check_launch("mi_paged_prefill_attention");
@@ -1126,8 +1144,9 @@ extern "C" int mi_paged_prefill_attention_mla(
   if (T < 0 || R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || Hkv > 65535)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention_mla: need T, R >= 0 and Hq a multiple of Hkv");
   const int G = Hq / Hkv;
-  if (G > 16)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: at most 16 query heads per KV head");
+  if (G > 64)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: at most 64 query heads per KV head");
+  const int Gw = G < 16 ? G : 16, parts = (G + 15) / 16;  // query heads per workgroup, workgroups per KV head
   if (head_dim_k != 192 || head_dim_v != 128)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention_mla: key width 192 (128 + 64) and value width 128 only");
   if (chunk_tokens <= 0 || chunk_tokens % 16)
@@ -1148,15 +1167,15 @@ extern "C" int mi_paged_prefill_attention_mla(
   p.v_sc = v_stride_chunk; p.v_st = (int32_t)v_stride_tok; p.v_sh = (int32_t)v_stride_head;
   p.bt = block_table; p.bt_stride = bt_stride; p.cu_q = cu_seqlens_q; p.lens = kv_lens;
   p.out = (uint16_t*)out; p.o_st = o_stride_tok; p.o_sh = o_stride_head;
-  p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G;
-  p.g_magic = 65536 / G + 1;
+  p.T = T; p.R = R; p.Hq = Hq; p.Hkv = Hkv; p.G = G; p.parts = parts;
+  p.g_magic = 65536 / Gw + 1;
   p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.skip_single = 0;  // one kernel serves every request, one-row requests included
   p.k_scale = nullptr; p.v_scale = nullptr;
   p.split_o = nullptr; p.split_lse = nullptr;
-  const int sbq = 8 * (32 / G);  // query tokens per workgroup (8 wavefronts x 32 rows)
+  const int sbq = 8 * (32 / Gw);  // query tokens per workgroup (8 wavefronts x 32 rows)
   const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0;  // staged tiles must not straddle chunks
   hipStream_t st = (hipStream_t)stream;
   hipEvent_t ev_a, ev_b;
@@ -1164,7 +1183,7 @@ extern "C" int mi_paged_prefill_attention_mla(
   if (timed) (void)hipEventRecord(ev_a, st);
   int n_split = 1;
   if (two_phase) {
-    dim3 lgrid(((T + sbq - 1) / sbq + R) * Hkv);
+    dim3 lgrid(((T + sbq - 1) / sbq + R) * Hkv * parts);
     const bool stagger = tune.prefill_two_phase == 1;
     // few query rows over long contexts: key ranges per request, partials in the workspace (which holds
     // nothing else here: one-row requests stay in the tile kernel)
@@ -1181,9 +1200,9 @@ extern "C" int mi_paged_prefill_attention_mla(
     if (f16) MI_PP_LAUNCH(false, 128, 192, true);
     else MI_PP_LAUNCH(false, 128, 192, false);
   } else {
-    dim3 grid((T + sbq - 1) / sbq + R, Hkv), block(64 * 8);
-    if (f16) hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2, true>), grid, block, 0, st, p);
-    else hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 2, 2, false>), grid, block, 0, st, p);
+    dim3 grid((T + sbq - 1) / sbq + R, Hkv * parts), block(64 * 8);
+    if (f16) hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 1, 2, true>), grid, block, 0, st, p);
+    else hipLaunchKernelGGL((paged_prefill_kernel<192, 128, 1, 2, false>), grid, block, 0, st, p);
   }
   if (timed) (void)hipEventRecord(ev_b, st);
   if (n_split > 1) {

@@ -120,12 +120,12 @@ def test_argument_validation_needs_no_gpu(mi):
     assert lib.mi_kv_append(None, None, 8, None, None, 8, 8, None, None, 0, 8, 2, None) == 0
     # unsupported head_dim / grouping are refused with a message
     one = ctypes.c_void_p(16)
-    rc = lib.mi_paged_decode_attention(one, 96, 96, one, one, 96, 96, 96, one, 1, one, one, 96, 96, one, 1 << 30,
-                                       1, 1, 1, 96, 16, 16, 0, 0.1, 0, None, None, 0, None, None)
+    rc = lib.mi_paged_decode_attention(one, 80, 80, one, one, 80, 80, 80, one, 1, one, one, 80, 80, one, 1 << 30,
+                                       1, 1, 1, 80, 16, 16, 0, 0.1, 0, None, None, 0, None, None)
     assert rc == -4 and b"head_dim" in lib.mi_last_error()
     rc = lib.mi_paged_decode_attention(one, 128, 128, one, one, 128, 128, 128, one, 1, one, one, 128, 128, one,
-                                       1 << 30, 1, 34, 2, 128, 16, 16, 0, 0.1, 0, None, None, 0, None, None)
-    assert rc == -4 and b"16 query heads" in lib.mi_last_error()
+                                       1 << 30, 1, 130, 2, 128, 16, 16, 0, 0.1, 0, None, None, 0, None, None)
+    assert rc == -4 and b"64 query heads" in lib.mi_last_error()
     rc = lib.mi_paged_decode_attention(one, 128, 128, one, one, 128, 128, 128, one, 1, one, one, 128, 128, one,
                                        1 << 30, 1, 8, 2, 128, 24, 16, 0, 0.1, 0, None, None, 0, None, None)
     assert rc == -2 and b"multiple of 16" in lib.mi_last_error()

@@ -73,6 +73,49 @@ def test_ragged_lengths_and_edges(mi, dev, chunk, subtiles, grid):
         mi.ops.set_tuning("decode_grid", 0)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("d", [96, 192, 256])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (32, 8), (12, 4), (16, 1)])
+def test_head_widths_96_192_256(mi, dev, d, Hq, Hkv, dtype):
+    """Head widths beside 64 and 128 (Phi-3-small / Gemma use 96 and 256, decompressed multi-latent keys 192):
+    ragged lengths around the tile and chunk edges, several chunk sizes and span cuts."""
+    for chunk in (16, 64, 256):
+        lens = torch.tensor([0, 1, 15, 16, 17, 33, chunk - 1, chunk, chunk + 1, 3 * chunk + 5, 1999], dtype=torch.int32)
+        cfg = mi.synthetic.DecodeConfig("w", lens.numel(), Hq, Hkv, d, 0, 0, chunk=chunk, seed=d + Hq + chunk)
+        case = mi.synthetic.make_decode_case(cfg, dev, lens=lens, dtype=dtype)
+        ref = _ref(case)
+        for split, grid in ((0, 0), (16, 4096), (512, 7)):
+            with mi.ops.tuning(decode_grid=grid):
+                out = _run_case(mi, case, split_tokens=split, max_kv_len=int(lens.max()))
+            _close(out, ref, 2e-2)
+            assert (out[case.kv_lens == 0] == 0).all(), "zero-length rows must be zeros"
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 1), (64, 2), (17, 1), (48, 2), (40, 2), (64, 1)])
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_more_than_16_query_heads_per_kv_head(mi, dev, Hq, Hkv, d):
+    """Up to 64 query heads share a KV head (multi-query models: Falcon-7B 71 -> 1 is beyond, Gemma-2B 8 -> 1 and
+    StarCoder 48 -> 1 within): every 16 of them take a wavefront of their own."""
+    lens = torch.tensor([0, 1, 17, 64, 65, 700, 2500], dtype=torch.int32)
+    cfg = mi.synthetic.DecodeConfig("mq", lens.numel(), Hq, Hkv, d, 0, 0, chunk=64, seed=Hq * 3 + d)
+    case = mi.synthetic.make_decode_case(cfg, dev, lens=lens)
+    ref = _ref(case)
+    for split, grid in ((0, 0), (64, 9), (16, 4096)):
+        with mi.ops.tuning(decode_grid=grid):
+            out = _run_case(mi, case, split_tokens=split, max_kv_len=int(lens.max()))
+        _close(out, ref, 2e-2)
+    # fp8 cache, width 128
+    if d == 128:
+        k8, ks = oa.quantize_chunks_fp8(case.k_cache.cpu())
+        v8, vs = oa.quantize_chunks_fp8(case.v_cache.cpu())
+        out = mi.ops.paged_decode_attention(case.q, k8.to(dev), v8.to(dev), case.kv_lens, case.block_table,
+                                            k_scales=ks.to(dev), v_scales=vs.to(dev))
+        torch.cuda.synchronize()
+        ref8 = oa.paged_decode_attention(case.q.cpu().squeeze(1), k8, v8, lens, case.block_table.cpu(), k_scales=ks,
+                                         v_scales=vs)
+        _close(out, ref8, 2e-2)
+
+
 def test_block_table_width_and_padding_rows(mi, dev):
     """Block table wider than needed (graph mode passes max_sequence_length) with -1 / 0 padding."""
     cfg = mi.synthetic.DecodeConfig("wide", 6, 32, 8, 128, 100, 2000, chunk=256, seed=5)
@@ -204,7 +247,7 @@ def test_rejects_bad_arguments(mi, dev):
     with pytest.raises(mi._lib.KernelError):
         mi.ops.paged_decode_attention(case.q, case.k_cache, case.v_cache, case.kv_lens, case.block_table,
                                       workspace=torch.empty(16, dtype=torch.uint8, device=dev), split_tokens=16)
-    q96 = torch.randn(2, 1, 8, 96, device=dev).bfloat16()
-    kc96 = torch.randn(4, 64, 2, 96, device=dev).bfloat16()
+    q80 = torch.randn(2, 1, 8, 80, device=dev).bfloat16()
+    kc80 = torch.randn(4, 64, 2, 80, device=dev).bfloat16()
     with pytest.raises(mi._lib.KernelError):
-        mi.ops.paged_decode_attention(q96, kc96, kc96, case.kv_lens, case.block_table)
+        mi.ops.paged_decode_attention(q80, kc80, kc80, case.kv_lens, case.block_table)

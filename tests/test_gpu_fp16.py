@@ -147,7 +147,7 @@ def _ulp_diff_f16(a, b):
 
 @pytest.mark.parametrize("norm", [None, "rms", "l2"])
 @pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64), (128, 40)])
+@pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64), (128, 40), (96, 96), (192, 64), (256, 256)])
 @pytest.mark.parametrize("vectorised", [1, -1])
 def test_norm_rope_follows_the_fp16_op_chain(mi, dev, norm, interleaved, d, rot, vectorised):
     """With faithful rounding the kernel rounds to fp16 wherever the unfused fp16 chain does: under 1 % of the

@@ -2,7 +2,7 @@
 
 Floating point: bf16 results within 2e-2 abs/rel of the fp32 formula; in the faithful
 rounding mode the kernel reproduces the bf16 op chain up to the last-place effects of
-cos/sin/rsqrt implementations (at most 2 bf16 ulps on a tiny fraction of elements).
+cos/sin/rsqrt implementations (a tiny fraction of elements, by at most 2 ulps of the head vector's largest element).
 """
 import pytest
 import torch
@@ -24,7 +24,8 @@ def _ulp_diff(a, b):
 
 @pytest.mark.parametrize("norm", [None, "rms", "l2"])
 @pytest.mark.parametrize("interleaved", [False, True])
-@pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64), (128, 96), (64, 32), (128, 40)])
+@pytest.mark.parametrize("d,rot", [(128, 128), (64, 64), (128, 64), (128, 96), (64, 32), (128, 40),
+                                   (96, 96), (96, 48), (96, 32), (192, 192), (192, 64), (256, 256), (256, 128), (256, 90)])
 @pytest.mark.parametrize("vectorised", [1, -1])
 def test_norm_rope_matches_unfused_chain(mi, dev, norm, interleaved, d, rot, vectorised):
     """Both kernels: 16 bytes per lane (taken when every rotary partner is a whole number of lanes
@@ -62,9 +63,12 @@ def _norm_rope_case(mi, dev, norm, interleaved, d, rot):
             err = (got.float() - ref.float()).abs()
             assert (err <= 2e-2 + 2e-2 * ref.float().abs()).all(), f"max err {err.max().item()}"
             if faithful:
-                ulps = _ulp_diff(got, ref)
-                assert ulps.max().item() <= 2
-                assert (ulps > 0).float().mean().item() < 0.01
+                # under 1 % of the elements differ at all (the device's rsqrt / cos / sin differ from the host's in
+                # the last bit), and those by at most 2 ulp of the head vector's largest element: a rotation whose
+                # two products nearly cancel turns one ulp of a product into many ulp of the small difference
+                assert (_ulp_diff(got, ref) > 0).float().mean().item() < 0.01
+                scale = ref.float().abs().amax(-1, keepdim=True)
+                assert (err <= 2 * 2.0 ** -7 * scale).all()
         assert torch.equal(kd.cpu(), k), "the key input must not be modified"
 
 
@@ -116,7 +120,7 @@ def test_fused_append_writes_rotated_key_and_raw_value(mi, dev, mode):
     assert (k_out.cpu().squeeze(1).float() - k_ref.float()).abs().max().item() <= 4e-2
 
 
-@pytest.mark.parametrize("d,hq,hkv", [(128, 32, 8), (128, 8, 8), (64, 12, 4), (128, 5, 1)])
+@pytest.mark.parametrize("d,hq,hkv", [(128, 32, 8), (128, 8, 8), (64, 12, 4), (128, 5, 1), (96, 32, 8), (192, 6, 2), (256, 16, 1)])
 @pytest.mark.parametrize("vectorised", [1, -1])
 @pytest.mark.parametrize("interleaved", [False, True])
 def test_mixed_qkv_input_equals_split_inputs(mi, dev, d, hq, hkv, vectorised, interleaved):

@@ -98,6 +98,57 @@ def test_two_phase_kernel_ragged_lengths(mi, dev, pingpong, chunk, Hq, Hkv, d):
         mi.ops.set_tuning("prefill_two_phase", 0)
 
 
+def _ragged_case(mi, dev, Hq, Hkv, d, chunk, dtype, seed, pad_rows=0):
+    q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 300, 3]
+    ctx = [0, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0, 40, 7, 1020]
+    kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
+    cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    gen = torch.Generator().manual_seed(seed)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, gen)
+    q = torch.randn(int(cu_q[-1]) + pad_rows, Hq, d, generator=gen).to(dtype).to(dev)
+    kc = torch.randn(N, chunk, Hkv, d, generator=gen).to(dtype).to(dev)
+    vc = torch.randn(N, chunk, Hkv, d, generator=gen).to(dtype).to(dev)
+    return q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev)
+
+
+def _check_padded(mi, q, kc, vc, cu_q, lens, bt, tol=2e-2):
+    out = mi.ops.paged_prefill_attention(q, kc, vc, cu_q, lens, bt, max_kv_len=int(lens.max()))
+    torch.cuda.synchronize()
+    T = int(cu_q[-1])
+    assert (out[T:] == 0).all(), "padding rows must be zeros"
+    ref = oa.paged_varlen_attention(q[:T].cpu(), kc.cpu(), vc.cpu(), cu_q.cpu(), lens.cpu(), bt.cpu())
+    got = out[:T].float().cpu()
+    assert torch.isfinite(got).all()
+    err = (got - ref).abs()
+    assert (err <= tol + tol * ref.abs()).all(), f"max err {err.max().item():.4e}"
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("chunk", [16, 64, 256])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (32, 8), (12, 4), (16, 1)])
+@pytest.mark.parametrize("d", [96, 192, 256])
+def test_head_widths_96_192_256(mi, dev, d, Hq, Hkv, chunk, dtype):
+    """Head widths beside 64 and 128 in prefill and mixed batches: ragged new-token counts and contexts, one-row
+    requests through the decode kernels (default) and through the prefill kernel (no workspace -> forced below by
+    the register-only knob), padding rows."""
+    q, kc, vc, cu_q, lens, bt = _ragged_case(mi, dev, Hq, Hkv, d, chunk, dtype, seed=d + Hq + chunk, pad_rows=3)
+    _check_padded(mi, q, kc, vc, cu_q, lens, bt)
+
+
+@pytest.mark.parametrize("kernel", ["two_phase", "registers", "split_keys"])
+@pytest.mark.parametrize("Hq,Hkv", [(32, 1), (64, 2), (17, 1), (48, 2), (40, 2), (64, 1)])
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_more_than_16_query_heads_per_kv_head(mi, dev, kernel, Hq, Hkv, d):
+    """Up to 64 query heads per KV head: every 16 of them (the last group: the rest) take workgroups of their own."""
+    if d == 256 and kernel != "registers":
+        pytest.skip("width 256 always takes the register-only kernel")
+    knobs = {"two_phase": {}, "registers": {"prefill_two_phase": -1}, "split_keys": {"prefill_kv_split": 3}}[kernel]
+    q, kc, vc, cu_q, lens, bt = _ragged_case(mi, dev, Hq, Hkv, d, 64, torch.bfloat16, seed=Hq + d, pad_rows=2)
+    with mi.ops.tuning(**knobs):
+        _check_padded(mi, q, kc, vc, cu_q, lens, bt)
+
+
 def test_stale_cache_rows_beyond_the_length_do_not_leak(mi, dev):
     """Slots past a request's last token may hold anything (NaN patterns included): the staged tiles
     re-read the last valid row instead of them."""
