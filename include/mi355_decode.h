@@ -82,7 +82,7 @@ typedef struct MiTuning {
 
 /*
  * Kernel timing.  mi_profile_enable(1) makes the attention entry points bracket their main
- * kernel (decode: the KV-streaming kernel; prefill, head_dim 128 or 64 with a chunk size that is a multiple of 64: the tile kernel, followed by
+ * kernel (decode: the KV-streaming kernel; prefill, head_dim 64, 96 or 128 with a chunk size that is a multiple of 64: the tile kernel, followed by
  * a second pair for the decode kernel of a mixed batch) with HIP events on the caller's
  * stream; mi_profile_collect waits for
  * the recorded pairs, writes their durations (milliseconds, HOST pointer) and returns how
@@ -170,8 +170,8 @@ int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t he
  * (megatron/core/transformer/attention.py:589-600):
  *   out[r,h] = softmax(q[r,h] . K_r[:len_r, h/G]^T * softmax_scale) . V_r[:len_r, h/G]
  *   K_r[j] = k_cache[block_table[r, j / chunk_tokens], j % chunk_tokens], G = Hq/Hkv.
- * q/out: bf16 `[R, Hq, d]` with the given token / head strides; d 64 or 128; G any value up to 16
- * (not only powers of two).  kv_lens int32 [R] (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] (the reference
+ * q/out: bf16 or fp16 `[R, Hq, d]` with the given token / head strides; d 64, 96, 128, 192 or 256 (an fp8 cache:
+ * 128); G any value up to 64 (not only powers of two; every 16 query heads of a KV head take a wavefront).  kv_lens int32 [R] (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] (the reference
  * passes max_sequence_length here, dynamic_context.py:791); the grid does not depend on
  * it.  `split_tokens` = minimum tokens one workgroup streams (0 = default 64).
  * kv_dtype MI_KV_FP8_E4M3 reads byte caches with k_scales/v_scales `[n_chunks, Hkv]`.
@@ -239,11 +239,13 @@ int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q
  * (megatron/core/transformer/attention.py:546-557): request r owns query rows
  * cu_seqlens_q[r]..cu_seqlens_q[r+1]-1 and kv_lens[r] keys; query i of Lq sees keys
  * j <= i + (Lk - Lq) (bottom-right aligned causal mask).  Rows past cu_seqlens_q[R] (token
- * padding) are zeroed.  head_dim 64 or 128; Hq / Hkv any value up to 16 (3, 5, 7 ... included).
+ * padding) are zeroed.  head_dim 64, 96, 128, 192 or 256; Hq / Hkv any value up to 64 (3, 5, 7 ... included; every
+ * 16 query heads of a KV head take workgroups of their own).
  * With a workspace of mi_prefill_workspace_bytes() bytes, requests that
  * have exactly one query row (the decode requests of a mixed batch) are streamed by the
  * decode kernels at full bandwidth; with workspace == NULL one kernel handles every request.
- * The same workspace lets the two-phase tile kernel (head_dim 128 or 64, chunk size a multiple of 64) cut the keys of every request into ranges when
+ * The same workspace lets the two-phase tile kernel (head_dim 64, 96 or 128, chunk size a multiple of 64; other
+ * widths and chunk sizes run a register-only kernel) cut the keys of every request into ranges when
  * the batch has few query rows over long contexts (a chunk of a prompt, a short turn after a long
  * history: without it a handful of workgroups would walk thousands of keys each): the ranges are
  * computed by separate workgroups and merged by log-sum-exp, as in the decode path.  `max_kv_len` (an

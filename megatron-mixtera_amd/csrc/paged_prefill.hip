@@ -360,8 +360,9 @@ __global__ __launch_bounds__(64 * WAVES) void paged_prefill_kernel(PrefillParams
 // bytes per staged K / V row.  head_dim 128: 288, measured conflict-free for the 16-row x 64-byte fragment
 // reads (272 is not), and 16 rows x 32 B of the transposing reads tile the banks twice; head_dim 64: 144
 // (36 dwords: the 16 rows of a fragment read start at 16 different multiples of four banks).
-// 192-wide keys (multi-latent attention): 416 (104 dwords = 8 x 13: the same bank pattern as 288).
-template <int HD> constexpr int pp_pitch() { return HD == 192 ? 416 : HD == 128 ? 288 : 144; }
+// 192-wide keys (multi-latent attention): 416 (104 dwords = 8 x 13: the same bank pattern as 288); head_dim 96:
+// 208 (52 dwords = 4 x 13: the same pattern as 144).
+template <int HD> constexpr int pp_pitch() { return HD == 192 ? 416 : HD == 128 ? 288 : HD == 96 ? 208 : 144; }
 constexpr int kPPTile = 64;   // keys per staged tile
 
 // FP8: the cache holds e4m3 bytes with one fp32 scale per (chunk, KV head); a piece is multiplied by
@@ -372,18 +373,23 @@ constexpr int kPPTile = 64;   // keys per staged tile
 // caches of multi-latent attention, whose value cache has its own strides.
 template <bool STAGGER, bool FP8, bool SPLIT, int HD, int HDK, bool F16>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
-  static_assert((HD == 128 && HDK == 128) || (HD == 64 && HDK == 64 && !FP8) || (HD == 128 && HDK == 192 && !FP8),
-                "head_dim 128, or 64 with a 16-bit cache, or 192 / 128 with 16-bit caches");
+  static_assert((HD == 128 && HDK == 128) || ((HD == 64 || HD == 96) && HDK == HD && !FP8) || (HD == 128 && HDK == 192 && !FP8),
+                "head_dim 128, or 64 / 96 with a 16-bit cache, or 192 / 128 with 16-bit caches");
   static_assert(!(FP8 && F16), "an fp8 cache is staged as bf16: bf16 queries only");
   constexpr bool MLA = HDK != HD;
   constexpr int KS = HDK / 32, DV = HD / 16, NQ = 2, NT = 4, WAVES = 8;
   constexpr int kKPitch = pp_pitch<HDK>(), kVPitch = pp_pitch<HD>();
-  constexpr int PPRK = HDK * 2 / 16;                 // 16-byte pieces per key row when it differs from a value row: 24
-  constexpr int NPK = kPPTile * PPRK / 512;          // key pieces per loader thread and tile: 3 | 2 | 1
-  constexpr int PPR = HD * 2 / 16;       // 16-byte pieces (8 elements) per key row: 16 | 8
-  constexpr int RPP = 512 / PPR;         // key rows the 512 loader threads cover in one pass: 32 | 64
-  constexpr int NPASS = kPPTile / RPP;   // passes (rows per thread) per tile: 2 | 1
-  constexpr int NH = HD / 64;            // 64-column halves of the output
+  constexpr int PPRK = HDK * 2 / 16;                 // 16-byte pieces per key row: 24 | 16 | 12 | 8
+  constexpr int PPR = HD * 2 / 16;                   // 16-byte pieces (8 elements) per value row: 16 | 12 | 8
+  // Rows of 16 or 8 pieces divide the 512 loader threads into whole rows (a thread keeps its piece index and
+  // takes rows lkey, lkey + RPP); rows of 24 or 12 pieces do not: a thread then takes pieces tid, tid + 512, ...
+  // of the tile's 64 * pieces-per-row, as far as they exist ("flat").
+  constexpr bool FLAT_K = 512 % PPRK != 0, FLAT_V = 512 % PPR != 0;
+  constexpr int NPK = (kPPTile * PPRK + 511) / 512;  // key pieces per loader thread and tile: 3 | 2 | 2 | 1
+  constexpr int RPP = 512 / PPR;         // value rows the 512 loader threads cover in one pass: 32 | - | 64
+  constexpr int NPASS = (kPPTile * PPR + 511) / 512;  // value pieces per loader thread and tile: 2 | 2 | 1
+  constexpr int NH = HD == 64 ? 1 : 2;   // column groups of the output: 64 + 64, 48 + 48, or 64
+  constexpr int EPG = HD / 16 / NH;      // 16-column blocks per group: 4 | 3 | 4
   constexpr int ESZ = FP8 ? 1 : 2;       // bytes per cache element
   constexpr int PIECE = FP8 ? 8 : 16;    // bytes one loader thread fetches of a row (8 elements)
   __shared__ __attribute__((aligned(16))) uint8_t Ks[2][kPPTile * kKPitch];
@@ -487,17 +493,25 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     const uint32_t row_off0 = (uint32_t)(lkey * v_tok_bytes + lpiece * PIECE);
     const uint32_t row_off1 = row_off0 + (uint32_t)(RPP * v_tok_bytes);  // (second pass, head_dim 128 only)
     const uint32_t piece_off = (uint32_t)(lpiece * PIECE);
-    // 192-wide keys: 24 pieces per row do not divide the 512 loader threads into whole rows, so a thread
-    // takes pieces tid, tid + 512 and tid + 1024 of the tile's 1536
-    uint32_t mk_row_off[NPK], mk_piece_off[NPK];
-    int mk_lds[NPK];
-    if constexpr (MLA) {
+    // flat loader roles (a piece index past the tile's last repeats piece 0 and is not stored)
+    uint32_t mk_row_off[NPK], mk_piece_off[NPK], mv_row_off[NPASS], mv_piece_off[NPASS];
+    int mk_lds[NPK], mv_lds[NPASS];
+    if constexpr (FLAT_K) {
 #pragma unroll
       for (int i = 0; i < NPK; ++i) {
-        const int idx = tid + 512 * i, row = idx / PPRK, piece = idx - row * PPRK;
+        const int idx = tid + 512 * i < kPPTile * PPRK ? tid + 512 * i : 0, row = idx / PPRK, piece = idx - row * PPRK;
         mk_row_off[i] = (uint32_t)(row * tok_bytes + piece * 16);
         mk_piece_off[i] = (uint32_t)(piece * 16);
         mk_lds[i] = row * kKPitch + piece * 16;
+      }
+    }
+    if constexpr (FLAT_V) {
+#pragma unroll
+      for (int i = 0; i < NPASS; ++i) {
+        const int idx = tid + 512 * i < kPPTile * PPR ? tid + 512 * i : 0, row = idx / PPR, piece = idx - row * PPR;
+        mv_row_off[i] = (uint32_t)(row * v_tok_bytes + piece * 16);
+        mv_piece_off[i] = (uint32_t)(piece * 16);
+        mv_lds[i] = row * kVPitch + piece * 16;
       }
     }
     float ksc_staged = 1.f, vsc_staged = 1.f;  // fp8: scales of the tile held in kreg / vreg (per-lane copies)
@@ -558,12 +572,21 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       }
     };
     auto tile_loads_k = [&](int64_t off, int room) {
-      if constexpr (MLA) {
+      if constexpr (FLAT_K) {
         const uint8_t* tb = kbase + off;
 #pragma unroll
         for (int i = 0; i < NPK; ++i) kreg[i] = ld16(tb + min(mk_row_off[i], (uint32_t)room + mk_piece_off[i]));
       } else {
         tile_loads(kbase, off, room, kreg);
+      }
+    };
+    auto tile_loads_v = [&](int64_t off, int room) {
+      if constexpr (FLAT_V) {
+        const uint8_t* tb = vbase + off;
+#pragma unroll
+        for (int i = 0; i < NPASS; ++i) vreg[i] = ld16(tb + min(mv_row_off[i], (uint32_t)room + mv_piece_off[i]));
+      } else {
+        tile_loads(vbase, off, room, vreg);
       }
     };
     // what goes into LDS for one staged piece: the bf16 bits, or (fp8) 8 bytes -> 8 bf16 of byte * scale
@@ -575,9 +598,10 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
                         pack2<F16>(c.x * scale, c.y * scale), pack2<F16>(d.x * scale, d.y * scale));
     };
     auto store_k = [&](int t) {
-      if constexpr (MLA) {
+      if constexpr (FLAT_K) {
 #pragma unroll
-        for (int i = 0; i < NPK; ++i) *reinterpret_cast<uint4*>(&Ks[t & 1][mk_lds[i]]) = kreg[i];
+        for (int i = 0; i < NPK; ++i)
+          if (tid + 512 * i < kPPTile * PPRK) *reinterpret_cast<uint4*>(&Ks[t & 1][mk_lds[i]]) = kreg[i];
         return;
       }
       uint8_t* dst = &Ks[t & 1][k_off];
@@ -586,6 +610,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     };
     auto vbuf = [](int t) { return (unsigned)(t + 3) % 3u; };  // tile -1 lives in buffer 2
     auto store_v = [&](int t) {
+      if constexpr (FLAT_V) {
+#pragma unroll
+        for (int i = 0; i < NPASS; ++i)
+          if (tid + 512 * i < kPPTile * PPR) *reinterpret_cast<uint4*>(&Vs[vbuf(t)][mv_lds[i]]) = vreg[i];
+        return;
+      }
       uint8_t* dst = &Vs[vbuf(t)][v_off];
       *reinterpret_cast<uint4*>(dst) = lds_piece(vreg[0], vsc_staged);
       if constexpr (NPASS == 2) *reinterpret_cast<uint4*>(dst + RPP * kVPitch) = lds_piece(vreg[1], vsc_staged);
@@ -632,22 +662,22 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         s[1][u] = mfma_16x16x32<F16>(kf[j], qf[1][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[1][u]);
       }
     };
-    // O^T += V^T P^T: group grp = (32-key step grp / 2, output columns 64 * (grp % 2) ..+63):
-    // 8 transposed reads, 8 MFMAs (+2 for the denominators in the odd groups)
+    // O^T += V^T P^T: group grp = (32-key step grp / NH, output column group grp % NH of 64 or 48 columns):
+    // 8 (6) transposed reads, 8 (6) MFMAs (+2 for the denominators in the last group of a step)
     auto pv_load = [&](int t, int grp, uint2 (&af)[4][2]) {
-      const uint8_t* vs = Vs[vbuf(t)] + vfrag_off + 32 * (grp / NH) * kVPitch + 128 * (grp % NH);
+      const uint8_t* vs = Vs[vbuf(t)] + vfrag_off + 32 * (grp / NH) * kVPitch + 32 * EPG * (grp % NH);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
+      for (int e = 0; e < EPG; ++e) {
         af[e][0] = lds_ld8_tr(vs + 32 * e);
         af[e][1] = lds_ld8_tr(vs + 16 * kVPitch + 32 * e);
       }
     };
     auto pv_mma = [&](int grp, const uint2 (&af)[4][2]) {
-      const int up = 2 * (grp / NH), e0 = 4 * (grp % NH);
+      const int up = 2 * (grp / NH), e0 = EPG * (grp % NH);
       const uint4 pp0 = make_uint4(pf[0][up].x, pf[0][up].y, pf[0][up + 1].x, pf[0][up + 1].y);
       const uint4 pp1 = make_uint4(pf[1][up].x, pf[1][up].y, pf[1][up + 1].x, pf[1][up + 1].y);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
+      for (int e = 0; e < EPG; ++e) {
         const uint4 a = make_uint4(af[e][0].x, af[e][0].y, af[e][1].x, af[e][1].y);
         acc[0][e0 + e] = mfma_16x16x32<F16>(a, pp0, acc[0][e0 + e]);
         acc[1][e0 + e] = mfma_16x16x32<F16>(a, pp1, acc[1][e0 + e]);
@@ -689,7 +719,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         MI_SB();
         sc_load(ts, 0, k0); MI_SB();
         pv_mma(1, a1);
-        tile_loads(vbase, off, room, vreg); MI_SB();
+        tile_loads_v(off, room); MI_SB();
         sc_load(ts, 1, k1); MI_SB(); sc_mma(0, k0); MI_SB();
         sc_load(ts, 2, k0); MI_SB(); sc_mma(1, k1); MI_SB();
         sc_load(ts, 3, k1); MI_SB(); sc_mma(2, k0); MI_SB();
@@ -719,7 +749,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       MI_SB();
       pv_load(ta, 3, a1); MI_SB();
       pv_mma(2, a0);
-      tile_loads(vbase, off_v, room_v, vreg); MI_SB();
+      tile_loads_v(off_v, room_v); MI_SB();
       if constexpr (MLA) {
         uint4 h0[3], h1[3];
         sc_load_half(ts, 0, 0, h0); MI_SB();
@@ -805,13 +835,13 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       const int pc0 = bt_row[c0.ci], pc1 = bt_row[c1.ci];
       const int64_t off0 = tile_offset(c0, pc0);
       tile_loads_k(off0, c0.room);
-      tile_loads(vbase, MLA ? tile_offset_v(c0, pc0) : off0, MLA ? c0.room_v : c0.room, vreg);
+      tile_loads_v(MLA ? tile_offset_v(c0, pc0) : off0, MLA ? c0.room_v : c0.room);
       store_k(0);
       store_v(0);
       __syncthreads();  // K(0), V(0) and the zero-filled buffer are visible; the staging registers are free
       const int64_t off1 = tile_offset(c1, pc1);
       tile_loads_k(off1, c1.room);  // K(1), V(1): stored by matrix(0)
-      tile_loads(vbase, MLA ? tile_offset_v(c1, pc1) : off1, MLA ? c1.room_v : c1.room, vreg);
+      tile_loads_v(MLA ? tile_offset_v(c1, pc1) : off1, MLA ? c1.room_v : c1.room);
       pc_cur = bt_row[cur.ci];
     }
     if (lead) __syncthreads();  // second group idles through phase 0
@@ -911,7 +941,7 @@ using namespace mi;
 // with thousands of keys to walk: then the keys are split so that about one workgroup per CU exists,
 // every one keeping at least sixteen 64-key tiles (a 512-token prompt is not worth the merge).  Host-side quantities only (the lengths live on the GPU).
 static int prefill_kv_splits(int T, int Hq, int Hkv, int head_dim, int max_kv_len) {
-  if ((head_dim != 128 && head_dim != 64) || max_kv_len <= 0) return 1;
+  if ((head_dim != 128 && head_dim != 64 && head_dim != 96) || max_kv_len <= 0) return 1;
   const int G = Hq / Hkv, Gw = G < 16 ? G : 16, parts = (G + 15) / 16;
   const int sbq = 8 * (32 / Gw);                         // query tokens per workgroup (8 wavefronts x 32 rows)
   const int64_t useful = (int64_t)Hkv * parts * ((T + sbq - 1) / sbq);
@@ -996,7 +1026,7 @@ static int launch_paged_prefill(
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_fp8: both scale arrays are required");
   // the two-phase tile kernel stages 64-key tiles that must not straddle chunks and exists for the common widths;
   // other chunk sizes and widths (and the knob) select the register-only kernel
-  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0 && (head_dim == 64 || head_dim == 128);
+  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0 && head_dim <= 128;
   if (fp8 && (head_dim != 128 || !two_phase || f16))
     return mi_fail(MI_ERR_UNSUPPORTED,
                    "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 128, a chunk size that is a "
@@ -1050,8 +1080,10 @@ static int launch_paged_prefill(
     if (fp8) MI_PP_LAUNCH(true, 128, 128, false);
     else if (head_dim == 128 && f16) MI_PP_LAUNCH(false, 128, 128, true);
     else if (head_dim == 128) MI_PP_LAUNCH(false, 128, 128, false);
-    else if (f16) MI_PP_LAUNCH(false, 64, 64, true);
-    else MI_PP_LAUNCH(false, 64, 64, false);
+    else if (head_dim == 64 && f16) MI_PP_LAUNCH(false, 64, 64, true);
+    else if (head_dim == 64) MI_PP_LAUNCH(false, 64, 64, false);
+    else if (f16) MI_PP_LAUNCH(false, 96, 96, true);
+    else MI_PP_LAUNCH(false, 96, 96, false);
     if (timed) (void)hipEventRecord(ev_b, st);
     if (n_split > 1) {
       if (f16) hipLaunchKernelGGL(prefill_split_merge_kernel<true>, dim3(T, Hq), dim3(head_dim), 0, st, p, n_split, head_dim);

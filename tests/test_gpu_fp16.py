@@ -79,7 +79,7 @@ def test_mismatched_types_are_rejected(mi, dev):
 
 
 @pytest.mark.parametrize("kernel", ["two_phase", "two_phase_lock_step", "registers", "split_keys"])
-@pytest.mark.parametrize("Hq,Hkv,d", [(32, 8, 128), (8, 8, 64), (12, 4, 128), (16, 1, 64)])
+@pytest.mark.parametrize("Hq,Hkv,d", [(32, 8, 128), (8, 8, 64), (12, 4, 128), (16, 1, 64), (32, 8, 96)])
 def test_prefill_and_mixed_batches(mi, dev, kernel, Hq, Hkv, d):
     knobs = {"two_phase": {}, "two_phase_lock_step": {"prefill_two_phase": 2}, "registers": {"prefill_two_phase": -1},
              "split_keys": {"prefill_kv_split": 3}}[kernel]

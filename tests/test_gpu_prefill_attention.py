@@ -76,9 +76,9 @@ def test_padded_requests_with_zero_lengths(mi, dev):
 @pytest.mark.parametrize("pingpong", [1, 2])
 @pytest.mark.parametrize("chunk", [64, 128, 256])
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 1), (16, 2)])
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 96])
 def test_two_phase_kernel_ragged_lengths(mi, dev, pingpong, chunk, Hq, Hkv, d):
-    """The two-phase tile kernel (head_dim 128 or 64, chunk a multiple of 64): new-token counts and cached
+    """The two-phase tile kernel (head_dim 128, 96 or 64, chunk a multiple of 64): new-token counts and cached
     contexts around every tile (64 keys), workgroup (256 rows) and chunk boundary, for 1, 2, 4, 8
     and 16 query heads per KV head, staggered and lock-step."""
     q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 500, 256, 257, 3]
@@ -129,16 +129,20 @@ def _check_padded(mi, q, kc, vc, cu_q, lens, bt, tol=2e-2):
 @pytest.mark.parametrize("Hq,Hkv", [(8, 8), (32, 8), (12, 4), (16, 1)])
 @pytest.mark.parametrize("d", [96, 192, 256])
 def test_head_widths_96_192_256(mi, dev, d, Hq, Hkv, chunk, dtype):
-    """Head widths beside 64 and 128 in prefill and mixed batches: ragged new-token counts and contexts, one-row
-    requests through the decode kernels (default) and through the prefill kernel (no workspace -> forced below by
-    the register-only knob), padding rows."""
+    """Head widths beside 64 and 128 in prefill and mixed batches (96: the two-phase tile kernel when the chunk size
+    allows, split keys included; 192 and 256: the register-only kernel): ragged new-token counts and contexts,
+    one-row requests through the decode kernels, padding rows."""
     q, kc, vc, cu_q, lens, bt = _ragged_case(mi, dev, Hq, Hkv, d, chunk, dtype, seed=d + Hq + chunk, pad_rows=3)
     _check_padded(mi, q, kc, vc, cu_q, lens, bt)
+    if d == 96 and chunk % 64 == 0:
+        for knobs in ({"prefill_kv_split": 3}, {"prefill_two_phase": 2}, {"prefill_two_phase": -1}):
+            with mi.ops.tuning(**knobs):
+                _check_padded(mi, q, kc, vc, cu_q, lens, bt)
 
 
 @pytest.mark.parametrize("kernel", ["two_phase", "registers", "split_keys"])
 @pytest.mark.parametrize("Hq,Hkv", [(32, 1), (64, 2), (17, 1), (48, 2), (40, 2), (64, 1)])
-@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("d", [64, 96, 128, 256])
 def test_more_than_16_query_heads_per_kv_head(mi, dev, kernel, Hq, Hkv, d):
     """Up to 64 query heads per KV head: every 16 of them (the last group: the rest) take workgroups of their own."""
     if d == 256 and kernel != "registers":

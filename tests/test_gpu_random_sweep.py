@@ -67,9 +67,9 @@ def widen_table(bt, extra, fill):
 
 def case_decode(mi, dev, rng, seed, fp8):
     gen = torch.Generator().manual_seed(seed)
-    d = rng.choice([64, 128])
+    d = 128 if fp8 else rng.choice([64, 128, 64, 128, 96, 192, 256])
     Hkv = rng.choice([1, 2, 3, 4, 8, 16])
-    G = rng.choice([1, 2, 3, 4, 5, 7, 8, 16])
+    G = rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 17, 24, 32] if Hkv <= 2 else [1, 2, 3, 4, 5, 7, 8, 16])
     Hq = Hkv * G
     chunk = rng.choice([16, 32, 48, 64, 80, 128, 256])
     R = rng.randint(1, 24)
@@ -125,9 +125,9 @@ def case_decode(mi, dev, rng, seed, fp8):
 
 def case_prefill(mi, dev, rng, seed, fp8):
     gen = torch.Generator().manual_seed(seed)
-    d = rng.choice([64, 128]) if not fp8 else 128
+    d = rng.choice([64, 128, 64, 128, 96, 96, 192, 256]) if not fp8 else 128
     Hkv = rng.choice([1, 2, 4, 8])
-    G = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16])
+    G = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 20, 32] if Hkv <= 2 else [1, 2, 3, 4, 5, 7, 8, 12, 16])
     Hq = Hkv * G
     chunk = rng.choice([16, 32, 64, 128, 256])
     R = rng.randint(1, 10)
@@ -370,7 +370,7 @@ def case_append_fp8(mi, dev, rng, seed):
 def case_norm_rope(mi, dev, rng, seed):
     gen = torch.Generator().manual_seed(seed)
     chunk = rng.choice([16, 64, 256])
-    d = rng.choice([64, 128])
+    d = rng.choice([64, 128, 64, 128, 96, 192, 256])
     rot = rng.choice([d, d // 2, d, 32])
     Hkv = rng.choice([1, 2, 4, 8])
     Hq = Hkv * rng.choice([1, 2, 3, 4, 5, 7])
