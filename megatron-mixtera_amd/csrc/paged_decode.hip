@@ -787,6 +787,9 @@ static int merge_groups(int grid_x, int R, int head_dim) {
   return g < 1 ? 1 : g;
 }
 
+// Requests one launch of the streaming kernels takes: their tile prefix sums and lengths sit in LDS.
+constexpr int kMaxRequestsPerLaunch = 7680;
+
 // Wavefronts along the heads: one per KV head and 16 query heads that share it.
 static int head_waves(int Hq, int Hkv) { return Hkv * ((Hq / Hkv + 15) / 16); }
 
@@ -876,8 +879,28 @@ int mi::launch_paged_decode(
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: one chunk must span less than 2 GiB");
   if (split_tokens < 0 || split_tokens % 16)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: split_tokens must be a non-negative multiple of 16");
-  if ((int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: batch too large for the in-LDS prefix sum (7680 requests)");
+  // The per-request prefix sums and lengths live in LDS (8 bytes per request): a larger batch is streamed in
+  // slices of kMaxRequestsPerLaunch requests, one after the other on the same stream and workspace.  Every
+  // argument check above is independent of the slice, so either all slices run or none does.
+  if (R > kMaxRequestsPerLaunch) {
+    const int64_t slots_all = (int64_t)decode_grid_size(Hq, Hkv, tune) + kMaxRequestsPerLaunch;
+    if (!workspace || workspace_bytes < slots_all * Hq * (head_dim + 1) * (int64_t)sizeof(float) +
+                                            (int64_t)kMaxRequestsPerLaunch * 2 * (int64_t)sizeof(int32_t))
+      return mi_fail(MI_ERR_WORKSPACE, "mi_paged_decode_attention: workspace too small (see mi_decode_workspace_bytes)");
+    for (int r0 = 0; r0 < R; r0 += kMaxRequestsPerLaunch) {
+      const int n = R - r0 < kMaxRequestsPerLaunch ? R - r0 : kMaxRequestsPerLaunch;
+      // with cu_seqlens_q the rows of q / out are addressed through it, else request r owns row r
+      const int64_t row0 = cu_seqlens_q ? 0 : r0;
+      const int rc = launch_paged_decode(
+          (const uint16_t*)q + row0 * q_stride_tok, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk,
+          kv_stride_tok, kv_stride_head, block_table + (int64_t)r0 * bt_stride, bt_stride, kv_lens + r0,
+          cu_seqlens_q ? cu_seqlens_q + r0 : nullptr, (uint16_t*)out + row0 * o_stride_tok, o_stride_tok, o_stride_head,
+          workspace, workspace_bytes, n, Hq, Hkv, head_dim, chunk_tokens, split_tokens, softmax_scale, kv_dtype, k_scales,
+          v_scales, dtype, tune, stream);
+      if (rc != MI_OK) return rc;
+    }
+    return MI_OK;
+  }
 
   const int grid_x = decode_grid_size(Hq, Hkv, tune);
   const int64_t slots = (int64_t)grid_x + R;
@@ -1107,8 +1130,20 @@ extern "C" int mi_paged_mla_decode_attention(
   if (kv_stride_tok < head_dim_k || kv_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_mla_decode_attention: bad token stride, or a chunk of 2 GiB or more");
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_mla_decode_attention: softmax_scale must be positive");
-  if ((int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: batch too large for the in-LDS prefix sum (7680 requests)");
+  if (R > kMaxRequestsPerLaunch) {  // slices, as in launch_paged_decode
+    if (!workspace || workspace_bytes < mi_mla_decode_workspace_bytes(kMaxRequestsPerLaunch, Hq, head_dim_v, tuning))
+      return mi_fail(MI_ERR_WORKSPACE, "mi_paged_mla_decode_attention: workspace too small (see mi_mla_decode_workspace_bytes)");
+    for (int r0 = 0; r0 < R; r0 += kMaxRequestsPerLaunch) {
+      const int n = R - r0 < kMaxRequestsPerLaunch ? R - r0 : kMaxRequestsPerLaunch;
+      const int rc = mi_paged_mla_decode_attention(
+          (const uint16_t*)q + (int64_t)r0 * q_stride_tok, q_stride_tok, q_stride_head, kv_cache, kv_stride_chunk,
+          kv_stride_tok, block_table + (int64_t)r0 * bt_stride, bt_stride, kv_lens + r0,
+          (uint16_t*)out + (int64_t)r0 * o_stride_tok, o_stride_tok, o_stride_head, workspace, workspace_bytes, n, Hq,
+          head_dim_k, head_dim_v, chunk_tokens, max_kv_len, softmax_scale, dtype, tuning, stream);
+      if (rc != MI_OK) return rc;
+    }
+    return MI_OK;
+  }
 
   const int groups = mla_groups(Hq);
   // Two kernels: the latent tile shared through LDS by the eight wavefronts of a workgroup (needs tiles

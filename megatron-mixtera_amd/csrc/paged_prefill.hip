@@ -1032,10 +1032,7 @@ static int launch_paged_prefill(
                    "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 128, a chunk size that is a "
                    "multiple of 64 and the two-phase tile kernel");
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
-  // Everything is checked before the first launch: the decode part of a mixed batch must not be rejected after
-  // the tile kernel has written its rows.
-  if (workspace && (int64_t)R * 2 * sizeof(int32_t) > 60 * 1024)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: batch too large for the in-LDS prefix sum (7680 requests)");
+  // (no limit on the number of requests: the decode part of a mixed batch runs in slices when it has to)
 
   PrefillParams p;
   p.q = (const uint16_t*)q; p.q_st = q_stride_tok; p.q_sh = q_stride_head;

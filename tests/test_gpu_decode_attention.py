@@ -116,6 +116,32 @@ def test_more_than_16_query_heads_per_kv_head(mi, dev, Hq, Hkv, d):
         _close(out, ref8, 2e-2)
 
 
+def test_more_requests_than_one_launch_takes(mi, dev):
+    """The streaming kernels keep 8 bytes per request in LDS, 7 680 requests per launch; the reference has no
+    such limit (a decode step without a graph pads to max_requests), so larger batches run in slices."""
+    R = 7680 + 7680 + 300
+    gen = torch.Generator().manual_seed(5)
+    lens = torch.randint(0, 70, (R,), generator=gen, dtype=torch.int32)
+    cfg = mi.synthetic.DecodeConfig("many", R, 8, 2, 64, 0, 0, chunk=16, seed=2)
+    case = mi.synthetic.make_decode_case(cfg, dev, lens=lens)
+    out = _run_case(mi, case, max_kv_len=70)
+    _close(out, _ref(case), 2e-2)
+    assert (out[case.kv_lens == 0] == 0).all()
+    # a mixed batch whose one-row requests exceed the limit: 3 prompts + R one-token requests
+    q_lens = [40, 1, 130] + [1] * R
+    kv = torch.cat([torch.tensor([100, 9, 130], dtype=torch.int32), lens.clamp(min=1)])
+    cu_q = torch.zeros(len(q_lens) + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+    bt, N = mi.synthetic.build_block_table(kv, 16, gen)
+    q = torch.randn(int(cu_q[-1]), 8, 64, generator=gen).bfloat16()
+    kc = torch.randn(N, 16, 2, 64, generator=gen).bfloat16()
+    vc = torch.randn(N, 16, 2, 64, generator=gen).bfloat16()
+    got = mi.ops.paged_prefill_attention(q.to(dev), kc.to(dev), vc.to(dev), cu_q.to(dev), kv.to(dev), bt.to(dev),
+                                         max_kv_len=int(kv.max()))
+    torch.cuda.synchronize()
+    _close(got, oa.paged_varlen_attention(q, kc, vc, cu_q, kv, bt), 2e-2)
+
+
 def test_block_table_width_and_padding_rows(mi, dev):
     """Block table wider than needed (graph mode passes max_sequence_length) with -1 / 0 padding."""
     cfg = mi.synthetic.DecodeConfig("wide", 6, 32, 8, 128, 100, 2000, chunk=256, seed=5)

@@ -71,6 +71,14 @@ def test_mla_decode_many_requests_fall_back_to_streaming(mi, dev):
     _check(mi, dev, q, cache, lens, bt, scale=0.07)
 
 
+def test_mla_decode_more_requests_than_one_launch_takes(mi, dev):
+    """Beyond 7 680 requests (8 bytes of LDS each) the call runs in slices."""
+    g = torch.Generator().manual_seed(21)
+    lens = torch.randint(0, 40, (7680 + 500,), generator=g).tolist()
+    q, cache, lens, bt = _case(mi, dev, lens, 8, 16, seed=22)
+    _check(mi, dev, q, cache, lens, bt, scale=0.07)
+
+
 def test_mla_decode_chunk_permutation_and_cache_view(mi, dev):
     """Moving the rows to other physical chunks changes nothing; a [N, C, 1, 576] cache view is accepted."""
     q, cache, lens, bt = _case(mi, dev, [100, 333, 64], 32, 64, seed=4)
