@@ -297,6 +297,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--hip-graph", action="store_true", help="replay the step as one captured HIP graph")
     ap.add_argument("--attention-only", action="store_true", help="time the attention call alone")
+    ap.add_argument("--separate-launches", action="store_true",
+                    help="decode workloads: norm / RoPE / append as a launch of its own before the attention call")
     ap.add_argument("--fp8-kv", action="store_true", help="cfg3 only: run the mixed batch over an fp8-e4m3 KV cache")
     ap.add_argument("--read-mib", type=int, default=1146,
                     help="stream_read only: buffer size (default: the 1.2 GB one cfg2 launch streams)")
@@ -580,7 +582,17 @@ def main():
     out = torch.empty_like(case.q)
     use_norm = "rms"
 
+    # the whole step inside the streaming kernel (16-bit caches, head_dim 64 / 128) unless asked otherwise
+    one_kernel = (not cfg.fp8 and not args.attention_only and not args.separate_launches
+                  and mi.ops.decode_step_supported(cfg.d, cfg.d, False, False))
+
     def step():
+        if one_kernel:
+            mi.ops.decode_step_attention(case.q, case.k_new, case.v_new, case.k_cache, case.v_cache, case.kv_lens,
+                                         case.block_table, q_weight=qw, k_weight=kw, eps=1e-5, norm=use_norm,
+                                         rotary_emb=table, positions=None, out=out, max_kv_len=max_len,
+                                         split_tokens=args.split_tokens)  # (positions: kv_lens - 1)
+            return
         if not args.attention_only:
             if cfg.fp8:
                 mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_in, key_out=k_rot, q_weight=qw, k_weight=kw, eps=1e-5,
@@ -643,6 +655,35 @@ def main():
     ms_per_step = elapsed * 1e3 / args.steps
     nbytes = mi.synthetic.decode_attention_bytes(lens_host.tolist(), cfg.Hq, cfg.Hkv, cfg.d, cfg.chunk,
                                        kv_bytes=1 if cfg.fp8 else 2, fp8_scales=cfg.fp8)
+
+    # The same step as three launches (norm / RoPE / append, then the attention-only streaming kernel, then the
+    # merge), timed right after: its streaming kernel does attention alone, so its rate is the one to hold
+    # against the HBM roofline kernel for kernel; the one-kernel step trades a little of that for a launch.
+    separate = None
+    if one_kernel:
+        def step_separate():
+            mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_in, value=case.v_new, q_weight=qw, k_weight=kw,
+                                    eps=1e-5, norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos,
+                                    k_cache=case.k_cache, v_cache=case.v_cache, block_table=case.block_table,
+                                    kv_lens=case.kv_lens)
+            mi.ops.paged_decode_attention(q_in, case.k_cache, case.v_cache, case.kv_lens, case.block_table, out=out,
+                                          max_kv_len=max_len, split_tokens=args.split_tokens)
+        for _ in range(args.warmup):
+            step_separate()
+        torch.cuda.synchronize()
+        lib.mi_profile_enable(1)
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step_separate()
+        torch.cuda.synchronize()
+        sep_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        n_sep = lib.mi_profile_collect(buf, args.steps)
+        lib.mi_profile_enable(0)
+        sep_kernel_ms = sum(buf[i] for i in range(min(n_sep, args.steps))) / max(1, min(n_sep, args.steps))
+        separate = {"ms_per_step": round(sep_ms, 5), "value": round(nbytes / (sep_ms * 1e-3) / 1e9, 1),
+                    "kernel": "paged_decode_stream_kernel", "kernel_ms": round(sep_kernel_ms, 5),
+                    "achieved": round(nbytes / (sep_kernel_ms * 1e-3) / 1e9, 1),
+                    "frac": round(nbytes / (sep_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
     value = nbytes / (ms_per_step * 1e-3) / 1e9
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9
 
@@ -661,6 +702,8 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": cfg.name + (", attention call only" if args.attention_only
+                                    else ", step = RMSNorm+RoPE+KV-append inside the paged decode attention kernel, then merge"
+                                    if one_kernel
                                     else ", step = fused RMSNorm+RoPE+KV-append then paged decode attention")
             + (", replayed as one HIP graph" if args.hip_graph else ""),
             "batch": case.q.size(0), "q_heads": cfg.Hq, "kv_heads": cfg.Hkv, "head_dim": cfg.d,
@@ -671,7 +714,7 @@ def main():
         "decode_steps_per_sec": round(1e3 / ms_per_step, 1),
         "roofline": {
             "bound": "hbm",
-            "kernel": "paged_decode_stream_kernel",
+            "kernel": "decode_step_stream_kernel" if one_kernel else "paged_decode_stream_kernel",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -681,6 +724,8 @@ def main():
             "traffic_source": TRAFFIC_SOURCE.get(args.workload),
         },
     }
+    if separate is not None:
+        result["separate_launches"] = separate
     if not args.no_cpu_baseline:
         sample = {"cfg1": 4, "cfg2": 64, "cfg3_decode": 64, "cfg4": 1, "cfg5": 16}[args.workload]
         result["cpu_baseline"] = cpu_baseline(case, cfg, sample, qw, kw, table, args.attention_only)

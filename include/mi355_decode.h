@@ -188,6 +188,39 @@ int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_str
                               int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
+ * One decode step of a layer in two launches instead of three: what mi_norm_rope_append (or
+ * mi_qkv_norm_rope_append) followed by mi_paged_decode_attention computes for R one-token requests, i.e.
+ * the sequence q_layernorm / k_layernorm (attention.py:1026-1030), apply_rotary_emb_query / _key
+ * (dynamic_context.py:566-631), append_key_value_cache (dynamic_context.py:511-545) and
+ * flash_attn_with_kvcache (attention.py:589-600).  The head norm, the rotary embedding and the append of the
+ * step's token ride in the streaming kernel: every span of keys prepares its query rows in registers, and the
+ * span that ends a request writes the request's new key and value rows into their cache slot
+ * (block_table[r, (kv_lens[r] - 1) / chunk_tokens], position (kv_lens[r] - 1) % chunk_tokens) before it reads
+ * them.  q holds the RAW queries: head h * G + u of request r at r * q_stride_tok + h * q_stride_group + u * d
+ * (a `[R, Hq, d]` tensor: q_stride_group = G * d; the QKV projection's output `[R, Hkv, (G + 2) * d]`:
+ * q_stride_group = (G + 2) * d, k_new = q + G * d, v_new = q + (G + 1) * d, both with head stride
+ * (G + 2) * d).  positions int64 [R] index rotary_angles; NULL = kv_lens[r] - 1, the position of the step's token
+ * in its request (what token_to_pos_ids holds on a decode step, and one load fewer on the way to the first
+ * product).  Same arithmetic and rounding points as
+ * mi_norm_rope_append (faithful_rounding as there); the normed queries are not written anywhere.
+ * Limits: 16-bit caches, head_dim 64 or 128, half-split rotary pairs with rot_dim / 2 a multiple of 32 (or
+ * interleaved pairs, or no rotary embedding); anything else is MI_ERR_UNSUPPORTED and takes the separate calls.
+ * Workspace as for mi_paged_decode_attention.  Rows with kv_lens[r] == 0 append nothing and produce zeros.
+ */
+int mi_decode_step_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new,
+                             int64_t k_stride_tok, int64_t k_stride_head, const void* v_new,
+                             int64_t v_stride_tok, int64_t v_stride_head, const void* q_weight,
+                             const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles,
+                             int64_t angles_stride, int32_t rot_dim, int32_t rotary_interleaved, float mscale,
+                             const int64_t* positions, void* k_cache, void* v_cache, int64_t kv_stride_chunk,
+                             int64_t kv_stride_tok, int64_t kv_stride_head, const int32_t* block_table,
+                             int64_t bt_stride, const int32_t* kv_lens, void* out, int64_t o_stride_tok,
+                             int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R,
+                             int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
+                             int32_t split_tokens, float softmax_scale, int32_t faithful_rounding,
+                             int32_t dtype, const MiTuning* tuning, void* stream);
+
+/*
  * mi_paged_decode_attention for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments and results as mi_paged_decode_attention, minus the workspace: the

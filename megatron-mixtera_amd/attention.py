@@ -105,6 +105,11 @@ class PagedSelfAttentionCore(torch.nn.Module):
             assert q_emb is k_emb or q_emb is None or k_emb is None or q_emb.data_ptr() == k_emb.data_ptr(), \
                 "the fused path takes one rotary table for query and key"
             emb = q_emb if q_emb is not None else k_emb
+        if self.fused and self._step_fusable(ctx, emb):
+            out = ctx.fused_decode_step_attention(
+                self.layer_number, mixed_qkv=mixed_qkv, num_query_heads=num_query_heads, rotary_pos_emb=emb,
+                softmax_scale=self.softmax_scale, **self._norm_args())
+            return out.reshape(out.size(0), out.size(1), -1)
         query = ctx.fused_qkv_norm_rope_append(
             self.layer_number, mixed_qkv, num_query_heads=num_query_heads, rotary_pos_emb=emb, config=self.config,
             q_weight=None if self.q_layernorm_weight is None else self.q_layernorm_weight.data,
@@ -121,6 +126,11 @@ class PagedSelfAttentionCore(torch.nn.Module):
         if self.fused:
             assert q_emb is k_emb or q_emb is None or k_emb is None or q_emb.data_ptr() == k_emb.data_ptr(), \
                 "the fused path takes one rotary table for query and key"
+            if self._step_fusable(ctx, q_emb if q_emb is not None else k_emb):
+                out = ctx.fused_decode_step_attention(
+                    self.layer_number, query, key, value, rotary_pos_emb=q_emb if q_emb is not None else k_emb,
+                    softmax_scale=self.softmax_scale, **self._norm_args())
+                return out.reshape(out.size(0), out.size(1), -1)
             ctx.fused_qk_norm_rope_append(
                 self.layer_number, query, key, value, rotary_pos_emb=q_emb if q_emb is not None else k_emb,
                 config=self.config, q_weight=None if self.q_layernorm_weight is None else self.q_layernorm_weight.data,
@@ -139,6 +149,17 @@ class PagedSelfAttentionCore(torch.nn.Module):
             if q_emb is not None:
                 query = ctx.apply_rotary_emb_query(query, q_emb, self.config, None, None)
         return self._attend(query, ctx)
+
+    def _norm_args(self) -> dict:
+        return dict(config=self.config, norm=self.qk_norm, eps=self.eps,
+                    q_weight=None if self.q_layernorm_weight is None else self.q_layernorm_weight.data,
+                    k_weight=None if self.k_layernorm_weight is None else self.k_layernorm_weight.data)
+
+    def _step_fusable(self, ctx, emb: Optional[Tensor]) -> bool:
+        """Decode-only steps over 16-bit caches run norm, RoPE, append and attention as one streaming kernel
+        (plus its merge) when the shapes allow; a context without that method keeps the separate launches."""
+        check = getattr(ctx, "decode_step_fusable", None)
+        return check is not None and check(self.head_dim, emb, self.config)
 
     def _attend(self, query: Tensor, ctx) -> Tensor:
         k_cache, v_cache, block_table = ctx.key_value_cache(self.layer_number)

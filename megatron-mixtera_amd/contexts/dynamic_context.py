@@ -518,6 +518,51 @@ class DynamicInferenceContext:
             faithful_rounding=faithful_rounding)
         return query
 
+    def decode_step_fusable(self, head_dim: int, rotary_pos_emb: Optional[Tensor], config=None) -> bool:
+        """Whether this step can run :meth:`fused_decode_step_attention`: a decode-only step over 16-bit per-head
+        caches with shapes the fused kernel has (``ops.decode_step_supported``)."""
+        if not self.is_decode_only() or self.cache_mla_latent or self.kv_cache_fp8:
+            return False
+        rot = 0 if rotary_pos_emb is None else rotary_pos_emb.size(-1)
+        interleaved = self._rope_flags(config) if config is not None else False
+        return ops.decode_step_supported(head_dim, rot, interleaved, False)
+
+    def fused_decode_step_attention(self, layer_number: int, query: Optional[Tensor] = None,
+                                    key: Optional[Tensor] = None, value: Optional[Tensor] = None, *,
+                                    mixed_qkv: Optional[Tensor] = None, num_query_heads: int = 0,
+                                    rotary_pos_emb: Optional[Tensor] = None, config=None,
+                                    q_weight: Optional[Tensor] = None, k_weight: Optional[Tensor] = None,
+                                    norm: Optional[str] = None, eps: float = 1e-5, mscale: float = 1.0,
+                                    softmax_scale: Optional[float] = None, faithful_rounding: bool = True) -> Tensor:
+        """A decode-only step of one layer in two launches: q/k norm, RoPE(q, k), append(k, v) and the attention
+        over the layer's cache (attention.py:1026-1030, 394-414, 589-600) -- :meth:`fused_qk_norm_rope_append`
+        (or :meth:`fused_qkv_norm_rope_append`) and ``flash_attn_with_kvcache`` in one streaming kernel plus its
+        merge.  Takes ``query`` / ``key`` / ``value`` ``[T, 1, H, d]`` or ``mixed_qkv`` ``[T, 1, (Hq + 2 Hkv) d]``;
+        returns the attention output ``[T, 1, Hq, d]`` (rows past the padded token count are left unwritten).
+        Row i is request i of the step: its token is appended at position ``kv_seq_lengths[i] - 1`` of the
+        request's chunks, which is where ``token_to_chunk_idx`` / ``token_to_local_position_within_kv_chunk``
+        point on a decode step; query and key rotate by that same position, which is what ``token_to_pos_ids``
+        and ``token_to_position_in_request`` hold on a decode step (``update_requests`` sets both to
+        ``request_kv_length_offsets``, dynamic_context.py:1248-1254; a one-token prompt starts at 0)."""
+        n = self.padded_active_token_count
+        k_cache, v_cache, block_table = self.key_value_cache(layer_number)
+        _, k_bound = self.attention_length_bounds()
+        common = dict(q_weight=q_weight, k_weight=k_weight, eps=eps, norm=norm, rotary_emb=rotary_pos_emb,
+                      positions=None,  # = kv_seq_lengths - 1, see the docstring
+                      rotary_interleaved=self._rope_flags(config) if config is not None else False, mscale=mscale,
+                      softmax_scale=softmax_scale, max_kv_len=k_bound, faithful_rounding=faithful_rounding)
+        if mixed_qkv is not None:
+            d = self.kv_channels
+            out = torch.empty((mixed_qkv.size(0), 1, num_query_heads, d), dtype=mixed_qkv.dtype, device=mixed_qkv.device)
+            ops.decode_step_attention(None, None, None, k_cache, v_cache, self.kv_seq_lengths, block_table,
+                                      mixed_qkv=mixed_qkv[:n], num_query_heads=num_query_heads,
+                                      num_kv_heads=self.num_kv_heads_per_partition, out=out[:n], **common)
+            return out
+        out = torch.empty_like(query)
+        ops.decode_step_attention(query[:n], key[:n], value[:n], k_cache, v_cache, self.kv_seq_lengths, block_table,
+                                  out=out[:n], **common)
+        return out
+
     def fused_qkv_norm_rope_append(self, layer_number: int, mixed_qkv: Tensor, *, num_query_heads: int,
                                    rotary_pos_emb: Optional[Tensor], config=None,
                                    q_weight: Optional[Tensor] = None, k_weight: Optional[Tensor] = None,

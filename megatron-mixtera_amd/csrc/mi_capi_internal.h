@@ -22,6 +22,24 @@ bool mi_profile_next(hipEvent_t* start, hipEvent_t* stop);
 
 namespace mi {
 int decode_grid_size(int Hq, int Hkv, const MiTuning& tune);
+// What a fused decode step hands the streaming kernel beside the attention arguments (see mi_decode_step_attention).
+struct FusedStepArgs {
+  int64_t q_stride_group;  // elements between the query-head groups of two KV heads (heads of a group are contiguous)
+  const void* k_new;
+  int64_t k_stride_tok, k_stride_head;
+  const void* v_new;
+  int64_t v_stride_tok, v_stride_head;
+  const void* q_weight;
+  const void* k_weight;
+  float eps;
+  int32_t norm_kind;
+  const float* rotary_angles;
+  int64_t angles_stride;
+  int32_t rot_dim, rotary_interleaved;
+  float mscale;
+  const int64_t* positions;
+  int32_t faithful_rounding;
+};
 // Shared by the decode entry point and by the mixed-batch path of the prefill entry point
 // (cu_seqlens_q non-null: only requests with one query row take part, at row cu_seqlens_q[r]).
 int launch_paged_decode(const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
@@ -31,5 +49,5 @@ int launch_paged_decode(const void* q, int64_t q_stride_tok, int64_t q_stride_he
                         int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq,
                         int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t split_tokens,
                         float softmax_scale, int32_t kv_dtype, const float* k_scales, const float* v_scales,
-                        int32_t dtype, const MiTuning& tune, void* stream);
+                        int32_t dtype, const MiTuning& tune, void* stream, const FusedStepArgs* fused = nullptr);
 }

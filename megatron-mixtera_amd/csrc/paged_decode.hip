@@ -35,6 +35,8 @@
 // A second kernel merges the partials of each request,
 //   o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max),
 // and writes zeros for zero-length (padded) rows.
+#include <stdio.h>
+
 #include "mi_common.h"
 
 #include <atomic>
@@ -64,6 +66,20 @@ struct DecodeParams {
   uint64_t chunk_magic;  // ceil(2^40 / chunk)
   int32_t R, Hq, Hkv, G, chunk, min_span_tiles, grid;
   int32_t parts;  // wavefronts per KV head: each takes up to 16 of the G query heads that share it
+  // Fused decode step only (FUSED kernels): `q` holds the raw queries of the step, head h * G + u of a row at
+  // h * q_gst + u * d; the step's new key / value rows, norm weights, rotary table and positions.
+  int64_t q_gst;
+  const uint16_t* nk;  // [R][Hkv][d]: head h of row r at r * nk_st + h * nk_hst
+  int64_t nk_st, nk_hst;
+  const uint16_t* nv;
+  int64_t nv_st, nv_hst;
+  const uint16_t* q_w;  // [d] or null
+  const uint16_t* k_w;
+  const float* emb;  // [max_pos][rot] angles or null
+  int64_t emb_stride;
+  const int64_t* pos;  // [R] rotary position of the step's token
+  int32_t rot, norm, interleaved, faithful;
+  float eps, mscale;
   float scale_log2;
 };
 
@@ -78,10 +94,17 @@ static __device__ __forceinline__ int chunk_of(int tok, uint64_t magic) {
 // HDK = width of the keys (and queries), HDV = width of the values (and of the output).  They differ
 // only for the latent cache of multi-latent attention (576 / 512: the value is the first 512 of the
 // shared 576-wide row, the caller points both cache arguments at the same buffer).
-template <int HDK, int HDV, int NT, bool FP8, bool F16>
+//
+// FUSED: the segment starts from the RAW queries of the step and does what the separate norm / rotary / append
+// launch does (same arithmetic and rounding points as norm_rope_append_kernel): every segment normalises and
+// rotates its query rows in registers; the segment that ends the request (`final_seg`: the only one that reads
+// the step's new token) first normalises and rotates the new key row of its KV head, writes it and the value
+// row into their cache slot, and orders that write before its own reads.  `q_lds` is then this wavefront's
+// piece of LDS for cos / sin of the request's position [2][HDK] and the key row [HDK] (fp32).
+template <int HDK, int HDV, int NT, bool FP8, bool F16, bool FUSED = false>
 static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int r, int row, int h, int hq0, int gq,
-                                                      int len, int start, int end, bool whole, int slot, int lane,
-                                                      uint8_t* q_lds) {
+                                                      int len, int start, int end, bool whole, bool final_seg,
+                                                      int slot, int lane, uint8_t* q_lds) {
   constexpr int KS = HDK / 32;
   // Wide keys (the 576-wide latent rows): the query fragments would take 72 registers per lane next
   // to 128 accumulator registers, so they live in this wavefront's piece of LDS instead (16 rows with
@@ -95,6 +118,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   constexpr int VD = FP8 ? 2 : DV / 2;  // dwords per token and lane of the value operand
   static_assert(HDK % 32 == 0 && HDV % 32 == 0 && HDK >= 64 && HDV >= 64, "head widths: multiples of 32");
   static_assert(!FP8 || (HDK == 128 && HDV == 128 && !F16), "fp8 KV: head_dim 128, bf16 queries");
+  static_assert(!FUSED || (!FP8 && HDK == HDV && (HDK == 64 || HDK == 128)), "fused step: head_dim 64 or 128, 16-bit cache");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
   // tile base addresses below run on the scalar unit instead of costing vector instructions.
@@ -116,7 +140,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   uint4 qf[Q_IN_LDS ? 1 : KS];
   const uint8_t* q_frag = q_lds + m16 * kQPitch + 16 * g;  // this lane's fragment of step kk: + 64 kk
   {
-    const uint16_t* qrow = p.q + (int64_t)row * p.q_st + (int64_t)hq * p.q_sh;
+    const uint16_t* qrow = FUSED ? p.q + (int64_t)row * p.q_st + (int64_t)h * p.q_gst + (int64_t)(hq - h * p.G) * HDK
+                                 : p.q + (int64_t)row * p.q_st + (int64_t)hq * p.q_sh;
     if (Q_IN_LDS) {
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk)
@@ -139,6 +164,212 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * ESZ;
   const int64_t chunk_bytes = p.kv_sc * ESZ;
   const uint32_t tok_bytes = (uint32_t)(p.kv_st * ESZ);
+
+  float* const cs = reinterpret_cast<float*>(q_lds);  // fused: [2][HDK]: cos | sin at the request's position
+  float* const kx = cs + 2 * HDK;                     // fused: [HDK]: the normalised key row (rotary partners)
+  const bool faithful = FUSED && p.faithful != 0;
+  // LDS traffic between the lanes of one wavefront: order it for the compiler, the hardware runs it in order
+  auto wave_sync = [] {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  // Requested here, ahead of the block-table round trip below, so that the two overlap: the rotary angles of
+  // elements lane, lane + 64 at the request's position and the norm weights of this lane's query elements.
+  constexpr int NA = (HDK + 63) / 64;
+  float ang[NA];
+  uint4 qwr[KS];
+  if constexpr (FUSED) {
+    if (p.emb) {
+      // (no position array: the step's token sits at the request's last position, which is already at hand)
+      const int64_t pos = p.pos ? p.pos[row] : (int64_t)(len - 1);
+#pragma unroll
+      for (int i = 0; i < NA; ++i) ang[i] = lane + 64 * i < p.rot ? p.emb[pos * p.emb_stride + lane + 64 * i] : 0.f;
+    }
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      qwr[kk] = (p.norm == MI_NORM_RMS && p.q_w) ? ld16(p.q_w + 32 * kk + 8 * g)
+                                                 : make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
+  }
+  auto fused_cos_sin = [&] {
+    if (p.emb) {
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int e = lane + 64 * i;
+        if (e >= HDK) break;
+        float c = 1.f, sn = 0.f;  // elements past the rotary width pass through
+        if (e < p.rot) {
+          const float a = ang[i];
+          c = cosf(a) * p.mscale;
+          sn = sinf(a) * p.mscale;
+          if (faithful) {
+            c = to_f32<F16>(f32_to_16<F16>(c));
+            sn = to_f32<F16>(f32_to_16<F16>(sn));
+          }
+        }
+        cs[e] = c;
+        cs[HDK + e] = sn;
+      }
+      wave_sync();
+    }
+  };
+  // ---- the step's new key / value rows of this KV head -> their cache slot (the request's last position) ----
+  // (With more than 16 query heads per KV head every wavefront of the head writes the same bytes: each one orders
+  // its own write before its own reads, and none has to wait for another.)
+  auto fused_append = [&] {
+    {
+      constexpr int LPV = HDK >= 128 ? 64 : 32, EPL = HDK / LPV;  // lane i owns elements i, i + LPV, ...
+      const bool on = lane < LPV;
+      const int i = on ? lane : 0;
+      const uint16_t* src = p.nk + (int64_t)row * p.nk_st + (int64_t)h * p.nk_hst;
+      float y[EPL];
+#pragma unroll
+      for (int w = 0; w < EPL; ++w) y[w] = on ? to_f32<F16>(src[i + w * LPV]) : 0.f;
+      if (p.norm != MI_NORM_NONE) {
+        float ss = y[0] * y[0] + y[1] * y[1];
+#pragma unroll
+        for (int w = 2; w < EPL; ++w) ss += y[w] * y[w];
+#pragma unroll
+        for (int o = LPV / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float rstd = rsqrtf(ss * (1.f / HDK) + p.eps);
+#pragma unroll
+        for (int w = 0; w < EPL; ++w) {
+          y[w] *= rstd;
+          if (p.norm == MI_NORM_RMS && p.k_w) y[w] *= to_f32<F16>(p.k_w[i + w * LPV]);
+          if (faithful) y[w] = to_f32<F16>(f32_to_16<F16>(y[w]));
+        }
+      }
+      float o[EPL];
+#pragma unroll
+      for (int w = 0; w < EPL; ++w) o[w] = y[w];
+      if (p.emb) {
+        if (on) {
+#pragma unroll
+          for (int w = 0; w < EPL; ++w) kx[i + w * LPV] = y[w];
+        }
+        wave_sync();
+        const int half = p.rot >> 1;
+#pragma unroll
+        for (int w = 0; w < EPL; ++w) {
+          const int e = i + w * LPV;
+          if (on && e < p.rot) {
+            const int partner = p.interleaved ? (e ^ 1) : (e < half ? e + half : e - half);
+            const float sign = p.interleaved ? ((e & 1) ? 1.f : -1.f) : (e < half ? -1.f : 1.f);
+            const float yp = kx[partner] * sign;
+            const float c = cs[e], sn = cs[HDK + e];
+            o[w] = faithful ? to_f32<F16>(f32_to_16<F16>(y[w] * c)) + to_f32<F16>(f32_to_16<F16>(yp * sn))
+                            : y[w] * c + yp * sn;
+          }
+        }
+      }
+      const int cpos = len - 1, ci = chunk_of(cpos, p.chunk_magic);
+      const int64_t slot_bytes = (int64_t)p.bt[(int64_t)r * p.bt_stride + ci] * chunk_bytes +
+                                 (int64_t)(cpos - ci * p.chunk) * tok_bytes;
+      uint16_t* kdst = reinterpret_cast<uint16_t*>(const_cast<uint8_t*>(kbase) + slot_bytes);
+      if (on) {
+#pragma unroll
+        for (int w = 0; w < EPL; ++w) kdst[i + w * LPV] = f32_to_16<F16>(o[w]);
+      }
+      const uint32_t* vsrc = reinterpret_cast<const uint32_t*>(p.nv + (int64_t)row * p.nv_st + (int64_t)h * p.nv_hst);
+      uint32_t* vdst = reinterpret_cast<uint32_t*>(const_cast<uint8_t*>(vbase) + slot_bytes);
+      for (int e = lane; e < HDV / 2; e += 64) vdst[e] = vsrc[e];
+      // The rows just written are read back below by other lanes of this same wavefront and by nobody else in
+      // this launch (it owns the request's last tiles): wait until the stores have reached the L2 (their
+      // acknowledgement), then keep the compiler from moving the loads up.  No cache has to be written back or
+      // invalidated for that -- the lines cannot sit in this CU's L1 (nothing read them before), and a wider
+      // scope would flush the L2 of the whole XCD under the other wavefronts' streams.
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+  };
+  // ---- this wavefront's query rows: lane (m16, g) holds elements 32 kk + 8 g .. + 7 of head m16 ----
+  auto fused_queries = [&] {
+    float x[KS][8];
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+      const uint32_t w4[4] = {qf[kk].x, qf[kk].y, qf[kk].z, qf[kk].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        x[kk][2 * j] = lo_to_f32<F16>(w4[j]);
+        x[kk][2 * j + 1] = hi_to_f32<F16>(w4[j]);
+      }
+    }
+    if (p.norm != MI_NORM_NONE) {
+      float ss = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss += x[kk][j] * x[kk][j];
+      ss += xor16(ss);
+      ss += xor32(ss);
+      const float rstd = rsqrtf(ss * (1.f / HDK) + p.eps);
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) {
+        const uint32_t w4[4] = {qwr[kk].x, qwr[kk].y, qwr[kk].z, qwr[kk].w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          float v = x[kk][j] * rstd;
+          if (p.norm == MI_NORM_RMS && p.q_w) v *= (j & 1) ? hi_to_f32<F16>(w4[j >> 1]) : lo_to_f32<F16>(w4[j >> 1]);
+          x[kk][j] = faithful ? to_f32<F16>(f32_to_16<F16>(v)) : v;
+        }
+      }
+    }
+    if (p.emb) {
+      // one rotated element: y cos + (partner, signed) sin, with the op chain's roundings when asked for
+      auto rotated = [&](float y, float yp, float c, float sn) {
+        return faithful ? to_f32<F16>(f32_to_16<F16>(y * c)) + to_f32<F16>(f32_to_16<F16>(yp * sn)) : y * c + yp * sn;
+      };
+      // cos | sin of elements 32 kk + 8 g + j .. + 3 (j = 0 or 4)
+      auto cos_sin = [&](int kk, int j, float (&c)[4], float (&sn)[4]) {
+        const float4 c4 = *reinterpret_cast<const float4*>(&cs[32 * kk + 8 * g + j]);
+        const float4 s4 = *reinterpret_cast<const float4*>(&cs[HDK + 32 * kk + 8 * g + j]);
+        c[0] = c4.x; c[1] = c4.y; c[2] = c4.z; c[3] = c4.w;
+        sn[0] = s4.x; sn[1] = s4.y; sn[2] = s4.z; sn[3] = s4.w;
+      };
+      // fragments ka < kb whose elements are each other's partners (half-split pairs), rotated in place
+      auto rotate_pair = [&](int ka, int kb) {
+#pragma unroll
+        for (int j0 = 0; j0 < 8; j0 += 4) {
+          float ca[4], sa[4], cb[4], sb[4];
+          cos_sin(ka, j0, ca, sa);
+          cos_sin(kb, j0, cb, sb);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float ya = x[ka][j0 + j], yb = x[kb][j0 + j];
+            x[ka][j0 + j] = rotated(ya, -yb, ca[j], sa[j]);
+            x[kb][j0 + j] = rotated(yb, ya, cb[j], sb[j]);
+          }
+        }
+      };
+      if (p.interleaved) {
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+#pragma unroll
+          for (int j0 = 0; j0 < 8; j0 += 4) {
+            float c[4], sn[4];
+            cos_sin(kk, j0, c, sn);
+#pragma unroll
+            for (int j = 0; j < 4; j += 2) {
+              if (32 * kk + 8 * g + j0 + j < p.rot) {  // (rot_dim is even: a pair lies within it or beyond)
+                const float ya = x[kk][j0 + j], yb = x[kk][j0 + j + 1];
+                x[kk][j0 + j] = rotated(ya, -yb, c[j], sn[j]);
+                x[kk][j0 + j + 1] = rotated(yb, ya, c[j + 1], sn[j + 1]);
+              }
+            }
+          }
+        }
+      } else if (KS == 4 && p.rot == 128) {  // partners 64 elements = two fragments apart
+        rotate_pair(0, 2 % KS);
+        rotate_pair(1, 3 % KS);
+      } else {  // rot_dim 64: fragments 0 and 1 pair up; fragments 2, 3 (head_dim 128) pass through
+        rotate_pair(0, 1);
+      }
+    }
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk)
+      qf[kk] = make_uint4(pack2<F16>(x[kk][0], x[kk][1]), pack2<F16>(x[kk][2], x[kk][3]),
+                          pack2<F16>(x[kk][4], x[kk][5]), pack2<F16>(x[kk][6], x[kk][7]));
+  };
 
   float m_run = -INFINITY, l_run = 0.f;
   f32x4_t acc[DV];
@@ -258,8 +489,26 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     }
   };
 
-  load_k(start);
-  load_v(start);
+  if constexpr (FUSED) {
+    // The segment that ends the request appends before it loads (its tiles hold the new token); every other
+    // segment gets its first loads under way and prepares its queries while they are in flight.
+    // (The value loads wait until the queries are done: with both tiles in flight the prologue would not fit the
+    // registers of three wavefronts per SIMD.)
+    if (final_seg) {
+      fused_cos_sin();
+      fused_append();
+      load_k(start);
+    } else {
+      load_k(start);
+      fused_cos_sin();
+    }
+    fused_queries();
+    __builtin_amdgcn_sched_barrier(0);
+    load_v(start);
+  } else {
+    load_k(start);
+    load_v(start);
+  }
   __builtin_amdgcn_sched_barrier(0);
   if (FP8) {  // the first tile lies in the opening chunk
     kcur.sc = ksc_tile = uniform_f(ksc_first);
@@ -421,7 +670,7 @@ static __device__ __forceinline__ bool decode_row(const DecodeParams& p, int r, 
 }
 
 // Span of this workgroup along the flattened sequence of TK-token tiles, then its segments one after
-// the other: seg(r, row, len, first token, one past the last token, whole request?, partial slot).
+// the other: seg(r, row, len, first token, one past the last token, whole request?, ends the request?, partial slot).
 // Every wavefront of the workgroup walks the same segments.  Dynamic LDS starts with the inclusive
 // prefix sums of tiles per request [R] and the request lengths [R].
 template <int TK, typename Seg>
@@ -487,7 +736,7 @@ static __device__ __forceinline__ void walk_segments(const DecodeParams& p, Seg 
       }
       int row;
       decode_row(p, r, row);
-      seg(r, row, len, tb * TK, min(te * TK, len), first && final, (int)blockIdx.x + r);
+      seg(r, row, len, tb * TK, min(te * TK, len), first && final, final, (int)blockIdx.x + r);
       t0 = rb + te;
     }
     ++r;
@@ -495,7 +744,7 @@ static __device__ __forceinline__ void walk_segments(const DecodeParams& p, Seg 
 }
 
 // The body of the register-streaming kernels: one wavefront per (virtual) KV head.
-template <int HDK, int HDV, int NT, bool FP8, bool F16>
+template <int HDK, int HDV, int NT, bool FP8, bool F16, bool FUSED = false>
 static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p) {
   extern __shared__ int cum[];
   const int lane = threadIdx.x & 63;
@@ -506,17 +755,26 @@ static __device__ __forceinline__ void decode_stream_body(const DecodeParams& p)
   const int part = hv - h * p.parts;
   const int hq0 = h * p.G + 16 * part;
   const int gq = min(16, p.G - 16 * part);
-  // wide keys: 16 query rows per wavefront behind the two integer arrays (see decode_segment)
+  // behind the two integer arrays, per wavefront: 16 query rows (wide keys) or the fused step's cos / sin / key
+  // row (see decode_segment)
   uint8_t* const q_lds = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15) +
-                         (size_t)wave * 16 * (HDK * 2 + 16);
-  walk_segments<16 * NT>(p, [&](int r, int row, int len, int start, int end, bool whole, int slot) {
-    decode_segment<HDK, HDV, NT, FP8, F16>(p, r, row, h, hq0, gq, len, start, end, whole, slot, lane, q_lds);
+                         (size_t)wave * (FUSED ? 3 * HDK * sizeof(float) : 16 * (HDK * 2 + 16));
+  walk_segments<16 * NT>(p, [&](int r, int row, int len, int start, int end, bool whole, bool final_seg, int slot) {
+    decode_segment<HDK, HDV, NT, FP8, F16, FUSED>(p, r, row, h, hq0, gq, len, start, end, whole, final_seg, slot, lane,
+                                                  q_lds);
   });
 }
 
 template <int HD, int NT, bool FP8, int MINW, bool F16>
 __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodeParams p) {
   decode_stream_body<HD, HD, NT, FP8, F16>(p);
+}
+
+// The same stream over the raw queries, keys and values of a decode step: head norm, rotary embedding and the
+// append of the new token ride in the segment prologues (see decode_segment).
+template <int HD, int NT, bool F16>
+__global__ __launch_bounds__(512, 3) void decode_step_stream_kernel(DecodeParams p) {
+  decode_stream_body<HD, HD, NT, false, F16, true>(p);
 }
 
 // Multi-latent attention, absorbed form: every query head attends to the same 576-wide latent rows
@@ -577,7 +835,7 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
   const int vfrag_off = (4 * g + (m16 >> 2)) * kMlaPitch + 2 * c0 + 8 * (m16 & 3);
   const uint4 ones = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
 
-  walk_segments<kMlaTile>(p, [&](int r, int row, int len, int start, int end, bool whole, int slot) {
+  walk_segments<kMlaTile>(p, [&](int r, int row, int len, int start, int end, bool whole, bool /*final_seg*/, int slot) {
     r = __builtin_amdgcn_readfirstlane(r);
     row = __builtin_amdgcn_readfirstlane(row);
     len = __builtin_amdgcn_readfirstlane(len);
@@ -848,7 +1106,7 @@ int mi::launch_paged_decode(
     void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
     int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
     int32_t split_tokens, float softmax_scale, int32_t kv_dtype, const float* k_scales,
-    const float* v_scales, int32_t dtype, const MiTuning& tune, void* stream) {
+    const float* v_scales, int32_t dtype, const MiTuning& tune, void* stream, const FusedStepArgs* fused) {
   if (R == 0) return MI_OK;
   if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
@@ -891,12 +1149,19 @@ int mi::launch_paged_decode(
       const int n = R - r0 < kMaxRequestsPerLaunch ? R - r0 : kMaxRequestsPerLaunch;
       // with cu_seqlens_q the rows of q / out are addressed through it, else request r owns row r
       const int64_t row0 = cu_seqlens_q ? 0 : r0;
+      FusedStepArgs fs;
+      if (fused) {
+        fs = *fused;
+        fs.k_new = (const uint16_t*)fs.k_new + r0 * fs.k_stride_tok;
+        fs.v_new = (const uint16_t*)fs.v_new + r0 * fs.v_stride_tok;
+        if (fs.positions) fs.positions += r0;
+      }
       const int rc = launch_paged_decode(
           (const uint16_t*)q + row0 * q_stride_tok, q_stride_tok, q_stride_head, k_cache, v_cache, kv_stride_chunk,
           kv_stride_tok, kv_stride_head, block_table + (int64_t)r0 * bt_stride, bt_stride, kv_lens + r0,
           cu_seqlens_q ? cu_seqlens_q + r0 : nullptr, (uint16_t*)out + row0 * o_stride_tok, o_stride_tok, o_stride_head,
           workspace, workspace_bytes, n, Hq, Hkv, head_dim, chunk_tokens, split_tokens, softmax_scale, kv_dtype, k_scales,
-          v_scales, dtype, tune, stream);
+          v_scales, dtype, tune, stream, fused ? &fs : nullptr);
       if (rc != MI_OK) return rc;
     }
     return MI_OK;
@@ -915,6 +1180,7 @@ int mi::launch_paged_decode(
   if (nt != 1 && nt != 2 && nt != 4) nt = kv_dtype == MI_KV_FP8_E4M3 ? 4 : 2;
   if (head_dim == 256) nt = 1;                 // (registers: 64 accumulators + 32 each for queries, keys, values)
   else if (head_dim == 192 && nt > 2) nt = 2;
+  if (fused) nt = 1;  // (the prologue's registers on top of two sub-tiles in flight would spill)
   while (chunk_tokens % (16 * nt)) nt >>= 1;  // a tile must not straddle two chunks
   const int minw = head_dim > 128 ? 2 : tune.decode_min_waves;
   const int tk = 16 * nt;
@@ -938,11 +1204,22 @@ int mi::launch_paged_decode(
   p.min_span_tiles = (min_span_tokens + tk - 1) / tk;
   p.grid = grid_x;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
+  if (fused) {
+    p.q_gst = fused->q_stride_group;
+    p.nk = (const uint16_t*)fused->k_new; p.nk_st = fused->k_stride_tok; p.nk_hst = fused->k_stride_head;
+    p.nv = (const uint16_t*)fused->v_new; p.nv_st = fused->v_stride_tok; p.nv_hst = fused->v_stride_head;
+    p.q_w = (const uint16_t*)fused->q_weight; p.k_w = (const uint16_t*)fused->k_weight;
+    p.emb = fused->rotary_angles; p.emb_stride = fused->angles_stride; p.pos = fused->positions;
+    p.rot = fused->rot_dim; p.norm = fused->norm_kind; p.interleaved = fused->rotary_interleaved;
+    p.faithful = fused->faithful_rounding; p.eps = fused->eps; p.mscale = fused->mscale;
+  }
 
   const int waves = head_waves(Hq, Hkv);
   const int wpb = pick_waves_per_block(waves, tune);
   dim3 grid(grid_x, waves / wpb), block(64 * wpb);
-  const size_t lds = (size_t)R * 2 * sizeof(int32_t);
+  // (fused step: per wavefront cos | sin | key row in fp32 behind the per-request arrays)
+  const size_t lds = fused ? (((size_t)R * 2 * sizeof(int32_t) + 15) & ~(size_t)15) + (size_t)wpb * 3 * head_dim * sizeof(float)
+                           : (size_t)R * 2 * sizeof(int32_t);
   hipStream_t st = (hipStream_t)stream;
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
@@ -962,7 +1239,12 @@ int mi::launch_paged_decode(
     if (nt == 2 && HD_ < 256) hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, (HD_ < 256 ? 2 : 1), false, 2, F16_>), grid, block, lds, st, p); \
     else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, false, 2, F16_>), grid, block, lds, st, p);               \
   } while (0)
-  if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true, false);
+#define MI_LAUNCH_STEP(HD_, F16_) hipLaunchKernelGGL((decode_step_stream_kernel<HD_, 1, F16_>), grid, block, lds, st, p)
+  if (fused && head_dim == 128 && f16) MI_LAUNCH_STEP(128, true);
+  else if (fused && head_dim == 128) MI_LAUNCH_STEP(128, false);
+  else if (fused && f16) MI_LAUNCH_STEP(64, true);
+  else if (fused) MI_LAUNCH_STEP(64, false);
+  else if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true, false);
   else if (head_dim == 128 && f16) MI_LAUNCH_DECODE(128, false, true);
   else if (head_dim == 128) MI_LAUNCH_DECODE(128, false, false);
   else if (head_dim == 64 && f16) MI_LAUNCH_DECODE(64, false, true);
@@ -975,6 +1257,7 @@ int mi::launch_paged_decode(
   else MI_LAUNCH_DECODE_WIDE(256, false);
 #undef MI_LAUNCH_DECODE
 #undef MI_LAUNCH_DECODE_WIDE
+#undef MI_LAUNCH_STEP
   if (timed) (void)hipEventRecord(ev_b, st);
   dim3 mgrid(Hq, R);
   const dim3 mblock(head_dim * merge_groups(p.grid, R, head_dim));
@@ -1008,6 +1291,61 @@ extern "C" int mi_paged_decode_attention(
                              kv_stride_head, block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok,
                              o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
                              split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, dtype, tune, stream);
+}
+
+extern "C" int mi_decode_step_attention(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new, int64_t k_stride_tok,
+    int64_t k_stride_head, const void* v_new, int64_t v_stride_tok, int64_t v_stride_head, const void* q_weight,
+    const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles, int64_t angles_stride,
+    int32_t rot_dim, int32_t rotary_interleaved, float mscale, const int64_t* positions, void* k_cache, void* v_cache,
+    int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head, const int32_t* block_table,
+    int64_t bt_stride, const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
+    int64_t workspace_bytes, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
+    int32_t split_tokens, float softmax_scale, int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning,
+    void* stream) {
+  const char* who = "mi_decode_step_attention";
+  char msg[160];
+  auto fail = [&](int code, const char* what) {
+    snprintf(msg, sizeof msg, "%s: %s", who, what);
+    return mi_fail(code, msg);
+  };
+  if (R == 0) return MI_OK;
+  MiTuning tune;
+  const int rc = mi_resolve_tuning(tuning, &tune, who);
+  if (rc != MI_OK) return rc;
+  if (!q || !k_new || !v_new || !k_cache || !v_cache) return fail(MI_ERR_NULL, "null pointer argument");
+  if (R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) return fail(MI_ERR_SHAPE, "need R >= 0 and Hq a multiple of Hkv");
+  if (head_dim != 64 && head_dim != 128)
+    return fail(MI_ERR_UNSUPPORTED, "head_dim must be 64 or 128 (other widths: the separate norm / rotary / append and attention calls)");
+  if (norm_kind != MI_NORM_NONE && norm_kind != MI_NORM_RMS && norm_kind != MI_NORM_L2)
+    return fail(MI_ERR_UNSUPPORTED, "unknown norm kind");
+  if (rotary_angles) {
+    if (rot_dim <= 0 || rot_dim > head_dim || (rot_dim & 1) || angles_stride < rot_dim)
+      return fail(MI_ERR_SHAPE, "rot_dim must be even and within head_dim");
+    // a lane holds 8 consecutive elements of every 32: half-split partners must sit a whole number of 32s away
+    if (!rotary_interleaved && (rot_dim / 2) % 32)
+      return fail(MI_ERR_UNSUPPORTED, "half-split rotary pairs need rot_dim / 2 to be a multiple of 32 (else: the separate calls)");
+  }
+  const int G = Hq / Hkv;
+  if (q_stride_group < (int64_t)G * head_dim) return fail(MI_ERR_SHAPE, "query group stride smaller than (Hq / Hkv) * head_dim");
+  if ((((uintptr_t)q | (uintptr_t)q_weight) & 15) || (q_stride_tok | q_stride_group) % 8)
+    return fail(MI_ERR_ALIGN, "q, the query norm weight and the q strides must keep rows 16-byte aligned");
+  if ((((uintptr_t)v_new | (uintptr_t)k_new) & 3) || ((v_stride_tok | v_stride_head) & 1))
+    return fail(MI_ERR_ALIGN, "new key / value rows must be 4-byte aligned");
+  FusedStepArgs fs;
+  fs.q_stride_group = q_stride_group;
+  fs.k_new = k_new; fs.k_stride_tok = k_stride_tok; fs.k_stride_head = k_stride_head;
+  fs.v_new = v_new; fs.v_stride_tok = v_stride_tok; fs.v_stride_head = v_stride_head;
+  fs.q_weight = q_weight; fs.k_weight = k_weight; fs.eps = eps; fs.norm_kind = norm_kind;
+  fs.rotary_angles = rotary_angles; fs.angles_stride = angles_stride; fs.rot_dim = rot_dim;
+  fs.rotary_interleaved = rotary_interleaved; fs.mscale = mscale; fs.positions = positions;
+  fs.faithful_rounding = faithful_rounding;
+  // (the remaining checks -- cache strides, chunk size, workspace -- are those of the attention entry point; the
+  // head stride of q is not used by the fused kernels)
+  return launch_paged_decode(q, q_stride_tok, head_dim, k_cache, v_cache, kv_stride_chunk, kv_stride_tok, kv_stride_head,
+                             block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok, o_stride_head, workspace,
+                             workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens, split_tokens, softmax_scale,
+                             MI_KV_16BIT, nullptr, nullptr, dtype, tune, stream, &fs);
 }
 
 // ---------------------------------------------------------------------------------------------

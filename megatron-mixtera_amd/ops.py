@@ -669,6 +669,97 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
 # ---------------------------------------------------------------------------------------------
 # context bookkeeping on the GPU
 # ---------------------------------------------------------------------------------------------
+def decode_step_supported(head_dim: int, rot_dim: int, rotary_interleaved: bool, fp8_cache: bool) -> bool:
+    """Whether :func:`decode_step_attention` has a kernel for these shapes (else: the separate calls)."""
+    if fp8_cache or head_dim not in (64, 128):
+        return False
+    return rot_dim == 0 or rotary_interleaved or (rot_dim // 2) % 32 == 0
+
+
+def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value: Optional[Tensor], k_cache: Tensor,
+                          v_cache: Tensor, kv_lens: Tensor, block_table: Tensor, *,
+                          mixed_qkv: Optional[Tensor] = None, num_query_heads: int = 0, num_kv_heads: int = 0,
+                          q_weight: Optional[Tensor] = None, k_weight: Optional[Tensor] = None, eps: float = 1e-5,
+                          norm: Optional[str] = None, rotary_emb: Optional[Tensor] = None,
+                          positions: Optional[Tensor] = None, rotary_interleaved: bool = False, mscale: float = 1.0,
+                          softmax_scale: Optional[float] = None, max_kv_len: Optional[int] = None,
+                          split_tokens: int = 0, out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
+                          faithful_rounding: bool = True) -> Tensor:
+    """One decode step of a layer in two launches: head norm + RoPE of the raw queries and of the step's new key
+    rows, the append of the new key / value rows at position ``kv_lens - 1`` and the attention over the cache --
+    what :func:`norm_rope_append` (or :func:`qkv_norm_rope_append`) followed by :func:`paged_decode_attention`
+    computes.  Inputs: ``query`` ``[R, (1,) Hq, d]``, ``key`` / ``value`` ``[R, (1,) Hkv, d]``, or ``mixed_qkv``
+    ``[R, (1,) (Hq + 2 Hkv) d]`` (the QKV projection's output) with the head counts.  Returns ``[R, (1,) Hq, d]``."""
+    lib = _lib.load()
+    if mixed_qkv is not None:
+        _require(query is None and key is None and value is None, "give either query / key / value or mixed_qkv")
+        _require(mixed_qkv.is_cuda and mixed_qkv.dtype in _DTYPE_CODES, "mixed_qkv must be a bf16 or fp16 device tensor")
+        four_d = mixed_qkv.dim() == 3
+        m2 = mixed_qkv[:, 0] if four_d else mixed_qkv
+        _require(not four_d or mixed_qkv.size(1) == 1, "mixed_qkv must be [R, 1, W]")
+        _require(m2.dim() == 2 and m2.stride(1) == 1, "mixed_qkv must be [R, W] with contiguous rows")
+        R, W = m2.shape
+        Hq, Hkv = int(num_query_heads), int(num_kv_heads)
+        _require(Hq > 0 and Hkv > 0 and Hq % Hkv == 0 and W % (Hq + 2 * Hkv) == 0, "mixed_qkv width / head counts")
+        D = W // (Hq + 2 * Hkv)
+        G = Hq // Hkv
+        group = (G + 2) * D
+        ref = m2
+        q_ptr, q_st, q_gst = m2.data_ptr(), m2.stride(0), group
+        k_ptr, k_st, k_hst = m2.data_ptr() + 2 * G * D, m2.stride(0), group
+        v_ptr, v_st, v_hst = m2.data_ptr() + 2 * (G + 1) * D, m2.stride(0), group
+        out_shape = (R, 1, Hq, D) if four_d else (R, Hq, D)
+    else:
+        q3, k3, v3 = _qo_view(query, "query"), _qo_view(key, "key"), _qo_view(value, "value")
+        R, Hq, D = q3.shape
+        Hkv = k3.size(1)
+        _require(tuple(k3.shape) == (R, Hkv, D) and tuple(v3.shape) == (R, Hkv, D) and Hq % max(Hkv, 1) == 0,
+                 "query / key / value shapes")
+        _require(q3.stride(1) == D, "query heads must be contiguous")
+        _require(k3.dtype == q3.dtype and v3.dtype == q3.dtype, "query / key / value must share one 16-bit type")
+        ref = q3
+        q_ptr, q_st, q_gst = q3.data_ptr(), q3.stride(0), (Hq // Hkv) * D
+        k_ptr, k_st, k_hst = k3.data_ptr(), k3.stride(0), k3.stride(1)
+        v_ptr, v_st, v_hst = v3.data_ptr(), v3.stride(0), v3.stride(1)
+        out_shape = tuple(query.shape)
+    stream = _stream(ref)
+    N, C, Hkv_c, Dk = k_cache.shape
+    _require(Dk == D and Hkv_c == Hkv and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
+    _require(k_cache.dtype == ref.dtype and v_cache.dtype == ref.dtype, "the caches must have the tensors' 16-bit type")
+    sc, st, sh = _cache_strides(k_cache)
+    _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
+    _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
+    _require(kv_lens.dtype == torch.int32 and kv_lens.is_contiguous(), "kv_lens must be contiguous int32")
+    _require(block_table.size(0) >= R and kv_lens.numel() >= R, "block_table / kv_lens shorter than the batch")
+    ang, a_stride, rot = _angles(rotary_emb)
+    _require(positions is None or (positions.dtype == torch.int64 and positions.is_contiguous()
+                                   and positions.numel() >= R), "positions must be int64 [>= R] (None: kv_lens - 1)")
+    for w in (q_weight, k_weight):
+        _require(w is None or (w.dtype == ref.dtype and w.numel() == D and w.is_contiguous()),
+                 "norm weights must be [d] of the tensors' 16-bit type")
+    if max_kv_len is None:
+        max_kv_len = block_table.size(1) * C
+    if softmax_scale is None:
+        softmax_scale = D ** -0.5
+    if out is None:
+        out = torch.empty(out_shape, dtype=ref.dtype, device=ref.device)
+    o3 = _qo_view(out, "out")
+    _require(tuple(o3.shape) == (R, Hq, D) and o3.dtype == ref.dtype, "out shape / dtype mismatch")
+    tune = _tuning_arg()
+    need = lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, C, max_kv_len, split_tokens, tune)
+    if workspace is None:
+        workspace = _workspace(ref.device, need)
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    _lib.check(lib.mi_decode_step_attention(
+        q_ptr, q_st, q_gst, k_ptr, k_st, k_hst, v_ptr, v_st, v_hst, _ptr(q_weight), _ptr(k_weight), float(eps),
+        _NORM_KINDS[norm], _ptr(ang), a_stride, rot, int(bool(rotary_interleaved)), float(mscale), _ptr(positions),
+        k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh, block_table.data_ptr(), block_table.stride(0),
+        kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1), _ptr(workspace), ws_bytes, R, Hq, Hkv, D, C,
+        int(split_tokens), float(softmax_scale), int(bool(faithful_rounding)), _dtype_code(ref, "query"), tune,
+        stream), "mi_decode_step_attention")
+    return out
+
+
 def update_requests(ctx, mask_i32: Tensor, new_tokens_i64: Tensor) -> None:
     """Enqueue the single-kernel ``update_requests`` on the state tensors of ``ctx`` (results land in
     ``ctx._counters`` / ``ctx._newly_paused_buf`` / ``ctx._finished_ids_buf`` / ``ctx._paused_tokens_buf``)."""

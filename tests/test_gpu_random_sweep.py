@@ -431,6 +431,80 @@ def case_norm_rope(mi, dev, rng, seed):
     assert (gk[untouched] == -1).all(), "rows outside the appended slots changed"
 
 
+def case_decode_step(mi, dev, rng, seed):
+    """The fused decode step: norm + RoPE + append inside the streaming kernel, against the checker's chain."""
+    gen = torch.Generator().manual_seed(seed)
+    d = rng.choice([64, 128])
+    Hkv = rng.choice([1, 2, 3, 4, 8])
+    G = rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 20] if Hkv <= 2 else [1, 2, 3, 4, 5, 7, 8])
+    Hq = Hkv * G
+    chunk = rng.choice([16, 32, 48, 64, 128, 256])
+    R = rng.randint(1, 20)
+    lens = rand_lens(rng, R, chunk, 1500)
+    norm = rng.choice([None, "rms", "l2"])
+    rotary = rng.choice(["none", "half", "half", "interleaved", "interleaved_part"] + (["half64"] if d == 128 else []))
+    rot = {"none": 0, "half": d, "half64": 64, "interleaved": d, "interleaved_part": rng.choice([24, 40, 62])}[rotary]
+    interleaved = rotary.startswith("interleaved")
+    grid = rng.choice([0, 0, 1, 3, 37, 500])
+    split = rng.choice([0, 0, 16, 64, 512])
+    waves = rng.choice([8, 8, 4, 2, 1])
+    mixed = rng.random() < 0.5
+    given_pos = rng.random() < 0.5
+    dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16])
+    _note(f"decode_step seed={seed} d={d} Hq={Hq} Hkv={Hkv} chunk={chunk} lens={lens} norm={norm} rotary={rotary} rot={rot} "
+          f"grid={grid} split={split} waves={waves} mixed={mixed} given_pos={given_pos} dtype={dtype}")
+    lens_t = torch.tensor(lens, dtype=torch.int32)
+    bt, N = mi.synthetic.build_block_table(lens_t, chunk, gen)
+    kc = (torch.randn(N + 1, chunk, Hkv, d, generator=gen) * 0.7).to(dtype)
+    vc = (torch.randn(N + 1, chunk, Hkv, d, generator=gen) * 0.7).to(dtype)
+    mixed_qkv = torch.randn(R, 1, Hkv * (G + 2) * d, generator=gen).to(dtype)
+    q, k, v = orn.split_mixed_qkv(mixed_qkv, Hq, Hkv)
+    qw = (1 + 0.02 * torch.randn(d, generator=gen)).to(dtype)
+    kw = (1 + 0.02 * torch.randn(d, generator=gen)).to(dtype)
+    pos = (lens_t.long() - 1).clamp(min=0)
+    table = orn.rotary_table(max(lens) + 2, rot, base=10000.0, interleaved=interleaved) if rot else None
+    q_ref = orn.norm_rope(q.squeeze(1), pos, table, norm=norm, weight=qw if norm == "rms" else None, eps=1e-5,
+                          interleaved=interleaved)
+    k_ref = orn.norm_rope(k.squeeze(1), pos, table, norm=norm, weight=kw if norm == "rms" else None, eps=1e-5,
+                          interleaved=interleaved)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    rows, ids, loc = oa.decode_slots(bt, lens_t, chunk)
+    oa.kv_append(kc_ref, vc_ref, k_ref[rows], v.squeeze(1)[rows], ids, loc)
+    ref = oa.paged_decode_attention(q_ref, kc_ref, vc_ref, lens_t, bt)
+    kcd, vcd = kc.to(dev), vc.to(dev)
+    common = dict(q_weight=qw.to(dev) if norm == "rms" else None, k_weight=kw.to(dev) if norm == "rms" else None, norm=norm,
+                  eps=1e-5, rotary_emb=None if table is None else table.to(dev), rotary_interleaved=interleaved,
+                  positions=pos.to(dev) if given_pos else None, split_tokens=split)
+    poison(dev)
+    with mi.ops.tuning(decode_grid=grid, decode_waves_per_block=waves):
+        if mixed:
+            out = mi.ops.decode_step_attention(None, None, None, kcd, vcd, lens_t.to(dev), bt.to(dev),
+                                               mixed_qkv=mixed_qkv.to(dev), num_query_heads=Hq, num_kv_heads=Hkv, **common)
+        else:
+            out = mi.ops.decode_step_attention(q.to(dev), k.to(dev), v.to(dev), kcd, vcd, lens_t.to(dev), bt.to(dev),
+                                               **common)
+        torch.cuda.synchronize()
+    close(out, ref, 2e-2, "decode step")
+    assert (out.cpu()[lens_t == 0] == 0).all(), "zero-length rows must be zeros"
+    gk, gv = kcd.cpu(), vcd.cpu()
+    assert torch.equal(gv.view(torch.int16), vc_ref.view(torch.int16)), "V cache differs"
+    errk = (gk.float() - kc_ref.float()).abs()
+    assert (errk <= 2e-2 + 2e-2 * kc_ref.float().abs()).all(), f"K cache err {errk.max().item()}"
+    untouched = torch.ones(N + 1, chunk, dtype=torch.bool)
+    untouched[ids, loc] = False
+    assert torch.equal(gk[untouched].view(torch.int16), kc[untouched].view(torch.int16)), "rows outside the appended slots changed"
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_random_decode_steps_match_the_checker(mi, dev, block):
+    for seed in range(90_000 + 50 * block, 90_000 + 50 * (block + 1)):
+        rng = random.Random(seed)
+        try:
+            case_decode_step(mi, dev, rng, seed)
+        except AssertionError as e:
+            raise AssertionError(f"{_last_case[0]}: {e}") from None
+
+
 WRITE_KINDS = {"append": case_append, "append_fp8": case_append_fp8, "norm_rope": case_norm_rope}
 
 
