@@ -31,20 +31,23 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 
 # HBM bytes per launch of the streaming kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
 # this same script, each counter scaled by what it reads for a plain 1 GiB device copy
-# (profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md).  Hardware counters cannot be
+# (profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md).  Hardware counters cannot be
 # read from inside the benchmark, so the figure is recorded here per workload; None = not collected.
-MEASURED_HBM_TRAFFIC_BYTES = {"cfg2": 1_226_800_000, "cfg4": 8_724_000_000, "cfg5": 9_070_100_000,
-                              # the mixed step (profiles/paged_prefill_pp_kernel_cfg3_mfma.md): tile kernel, stream kernel
-                              "cfg3_tile": 402_300_000, "cfg3_stream": 2_195_700_000}
+MEASURED_HBM_TRAFFIC_BYTES = {
+    # decode workloads: "<cfg>" = the attention-only streaming kernel, "<cfg>_step" = the one-kernel decode step
+    "cfg2": 1_226_700_000, "cfg2_step": 1_215_100_000, "cfg4": 8_724_600_000, "cfg4_step": 8_635_100_000,
+    "cfg5": 9_070_700_000,
+    # the mixed step: tile kernel, stream kernel
+    "cfg3_tile": 401_600_000, "cfg3_stream": 2_195_400_000}
 # Where each figure above was read, so that a reader of the JSON line can tell a stale constant from a fresh one:
 # the summary file and the last commit that touched the kernel when the counters were collected.
-TRAFFIC_SOURCE = {
-    "cfg2": "profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
-    "cfg4": "profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
-    "cfg5": "profiles/paged_decode_stream_kernel_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
-    "cfg3_tile": "profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
-    "cfg3_stream": "profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernel as of commit 45971b2)",
-}
+_DECODE_TRAFFIC = ("profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                   "kernels as of commit bc375af)")
+_MIXED_TRAFFIC = ("profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
+                  "commit bc375af)")
+TRAFFIC_SOURCE = {"cfg2": _DECODE_TRAFFIC, "cfg2_step": _DECODE_TRAFFIC, "cfg4": _DECODE_TRAFFIC,
+                  "cfg4_step": _DECODE_TRAFFIC, "cfg5": _DECODE_TRAFFIC, "cfg3_tile": _MIXED_TRAFFIC,
+                  "cfg3_stream": _MIXED_TRAFFIC}
 
 
 # Single-kernel workloads for the rows built around the path (multi-latent decode, the tail of a step).
@@ -683,7 +686,9 @@ def main():
         separate = {"ms_per_step": round(sep_ms, 5), "value": round(nbytes / (sep_ms * 1e-3) / 1e9, 1),
                     "kernel": "paged_decode_stream_kernel", "kernel_ms": round(sep_kernel_ms, 5),
                     "achieved": round(nbytes / (sep_kernel_ms * 1e-3) / 1e9, 1),
-                    "frac": round(nbytes / (sep_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                    "frac": round(nbytes / (sep_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
+                    "traffic_source": TRAFFIC_SOURCE.get(args.workload)}
     value = nbytes / (ms_per_step * 1e-3) / 1e9
     achieved = nbytes / (kernel_ms * 1e-3) / 1e9
 
@@ -720,8 +725,8 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
             "kernel_ms": round(kernel_ms, 5),
-            "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
-            "traffic_source": TRAFFIC_SOURCE.get(args.workload),
+            "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload + "_step" if one_kernel else args.workload),
+            "traffic_source": TRAFFIC_SOURCE.get(args.workload + "_step" if one_kernel else args.workload),
         },
     }
     if separate is not None:
