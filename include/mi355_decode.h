@@ -431,6 +431,27 @@ int mi_update_requests(int32_t* request_ids, int32_t* request_query_lengths,
                        int32_t chunk_size_tokens, int32_t max_requests, void* stream);
 
 /*
+ * The tensor writes of DynamicInferenceContext.add_request (dynamic_context.py:976-1015) as one kernel, after
+ * the caller has made the reference's host-side checks (token / request / chunk / sequence-length overflow,
+ * dynamic_context.py:945-974) and lowered the allocator's count by `chunk_count`: the request's row of every
+ * per-request tensor, the first `chunk_count` entries of its chunk-table row = chunk_bag[stack_first ..
+ * stack_first + chunk_count - 1] (the ids the allocator hands out, in stack order; stack_first = the
+ * allocator's count after the pop), and the rows token_begin .. token_begin + prompt_length - 1 of the per-token
+ * tensors (input id, position, request row, position in request, chunk, position in chunk).  prompt_tokens int64
+ * [prompt_length] on the device.
+ */
+int mi_add_request(int32_t* request_ids, int32_t* request_query_lengths, int32_t* request_output_lengths,
+                   int32_t* request_kv_length_offsets, int32_t* request_kv_chunk_counts,
+                   int32_t* request_last_kv_chunk_id, int32_t* request_last_kv_chunk_offset,
+                   int32_t* request_to_kv_chunk_ids, int64_t table_stride, int64_t* token_to_input_ids,
+                   int64_t* token_to_pos_ids, int64_t* token_to_request_idx,
+                   int64_t* token_to_position_in_request, int64_t* token_to_chunk_idx,
+                   int64_t* token_to_local_position_within_kv_chunk, const int32_t* chunk_bag,
+                   const int64_t* prompt_tokens, int32_t request_row, int32_t token_begin,
+                   int32_t prompt_length, int32_t chunk_count, int32_t stack_first, int32_t chunk_size_tokens,
+                   int32_t request_id, int32_t output_length, void* stream);
+
+/*
  * The decode-only part of DynamicInferenceContext.initialize_attention_state
  * (dynamic_context.py:733-741, 747-750, 785-787, 816-818) as one kernel: copies query lengths,
  * kv lengths (offset + query length) and block-table rows of the active requests into the

@@ -77,6 +77,7 @@ SIGNATURES = {
         c_int, [_P] * 8 + [_I64, _I32] + [_P] * 15 + [_I32] * 7 + [_P]),
     "mi_step_attention_state": (
         c_int, [_P, _P, _P, _I64, _I32, _P, _P, _P, _P, _P, _I64, _P, _P, _P, _P] + [_I32] * 6 + [_P]),
+    "mi_add_request": (c_int, [_P] * 8 + [_I64] + [_P] * 8 + [_I32] * 8 + [_P]),
     "mi_decode_attention_state": (
         c_int, [_P, _P, _P, _I64, _I32, _P, _P, _P, _I64, _P, _P, _P, _I32, _I32, _I32, _I32, _I32, _P]),
     "mi_last_token_gather": (c_int, [_P, _I64, _P, _I64, _P, _I32, _I32, _I32, _P]),

@@ -813,6 +813,16 @@ class DynamicInferenceContext:
             raise MaxSequenceLengthOverflowError(request_id)
 
         row = self.total_request_count
+        if self.fused_bookkeeping and length > 0:
+            # every write below as one launch (the popped ids are read from the allocator's stack on the GPU)
+            prompt = tokens.reshape(-1).to(device=self.device, dtype=torch.int64).contiguous()
+            ops.add_request(self, row, self.active_token_count, prompt, n_chunks,
+                            self.chunk_allocator.chunk_count_avail, request_id, length + num_tokens_to_generate)
+            self.total_request_count += 1
+            self.active_token_count += length
+            self._host_max_query_len = max(self._host_max_query_len, length)
+            self._host_kv_len_bound = max(self._host_kv_len_bound, length)
+            return
         self.request_ids[row] = request_id
         self.request_query_lengths[row] = length
         self.request_output_lengths[row] = length + num_tokens_to_generate

@@ -781,6 +781,26 @@ def update_requests(ctx, mask_i32: Tensor, new_tokens_i64: Tensor) -> None:
         ctx.chunk_size_tokens, ctx.max_requests, _stream(table)), "mi_update_requests")
 
 
+def add_request(ctx, row: int, token_begin: int, tokens_i64: Tensor, n_chunks: int, stack_first: int,
+                request_id: int, output_length: int) -> None:
+    """The tensor writes of ``add_request`` in one launch: request row ``row``, its chunk-table entries
+    ``chunk_bag[stack_first : stack_first + n_chunks]`` and the token rows from ``token_begin`` on."""
+    lib = _lib.load()
+    table = ctx.request_to_kv_chunk_ids
+    _require(tokens_i64.dtype == torch.int64 and tokens_i64.is_contiguous() and tokens_i64.device == table.device,
+             "prompt tokens must be a contiguous int64 tensor on the context's device")
+    _lib.check(lib.mi_add_request(
+        ctx.request_ids.data_ptr(), ctx.request_query_lengths.data_ptr(), ctx.request_output_lengths.data_ptr(),
+        ctx.request_kv_length_offsets.data_ptr(), ctx.request_kv_chunk_counts.data_ptr(),
+        ctx.request_last_kv_chunk_id.data_ptr(), ctx.request_last_kv_chunk_offset.data_ptr(), table.data_ptr(),
+        table.stride(0), ctx.token_to_input_ids.data_ptr(), ctx.token_to_pos_ids.data_ptr(),
+        ctx.token_to_request_idx.data_ptr(), ctx.token_to_position_in_request.data_ptr(),
+        ctx.token_to_chunk_idx.data_ptr(), ctx.token_to_local_position_within_kv_chunk.data_ptr(),
+        ctx.chunk_allocator.chunk_bag.data_ptr(), tokens_i64.data_ptr(), int(row), int(token_begin),
+        tokens_i64.numel(), int(n_chunks), int(stack_first), ctx.chunk_size_tokens, int(request_id),
+        int(output_length), _stream(table)), "mi_add_request")
+
+
 def decode_attention_state(ctx, n_active_requests: int, padded_tokens: int) -> None:
     """Fill the fixed-address length / block-table mirrors and the padded token rows in one launch."""
     lib = _lib.load()

@@ -173,6 +173,29 @@ def test_random_request_streams_match_restatement(mi, Ctx, dev, seed):
         assert "paused" in events and "resumed" in events
 
 
+def test_add_request_kernel_equals_the_indexed_writes(mi, Ctx, dev):
+    """Prompts of one token, around the chunk size and over several launch blocks: the one-launch admission leaves
+    every state tensor as the reference's sequence of indexed writes does (dynamic_context.py:976-1015)."""
+    a = small_ctx(Ctx, dev, fused_bookkeeping=True)
+    b = small_ctx(Ctx, dev, fused_bookkeeping=False)
+    gen = torch.Generator().manual_seed(4)
+    for rid, n in enumerate([1, 127, 128, 129, 300, 512, 5]):
+        toks = torch.randint(0, 50000, (n,), generator=gen)
+        budget = None if rid % 2 else 3
+        for c in (a, b):
+            try:
+                c.add_request(100 + rid, toks.to(dev), budget)
+                err = ""
+            except mi.ContextOverflowError as e:
+                err = type(e).__name__
+            c._last_err = err
+        assert a._last_err == b._last_err
+        assert _snapshot_product(a) == _snapshot_product(b), f"after request {rid} ({n} tokens)"
+    assert a.total_request_count >= 5
+    untouched = a.request_to_kv_chunk_ids[a.total_request_count:]
+    assert (untouched == -1).all()
+
+
 def test_kernel_and_torch_op_sequence_agree_on_a_wide_batch(mi, Ctx, dev):
     """More rows than one pass of the workgroup (max_requests > 256): both GPU paths, step by step."""
     set_rounder(Ctx, 4)
