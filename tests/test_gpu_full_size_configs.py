@@ -160,3 +160,51 @@ def test_cfg3_mixed_batch_full_size(mi, dev):
     ref = oa.paged_varlen_attention(q[a:a + 64].cpu(), kcc, vcc, torch.tensor([0, 64], dtype=torch.int32),
                                     (lens[r:r + 1] - 2048 + 64).cpu(), rows)
     _close(out[a:a + 64], ref, 2e-2, f"cfg3 prompt {r}, first 64 rows")
+
+
+@pytest.mark.parametrize("name,need", [("cfg2", 6), ("cfg4", 24)])
+def test_one_kernel_decode_step_full_size(mi, dev, name, need):
+    """The benchmark's default step at full size (configuration 2: batch 64, U[512, 8192]; configuration 4: batch 16
+    x 131 072): RMSNorm + RoPE + append + attention in the streaming kernel against the separate launches -- the
+    appended cache rows bit for bit, the outputs within 8e-3 -- and three sampled rows against the checker's chain."""
+    from oracle import rope_norm as orn
+    _need_free(need)
+    cfg = mi.synthetic.CONFIGS[name]
+    case = mi.synthetic.make_decode_case(cfg, dev, on_device_rng=True)
+    R, d = case.q.size(0), cfg.d
+    mx = int(case.kv_lens.max())
+    gen = torch.Generator().manual_seed(11)
+    qw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16()
+    kw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16()
+    table = mi.synthetic.rotary_angle_table(mx + 1, d, base=500000.0)
+    pos = (case.kv_lens.long() - 1).contiguous()
+    common = dict(q_weight=qw.to(dev), k_weight=kw.to(dev), eps=1e-5, norm="rms", rotary_emb=table.to(dev))
+    # where the step's token lands: the caches are too large to clone, so the appended rows are compared by slot
+    lens_h, bt_h = case.kv_lens.cpu().long(), case.block_table.cpu().long()
+    slot_chunk = bt_h[torch.arange(R), (lens_h - 1) // cfg.chunk].to(dev)
+    slot_pos = ((lens_h - 1) % cfg.chunk).to(dev)
+
+    out_a = mi.ops.decode_step_attention(case.q, case.k_new, case.v_new, case.k_cache, case.v_cache, case.kv_lens,
+                                         case.block_table, positions=None, max_kv_len=mx, **common)
+    torch.cuda.synchronize()
+    k_rows_a = case.k_cache[slot_chunk, slot_pos].clone()
+    v_rows_a = case.v_cache[slot_chunk, slot_pos].clone()
+    case.k_cache[slot_chunk, slot_pos] = 0   # make sure the second path writes them again
+    case.v_cache[slot_chunk, slot_pos] = 0
+    q_b = torch.empty_like(case.q)
+    with mi.ops.tuning(norm_rope_vectorised=-1):
+        mi.ops.norm_rope_append(case.q, case.k_new, value=case.v_new, query_out=q_b, q_positions=pos, k_positions=pos,
+                                k_cache=case.k_cache, v_cache=case.v_cache, block_table=case.block_table,
+                                kv_lens=case.kv_lens, **common)
+    out_b = mi.ops.paged_decode_attention(q_b, case.k_cache, case.v_cache, case.kv_lens, case.block_table, max_kv_len=mx)
+    torch.cuda.synchronize()
+    assert torch.equal(case.k_cache[slot_chunk, slot_pos], k_rows_a), "appended key rows differ from the separate launch"
+    assert torch.equal(case.v_cache[slot_chunk, slot_pos], v_rows_a)
+    assert torch.equal(v_rows_a, case.v_new.squeeze(1))
+    diff = (out_a.float() - out_b.float()).abs().max().item()
+    assert diff <= 8e-3, f"one-kernel step and separate launches differ by {diff:.3e}"
+    for r in (0, R // 2, R - 1):
+        rows, (kc, vc) = _compact(case.block_table[r:r + 1], case.k_cache.size(0), case.k_cache, case.v_cache)
+        q_ref = orn.norm_rope(case.q[r:r + 1].cpu().squeeze(1), pos[r:r + 1].cpu(), table, norm="rms", weight=qw, eps=1e-5)
+        ref = oa.paged_decode_attention(q_ref, kc, vc, case.kv_lens[r:r + 1].cpu(), rows)
+        _close(out_a[r:r + 1], ref, 2e-2, f"{name} row {r}")
