@@ -157,7 +157,10 @@ int mi_kv_append_fp8(const void* key_bf16, const void* value_bf16, int64_t src_s
 
 /*
  * Bytes of workspace mi_paged_decode_attention needs for these sizes on the current
- * device (partials of the workgroups that share a request + per-request bookkeeping).
+ * device (partials of the workgroups that share a request + per-request bookkeeping).  The size
+ * depends on R, the head counts, head_dim, the device's CU count and the grid knobs of `tuning`;
+ * chunk_tokens, max_kv_len and split_tokens are accepted for symmetry with the attention call and
+ * do not change it.  -1 = a knob out of range.
  */
 int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                   int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
