@@ -38,7 +38,7 @@ def test_mla_prefill_matches_checker(mi, dev, H, chunk):
 
 
 @pytest.mark.parametrize("pingpong", [-1, 1, 2])  # register-only kernel, two-phase, two-phase in lock-step
-@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (8, 2), (16, 1)])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (8, 2), (16, 1), (20, 1), (64, 2)])
 def test_mla_prefill_kernel_choice_and_grouped_heads(mi, dev, pingpong, Hq, Hkv):
     """The two-phase tile kernel (both wave schedules) and the register kernel, with several query heads
     per key head, over lengths either side of the 64-key tiles and the chunk size."""
