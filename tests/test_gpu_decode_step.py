@@ -169,3 +169,21 @@ def test_fused_step_rejects_what_it_has_no_kernel_for(mi, dev):
     c96 = torch.zeros(4, 64, 2, 96, dtype=torch.bfloat16, device=dev)
     with pytest.raises(mi._lib.KernelError, match="head_dim"):
         mi.ops.decode_step_attention(q96, k96, k96, c96, c96, case.kv_lens, case.block_table)
+
+
+def test_fused_step_more_requests_than_one_launch_takes(mi, dev):
+    """Beyond 7 680 requests the step runs in slices: queries, new rows, positions, lengths and table rows of a
+    slice all start at the slice's first request."""
+    R = 7680 + 900
+    gen = torch.Generator().manual_seed(6)
+    lens = torch.randint(0, 50, (R,), generator=gen).tolist()
+    table = orn.rotary_table(64, 64, base=10000.0)
+    case, lens, qw, kw, pos = _step_case(mi, dev, Hq=4, Hkv=2, d=64, chunk=16, lens=lens, dtype=torch.bfloat16, seed=8)
+    pos = (lens.long() - 1).clamp(min=0)
+    (out_a, kc_a, vc_a), (out_b, kc_b, vc_b) = _run_both(mi, dev, case, lens, qw, kw, pos, norm="rms", table=table,
+                                                         interleaved=False, mixed=False, max_kv_len=50)
+    dummy = case.k_cache.size(0) - 1
+    assert torch.equal(kc_a[:dummy], kc_b[:dummy]) and torch.equal(vc_a[:dummy], vc_b[:dummy])
+    assert (out_a.float() - out_b.float()).abs().max().item() <= 8e-3
+    ref, _, _ = _oracle(case, lens, qw, kw, pos, norm="rms", table=table, interleaved=False)
+    _close(out_a, ref, 2e-2, "sliced fused step vs checker")
