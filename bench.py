@@ -60,6 +60,11 @@ SECONDARY_WORKLOADS = {
     "mla_prefill_h16": ("mla_prefill", dict(H=16, n=8, new=2048, ctx=2048)),
     "mla_prefill_h128": ("mla_prefill", dict(H=128, n=2, new=2048, ctx=2048)),
     "prefill_d64": ("prefill", dict(Hq=32, Hkv=8, d=64, n=8, new=2048, ctx=2048)),
+    "prefill_d96": ("prefill", dict(Hq=32, Hkv=8, d=96, n=8, new=2048, ctx=2048)),
+    "prefill_d128": ("prefill", dict(Hq=32, Hkv=8, d=128, n=8, new=2048, ctx=2048)),
+    "prefill_d192": ("prefill", dict(Hq=32, Hkv=8, d=192, n=8, new=2048, ctx=2048)),
+    "prefill_d256": ("prefill", dict(Hq=32, Hkv=8, d=256, n=8, new=2048, ctx=2048)),
+    "prefill_d128_mqa": ("prefill", dict(Hq=64, Hkv=2, d=128, n=8, new=2048, ctx=2048)),
     "sampling_top_k": ("sampling", dict(R=64, V=128256, top_k=50, top_p=0.0)),
     "sampling_top_p": ("sampling", dict(R=64, V=128256, top_k=0, top_p=0.9)),
     "sampling_greedy": ("sampling", dict(R=64, V=128256, top_k=1, top_p=0.0)),
@@ -109,7 +114,7 @@ def run_secondary(args, mi, lib, torch, dev):
         pairs = n * (new * ctx + new * (new + 1) // 2)          # (query row, visible key) pairs per head
         flops = 2 * Hq * (dk + dv) * pairs
         nbytes = n * (new + ctx) * Hkv * (dk + dv) * 2 + n * new * Hq * (dk + dv) * 2
-        kernel = "paged_prefill_pp_kernel"
+        kernel = "paged_prefill_pp_kernel" if dk <= 128 or mla else "paged_prefill_kernel"
         what = (f"paged varlen causal attention, {n} x {new} new tokens over {ctx} cached, {Hq}/{Hkv} heads, "
                 f"keys {dk} / values {dv} wide, chunk 256")
         dtype = "bf16 (fp32 accumulate)"
@@ -294,7 +299,7 @@ def parse_args():
     ap.add_argument("--workload", default="cfg2",
                     choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", "cu_probes", *SECONDARY_WORKLOADS],
                     help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch; the "
-                         "mla_* / prefill_d64 / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
+                         "mla_* / prefill_d* / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
     ap.add_argument("--split-tokens", type=int, default=0)
     ap.add_argument("--subtiles", type=int, default=0, help="16-token sub-tiles per loop iteration (1, 2 or 4)")
     ap.add_argument("--no-cpu-baseline", action="store_true")

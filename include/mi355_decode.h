@@ -82,8 +82,8 @@ typedef struct MiTuning {
 
 /*
  * Kernel timing.  mi_profile_enable(1) makes the attention entry points bracket their main
- * kernel (decode: the KV-streaming kernel; prefill, head_dim 64, 96 or 128 with a chunk size that is a multiple of 64: the tile kernel, followed by
- * a second pair for the decode kernel of a mixed batch) with HIP events on the caller's
+ * kernel (decode: the KV-streaming kernel; prefill: the tile kernel, followed by a second pair
+ * for the decode kernel of a mixed batch when a workspace is passed) with HIP events on the caller's
  * stream; mi_profile_collect waits for
  * the recorded pairs, writes their durations (milliseconds, HOST pointer) and returns how
  * many there were.  Keep it off while capturing a graph.

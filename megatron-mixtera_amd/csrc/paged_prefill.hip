@@ -1094,6 +1094,9 @@ static int launch_paged_prefill(
     const int sbq = waves * ((16 * nq) / Gw);  // query tokens per workgroup: whole tokens in each wavefront's rows
     dim3 grid((T + sbq - 1) / sbq + R, Hkv * parts), block(64 * waves);
     const int nt = (tune.prefill_tile_subtiles == 1 || head_dim >= 192) ? 1 : 2;
+    hipEvent_t ev_a, ev_b;
+    const bool timed = mi_profile_next(&ev_a, &ev_b);
+    if (timed) (void)hipEventRecord(ev_a, st);
 #define MI_LAUNCH_PREFILL(HD_, F16_)                                                                           \
   do {                                                                                                         \
     if (nq == 4 && nt == 1) hipLaunchKernelGGL((paged_prefill_kernel<HD_, HD_, 1, 4, F16_>), grid, block, 0, st, p);  \
@@ -1112,6 +1115,7 @@ static int launch_paged_prefill(
     else if (f16) hipLaunchKernelGGL((paged_prefill_kernel<256, 256, 1, 1, true, 8>), grid, block, 0, st, p);
     else hipLaunchKernelGGL((paged_prefill_kernel<256, 256, 1, 1, false, 8>), grid, block, 0, st, p);
 #undef MI_LAUNCH_PREFILL
+    if (timed) (void)hipEventRecord(ev_b, st);
   }
   const int rc = mi_check_launch("mi_paged_prefill_attention");
   if (rc != MI_OK || !p.skip_single) return rc;
