@@ -114,7 +114,7 @@ def run_secondary(args, mi, lib, torch, dev):
         pairs = n * (new * ctx + new * (new + 1) // 2)          # (query row, visible key) pairs per head
         flops = 2 * Hq * (dk + dv) * pairs
         nbytes = n * (new + ctx) * Hkv * (dk + dv) * 2 + n * new * Hq * (dk + dv) * 2
-        kernel = "paged_prefill_pp_kernel" if dk <= 128 or mla else "paged_prefill_kernel"
+        kernel = "paged_prefill_pp_kernel"
         what = (f"paged varlen causal attention, {n} x {new} new tokens over {ctx} cached, {Hq}/{Hkv} heads, "
                 f"keys {dk} / values {dv} wide, chunk 256")
         dtype = "bf16 (fp32 accumulate)"

@@ -362,8 +362,10 @@ __global__ __launch_bounds__(64 * WAVES) void paged_prefill_kernel(PrefillParams
 // (36 dwords: the 16 rows of a fragment read start at 16 different multiples of four banks).
 // 192-wide keys (multi-latent attention): 416 (104 dwords = 8 x 13: the same bank pattern as 288); head_dim 96:
 // 208 (52 dwords = 4 x 13: the same pattern as 144).
-template <int HD> constexpr int pp_pitch() { return HD == 192 ? 416 : HD == 128 ? 288 : HD == 96 ? 208 : 144; }
-constexpr int kPPTile = 64;   // keys per staged tile
+// head_dim 256: 544 (136 dwords = 8 x 17).
+template <int HD> constexpr int pp_pitch() { return HD == 256 ? 544 : HD == 192 ? 416 : HD == 128 ? 288 : HD == 96 ? 208 : 144; }
+// keys per staged tile: 64; 32 at head_dim 256, where five 64-key buffers would not fit the 160 KB of LDS
+template <int HD> constexpr int pp_tile() { return HD == 256 ? 32 : 64; }
 
 // FP8: the cache holds e4m3 bytes with one fp32 scale per (chunk, KV head); a piece is multiplied by
 // its chunk's scale and rounded to bf16 on its way into LDS, so both matrix phases are the bf16 ones.
@@ -373,11 +375,16 @@ constexpr int kPPTile = 64;   // keys per staged tile
 // caches of multi-latent attention, whose value cache has its own strides.
 template <bool STAGGER, bool FP8, bool SPLIT, int HD, int HDK, bool F16>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
-  static_assert((HD == 128 && HDK == 128) || ((HD == 64 || HD == 96) && HDK == HD && !FP8) || (HD == 128 && HDK == 192 && !FP8),
-                "head_dim 128, or 64 / 96 with a 16-bit cache, or 192 / 128 with 16-bit caches");
+  static_assert((HD == 128 && HDK == 128) || ((HD == 64 || HD == 96 || HD == 192 || HD == 256) && HDK == HD && !FP8) ||
+                    (HD == 128 && HDK == 192 && !FP8),
+                "head_dim 128, or 64 / 96 / 192 / 256 with a 16-bit cache, or 192 / 128 with 16-bit caches");
   static_assert(!(FP8 && F16), "an fp8 cache is staged as bf16: bf16 queries only");
   constexpr bool MLA = HDK != HD;
-  constexpr int KS = HDK / 32, DV = HD / 16, NQ = 2, NT = 4, WAVES = 8;
+  // Wide heads (192, 256): 16 rows per wavefront instead of 32 -- the accumulators of 32 rows (96 / 128 registers)
+  // plus query fragments (48 / 64) leave no room for the operand fragments in a wavefront's 256 registers.
+  constexpr bool WIDE = HD >= 192;
+  constexpr int kPPTile = pp_tile<HD>();
+  constexpr int KS = HDK / 32, DV = HD / 16, NQ = WIDE ? 1 : 2, NT = kPPTile / 16, WAVES = 8;
   constexpr int kKPitch = pp_pitch<HDK>(), kVPitch = pp_pitch<HD>();
   constexpr int PPRK = HDK * 2 / 16;                 // 16-byte pieces per key row: 24 | 16 | 12 | 8
   constexpr int PPR = HD * 2 / 16;                   // 16-byte pieces (8 elements) per value row: 16 | 12 | 8
@@ -388,7 +395,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   constexpr int NPK = (kPPTile * PPRK + 511) / 512;  // key pieces per loader thread and tile: 3 | 2 | 2 | 1
   constexpr int RPP = 512 / PPR;         // value rows the 512 loader threads cover in one pass: 32 | - | 64
   constexpr int NPASS = (kPPTile * PPR + 511) / 512;  // value pieces per loader thread and tile: 2 | 2 | 1
-  constexpr int NH = HD == 64 ? 1 : 2;   // column groups of the output: 64 + 64, 48 + 48, or 64
+  constexpr int NH = HD == 64 ? 1 : WIDE ? HD / 64 : 2;   // column groups of the output: 64 + 64, 48 + 48, 64, or 3 / 4 x 64
   constexpr int EPG = HD / 16 / NH;      // 16-column blocks per group: 4 | 3 | 4
   constexpr int ESZ = FP8 ? 1 : 2;       // bytes per cache element
   constexpr int PIECE = FP8 ? 8 : 16;    // bytes one loader thread fetches of a row (8 elements)
@@ -640,12 +647,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       for (int kk = 0; kk < KS; ++kk) kf[kk] = *reinterpret_cast<const uint4*>(ks + 64 * kk);
     };
     auto sc_mma = [&](int u, const uint4 (&kf)[KS]) {
-      s[0][u] = mfma_16x16x32<F16>(kf[0], qf[0][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
-      s[1][u] = mfma_16x16x32<F16>(kf[0], qf[1][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+      for (int nt = 0; nt < NQ; ++nt) s[nt][u] = mfma_16x16x32<F16>(kf[0], qf[nt][0], f32x4_t{0.f, 0.f, 0.f, 0.f});
 #pragma unroll
       for (int kk = 1; kk < KS; ++kk) {
-        s[0][u] = mfma_16x16x32<F16>(kf[kk], qf[0][kk], s[0][u]);
-        s[1][u] = mfma_16x16x32<F16>(kf[kk], qf[1][kk], s[1][u]);
+#pragma unroll
+        for (int nt = 0; nt < NQ; ++nt) s[nt][u] = mfma_16x16x32<F16>(kf[kk], qf[nt][kk], s[nt][u]);
       }
     };
     // 192-wide keys: a sub-tile's product in two halves of three fragments (half the fragment registers)
@@ -658,8 +665,9 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 #pragma unroll
       for (int j = 0; j < 3; ++j) {
         const int kk = 3 * half + j;
-        s[0][u] = mfma_16x16x32<F16>(kf[j], qf[0][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[0][u]);
-        s[1][u] = mfma_16x16x32<F16>(kf[j], qf[1][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[1][u]);
+#pragma unroll
+        for (int nt = 0; nt < NQ; ++nt)
+          s[nt][u] = mfma_16x16x32<F16>(kf[j], qf[nt][kk % KS], kk == 0 ? f32x4_t{0.f, 0.f, 0.f, 0.f} : s[nt][u]);
       }
     };
     // O^T += V^T P^T: group grp = (32-key step grp / NH, output column group grp % NH of 64 or 48 columns):
@@ -674,17 +682,18 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     };
     auto pv_mma = [&](int grp, const uint2 (&af)[4][2]) {
       const int up = 2 * (grp / NH), e0 = EPG * (grp % NH);
-      const uint4 pp0 = make_uint4(pf[0][up].x, pf[0][up].y, pf[0][up + 1].x, pf[0][up + 1].y);
-      const uint4 pp1 = make_uint4(pf[1][up].x, pf[1][up].y, pf[1][up + 1].x, pf[1][up + 1].y);
+      uint4 pp[NQ];
+#pragma unroll
+      for (int nt = 0; nt < NQ; ++nt) pp[nt] = make_uint4(pf[nt][up].x, pf[nt][up].y, pf[nt][up + 1].x, pf[nt][up + 1].y);
 #pragma unroll
       for (int e = 0; e < EPG; ++e) {
         const uint4 a = make_uint4(af[e][0].x, af[e][0].y, af[e][1].x, af[e][1].y);
-        acc[0][e0 + e] = mfma_16x16x32<F16>(a, pp0, acc[0][e0 + e]);
-        acc[1][e0 + e] = mfma_16x16x32<F16>(a, pp1, acc[1][e0 + e]);
+#pragma unroll
+        for (int nt = 0; nt < NQ; ++nt) acc[nt][e0 + e] = mfma_16x16x32<F16>(a, pp[nt], acc[nt][e0 + e]);
       }
       if (grp % NH == NH - 1) {  // once per 32-key step
-        accl[0] = mfma_16x16x32<F16>(ones, pp0, accl[0]);
-        accl[1] = mfma_16x16x32<F16>(ones, pp1, accl[1]);
+#pragma unroll
+        for (int nt = 0; nt < NQ; ++nt) accl[nt] = mfma_16x16x32<F16>(ones, pp[nt], accl[nt]);
       }
     };
 #define MI_SB() __builtin_amdgcn_sched_barrier(0)
@@ -700,6 +709,46 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       uint2 a0[4][2], a1[4][2];
       uint4 k0[KS], k1[KS];
       const int ta = it - 1, ts = it;
+      if constexpr (WIDE) {
+        // One list of operand groups -- the value groups of tile it-1 (a 32-key step x 64 output columns each), then
+        // the 16-key score groups of tile it; the fragments of group i+1 are requested before the MFMAs of group i,
+        // in alternating registers.  Staging rides behind the first three groups.
+        constexpr int NPV = (kPPTile / 32) * NH, NG = NPV + NT;
+        static_assert(NG >= 3, "the staging hooks sit behind groups 0, 1 and 2");
+        uint2 ab[2][4][2];
+        uint4 kb[2][KS];
+        auto load = [&](int i) {
+          if (i < NPV) pv_load(ta, i, ab[i & 1]);
+          else sc_load(ts, i - NPV, kb[(i - NPV) & 1]);
+        };
+        auto mma = [&](int i) {
+          if (i < NPV) pv_mma(i, ab[i & 1]);
+          else sc_mma(i - NPV, kb[(i - NPV) & 1]);
+        };
+        int64_t off = 0;
+        int room = 0;
+        load(0);
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+          if (i + 1 < NG) load(i + 1);
+          MI_SB();
+          mma(i);
+          if (i == 0) {
+            store_k(it + 1);
+            store_v(it + 1);
+          } else if (i == 1) {
+            off = tile_offset(cur, pc_cur);
+            room = cur.room;
+            tile_loads_k(off, room);
+            cursor_next(cur);
+            pc_cur = bt_row[cur.ci];  // block-table entry of tile it+3, consumed one iteration from now
+          } else if (i == 2) {
+            tile_loads_v(off, room);
+          }
+          MI_SB();
+        }
+        return;
+      }
       if constexpr (HD == 64) {  // half the matrix work per tile: two value groups, four 4-MFMA score groups
         pv_load(ta, 0, a0);
         pv_load(ta, 1, a1); MI_SB();
@@ -789,11 +838,15 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         float tmax = fmaxf(fmaxf(s[nt][0][0], s[nt][0][1]), s[nt][0][2]);
         tmax = fmaxf(fmaxf(tmax, s[nt][0][3]), s[nt][1][0]);
         tmax = fmaxf(fmaxf(tmax, s[nt][1][1]), s[nt][1][2]);
-        tmax = fmaxf(fmaxf(tmax, s[nt][1][3]), s[nt][2][0]);
-        tmax = fmaxf(fmaxf(tmax, s[nt][2][1]), s[nt][2][2]);
-        tmax = fmaxf(fmaxf(tmax, s[nt][2][3]), s[nt][3][0]);
-        tmax = fmaxf(fmaxf(tmax, s[nt][3][1]), s[nt][3][2]);
-        tmax = fmaxf(tmax, s[nt][3][3]);
+        if constexpr (NT == 4) {
+          tmax = fmaxf(fmaxf(tmax, s[nt][1][3]), s[nt][2][0]);
+          tmax = fmaxf(fmaxf(tmax, s[nt][2][1]), s[nt][2][2]);
+          tmax = fmaxf(fmaxf(tmax, s[nt][2][3]), s[nt][3][0]);
+          tmax = fmaxf(fmaxf(tmax, s[nt][3][1]), s[nt][3][2]);
+          tmax = fmaxf(tmax, s[nt][3][3]);
+        } else {
+          tmax = fmaxf(tmax, s[nt][1][3]);
+        }
         tmax = rowgroup_max(tmax);
         const float m_raw = fmaxf(m_run[nt], tmax);
         const float m_use = m_raw == -INFINITY ? 0.f : m_raw;
@@ -898,7 +951,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 // Rows whose keys were split over several workgroups: o = sum_s 2^(lse_s - max) o_s / sum_s 2^(lse_s - max).
 // Grid (T, Hq), head_dim threads = the output values of one (row, head).
 template <bool F16>
-__global__ __launch_bounds__(128) void prefill_split_merge_kernel(PrefillParams p, int n_split, int head_dim) {
+__global__ __launch_bounds__(256) void prefill_split_merge_kernel(PrefillParams p, int n_split, int head_dim) {
   const int row = blockIdx.x, head = blockIdx.y, d = threadIdx.x;
   if (row >= p.cu_q[p.R]) return;  // padding rows: zeroed by the tile kernel
   if (p.skip_single) {             // one-row requests were left to the decode kernels
@@ -941,9 +994,9 @@ using namespace mi;
 // with thousands of keys to walk: then the keys are split so that about one workgroup per CU exists,
 // every one keeping at least sixteen 64-key tiles (a 512-token prompt is not worth the merge).  Host-side quantities only (the lengths live on the GPU).
 static int prefill_kv_splits(int T, int Hq, int Hkv, int head_dim, int max_kv_len) {
-  if ((head_dim != 128 && head_dim != 64 && head_dim != 96) || max_kv_len <= 0) return 1;
+  if (max_kv_len <= 0) return 1;
   const int G = Hq / Hkv, Gw = G < 16 ? G : 16, parts = (G + 15) / 16;
-  const int sbq = 8 * (32 / Gw);                         // query tokens per workgroup (8 wavefronts x 32 rows)
+  const int sbq = 8 * ((head_dim >= 192 ? 16 : 32) / Gw);  // query tokens per workgroup (8 wavefronts x 32 or 16 rows)
   const int64_t useful = (int64_t)Hkv * parts * ((T + sbq - 1) / sbq);
   const int cus = 256;
   if (useful >= cus) return 1;
@@ -1024,9 +1077,9 @@ static int launch_paged_prefill(
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: unknown kv_dtype");
   if (fp8 && (!k_scales || !v_scales))
     return mi_fail(MI_ERR_NULL, "mi_paged_prefill_attention_fp8: both scale arrays are required");
-  // the two-phase tile kernel stages 64-key tiles that must not straddle chunks and exists for the common widths;
-  // other chunk sizes and widths (and the knob) select the register-only kernel
-  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0 && head_dim <= 128;
+  // the two-phase tile kernel stages 64-key tiles that must not straddle chunks; other chunk sizes (and the knob)
+  // select the register-only kernel
+  const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0;
   if (fp8 && (head_dim != 128 || !two_phase || f16))
     return mi_fail(MI_ERR_UNSUPPORTED,
                    "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 128, a chunk size that is a "
@@ -1053,7 +1106,7 @@ static int launch_paged_prefill(
 
   hipStream_t st = (hipStream_t)stream;
   if (two_phase) {
-    const int sbq_lds = 8 * (32 / Gw);  // 8 wavefronts x whole tokens in a wavefront's 32 rows
+    const int sbq_lds = 8 * ((head_dim >= 192 ? 16 : 32) / Gw);  // 8 wavefronts x whole tokens in a wavefront's 32 (wide heads: 16) rows
     dim3 lgrid(((T + sbq_lds - 1) / sbq_lds + R) * Hkv * parts);
     hipEvent_t ev_a, ev_b;
     const bool timed = mi_profile_next(&ev_a, &ev_b);
@@ -1079,8 +1132,12 @@ static int launch_paged_prefill(
     else if (head_dim == 128) MI_PP_LAUNCH(false, 128, 128, false);
     else if (head_dim == 64 && f16) MI_PP_LAUNCH(false, 64, 64, true);
     else if (head_dim == 64) MI_PP_LAUNCH(false, 64, 64, false);
-    else if (f16) MI_PP_LAUNCH(false, 96, 96, true);
-    else MI_PP_LAUNCH(false, 96, 96, false);
+    else if (head_dim == 96 && f16) MI_PP_LAUNCH(false, 96, 96, true);
+    else if (head_dim == 96) MI_PP_LAUNCH(false, 96, 96, false);
+    else if (head_dim == 192 && f16) MI_PP_LAUNCH(false, 192, 192, true);
+    else if (head_dim == 192) MI_PP_LAUNCH(false, 192, 192, false);
+    else if (f16) MI_PP_LAUNCH(false, 256, 256, true);
+    else MI_PP_LAUNCH(false, 256, 256, false);
     if (timed) (void)hipEventRecord(ev_b, st);
     if (n_split > 1) {
       if (f16) hipLaunchKernelGGL(prefill_split_merge_kernel<true>, dim3(T, Hq), dim3(head_dim), 0, st, p, n_split, head_dim);

@@ -129,12 +129,13 @@ def _check_padded(mi, q, kc, vc, cu_q, lens, bt, tol=2e-2):
 @pytest.mark.parametrize("Hq,Hkv", [(8, 8), (32, 8), (12, 4), (16, 1)])
 @pytest.mark.parametrize("d", [96, 192, 256])
 def test_head_widths_96_192_256(mi, dev, d, Hq, Hkv, chunk, dtype):
-    """Head widths beside 64 and 128 in prefill and mixed batches (96: the two-phase tile kernel when the chunk size
-    allows, split keys included; 192 and 256: the register-only kernel): ragged new-token counts and contexts,
-    one-row requests through the decode kernels, padding rows."""
+    """Head widths beside 64 and 128 in prefill and mixed batches (the two-phase tile kernel when the chunk size
+    allows -- 16 rows per wavefront at 192 and 256, 32-key tiles at 256 -- split keys, the lock-step schedule and the
+    register-only kernel included): ragged new-token counts and contexts, one-row requests through the decode
+    kernels, padding rows."""
     q, kc, vc, cu_q, lens, bt = _ragged_case(mi, dev, Hq, Hkv, d, chunk, dtype, seed=d + Hq + chunk, pad_rows=3)
     _check_padded(mi, q, kc, vc, cu_q, lens, bt)
-    if d == 96 and chunk % 64 == 0:
+    if chunk % 64 == 0:
         for knobs in ({"prefill_kv_split": 3}, {"prefill_two_phase": 2}, {"prefill_two_phase": -1}):
             with mi.ops.tuning(**knobs):
                 _check_padded(mi, q, kc, vc, cu_q, lens, bt)
@@ -142,11 +143,9 @@ def test_head_widths_96_192_256(mi, dev, d, Hq, Hkv, chunk, dtype):
 
 @pytest.mark.parametrize("kernel", ["two_phase", "registers", "split_keys"])
 @pytest.mark.parametrize("Hq,Hkv", [(32, 1), (64, 2), (17, 1), (48, 2), (40, 2), (64, 1)])
-@pytest.mark.parametrize("d", [64, 96, 128, 256])
+@pytest.mark.parametrize("d", [64, 96, 128, 192, 256])
 def test_more_than_16_query_heads_per_kv_head(mi, dev, kernel, Hq, Hkv, d):
     """Up to 64 query heads per KV head: every 16 of them (the last group: the rest) take workgroups of their own."""
-    if d == 256 and kernel != "registers":
-        pytest.skip("width 256 always takes the register-only kernel")
     knobs = {"two_phase": {}, "registers": {"prefill_two_phase": -1}, "split_keys": {"prefill_kv_split": 3}}[kernel]
     q, kc, vc, cu_q, lens, bt = _ragged_case(mi, dev, Hq, Hkv, d, 64, torch.bfloat16, seed=Hq + d, pad_rows=2)
     with mi.ops.tuning(**knobs):
