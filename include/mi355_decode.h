@@ -280,8 +280,8 @@ int mi_paged_mla_decode_attention(const void* q, int64_t q_stride_tok, int64_t q
  * With a workspace of mi_prefill_workspace_bytes() bytes, requests that
  * have exactly one query row (the decode requests of a mixed batch) are streamed by the
  * decode kernels at full bandwidth; with workspace == NULL one kernel handles every request.
- * The same workspace lets the two-phase tile kernel (head_dim 64, 96 or 128, chunk size a multiple of 64; other
- * widths and chunk sizes run a register-only kernel) cut the keys of every request into ranges when
+ * The same workspace lets the two-phase tile kernel (chunk size a multiple of 64; other
+ * chunk sizes run a register-only kernel) cut the keys of every request into ranges when
  * the batch has few query rows over long contexts (a chunk of a prompt, a short turn after a long
  * history: without it a handful of workgroups would walk thousands of keys each): the ranges are
  * computed by separate workgroups and merged by log-sum-exp, as in the decode path.  `max_kv_len` (an
