@@ -54,18 +54,26 @@ struct NormRopeParams {
   int64_t bt_stride;
   const int32_t* lens;
   int32_t T, Hq, Hkv, d, rot, chunk, norm, interleaved, faithful, q_group;
+  uint32_t q_group_magic;  // ceil(2^32 / q_group): h / q_group = umulhi(h, magic) for q_group > 1 (h * q_group < 2^32)
   float eps, mscale;
 };
 
 // one rounding to the tensors' 16-bit type and back
 template <bool F16>
 static __device__ __forceinline__ float round16(float x) { return to_f32<F16>(f32_to_16<F16>(x)); }
+// the same for two values: one packed conversion and two unpacks
+template <bool F16>
+static __device__ __forceinline__ void round16_pair(float& a, float& b) {
+  const uint32_t packed = pack2<F16>(a, b);
+  a = lo_to_f32<F16>(packed);
+  b = hi_to_f32<F16>(packed);
+}
 
 // First element of head vector `vec` (query heads first, then key heads) of token t.
 static __device__ __forceinline__ const uint16_t* head_vector(const NormRopeParams& p, int t, int vec) {
   if (vec < p.Hq) {
     if (p.q_gst == 0) return p.q + (int64_t)t * p.q_st + (int64_t)vec * p.d;  // one group: contiguous heads
-    const int g = vec / p.q_group;
+    const int g = p.q_group == 1 ? vec : (int)__umulhi((uint32_t)vec, p.q_group_magic);
     return p.q + (int64_t)t * p.q_st + (int64_t)g * p.q_gst + (int64_t)(vec - g * p.q_group) * p.d;
   }
   return p.k + (int64_t)t * p.k_st + (int64_t)(vec - p.Hq) * p.k_hst;
@@ -133,7 +141,10 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
           }
           if ((which == 0 && p.Hq == 0) || (which == 1 && p.Hkv == 0)) continue;
           const float a = p.emb[(which ? kp : qp) * p.emb_stride + e];
-          float c = cosf(a) * p.mscale, sn = sinf(a) * p.mscale;
+          float c, sn;
+          rotary_sincos(a, &sn, &c);
+          c *= p.mscale;
+          sn *= p.mscale;
           if (faithful) {
             c = round16<F16>(c);
             sn = round16<F16>(sn);
@@ -223,9 +234,9 @@ __global__ __launch_bounds__(256) void norm_rope_append_kernel(NormRopeParams p)
 // the kernel is latency-bound unless enough workgroups are resident and independent loads are in
 // flight meanwhile: the first pass's head vector and the value row are requested before the chain,
 // and cos / sin / norm weights live in LDS or packed registers to stay within 64 VGPRs (8 waves per
-// SIMD).  Each angle's cos or sin is evaluated by exactly one thread of the workgroup.
+// SIMD).  Each angle's cos and sin are evaluated by exactly one thread of the workgroup.
 template <int D, bool F16>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) void norm_rope_append_vec_kernel(NormRopeParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(6, 8))) void norm_rope_append_vec_kernel(NormRopeParams p) {
   constexpr int LPV = D / 8;        // lanes that hold a head vector
   constexpr int LPG = LPV <= 8 ? 8 : LPV <= 16 ? 16 : 32;  // lane group of a head vector (a power of two)
   constexpr int VPW = 64 / LPG;     // head vectors per wave
@@ -275,28 +286,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
   __shared__ __align__(16) float cs_lds[2][2][D];  // [query | key position][cos | sin][element]
   const int half = p.rot >> 1;
   int src_lane = lane;   // lane holding the half-split partner elements (same j)
-  float psign = 0.f;     // sign of the partner term for half-split pairs
   bool same = true;      // query and key positions agree (uniform over the workgroup)
   if (p.emb) {
     const int64_t qp = p.q_pos ? p.q_pos[t] : 0;
     const int64_t kp = p.k_pos ? p.k_pos[t] : qp;
     same = kp == qp && p.Hq > 0;
-    for (int job = threadIdx.x; job < 4 * D; job += 256) {
-      const int which = job / (2 * D), fn = (job / D) & 1, e = job % D;
+    // one thread per (position, element): cos and sin together; the sine carries the sign of the partner term
+    // (half-split pairs: minus in the first half; interleaved pairs: minus at even elements)
+    for (int job = threadIdx.x; job < 2 * D; job += 256) {
+      const int which = job / D, e = job % D;
       if (which == 1 && same) break;
       if ((which == 0 && p.Hq == 0) || (which == 1 && p.Hkv == 0)) continue;
-      float r = fn ? 0.f : 1.f;
+      float c = 1.f, sn = 0.f;
       if (e < p.rot) {
-        const float a = p.emb[(which ? kp : qp) * p.emb_stride + e];
-        r = (fn ? sinf(a) : cosf(a)) * p.mscale;
-        if (faithful) r = round16<F16>(r);
+        rotary_sincos(p.emb[(which ? kp : qp) * p.emb_stride + e], &sn, &c);
+        c *= p.mscale;
+        sn *= p.mscale;
+        if (faithful) {
+          c = round16<F16>(c);
+          sn = round16<F16>(sn);
+        }
+        if (p.interleaved ? (e & 1) == 0 : e < half) sn = -sn;
       }
-      cs_lds[which][fn][e] = r;
+      cs_lds[which][0][e] = c;
+      cs_lds[which][1][e] = sn;
     }
     if (!p.interleaved) {
       const int pe = e0 < half ? e0 + half : e0 - half;  // partner of this lane's first element
       src_lane = lane - li + pe / 8;
-      psign = e0 < half ? -1.f : 1.f;
     }
   }
   // norm weights of this lane's elements, kept packed
@@ -315,6 +332,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
   }
   if (p.emb) __syncthreads();
 
+  // The loop below is bound by vector-instruction issue (about as many instructions as a copy of the same bytes
+  // leaves time for), so everything uniform is decided by scalar branches around whole element loops, lane
+  // exchanges are single data-parallel moves where the distance allows, and cos = 1 / sin = 0 past the rotary
+  // width make the rotation a pass-through there without a per-element test (non-finite inputs excepted: then the
+  // select below keeps the reference's behaviour).
+  const bool any_norm = p.norm != MI_NORM_NONE, rms = p.norm == MI_NORM_RMS;
+  const int plane = half >> 3;                         // lanes between the partners of a half-split pair
+  const bool pow2 = (half & 7) == 0 && plane > 0 && (plane & (plane - 1)) == 0 && 2 * plane <= LPG;
+  const bool full_rot = p.rot == D;
   for (int vec0 = blockIdx.y * VPB; vec0 < nvec; vec0 += gridDim.y * VPB) {
     const int vec = vec0 + slot;
     const bool active = vec < nvec;  // uniform over the LPV lanes of a vector
@@ -327,20 +353,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
       for (int j = 0; j < 4; ++j) { y[2 * j] = lo_to_f32<F16>(w4[j]); y[2 * j + 1] = hi_to_f32<F16>(w4[j]); }
     }
     raw = load_vec(vec + gridDim.y * VPB);  // next pass, in flight during this one
-    if (p.norm != MI_NORM_NONE) {
+    if (any_norm) {
       float ss = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) ss += y[j] * y[j];
-#pragma unroll
-      for (int o = LPG / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      ss = lane_group_sum<LPG>(ss);
       const float rstd = rsqrtf(ss * (1.f / D) + p.eps);
-      const uint4 wr = is_q ? wq_raw : wk_raw;
-      const uint32_t w4[4] = {wr.x, wr.y, wr.z, wr.w};
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float v = y[j] * rstd;
-        if (p.norm == MI_NORM_RMS) v *= (j & 1) ? hi_to_f32<F16>(w4[j >> 1]) : lo_to_f32<F16>(w4[j >> 1]);
-        y[j] = faithful ? round16<F16>(v) : v;
+      for (int j = 0; j < 8; ++j) y[j] *= rstd;
+      if (rms) {
+        const uint4 wr = is_q ? wq_raw : wk_raw;
+        const uint32_t w4[4] = {wr.x, wr.y, wr.z, wr.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { y[2 * j] *= lo_to_f32<F16>(w4[j]); y[2 * j + 1] *= hi_to_f32<F16>(w4[j]); }
+      }
+      if (faithful) {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) round16_pair<F16>(y[j], y[j + 1]);
       }
     }
     float o[8];
@@ -348,7 +377,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
     for (int j = 0; j < 8; ++j) o[j] = y[j];
     if (p.emb) {
       const int which = (is_q || same) ? 0 : 1;
-      float c[8], sn[8];
+      float c[8], sn[8], yp[8];
 #pragma unroll
       for (int j = 0; j < 8; j += 4) {
         const float4 c4 = *reinterpret_cast<const float4*>(&cs_lds[which][0][e0 + j]);
@@ -356,13 +385,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(8, 8))) voi
         c[j] = c4.x; c[j + 1] = c4.y; c[j + 2] = c4.z; c[j + 3] = c4.w;
         sn[j] = s4.x; sn[j + 1] = s4.y; sn[j + 2] = s4.z; sn[j + 3] = s4.w;
       }
+      if (p.interleaved) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        float yp;
-        if (p.interleaved) yp = (j & 1) ? y[j ^ 1] : -y[j ^ 1];
-        else yp = __shfl(y[j], src_lane, 64) * psign;
-        // elements past the rotary width carry cos = 1, sin = 0 in the table
-        if (e0 + j < p.rot) o[j] = faithful ? round16<F16>(y[j] * c[j]) + round16<F16>(yp * sn[j]) : y[j] * c[j] + yp * sn[j];
+        for (int j = 0; j < 8; ++j) yp[j] = y[j ^ 1];
+      } else if (pow2) {  // the partner lane is lane ^ plane
+#define MI_PARTNERS(P_)                                  \
+  _Pragma("unroll") for (int j = 0; j < 8; ++j) yp[j] = lane_xor<P_>(y[j])
+        if (plane == 8) { MI_PARTNERS(8); }
+        else if (plane == 4) { MI_PARTNERS(4); }
+        else if (plane == 16) { MI_PARTNERS(16); }
+        else if (plane == 2) { MI_PARTNERS(2); }
+        else { MI_PARTNERS(1); }
+#undef MI_PARTNERS
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) yp[j] = __shfl(y[j], src_lane, 64);
+      }
+      if (faithful) {
+#pragma unroll
+        for (int j = 0; j < 8; j += 2) {
+          float a0 = y[j] * c[j], a1 = y[j + 1] * c[j + 1], b0 = yp[j] * sn[j], b1 = yp[j + 1] * sn[j + 1];
+          round16_pair<F16>(a0, a1);
+          round16_pair<F16>(b0, b1);
+          o[j] = a0 + b0;
+          o[j + 1] = a1 + b1;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = y[j] * c[j] + yp[j] * sn[j];
+      }
+      if (!full_rot) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = e0 + j < p.rot ? o[j] : y[j];
       }
     }
     if (active && lane_on) {
@@ -393,6 +447,7 @@ int norm_rope_launch(NormRopeParams& p, int32_t dtype, const MiTuning* tuning, h
     return mi_fail(code, msg);
   };
   if (p.T == 0) return MI_OK;
+  p.q_group_magic = p.q_group > 1 ? (uint32_t)((((uint64_t)1 << 32) + p.q_group - 1) / p.q_group) : 0u;
   MiTuning tune;
   const int rc_t = mi_resolve_tuning(tuning, &tune, name);
   if (rc_t != MI_OK) return rc_t;

@@ -200,8 +200,9 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
         float c = 1.f, sn = 0.f;  // elements past the rotary width pass through
         if (e < p.rot) {
           const float a = ang[i];
-          c = cosf(a) * p.mscale;
-          sn = sinf(a) * p.mscale;
+          rotary_sincos(a, &sn, &c);
+          c *= p.mscale;
+          sn *= p.mscale;
           if (faithful) {
             c = to_f32<F16>(f32_to_16<F16>(c));
             sn = to_f32<F16>(f32_to_16<F16>(sn));

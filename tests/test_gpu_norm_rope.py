@@ -72,6 +72,34 @@ def _norm_rope_case(mi, dev, norm, interleaved, d, rot):
         assert torch.equal(kd.cpu(), k), "the key input must not be modified"
 
 
+@pytest.mark.parametrize("vectorised", [1, -1])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+def test_large_rotary_angles(mi, dev, vectorised, dtype):
+    """Angles far beyond one turn: rows of the table reach 1e3, 1e5, 1e6 (the kernels' own range reduction) and 3e7 rad
+    (the library functions behind it); the result still equals the op-by-op chain, whose cos / sin are the host's."""
+    gen = torch.Generator().manual_seed(5)
+    T, Hq, Hkv, d = 64, 4, 2, 128
+    tops = [1e3, 1e5, 1e6, 3e7]
+    table = torch.stack([torch.rand(d, generator=gen) * tops[i % 4] for i in range(T)]).float()
+    table[:, d // 2:] = table[:, :d // 2]  # half-split pairs share an angle
+    pos = torch.randperm(T, generator=gen)
+    q = torch.randn(T, 1, Hq, d, generator=gen).to(dtype)
+    k = torch.randn(T, 1, Hkv, d, generator=gen).to(dtype)
+    q_ref = orn.norm_rope(q.squeeze(1), pos, table, norm=None)
+    k_ref = orn.norm_rope(k.squeeze(1), pos, table, norm=None)
+    with mi.ops.tuning(norm_rope_vectorised=vectorised):
+        qd, kd = q.to(dev).clone(), k.to(dev)
+        k_out = torch.empty_like(kd)
+        mi.ops.norm_rope_append(qd, kd, key_out=k_out, rotary_emb=table.to(dev), q_positions=pos.to(dev),
+                                k_positions=pos.to(dev), faithful_rounding=True)
+        torch.cuda.synchronize()
+    ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -10
+    for got, ref in ((qd.cpu().squeeze(1), q_ref), (k_out.cpu().squeeze(1), k_ref)):
+        err = (got.float() - ref.float()).abs()
+        assert (got != ref).float().mean().item() < 0.01
+        assert (err <= 2 * ulp * ref.float().abs().amax(-1, keepdim=True)).all(), f"max err {err.max().item()}"
+
+
 def test_position_zero_is_identity_and_passthrough_tail(mi, dev):
     T, H, d, rot = 5, 4, 128, 64
     x = torch.randn(T, 1, H, d).bfloat16().to(dev)
