@@ -219,6 +219,14 @@ static __device__ void find_crossing(const uint64_t* hist, uint64_t above, uint6
 }
 
 constexpr int kMemberCap = 4096;  // members of the chosen value bin that fit the LDS list
+// Top-k with a small k (the usual 20-100) needs none of the row-wide histogram passes: a threshold is estimated
+// from kMemberCap values spread over the row so that about kCandidateTarget elements lie at or above it, ONE pass
+// finds the maximum and lists those candidates, and the exact k-th largest value and the draw are then worked out
+// on the list.  When the estimate misses (fewer than k candidates, or more than the list holds: flat rows), the
+// general path below runs instead; the result is the same either way.
+constexpr int kFastTopK = 256;          // largest k the one-pass form is tried for
+constexpr int kFastMinVocab = 16384;    // smallest row it is tried for
+constexpr int kCandidateTarget = 1024;  // expected candidates (standard deviation ~ target / sqrt(sample rank))
 
 template <int DT, int VEC>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) {
@@ -231,6 +239,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   __shared__ int32_t pick[2];
   __shared__ uint32_t member_count;
   __shared__ uint32_t member_key[kMemberCap];
+  __shared__ int32_t member_idx[kMemberCap];    // one-pass top-k only: vocabulary index of a candidate
   __shared__ uint64_t member_mass[kMemberCap];
 
   const int r = blockIdx.x;
@@ -239,13 +248,69 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   const bool greedy = p.top_k == 1;
   const RowReader<DT, VEC> rd{reinterpret_cast<const uint8_t*>(p.logits) + (int64_t)r * p.stride * (DT != 0 ? 2 : 4), V,
                                 p.inv_temperature, !greedy && p.inv_temperature != 1.0f};
-  constexpr int U = 8;  // loads in flight per thread
+  constexpr int U = VEC == 8 ? 4 : 8;  // 16-byte loads in flight per thread (32 values either way)
 
   // ---- pass A: maximum (lowest index among equals, NaN counts as largest) and finite minimum ----
   // (a thread meets its elements in rising index order, so "strictly greater" keeps the first)
   uint32_t bk = 0; int bi = 0x7fffffff; float mn = INFINITY;
   const bool filtering = !greedy && (p.top_k > 1 || p.top_p > 0.f);
-  if (filtering) {
+  // `digit_select`: the key with exactly `target` list members (weights: 1, or the members' masses) above it, by four
+  // 8-bit digit passes over member_key[0..n) starting from `above` (the weight already counted above the list).
+  // With last_digit > 0 the low digits stay zero: a key at or below the exact one (a threshold that errs on the
+  // side of more members).
+  auto digit_select = [&](int n, uint64_t target, uint64_t above, bool by_mass, int last_digit) -> uint32_t {
+    uint32_t pmask = 0, pval = 0;
+    for (int d = 3; d >= last_digit; --d) {
+      __syncthreads();
+      if (tid < 256) hist[tid] = 0;
+      __syncthreads();
+      for (int j0 = 0; j0 < n; j0 += kSampleThreads) {
+        const int j = j0 + tid;
+        const bool in = j < n;
+        const uint32_t k = in ? member_key[j] : 0;
+        hist_add(hist, 255 - (int)((k >> (8 * d)) & 255u), in && (k & pmask) == pval, lane,
+                 [&] { return by_mass ? member_mass[j] : (uint64_t)1; });
+      }
+      __syncthreads();
+      if (wave == 0) find_crossing(hist, above, target, res, lane);
+      __syncthreads();
+      const uint32_t digit = 255u - (uint32_t)res[0];  // the crossing lies inside the list, so a digit is always found
+      above = res[1];
+      pmask |= 0xffu << (8 * d);
+      pval |= digit << (8 * d);
+    }
+    return pval;
+  };
+  const bool one_pass = !greedy && p.top_k > 1 && p.top_k <= kFastTopK && V >= kFastMinVocab;
+  if (one_pass) {
+    // threshold: the rank-th largest of kMemberCap sampled values, rank chosen for ~kCandidateTarget candidates
+    const int blk = V / kSampleThreads;  // >= 16: thread t samples elements t * blk .. + 3
+#pragma unroll
+    for (int j = 0; j < kMemberCap / kSampleThreads; ++j)
+      member_key[tid * (kMemberCap / kSampleThreads) + j] = order_key(rd.at(tid * blk + j));
+    const int rank = (int)(((int64_t)kCandidateTarget * kMemberCap + V - 1) / V);
+    // (the upper 16 bits of the key are enough: sign, exponent and 7 bits of the fraction)
+    const uint32_t tau = digit_select(kMemberCap, (uint64_t)(rank - 1), 0, false, 2);
+    if (tid == 0) member_count = 0;
+    __syncthreads();  // the sample has been read by everyone; the list is reused for the candidates
+    sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
+      const uint32_t k = order_key(x);
+      const bool up = in && k > bk;
+      bk = up ? k : bk; bi = up ? i : bi;
+      const bool cand = in && k >= tau;
+      const uint64_t m = __builtin_amdgcn_ballot_w64(cand);
+      if (m == 0) return;
+      uint32_t base = 0;
+      const int first = __builtin_ctzll(m);
+      if (lane == first) base = atomicAdd(&member_count, (uint32_t)__builtin_popcountll(m));
+      base = __builtin_amdgcn_readlane(base, first);
+      const uint32_t at = base + (uint32_t)__builtin_popcountll(m & (((uint64_t)1 << lane) - 1));
+      if (cand && at < (uint32_t)kMemberCap) {
+        member_key[at] = k;
+        member_idx[at] = i;
+      }
+    });
+  } else if (filtering) {
     sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
       const uint32_t k = order_key(x);
       const bool up = in && k > bk;
@@ -285,7 +350,29 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   if (drawable) {
     const bool by_count = p.top_k > 1;
     const bool filtered = by_count || p.top_p > 0.f;
-    if (filtered) {
+    bool cut_from_list = false;
+    int n_candidates = 0;
+    if (one_pass) {
+      n_candidates = (int)member_count;  // (published by the barrier of the maximum's reduction)
+      if (n_candidates >= p.top_k && n_candidates <= kMemberCap) {
+        cut_key = digit_select(n_candidates, (uint64_t)(p.top_k - 1), 0, false, 0);
+        cut_from_list = true;
+      } else {
+        // the general path needs the finite minimum, which the one-pass sweep did not track
+        sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int, float x, bool in) {
+          mn = (in && x > -INFINITY) ? fminf(mn, x) : mn;
+        });
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) mn = fminf(mn, __shfl_xor(mn, m, 64));
+        __syncthreads();
+        if (lane == 0) red_min[wave] = mn;
+        __syncthreads();
+        mn = red_min[0];
+#pragma unroll
+        for (int w = 1; w < kSampleWaves; ++w) mn = fminf(mn, red_min[w]);
+      }
+    }
+    if (filtered && !cut_from_list) {
       // ---- pass B: 256 linear bins over [mx - range, mx], bin 0 = largest values ----
       float range = mx - mn;
       if (!by_count) range = fminf(range, 32.f);  // mass below exp(-32) cannot move a top-p cut
@@ -368,67 +455,108 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
       }
     }
 
-    // ---- draw: inverse CDF over the kept elements in vocabulary order ----
-    auto kept_mass = [&](float x) -> uint64_t { return order_key(x) >= cut_key ? mass_of(x, neg_mx) : 0; };
-    const int L1 = ((V + kSampleWaves - 1) / kSampleWaves + 63) & ~63;  // elements per first-level range
-    {
-      const int a = min(wave * L1, V), b = min(a + L1, V);
-      uint64_t s = 0;
-      sweep<U>(rd, a, b, lane, 64, [&](int, float x, bool in) { s += in ? kept_mass(x) : 0; });
-      s = wave_sum_u64(s);
-      if (lane == 0) wsum[wave] = s;
-    }
-    __syncthreads();
-    uint64_t total = 0;
-#pragma unroll
-    for (int w = 0; w < kSampleWaves; ++w) total += wsum[w];
-    // total > 0: the maximum itself is always kept and has the largest mass
-    uint64_t want = (uint64_t)((double)p.uniform[r] * (double)total);
-    want = want < total ? want : total - 1;
-    int w1 = 0;
-#pragma unroll
-    for (int w = 0; w < kSampleWaves - 1; ++w) {
-      const bool pass = w == w1 && want >= wsum[w];
-      want -= pass ? wsum[w] : 0;
-      w1 += pass ? 1 : 0;
-    }
-    // (ranges after the last non-empty one hold no mass, so w1 stops inside the vocabulary)
-    const int a1 = min(w1 * L1, V), b1 = min(a1 + L1, V);
-    const int L2 = (L1 / kSampleWaves + 63) & ~63;  // elements per second-level range
-    __syncthreads();
-    {
-      const int a = min(a1 + wave * L2, b1), b = min(a + L2, b1);
-      uint64_t s = 0;
-      sweep<1>(rd, a, b, lane, 64, [&](int, float x, bool in) { s += in ? kept_mass(x) : 0; });
-      s = wave_sum_u64(s);
-      if (lane == 0) wsum[wave] = s;
-    }
-    __syncthreads();
-    int w2 = 0;
-#pragma unroll
-    for (int w = 0; w < kSampleWaves - 1; ++w) {
-      const bool pass = w == w2 && want >= wsum[w];
-      want -= pass ? wsum[w] : 0;
-      w2 += pass ? 1 : 0;
-    }
-    const int a2 = min(a1 + w2 * L2, b1), b2 = min(a2 + L2, b1);
-    if (wave == 0) {
-      // third level: each lane owns a contiguous run of the sub-range
-      const int per = L2 / 64;
-      const int a = min(a2 + lane * per, b2), b = min(a + per, b2);
-      uint64_t s = 0;
-      for (int i = a; i < b; ++i) s += kept_mass(rd.at(i));
-      const uint64_t incl = wave_scan_incl_u64(s, lane);
-      const uint64_t m = __builtin_amdgcn_ballot_w64(incl > want);
-      const int owner = m ? __builtin_ctzll(m) : 63;
-      if (lane == owner) {
-        uint64_t run = incl - s;
-        int found = b > a ? b - 1 : bi;
-        for (int i = a; i < b; ++i) {
-          run += kept_mass(rd.at(i));
-          if (run > want) { found = i; break; }
+    // ---- draw on the candidate list: the kept elements are among the candidates, so when they are few the
+    // inverse CDF in vocabulary order is a direct count over the list (each thread owns one kept element and sums
+    // the masses of those at or before it) ----
+    bool drawn = false;
+    if (cut_from_list) {
+      __syncthreads();
+      if (tid == 0) member_count = 0;
+      __syncthreads();
+      for (int j0 = 0; j0 < n_candidates; j0 += kSampleThreads) {
+        const int j = j0 + tid;
+        const bool kept = j < n_candidates && member_key[j] >= cut_key;
+        const uint64_t m = __builtin_amdgcn_ballot_w64(kept);
+        if (m == 0) continue;
+        uint32_t base = 0;
+        const int first = __builtin_ctzll(m);
+        if (lane == first) base = atomicAdd(&member_count, (uint32_t)__builtin_popcountll(m));
+        base = __builtin_amdgcn_readlane(base, first);
+        const uint32_t at = base + (uint32_t)__builtin_popcountll(m & (((uint64_t)1 << lane) - 1));
+        // (vocabulary index and mass of a kept element in one word: a mass fits 32 bits)
+        if (kept) member_mass[at] = ((uint64_t)(uint32_t)member_idx[j] << 32) | mass_of(order_key_value(member_key[j]), neg_mx);
+      }
+      __syncthreads();
+      const int n_kept = (int)member_count;
+      if (n_kept <= kSampleThreads) {
+        const uint64_t mine = tid < n_kept ? member_mass[tid] : 0;
+        const uint32_t my_idx = (uint32_t)(mine >> 32);
+        uint64_t total = 0, upto = 0;  // all kept mass; kept mass at vocabulary indices <= mine
+        for (int m = 0; m < n_kept; ++m) {
+          const uint64_t e = member_mass[m];  // the same word for every lane: a broadcast read
+          const uint64_t w = e & 0xffffffffu;
+          total += w;
+          upto += (uint32_t)(e >> 32) <= my_idx ? w : 0;
         }
-        pick[0] = found;
+        uint64_t want = (uint64_t)((double)p.uniform[r] * (double)total);
+        want = want < total ? want : total - 1;
+        const uint64_t w_mine = mine & 0xffffffffu;
+        if (tid < n_kept && upto > want && upto - w_mine <= want) pick[0] = (int)my_idx;
+        drawn = true;
+      }
+    }
+    auto kept_mass = [&](float x) -> uint64_t { return order_key(x) >= cut_key ? mass_of(x, neg_mx) : 0; };
+    if (!drawn) {
+      const int L1 = ((V + kSampleWaves - 1) / kSampleWaves + 63) & ~63;  // elements per first-level range
+      {
+        const int a = min(wave * L1, V), b = min(a + L1, V);
+        uint64_t s = 0;
+        sweep<U>(rd, a, b, lane, 64, [&](int, float x, bool in) { s += in ? kept_mass(x) : 0; });
+        s = wave_sum_u64(s);
+        if (lane == 0) wsum[wave] = s;
+      }
+      __syncthreads();
+      uint64_t total = 0;
+#pragma unroll
+      for (int w = 0; w < kSampleWaves; ++w) total += wsum[w];
+      // total > 0: the maximum itself is always kept and has the largest mass
+      uint64_t want = (uint64_t)((double)p.uniform[r] * (double)total);
+      want = want < total ? want : total - 1;
+      int w1 = 0;
+#pragma unroll
+      for (int w = 0; w < kSampleWaves - 1; ++w) {
+        const bool pass = w == w1 && want >= wsum[w];
+        want -= pass ? wsum[w] : 0;
+        w1 += pass ? 1 : 0;
+      }
+      // (ranges after the last non-empty one hold no mass, so w1 stops inside the vocabulary)
+      const int a1 = min(w1 * L1, V), b1 = min(a1 + L1, V);
+      const int L2 = (L1 / kSampleWaves + 63) & ~63;  // elements per second-level range
+      __syncthreads();
+      {
+        const int a = min(a1 + wave * L2, b1), b = min(a + L2, b1);
+        uint64_t s = 0;
+        sweep<1>(rd, a, b, lane, 64, [&](int, float x, bool in) { s += in ? kept_mass(x) : 0; });
+        s = wave_sum_u64(s);
+        if (lane == 0) wsum[wave] = s;
+      }
+      __syncthreads();
+      int w2 = 0;
+#pragma unroll
+      for (int w = 0; w < kSampleWaves - 1; ++w) {
+        const bool pass = w == w2 && want >= wsum[w];
+        want -= pass ? wsum[w] : 0;
+        w2 += pass ? 1 : 0;
+      }
+      const int a2 = min(a1 + w2 * L2, b1), b2 = min(a2 + L2, b1);
+      if (wave == 0) {
+        // third level: each lane owns a contiguous run of the sub-range
+        const int per = L2 / 64;
+        const int a = min(a2 + lane * per, b2), b = min(a + per, b2);
+        uint64_t s = 0;
+        for (int i = a; i < b; ++i) s += kept_mass(rd.at(i));
+        const uint64_t incl = wave_scan_incl_u64(s, lane);
+        const uint64_t m = __builtin_amdgcn_ballot_w64(incl > want);
+        const int owner = m ? __builtin_ctzll(m) : 63;
+        if (lane == owner) {
+          uint64_t run = incl - s;
+          int found = b > a ? b - 1 : bi;
+          for (int i = a; i < b; ++i) {
+            run += kept_mass(rd.at(i));
+            if (run > want) { found = i; break; }
+          }
+          pick[0] = found;
+        }
       }
     }
     __syncthreads();

@@ -51,14 +51,15 @@ _retired_workspaces: list = []   # outgrown buffers stay alive: work already enq
 _workspace_override: list = []   # innermost ``use_workspace`` buffer
 
 
-def _workspace(device: torch.device, nbytes: int) -> Optional[Tensor]:
+def _workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> Optional[Tensor]:
+    """Scratch for a call on ``stream`` (the handle the caller already looked up; default: the current one)."""
     if nbytes <= 0:
         return None
     if _workspace_override:
         ws = _workspace_override[-1]
         _require(ws.device == device and ws.numel() >= nbytes, "the workspace given to use_workspace is too small")
         return ws
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    key = (device, torch.cuda.current_stream(device).cuda_stream if stream is None else stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
@@ -307,7 +308,7 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
                            v_scales: Optional[Tensor] = None) -> Tensor:
     """One query token per request against the paged cache; returns a tensor shaped like ``q``."""
     lib = _lib.load()
-    _stream(q)  # device check first: there is no CPU path
+    stream = _stream(q)  # device check first: there is no CPU path
     q3 = _qo_view(q, "q")
     R, Hq, D = q3.shape
     N, C, Hkv, Dk = k_cache.shape
@@ -337,14 +338,14 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
     tune = _tuning_arg()
     need = lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, C, max_kv_len, split_tokens, tune)
     if workspace is None:
-        workspace = _workspace(q.device, need)
+        workspace = _workspace(q.device, need, stream)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _lib.check(lib.mi_paged_decode_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
         block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
         _ptr(workspace), ws_bytes, R, Hq, Hkv, D, C, int(max_kv_len), int(split_tokens), float(softmax_scale),
         MI_KV_FP8_E4M3 if fp8 else MI_KV_16BIT, _ptr(k_scales), _ptr(v_scales), _dtype_code(q3, "q"), tune,
-        _stream(q)), "mi_paged_decode_attention")
+        stream), "mi_paged_decode_attention")
     return out
 
 
@@ -748,7 +749,7 @@ def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value:
     tune = _tuning_arg()
     need = lib.mi_decode_workspace_bytes(R, Hq, Hkv, D, C, max_kv_len, split_tokens, tune)
     if workspace is None:
-        workspace = _workspace(ref.device, need)
+        workspace = _workspace(ref.device, need, stream)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     _lib.check(lib.mi_decode_step_attention(
         q_ptr, q_st, q_gst, k_ptr, k_st, k_hst, v_ptr, v_st, v_hst, _ptr(q_weight), _ptr(k_weight), float(eps),

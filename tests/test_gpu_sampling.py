@@ -180,6 +180,33 @@ def test_draw_frequencies_follow_the_kept_probabilities(mi, dev, mode):
     assert ((freq - pr).abs() <= 5 * sigma + 1e-6).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("k", [2, 10, 200, 256, 257])
+def test_top_k_one_pass_form_and_its_fallbacks(mi, dev, dtype, k):
+    """Rows of 32 768 and a small k take the form that lists candidates above a sampled threshold in one pass; rows
+    where the estimate cannot work -- flat (every value a candidate), a few finite values (fewer candidates than k),
+    a spike in an otherwise flat row, half the row tied at the maximum -- must come out the same through the general
+    path.  k = 257 never takes the one-pass form."""
+    V = 32768
+    x = _logits(10, V, 900 + k, dtype)
+    x[0, :] = -0.75                                             # flat: every entry equals the cut
+    x[1, :] = float("-inf"); x[1, [5, 17000, 32767]] = torch.tensor([0.5, 1.5, 1.0], dtype=dtype)  # three finite values
+    x[2, :] = 0.25; x[2, 12345] = 9.0                           # one spike over a flat row
+    x[3, : V // 2] = 3.0                                        # half the row tied at the top
+    x[4, ::2] = float("-inf")                                   # every other entry pre-masked
+    x[5] = (torch.arange(V).float() / V).to(dtype)              # sorted ascending: the sample sees every level
+    x[6] = (torch.arange(V, 0, -1).float() / V).to(dtype)
+    u = torch.rand(10, generator=torch.Generator().manual_seed(k))
+    s, _, cut = mi.ops.sample_from_logits(x.to(dev), top_k=k, uniform=u.to(dev), return_cut=True)
+    xs = osm.scaled_logits(x, 1.0)
+    kth = torch.topk(xs, k, dim=-1).values[:, -1]
+    assert torch.equal(cut.cpu(), kth)
+    _check_draw(xs, kth, u, s.cpu())
+    assert s[1].item() in (5, 17000, 32767) and (k > 1 and s[2].item() >= 0)
+    s2, _ = mi.ops.sample_from_logits(x.to(dev), top_k=k, uniform=u.to(dev))
+    assert torch.equal(s, s2)
+
+
 def test_extreme_rows(mi, dev):
     V = 4096
     x = _logits(6, V, 41)
