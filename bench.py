@@ -67,6 +67,7 @@ SECONDARY_WORKLOADS = {
     "prefill_d128_mqa": ("prefill", dict(Hq=64, Hkv=2, d=128, n=8, new=2048, ctx=2048)),
     "sampling_top_k": ("sampling", dict(R=64, V=128256, top_k=50, top_p=0.0)),
     "sampling_top_p": ("sampling", dict(R=64, V=128256, top_k=0, top_p=0.9)),
+    "sampling_top_p_peaked": ("sampling", dict(R=64, V=128256, top_k=0, top_p=0.9, peaked=True)),
     "sampling_greedy": ("sampling", dict(R=64, V=128256, top_k=1, top_p=0.0)),
     "log_probs_bf16": ("log_probs", dict(T=4096, V=131072, bf16=True)),
     "log_probs_fp32": ("log_probs", dict(T=4096, V=131072, bf16=False)),
@@ -121,13 +122,19 @@ def run_secondary(args, mi, lib, torch, dev):
         timed_by_library = True
     elif kind == "sampling":
         R, V = prm["R"], prm["V"]
-        logits = (torch.randn(R, V, generator=gen) * 3).to(dev)
+        logits = torch.randn(R, V, generator=gen) * 3
+        if prm.get("peaked"):  # a language model's rows: a few dozen tokens far above the rest
+            logits *= 2.0 / 3.0
+            for r in range(R):
+                logits[r, torch.randperm(V, generator=gen)[:32]] += torch.rand(32, generator=gen) * 6 + 9
+        logits = logits.to(dev)
         u = torch.rand(R, generator=gen).to(dev)
         step = lambda: mi.ops.sample_from_logits(logits, top_k=prm["top_k"], top_p=prm["top_p"], temperature=0.8,
                                                  uniform=u)
         nbytes = R * V * 4 + R * 12
         kernel = "sample_kernel"
-        what = f"sampling of {R} rows of {V} fp32 logits, top_k {prm['top_k']}, top_p {prm['top_p']}, temperature 0.8"
+        what = (f"sampling of {R} rows of {V} fp32 logits ({'32 tokens 9-15 above a N(0, 2) bulk' if prm.get('peaked') else 'N(0, 3)'}), "
+                f"top_k {prm['top_k']}, top_p {prm['top_p']}, temperature 0.8")
         dtype = "fp32 logits, 2^-32 fixed-point mass"
         timed_by_library = False
     else:

@@ -222,8 +222,10 @@ constexpr int kMemberCap = 4096;  // members of the chosen value bin that fit th
 // Top-k with a small k (the usual 20-100) needs none of the row-wide histogram passes: a threshold is estimated
 // from kMemberCap values spread over the row so that about kCandidateTarget elements lie at or above it, ONE pass
 // finds the maximum and lists those candidates, and the exact k-th largest value and the draw are then worked out
-// on the list.  When the estimate misses (fewer than k candidates, or more than the list holds: flat rows), the
-// general path below runs instead; the result is the same either way.
+// on the list.  Top-p does the same with one more pass for the row's total mass; its cut lies inside the list
+// whenever the candidates alone hold more than top_p of that mass (peaked rows: the usual case).  When the estimate
+// misses (fewer than k candidates, more than the list holds -- flat rows --, too little mass), the general path
+// below runs instead; the result is the same either way.
 constexpr int kFastTopK = 256;          // largest k the one-pass form is tried for
 constexpr int kFastMinVocab = 16384;    // smallest row it is tried for
 constexpr int kCandidateTarget = 1024;  // expected candidates (standard deviation ~ target / sqrt(sample rank))
@@ -281,23 +283,24 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
     }
     return pval;
   };
-  const bool one_pass = !greedy && p.top_k > 1 && p.top_k <= kFastTopK && V >= kFastMinVocab;
+  const bool one_pass = !greedy && V >= kFastMinVocab &&
+                        (p.top_k > 1 ? p.top_k <= kFastTopK : p.top_p > 0.f);  // (top-p: one more pass for the total mass)
+  constexpr int kSamplesPerThread = kMemberCap / kSampleThreads;
+  uint32_t tau = 0;
   if (one_pass) {
     // threshold: the rank-th largest of kMemberCap sampled values, rank chosen for ~kCandidateTarget candidates
     const int blk = V / kSampleThreads;  // >= 16: thread t samples elements t * blk .. + 3
 #pragma unroll
-    for (int j = 0; j < kMemberCap / kSampleThreads; ++j)
-      member_key[tid * (kMemberCap / kSampleThreads) + j] = order_key(rd.at(tid * blk + j));
+    for (int j = 0; j < kSamplesPerThread; ++j)
+      member_key[tid * kSamplesPerThread + j] = order_key(rd.at(tid * blk + j));
     const int rank = (int)(((int64_t)kCandidateTarget * kMemberCap + V - 1) / V);
     // (the upper 16 bits of the key are enough: sign, exponent and 7 bits of the fraction)
-    const uint32_t tau = digit_select(kMemberCap, (uint64_t)(rank - 1), 0, false, 2);
+    tau = digit_select(kMemberCap, (uint64_t)(rank - 1), 0, false, 2);
     if (tid == 0) member_count = 0;
     __syncthreads();  // the sample has been read by everyone; the list is reused for the candidates
-    sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
-      const uint32_t k = order_key(x);
-      const bool up = in && k > bk;
-      bk = up ? k : bk; bi = up ? i : bi;
-      const bool cand = in && k >= tau;
+    // one pass: the maximum (and, for top-p, which falls back to the general path often enough, the finite
+    // minimum) and the list of candidates
+    auto list_candidate = [&](uint32_t k, int i, bool cand) {
       const uint64_t m = __builtin_amdgcn_ballot_w64(cand);
       if (m == 0) return;
       uint32_t base = 0;
@@ -309,7 +312,23 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
         member_key[at] = k;
         member_idx[at] = i;
       }
-    });
+    };
+    if (p.top_k > 1) {
+      sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
+        const uint32_t k = order_key(x);
+        const bool up = in && k > bk;
+        bk = up ? k : bk; bi = up ? i : bi;
+        list_candidate(k, i, in && k >= tau);
+      });
+    } else {  // (half the loads in flight: with the minimum the full count no longer fits the registers)
+      sweep<U / 2>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
+        const uint32_t k = order_key(x);
+        const bool up = in && k > bk;
+        bk = up ? k : bk; bi = up ? i : bi;
+        mn = (in && x > -INFINITY) ? fminf(mn, x) : mn;
+        list_candidate(k, i, in && k >= tau);
+      });
+    }
   } else if (filtering) {
     sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int i, float x, bool in) {
       const uint32_t k = order_key(x);
@@ -354,11 +373,52 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
     int n_candidates = 0;
     if (one_pass) {
       n_candidates = (int)member_count;  // (published by the barrier of the maximum's reduction)
-      if (n_candidates >= p.top_k && n_candidates <= kMemberCap) {
-        cut_key = digit_select(n_candidates, (uint64_t)(p.top_k - 1), 0, false, 0);
+      bool usable = n_candidates <= kMemberCap && (by_count ? n_candidates >= p.top_k : n_candidates > 0);
+      uint64_t target = by_count ? (uint64_t)(p.top_k - 1) : 0;
+      if (usable && !by_count) {
+        // top-p: the row's total mass (one more pass), then the candidates' masses; the cut lies inside the list
+        // when those alone exceed top_p of the total
+        auto workgroup_sum = [&](uint64_t v) -> uint64_t {
+          v = wave_sum_u64(v);
+          __syncthreads();
+          if (lane == 0) wsum[wave] = v;
+          __syncthreads();
+          uint64_t t = 0;
+#pragma unroll
+          for (int w = 0; w < kSampleWaves; ++w) t += wsum[w];
+          return t;
+        };
+        uint64_t c = 0;
+        for (int j = tid; j < n_candidates; j += kSampleThreads) {
+          const uint64_t m = mass_of(order_key_value(member_key[j]), neg_mx);
+          member_mass[j] = m;
+          c += m;
+        }
+        c = workgroup_sum(c);
+        // Worth the pass?  The mass below the threshold is many small terms, so the sample estimates it well
+        // (unlike the mass above it, which a few elements can hold); 10 % on top of the estimate as margin.
+        // (the sampled values are read again rather than kept in registers through the passes above)
+        uint64_t below = 0;
+#pragma unroll
+        for (int j = 0; j < kSamplesPerThread; ++j) {
+          const float x = rd.at(tid * (V / kSampleThreads) + j);
+          below += order_key(x) < tau ? mass_of(x, neg_mx) : 0;
+        }
+        const double rest = (double)workgroup_sum(below) * ((double)V / kMemberCap) * 1.1;
+        usable = (double)c > (double)p.top_p * ((double)c + rest);
+        if (usable) {
+          uint64_t z = 0;
+          sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int, float x, bool in) { z += in ? mass_of(x, neg_mx) : 0; });
+          z = workgroup_sum(z);
+          target = (uint64_t)((double)p.top_p * (double)z);
+          usable = c > target;
+        }
+      }
+      if (usable) {
+        cut_key = digit_select(n_candidates, target, 0, !by_count, 0);
         cut_from_list = true;
-      } else {
-        // the general path needs the finite minimum, which the one-pass sweep did not track
+      } else if (by_count) {
+        // the general path needs the finite minimum, which the one-pass sweep did not track for top-k
         sweep<U>(rd, 0, V, tid, kSampleThreads, [&](int, float x, bool in) {
           mn = (in && x > -INFINITY) ? fminf(mn, x) : mn;
         });

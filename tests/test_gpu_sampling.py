@@ -132,7 +132,10 @@ def test_top_p_cut_meets_the_definition(mi, dev, dtype, V, top_p):
     x[2] *= 0.05           # nearly flat row: the prefix is long
     x[5, V // 3:] = float("-inf")
     u = torch.rand(R, generator=torch.Generator().manual_seed(V))
-    temperature = 0.9
+    _check_top_p(mi, dev, x, top_p, 0.9, u)
+
+
+def _check_top_p(mi, dev, x, top_p, temperature, u):
     s, _, cut = mi.ops.sample_from_logits(x.to(dev), top_p=top_p, temperature=temperature, uniform=u.to(dev),
                                           return_cut=True)
     cut = cut.cpu()
@@ -147,6 +150,25 @@ def test_top_p_cut_meets_the_definition(mi, dev, dtype, V, top_p):
     clear = ((above - top_p).abs() > TOL) & ((down_to - top_p).abs() > TOL)
     assert torch.equal(cut[clear], want_cut[clear])
     _check_draw(xs, cut, u, s.cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("top_p", [0.3, 0.9])
+def test_top_p_one_pass_form_and_its_fallbacks(mi, dev, dtype, top_p):
+    """Top-p on rows of 32 768: peaked rows find their cut among the listed candidates, the others (flat, nearly
+    flat, a few finite values, half the row tied at the top) go through the general path; both must meet the
+    definition."""
+    V = 32768
+    x = _logits(10, V, 1200 + int(10 * top_p), dtype, spread=5.0)   # rows 7-9: peaked random rows
+    x[0, :] = -0.75
+    x[1, :] = float("-inf"); x[1, [5, 17000, 32767]] = torch.tensor([0.5, 1.5, 1.0], dtype=dtype)
+    x[2, :] = 0.25; x[2, 12345] = 9.0
+    x[3, : V // 2] = 3.0
+    x[4, ::2] = float("-inf")
+    x[5] = (torch.arange(V).float() / V * 30).to(dtype)
+    x[6] *= 0.02
+    u = torch.rand(10, generator=torch.Generator().manual_seed(int(100 * top_p)))
+    _check_top_p(mi, dev, x, top_p, 1.0, u)
 
 
 def test_no_filter_draws_from_the_full_softmax(mi, dev):
