@@ -220,15 +220,16 @@ static __device__ void find_crossing(const uint64_t* hist, uint64_t above, uint6
 
 constexpr int kMemberCap = 4096;  // members of the chosen value bin that fit the LDS list
 // Top-k with a small k (the usual 20-100) needs none of the row-wide histogram passes: a threshold is estimated
-// from kMemberCap values spread over the row so that about kCandidateTarget elements lie at or above it, ONE pass
+// from kMemberCap values spread over the row so that a thousand or a few thousand elements lie at or above it, ONE pass
 // finds the maximum and lists those candidates, and the exact k-th largest value and the draw are then worked out
 // on the list.  Top-p does the same with one more pass for the row's total mass; its cut lies inside the list
 // whenever the candidates alone hold more than top_p of that mass (peaked rows: the usual case).  When the estimate
 // misses (fewer than k candidates, more than the list holds -- flat rows --, too little mass), the general path
 // below runs instead; the result is the same either way.
-constexpr int kFastTopK = 256;          // largest k the one-pass form is tried for
+constexpr int kFastTopK = 768;          // largest k the one-pass form is tried for
 constexpr int kFastMinVocab = 16384;    // smallest row it is tried for
-constexpr int kCandidateTarget = 1024;  // expected candidates (standard deviation ~ target / sqrt(sample rank))
+// expected candidates: 1 024, or 4 k up to 3 072 (standard deviation ~ target / sqrt(sample rank), i.e. ~10-18 %)
+static __device__ __forceinline__ int candidate_target(int top_k) { return max(1024, min(4 * top_k, 3072)); }
 
 template <int DT, int VEC>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) {
@@ -288,12 +289,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   constexpr int kSamplesPerThread = kMemberCap / kSampleThreads;
   uint32_t tau = 0;
   if (one_pass) {
-    // threshold: the rank-th largest of kMemberCap sampled values, rank chosen for ~kCandidateTarget candidates
+    // threshold: the rank-th largest of kMemberCap sampled values, rank chosen for ~candidate_target(k) candidates
     const int blk = V / kSampleThreads;  // >= 16: thread t samples elements t * blk .. + 3
 #pragma unroll
     for (int j = 0; j < kSamplesPerThread; ++j)
       member_key[tid * kSamplesPerThread + j] = order_key(rd.at(tid * blk + j));
-    const int rank = (int)(((int64_t)kCandidateTarget * kMemberCap + V - 1) / V);
+    const int rank = min(kMemberCap / 2, (int)(((int64_t)candidate_target(p.top_k) * kMemberCap + V - 1) / V));
     // (the upper 16 bits of the key are enough: sign, exponent and 7 bits of the fraction)
     tau = digit_select(kMemberCap, (uint64_t)(rank - 1), 0, false, 2);
     if (tid == 0) member_count = 0;

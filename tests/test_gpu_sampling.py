@@ -203,12 +203,12 @@ def test_draw_frequencies_follow_the_kept_probabilities(mi, dev, mode):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("k", [2, 10, 200, 256, 257])
+@pytest.mark.parametrize("k", [2, 10, 200, 256, 257, 768, 769])
 def test_top_k_one_pass_form_and_its_fallbacks(mi, dev, dtype, k):
     """Rows of 32 768 and a small k take the form that lists candidates above a sampled threshold in one pass; rows
     where the estimate cannot work -- flat (every value a candidate), a few finite values (fewer candidates than k),
     a spike in an otherwise flat row, half the row tied at the maximum -- must come out the same through the general
-    path.  k = 257 never takes the one-pass form."""
+    path.  k = 769 never takes the one-pass form."""
     V = 32768
     x = _logits(10, V, 900 + k, dtype)
     x[0, :] = -0.75                                             # flat: every entry equals the cut
