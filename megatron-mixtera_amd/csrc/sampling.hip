@@ -397,7 +397,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
         }
         c = workgroup_sum(c);
         // Worth the pass?  The mass below the threshold is many small terms, so the sample estimates it well
-        // (unlike the mass above it, which a few elements can hold); 10 % on top of the estimate as margin.
+        // (unlike the mass above it, which a few elements can hold); a quarter on top of the estimate as margin, so
+        // that rows on the edge do not pay for the total-mass pass and then fail.
         // (the sampled values are read again rather than kept in registers through the passes above)
         uint64_t below = 0;
 #pragma unroll
@@ -405,7 +406,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
           const float x = rd.at(tid * (V / kSampleThreads) + j);
           below += order_key(x) < tau ? mass_of(x, neg_mx) : 0;
         }
-        const double rest = (double)workgroup_sum(below) * ((double)V / kMemberCap) * 1.1;
+        const double rest = (double)workgroup_sum(below) * ((double)V / kMemberCap) * 1.25;
         usable = (double)c > (double)p.top_p * ((double)c + rest);
         if (usable) {
           uint64_t z = 0;
