@@ -173,17 +173,32 @@ def test_stale_cache_rows_beyond_the_length_do_not_leak(mi, dev):
     assert torch.equal(out, ref)
 
 
-def test_chunked_prefill_is_consistent_at_full_size(mi, dev):
-    """Size-independent property on the cfg3-sized prompts (8 x 2048 tokens over U[0,4096] cached):
+@pytest.mark.parametrize("d", [128, 96, 192, 256])
+def test_chunked_prefill_is_consistent_at_full_size(mi, dev, d):
+    """Size-independent property on the cfg3-sized prompts (8 x 2048 tokens over U[0,4096] cached), at head_dim 128
+    and at the widths whose tile kernel has a shape of its own (96: 208-byte rows; 192 / 256: 16 rows per wavefront,
+    32-key tiles at 256):
     the rows of the second half of every prompt, computed with the first half already counted as
     cached context, equal the same rows of the single full call bit for bit (same tiles, same order),
-    and the block table can be permuted without changing a bit."""
+    and the block table can be permuted without changing a bit.  The last 48 rows of the first and the last
+    prompt are also checked against the fp32 checker."""
     q, kc, vc, cu_q, lens, bt = mi.synthetic.make_prefill_case(
         dev, n_prefill=8, new_tokens=2048, ctx_lo=0, ctx_hi=4096, n_decode=0, dec_lo=1, dec_hi=2,
-        Hq=32, Hkv=8, d=128, chunk=256, seed=1003, on_device_rng=True)
+        Hq=32, Hkv=8, d=d, chunk=256, seed=1003 + d, on_device_rng=True)
     full = mi.ops.paged_prefill_attention(q, kc, vc, cu_q, lens, bt, max_kv_len=int(lens.max()))
     torch.cuda.synchronize()
     assert torch.isfinite(full).all()
+    for r in (0, 7):
+        # the request's chunks alone, compacted, so that only a few megabytes travel to the host
+        L = int(lens[r])
+        nch = (L + 255) // 256
+        ids = bt[r, :nch].long()
+        end = int(cu_q[r + 1])
+        ref = oa.paged_varlen_attention(q[end - 48:end].cpu(), kc[ids].cpu(), vc[ids].cpu(),
+                                        torch.tensor([0, 48], dtype=torch.int32), torch.tensor([L], dtype=torch.int32),
+                                        torch.arange(nch, dtype=torch.int32)[None])
+        err = (full[end - 48:end].float().cpu() - ref).abs()
+        assert (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"request {r}: max err {err.max().item():.3e}"
     # second halves only: 1024 new tokens per request, same kv lengths
     rows = torch.cat([torch.arange(int(cu_q[r]) + 1024, int(cu_q[r + 1]), device=dev) for r in range(8)])
     cu_half = torch.arange(0, 8 * 1024 + 1, 1024, dtype=torch.int32, device=dev)
