@@ -886,10 +886,26 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
       const int T = start + t * kMlaTile;
       // ---- S^T = K Q^T: this wavefront's share, then the whole tile through LDS -----------
       {
+        // Key fragments in batches of KB, the reads of batch b+1 issued before the products of batch b (scheduling
+        // barriers keep that order): read-wait-multiply one fragment at a time pays the LDS latency KSW times.
+        constexpr int KB = KSW % 6 == 0 ? 6 : 3, NB = KSW / KB;
+        static_assert(KSW % KB == 0, "18 or 9 fragments");
         const uint8_t* ks = buf + kfrag_off + 16 * su * kMlaPitch + 64 * k0;
         f32x4_t sacc = {0.f, 0.f, 0.f, 0.f};
+        uint4 kf[2][KB];
 #pragma unroll
-        for (int kk = 0; kk < KSW; ++kk) sacc = mfma_16x16x32<F16>(lds_ld16(ks + 64 * kk), qf[kk], sacc);
+        for (int j = 0; j < KB; ++j) kf[0][j] = *reinterpret_cast<const uint4*>(ks + 64 * j);
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          if (b + 1 < NB) {
+#pragma unroll
+            for (int j = 0; j < KB; ++j) kf[(b + 1) & 1][j] = *reinterpret_cast<const uint4*>(ks + 64 * (KB * (b + 1) + j));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int j = 0; j < KB; ++j) sacc = mfma_16x16x32<F16>(kf[b & 1][j], qf[KB * b + j], sacc);
+          __builtin_amdgcn_sched_barrier(0);
+        }
         sbuf[((k0 ? 1 : 0) * 4 + su) * 64 + lane] = make_float4(sacc[0], sacc[1], sacc[2], sacc[3]);
       }
       __syncthreads();
