@@ -505,6 +505,95 @@ def test_random_decode_steps_match_the_checker(mi, dev, block):
             raise AssertionError(f"{_last_case[0]}: {e}") from None
 
 
+def case_sampling(mi, dev, rng, seed):
+    """Sampling over rows of random shapes -- Gaussian, peaked like a language model's, flat, heavy ties, a few finite
+    values, pre-masked halves -- through greedy, top-k (small k: the one-pass form and its fallbacks; large k), top-p
+    and plain temperature sampling, in fp32 or bf16, aligned or not."""
+    from oracle import sampling as osm
+    gen = torch.Generator().manual_seed(seed)
+    V = rng.choice([50, 1000, 4097, 16384, 20000, 32768, 50257, 65536])
+    R = rng.randint(1, 6)
+    dtype = rng.choice([torch.float32, torch.bfloat16])
+    mode = rng.choice(["greedy", "top_k", "top_k", "top_p", "top_p", "none"])
+    temperature = rng.choice([1.0, 0.7, 1.3])
+    x = torch.randn(R, V, generator=gen) * rng.choice([0.05, 1.0, 3.0, 6.0])
+    shapes = []
+    for r in range(R):
+        shape = rng.choice(["gauss", "gauss", "peaked", "flat", "ties", "few", "masked", "sorted"])
+        shapes.append(shape)
+        if shape == "peaked":
+            n = rng.randint(1, 40)
+            x[r, torch.randperm(V, generator=gen)[:n]] += torch.rand(n, generator=gen) * 6 + 8
+        elif shape == "flat":
+            x[r] = rng.uniform(-3, 3)
+        elif shape == "ties":
+            x[r] = torch.randint(0, rng.choice([2, 5, 40]), (V,), generator=gen).float() * 0.5
+        elif shape == "few":
+            keep = torch.randperm(V, generator=gen)[:rng.randint(1, 5)]
+            vals = x[r, keep].clone()
+            x[r] = float("-inf")
+            x[r, keep] = vals
+        elif shape == "masked":
+            x[r, torch.randperm(V, generator=gen)[: V // 2]] = float("-inf")
+        elif shape == "sorted":
+            x[r] = torch.sort(x[r], descending=rng.random() < 0.5).values
+    x = x.to(dtype)
+    if rng.random() < 0.3 and V > 100:   # a row stride that breaks the 16-byte alignment of the rows
+        wide = torch.zeros(R, V + 3, dtype=dtype)
+        wide[:, :V] = x
+        xd = wide.to(dev)[:, :V]
+    else:
+        xd = x.to(dev)
+    u = torch.rand(R, generator=gen)
+    k = rng.choice([2, 5, 50, 200, 256, 300, 768, 1000, 5000])
+    k = max(2, min(k, V))
+    top_p = rng.choice([0.05, 0.3, 0.5, 0.9, 0.99])
+    _note(f"sampling seed={seed} V={V} R={R} dtype={dtype} mode={mode} T={temperature} k={k} top_p={top_p} rows={shapes} "
+          f"aligned={xd.is_contiguous()}")
+    poison(dev)
+    xs = osm.scaled_logits(x, temperature)
+    if mode == "greedy":
+        s, _ = mi.ops.sample_from_logits(xd, top_k=1)
+        assert torch.equal(s.cpu(), osm.sample_from_logits(x, top_k=1))
+        return
+    kwargs = {"top_k": dict(top_k=k), "top_p": dict(top_p=top_p), "none": {}}[mode]
+    s, _, cut = mi.ops.sample_from_logits(xd, temperature=temperature, uniform=u.to(dev), return_cut=True, **kwargs)
+    torch.cuda.synchronize()
+    s, cut = s.cpu(), cut.cpu()
+    assert ((s >= 0) & (s < V)).all()
+    if mode == "top_k":
+        kth = torch.topk(xs, k, dim=-1).values[:, -1]
+        assert torch.equal(cut, kth), f"top-k cut {cut.tolist()} != {kth.tolist()}"
+    elif mode == "top_p":
+        pr = xs.double().softmax(-1)
+        above = (pr * (xs > cut[:, None])).sum(-1)
+        down_to = (pr * (xs >= cut[:, None])).sum(-1)
+        assert (above <= top_p + 2e-6).all() and (down_to > top_p - 2e-6).all(), "top-p cut violates the definition"
+    else:
+        assert torch.isinf(cut).all() and (cut < 0).all()
+    # the drawn index lies in the kept set, and its CDF bracket holds u within the margin
+    keep = xs >= cut[:, None]
+    pr = osm.kept_probabilities(xs, keep)
+    cdf = pr.cumsum(-1)
+    idx = torch.arange(R)
+    assert keep[idx, s].all(), "a filtered entry was drawn"
+    hi = cdf[idx, s]
+    lo = hi - pr[idx, s]
+    assert ((lo - 2e-6 <= u.double()) & (u.double() <= hi + 2e-6)).all(), "draw outside its CDF bracket"
+    s2, _ = mi.ops.sample_from_logits(xd, temperature=temperature, uniform=u.to(dev), **kwargs)
+    assert torch.equal(s2.cpu(), s), "a repeated call drew other tokens"
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_random_sampling_cases_match_the_checker(mi, dev, block):
+    for seed in range(110_000 + 60 * block, 110_000 + 60 * (block + 1)):
+        rng = random.Random(seed)
+        try:
+            case_sampling(mi, dev, rng, seed)
+        except AssertionError as e:
+            raise AssertionError(f"{_last_case[0]}: {e}") from None
+
+
 WRITE_KINDS = {"append": case_append, "append_fp8": case_append_fp8, "norm_rope": case_norm_rope}
 
 
