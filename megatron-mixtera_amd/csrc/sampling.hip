@@ -263,10 +263,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
   // side of more members).
   auto digit_select = [&](int n, uint64_t target, uint64_t above, bool by_mass, int last_digit) -> uint32_t {
     uint32_t pmask = 0, pval = 0;
+    __syncthreads();
+    if (tid < 256) hist[tid] = 0;
+    __syncthreads();
     for (int d = 3; d >= last_digit; --d) {
-      __syncthreads();
-      if (tid < 256) hist[tid] = 0;
-      __syncthreads();
       for (int j0 = 0; j0 < n; j0 += kSampleThreads) {
         const int j = j0 + tid;
         const bool in = j < n;
@@ -275,7 +275,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
                  [&] { return by_mass ? member_mass[j] : (uint64_t)1; });
       }
       __syncthreads();
-      if (wave == 0) find_crossing(hist, above, target, res, lane);
+      if (wave == 0) {  // the wavefront that reads the bins also clears them for the next digit: two barriers a pass
+        find_crossing(hist, above, target, res, lane);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) hist[4 * lane + j] = 0;
+      }
       __syncthreads();
       const uint32_t digit = 255u - (uint32_t)res[0];  // the crossing lies inside the list, so a digit is always found
       above = res[1];
@@ -541,19 +545,21 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(SampleParams p) 
       __syncthreads();
       const int n_kept = (int)member_count;
       if (n_kept <= kSampleThreads) {
-        const uint64_t mine = tid < n_kept ? member_mass[tid] : 0;
-        const uint32_t my_idx = (uint32_t)(mine >> 32);
-        uint64_t total = 0, upto = 0;  // all kept mass; kept mass at vocabulary indices <= mine
-        for (int m = 0; m < n_kept; ++m) {
-          const uint64_t e = member_mass[m];  // the same word for every lane: a broadcast read
-          const uint64_t w = e & 0xffffffffu;
-          total += w;
-          upto += (uint32_t)(e >> 32) <= my_idx ? w : 0;
+        if (wave * 64 < n_kept) {  // only the wavefronts that own a kept element walk the list
+          const uint64_t mine = tid < n_kept ? member_mass[tid] : 0;
+          const uint32_t my_idx = (uint32_t)(mine >> 32);
+          uint64_t total = 0, upto = 0;  // all kept mass; kept mass at vocabulary indices <= mine
+          for (int m = 0; m < n_kept; ++m) {
+            const uint64_t e = member_mass[m];  // the same word for every lane: a broadcast read
+            const uint64_t w = e & 0xffffffffu;
+            total += w;
+            upto += (uint32_t)(e >> 32) <= my_idx ? w : 0;
+          }
+          uint64_t want = (uint64_t)((double)p.uniform[r] * (double)total);
+          want = want < total ? want : total - 1;
+          const uint64_t w_mine = mine & 0xffffffffu;
+          if (tid < n_kept && upto > want && upto - w_mine <= want) pick[0] = (int)my_idx;
         }
-        uint64_t want = (uint64_t)((double)p.uniform[r] * (double)total);
-        want = want < total ? want : total - 1;
-        const uint64_t w_mine = mine & 0xffffffffu;
-        if (tid < n_kept && upto > want && upto - w_mine <= want) pick[0] = (int)my_idx;
         drawn = true;
       }
     }
