@@ -51,21 +51,28 @@ static __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
   const uint32_t lo = __shfl_xor((uint32_t)v, m, 64), hi = __shfl_xor((uint32_t)(v >> 32), m, 64);
   return ((uint64_t)hi << 32) | lo;
 }
-static __device__ __forceinline__ uint64_t shfl_up_u64(uint64_t v, int d) {
-  const uint32_t lo = __shfl_up((uint32_t)v, d, 64), hi = __shfl_up((uint32_t)(v >> 32), d, 64);
-  return ((uint64_t)hi << 32) | lo;
-}
 static __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
 #pragma unroll
   for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_u64(v, m);
   return v;
 }
-static __device__ __forceinline__ uint64_t wave_scan_incl_u64(uint64_t v, int lane) {
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const uint64_t o = shfl_up_u64(v, d);
-    if (lane >= d) v += o;
-  }
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (shifts by 1, 2, 4, 8 inside a row of 16
+// lanes, then the last lane of row 0 / 2 broadcast into row 1 / 3 and lane 31 into the upper half): six steps of two
+// moves and one 64-bit add, where the shuffle form costs twelve dependent trips through the LDS crossbar.  Lanes
+// without a source receive zero.
+template <int CTRL, int ROW_MASK>
+static __device__ __forceinline__ uint64_t dpp_u64(uint64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, CTRL, ROW_MASK, 0xF, false);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), CTRL, ROW_MASK, 0xF, false);
+  return ((uint64_t)hi << 32) | lo;
+}
+static __device__ __forceinline__ uint64_t wave_scan_incl_u64(uint64_t v, int /*lane*/) {
+  v += dpp_u64<0x111, 0xF>(v);  // row_shr:1
+  v += dpp_u64<0x112, 0xF>(v);  // row_shr:2
+  v += dpp_u64<0x114, 0xF>(v);  // row_shr:4
+  v += dpp_u64<0x118, 0xF>(v);  // row_shr:8
+  v += dpp_u64<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
+  v += dpp_u64<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
   return v;
 }
 
