@@ -47,15 +47,6 @@ static __device__ __forceinline__ float order_key_value(uint32_t k) {
   return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-static __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
-  const uint32_t lo = __shfl_xor((uint32_t)v, m, 64), hi = __shfl_xor((uint32_t)(v >> 32), m, 64);
-  return ((uint64_t)hi << 32) | lo;
-}
-static __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
-#pragma unroll
-  for (int m = 32; m >= 1; m >>= 1) v += shfl_xor_u64(v, m);
-  return v;
-}
 // Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves (shifts by 1, 2, 4, 8 inside a row of 16
 // lanes, then the last lane of row 0 / 2 broadcast into row 1 / 3 and lane 31 into the upper half): six steps of two
 // moves and one 64-bit add, where the shuffle form costs twelve dependent trips through the LDS crossbar.  Lanes
@@ -74,6 +65,13 @@ static __device__ __forceinline__ uint64_t wave_scan_incl_u64(uint64_t v, int /*
   v += dpp_u64<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3
   v += dpp_u64<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
   return v;
+}
+// Sum over the 64 lanes, in every lane: the scan above, then its last lane's value.
+static __device__ __forceinline__ uint64_t wave_sum_u64(uint64_t v) {
+  v = wave_scan_incl_u64(v, 0);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 63);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 63);
+  return ((uint64_t)hi << 32) | lo;
 }
 
 // One row of logits.  DT = element type (0 fp32, 1 bf16, 2 fp16); VEC = elements per 16-byte load (4 fp32,
