@@ -56,7 +56,8 @@ int mi_resolve_tuning(const MiTuning* given, MiTuning* out, const char* who) {
   if (t.norm_rope_vectorised != 1 && t.norm_rope_vectorised != 2 && t.norm_rope_vectorised != -1)
     return bad("norm_rope_vectorised must be 0 (default), 1 or -1 (never)");
   if (t.mla_decode_lds == 0) t.mla_decode_lds = 1;
-  if (t.mla_decode_lds != 1 && t.mla_decode_lds != -1) return bad("mla_decode_lds must be 0 (default) or -1 (streaming kernel)");
+  if (t.mla_decode_lds != 1 && t.mla_decode_lds != -1 && t.mla_decode_lds != 2)
+    return bad("mla_decode_lds must be 0 (default), -1 (streaming kernel) or 2 (eight-wavefront LDS kernel at every head count)");
   *out = t;
   return MI_OK;
 }

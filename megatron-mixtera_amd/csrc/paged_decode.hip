@@ -40,6 +40,7 @@
 #include "mi_common.h"
 
 #include <atomic>
+#include <type_traits>
 #include "mi_capi_internal.h"
 
 namespace mi {
@@ -992,6 +993,341 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
   });
 }
 
+// ---------------------------------------------------------------------------------------------
+// Multi-latent attention decode, 128 query heads per workgroup.
+//
+// With 128 heads the latent rows carry 242 flop per byte: the matrix cores, not memory, are the bound,
+// and what feeds them is LDS.  A wavefront takes in no more than ~18 B/clk of fragments whatever runs
+// beside it, so what counts is how many products each fragment read serves.  Here a workgroup is four
+// wavefronts, one per SIMD with the SIMD's whole register file (512 registers per lane); wavefront w
+// owns query heads 32 w .. 32 w + 31 (two 16-row tiles: every key fragment and every transposed value
+// fragment feeds two products) and all 512 output columns (256 accumulator registers), and shares
+// nothing with the others but the staged rows: no score exchange, one barrier per tile.
+// 32-token tiles (37 KB) in three LDS buffers: in iteration t the score product reads tile t, then
+// tile t+1 goes from registers to LDS, the barrier, the loads of tile t+2 are issued, softmax, value
+// product of tile t -- and the first key fragments of tile t+1 are requested under its last products.
+// (Three buffers: a wavefront past the barrier of iteration t+1 stores tile t+2 while a slower one
+// may still read values of tile t.)  The accumulators are rescaled only when a running maximum
+// moves by more than a factor 256: they live in accumulation registers, out of the vector ALU's
+// reach, and a rescale is ~770 instructions; until then probabilities are taken against the older
+// maximum (at most 256, exact in fp32 sums and within the 16-bit types' range).
+// ---------------------------------------------------------------------------------------------
+constexpr int kMlaHeadsTile = 32;  // tokens per staged tile of the 128-head kernel
+// A tile arrives in LDS by direct loads: each instruction puts its 64 lanes' 16-byte pieces side by side (1 KB), so a
+// tile is 37 instructions over a line of 32 x 73 pieces (72 of a row + the 16 bytes of row padding, which receive a
+// copy of the row's last piece), and a buffer is 37 KB.
+constexpr int kMlaHeadsLoads = (kMlaHeadsTile * (kMlaPitch / 16) + 63) / 64;
+constexpr int kMlaHeadsBuf = kMlaHeadsLoads * 1024;
+constexpr bool mla_piece_division_ok() {
+  for (unsigned u = 0; u < 64u * kMlaHeadsLoads; ++u)
+    if (((u * 14365u) >> 20) != u / 73u) return false;
+  return true;
+}
+static_assert(kMlaPitch == 73 * 16 && mla_piece_division_ok(), "piece -> (row, column) by multiplication");
+
+template <bool F16>
+__global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodeParams p) {
+  constexpr int HDV = 512, KS = 576 / 32, NE = HDV / 16, TK = kMlaHeadsTile;
+  constexpr int KB = 3, NKG = 2 * KS / KB;   // key fragments per group; groups per tile (two 16-token sub-tiles)
+  constexpr int VB = 2, NVG = NE / VB;       // 16-column output blocks per group; groups per tile
+  // log2 of the factor a row's maximum may grow before the reference of its exponentials follows: probabilities
+  // up to that factor must fit the 16-bit type (fp16: 65 504)
+  constexpr float kLazy = F16 ? 8.f : 30.f;
+  extern __shared__ int cum[];
+  uint8_t* const tiles = reinterpret_cast<uint8_t*>(cum) + (((size_t)p.R * 8 + 15) & ~(size_t)15);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int m16 = lane & 15, g = lane >> 4;
+  const int hq0 = (blockIdx.y * 4 + wave) * 32 + m16;  // this lane's query head in the first row tile (+16: second)
+  const int64_t chunk_bytes = p.kv_sc * 2;
+  const uint32_t tok_bytes = (uint32_t)(p.kv_st * 2);
+  // the LDS byte address of the tile buffers, for the direct loads
+  const uint32_t tiles_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)tiles;
+  const int kfrag_off = m16 * kMlaPitch + 16 * g;
+  const int vfrag_off = (4 * g + (m16 >> 2)) * kMlaPitch + 8 * (m16 & 3);
+  const uint4 ones = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
+#define MI_SB() __builtin_amdgcn_sched_barrier(0)
+
+  walk_segments<TK>(p, [&](int r, int row, int len, int start, int end, bool whole, bool /*final_seg*/, int slot) {
+    r = __builtin_amdgcn_readfirstlane(r);
+    row = __builtin_amdgcn_readfirstlane(row);
+    len = __builtin_amdgcn_readfirstlane(len);
+    start = __builtin_amdgcn_readfirstlane(start);
+    end = __builtin_amdgcn_readfirstlane(end);
+    slot = __builtin_amdgcn_readfirstlane(slot);
+    const int last = min(end, len) - 1;
+    const int ntile = (end - start + TK - 1) / TK;
+    const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
+
+    uint4 qf[2][KS];
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const uint16_t* qrow = p.q + (int64_t)row * p.q_st + (int64_t)(hq0 + 16 * h2) * p.q_sh + 8 * g;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) qf[h2][kk] = ld16(qrow + 32 * kk);
+    }
+    // A tile lies in one chunk (the launcher requires a chunk size that is a multiple of 32); rows past
+    // the segment's last token re-read that token's row (their probabilities are forced to zero).
+    // Tile t goes straight from memory into buffer t % 3: wavefront w issues loads w, w + 4, ... of the tile's 37;
+    // lane l of load k fills piece 64 k + l of the buffer's line.  The loads count on the vector-memory counter.
+    auto tile_buf = [&](int t) { return (unsigned)t % 3u * (unsigned)kMlaHeadsBuf; };
+    auto fetch = [&](int t) {
+      const int T = start + t * TK;
+      const int ci = chunk_of(T, p.chunk_magic);
+      const int pc = __builtin_amdgcn_readfirstlane(bt_row[ci]);
+      const uint8_t* src = p.kc + (int64_t)pc * chunk_bytes + (int64_t)(uint32_t)(T - ci * p.chunk) * tok_bytes;
+      const uint32_t row_lim = (uint32_t)min(last - T, TK - 1);
+      const uint32_t dst = tiles_lds + tile_buf(t);
+      uint32_t ln = (uint32_t)lane;
+      asm volatile("" : "+v"(ln));  // opaque: the ten piece addresses are worked out here, not kept in registers across tiles
+#pragma unroll
+      for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
+        const int k = wave + 4 * i;
+        if (k < kMlaHeadsLoads) {  // wave-uniform
+          const uint32_t u = 64u * (uint32_t)k + ln;
+          const uint32_t prow = (u * 14365u) >> 20, pcol = u - 73u * prow;
+          const uint8_t* g_src = src + min(prow, row_lim) * tok_bytes + 16u * min(pcol, 71u);
+          const uint32_t m0 = __builtin_amdgcn_readfirstlane(dst + 1024u * (uint32_t)k);
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(g_src) : "memory");
+          MI_SB();  // one address at a time: the registers are needed elsewhere
+        }
+      }
+    };
+    auto fetch_wait = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    // key group i of a tile: fragments KB (i % (KS / KB)) .. + KB - 1 of 16-token sub-tile i / (KS / KB)
+    auto load_k = [&](const uint8_t* buf, int i, uint4 (&kf)[KB]) {
+      const uint8_t* ks = buf + kfrag_off + 16 * (i / (KS / KB)) * kMlaPitch + 64 * KB * (i % (KS / KB));
+#pragma unroll
+      for (int j = 0; j < KB; ++j) kf[j] = *reinterpret_cast<const uint4*>(ks + 64 * j);
+    };
+    // value group j: output columns 16 VB j .. + 16 VB - 1, all 32 tokens, transposed
+    auto load_v = [&](const uint8_t* buf, int j, uint2 (&vf)[VB][2]) {
+      const uint8_t* vs = buf + vfrag_off + 32 * VB * j;
+#pragma unroll
+      for (int e = 0; e < VB; ++e) {
+        vf[e][0] = lds_ld8_tr(vs + 32 * e);
+        vf[e][1] = lds_ld8_tr(vs + 16 * kMlaPitch + 32 * e);
+      }
+    };
+
+    __syncthreads();  // every wavefront is done with the previous segment's buffers
+    fetch(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), in the compiler's sight
+    // (the query fragments count as used here: the compiler then waits for their loads now and not in the tile loop,
+    // where a wait on the vector-memory counter waits for the direct loads in flight as well)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk)
+        asm volatile("" ::"v"(qf[h2][kk].x), "v"(qf[h2][kk].y), "v"(qf[h2][kk].z), "v"(qf[h2][kk].w));
+    if (ntile > 1) fetch(1);
+    __syncthreads();
+
+    // The accumulators live in accumulation registers, out of the vector ALU's reach, and any other definition of
+    // theirs than a matrix product or a zero makes the compiler keep all 256 in vector registers (and the query
+    // fragments in scratch memory).  So the tile loop never rescales them: exponentials are taken against the row
+    // maxima of the first tile, and when a later maximum leaves the window above those (kLazy: hardly ever) the
+    // wavefront moves its sums into this segment's rows of the partial-output buffer -- no other workgroup touches
+    // those -- and finishes the segment in a second, slow loop that follows every maximum and keeps them there.
+    float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.f, 0.f};
+    const float mul = p.scale_log2;
+    // scores of tile t (key fragments of its first group already requested into kf[0]); requests the first value
+    // fragments; masks the tokens past the segment's end; row maxima in the exponent's unit
+    auto scores = [&](int t, const uint8_t* buf, uint4 (&kf)[2][KB], uint2 (&vf0)[VB][2], f32x4_t (&sc)[2][2], float (&tmax)[2]) {
+#pragma unroll
+      for (int i = 0; i < NKG; ++i) {
+        if (i + 1 < NKG) load_k(buf, i + 1, kf[(i + 1) & 1]);
+        else load_v(buf, 0, vf0);
+        MI_SB();
+        const int u = i / (KS / KB), k0 = KB * (i % (KS / KB));
+#pragma unroll
+        for (int j = 0; j < KB; ++j) {
+#pragma unroll
+          for (int h2 = 0; h2 < 2; ++h2)
+            sc[h2][u] = mfma_16x16x32<F16>(kf[i & 1][j], qf[h2][k0 + j], (k0 + j) ? sc[h2][u] : f32x4_t{0.f, 0.f, 0.f, 0.f});
+        }
+        MI_SB();
+      }
+      const int T = start + t * TK;
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        if (T + TK > end) {  // only the last tile of a segment has masked tokens
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            const int tok0 = T + 16 * u + 4 * g;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (tok0 + i >= end) sc[h2][u][i] = -INFINITY;
+          }
+        }
+        const float mx = fmaxf(fmaxf(fmaxf(sc[h2][0][0], sc[h2][0][1]), fmaxf(sc[h2][0][2], sc[h2][0][3])),
+                               fmaxf(fmaxf(sc[h2][1][0], sc[h2][1][1]), fmaxf(sc[h2][1][2], sc[h2][1][3])));
+        tmax[h2] = rowgroup_max(mx) * mul;
+      }
+    };
+    // probabilities of a tile against m_run, as the B operand of the value product
+    auto probabilities = [&](const f32x4_t (&sc)[2][2], uint4 (&pp)[2]) {
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const float neg = -m_run[h2];
+        uint32_t w[4];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const float p0 = fast_exp2(__builtin_fmaf(sc[h2][u][0], mul, neg));
+          const float p1 = fast_exp2(__builtin_fmaf(sc[h2][u][1], mul, neg));
+          const float p2 = fast_exp2(__builtin_fmaf(sc[h2][u][2], mul, neg));
+          const float p3 = fast_exp2(__builtin_fmaf(sc[h2][u][3], mul, neg));
+          w[2 * u] = pack2<F16>(p0, p1);
+          w[2 * u + 1] = pack2<F16>(p2, p3);
+        }
+        pp[h2] = make_uint4(w[0], w[1], w[2], w[3]);
+        MI_SB();
+      }
+    };
+
+    int t = 0;
+    {
+      f32x4_t acc[2][NE];
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+        for (int e = 0; e < NE; ++e) acc[h2][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      uint4 kf[2][KB];
+      uint2 vf[2][VB][2];
+      load_k(tiles + tile_buf(0), 0, kf[0]);
+      for (; t < ntile; ++t) {
+        const uint8_t* buf = tiles + tile_buf(t);
+        f32x4_t sc[2][2];
+        float tmax[2];
+        scores(t, buf, kf, vf[0], sc, tmax);
+        if (t == 0) {
+          m_run[0] = tmax[0];
+          m_run[1] = tmax[1];
+        }
+        if (__builtin_amdgcn_ballot_w64(tmax[0] > m_run[0] + kLazy || tmax[1] > m_run[1] + kLazy)) break;
+        // ---- tile t+1 has landed (every wavefront waits for its own loads, then the barrier); tile t+2 sets
+        // out into the buffer of tile t-1, which nobody reads any more ----------------------------------
+        fetch_wait();
+        __syncthreads();
+        if (t + 2 < ntile) fetch(t + 2);
+        uint4 pp[2];
+        probabilities(sc, pp);
+        // ---- O^T += V^T P^T: one 32-token product per 16 columns and row tile; row sums from ones ----
+        const uint8_t* nbuf = tiles + tile_buf(t + 1);
+#pragma unroll
+        for (int j = 0; j < NVG; ++j) {
+          if (j + 1 < NVG) load_v(buf, j + 1, vf[(j + 1) & 1]);
+          else if (t + 1 < ntile) load_k(nbuf, 0, kf[0]);
+          MI_SB();
+#pragma unroll
+          for (int e = 0; e < VB; ++e) {
+            const uint4 a = make_uint4(vf[j & 1][e][0].x, vf[j & 1][e][0].y, vf[j & 1][e][1].x, vf[j & 1][e][1].y);
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) acc[h2][VB * j + e] = mfma_16x16x32<F16>(a, pp[h2], acc[h2][VB * j + e]);
+          }
+          if (j == 0) {
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2)
+              l_run[h2] += mfma_16x16x32<F16>(ones, pp[h2], f32x4_t{0.f, 0.f, 0.f, 0.f})[0];
+          }
+          MI_SB();
+        }
+      }
+      // ---- the sums leave the registers: acc[h2][e][i] is output column 16 e + 4 g + i of head hq0 + 16 h2.
+      // The segment's result when every tile is done; otherwise as they are, for the loop below ---------
+      const bool done = t >= ntile;
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const float inv = done ? 1.f / l_run[h2] : 1.f;
+        const int hq = hq0 + 16 * h2;
+        const int64_t prow = (int64_t)slot * p.Hq + hq;
+        if (done && whole) {
+          uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + 4 * g;
+#pragma unroll
+          for (int e = 0; e < NE; ++e)
+            st8(o + 16 * e, make_uint2(pack2<F16>(acc[h2][e][0] * inv, acc[h2][e][1] * inv),
+                                       pack2<F16>(acc[h2][e][2] * inv, acc[h2][e][3] * inv)));
+        } else {
+          float* o = p.part_o + prow * HDV + 4 * g;
+#pragma unroll
+          for (int e = 0; e < NE; ++e)
+            *reinterpret_cast<float4*>(o + 16 * e) =
+                make_float4(acc[h2][e][0] * inv, acc[h2][e][1] * inv, acc[h2][e][2] * inv, acc[h2][e][3] * inv);
+          if (done && g == 0) p.part_lse[prow] = m_run[h2] + fast_log2(l_run[h2]);
+        }
+      }
+    }
+    if (t < ntile) {
+      // ---- the slow loop: sums in memory, every lane reading back only what it wrote itself (the fences make
+      // its own earlier stores what its loads see) ---------------------------------------------------------
+      float* const po0 = p.part_o + ((int64_t)slot * p.Hq + hq0) * HDV + 4 * g;
+      float* const po1 = po0 + (int64_t)16 * HDV;
+      for (; t < ntile; ++t) {
+        const uint8_t* buf = tiles + tile_buf(t);
+        uint4 kf[2][KB];
+        uint2 vf[2][VB][2];
+        f32x4_t sc[2][2];
+        float tmax[2], alpha[2];
+        load_k(buf, 0, kf[0]);
+        scores(t, buf, kf, vf[0], sc, tmax);
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const float m_new = fmaxf(m_run[h2], tmax[h2]);
+          alpha[h2] = fast_exp2(m_run[h2] - m_new);
+          m_run[h2] = m_new;
+        }
+        fetch_wait();
+        __syncthreads();
+        if (t + 2 < ntile) fetch(t + 2);
+        uint4 pp[2];
+        probabilities(sc, pp);
+        __threadfence();
+#pragma unroll
+        for (int j = 0; j < NVG; ++j) {
+          if (j + 1 < NVG) load_v(buf, j + 1, vf[(j + 1) & 1]);
+          MI_SB();
+#pragma unroll
+          for (int e = 0; e < VB; ++e) {
+            const uint4 a = make_uint4(vf[j & 1][e][0].x, vf[j & 1][e][0].y, vf[j & 1][e][1].x, vf[j & 1][e][1].y);
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+              const f32x4_t add = mfma_16x16x32<F16>(a, pp[h2], f32x4_t{0.f, 0.f, 0.f, 0.f});
+              float4* o = reinterpret_cast<float4*>((h2 ? po1 : po0) + 16 * (VB * j + e));
+              float4 v = *o;
+              v.x = __builtin_fmaf(v.x, alpha[h2], add[0]); v.y = __builtin_fmaf(v.y, alpha[h2], add[1]);
+              v.z = __builtin_fmaf(v.z, alpha[h2], add[2]); v.w = __builtin_fmaf(v.w, alpha[h2], add[3]);
+              *o = v;
+            }
+          }
+          MI_SB();
+        }
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2)
+          l_run[h2] = l_run[h2] * alpha[h2] + mfma_16x16x32<F16>(ones, pp[h2], f32x4_t{0.f, 0.f, 0.f, 0.f})[0];
+      }
+      __threadfence();
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const float inv = 1.f / l_run[h2];
+        const int hq = hq0 + 16 * h2;
+        float* po = h2 ? po1 : po0;
+        uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + 4 * g;
+#pragma unroll 4
+        for (int e = 0; e < NE; ++e) {
+          float4 v = *reinterpret_cast<const float4*>(po + 16 * e);
+          v.x *= inv; v.y *= inv; v.z *= inv; v.w *= inv;
+          if (whole) st8(o + 16 * e, make_uint2(pack2<F16>(v.x, v.y), pack2<F16>(v.z, v.w)));
+          else *reinterpret_cast<float4*>(po + 16 * e) = v;
+        }
+        if (!whole && g == 0) p.part_lse[(int64_t)slot * p.Hq + hq] = m_run[h2] + fast_log2(l_run[h2]);
+      }
+    }
+  });
+#undef MI_SB
+}
+
 // One workgroup per (request, query head): merge the partials of the workgroups that
 // shared the request; zero-length rows get zeros.  blockDim.x = HD * S: S groups of HD threads take the
 // segments round-robin in batches of 8 (a request cut over hundreds of workgroups is a chain of dependent
@@ -1444,14 +1780,23 @@ static int mla_grid_size(int groups, const MiTuning& tune) {
   return grid < 1 ? 1 : grid;
 }
 static int mla_groups(int Hq) { return Hq <= 16 ? 1 : Hq / 16; }
+// the 128-heads-per-workgroup kernel: one workgroup per CU, Hq / 128 of them per span
+static bool mla_heads_kernel_shape(int Hq, int chunk_tokens) { return Hq % 128 == 0 && chunk_tokens % kMlaHeadsTile == 0; }
+static int mla_heads_grid_size(int Hq, const MiTuning& tune) {
+  if (tune.decode_grid > 0) return tune.decode_grid;
+  const int grid = device_cu_count() / (Hq / 128);
+  return grid < 1 ? 1 : grid;
+}
 }  // namespace mi
 
 extern "C" int64_t mi_mla_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t head_dim_v, const MiTuning* tuning) {
   if (R <= 0 || Hq <= 0 || head_dim_v <= 0) return 0;
   MiTuning tune;
   if (mi_resolve_tuning(tuning, &tune, "mi_mla_decode_workspace_bytes") != MI_OK) return -1;
-  // (the per-wavefront kernel uses the larger grid of the two: enough for either)
-  const int64_t slots = (int64_t)mla_grid_size(mla_groups(Hq), tune) + R;
+  // (the largest grid any of the kernels may take for this head count: enough for each of them)
+  int grid = mla_grid_size(mla_groups(Hq), tune);
+  if (Hq % 128 == 0 && mla_heads_grid_size(Hq, tune) > grid) grid = mla_heads_grid_size(Hq, tune);
+  const int64_t slots = (int64_t)grid + R;
   return slots * Hq * (head_dim_v + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
 
@@ -1508,8 +1853,13 @@ extern "C" int mi_paged_mla_decode_attention(
   const bool shared_tile = chunk_tokens % kMlaTile == 0 && tune.mla_decode_lds > 0 && lds_shared <= 160 * 1024;
   const int parts = (groups % 2 == 0) ? 4 : 8;            // output-column parts per head group
   const int wg_y = shared_tile ? groups / (8 / parts) : 0;  // workgroups per span (shared-tile kernel)
+  // Multiples of 128 heads: four wavefronts with 32 heads each (mla_decode_lds = 2 keeps the kernel above)
+  const size_t lds_heads = lds_head + (size_t)3 * kMlaHeadsBuf;
+  const bool heads_tile = mla_heads_kernel_shape(Hq, chunk_tokens) && tune.mla_decode_lds == 1 && lds_heads <= 160 * 1024;
   int grid_x = mla_grid_size(groups, tune);
-  if (shared_tile && tune.decode_grid <= 0) {
+  if (heads_tile) {
+    grid_x = mla_heads_grid_size(Hq, tune);
+  } else if (shared_tile && tune.decode_grid <= 0) {
     grid_x = device_cu_count() / wg_y;
     if (grid_x < 1) grid_x = 1;
   }
@@ -1532,13 +1882,13 @@ extern "C" int mi_paged_mla_decode_attention(
   p.k_scale = nullptr; p.v_scale = nullptr;
   p.R = R; p.Hq = Hq; p.Hkv = groups; p.G = Hq < 16 ? Hq : 16; p.parts = 1; p.chunk = chunk_tokens;
   p.chunk_magic = (((uint64_t)1 << 40) + chunk_tokens - 1) / chunk_tokens;
-  p.min_span_tiles = shared_tile ? 64 / kMlaTile : 64 / 16;
+  p.min_span_tiles = heads_tile ? 64 / kMlaHeadsTile : shared_tile ? 64 / kMlaTile : 64 / 16;
   p.grid = grid_x;
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
 
   hipStream_t st = (hipStream_t)stream;
   const int wpb = mla_waves_per_block(groups);
-  const size_t lds = shared_tile ? lds_shared : lds_head + (size_t)wpb * 16 * (576 * 2 + 16);
+  const size_t lds = heads_tile ? lds_heads : shared_tile ? lds_shared : lds_head + (size_t)wpb * 16 * (576 * 2 + 16);
   if (lds > 160 * 1024)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_mla_decode_attention: batch too large for the LDS of one workgroup");
   static std::atomic<bool> lds_limit_raised[64];  // per device: more than the default 64 KB of dynamic LDS
@@ -1551,7 +1901,9 @@ extern "C" int mi_paged_mla_decode_attention(
         hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<4, false>, attr, 160 * 1024) != hipSuccess ||
         hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<4, true>, attr, 160 * 1024) != hipSuccess ||
         hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8, false>, attr, 160 * 1024) != hipSuccess ||
-        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8, true>, attr, 160 * 1024) != hipSuccess)
+        hipFuncSetAttribute((const void*)paged_mla_decode_lds_kernel<8, true>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_heads_kernel<false>, attr, 160 * 1024) != hipSuccess ||
+        hipFuncSetAttribute((const void*)paged_mla_decode_heads_kernel<true>, attr, 160 * 1024) != hipSuccess)
       return mi_fail(MI_ERR_LAUNCH, "mi_paged_mla_decode_attention: cannot raise the dynamic LDS limit");
     lds_limit_raised[dev_id].store(true, std::memory_order_release);
   }
@@ -1560,7 +1912,9 @@ extern "C" int mi_paged_mla_decode_attention(
   if (timed) (void)hipEventRecord(ev_a, st);
 #define MI_LAUNCH_MLA(F16_)                                                                                       \
   do {                                                                                                            \
-    if (shared_tile && parts == 4)                                                                                \
+    if (heads_tile)                                                                                               \
+      hipLaunchKernelGGL((paged_mla_decode_heads_kernel<F16_>), dim3(grid_x, Hq / 128), dim3(256), lds, st, p);    \
+    else if (shared_tile && parts == 4)                                                                           \
       hipLaunchKernelGGL((paged_mla_decode_lds_kernel<4, F16_>), dim3(grid_x, wg_y), dim3(512), lds, st, p);       \
     else if (shared_tile)                                                                                         \
       hipLaunchKernelGGL((paged_mla_decode_lds_kernel<8, F16_>), dim3(grid_x, wg_y), dim3(512), lds, st, p);       \

@@ -30,11 +30,12 @@ def _check(mi, dev, q, cache, lens, bt, scale):
     return out
 
 
-@pytest.fixture(params=[0, -1], ids=["lds_tile", "streaming"])
+@pytest.fixture(params=[0, -1, 2], ids=["lds_tile", "streaming", "lds_tile_eight_wavefronts"])
 def kernel_choice(request, mi):
-    """Both decode kernels: latent tiles shared through LDS (chunk sizes that are multiples of 64 only;
-    other sizes stream either way) and one streaming wavefront per head group."""
-    mi.ops.set_tuning("mla_decode_lds", request.param)  # 0 = default (the LDS-tile kernel), -1 = never
+    """The decode kernels: latent tiles shared through LDS (chunk sizes that are multiples of 64, or of 32 at
+    multiples of 128 heads, where the default is the four-wavefront kernel with 32 heads per wavefront and 2 asks
+    for the eight-wavefront one; other sizes stream either way) and one streaming wavefront per head group."""
+    mi.ops.set_tuning("mla_decode_lds", request.param)  # 0 = default (an LDS-tile kernel), -1 = never
     yield request.param
     mi.ops.set_tuning("mla_decode_lds", 0)
 
@@ -61,6 +62,39 @@ def test_mla_decode_long_contexts_and_splits(mi, dev, Hq, kernel_choice):
             _check(mi, dev, q, cache, lens, bt, scale=0.07)
         finally:
             mi.ops.set_tuning("decode_grid", 0)
+
+
+@pytest.mark.parametrize("Hq", [128, 256])
+@pytest.mark.parametrize("chunk", [32, 96, 256])
+def test_mla_decode_128_heads_per_workgroup(mi, dev, Hq, chunk):
+    """The four-wavefront kernel (multiples of 128 heads, chunk sizes that are multiples of 32): tile edges, empty
+    requests, requests cut over workgroups, forced grids."""
+    lens = [0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, chunk - 1, chunk, chunk + 1, 3 * chunk + 5, 700, 0, 2049]
+    q, cache, lens, bt = _case(mi, dev, lens, Hq, chunk, seed=Hq + chunk)
+    out = _check(mi, dev, q, cache, lens, bt, scale=(128 + 64) ** -0.5)
+    assert (out.cpu()[lens == 0] == 0).all()
+    for grid in (1, 5, 64):
+        with mi.ops.tuning(decode_grid=grid):
+            _check(mi, dev, q, cache, lens, bt, scale=(128 + 64) ** -0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("choice", [0, 2])
+def test_mla_decode_128_heads_scores_that_keep_growing(mi, dev, dtype, choice):
+    """Keys whose scores grow along the sequence by far more than a factor 2^30: the four-wavefront kernel leaves its
+    fast loop (exponentials against the first tile's maxima) for the one that follows every maximum, in the middle
+    of a segment, whole requests and cut ones alike."""
+    lens = [900, 333, 64, 2500, 33]
+    q, cache, lens, bt = _case(mi, dev, lens, 128, 64, seed=11)
+    cache = cache.float()
+    for r in range(lens.numel()):
+        pos = torch.arange(int(lens[r]))
+        # (only the 64 values past the value part of a row grow: the outputs keep their size and the tolerance its meaning)
+        cache[bt[r, pos // 64].long(), pos % 64, DV:] *= (1.0 + 0.05 * pos)[:, None]
+    q, cache = q.to(dtype), cache.to(dtype)
+    for grid in (0, 7):
+        with mi.ops.tuning(mla_decode_lds=choice, decode_grid=grid):
+            _check(mi, dev, q, cache, lens, bt, scale=0.07)
 
 
 def test_mla_decode_many_requests_fall_back_to_streaming(mi, dev):
