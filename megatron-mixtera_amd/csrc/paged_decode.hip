@@ -1003,14 +1003,12 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
 // owns query heads 32 w .. 32 w + 31 (two 16-row tiles: every key fragment and every transposed value
 // fragment feeds two products) and all 512 output columns (256 accumulator registers), and shares
 // nothing with the others but the staged rows: no score exchange, one barrier per tile.
-// 32-token tiles (37 KB) in three LDS buffers: in iteration t the score product reads tile t, then
-// tile t+1 goes from registers to LDS, the barrier, the loads of tile t+2 are issued, softmax, value
-// product of tile t -- and the first key fragments of tile t+1 are requested under its last products.
-// (Three buffers: a wavefront past the barrier of iteration t+1 stores tile t+2 while a slower one
-// may still read values of tile t.)  The accumulators are rescaled only when a running maximum
-// moves by more than a factor 256: they live in accumulation registers, out of the vector ALU's
-// reach, and a rescale is ~770 instructions; until then probabilities are taken against the older
-// maximum (at most 256, exact in fp32 sums and within the 16-bit types' range).
+// 32-token tiles (37 KB) in four LDS buffers, filled by direct loads from memory (no staging registers, no LDS
+// stores): iteration t requests tile t+2, multiplies the scores of tile t, waits until its own loads of tile t+1
+// have landed, passes the barrier, then softmax and the value product of tile t -- with the first key fragments
+// of tile t+1 requested under its last products.  (Four buffers: tile t+2 replaces tile t-2, which every
+// wavefront left before the barrier of iteration t-1; a wavefront may still be reading values of tile t-1.)
+// The accumulators are never rescaled in that loop (see there).
 // ---------------------------------------------------------------------------------------------
 constexpr int kMlaHeadsTile = 32;  // tokens per staged tile of the 128-head kernel
 // A tile arrives in LDS by direct loads: each instruction puts its 64 lanes' 16-byte pieces side by side (1 KB), so a
@@ -1061,18 +1059,21 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
     const int ntile = (end - start + TK - 1) / TK;
     const int32_t* bt_row = p.bt + (int64_t)r * p.bt_stride;
 
+    auto load_q = [&](uint4 (&qf)[2][KS]) {
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        const uint16_t* qrow = p.q + (int64_t)row * p.q_st + (int64_t)(hq0 + 16 * h2) * p.q_sh + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) qf[h2][kk] = ld16(qrow + 32 * kk);
+      }
+    };
     uint4 qf[2][KS];
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-      const uint16_t* qrow = p.q + (int64_t)row * p.q_st + (int64_t)(hq0 + 16 * h2) * p.q_sh + 8 * g;
-#pragma unroll
-      for (int kk = 0; kk < KS; ++kk) qf[h2][kk] = ld16(qrow + 32 * kk);
-    }
+    load_q(qf);
     // A tile lies in one chunk (the launcher requires a chunk size that is a multiple of 32); rows past
     // the segment's last token re-read that token's row (their probabilities are forced to zero).
     // Tile t goes straight from memory into buffer t % 3: wavefront w issues loads w, w + 4, ... of the tile's 37;
     // lane l of load k fills piece 64 k + l of the buffer's line.  The loads count on the vector-memory counter.
-    auto tile_buf = [&](int t) { return (unsigned)t % 3u * (unsigned)kMlaHeadsBuf; };
+    auto tile_buf = [&](int t) { return ((unsigned)t & 3u) * (unsigned)kMlaHeadsBuf; };
     auto fetch = [&](int t) {
       const int T = start + t * TK;
       const int ci = chunk_of(T, p.chunk_magic);
@@ -1080,8 +1081,10 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
       const uint8_t* src = p.kc + (int64_t)pc * chunk_bytes + (int64_t)(uint32_t)(T - ci * p.chunk) * tok_bytes;
       const uint32_t row_lim = (uint32_t)min(last - T, TK - 1);
       const uint32_t dst = tiles_lds + tile_buf(t);
-      uint32_t ln = (uint32_t)lane;
-      asm volatile("" : "+v"(ln));  // opaque: the ten piece addresses are worked out here, not kept in registers across tiles
+      // (the lane number taken afresh and opaque: the ten piece addresses are worked out here, tile after tile,
+      // instead of living in registers -- or scratch memory -- across the loop)
+      uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+      asm volatile("" : "+v"(ln));
 #pragma unroll
       for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
         const int k = wave + 4 * i;
@@ -1095,7 +1098,14 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         }
       }
     };
-    auto fetch_wait = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    // tile t+1 has landed for this wavefront: nothing in flight but its loads of tile t+2 (ten for wavefront 0, nine
+    // for the others), which were issued after those of tile t+1 and complete after them
+    auto fetch_wait = [&](int t) {
+      if (t + 2 >= ntile) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      else if (wave == 0) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    };
+    static_assert(kMlaHeadsLoads == 37, "wavefront 0 issues ten loads per tile, the others nine");
     // key group i of a tile: fragments KB (i % (KS / KB)) .. + KB - 1 of 16-token sub-tile i / (KS / KB)
     auto load_k = [&](const uint8_t* buf, int i, uint4 (&kf)[KB]) {
       const uint8_t* ks = buf + kfrag_off + 16 * (i / (KS / KB)) * kMlaPitch + 64 * KB * (i % (KS / KB));
@@ -1135,7 +1145,8 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
     const float mul = p.scale_log2;
     // scores of tile t (key fragments of its first group already requested into kf[0]); requests the first value
     // fragments; masks the tokens past the segment's end; row maxima in the exponent's unit
-    auto scores = [&](int t, const uint8_t* buf, uint4 (&kf)[2][KB], uint2 (&vf0)[VB][2], f32x4_t (&sc)[2][2], float (&tmax)[2]) {
+    auto scores = [&](int t, const uint8_t* buf, const uint4 (&qf)[2][KS], uint4 (&kf)[2][KB], uint2 (&vf0)[VB][2],
+                      f32x4_t (&sc)[2][2], float (&tmax)[2]) {
 #pragma unroll
       for (int i = 0; i < NKG; ++i) {
         if (i + 1 < NKG) load_k(buf, i + 1, kf[(i + 1) & 1]);
@@ -1154,9 +1165,11 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2) {
         if (T + TK > end) {  // only the last tile of a segment has masked tokens
+          uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+          asm volatile("" : "+v"(ln));
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
-            const int tok0 = T + 16 * u + 4 * g;
+            const int tok0 = T + 16 * u + 4 * (int)(ln >> 4);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
               if (tok0 + i >= end) sc[h2][u][i] = -INFINITY;
@@ -1201,17 +1214,16 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         const uint8_t* buf = tiles + tile_buf(t);
         f32x4_t sc[2][2];
         float tmax[2];
-        scores(t, buf, kf, vf[0], sc, tmax);
+        if (t + 2 < ntile) fetch(t + 2);  // into the buffer of tile t-2, which every wavefront has left
+        scores(t, buf, qf, kf, vf[0], sc, tmax);
         if (t == 0) {
           m_run[0] = tmax[0];
           m_run[1] = tmax[1];
         }
         if (__builtin_amdgcn_ballot_w64(tmax[0] > m_run[0] + kLazy || tmax[1] > m_run[1] + kLazy)) break;
-        // ---- tile t+1 has landed (every wavefront waits for its own loads, then the barrier); tile t+2 sets
-        // out into the buffer of tile t-1, which nobody reads any more ----------------------------------
-        fetch_wait();
+        // ---- tile t+1 has landed: every wavefront waits for its own loads, then the barrier ------------
+        fetch_wait(t);
         __syncthreads();
-        if (t + 2 < ntile) fetch(t + 2);
         uint4 pp[2];
         probabilities(sc, pp);
         // ---- O^T += V^T P^T: one 32-token product per 16 columns and row tile; row sums from ones ----
@@ -1264,23 +1276,28 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
       // its own earlier stores what its loads see) ---------------------------------------------------------
       float* const po0 = p.part_o + ((int64_t)slot * p.Hq + hq0) * HDV + 4 * g;
       float* const po1 = po0 + (int64_t)16 * HDV;
+      // (the query fragments are fetched again: kept alive across the stores above, some of them would live in
+      // scratch memory -- in the fast loop as well)
+      uint4 qs[2][KS];
+      load_q(qs);
+      const int t_handover = t;
       for (; t < ntile; ++t) {
         const uint8_t* buf = tiles + tile_buf(t);
         uint4 kf[2][KB];
         uint2 vf[2][VB][2];
         f32x4_t sc[2][2];
         float tmax[2], alpha[2];
+        if (t + 2 < ntile && t != t_handover) fetch(t + 2);  // (the fast loop has issued the hand-over tile's already)
         load_k(buf, 0, kf[0]);
-        scores(t, buf, kf, vf[0], sc, tmax);
+        scores(t, buf, qs, kf, vf[0], sc, tmax);
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
           const float m_new = fmaxf(m_run[h2], tmax[h2]);
           alpha[h2] = fast_exp2(m_run[h2] - m_new);
           m_run[h2] = m_new;
         }
-        fetch_wait();
+        fetch_wait(t);
         __syncthreads();
-        if (t + 2 < ntile) fetch(t + 2);
         uint4 pp[2];
         probabilities(sc, pp);
         __threadfence();
@@ -1854,7 +1871,7 @@ extern "C" int mi_paged_mla_decode_attention(
   const int parts = (groups % 2 == 0) ? 4 : 8;            // output-column parts per head group
   const int wg_y = shared_tile ? groups / (8 / parts) : 0;  // workgroups per span (shared-tile kernel)
   // Multiples of 128 heads: four wavefronts with 32 heads each (mla_decode_lds = 2 keeps the kernel above)
-  const size_t lds_heads = lds_head + (size_t)3 * kMlaHeadsBuf;
+  const size_t lds_heads = lds_head + (size_t)4 * kMlaHeadsBuf;
   const bool heads_tile = mla_heads_kernel_shape(Hq, chunk_tokens) && tune.mla_decode_lds == 1 && lds_heads <= 160 * 1024;
   int grid_x = mla_grid_size(groups, tune);
   if (heads_tile) {
