@@ -1071,20 +1071,41 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
     load_q(qf);
     // A tile lies in one chunk (the launcher requires a chunk size that is a multiple of 32); rows past
     // the segment's last token re-read that token's row (their probabilities are forced to zero).
-    // Tile t goes straight from memory into buffer t % 3: wavefront w issues loads w, w + 4, ... of the tile's 37;
+    // Tile t goes straight from memory into buffer t % 4: wavefront w issues loads w, w + 4, ... of the tile's 37;
     // lane l of load k fills piece 64 k + l of the buffer's line.  The loads count on the vector-memory counter.
     auto tile_buf = [&](int t) { return ((unsigned)t & 3u) * (unsigned)kMlaHeadsBuf; };
-    auto fetch = [&](int t) {
+    // The block-table entry of tile t's chunk, by a scalar load the compiler does not see: a vector load in the tile
+    // loop would make it wait on the vector-memory counter, i.e. for every direct load in flight.  request / arrived
+    // are the two halves (the value may only be used after `arrived`); tiles past the segment ask for its last chunk.
+    const int ci_last = chunk_of(last, p.chunk_magic);
+    auto bt_request = [&](int t) {
+      const int byte_off = 4 * min(chunk_of(start + t * TK, p.chunk_magic), ci_last);
+      int pc;
+      asm volatile("s_load_dword %0, %1, %2" : "=s"(pc) : "s"(bt_row), "s"(byte_off) : "memory");
+      return pc;
+    };
+    auto bt_arrived = [&](int& pc) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(pc)::"memory"); };
+    auto fetch = [&](int t, int pc, const uint32_t* piece_off = nullptr) {
       const int T = start + t * TK;
       const int ci = chunk_of(T, p.chunk_magic);
-      const int pc = __builtin_amdgcn_readfirstlane(bt_row[ci]);
       const uint8_t* src = p.kc + (int64_t)pc * chunk_bytes + (int64_t)(uint32_t)(T - ci * p.chunk) * tok_bytes;
       const uint32_t row_lim = (uint32_t)min(last - T, TK - 1);
       const uint32_t dst = tiles_lds + tile_buf(t);
-      // (the lane number taken afresh and opaque: the ten piece addresses are worked out here, tile after tile,
-      // instead of living in registers -- or scratch memory -- across the loop)
+      if (piece_off && row_lim == TK - 1) {  // a whole tile in the fast loop: scalar base + the lane's fixed offsets
+#pragma unroll
+        for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
+          const int k = wave + 4 * i;
+          if (k < kMlaHeadsLoads) {  // wave-uniform
+            const uint32_t m0 = __builtin_amdgcn_readfirstlane(dst + 1024u * (uint32_t)k);
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(piece_off[i]), "s"(src)
+                         : "memory");
+          }
+        }
+        return;
+      }
+      // a segment's last tile: rows past its last token re-read that token's row
       uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-      asm volatile("" : "+v"(ln));
+      asm volatile("" : "+v"(ln));  // (opaque: these addresses are worked out here, not kept in registers across tiles)
 #pragma unroll
       for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
         const int k = wave + 4 * i;
@@ -1123,7 +1144,10 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
     };
 
     __syncthreads();  // every wavefront is done with the previous segment's buffers
-    fetch(0);
+    int pc0 = bt_request(0), pc1 = bt_request(1);
+    bt_arrived(pc1);
+    bt_arrived(pc0);
+    fetch(0, pc0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), in the compiler's sight
     // (the query fragments count as used here: the compiler then waits for their loads now and not in the tile loop,
     // where a wait on the vector-memory counter waits for the direct loads in flight as well)
@@ -1132,7 +1156,8 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk)
         asm volatile("" ::"v"(qf[h2][kk].x), "v"(qf[h2][kk].y), "v"(qf[h2][kk].z), "v"(qf[h2][kk].w));
-    if (ntile > 1) fetch(1);
+    if (ntile > 1) fetch(1, pc1);
+    int pc_ahead = bt_request(2);  // of the tile the loops fetch next; each iteration asks for the one after
     __syncthreads();
 
     // The accumulators live in accumulation registers, out of the vector ALU's reach, and any other definition of
@@ -1209,12 +1234,27 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         for (int e = 0; e < NE; ++e) acc[h2][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       uint4 kf[2][KB];
       uint2 vf[2][VB][2];
+      // where this lane's piece of direct load k = wave + 4 i of a whole tile comes from, relative to the tile's first
+      // row: piece 64 k + lane of the line = (row, 16-byte column) = divmod by 73, the padding column doubling the last
+      // one.  (Worked out per segment, from an opaque copy of the lane number so that it stays so: alive across the
+      // whole kernel they would live in scratch memory.)
+      uint32_t piece_off[(kMlaHeadsLoads + 3) / 4];
+      uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+      asm volatile("" : "+v"(ln));
+#pragma unroll
+      for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
+        const uint32_t u = 64u * (uint32_t)(wave + 4 * i) + ln;
+        const uint32_t prow = (u * 14365u) >> 20, pcol = u - 73u * prow;
+        piece_off[i] = min(prow, (uint32_t)TK - 1) * tok_bytes + 16u * min(pcol, 71u);
+      }
       load_k(tiles + tile_buf(0), 0, kf[0]);
       for (; t < ntile; ++t) {
         const uint8_t* buf = tiles + tile_buf(t);
         f32x4_t sc[2][2];
         float tmax[2];
-        if (t + 2 < ntile) fetch(t + 2);  // into the buffer of tile t-2, which every wavefront has left
+        bt_arrived(pc_ahead);
+        if (t + 2 < ntile) fetch(t + 2, pc_ahead, piece_off);  // into the buffer of tile t-2, which every wavefront has left
+        pc_ahead = bt_request(t + 3);
         scores(t, buf, qf, kf, vf[0], sc, tmax);
         if (t == 0) {
           m_run[0] = tmax[0];
@@ -1287,7 +1327,11 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         uint2 vf[2][VB][2];
         f32x4_t sc[2][2];
         float tmax[2], alpha[2];
-        if (t + 2 < ntile && t != t_handover) fetch(t + 2);  // (the fast loop has issued the hand-over tile's already)
+        if (t != t_handover) {  // (the fast loop has dealt with the hand-over tile's already)
+          bt_arrived(pc_ahead);
+          if (t + 2 < ntile) fetch(t + 2, pc_ahead);
+          pc_ahead = bt_request(t + 3);
+        }
         load_k(buf, 0, kf[0]);
         scores(t, buf, qs, kf, vf[0], sc, tmax);
 #pragma unroll
