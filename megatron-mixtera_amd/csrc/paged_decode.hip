@@ -1043,8 +1043,22 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
   const uint32_t tok_bytes = (uint32_t)(p.kv_st * 2);
   // the LDS byte address of the tile buffers, for the direct loads
   const uint32_t tiles_lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)tiles;
-  const int kfrag_off = m16 * kMlaPitch + 16 * g;
-  const int vfrag_off = (4 * g + (m16 >> 2)) * kMlaPitch + 8 * (m16 & 3);
+  // The lane number, computed where it is asked for (volatile: neither hoisted nor shared between its uses).
+  auto lane_now = []() {
+    uint32_t ln;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=&v"(ln));
+    return ln;
+  };
+  // Where a lane's key fragments (the A operand of the scores) and transposed value fragments start within a tile.
+  // Worked out afresh for every tile from an opaque copy of the lane number: kept in a register across the kernel,
+  // such a value ends up in scratch memory, and its reload in the tile loop waits on the vector-memory counter --
+  // for every direct load in flight.
+  auto frag_offsets = [&](int& kfrag_off, int& vfrag_off) {
+    const uint32_t ln = lane_now();
+    const int m = ln & 15, gq = ln >> 4;
+    kfrag_off = m * kMlaPitch + 16 * gq;
+    vfrag_off = (4 * gq + (m >> 2)) * kMlaPitch + 8 * (m & 3);
+  };
   const uint4 ones = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
 #define MI_SB() __builtin_amdgcn_sched_barrier(0)
 
@@ -1085,27 +1099,26 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
       return pc;
     };
     auto bt_arrived = [&](int& pc) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(pc)::"memory"); };
-    auto fetch = [&](int t, int pc, const uint32_t* piece_off = nullptr) {
+    auto tile_src = [&](int t, int pc) {
       const int T = start + t * TK;
       const int ci = chunk_of(T, p.chunk_magic);
-      const uint8_t* src = p.kc + (int64_t)pc * chunk_bytes + (int64_t)(uint32_t)(T - ci * p.chunk) * tok_bytes;
-      const uint32_t row_lim = (uint32_t)min(last - T, TK - 1);
-      const uint32_t dst = tiles_lds + tile_buf(t);
-      if (piece_off && row_lim == TK - 1) {  // a whole tile in the fast loop: scalar base + the lane's fixed offsets
-#pragma unroll
-        for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
-          const int k = wave + 4 * i;
-          if (k < kMlaHeadsLoads) {  // wave-uniform
-            const uint32_t m0 = __builtin_amdgcn_readfirstlane(dst + 1024u * (uint32_t)k);
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(piece_off[i]), "s"(src)
-                         : "memory");
-          }
-        }
-        return;
+      return p.kc + (int64_t)pc * chunk_bytes + (int64_t)(uint32_t)(T - ci * p.chunk) * tok_bytes;
+    };
+    auto whole_tile = [&](int t) { return last - (start + t * TK) >= TK - 1; };
+    // direct load i (of this wavefront's nine or ten) of a whole tile: scalar base + the lane's fixed offset
+    auto fetch_piece = [&](int t, const uint8_t* src, int i, uint32_t piece_off_i) {
+      const int k = wave + 4 * i;
+      if (k < kMlaHeadsLoads) {  // wave-uniform
+        const uint32_t m0 = __builtin_amdgcn_readfirstlane(tiles_lds + tile_buf(t) + 1024u * (uint32_t)k);
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(piece_off_i), "s"(src) : "memory");
       }
-      // a segment's last tile: rows past its last token re-read that token's row
-      uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-      asm volatile("" : "+v"(ln));  // (opaque: these addresses are worked out here, not kept in registers across tiles)
+    };
+    // any tile, all of this wavefront's loads at once: rows past the segment's last token re-read that token's row
+    auto fetch = [&](int t, int pc) {
+      const uint8_t* src = tile_src(t, pc);
+      const uint32_t row_lim = (uint32_t)min(last - (start + t * TK), TK - 1);
+      const uint32_t dst = tiles_lds + tile_buf(t);
+      const uint32_t ln = lane_now();
 #pragma unroll
       for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
         const int k = wave + 4 * i;
@@ -1120,7 +1133,8 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
       }
     };
     // tile t+1 has landed for this wavefront: nothing in flight but its loads of tile t+2 (ten for wavefront 0, nine
-    // for the others), which were issued after those of tile t+1 and complete after them
+    // for the others), which were issued after those of tile t+1 and complete after them (those of tile t+3 are
+    // issued after this wait)
     auto fetch_wait = [&](int t) {
       if (t + 2 >= ntile) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       else if (wave == 0) asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
@@ -1128,13 +1142,13 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
     };
     static_assert(kMlaHeadsLoads == 37, "wavefront 0 issues ten loads per tile, the others nine");
     // key group i of a tile: fragments KB (i % (KS / KB)) .. + KB - 1 of 16-token sub-tile i / (KS / KB)
-    auto load_k = [&](const uint8_t* buf, int i, uint4 (&kf)[KB]) {
+    auto load_k = [&](const uint8_t* buf, int kfrag_off, int i, uint4 (&kf)[KB]) {
       const uint8_t* ks = buf + kfrag_off + 16 * (i / (KS / KB)) * kMlaPitch + 64 * KB * (i % (KS / KB));
 #pragma unroll
       for (int j = 0; j < KB; ++j) kf[j] = *reinterpret_cast<const uint4*>(ks + 64 * j);
     };
     // value group j: output columns 16 VB j .. + 16 VB - 1, all 32 tokens, transposed
-    auto load_v = [&](const uint8_t* buf, int j, uint2 (&vf)[VB][2]) {
+    auto load_v = [&](const uint8_t* buf, int vfrag_off, int j, uint2 (&vf)[VB][2]) {
       const uint8_t* vs = buf + vfrag_off + 32 * VB * j;
 #pragma unroll
       for (int e = 0; e < VB; ++e) {
@@ -1143,11 +1157,34 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
       }
     };
 
+    // where this lane's piece of direct load k = wave + 4 i of a whole tile comes from, relative to the tile's first
+    // row: piece 64 k + lane of the line = (row, 16-byte column) = divmod by 73, the padding column doubling the last
+    // one.  (Worked out per segment, from a lane number of its own so that it stays so: alive across the whole kernel
+    // they would live in scratch memory.)
+    uint32_t piece_off[(kMlaHeadsLoads + 3) / 4];
+    {
+      const uint32_t ln = lane_now();
+#pragma unroll
+      for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
+        const uint32_t u = 64u * (uint32_t)(wave + 4 * i) + ln;
+        const uint32_t prow = (u * 14365u) >> 20, pcol = u - 73u * prow;
+        piece_off[i] = min(prow, (uint32_t)TK - 1) * tok_bytes + 16u * min(pcol, 71u);
+      }
+    }
+    // a tile of the prologue: whole ones by the fixed offsets, the segment's last one the general way
+    auto fetch_first = [&](int t, int pc) {
+      if (!whole_tile(t)) return fetch(t, pc);
+      const uint8_t* src = tile_src(t, pc);
+#pragma unroll
+      for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) fetch_piece(t, src, i, piece_off[i]);
+    };
+
     __syncthreads();  // every wavefront is done with the previous segment's buffers
-    int pc0 = bt_request(0), pc1 = bt_request(1);
+    int pc0 = bt_request(0), pc1 = bt_request(1), pc2 = bt_request(2);
+    bt_arrived(pc2);
     bt_arrived(pc1);
     bt_arrived(pc0);
-    fetch(0, pc0);
+    fetch_first(0, pc0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0), in the compiler's sight
     // (the query fragments count as used here: the compiler then waits for their loads now and not in the tile loop,
     // where a wait on the vector-memory counter waits for the direct loads in flight as well)
@@ -1156,8 +1193,9 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 #pragma unroll
       for (int kk = 0; kk < KS; ++kk)
         asm volatile("" ::"v"(qf[h2][kk].x), "v"(qf[h2][kk].y), "v"(qf[h2][kk].z), "v"(qf[h2][kk].w));
-    if (ntile > 1) fetch(1, pc1);
-    int pc_ahead = bt_request(2);  // of the tile the loops fetch next; each iteration asks for the one after
+    if (ntile > 1) fetch_first(1, pc1);
+    if (ntile > 2) fetch_first(2, pc2);
+    int pc_ahead = bt_request(3);  // of the tile the loops fetch next; each iteration asks for the one after
     __syncthreads();
 
     // The accumulators live in accumulation registers, out of the vector ALU's reach, and any other definition of
@@ -1170,12 +1208,12 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
     const float mul = p.scale_log2;
     // scores of tile t (key fragments of its first group already requested into kf[0]); requests the first value
     // fragments; masks the tokens past the segment's end; row maxima in the exponent's unit
-    auto scores = [&](int t, const uint8_t* buf, const uint4 (&qf)[2][KS], uint4 (&kf)[2][KB], uint2 (&vf0)[VB][2],
-                      f32x4_t (&sc)[2][2], float (&tmax)[2]) {
+    auto scores = [&](int t, const uint8_t* buf, int kfrag_off, int vfrag_off, const uint4 (&qf)[2][KS], uint4 (&kf)[2][KB],
+                      uint2 (&vf0)[VB][2], f32x4_t (&sc)[2][2], float (&tmax)[2]) {
 #pragma unroll
       for (int i = 0; i < NKG; ++i) {
-        if (i + 1 < NKG) load_k(buf, i + 1, kf[(i + 1) & 1]);
-        else load_v(buf, 0, vf0);
+        if (i + 1 < NKG) load_k(buf, kfrag_off, i + 1, kf[(i + 1) & 1]);
+        else load_v(buf, vfrag_off, 0, vf0);
         MI_SB();
         const int u = i / (KS / KB), k0 = KB * (i % (KS / KB));
 #pragma unroll
@@ -1190,8 +1228,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 #pragma unroll
       for (int h2 = 0; h2 < 2; ++h2) {
         if (T + TK > end) {  // only the last tile of a segment has masked tokens
-          uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-          asm volatile("" : "+v"(ln));
+          const uint32_t ln = lane_now();
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
             const int tok0 = T + 16 * u + 4 * (int)(ln >> 4);
@@ -1234,28 +1271,18 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         for (int e = 0; e < NE; ++e) acc[h2][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       uint4 kf[2][KB];
       uint2 vf[2][VB][2];
-      // where this lane's piece of direct load k = wave + 4 i of a whole tile comes from, relative to the tile's first
-      // row: piece 64 k + lane of the line = (row, 16-byte column) = divmod by 73, the padding column doubling the last
-      // one.  (Worked out per segment, from an opaque copy of the lane number so that it stays so: alive across the
-      // whole kernel they would live in scratch memory.)
-      uint32_t piece_off[(kMlaHeadsLoads + 3) / 4];
-      uint32_t ln = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-      asm volatile("" : "+v"(ln));
-#pragma unroll
-      for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
-        const uint32_t u = 64u * (uint32_t)(wave + 4 * i) + ln;
-        const uint32_t prow = (u * 14365u) >> 20, pcol = u - 73u * prow;
-        piece_off[i] = min(prow, (uint32_t)TK - 1) * tok_bytes + 16u * min(pcol, 71u);
+      {
+        int kfo, vfo;
+        frag_offsets(kfo, vfo);
+        load_k(tiles + tile_buf(0), kfo, 0, kf[0]);
       }
-      load_k(tiles + tile_buf(0), 0, kf[0]);
       for (; t < ntile; ++t) {
         const uint8_t* buf = tiles + tile_buf(t);
         f32x4_t sc[2][2];
         float tmax[2];
-        bt_arrived(pc_ahead);
-        if (t + 2 < ntile) fetch(t + 2, pc_ahead, piece_off);  // into the buffer of tile t-2, which every wavefront has left
-        pc_ahead = bt_request(t + 3);
-        scores(t, buf, qf, kf, vf[0], sc, tmax);
+        int kfrag_off, vfrag_off;
+        frag_offsets(kfrag_off, vfrag_off);
+        scores(t, buf, kfrag_off, vfrag_off, qf, kf, vf[0], sc, tmax);
         if (t == 0) {
           m_run[0] = tmax[0];
           m_run[1] = tmax[1];
@@ -1264,14 +1291,22 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         // ---- tile t+1 has landed: every wavefront waits for its own loads, then the barrier ------------
         fetch_wait(t);
         __syncthreads();
+        // ---- tile t+3 sets out into the buffer of tile t-1, which every wavefront has left: its loads are issued
+        // one by one under the products below (all at once here when it is the segment's last, partial tile) ----
+        bt_arrived(pc_ahead);
+        const bool more = t + 3 < ntile, piecewise = more && whole_tile(t + 3);
+        const uint8_t* const src_ahead = tile_src(t + 3, pc_ahead);
+        if (more && !piecewise) fetch(t + 3, pc_ahead);
+        pc_ahead = bt_request(t + 4);
         uint4 pp[2];
         probabilities(sc, pp);
         // ---- O^T += V^T P^T: one 32-token product per 16 columns and row tile; row sums from ones ----
         const uint8_t* nbuf = tiles + tile_buf(t + 1);
+        static_assert(NVG >= (kMlaHeadsLoads + 3) / 4, "one direct load per group of products");
 #pragma unroll
         for (int j = 0; j < NVG; ++j) {
-          if (j + 1 < NVG) load_v(buf, j + 1, vf[(j + 1) & 1]);
-          else if (t + 1 < ntile) load_k(nbuf, 0, kf[0]);
+          if (j + 1 < NVG) load_v(buf, vfrag_off, j + 1, vf[(j + 1) & 1]);
+          else if (t + 1 < ntile) load_k(nbuf, kfrag_off, 0, kf[0]);
           MI_SB();
 #pragma unroll
           for (int e = 0; e < VB; ++e) {
@@ -1279,6 +1314,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 #pragma unroll
             for (int h2 = 0; h2 < 2; ++h2) acc[h2][VB * j + e] = mfma_16x16x32<F16>(a, pp[h2], acc[h2][VB * j + e]);
           }
+          if (j < (kMlaHeadsLoads + 3) / 4 && piecewise) fetch_piece(t + 3, src_ahead, j, piece_off[j]);
           if (j == 0) {
 #pragma unroll
             for (int h2 = 0; h2 < 2; ++h2)
@@ -1320,20 +1356,17 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
       // scratch memory -- in the fast loop as well)
       uint4 qs[2][KS];
       load_q(qs);
-      const int t_handover = t;
       for (; t < ntile; ++t) {
         const uint8_t* buf = tiles + tile_buf(t);
         uint4 kf[2][KB];
         uint2 vf[2][VB][2];
         f32x4_t sc[2][2];
         float tmax[2], alpha[2];
-        if (t != t_handover) {  // (the fast loop has dealt with the hand-over tile's already)
-          bt_arrived(pc_ahead);
-          if (t + 2 < ntile) fetch(t + 2, pc_ahead);
-          pc_ahead = bt_request(t + 3);
-        }
-        load_k(buf, 0, kf[0]);
-        scores(t, buf, qs, kf, vf[0], sc, tmax);
+
+        int kfrag_off, vfrag_off;
+        frag_offsets(kfrag_off, vfrag_off);
+        load_k(buf, kfrag_off, 0, kf[0]);
+        scores(t, buf, kfrag_off, vfrag_off, qs, kf, vf[0], sc, tmax);
 #pragma unroll
         for (int h2 = 0; h2 < 2; ++h2) {
           const float m_new = fmaxf(m_run[h2], tmax[h2]);
@@ -1342,12 +1375,15 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         }
         fetch_wait(t);
         __syncthreads();
+        bt_arrived(pc_ahead);
+        if (t + 3 < ntile) fetch(t + 3, pc_ahead);
+        pc_ahead = bt_request(t + 4);
         uint4 pp[2];
         probabilities(sc, pp);
         __threadfence();
 #pragma unroll
         for (int j = 0; j < NVG; ++j) {
-          if (j + 1 < NVG) load_v(buf, j + 1, vf[(j + 1) & 1]);
+          if (j + 1 < NVG) load_v(buf, vfrag_off, j + 1, vf[(j + 1) & 1]);
           MI_SB();
 #pragma unroll
           for (int e = 0; e < VB; ++e) {
