@@ -90,7 +90,7 @@ def run_secondary(args, mi, lib, torch, dev):
         step = lambda: mi.ops.paged_mla_decode_attention(q, cache, lens_d, bt_d, softmax_scale=0.072, out=out)
         nbytes = int(lens.sum()) * 576 * 2 + B * Hq * (576 + 512) * 2 + int(((lens + 255) // 256).sum()) * 4 + B * 4
         flops = int(lens.sum()) * Hq * (576 + 512) * 2
-        kernel = "paged_mla_decode_lds_kernel"
+        kernel = "paged_mla_decode_heads_kernel" if Hq % 128 == 0 else "paged_mla_decode_lds_kernel"
         what = (f"absorbed multi-latent decode attention, {Hq} query heads, batch {B}, latent rows of 576 bf16, "
                 f"context U[{prm['lo']},{prm['hi']}], chunk 256")
         dtype = "bf16 (fp32 accumulate)"

@@ -75,8 +75,10 @@ typedef struct MiTuning {
   int32_t norm_rope_vectorised;   /* 16-byte-per-lane norm / rotary kernel: 0 = default (from 256 tokens up, where
                                      alignment and rotary width allow), 1 = wherever they allow, -1 = never */
   int32_t mla_decode_lds;         /* multi-latent decode: 0 = default (latent tiles shared through LDS when the chunk
-                                     size is a multiple of 64 and the call has at most 768 requests), -1 = one
-                                     streaming wavefront per 16-head group always */
+                                     size is a multiple of 64 and the call has at most 768 requests; with a multiple
+                                     of 128 query heads and a chunk size that is a multiple of 32, by the kernel of
+                                     four wavefronts with 32 heads each), 2 = the eight-wavefront LDS kernel at
+                                     every head count, -1 = one streaming wavefront per 16-head group always */
   int32_t reserved[5];            /* must be 0 */
 } MiTuning;
 

@@ -188,16 +188,23 @@ def case_prefill(mi, dev, rng, seed, fp8):
 
 def case_mla_decode(mi, dev, rng, seed):
     gen = torch.Generator().manual_seed(seed)
-    Hq = rng.choice([1, 2, 4, 8, 16, 32, 48, 64, 128])
-    chunk = rng.choice([16, 32, 64, 128, 256])
+    Hq = rng.choice([1, 2, 4, 8, 16, 32, 48, 64, 128, 128, 128, 256])
+    chunk = rng.choice([16, 32, 64, 96, 128, 256])
     R = rng.randint(1, 12)
     lens = rand_lens(rng, R, chunk, 1200)
     grid = rng.choice([0, 0, 1, 5, 41])
-    lds = rng.choice([0, 0, -1])
-    _note(f"mla_decode seed={seed} Hq={Hq} chunk={chunk} lens={lens} grid={grid} lds={lds}")
+    lds = rng.choice([0, 0, -1, 2])
+    grow = rng.choice([0.0, 0.0, 0.0, 0.05])  # scores that keep growing along the sequence (through the 64 values past
+    # the value part of a row, so the outputs keep their size): row maxima that leave any window above the first tile's
+    _note(f"mla_decode seed={seed} Hq={Hq} chunk={chunk} lens={lens} grid={grid} lds={lds} grow={grow}")
     lens_t = torch.tensor(lens, dtype=torch.int32)
     bt, N = mi.synthetic.build_block_table(lens_t, chunk, gen)
-    cache = (torch.randn(N + 2, chunk, 576, generator=gen) * 0.5).bfloat16()
+    cache = torch.randn(N + 2, chunk, 576, generator=gen) * 0.5
+    if grow:
+        for r in range(R):
+            pos = torch.arange(lens[r])
+            cache[bt[r, pos // chunk].long(), pos % chunk, 512:] *= (1.0 + grow * pos)[:, None]
+    cache = cache.bfloat16()
     q = torch.randn(R, 1, Hq, 576, generator=gen).bfloat16()
     mi.ops.set_tuning("decode_grid", grid)
     mi.ops.set_tuning("mla_decode_lds", lds)
