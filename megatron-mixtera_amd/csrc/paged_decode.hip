@@ -802,7 +802,11 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_stream_kernel(DecodeP
 // Two barriers per tile; the global loads of tile t+1 are in flight in registers while tile t computes.
 // ---------------------------------------------------------------------------------------------
 constexpr int kMlaTile = 64;                 // tokens per staged tile
-constexpr int kMlaPitch = 576 * 2 + 16;      // LDS bytes per staged row: 16 rows of a fragment read cover all banks
+// LDS bytes per staged row.  (By counter a 16-byte fragment read takes 4 conflict cycles on top of its 4 and a
+// transposing 8-byte read 2 on top of its 2 at this pitch -- 292 dwords = 36 mod 64; 1 184 bytes, as in the kernel
+// for 128 heads below, has none, but two 64-token buffers of it leave room for 512 requests' prefix sums instead
+// of 768, and this kernel is no faster for it.)
+constexpr int kMlaPitch = 576 * 2 + 16;
 
 template <int PARTS, bool F16>
 __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodeParams p) {
@@ -1011,17 +1015,21 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
 // The accumulators are never rescaled in that loop (see there).
 // ---------------------------------------------------------------------------------------------
 constexpr int kMlaHeadsTile = 32;  // tokens per staged tile of the 128-head kernel
+// LDS bytes per staged row: 296 dwords = 40 mod 64, an odd multiple of 8 banks.  A 16-byte fragment read is served in
+// passes of {rows 0-7 at piece g, rows 8-15 at piece g + 1} and a transposing 8-byte read in passes of eight rows: both
+// then cover the 64 banks exactly once (no conflict cycle by counter; at 1 168 bytes: 4 and 2 per read).
+constexpr int kMlaHeadsPitch = 576 * 2 + 32;
 // A tile arrives in LDS by direct loads: each instruction puts its 64 lanes' 16-byte pieces side by side (1 KB), so a
-// tile is 37 instructions over a line of 32 x 73 pieces (72 of a row + the 16 bytes of row padding, which receive a
-// copy of the row's last piece), and a buffer is 37 KB.
-constexpr int kMlaHeadsLoads = (kMlaHeadsTile * (kMlaPitch / 16) + 63) / 64;
+// tile is 37 instructions over a line of 32 x 74 pieces (72 of a row + the 32 bytes of row padding, which receive
+// copies of the row's last piece), and a buffer is 37 KB -- exactly.
+constexpr int kMlaHeadsLoads = (kMlaHeadsTile * (kMlaHeadsPitch / 16) + 63) / 64;
 constexpr int kMlaHeadsBuf = kMlaHeadsLoads * 1024;
 constexpr bool mla_piece_division_ok() {
   for (unsigned u = 0; u < 64u * kMlaHeadsLoads; ++u)
-    if (((u * 14365u) >> 20) != u / 73u) return false;
+    if (((u * 14170u) >> 20) != u / 74u) return false;
   return true;
 }
-static_assert(kMlaPitch == 73 * 16 && mla_piece_division_ok(), "piece -> (row, column) by multiplication");
+static_assert(kMlaHeadsPitch == 74 * 16 && mla_piece_division_ok(), "piece -> (row, column) by multiplication");
 
 template <bool F16>
 __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodeParams p) {
@@ -1056,8 +1064,8 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
   auto frag_offsets = [&](int& kfrag_off, int& vfrag_off) {
     const uint32_t ln = lane_now();
     const int m = ln & 15, gq = ln >> 4;
-    kfrag_off = m * kMlaPitch + 16 * gq;
-    vfrag_off = (4 * gq + (m >> 2)) * kMlaPitch + 8 * (m & 3);
+    kfrag_off = m * kMlaHeadsPitch + 16 * gq;
+    vfrag_off = (4 * gq + (m >> 2)) * kMlaHeadsPitch + 8 * (m & 3);
   };
   const uint4 ones = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
 #define MI_SB() __builtin_amdgcn_sched_barrier(0)
@@ -1124,7 +1132,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
         const int k = wave + 4 * i;
         if (k < kMlaHeadsLoads) {  // wave-uniform
           const uint32_t u = 64u * (uint32_t)k + ln;
-          const uint32_t prow = (u * 14365u) >> 20, pcol = u - 73u * prow;
+          const uint32_t prow = (u * 14170u) >> 20, pcol = u - 74u * prow;
           const uint8_t* g_src = src + min(prow, row_lim) * tok_bytes + 16u * min(pcol, 71u);
           const uint32_t m0 = __builtin_amdgcn_readfirstlane(dst + 1024u * (uint32_t)k);
           asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(g_src) : "memory");
@@ -1143,7 +1151,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
     static_assert(kMlaHeadsLoads == 37, "wavefront 0 issues ten loads per tile, the others nine");
     // key group i of a tile: fragments KB (i % (KS / KB)) .. + KB - 1 of 16-token sub-tile i / (KS / KB)
     auto load_k = [&](const uint8_t* buf, int kfrag_off, int i, uint4 (&kf)[KB]) {
-      const uint8_t* ks = buf + kfrag_off + 16 * (i / (KS / KB)) * kMlaPitch + 64 * KB * (i % (KS / KB));
+      const uint8_t* ks = buf + kfrag_off + 16 * (i / (KS / KB)) * kMlaHeadsPitch + 64 * KB * (i % (KS / KB));
 #pragma unroll
       for (int j = 0; j < KB; ++j) kf[j] = *reinterpret_cast<const uint4*>(ks + 64 * j);
     };
@@ -1153,12 +1161,12 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 #pragma unroll
       for (int e = 0; e < VB; ++e) {
         vf[e][0] = lds_ld8_tr(vs + 32 * e);
-        vf[e][1] = lds_ld8_tr(vs + 16 * kMlaPitch + 32 * e);
+        vf[e][1] = lds_ld8_tr(vs + 16 * kMlaHeadsPitch + 32 * e);
       }
     };
 
     // where this lane's piece of direct load k = wave + 4 i of a whole tile comes from, relative to the tile's first
-    // row: piece 64 k + lane of the line = (row, 16-byte column) = divmod by 73, the padding column doubling the last
+    // row: piece 64 k + lane of the line = (row, 16-byte column) = divmod by 74, the padding columns doubling the last
     // one.  (Worked out per segment, from a lane number of its own so that it stays so: alive across the whole kernel
     // they would live in scratch memory.)
     uint32_t piece_off[(kMlaHeadsLoads + 3) / 4];
@@ -1167,7 +1175,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 #pragma unroll
       for (int i = 0; i < (kMlaHeadsLoads + 3) / 4; ++i) {
         const uint32_t u = 64u * (uint32_t)(wave + 4 * i) + ln;
-        const uint32_t prow = (u * 14365u) >> 20, pcol = u - 73u * prow;
+        const uint32_t prow = (u * 14170u) >> 20, pcol = u - 74u * prow;
         piece_off[i] = min(prow, (uint32_t)TK - 1) * tok_bytes + 16u * min(pcol, 71u);
       }
     }
