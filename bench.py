@@ -38,14 +38,18 @@ MEASURED_HBM_TRAFFIC_BYTES = {
     "cfg2": 1_226_700_000, "cfg2_step": 1_215_100_000, "cfg4": 8_724_600_000, "cfg4_step": 8_635_100_000,
     "cfg5": 9_070_700_000,
     # the mixed step: tile kernel, stream kernel
-    "cfg3_tile": 401_600_000, "cfg3_stream": 2_195_400_000}
+    "cfg3_tile": 401_600_000, "cfg3_stream": 2_195_400_000,
+    # multi-latent decode at 128 heads (reads + the partial results it writes)
+    "mla_decode_h128": 454_500_000, "mla_decode_h128_long": 1_305_000_000}
 # Where each figure above was read, so that a reader of the JSON line can tell a stale constant from a fresh one:
 # the summary file and the last commit that touched the kernel when the counters were collected.
 _DECODE_TRAFFIC = ("profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                    "kernels as of commit bc375af)")
 _MIXED_TRAFFIC = ("profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
                   "commit bc375af)")
-TRAFFIC_SOURCE = {"cfg2": _DECODE_TRAFFIC, "cfg2_step": _DECODE_TRAFFIC, "cfg4": _DECODE_TRAFFIC,
+_MLA_HEADS_TRAFFIC = ("profiles/paged_mla_decode_heads_kernel_h128_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
+                      "kernel as of commit 3b3c0d1)")
+TRAFFIC_SOURCE = {"mla_decode_h128": _MLA_HEADS_TRAFFIC, "mla_decode_h128_long": _MLA_HEADS_TRAFFIC, "cfg2": _DECODE_TRAFFIC, "cfg2_step": _DECODE_TRAFFIC, "cfg4": _DECODE_TRAFFIC,
                   "cfg4_step": _DECODE_TRAFFIC, "cfg5": _DECODE_TRAFFIC, "cfg3_tile": _MIXED_TRAFFIC,
                   "cfg3_stream": _MIXED_TRAFFIC}
 
@@ -179,7 +183,9 @@ def run_secondary(args, mi, lib, torch, dev):
                  "frac": round(flops / kernel_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)} if mfma_bound else
                 {"bound": "hbm", "kernel": kernel, "achieved": round(nbytes / kernel_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
                  "unit": "GB/s", "frac": round(nbytes / kernel_ms / 1e6 / HBM_PEAK_GBPS, 4)})
-    roofline.update({"kernel_ms": round(kernel_ms, 5), "traffic": None})
+    roofline.update({"kernel_ms": round(kernel_ms, 5), "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload)})
+    if args.workload in TRAFFIC_SOURCE:
+        roofline["traffic_source"] = TRAFFIC_SOURCE[args.workload]
     print(json.dumps({
         "metric": f"{args.workload}_GBps", "value": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
