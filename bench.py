@@ -48,7 +48,7 @@ _DECODE_TRAFFIC = ("profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md
 _MIXED_TRAFFIC = ("profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
                   "commit bc375af)")
 _MLA_HEADS_TRAFFIC = ("profiles/paged_mla_decode_heads_kernel_h128_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
-                      "kernel as of commit 3b3c0d1)")
+                      "kernel as of commit c8e09ff; the row pitch changed since, the traffic does not depend on it)")
 TRAFFIC_SOURCE = {"mla_decode_h128": _MLA_HEADS_TRAFFIC, "mla_decode_h128_long": _MLA_HEADS_TRAFFIC, "cfg2": _DECODE_TRAFFIC, "cfg2_step": _DECODE_TRAFFIC, "cfg4": _DECODE_TRAFFIC,
                   "cfg4_step": _DECODE_TRAFFIC, "cfg5": _DECODE_TRAFFIC, "cfg3_tile": _MIXED_TRAFFIC,
                   "cfg3_stream": _MIXED_TRAFFIC}
