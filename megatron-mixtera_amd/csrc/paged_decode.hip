@@ -1008,11 +1008,11 @@ __global__ __launch_bounds__(512, 2) void paged_mla_decode_lds_kernel(DecodePara
 // fragment feeds two products) and all 512 output columns (256 accumulator registers), and shares
 // nothing with the others but the staged rows: no score exchange, one barrier per tile.
 // 32-token tiles (37 KB) in four LDS buffers, filled by direct loads from memory (no staging registers, no LDS
-// stores): iteration t requests tile t+2, multiplies the scores of tile t, waits until its own loads of tile t+1
-// have landed, passes the barrier, then softmax and the value product of tile t -- with the first key fragments
-// of tile t+1 requested under its last products.  (Four buffers: tile t+2 replaces tile t-2, which every
-// wavefront left before the barrier of iteration t-1; a wavefront may still be reading values of tile t-1.)
-// The accumulators are never rescaled in that loop (see there).
+// stores): iteration t multiplies the scores of tile t, waits until its own loads of tile t+1 have landed, passes
+// the barrier, then softmax and the value product of tile t -- under whose products it issues, one by one, the
+// loads of tile t+3, and at whose end it requests the first key fragments of tile t+1.  (Four buffers: tile t+3
+// replaces tile t-1, which every wavefront left before the barrier of iteration t; tiles t+1 and t+2 are in LDS
+// or on their way.)  The accumulators are never rescaled in that loop (see there).
 // ---------------------------------------------------------------------------------------------
 constexpr int kMlaHeadsTile = 32;  // tokens per staged tile of the 128-head kernel
 // LDS bytes per staged row: 296 dwords = 40 mod 64, an odd multiple of 8 banks.  A 16-byte fragment read is served in
@@ -1118,7 +1118,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
       const int k = wave + 4 * i;
       if (k < kMlaHeadsLoads) {  // wave-uniform
         const uint32_t m0 = __builtin_amdgcn_readfirstlane(tiles_lds + tile_buf(t) + 1024u * (uint32_t)k);
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(piece_off_i), "s"(src) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0), "v"(piece_off_i), "s"(src) : "memory", "m0");
       }
     };
     // any tile, all of this wavefront's loads at once: rows past the segment's last token re-read that token's row
@@ -1135,7 +1135,7 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
           const uint32_t prow = (u * 14170u) >> 20, pcol = u - 74u * prow;
           const uint8_t* g_src = src + min(prow, row_lim) * tok_bytes + 16u * min(pcol, 71u);
           const uint32_t m0 = __builtin_amdgcn_readfirstlane(dst + 1024u * (uint32_t)k);
-          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(g_src) : "memory");
+          asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(g_src) : "memory", "m0");
           MI_SB();  // one address at a time: the registers are needed elsewhere
         }
       }
