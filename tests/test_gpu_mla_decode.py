@@ -51,7 +51,7 @@ def test_mla_decode_matches_checker(mi, dev, Hq, chunk, kernel_choice):
     assert (out.cpu()[lens == 0] == 0).all()
 
 
-@pytest.mark.parametrize("Hq", [16, 64])
+@pytest.mark.parametrize("Hq", [16, 64, 128])
 def test_mla_decode_long_contexts_and_splits(mi, dev, Hq, kernel_choice):
     """Enough tokens that every request is cut over many workgroups and merged."""
     q, cache, lens, bt = _case(mi, dev, [20000, 4097, 12345, 1], Hq, 64, seed=9)
