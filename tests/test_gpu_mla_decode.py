@@ -113,10 +113,16 @@ def test_mla_decode_more_requests_than_one_launch_takes(mi, dev):
     _check(mi, dev, q, cache, lens, bt, scale=0.07)
 
 
-def test_mla_decode_chunk_permutation_and_cache_view(mi, dev):
-    """Moving the rows to other physical chunks changes nothing; a [N, C, 1, 576] cache view is accepted."""
-    q, cache, lens, bt = _case(mi, dev, [100, 333, 64], 32, 64, seed=4)
+@pytest.mark.parametrize("Hq", [32, 128])
+def test_mla_decode_chunk_permutation_and_cache_view(mi, dev, Hq):
+    """Moving the rows to other physical chunks changes nothing; a [N, C, 1, 576] cache view is accepted; so is a
+    cache that is a slice of a wider buffer (a token stride beyond 576 values)."""
+    q, cache, lens, bt = _case(mi, dev, [100, 333, 64], Hq, 64, seed=4)
     a = mi.ops.paged_mla_decode_attention(q.to(dev), cache.to(dev), lens.to(dev), bt.to(dev), softmax_scale=0.1)
+    wide = torch.zeros(cache.size(0), cache.size(1), 640, dtype=cache.dtype)
+    wide[..., :DK] = cache
+    c = mi.ops.paged_mla_decode_attention(q.to(dev), wide.to(dev)[..., :DK], lens.to(dev), bt.to(dev), softmax_scale=0.1)
+    assert torch.equal(a, c)
     N = cache.size(0)
     perm = torch.randperm(N, generator=torch.Generator().manual_seed(1))
     moved = torch.empty_like(cache)
