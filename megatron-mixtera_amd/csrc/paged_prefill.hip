@@ -357,13 +357,13 @@ __global__ __launch_bounds__(64 * WAVES) void paged_prefill_kernel(PrefillParams
 // permute work; the softmax denominator is accumulated by the matrix cores (an all-ones A fragment), and
 // the cross-lane maximum uses the lane-swap instructions instead of LDS permutes.
 // ---------------------------------------------------------------------------------------------
-// bytes per staged K / V row.  head_dim 128: 288, measured conflict-free for the 16-row x 64-byte fragment
-// reads (272 is not), and 16 rows x 32 B of the transposing reads tile the banks twice; head_dim 64: 144
-// (36 dwords: the 16 rows of a fragment read start at 16 different multiples of four banks).
-// 192-wide keys (multi-latent attention): 416 (104 dwords = 8 x 13: the same bank pattern as 288); head_dim 96:
-// 208 (52 dwords = 4 x 13: the same pattern as 144).
-// head_dim 256: 544 (136 dwords = 8 x 17).
-template <int HD> constexpr int pp_pitch() { return HD == 256 ? 544 : HD == 192 ? 416 : HD == 128 ? 288 : HD == 96 ? 208 : 144; }
+// bytes per staged K / V row: the row width plus padding that makes the pitch an odd multiple of 8 banks (32 bytes).
+// A 16-byte fragment read is served in passes of {rows 0-7 at piece g, rows 8-15 at piece g + 1}, a transposing
+// 8-byte read in passes of eight rows; both cover the 64 banks exactly once at such a pitch (288 = 8 x 9 dwords
+// reads 0 conflict cycles by counter; 4 x odd dwords -- 144 or 208, as head_dim 64 and 96 once had -- costs a
+// fragment read 4 cycles on top of its 4 and a transposing read 2 on top of its 2).
+// head_dim 64: 160 (8 x 5 dwords), 96: 224 (8 x 7), 128: 288, 192-wide keys: 416 (8 x 13), 256: 544 (8 x 17).
+template <int HD> constexpr int pp_pitch() { return HD == 256 ? 544 : HD == 192 ? 416 : HD == 128 ? 288 : HD == 96 ? 224 : 160; }
 // keys per staged tile: 64; 32 at head_dim 256, where five 64-key buffers would not fit the 160 KB of LDS
 template <int HD> constexpr int pp_tile() { return HD == 256 ? 32 : 64; }
 
