@@ -1320,7 +1320,25 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
           for (int e = 0; e < VB; ++e) {
             const uint4 a = make_uint4(vf[j & 1][e][0].x, vf[j & 1][e][0].y, vf[j & 1][e][1].x, vf[j & 1][e][1].y);
 #pragma unroll
-            for (int h2 = 0; h2 < 2; ++h2) acc[h2][VB * j + e] = mfma_16x16x32<F16>(a, pp[h2], acc[h2][VB * j + e]);
+            for (int h2 = 0; h2 < 2; ++h2) {
+              if (VB * j + e >= NE - 3) {
+                // The compiler gives every matrix product of the kernel its result in accumulation registers; 256 sums
+                // + 16 scores + 8 row sums are 280 of the 256 there are, so it keeps 24 sums in vector registers and
+                // moves them in and out around their products (108 moves per tile).  These six tiles are therefore
+                // multiplied in the vector-register form, by hand: their registers are touched by nothing else in the
+                // loop (next by the same product one tile later, then by the epilogue), the fragment operands come
+                // from LDS reads the compiler waits for, and the probabilities were written many instructions ago
+                // (the s_nop covers the two wait states a vector write needs before a product reads it).
+                typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+                const u32x4_t av = {a.x, a.y, a.z, a.w}, bv = {pp[h2].x, pp[h2].y, pp[h2].z, pp[h2].w};
+                if constexpr (F16)
+                  asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[h2][VB * j + e]) : "v"(av), "v"(bv));
+                else
+                  asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[h2][VB * j + e]) : "v"(av), "v"(bv));
+              } else {
+                acc[h2][VB * j + e] = mfma_16x16x32<F16>(a, pp[h2], acc[h2][VB * j + e]);
+              }
+            }
           }
           if (j < (kMlaHeadsLoads + 3) / 4 && piecewise) fetch_piece(t + 3, src_ahead, j, piece_off[j]);
           if (j == 0) {
