@@ -1349,6 +1349,9 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
           MI_SB();
         }
       }
+      // (the hand-written products above are not known to the compiler as such: the wait states a vector instruction
+      // needs before it reads a matrix result, spelled out)
+      asm volatile("s_nop 15\n\ts_nop 7" ::: "memory");
       // ---- the sums leave the registers: acc[h2][e][i] is output column 16 e + 4 g + i of head hq0 + 16 h2.
       // The segment's result when every tile is done; otherwise as they are, for the loop below ---------
       const bool done = t >= ntile;
