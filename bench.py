@@ -258,7 +258,7 @@ def run_cu_probes(args, mi, torch, dev):
     blib = ctypes.CDLL(str(path))
     P, I = ctypes.c_void_p, ctypes.c_int32
     blib.mi_bench_read_probe.restype = ctypes.c_int
-    blib.mi_bench_read_probe.argtypes = [I, I, I, I, P, P, P, P]
+    blib.mi_bench_read_probe.argtypes = [I, I, I, I, I, P, P, P, P]
     blib.mi_bench_coexec_probe.restype = ctypes.c_int
     blib.mi_bench_coexec_probe.argtypes = [I, I, I, I, P, P, P]
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
@@ -270,14 +270,16 @@ def run_cu_probes(args, mi, torch, dev):
     reads = {}
     iters = 2000
     for mode, name in ((0, "lds_b128"), (1, "lds_tr_b64"), (2, "global_b128_l1_resident")):
-        for waves in (1, 4, 8, 16):
-            for _ in range(2):
-                assert blib.mi_bench_read_probe(mode, waves, cus, iters, cyc.data_ptr(), sink.data_ptr(), gsrc.data_ptr(), stream) == 0
-            torch.cuda.synchronize()
-            worst = int(cyc[:waves].max())
-            nbytes = iters * 16 * 1024 * waves
-            reads[f"{name}_{waves}_waves"] = {"bytes_per_clk_per_cu": round(nbytes / worst, 1),
-                                              "bytes_per_clk_per_wave": round(nbytes / worst / waves, 2)}
+        for depth in (1, 4, 16):   # fragments a wavefront has in flight before it waits for the first
+            for waves in (1, 4, 8, 16):
+                for _ in range(2):
+                    assert blib.mi_bench_read_probe(mode, depth, waves, cus, iters, cyc.data_ptr(), sink.data_ptr(),
+                                                    gsrc.data_ptr(), stream) == 0
+                torch.cuda.synchronize()
+                worst = int(cyc[:waves].max())
+                nbytes = iters * 16 * 1024 * waves
+                reads[f"{name}_{depth}_in_flight_{waves}_waves"] = {"bytes_per_clk_per_cu": round(nbytes / worst, 1),
+                                                                    "bytes_per_clk_per_wave": round(nbytes / worst / waves, 2)}
     names = {0: "idle", 1: "mfma_16x16x32", 2: "mfma_32x32x16", 3: "fma", 4: "exp2"}
     per_iter = {1: 32, 2: 16, 3: 32, 4: 32}
     coexec = {}
@@ -293,15 +295,37 @@ def run_cu_probes(args, mi, torch, dev):
                 entry["b_clk_per_instr"] = round(c[4] / (iters * per_iter[b]), 2)
             entry["core_clock_mhz"] = round(c[0] / max(c[8], 1) * 100)
             coexec[f"{names[a]}+{names[b]}" + ("_all_cus" if wgs > 1 else "_one_cu")] = entry
+    blib.mi_bench_woven_probe.restype = ctypes.c_int
+    blib.mi_bench_woven_probe.argtypes = [I, I, I, I, P, P, P]
+    woven = {}
+    iters = 2000
+    for rows in (64, 32):
+        for weave, name in ((1, "woven"), (0, "vector_work_after_the_products")):
+            for wgs in (1, cus):
+                for _ in range(2):
+                    assert blib.mi_bench_woven_probe(rows, weave, wgs, iters, cyc.data_ptr(), sink.data_ptr(), stream) == 0
+                torch.cuda.synchronize()
+                c = cyc.tolist()
+                clk = max(c[:256 // rows]) / iters   # every wavefront of the workgroup does `iters` tiles
+                # a 16x16x32 product occupies a SIMD's matrix core for 16 clocks (mfma_16x16x32+idle above);
+                # a SIMD's wavefronts together issue 128 of them per `clk`
+                woven[f"{rows}_rows_per_wavefront_{name}" + ("_all_cus" if wgs > 1 else "_one_cu")] = {
+                    "clk_per_tile": round(clk, 1), "matrix_core_busy": round(128 * 16 / clk, 3),
+                    "core_clock_mhz": round(c[0] / max(c[8], 1) * 100)}
     elapsed = time.perf_counter() - t0
     print(json.dumps({
-        "metric": "cu_probes", "value": reads["lds_b128_16_waves"]["bytes_per_clk_per_cu"], "unit": "LDS B/clk/CU",
+        "metric": "cu_probes", "value": reads["lds_b128_16_in_flight_16_waves"]["bytes_per_clk_per_cu"], "unit": "LDS B/clk/CU",
         "n_gpus": 1, "steps": 1, "warmup": 0, "ms_per_step": round(elapsed * 1e3, 1), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u8 / bf16 / f32", "data": "synthetic",
         "config": {"workload": "probes of one compute unit: fragment reads from LDS and through the vector L1 "
                                "(bytes per core clock), matrix / vector co-execution of two wavefronts of a SIMD "
                                "(core clocks per instruction; a = wavefronts 0-3, b = wavefronts 4-7), core clock"},
-        "reads": reads, "coexec": coexec}), flush=True)
+        "reads": reads, "coexec": coexec,
+        "attention_tile_in_one_instruction_stream": {
+            "what": "64 keys x 128 values x (64 query rows per wavefront, one wavefront a SIMD | 32 rows, two a SIMD): "
+                    "per SIMD and tile 128 products 16x16x32, the key / value fragment reads and the softmax's vector "
+                    "arithmetic in one instruction stream per wavefront",
+            **woven}}), flush=True)
 
 
 def parse_args():
