@@ -466,11 +466,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       qf[nt][kk] = valid ? ld16(qrow + 32 * kk + 8 * g) : make_uint4(0, 0, 0, 0);
   }
 
-  float m_run[NQ];
+  float m_run[NQ], neg_run[NQ];
   f32x4_t acc[NQ][DV], accl[NQ];
 #pragma unroll
   for (int nt = 0; nt < NQ; ++nt) {
     m_run[nt] = -INFINITY;
+    neg_run[nt] = 0.f;
     accl[nt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int e = 0; e < DV; ++e) acc[nt][e] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -629,6 +630,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     };
 
     const float scale = p.scale_log2;
+    const float win = (F16 ? 8.f : 30.f) / scale;  // probabilities stay below 2^8 (fp16 operands) or 2^30
     const uint4 ones = make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
     f32x4_t s[NQ][NT];
     uint2 pf[NQ][NT];
@@ -847,12 +849,25 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         } else {
           tmax = fmaxf(tmax, s[nt][1][3]);
         }
-        tmax = rowgroup_max(tmax);
-        const float m_raw = fmaxf(m_run[nt], tmax);
-        const float m_use = m_raw == -INFINITY ? 0.f : m_raw;
-        const float alpha = fast_exp2((m_run[nt] - m_use) * scale);
-        const float neg = -m_use * scale;
-        m_run[nt] = m_raw;
+        // The reference the exponentials are taken against moves only when a score of this lane exceeds it by a
+        // window (2^kWin as the largest probability): the exchange within the row group, the rescale factor and
+        // the rescale are then rare instead of once per tile.
+        if (__builtin_amdgcn_ballot_w64(tmax > m_run[nt] + win)) {
+          tmax = rowgroup_max(tmax);
+          const float m_raw = fmaxf(m_run[nt], tmax);
+          const float m_use = m_raw == -INFINITY ? 0.f : m_raw;
+          const float alpha = fast_exp2((m_run[nt] - m_use) * scale);
+          neg_run[nt] = -m_use * scale;
+          m_run[nt] = m_raw;
+          if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+            for (int e = 0; e < DV; ++e) {
+              acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
+            }
+            accl[nt][0] *= alpha; accl[nt][1] *= alpha; accl[nt][2] *= alpha; accl[nt][3] *= alpha;
+          }
+        }
+        const float neg = neg_run[nt];
 #pragma unroll
         for (int u = 0; u < NT; ++u) {
           const float p0 = fast_exp2(__builtin_fmaf(s[nt][u][0], scale, neg));
@@ -860,13 +875,6 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
           const float p2 = fast_exp2(__builtin_fmaf(s[nt][u][2], scale, neg));
           const float p3 = fast_exp2(__builtin_fmaf(s[nt][u][3], scale, neg));
           pf[nt][u] = make_uint2(pack2<F16>(p0, p1), pack2<F16>(p2, p3));
-        }
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
-#pragma unroll
-          for (int e = 0; e < DV; ++e) {
-            acc[nt][e][0] *= alpha; acc[nt][e][1] *= alpha; acc[nt][e][2] *= alpha; acc[nt][e][3] *= alpha;
-          }
-          accl[nt][0] *= alpha; accl[nt][1] *= alpha; accl[nt][2] *= alpha; accl[nt][3] *= alpha;
         }
       }
     };

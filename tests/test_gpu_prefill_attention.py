@@ -141,6 +141,26 @@ def test_head_widths_96_192_256(mi, dev, d, Hq, Hkv, chunk, dtype):
                 _check_padded(mi, q, kc, vc, cu_q, lens, bt)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("kernel", ["two_phase", "registers", "split_keys"])
+@pytest.mark.parametrize("d", [64, 96, 128, 192, 256])
+def test_scores_that_keep_growing_along_the_context(mi, dev, d, kernel, dtype):
+    """Keys grow with their position (x52 at token 1 020), so a row's largest score moves up by far more than any
+    window a kernel takes its exponentials within (2^8 for fp16 operands, 2^30 for bf16), tile after tile; rows
+    whose query points the other way see it fall instead."""
+    knobs = {"two_phase": {}, "registers": {"prefill_two_phase": -1}, "split_keys": {"prefill_kv_split": 3}}[kernel]
+    chunk = 64
+    q, kc, vc, cu_q, lens, bt = _ragged_case(mi, dev, 16, 4, d, chunk, dtype, seed=700 + d)
+    pos = torch.arange(chunk, device=dev)
+    kf = kc.float()
+    for r in range(bt.size(0)):
+        for ci in range((int(lens[r]) + chunk - 1) // chunk):
+            kf[int(bt[r, ci])] *= (1 + 0.05 * (ci * chunk + pos)).view(-1, 1, 1)
+    kc = kf.to(dtype)
+    with mi.ops.tuning(**knobs):
+        _check(mi, q, kc, vc, cu_q, lens, bt)
+
+
 @pytest.mark.parametrize("kernel", ["two_phase", "registers", "split_keys"])
 @pytest.mark.parametrize("Hq,Hkv", [(32, 1), (64, 2), (17, 1), (48, 2), (40, 2), (64, 1)])
 @pytest.mark.parametrize("d", [64, 96, 128, 192, 256])
