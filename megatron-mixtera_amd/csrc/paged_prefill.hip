@@ -829,9 +829,13 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
 #pragma unroll
       for (int nt = 0; nt < NQ; ++nt) {
         if (need_mask) {
+          int Tm = T;
+          // keeps the token positions below out of the tiles that need no mask (the 192-wide keys of the
+          // multi-latent form have no register to spare for it)
+          if constexpr (!MLA) asm volatile("" : "+s"(Tm));
 #pragma unroll
           for (int u = 0; u < NT; ++u) {
-            const int tok0 = T + 16 * u + 4 * g;
+            const int tok0 = Tm + 16 * u + 4 * g;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
               if (tok0 + i > qpos[nt]) s[nt][u][i] = -INFINITY;
