@@ -702,11 +702,15 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // The whole matrix phase of iteration it: O^T += V^T P^T of tile it-1, S^T = K Q^T of tile it,
     // and -- spread over the first MFMA groups, whose shadow hides the address arithmetic --
     // the staging: store K(it+1) and V(it+1) (fetched during the previous matrix phase) into
-    // LDS, then fetch K(it+2) and V(it+2).  (Reading fragments ahead during the vector phase, or
-    // moving score groups there, was measured slower: a wave sustains only ~32 B/clk of LDS reads
-    // and the vector phase has no issue slots to spare.)
+    // LDS, then fetch K(it+2) and V(it+2).  (Moving score groups to the vector phase was measured
+    // slower; so was reading more than one group of fragments ahead there: the registers run out.)
     Cursor cur = cursor_at(tb + 2);  // the tile fetched during iteration 0
     int pc_cur = 0;             // its block-table entry (a per-lane copy, made scalar at its use)
+    // Head width 128, whose matrix phase is the longer one: the fragments of its first value group are requested at
+    // the end of the vector phase before it (their tile was staged two phases earlier) and waited for at that
+    // phase's barrier, so the matrix phase starts on loaded registers instead of on an LDS round trip.
+    constexpr bool kAhead = !WIDE && !MLA && HD == 128;
+    uint2 a_first[4][2];
     auto matrix_phase = [&](int it) {
       uint2 a0[4][2], a1[4][2];
       uint4 k0[KS], k1[KS];
@@ -777,9 +781,9 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         sc_mma(3, k1);
         return;
       }
-      pv_load(ta, 0, a0);
+      if constexpr (!kAhead) pv_load(ta, 0, a_first);
       pv_load(ta, 1, a1); MI_SB();
-      pv_mma(0, a0);
+      pv_mma(0, a_first);
       store_k(it + 1);
       store_v(it + 1); MI_SB();
       pv_load(ta, 2, a0); MI_SB();
@@ -881,6 +885,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
           pf[nt][u] = make_uint2(pack2<F16>(p0, p1), pack2<F16>(p2, p3));
         }
       }
+      if constexpr (kAhead) pv_load(t, 0, a_first);  // for the matrix phase of iteration t + 1
     };
     // Staging rides in the matrix phase (LDS-write and memory ports are idle there).  Phase
     // numbers: group 0 runs matrix(it) in phase 2it and vector(it) in 2it+1, group 1 one phase
@@ -915,6 +920,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
     // wave whose rows cannot see a tile would only wait at the barriers instead; its scores there
     // are all masked, p = 0).  Iteration 0 "accumulates" tile -1: zero probabilities times a
     // zero-filled V buffer; iteration ntl computes scores of a stale K buffer that nobody uses.
+    if constexpr (kAhead) pv_load(-1, 0, a_first);
     for (int it = 0; it <= ntl; ++it) {
       // (scheduling barriers: MFMAs touch no memory, so nothing else stops the compiler from
       // sinking them past the workgroup barrier into the other phase)
