@@ -819,6 +819,23 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
         sc_mma_half(3, 1, h1);
         return;
       }
+      if constexpr (kAhead) {
+        // the next group's four key fragments requested one by one between this group's products, not in a burst:
+        // the four wavefronts in this phase run in step and would otherwise queue at the LDS together
+        auto weave = [&]() {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);  // two MFMAs
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+          }
+        };
+        sc_load(ts, 0, k0); pv_mma(3, a1); weave(); MI_SB();
+        sc_load(ts, 1, k1); sc_mma(0, k0); weave(); MI_SB();
+        sc_load(ts, 2, k0); sc_mma(1, k1); weave(); MI_SB();
+        sc_load(ts, 3, k1); sc_mma(2, k0); weave(); MI_SB();
+        sc_mma(3, k1);
+        return;
+      }
       sc_load(ts, 0, k0); MI_SB();
       pv_mma(3, a1); MI_SB();
       sc_load(ts, 1, k1); MI_SB(); sc_mma(0, k0); MI_SB();
