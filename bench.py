@@ -300,7 +300,7 @@ def run_cu_probes(args, mi, torch, dev):
     woven = {}
     iters = 2000
     for rows in (64, 32):
-        for weave, name in ((1, "woven"), (0, "vector_work_after_the_products")):
+        for weave, name in ((1, "woven"), (0, "vector_work_after_the_products"), (2, "woven_fma_and_exponential_only")):
             for wgs in (1, cus):
                 for _ in range(2):
                     assert blib.mi_bench_woven_probe(rows, weave, wgs, iters, cyc.data_ptr(), sink.data_ptr(), stream) == 0

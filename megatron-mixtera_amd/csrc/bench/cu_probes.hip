@@ -156,7 +156,9 @@ static __device__ __forceinline__ uint2 lds_tr(const uint8_t* p) {
 // products 16x16x32; ROWS exponentials per lane with their max / fma / sum; scores out of, probabilities into, the
 // product operands.  ROWS 64: four wavefronts a workgroup, the SIMD's whole register file each; ROWS 32: eight.
 // WEAVE: vector work between the matrix instructions (true) or all of it after them (false).
-template <int ROWS, bool WEAVE>
+// LEAN: per score only fma + exponential (+ pack): no running maximum, no sum (a kernel that takes its exponentials
+// against a fixed reference and lets the matrix cores add the denominators).
+template <int ROWS, bool WEAVE, bool LEAN>
 __global__ __launch_bounds__(ROWS == 64 ? 256 : 512, 1) void woven_probe(long long* cycles, float* sink, int iters) {
   constexpr int R16 = ROWS / 16, kGroups = 16 * R16;
   __shared__ __attribute__((aligned(16))) uint8_t lds[2][64 * kPitch];  // a key and a value tile (contents do not matter)
@@ -211,9 +213,9 @@ __global__ __launch_bounds__(ROWS == 64 ? 256 : 512, 1) void woven_probe(long lo
       acc_o[grp % (8 * R16)] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
           __builtin_bit_cast(bf16x8_t, vf[f & 3]), __builtin_bit_cast(bf16x8_t, pr[grp % (2 * R16)]), acc_o[grp % (8 * R16)], 0, 0, 0);
       if (WEAVE) {  // the softmax arithmetic of one score of the previous tile
-        mx = fmaxf(mx, sprev[grp]);
+        if (!LEAN) mx = fmaxf(mx, sprev[grp]);
         const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sprev[grp], scale, -mx));
-        sum += e;
+        if (!LEAN) sum += e;
         e_keep[grp] = e;
       }
       SB();
@@ -260,16 +262,18 @@ __global__ __launch_bounds__(ROWS == 64 ? 256 : 512, 1) void woven_probe(long lo
 }  // namespace
 
 // rows 64: four wavefronts a workgroup, 128 matrix instructions per wavefront and tile; rows 32: eight wavefronts, 64 each.
-// `weave` 1: vector work between the matrix instructions, 0: after them.  cycles_out (device, int64 [16]): [w] core
+// `weave` 1: vector work between the matrix instructions, 0: after them, 2: between them and only fma + exponential per score.  cycles_out (device, int64 [16]): [w] core
 // clocks of wavefront w (< 8) of workgroup 0, [8 + w] its wall-clock ticks.  sink: device, workgroups * 512 floats.
 extern "C" int mi_bench_woven_probe(int32_t rows, int32_t weave, int32_t workgroups, int32_t iters, long long* cycles_out,
                                     float* sink, void* stream) {
   if (!cycles_out || !sink || workgroups < 1 || iters < 1 || (rows != 32 && rows != 64)) return -1;
   hipStream_t st = (hipStream_t)stream;
-  if (rows == 64 && weave) hipLaunchKernelGGL((woven_probe<64, true>), dim3(workgroups), dim3(256), 0, st, cycles_out, sink, iters);
-  else if (rows == 64) hipLaunchKernelGGL((woven_probe<64, false>), dim3(workgroups), dim3(256), 0, st, cycles_out, sink, iters);
-  else if (weave) hipLaunchKernelGGL((woven_probe<32, true>), dim3(workgroups), dim3(512), 0, st, cycles_out, sink, iters);
-  else hipLaunchKernelGGL((woven_probe<32, false>), dim3(workgroups), dim3(512), 0, st, cycles_out, sink, iters);
+  if (rows == 64 && weave == 2) hipLaunchKernelGGL((woven_probe<64, true, true>), dim3(workgroups), dim3(256), 0, st, cycles_out, sink, iters);
+  else if (rows == 64 && weave) hipLaunchKernelGGL((woven_probe<64, true, false>), dim3(workgroups), dim3(256), 0, st, cycles_out, sink, iters);
+  else if (rows == 64) hipLaunchKernelGGL((woven_probe<64, false, false>), dim3(workgroups), dim3(256), 0, st, cycles_out, sink, iters);
+  else if (weave == 2) hipLaunchKernelGGL((woven_probe<32, true, true>), dim3(workgroups), dim3(512), 0, st, cycles_out, sink, iters);
+  else if (weave) hipLaunchKernelGGL((woven_probe<32, true, false>), dim3(workgroups), dim3(512), 0, st, cycles_out, sink, iters);
+  else hipLaunchKernelGGL((woven_probe<32, false, false>), dim3(workgroups), dim3(512), 0, st, cycles_out, sink, iters);
   return hipGetLastError() == hipSuccess ? 0 : -2;
 }
 
