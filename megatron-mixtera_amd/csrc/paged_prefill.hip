@@ -355,7 +355,9 @@ __global__ __launch_bounds__(64 * WAVES) void paged_prefill_kernel(PrefillParams
 //
 // V fragments come out of LDS already transposed (ds_read_b64_tr_b16, 288-byte V pitch), so there is no
 // permute work; the softmax denominator is accumulated by the matrix cores (an all-ones A fragment), and
-// the cross-lane maximum uses the lane-swap instructions instead of LDS permutes.
+// the cross-lane maximum uses the lane-swap instructions instead of LDS permutes -- and is taken only when
+// some score of a tile exceeds the reference of its row by a window (2^30 as the largest probability with bf16
+// operands, 2^8 with fp16 ones): the exponentials are taken against a reference that rarely moves.
 // ---------------------------------------------------------------------------------------------
 // bytes per staged K / V row: the row width plus padding that makes the pitch an odd multiple of 8 banks (32 bytes).
 // A 16-byte fragment read is served in passes of {rows 0-7 at piece g, rows 8-15 at piece g + 1}, a transposing
@@ -843,7 +845,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       sc_load(ts, 3, k1); MI_SB(); sc_mma(2, k0); MI_SB();
       sc_mma(3, k1);
     };
-    // ---- online softmax of tile t: s -> pf, rescale of the accumulators when a maximum moved ----
+    // ---- online softmax of tile t: s -> pf, rescale of the accumulators when the reference moved ----
     auto softmax = [&](int t) {  // t counts from this workgroup's first tile
       const int T = (tb + t) * kPPTile;
       const bool need_mask = T + kPPTile - 1 > full_until;
