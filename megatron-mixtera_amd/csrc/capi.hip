@@ -42,9 +42,9 @@ int mi_resolve_tuning(const MiTuning* given, MiTuning* out, const char* who) {
   if (t.decode_grid < 0 || t.decode_grid > 65535) return bad("decode_grid must be 0 (automatic) or 1..65535");
   if (t.decode_waves_per_block == 0) t.decode_waves_per_block = 8;
   if (t.decode_waves_per_block < 1 || t.decode_waves_per_block > 8) return bad("decode_waves_per_block must be 0 (default) or 1..8");
-  if (t.prefill_two_phase == 0) t.prefill_two_phase = 1;
-  if (t.prefill_two_phase != 1 && t.prefill_two_phase != 2 && t.prefill_two_phase != -1)
-    return bad("prefill_two_phase must be 0 (default), 1, 2 or -1 (register-only kernel)");
+  if (t.prefill_two_phase == 0) t.prefill_two_phase = 3;
+  if (t.prefill_two_phase != 1 && t.prefill_two_phase != 2 && t.prefill_two_phase != 3 && t.prefill_two_phase != -1)
+    return bad("prefill_two_phase must be 0 (default), 1, 2, 3 (one-stream tile kernel) or -1 (register-only kernel)");
   if (t.prefill_tile_subtiles == 0) t.prefill_tile_subtiles = 2;
   if (t.prefill_tile_subtiles != 1 && t.prefill_tile_subtiles != 2) return bad("prefill_tile_subtiles must be 0 (default), 1 or 2");
   if (t.prefill_row_tiles == 0) t.prefill_row_tiles = 2;

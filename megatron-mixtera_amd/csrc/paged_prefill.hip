@@ -17,59 +17,9 @@
 // (request, KV head), so they pull identical K/V lines at about the same time.
 #include "mi_common.h"
 #include "mi_capi_internal.h"
+#include "paged_prefill_params.h"
 
 namespace mi {
-
-struct PrefillParams {
-  const uint16_t* q;
-  int64_t q_st, q_sh;
-  const uint8_t* kc;
-  const uint8_t* vc;
-  int64_t kv_sc;
-  int32_t kv_st, kv_sh;
-  int64_t v_sc;          // value cache strides (register-only kernel; equal to the key cache's otherwise)
-  int32_t v_st, v_sh;
-  const int32_t* bt;
-  int64_t bt_stride;
-  const int32_t* cu_q;
-  const int32_t* lens;
-  uint16_t* out;
-  int64_t o_st, o_sh;
-  uint64_t chunk_magic;  // ceil(2^40 / chunk)
-  int32_t T, R, Hq, Hkv, G, g_magic, chunk;  // g_magic = 65536 / G + 1: (n * g_magic) >> 16 == n / G for n <= 64, G <= 16
-  int32_t parts;         // workgroups per KV head along the query heads: each takes up to 16 of the G that share it
-  int32_t skip_single;  // requests with exactly one query row are handled by the decode kernels
-  float scale_log2;
-  const float* k_scale;  // fp8 KV only: [n_chunks][Hkv]
-  const float* v_scale;
-  // Two-phase tile kernel only: the keys of a request cut into gridDim.y ranges, one workgroup each;
-  // with more than one range the workgroups write fp32 partials [range][T][Hq][128] and their
-  // log-sum-exps [range][T][Hq] (log2 domain) and a merge kernel finishes the rows.
-  float* split_o;
-  float* split_lse;
-};
-
-// The query heads one workgroup serves: with at most 16 query heads per KV head, all G of KV head `hv`; with more,
-// `parts` workgroups share a KV head and take 16 query heads each (the last one the rest).
-struct HeadSlice {
-  int h;        // KV head
-  int hq0;      // first query head
-  int G;        // query heads (1..16)
-  int g_magic;  // 65536 / G + 1
-};
-static __device__ __forceinline__ HeadSlice head_slice(const PrefillParams& p, int hv) {
-  HeadSlice s;
-  if (p.parts <= 1) {
-    s.h = hv; s.hq0 = hv * p.G; s.G = p.G; s.g_magic = p.g_magic;
-  } else {
-    s.h = hv / p.parts;
-    const int part = hv - s.h * p.parts;
-    s.hq0 = s.h * p.G + 16 * part;
-    s.G = min(16, p.G - 16 * part);
-    s.g_magic = 65536 / s.G + 1;
-  }
-  return s;
-}
 
 // NQ = 16-row tiles per wave, WAVES wavefronts per workgroup (256 rows for the narrow heads, 128 at width 256).
 // HDK = width of queries and keys, HDV = width of values and of the output (they differ for the
@@ -1148,7 +1098,7 @@ static int launch_paged_prefill(
     hipEvent_t ev_a, ev_b;
     const bool timed = mi_profile_next(&ev_a, &ev_b);
     if (timed) (void)hipEventRecord(ev_a, st);
-    const bool stagger = tune.prefill_two_phase == 1;
+    const bool stagger = tune.prefill_two_phase != 2;
     // key ranges per request (with a workspace only): partials behind the decode part's scratch
     int n_split = 1;
     if (workspace) {
@@ -1164,7 +1114,9 @@ static int launch_paged_prefill(
         workspace_bytes = dec_bytes;
       }
     }
-    if (fp8) MI_PP_LAUNCH(true, 128, 128, false);
+    // head_dim 128 over a 16-bit cache: the one-stream tile kernel when asked for
+    if (!fp8 && head_dim == 128 && tune.prefill_two_phase == 3) launch_prefill_woven(p, lgrid, f16, st);
+    else if (fp8) MI_PP_LAUNCH(true, 128, 128, false);
     else if (head_dim == 128 && f16) MI_PP_LAUNCH(false, 128, 128, true);
     else if (head_dim == 128) MI_PP_LAUNCH(false, 128, 128, false);
     else if (head_dim == 64 && f16) MI_PP_LAUNCH(false, 64, 64, true);
@@ -1311,7 +1263,7 @@ extern "C" int mi_paged_prefill_attention_mla(
   int n_split = 1;
   if (two_phase) {
     dim3 lgrid(((T + sbq - 1) / sbq + R) * Hkv * parts);
-    const bool stagger = tune.prefill_two_phase == 1;
+    const bool stagger = tune.prefill_two_phase != 2;
     // few query rows over long contexts: key ranges per request, partials in the workspace (which holds
     // nothing else here: one-row requests stay in the tile kernel)
     if (workspace) {
