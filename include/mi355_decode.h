@@ -66,8 +66,9 @@ typedef struct MiTuning {
   int32_t decode_wgs_per_cu;      /* decode kernel, workgroups of 8 wavefronts per CU: 0 = default (1), 1..8 */
   int32_t decode_grid;            /* decode kernels, spans the tile sequence is cut into: 0 = automatic, 1..65535 */
   int32_t decode_waves_per_block; /* decode kernel, KV heads per workgroup: 0 = default (8), 1..8 */
-  int32_t prefill_two_phase;      /* prefill: 0 = default (1), 1 = two-phase tile kernel, 2 = the same with its
-                                     wave groups in lock-step, -1 = register-only kernel */
+  int32_t prefill_two_phase;      /* prefill tile kernel: 0 = default (3), 1 = two-phase kernel, 2 = the same with its
+                                     wave groups in lock-step, 3 = one-stream kernel where it applies (head_dim 128 over a
+                                     16-bit cache; the two-phase kernel elsewhere), -1 = register-only kernel */
   int32_t prefill_tile_subtiles;  /* register-only prefill kernel, 16-key sub-tiles per iteration: 0 = default (2), 1, 2 */
   int32_t prefill_row_tiles;      /* register-only prefill kernel, 16-row tiles per wavefront: 0 = default (2), 2, 4 */
   int32_t prefill_kv_split;       /* two-phase kernel, key ranges per request: 0 = from T and max_kv_len, -1 = never,

@@ -40,19 +40,26 @@ constexpr int kWvPitch = 288;                    // LDS bytes per staged row (25
 constexpr int kWvPieces = kWvPitch / 16;         // 16-byte pieces per staged row
 constexpr int kWvLoads = kWvTile * kWvPieces / 64;  // direct loads (64 lanes x 16 bytes) per tile: 18
 constexpr int kWvBuf = kWvLoads * 1024;          // bytes per tile buffer
+constexpr int kWvDepth = 1;                      // tiles between the issue of a tile's loads and the barrier that needs them
+constexpr int kWvAhead = 3;                      // fragments requested ahead of their products (the stream: 16 per 32-key slot)
+constexpr int kWvRing = 4;                       // fragment registers: fragment n lives in slot n % kWvRing
+static_assert(kWvAhead < kWvRing && kWvAhead <= 8 && 16 % kWvRing == 0, "next slot's key fragments are requested after the tile's barrier");
 constexpr bool wv_piece_division_ok() {
   for (unsigned u = 0; u < 64u * kWvLoads; ++u)
     if (((u * 3641u) >> 16) != u / 18u) return false;
   return true;
 }
-static_assert(kWvPieces == 18 && kWvBuf == kWvTile * kWvPitch && wv_piece_division_ok(), "piece -> (row, column) by multiplication");
+static_assert((kWvDepth == 1 || kWvDepth == 2) && kWvPieces == 18 && kWvBuf == kWvTile * kWvPitch && wv_piece_division_ok(), "piece -> (row, column) by multiplication");
 
 template <bool SPLIT, bool F16>
 __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillParams p) {
   constexpr int HD = 128, KS = HD / 32, DV = HD / 16, NQ = 2, WAVES = 8;
   constexpr int PITCH = kWvPitch, BUF = kWvBuf;
-  __shared__ __attribute__((aligned(16))) uint8_t Ks[2][BUF];
-  __shared__ __attribute__((aligned(16))) uint8_t Vs[3][BUF];
+  // DEPTH: how many tiles ahead of their barrier the loads of a tile pair are issued.  Key tile t lives in
+  // Ks[t % KBUFS], value tile t in Vs[(t + 1) % VBUFS] (values are multiplied one tile after their keys).
+  constexpr int DEPTH = kWvDepth, KBUFS = DEPTH + 1, VBUFS = DEPTH + 2;
+  __shared__ __attribute__((aligned(16))) uint8_t Ks[KBUFS][BUF];
+  __shared__ __attribute__((aligned(16))) uint8_t Vs[VBUFS][BUF];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -211,7 +218,8 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
     // S[x]: scores of the even (x = 0) / odd (x = 1) 32-key steps, P[x]: their probabilities as the B operand
     f32x4_t S[2][NQ][2];
     uint4 P[2][NQ];
-    uint4 fr[4];  // fragments in flight: fragment n of the stream lives in fr[n & 3]
+    constexpr int AHEAD = kWvAhead, RING = kWvRing;
+    uint4 fr[RING];  // fragments in flight: fragment n of the stream lives in fr[n % RING]
 #pragma unroll
     for (int nt = 0; nt < NQ; ++nt) {
       P[0][nt] = P[1][nt] = make_uint4(0u, 0u, 0u, 0u);
@@ -270,26 +278,42 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
       const f32x4_t (&Sx)[NQ][2] = S[1 - H];
       uint4 (&Px)[NQ] = P[1 - H];
       const uint4 (&Pv)[NQ] = P[H];
-      // fragment n of the slot's stream: 0-7 key fragments, 8-15 value fragments, 16-18 the next slot's first keys
+      // fragment n of the slot's stream: 0-7 key fragments, 8-15 value fragments, from 16 the next slot's first keys
       auto request = [&](int n) {
-        if (n < 8) fr[n & 3] = read_k(ka, H, n);
-        else if (n < 16) fr[n & 3] = read_v(va, H, n - 8);
-        else fr[n & 3] = H == 0 ? read_k(ka, 1, n - 16) : read_k(ka_next, 0, n - 16);
+        if (n < 8) fr[n % RING] = read_k(ka, H, n);
+        else if (n < 16) fr[n % RING] = read_v(va, H, n - 8);
+        else fr[n % RING] = H == 0 ? read_k(ka, 1, n - 16) : read_k(ka_next, 0, n - 16);
+      };
+      // The probabilities of S[1-H], two scores ("chunk") at a time in three stages -- scale and subtract, exponential,
+      // pack -- one stage of three different chunks per position, so that no instruction waits for the one before it:
+      // position n holds stage one of chunk n, stage two of chunk n - 1, stage three of chunk n - 2.
+      float xs[8][2], ps[8][2];
+      auto exp_stages = [&](int n) {
+        if (n >= 2 && n < 10) {
+          const int c = n - 2, nt = c >> 2, d = 2 * ((c >> 1) & 1) + (c & 1);
+          const uint32_t w = pack2<F16>(ps[c][0], ps[c][1]);
+          if (d == 0) Px[nt].x = w; else if (d == 1) Px[nt].y = w; else if (d == 2) Px[nt].z = w; else Px[nt].w = w;
+        }
+        if (n >= 1 && n < 9) {
+          ps[n - 1][0] = fast_exp2(xs[n - 1][0]);
+          ps[n - 1][1] = fast_exp2(xs[n - 1][1]);
+        }
+        if (n < 8) {
+          const int nt = n >> 2, u = (n >> 1) & 1, q2 = 2 * (n & 1);
+          xs[n][0] = __builtin_fmaf(Sx[nt][u][q2], scale, neg_run[nt]);
+          xs[n][1] = __builtin_fmaf(Sx[nt][u][q2 + 1], scale, neg_run[nt]);
+        }
       };
       // scores: sub-tiles alternate, so a product meets its accumulator again four products later
 #pragma unroll
       for (int n = 0; n < 8; ++n) {
-        request(n + 3);
+        request(n + AHEAD);
         MI_SB();
         const int u = n & 1, kk = n >> 1;
-        Sn[0][u] = mfma_16x16x32<F16>(fr[n & 3], qf[0][kk], kk ? Sn[0][u] : zero4);
-        Sn[1][u] = mfma_16x16x32<F16>(fr[n & 3], qf[1][kk], kk ? Sn[1][u] : zero4);
+        Sn[0][u] = mfma_16x16x32<F16>(fr[n % RING], qf[0][kk], kk ? Sn[0][u] : zero4);
+        Sn[1][u] = mfma_16x16x32<F16>(fr[n % RING], qf[1][kk], kk ? Sn[1][u] : zero4);
         MI_SB();
-        if (n == 0) exp_chunk(Sx, Px, 0);
-        if (n == 2) exp_chunk(Sx, Px, 1);
-        if (n == 3) exp_chunk(Sx, Px, 2);
-        if (n == 5) exp_chunk(Sx, Px, 3);
-        if (n == 6) exp_chunk(Sx, Px, 4);
+        exp_stages(n);
         MI_SB();
       }
       if constexpr (H == 1) at_barrier();
@@ -298,15 +322,13 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
       // values; beside them the last probabilities, then mask and maximum of the scores just multiplied
 #pragma unroll
       for (int n = 8; n < 16; ++n) {
-        request(n + 3);
+        request(n + AHEAD);
         MI_SB();
         const int e = n - 8;
-        acc[0][e] = mfma_16x16x32<F16>(fr[n & 3], Pv[0], acc[0][e]);
-        acc[1][e] = mfma_16x16x32<F16>(fr[n & 3], Pv[1], acc[1][e]);
+        acc[0][e] = mfma_16x16x32<F16>(fr[n % RING], Pv[0], acc[0][e]);
+        acc[1][e] = mfma_16x16x32<F16>(fr[n % RING], Pv[1], acc[1][e]);
         MI_SB();
-        if (n == 8) exp_chunk(Sx, Px, 5);
-        if (n == 9) exp_chunk(Sx, Px, 6);
-        if (n == 10) exp_chunk(Sx, Px, 7);
+        if (n < 10) exp_stages(n);
         if constexpr (H == 1) under_products(n - 8);
         if (n == 11 && MASK) {
           const int tok0 = key0 + 4 * g;
@@ -344,11 +366,17 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
     };
 
     // ---- prologue: clear the buffers (the value tile "before the first" must hold zeros), start the first tiles ----
-    for (int i = tid * 16; i < 2 * BUF; i += 512 * 16) *reinterpret_cast<uint4*>(&Ks[0][0] + i) = make_uint4(0u, 0u, 0u, 0u);
-    for (int i = tid * 16; i < 3 * BUF; i += 512 * 16) *reinterpret_cast<uint4*>(&Vs[0][0] + i) = make_uint4(0u, 0u, 0u, 0u);
-    const Cursor c0 = cursor_at(tb), c1 = cursor_at(tb + 1);
-    Cursor cur = cursor_at(tb + 2);
-    const int pc0 = __builtin_amdgcn_readfirstlane(bt_row[c0.ci]), pc1 = __builtin_amdgcn_readfirstlane(bt_row[c1.ci]);
+    for (int i = tid * 16; i < KBUFS * BUF; i += 512 * 16) *reinterpret_cast<uint4*>(&Ks[0][0] + i) = make_uint4(0u, 0u, 0u, 0u);
+    for (int i = tid * 16; i < VBUFS * BUF; i += 512 * 16) *reinterpret_cast<uint4*>(&Vs[0][0] + i) = make_uint4(0u, 0u, 0u, 0u);
+    Cursor cur = cursor_at(tb + DEPTH + 1);
+    int64_t off_first[DEPTH + 1];   // tiles tb .. tb + DEPTH, started here
+    uint32_t nrec_first[DEPTH + 1];
+#pragma unroll
+    for (int i = 0; i <= DEPTH; ++i) {
+      const Cursor c = cursor_at(tb + i);
+      off_first[i] = tile_off(c, __builtin_amdgcn_readfirstlane(bt_row[c.ci]));
+      nrec_first[i] = tile_nrec(c);
+    }
     int pc_next = __builtin_amdgcn_readfirstlane(bt_row[cur.ci]);
     // (the query fragments count as used here: the compiler then waits for their loads now and not in the tile
     // loop, where a wait on the vector-memory counter would wait for the direct loads in flight as well)
@@ -361,45 +389,51 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
     int64_t off_prev;
     uint32_t nrec_prev;
     {
-      const int64_t off0 = tile_off(c0, pc0), off1 = tile_off(c1, pc1);
-      const u32x4_t rk0 = tile_rsrc(kbase, off0, tile_nrec(c0)), rv0 = tile_rsrc(vbase, off0, tile_nrec(c0));
-      const u32x4_t rk1 = tile_rsrc(kbase, off1, tile_nrec(c1));
+      const u32x4_t rk0 = tile_rsrc(kbase, off_first[0], nrec_first[0]);
 #pragma unroll
       for (int i = 0; i < 5; ++i)
-        if (ld_key[i]) issue_load(i, rk0, rk0, ks_lds, ks_lds);            // key tile 0 -> Ks[0]
+        if (ld_key[i]) issue_load(i, rk0, rk0, ks_lds, ks_lds);  // key tile 0 -> Ks[0]
 #pragma unroll
-      for (int i = 0; i < 5; ++i) issue_load(i, rk1, rv0, ks_lds + BUF, vs_lds + BUF);  // key tile 1 -> Ks[1], value tile 0 -> Vs[1]
-      off_prev = off1;
-      nrec_prev = tile_nrec(c1);
+      for (int t = 1; t <= DEPTH; ++t) {  // the pairs {key tile t -> Ks[t], value tile t - 1 -> Vs[t]}
+        const u32x4_t rk = tile_rsrc(kbase, off_first[t], nrec_first[t]);
+        const u32x4_t rv = tile_rsrc(vbase, off_first[t - 1], nrec_first[t - 1]);
+#pragma unroll
+        for (int i = 0; i < 5; ++i) issue_load(i, rk, rv, ks_lds + t * BUF, vs_lds + t * BUF);
+      }
+      off_prev = off_first[DEPTH];
+      nrec_prev = nrec_first[DEPTH];
     }
-    asm volatile("s_waitcnt vmcnt(5)" ::: "memory");  // key tile 0 has landed (this wavefront's share)
+    // key tile 0 has landed (this wavefront's share): only the DEPTH pairs issued after it may still be on their way
+    if constexpr (DEPTH == 1) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
     __builtin_amdgcn_s_barrier();
     MI_SB();
 
     const int t_mask = max(0, (full_until + 1) >> 6);              // first tile with a masked score for this wavefront
     const int jm = min(max(t_mask - tb, 0), ntl);                  // iterations [0, jm) need no mask
     int j = 0;
-    int vb = 0;  // j % 3
-    fr[0] = read_k(k_lane, 0, 0);
-    fr[1] = read_k(k_lane, 0, 1);
-    fr[2] = read_k(k_lane, 0, 2);
+    int kbi = 0, vbi = 0;  // j % KBUFS, j % VBUFS
+#pragma unroll
+    for (int n = 0; n < AHEAD; ++n) fr[n] = read_k(k_lane, 0, n);
 
-    // iteration j: scores of key tile j (Ks[j & 1]), values of tile j-1 (Vs[j % 3]); after its barrier key tile j+1
-    // and value tile j are in LDS, and the loads of key tile j+2 (into Ks[j & 1]) and value tile j+1 (into
-    // Vs[(j + 2) % 3]) set out under the products that follow.
+    // iteration j: scores of key tile j (Ks[j % KBUFS]), values of tile j-1 (Vs[j % VBUFS]); after its barrier key tile
+    // j+1 and value tile j are in LDS, and the loads of key tile j+DEPTH+1 (into the buffer of key tile j, which every
+    // wavefront has left) and value tile j+DEPTH (into the buffer of value tile j-2) set out under the products that follow.
     auto iteration = [&](auto Mc) {
-      const int kb = (j & 1) * BUF;
+      const int kb = kbi * BUF;
       const uint8_t* ka = k_lane + kb;
-      const uint8_t* ka_next = k_lane + (BUF - kb);
-      const uint8_t* va = v_lane + vb * BUF;
+      const uint8_t* ka_next = k_lane + (kbi == KBUFS - 1 ? 0 : kbi + 1) * BUF;
+      const uint8_t* va = v_lane + vbi * BUF;
       const int key0 = (tb + j) * kWvTile;
       u32x4_t rs_k, rs_v;
       const uint32_t kdst = ks_lds + (uint32_t)kb;
-      const uint32_t vdst = vs_lds + (uint32_t)((vb == 0 ? 2 : vb - 1) * BUF);  // (j + 2) % 3
+      const uint32_t vdst = vs_lds + (uint32_t)((vbi == 0 ? VBUFS - 1 : vbi - 1) * BUF);  // (j - 1) % VBUFS
       slot(std::integral_constant<int, 0>{}, Mc, ka, ka_next, va, key0, [] {}, [](int) {});
       slot(std::integral_constant<int, 1>{}, Mc, ka, ka_next, va, key0 + 32,
            [&] {
-             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's share of key tile j+1 and value tile j
+             // this wavefront's share of key tile j+1 and value tile j has landed: only younger pairs are on their way
+             if constexpr (DEPTH == 1) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+             else asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
              __builtin_amdgcn_s_barrier();
              bt_arrived(pc_next);
              const int64_t off = tile_off(cur, pc_next);
@@ -415,14 +449,15 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
              if (i < 5) issue_load(i, rs_k, rs_v, kdst, vdst);
            });
       ++j;
-      vb = vb == 2 ? 0 : vb + 1;
+      kbi = kbi == KBUFS - 1 ? 0 : kbi + 1;
+      vbi = vbi == VBUFS - 1 ? 0 : vbi + 1;
     };
     for (; j < jm;) iteration(std::false_type{});
     for (; j < ntl;) iteration(std::true_type{});
 
-    // ---- drain: the last two steps' values (tile ntl - 1 in Vs[ntl % 3]); S[1] is masked and checked already ----
+    // ---- drain: the last two steps' values (tile ntl - 1 in Vs[ntl % VBUFS]); S[1] is masked and checked already ----
     {
-      const uint8_t* va = v_lane + vb * BUF;
+      const uint8_t* va = v_lane + vbi * BUF;
       auto values = [&](int half, const uint4 (&Pv)[NQ]) {
 #pragma unroll
         for (int e = 0; e < DV; ++e) {

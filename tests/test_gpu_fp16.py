@@ -78,10 +78,11 @@ def test_mismatched_types_are_rejected(mi, dev):
         mi.ops.paged_decode_attention(case.q, k8, k8, case.kv_lens, case.block_table, k_scales=sc, v_scales=sc)
 
 
-@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_lock_step", "registers", "split_keys"])
+@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_staggered", "two_phase_lock_step", "registers", "split_keys"])
 @pytest.mark.parametrize("Hq,Hkv,d", [(32, 8, 128), (8, 8, 64), (12, 4, 128), (16, 1, 64), (32, 8, 96)])
 def test_prefill_and_mixed_batches(mi, dev, kernel, Hq, Hkv, d):
-    knobs = {"two_phase": {}, "two_phase_lock_step": {"prefill_two_phase": 2}, "registers": {"prefill_two_phase": -1},
+    knobs = {"two_phase": {}, "two_phase_staggered": {"prefill_two_phase": 1}, "two_phase_lock_step": {"prefill_two_phase": 2},
+             "registers": {"prefill_two_phase": -1},
              "split_keys": {"prefill_kv_split": 3}}[kernel]
     q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 500, 256, 257, 3]
     ctx = [700, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0, 40, 7, 64, 63, 1020]

@@ -73,14 +73,15 @@ def test_padded_requests_with_zero_lengths(mi, dev):
     assert (out.float().cpu() - ref).abs().max().item() < 2e-2
 
 
-@pytest.mark.parametrize("pingpong", [1, 2])
+@pytest.mark.parametrize("pingpong", [1, 2, 3])
 @pytest.mark.parametrize("chunk", [64, 128, 256])
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 1), (16, 2)])
 @pytest.mark.parametrize("d", [128, 64, 96])
 def test_two_phase_kernel_ragged_lengths(mi, dev, pingpong, chunk, Hq, Hkv, d):
-    """The two-phase tile kernel (head_dim 128, 96 or 64, chunk a multiple of 64): new-token counts and cached
+    """The tile kernels (head_dim 128, 96 or 64, chunk a multiple of 64): new-token counts and cached
     contexts around every tile (64 keys), workgroup (256 rows) and chunk boundary, for 1, 2, 4, 8
-    and 16 query heads per KV head, staggered and lock-step."""
+    and 16 query heads per KV head; the two-phase kernel staggered (1) and in lock-step (2), and the one-stream
+    kernel that serves head_dim 128 by default (3; other widths fall back to the two-phase kernel)."""
     q_lens = [1, 2, 15, 16, 17, 63, 64, 65, 128, 200, 1, 97, 500, 256, 257, 3]
     ctx = [0, 5, 0, 16, 31, 0, 100, 1, 0, 333, 0, 40, 7, 64, 63, 1020]
     kv_lens = torch.tensor([a + b for a, b in zip(q_lens, ctx)], dtype=torch.int32)
@@ -142,13 +143,15 @@ def test_head_widths_96_192_256(mi, dev, d, Hq, Hkv, chunk, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
-@pytest.mark.parametrize("kernel", ["two_phase", "registers", "split_keys"])
+@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_staggered", "registers", "split_keys", "split_keys_staggered"])
 @pytest.mark.parametrize("d", [64, 96, 128, 192, 256])
 def test_scores_that_keep_growing_along_the_context(mi, dev, d, kernel, dtype):
     """Keys grow with their position (x52 at token 1 020), so a row's largest score moves up by far more than any
     window a kernel takes its exponentials within (2^8 for fp16 operands, 2^30 for bf16), tile after tile; rows
     whose query points the other way see it fall instead."""
-    knobs = {"two_phase": {}, "registers": {"prefill_two_phase": -1}, "split_keys": {"prefill_kv_split": 3}}[kernel]
+    knobs = {"two_phase": {}, "two_phase_staggered": {"prefill_two_phase": 1}, "registers": {"prefill_two_phase": -1},
+             "split_keys": {"prefill_kv_split": 3},
+             "split_keys_staggered": {"prefill_kv_split": 3, "prefill_two_phase": 1}}[kernel]
     chunk = 64
     q, kc, vc, cu_q, lens, bt = _ragged_case(mi, dev, 16, 4, d, chunk, dtype, seed=700 + d)
     pos = torch.arange(chunk, device=dev)
@@ -300,14 +303,14 @@ def test_split_keys_with_padding_rows_and_fp8(mi, dev):
     assert (err8 <= 2.5e-2 + 2.5e-2 * ref8.abs()).all() and (out8[53:] == 0).all()
 
 
-@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_no_offset", "registers", "registers_64_rows", "split_keys"])
+@pytest.mark.parametrize("kernel", ["two_phase", "two_phase_staggered", "two_phase_no_offset", "registers", "registers_64_rows", "split_keys"])
 @pytest.mark.parametrize("Hq,Hkv", [(12, 4), (10, 2), (28, 4), (6, 1), (12, 1), (15, 1)])
 @pytest.mark.parametrize("d", [128, 64])
 def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, d):
     """3, 5, 6, 7, 12 or 15 query heads per KV head (Llama-3.2-3B, Qwen2.5-14B, Qwen2-7B ... have such groups):
     a wavefront's 32 (64) rows then hold as many whole tokens as fit, the rest are padding rows.  Every
     prefill kernel, lengths either side of the per-workgroup token counts (48 tokens at a group of 5)."""
-    knobs = {"two_phase": {}, "two_phase_no_offset": {"prefill_two_phase": 2},
+    knobs = {"two_phase": {}, "two_phase_staggered": {"prefill_two_phase": 1}, "two_phase_no_offset": {"prefill_two_phase": 2},
              "registers": {"prefill_two_phase": -1},
              "registers_64_rows": {"prefill_two_phase": -1, "prefill_row_tiles": 4},
              "split_keys": {"prefill_kv_split": 3}}[kernel]

@@ -145,7 +145,7 @@ def case_prefill(mi, dev, rng, seed, fp8):
             ctx.append(rng.choice([0, 0, 5, chunk - 1, chunk, rng.randint(0, 700)]))
     if sum(q_lens) == 0:
         q_lens[0] = 3
-    pp = rng.choice([0, 0, 2, -1])  # two-phase tile kernel (default), the same in lock-step, register-only kernel
+    pp = rng.choice([0, 0, 1, 2, -1])  # default tile kernel (one stream at head_dim 128), two-phase staggered / lock-step, register-only
     ksplit = rng.choice([0, 0, -1, 3, 8])  # key ranges per request in the tile kernel (0 = automatic, -1 = never)
     # keys of later physical chunks up to 41 times larger: maxima that keep moving.  Not over an fp8 cache: scores in
     # the hundreds amplify the rounding of its dequantised keys to the 16-bit operand type beyond the 2.5e-2 bound
@@ -250,7 +250,7 @@ def case_mla_prefill(mi, dev, rng, seed):
             ctx.append(rng.choice([0, 0, 5, chunk - 1, chunk, rng.randint(0, 700)]))
     if sum(q_lens) == 0:
         q_lens[0] = 5
-    pp = rng.choice([0, 0, 2, -1])  # two-phase tile kernel (default), the same in lock-step, register-only kernel
+    pp = rng.choice([0, 0, 1, 2, -1])  # default tile kernel (one stream at head_dim 128), two-phase staggered / lock-step, register-only
     ksplit = rng.choice([0, 0, -1, 3, 8])
     joint = rng.random() < 0.4
     _note(f"mla_prefill seed={seed} Hq={Hkv * G} Hkv={Hkv} chunk={chunk} q_lens={q_lens} ctx={ctx} pingpong={pp} joint={joint}")
