@@ -119,7 +119,7 @@ def run_secondary(args, mi, lib, torch, dev):
         pairs = n * (new * ctx + new * (new + 1) // 2)          # (query row, visible key) pairs per head
         flops = 2 * Hq * (dk + dv) * pairs
         nbytes = n * (new + ctx) * Hkv * (dk + dv) * 2 + n * new * Hq * (dk + dv) * 2
-        kernel = "paged_prefill_pp_kernel"
+        kernel = "paged_prefill_woven_kernel" if (not mla and dk == 128) else "paged_prefill_pp_kernel"
         what = (f"paged varlen causal attention, {n} x {new} new tokens over {ctx} cached, {Hq}/{Hkv} heads, "
                 f"keys {dk} / values {dv} wide, chunk 256")
         dtype = "bf16 (fp32 accumulate)"
@@ -186,13 +186,13 @@ def run_secondary(args, mi, lib, torch, dev):
     roofline.update({"kernel_ms": round(kernel_ms, 5), "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload)})
     if args.workload in TRAFFIC_SOURCE:
         roofline["traffic_source"] = TRAFFIC_SOURCE[args.workload]
-    print(json.dumps({
+    return ({
         "metric": f"{args.workload}_GBps", "value": round(nbytes / (ms_per_step * 1e-3) / 1e9, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
         "config": {"workload": what, "algorithmic_bytes_per_step": nbytes, "flops_per_step": flops,
                    "call_ms_by_events": round(call_ms, 5)},
-        "roofline": roofline}), flush=True)
+        "roofline": roofline})
 
 
 def run_stream_read(args, mi, torch, dev):
@@ -233,7 +233,7 @@ def run_stream_read(args, mi, torch, dev):
         results[name] = {"kernel_ms_mean": sum(ms) / len(ms), "kernel_ms_min": ms[0], "ms_per_step": elapsed * 1e3 / args.steps}
     best = results["nontemporal"]
     achieved = nbytes / best["kernel_ms_mean"] / 1e6
-    print(json.dumps({
+    return ({
         "metric": "stream_read_GBps", "value": round(nbytes / (best["ms_per_step"] * 1e-3) / 1e9, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(best["ms_per_step"], 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
@@ -244,88 +244,7 @@ def run_stream_read(args, mi, torch, dev):
                    "best_launch_GBps": round(nbytes / best["kernel_ms_min"] / 1e6, 1)},
         "roofline": {"bound": "hbm", "kernel": "stream_read_kernel", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "kernel_ms": round(best["kernel_ms_mean"], 5), "traffic": None}}), flush=True)
-
-
-def run_cu_probes(args, mi, torch, dev):
-    """Calibration leg: what one compute unit delivers to the prefill tile kernel (csrc/bench/cu_probes.hip) --
-    LDS fragment reads per wavefront and per CU, the same fragments through the vector L1, how matrix and vector
-    instructions of two wavefronts of a SIMD overlap, and the core clock a matrix-bound kernel really runs at."""
-    path = mi._lib.PKG_DIR / "libmi355_bench.so"
-    if not path.exists():
-        print(f"{path} not found: build first (python megatron-mixtera_amd/build.py)", file=sys.stderr)
-        sys.exit(2)
-    blib = ctypes.CDLL(str(path))
-    P, I = ctypes.c_void_p, ctypes.c_int32
-    blib.mi_bench_read_probe.restype = ctypes.c_int
-    blib.mi_bench_read_probe.argtypes = [I, I, I, I, I, P, P, P, P]
-    blib.mi_bench_coexec_probe.restype = ctypes.c_int
-    blib.mi_bench_coexec_probe.argtypes = [I, I, I, I, P, P, P]
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    cyc = torch.zeros(16, dtype=torch.int64, device=dev)
-    sink = torch.zeros(cus * 1024, dtype=torch.int32, device=dev)
-    gsrc = torch.ones(cus * 64 * 2048, dtype=torch.uint8, device=dev)
-    stream = torch.cuda.current_stream().cuda_stream
-    t0 = time.perf_counter()
-    reads = {}
-    iters = 2000
-    for mode, name in ((0, "lds_b128"), (1, "lds_tr_b64"), (2, "global_b128_l1_resident")):
-        for depth in (1, 4, 16):   # fragments a wavefront has in flight before it waits for the first
-            for waves in (1, 4, 8, 16):
-                for _ in range(2):
-                    assert blib.mi_bench_read_probe(mode, depth, waves, cus, iters, cyc.data_ptr(), sink.data_ptr(),
-                                                    gsrc.data_ptr(), stream) == 0
-                torch.cuda.synchronize()
-                worst = int(cyc[:waves].max())
-                nbytes = iters * 16 * 1024 * waves
-                reads[f"{name}_{depth}_in_flight_{waves}_waves"] = {"bytes_per_clk_per_cu": round(nbytes / worst, 1),
-                                                                    "bytes_per_clk_per_wave": round(nbytes / worst / waves, 2)}
-    names = {0: "idle", 1: "mfma_16x16x32", 2: "mfma_32x32x16", 3: "fma", 4: "exp2"}
-    per_iter = {1: 32, 2: 16, 3: 32, 4: 32}
-    coexec = {}
-    iters = 20000
-    for a, b in ((1, 0), (2, 0), (3, 0), (4, 0), (3, 3), (1, 3), (1, 4), (2, 3), (2, 4), (1, 1)):
-        for wgs in (1, cus):   # one workgroup alone; every CU busy (the clock a loaded chip runs at)
-            for _ in range(2):
-                assert blib.mi_bench_coexec_probe(a, b, wgs, iters, cyc.data_ptr(), sink.data_ptr(), stream) == 0
-            torch.cuda.synchronize()
-            c = cyc.tolist()
-            entry = {"a_clk_per_instr": round(c[0] / (iters * per_iter[a]), 2)}
-            if b:
-                entry["b_clk_per_instr"] = round(c[4] / (iters * per_iter[b]), 2)
-            entry["core_clock_mhz"] = round(c[0] / max(c[8], 1) * 100)
-            coexec[f"{names[a]}+{names[b]}" + ("_all_cus" if wgs > 1 else "_one_cu")] = entry
-    blib.mi_bench_woven_probe.restype = ctypes.c_int
-    blib.mi_bench_woven_probe.argtypes = [I, I, I, I, P, P, P]
-    woven = {}
-    iters = 2000
-    for rows in (64, 32):
-        for weave, name in ((1, "woven"), (0, "vector_work_after_the_products"), (2, "woven_fma_and_exponential_only")):
-            for wgs in (1, cus):
-                for _ in range(2):
-                    assert blib.mi_bench_woven_probe(rows, weave, wgs, iters, cyc.data_ptr(), sink.data_ptr(), stream) == 0
-                torch.cuda.synchronize()
-                c = cyc.tolist()
-                clk = max(c[:256 // rows]) / iters   # every wavefront of the workgroup does `iters` tiles
-                # a 16x16x32 product occupies a SIMD's matrix core for 16 clocks (mfma_16x16x32+idle above);
-                # a SIMD's wavefronts together issue 128 of them per `clk`
-                woven[f"{rows}_rows_per_wavefront_{name}" + ("_all_cus" if wgs > 1 else "_one_cu")] = {
-                    "clk_per_tile": round(clk, 1), "matrix_core_busy": round(128 * 16 / clk, 3),
-                    "core_clock_mhz": round(c[0] / max(c[8], 1) * 100)}
-    elapsed = time.perf_counter() - t0
-    print(json.dumps({
-        "metric": "cu_probes", "value": reads["lds_b128_16_in_flight_16_waves"]["bytes_per_clk_per_cu"], "unit": "LDS B/clk/CU",
-        "n_gpus": 1, "steps": 1, "warmup": 0, "ms_per_step": round(elapsed * 1e3, 1), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "u8 / bf16 / f32", "data": "synthetic",
-        "config": {"workload": "probes of one compute unit: fragment reads from LDS and through the vector L1 "
-                               "(bytes per core clock), matrix / vector co-execution of two wavefronts of a SIMD "
-                               "(core clocks per instruction; a = wavefronts 0-3, b = wavefronts 4-7), core clock"},
-        "reads": reads, "coexec": coexec,
-        "attention_tile_in_one_instruction_stream": {
-            "what": "64 keys x 128 values x (64 query rows per wavefront, one wavefront a SIMD | 32 rows, two a SIMD): "
-                    "per SIMD and tile 128 products 16x16x32, the key / value fragment reads and the softmax's vector "
-                    "arithmetic in one instruction stream per wavefront",
-            **woven}}), flush=True)
+                     "kernel_ms": round(best["kernel_ms_mean"], 5), "traffic": None}})
 
 
 def parse_args():
@@ -334,7 +253,7 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", "cu_probes", *SECONDARY_WORKLOADS],
+                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", *SECONDARY_WORKLOADS],
                     help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch; the "
                          "mla_* / prefill_d* / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
     ap.add_argument("--split-tokens", type=int, default=0)
@@ -348,6 +267,11 @@ def parse_args():
     ap.add_argument("--read-mib", type=int, default=1146,
                     help="stream_read only: buffer size (default: the 1.2 GB one cfg2 launch streams)")
     ap.add_argument("--read-wgs-per-cu", type=int, default=2, help="stream_read only: workgroups per CU")
+    ap.add_argument("--cpu-budget-s", type=float, default=12.0, help="seconds of CPU work for the cpu_baseline leg")
+    ap.add_argument("--sustained-launches", type=int, default=1000,
+                    help="cfg3: back-to-back launches of the tile kernel for the power-capped figure (0 = skip)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="default cfg2 run only: do not append the cfg3 / cfg4 / cfg5 legs (other_configs)")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="also run a plain device copy of this many MiB (a known-size reference for "
                          "scaling hardware traffic counters collected by an external profiler)")
@@ -364,6 +288,50 @@ def _compact_chunks(torch, table_rows, n_pool, *tensors):
     return new_rows, [None if t is None else t[used.to(t.device)].cpu() for t in tensors]
 
 
+class BoardPower:
+    """Board power while a leg runs: a thread reads the amdgpu hwmon files (the driver's running average, which
+    follows the load with a lag of a few hundred milliseconds, so only legs of about a second say anything)."""
+
+    def __init__(self):
+        import glob
+        inp = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+                     + glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average"))
+        cap = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"))
+        self.path = inp[0] if inp else None
+        self.cap_w = self._read(cap[0]) if cap else None
+        self.samples = []
+        self._stop = False
+        self._thread = None
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return int(f.read().strip()) / 1e6
+        except (OSError, ValueError):
+            return None
+
+    def __enter__(self):
+        import threading
+        if self.path:
+            def loop():
+                while not self._stop:
+                    self.samples.append((time.perf_counter(), self._read(self.path)))
+                    time.sleep(0.01)
+            self._thread = threading.Thread(target=loop, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread:
+            self._thread.join()
+
+    def mean_w(self, t_from: float, t_to: float):
+        vals = [w for t, w in self.samples if w is not None and t_from <= t <= t_to]
+        return round(sum(vals) / len(vals), 1) if vals else None
+
+
 def _time_cpu(torch, one_pass, budget_s: float = 12.0):
     """Median pass time after one warm-up: at least 3 timed passes, about ``budget_s`` seconds of CPU work."""
     torch.set_num_threads(os.cpu_count() or 1)
@@ -376,7 +344,7 @@ def _time_cpu(torch, one_pass, budget_s: float = 12.0):
     return sorted(times[1:])[len(times[1:]) // 2], len(times) - 1
 
 
-def cpu_baseline(case, cfg, sample_requests: int, qw, kw, table, attention_only: bool):
+def cpu_baseline(case, cfg, sample_requests: int, qw, kw, table, attention_only: bool, budget_s: float = 12.0):
     """Time the CPU checker on the first ``sample_requests`` requests of the same seeded batch, doing what the GPU
     step does: unfused q/k RMSNorm + RoPE (op by op in bf16), the scatter append of the new key / value rows
     (quantising for an fp8 cache), then gather through the block table + fp32 attention."""
@@ -408,7 +376,7 @@ def cpu_baseline(case, cfg, sample_requests: int, qw, kw, table, attention_only:
                 oa.kv_append(kc, vc, kn[rows], v_new[rows], ids, loc)
         return oa.paged_decode_attention(qn, kc, vc, lens, bt, k_scales=ks, v_scales=vs)
 
-    t, passes = _time_cpu(torch, one_pass)
+    t, passes = _time_cpu(torch, one_pass, budget_s)
     nbytes = oa.decode_attention_bytes(lens.tolist(), cfg.Hq, cfg.Hkv, cfg.d, cfg.chunk,
                                        kv_bytes=1 if cfg.fp8 else 2, fp8_scales=cfg.fp8)
     what = ("fp32 gather + softmax checker" if attention_only else
@@ -419,7 +387,7 @@ def cpu_baseline(case, cfg, sample_requests: int, qw, kw, table, attention_only:
 
 
 def cpu_baseline_mixed(q, k_new, v_new, kc, vc, cu_q, lens, bt, qw, kw, table, n_prefill: int, n_decode: int,
-                       Hq: int, Hkv: int, d: int, chunk: int):
+                       Hq: int, Hkv: int, d: int, chunk: int, budget_s: float = 12.0):
     """The mixed step on the CPU checker for a bounded sample of the batch: the first ``n_prefill`` prefill
     requests and the first ``n_decode`` one-token requests -- unfused RMSNorm + RoPE of their new tokens, scatter
     append, varlen causal attention through the block table."""
@@ -453,7 +421,7 @@ def cpu_baseline_mixed(q, k_new, v_new, kc, vc, cu_q, lens, bt, qw, kw, table, n
         oa.kv_append(kcc, vcc, kn, vs_new, ids, loc)
         return oa.paged_varlen_attention(qn, kcc, vcc, cu_s, lens_s, bt_s)
 
-    t, passes = _time_cpu(torch, one_pass)
+    t, passes = _time_cpu(torch, one_pass, budget_s)
     lk = lens_s.long()
     is_pre = lq > 1
     dec_bytes = oa.decode_attention_bytes(lk[~is_pre].tolist(), Hq, Hkv, d, chunk)
@@ -529,6 +497,37 @@ def run_mixed_batch(args, mi, lib, torch, dev):
     tile_ms = sum(buf[i] for i in range(0, n_ev, 2)) / max(1, n_ev // 2)
     stream_ms = sum(buf[i] for i in range(1, n_ev, 2)) / max(1, n_ev // 2)
 
+    # The tile kernel alone, launched back to back for about a second (the prefill requests only, no workspace, so
+    # the call is that one kernel), with the board power read beside it: this kernel runs the board into its power
+    # cap, and what a power-capped kernel reaches is set by the energy it spends, not by its schedule.
+    sustained = None
+    if args.sustained_launches > 0:
+        n_pre = int((cu_q[1:] - cu_q[:-1] > 1).sum())
+        t_pre = int(cu_q[n_pre])
+        cu_pre, lens_pre, bt_pre = cu_q[:n_pre + 1].contiguous(), lens[:n_pre].contiguous(), bt[:n_pre].contiguous()
+        q_pre, out_pre = q_rot[:t_pre], out[:t_pre]
+        def tile_only():
+            mi.ops.paged_prefill_attention(q_pre, kc, vc, cu_pre, lens_pre, bt_pre, max_kv_len=max_len, out=out_pre,
+                                           k_scales=ks, v_scales=vs)
+        for _ in range(5):
+            tile_only()
+        torch.cuda.synchronize()
+        with BoardPower() as power:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t_a = time.perf_counter()
+            e0.record()
+            for _ in range(args.sustained_launches):
+                tile_only()
+            e1.record()
+            torch.cuda.synchronize()
+            t_b = time.perf_counter()
+        sus_ms = e0.elapsed_time(e1) / args.sustained_launches
+        sustained = {"launches": args.sustained_launches, "kernel_ms": round(sus_ms, 5),
+                     "achieved": None, "board_power_w": power.mean_w(t_a + 0.6 * (t_b - t_a), t_b),
+                     "power_cap_w": power.cap_w,
+                     "what": "the prefill requests' tile kernel launched back to back; board power = mean of the "
+                             "driver's hwmon reading over the last 40 % of the run"}
+
     lq = (cu_q[1:] - cu_q[:-1]).cpu().long()
     lk = lens.cpu().long()
     pre = lq > 1
@@ -550,7 +549,8 @@ def run_mixed_batch(args, mi, lib, torch, dev):
                                + (" (fp8-e4m3 KV cache, quantising append)" if args.fp8_kv else ""),
                    "new_tokens": T, "requests": int(lens.numel()), "algorithmic_bytes_per_step": total_bytes,
                    "prefill_flops_per_step": flops},
-        "roofline": {"bound": "mfma", "kernel": "paged_prefill_pp_kernel", "achieved": round(flops / tile_ms / 1e9, 1),
+        "roofline": {"bound": "mfma", "kernel": "paged_prefill_pp_kernel" if args.fp8_kv else "paged_prefill_woven_kernel",
+                     "achieved": round(flops / tile_ms / 1e9, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / tile_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "kernel_ms": round(tile_ms, 5),
                      "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_tile"],
@@ -562,10 +562,15 @@ def run_mixed_batch(args, mi, lib, torch, dev):
                                  "traffic": None if args.fp8_kv else MEASURED_HBM_TRAFFIC_BYTES["cfg3_stream"],
                                  "traffic_source": None if args.fp8_kv else TRAFFIC_SOURCE["cfg3_stream"]},
     }
+    if sustained is not None:
+        sustained["achieved"] = round(flops / sustained["kernel_ms"] / 1e9, 1)
+        sustained["frac"] = round(flops / sustained["kernel_ms"] / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)
+        result["roofline"]["sustained"] = sustained
     if not args.no_cpu_baseline and not args.fp8_kv:
         result["cpu_baseline"] = cpu_baseline_mixed(q, k_new, v_new, kc, vc, cu_q, lens, bt, qw, kw, table,
-                                                    n_prefill=1, n_decode=15, Hq=Hq, Hkv=Hkv, d=d, chunk=chunk)
-    print(json.dumps(result), flush=True)
+                                                    n_prefill=1, n_decode=15, Hq=Hq, Hkv=Hkv, d=d, chunk=chunk,
+                                                    budget_s=args.cpu_budget_s)
+    return result
 
 
 def main():
@@ -574,6 +579,8 @@ def main():
         print(f"bench.py measures one GPU: this build's hot path is a single-GPU kernel path and --gpus "
               f"{args.gpus} is not supported (no collectives are part of it).", file=sys.stderr)
         sys.exit(2)
+
+    import copy
 
     import torch
 
@@ -589,19 +596,37 @@ def main():
     if args.subtiles:
         mi.ops.set_tuning("decode_tile_subtiles", args.subtiles)  # (passed with every call of the ops module)
 
-    if args.workload == "cfg3":
-        run_mixed_batch(args, mi, lib, torch, dev)
-        return
-    if args.workload == "stream_read":
-        run_stream_read(args, mi, torch, dev)
-        return
-    if args.workload == "cu_probes":
-        run_cu_probes(args, mi, torch, dev)
-        return
-    if args.workload in SECONDARY_WORKLOADS:
-        run_secondary(args, mi, lib, torch, dev)
-        return
+    result = run_workload(args, mi, lib, torch, dev)
+    # The default run carries the other single-GPU configurations beside the headline one: the mixed batch (cfg3),
+    # the long-context batch (cfg4) and the fp8 cache (cfg5), each with its own roofline and a short CPU leg.
+    plain = not (args.hip_graph or args.attention_only or args.separate_launches or args.fp8_kv or args.subtiles
+                 or args.split_tokens or args.calibrate_copy_mib)
+    if args.workload == "cfg2" and plain and not args.no_other_configs:
+        others = {}
+        for name, steps in (("cfg3", 20), ("cfg4", 20), ("cfg5", 10)):
+            sub = copy.copy(args)
+            sub.workload, sub.steps, sub.warmup, sub.cpu_budget_s = name, min(args.steps, steps), min(args.warmup, 3), 3.0
+            torch.cuda.empty_cache()
+            r = run_workload(sub, mi, lib, torch, dev)
+            others[name] = {k: r[k] for k in ("value", "unit", "steps", "ms_per_step", "dtype", "config", "roofline",
+                                              "roofline_decode_part", "separate_launches", "cpu_baseline") if k in r}
+        result["other_configs"] = others
+    print(json.dumps(result), flush=True)
 
+
+def run_workload(args, mi, lib, torch, dev):
+    """One workload -> its result line as a dictionary."""
+    if args.workload == "cfg3":
+        return run_mixed_batch(args, mi, lib, torch, dev)
+    if args.workload == "stream_read":
+        return run_stream_read(args, mi, torch, dev)
+    if args.workload in SECONDARY_WORKLOADS:
+        return run_secondary(args, mi, lib, torch, dev)
+    return run_decode_config(args, mi, lib, torch, dev)
+
+
+def run_decode_config(args, mi, lib, torch, dev):
+    """cfg1 / cfg2 / cfg4 / cfg5 (and cfg3's decode part alone): one decode step per timed step."""
     cfg = mi.synthetic.CONFIGS[args.workload]
     case = mi.synthetic.make_decode_case(cfg, dev, on_device_rng=True)
     if cfg.fp8:
@@ -777,8 +802,8 @@ def main():
         result["separate_launches"] = separate
     if not args.no_cpu_baseline:
         sample = {"cfg1": 4, "cfg2": 64, "cfg3_decode": 64, "cfg4": 1, "cfg5": 16}[args.workload]
-        result["cpu_baseline"] = cpu_baseline(case, cfg, sample, qw, kw, table, args.attention_only)
-    print(json.dumps(result), flush=True)
+        result["cpu_baseline"] = cpu_baseline(case, cfg, sample, qw, kw, table, args.attention_only, args.cpu_budget_s)
+    return result
 
 
 if __name__ == "__main__":
