@@ -69,6 +69,9 @@ SECONDARY_WORKLOADS = {
     "prefill_d192": ("prefill", dict(Hq=32, Hkv=8, d=192, n=8, new=2048, ctx=2048)),
     "prefill_d256": ("prefill", dict(Hq=32, Hkv=8, d=256, n=8, new=2048, ctx=2048)),
     "prefill_d128_mqa": ("prefill", dict(Hq=64, Hkv=2, d=128, n=8, new=2048, ctx=2048)),
+    # the projections either side of the path at decode size (cfg2's layer: hidden 4096, 32 / 8 heads of 128)
+    "qkv_proj_decode": ("linear", dict(T=64, N=6144, K=4096, bias=True)),
+    "out_proj_decode": ("linear", dict(T=64, N=4096, K=4096, bias=False)),
     "sampling_top_k": ("sampling", dict(R=64, V=128256, top_k=50, top_p=0.0)),
     "sampling_top_p": ("sampling", dict(R=64, V=128256, top_k=0, top_p=0.9)),
     "sampling_top_p_peaked": ("sampling", dict(R=64, V=128256, top_k=0, top_p=0.9, peaked=True)),
@@ -122,6 +125,20 @@ def run_secondary(args, mi, lib, torch, dev):
         kernel = "paged_prefill_woven_kernel" if (not mla and dk == 128) else "paged_prefill_pp_kernel"
         what = (f"paged varlen causal attention, {n} x {new} new tokens over {ctx} cached, {Hq}/{Hkv} heads, "
                 f"keys {dk} / values {dv} wide, chunk 256")
+        dtype = "bf16 (fp32 accumulate)"
+        timed_by_library = True
+    elif kind == "linear":
+        T, N, K = prm["T"], prm["N"], prm["K"]
+        x = (torch.randn(T, K, generator=gen) * 0.5).bfloat16().to(dev)
+        w = torch.empty(N, K, dtype=torch.bfloat16, device=dev).normal_(0, K ** -0.5)
+        bias_t = torch.randn(N, generator=gen).bfloat16().to(dev) if prm["bias"] else None
+        out = torch.empty(T, N, dtype=torch.bfloat16, device=dev)
+        step = lambda: mi.ops.linear_decode(x, w, bias_t, out=out)
+        nbytes = N * K * 2 + T * K * 2 + T * N * 2 + (N * 2 if prm["bias"] else 0)
+        flops = 2 * T * N * K
+        kernel = "linear_decode_kernel"
+        what = (f"y[{T}, {N}] = x[{T}, {K}] . W[{N}, {K}]^T{' + bias' if prm['bias'] else ''}: the weight matrix streamed "
+                f"once, fp32 partial sums over slices of K and their reduction launch included in the step")
         dtype = "bf16 (fp32 accumulate)"
         timed_by_library = True
     elif kind == "sampling":
@@ -184,6 +201,19 @@ def run_secondary(args, mi, lib, torch, dev):
                 {"bound": "hbm", "kernel": kernel, "achieved": round(nbytes / kernel_ms / 1e6, 1), "peak": HBM_PEAK_GBPS,
                  "unit": "GB/s", "frac": round(nbytes / kernel_ms / 1e6 / HBM_PEAK_GBPS, 4)})
     roofline.update({"kernel_ms": round(kernel_ms, 5), "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload)})
+    if kind == "linear":
+        # the library's GEMM on the same operands, timed the same way (what the reference's linear layers call)
+        lin = lambda: torch.nn.functional.linear(x, w, bias_t)
+        for _ in range(args.warmup):
+            lin()
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+        for a, b2 in ev:
+            a.record()
+            lin()
+            b2.record()
+        torch.cuda.synchronize()
+        roofline["library_gemm_ms"] = round(sum(a.elapsed_time(b2) for a, b2 in ev) / args.steps, 5)
+        roofline["call_ms"] = round(call_ms, 5)
     if args.workload in TRAFFIC_SOURCE:
         roofline["traffic_source"] = TRAFFIC_SOURCE[args.workload]
     return ({

@@ -551,6 +551,45 @@ int mi_sample_from_logits(const void* logits, int64_t stride_row, int32_t logits
                           const int32_t* request_output_lengths, int64_t termination_id,
                           uint8_t* active_request_mask, void* stream);
 
+/*
+ * The projections either side of the attention path at decode size (at most 256 tokens a call):
+ *   y[T, N] = x[T, K] . W[N, K]^T (+ bias[N]),   16-bit x / W / bias / y, fp32 accumulation.
+ * The weight matrix is streamed from HBM once (it is the traffic: 50 MB for 4096 -> 6144), its rows riding
+ * through the matrix cores; K is cut into slices of at most 512 columns whose fp32 partial sums [slice][T][N]
+ * live in the caller's workspace and are added in a fixed order by a second small launch (results do not depend
+ * on timing).  N a multiple of 16, K a multiple of 32; x, W and y rows 16-byte aligned (y: 8-byte).
+ *
+ * mi_linear_qkv_decode_step replaces `mixed_qkv, _ = self.linear_qkv(hidden_states)` of
+ * Attention.get_query_key_value_tensors (megatron/core/transformer/attention.py:985-992; ColumnParallelLinear at
+ * tensor-parallel size 1, megatron/core/tensor_parallel/layers.py:946-1010): qkv_weight is
+ * `[(Hq + 2 Hkv) d, hidden]` with the rows of KV group h laid out as [G query heads | key | value], so mixed_qkv
+ * is the `[T, Hkv, (G + 2) d]` tensor that mi_decode_step_attention and mi_qkv_norm_rope_append read as it is:
+ * the split, q / k head norm, rotary embedding and cache append of attention.py:994-1030 and :394-414 then run in
+ * THEIR prologue, and no per-head q / k / v tensor is ever written.
+ *
+ * mi_attention_out_linear_proj replaces `output, bias = self.linear_proj(core_attn_out)` (attention.py:829-845;
+ * RowParallelLinear with skip_bias_add, layers.py:1225-1290: the bias is handed back to the caller, not added):
+ * core_attn_out is the `[T, Hq d]` output of the attention call, proj_weight `[hidden, Hq d]`.
+ *
+ * mi_linear_decode is the product itself, for any (N, K) within the limits above.
+ */
+int64_t mi_linear_decode_workspace_bytes(int32_t T, int32_t N, int32_t K);
+
+int mi_linear_decode(const void* x, int64_t x_stride_tok, const void* weight, int64_t w_stride_row,
+                     const void* bias, void* out, int64_t out_stride_tok, void* workspace,
+                     int64_t workspace_bytes, int32_t T, int32_t N, int32_t K, int32_t dtype, void* stream);
+
+int mi_linear_qkv_decode_step(const void* hidden_states, int64_t x_stride_tok, const void* qkv_weight,
+                              int64_t w_stride_row, const void* qkv_bias, void* mixed_qkv,
+                              int64_t out_stride_tok, void* workspace, int64_t workspace_bytes, int32_t T,
+                              int32_t hidden_size, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t dtype,
+                              void* stream);
+
+int mi_attention_out_linear_proj(const void* core_attn_out, int64_t x_stride_tok, const void* proj_weight,
+                                 int64_t w_stride_row, void* output, int64_t out_stride_tok, void* workspace,
+                                 int64_t workspace_bytes, int32_t T, int32_t hidden_size, int32_t Hq,
+                                 int32_t head_dim, int32_t dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,9 +15,11 @@ Public surface (same names as the reference wherever one exists):
 * :mod:`step` -- ``generate_output_tokens_dynamic_batch``: one engine step on a context with the
   model behind a callable (reference: the same file, :411-546).
 """
-from . import ops, sampling, step, synthetic  # noqa: F401
+from . import attention, ops, sampling, step, synthetic  # noqa: F401
 from .attention import (  # noqa: F401
+    DecodeLinear,
     PagedSelfAttentionCore,
+    PagedSelfAttentionLayer,
     adjust_key_value_for_inference,
     flash_decode_and_prefill,
 )

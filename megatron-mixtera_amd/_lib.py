@@ -88,6 +88,12 @@ SIGNATURES = {
         c_int,
         [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F,
          _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _P, _P]),
+    "mi_linear_decode_workspace_bytes": (_I64, [_I32, _I32, _I32]),
+    "mi_linear_decode": (c_int, [_P, _I64, _P, _I64, _P, _P, _I64, _P, _I64, _I32, _I32, _I32, _I32, _P]),
+    "mi_linear_qkv_decode_step": (
+        c_int, [_P, _I64, _P, _I64, _P, _P, _I64, _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
+    "mi_attention_out_linear_proj": (
+        c_int, [_P, _I64, _P, _I64, _P, _I64, _P, _I64, _I32, _I32, _I32, _I32, _I32, _P]),
     "mi_qkv_norm_rope_append": (
         c_int,
         [_P, _I64, _P, _I64, _P, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F,

@@ -175,3 +175,61 @@ class PagedSelfAttentionCore(torch.nn.Module):
         out = flash_decode_and_prefill(query, k_cache, v_cache, max_q, max_k, cu_q, cu_k, kv_lens, block_table,
                                        softmax_scale=self.softmax_scale, k_scales=k_scales, v_scales=v_scales)
         return out.reshape(out.size(0), out.size(1), -1)
+
+
+class DecodeLinear(torch.nn.Module):
+    """``linear_qkv`` / ``linear_proj`` of the attention layer at tensor-parallel size 1, with the reference's call
+    contract (megatron/core/tensor_parallel/layers.py:946-1010 ColumnParallelLinear, :1225-1290 RowParallelLinear):
+    ``forward(input_) -> (output, output_bias)``, where the bias is added to the output unless ``skip_bias_add`` and
+    is handed back instead when it is.  Steps of at most 256 rows run the weight-streaming kernel
+    (``ops.linear_decode``); larger (prompt-sized) inputs are plain library GEMMs.
+    """
+
+    DECODE_ROWS = 256
+
+    def __init__(self, input_size: int, output_size: int, *, bias: bool = True, skip_bias_add: bool = False,
+                 dtype: torch.dtype = torch.bfloat16, device=None):
+        super().__init__()
+        self.input_size, self.output_size, self.skip_bias_add = input_size, output_size, skip_bias_add
+        self.weight = torch.nn.Parameter(torch.empty(output_size, input_size, dtype=dtype, device=device))
+        self.bias = torch.nn.Parameter(torch.zeros(output_size, dtype=dtype, device=device)) if bias else None
+
+    def forward(self, input_: Tensor):
+        from . import ops
+        add = None if (self.bias is None or self.skip_bias_add) else self.bias.data
+        rows = input_.numel() // input_.size(-1)
+        if rows <= self.DECODE_ROWS:
+            output = ops.linear_decode(input_, self.weight.data, add)
+        else:
+            output = torch.nn.functional.linear(input_, self.weight, add)
+        return output, (self.bias if self.skip_bias_add else None)
+
+
+class PagedSelfAttentionLayer(torch.nn.Module):
+    """One attention layer of the dynamic inference path from hidden states to hidden states: what
+    ``Attention.forward`` does with a dynamic ``inference_context`` (attention.py:603-847) --
+    ``get_query_key_value_tensors`` (:985-1030), ``_adjust_key_value_for_inference`` (:394-414), rotary embedding of
+    the query (:740-790), ``flash_decode_and_prefill`` (:470-601) and ``linear_proj`` (:829-845) -- as three launches
+    on a decode step: the QKV projection writes the mixed ``[T, Hkv, (G + 2) d]`` tensor, the streaming kernel reads it
+    directly (split, head norm, rotary embedding and cache append in its prologue) and the output projection follows
+    the merge.  Returns ``(output, bias)`` like the reference.
+    """
+
+    def __init__(self, layer_number: int, hidden_size: int, num_query_heads: int, num_kv_heads: int, head_dim: int, *,
+                 qk_norm: Optional[str] = None, eps: float = 1e-5, add_qkv_bias: bool = False,
+                 add_bias_linear: bool = False, softmax_scale: Optional[float] = None, rotary_interleaved: bool = False,
+                 dtype: torch.dtype = torch.bfloat16, device=None):
+        super().__init__()
+        self.num_query_heads, self.num_kv_heads, self.head_dim = num_query_heads, num_kv_heads, head_dim
+        self.linear_qkv = DecodeLinear(hidden_size, (num_query_heads + 2 * num_kv_heads) * head_dim,
+                                       bias=add_qkv_bias or add_bias_linear, skip_bias_add=False, dtype=dtype, device=device)
+        self.core = PagedSelfAttentionCore(layer_number, head_dim, qk_norm=qk_norm, eps=eps, softmax_scale=softmax_scale,
+                                           rotary_interleaved=rotary_interleaved, dtype=dtype, device=device)
+        self.linear_proj = DecodeLinear(num_query_heads * head_dim, hidden_size, bias=add_bias_linear,
+                                        skip_bias_add=True, dtype=dtype, device=device)
+
+    def forward(self, hidden_states: Tensor, inference_context,
+                rotary_pos_emb: Optional[Tuple[Tensor, Tensor]] = None):
+        mixed_qkv, _ = self.linear_qkv(hidden_states)
+        core_attn_out = self.core.forward_mixed_qkv(mixed_qkv, self.num_query_heads, inference_context, rotary_pos_emb)
+        return self.linear_proj(core_attn_out)

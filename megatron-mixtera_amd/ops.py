@@ -48,15 +48,23 @@ def _cache_strides(cache: Tensor) -> Tuple[int, int, int]:
 # overlap, so each stream gets its own.
 _workspaces: dict = {}
 _retired_workspaces: list = []   # outgrown buffers stay alive: work already enqueued may still use them
-_workspace_override: list = []   # innermost ``use_workspace`` buffer
+_override_local = threading.local()   # ``use_workspace`` buffers of THIS thread (innermost last)
+
+
+def _override_stack() -> list:
+    stack = getattr(_override_local, "stack", None)
+    if stack is None:
+        stack = _override_local.stack = []
+    return stack
 
 
 def _workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) -> Optional[Tensor]:
     """Scratch for a call on ``stream`` (the handle the caller already looked up; default: the current one)."""
     if nbytes <= 0:
         return None
-    if _workspace_override:
-        ws = _workspace_override[-1]
+    override = _override_stack()
+    if override:
+        ws = override[-1]
         _require(ws.device == device and ws.numel() >= nbytes, "the workspace given to use_workspace is too small")
         return ws
     key = (device, torch.cuda.current_stream(device).cuda_stream if stream is None else stream)
@@ -64,24 +72,27 @@ def _workspace(device: torch.device, nbytes: int, stream: Optional[int] = None) 
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
             _retired_workspaces.append(ws)
+            if len(_retired_workspaces) > 8:  # enqueued work may still use them: wait for it once, then let them go
+                torch.cuda.synchronize(device)
+                _retired_workspaces.clear()
         ws = torch.empty(max(nbytes, 2 * (0 if ws is None else ws.numel())), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 
 
 class use_workspace:
-    """Context manager: attention calls inside use ``buffer`` as their scratch instead of the
-    per-device one (graph capture needs a buffer that is never re-allocated)."""
+    """Context manager: attention calls this thread makes inside use ``buffer`` as their scratch instead of the
+    per-stream one (graph capture needs a buffer that is never re-allocated).  Other threads are not affected."""
 
     def __init__(self, buffer: Tensor):
         self.buffer = buffer
 
     def __enter__(self):
-        _workspace_override.append(self.buffer)
+        _override_stack().append(self.buffer)
         return self.buffer
 
     def __exit__(self, *exc):
-        _workspace_override.pop()
+        _override_stack().pop()
         return False
 
 
@@ -416,7 +427,7 @@ def paged_mla_decode_attention(q: Tensor, kv_cache: Tensor, kv_lens: Tensor, blo
     o3 = _qo_view(out, "out")
     _require(tuple(o3.shape) == (R, Hq, head_dim_v), "out shape mismatch")
     tune = _tuning_arg()
-    workspace = _workspace(q.device, lib.mi_mla_decode_workspace_bytes(R, Hq, head_dim_v, tune))
+    workspace = _workspace(q.device, lib.mi_mla_decode_workspace_bytes(R, Hq, head_dim_v, tune), stream)
     _lib.check(lib.mi_paged_mla_decode_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), kv_cache.data_ptr(), kv_cache.stride(0), kv_cache.stride(1),
         block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
@@ -457,10 +468,11 @@ def paged_prefill_attention_mla(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_
         max_kv_len = block_table.size(1) * C
     tune = _tuning_arg()
     need = lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, Dv, int(max_kv_len), 0, tune)
-    if _workspace_override and _workspace_override[-1].numel() < need:
+    override = _override_stack()
+    if override and override[-1].numel() < need:
         workspace = None  # the split of the keys is optional here: a caller-sized workspace that is too small turns it off
     else:
-        workspace = _workspace(q.device, need)
+        workspace = _workspace(q.device, need, stream)
     ws_bytes = 0 if workspace is None else workspace.numel()
     _lib.check(lib.mi_paged_prefill_attention_mla(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), ksc, kst, ksh, v_cache.data_ptr(), vsc, vst, vsh,
@@ -508,7 +520,8 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
     o3 = _qo_view(out, "out")
     _require(tuple(o3.shape) == (T, Hq, D) and o3.dtype == q3.dtype, "out shape / dtype mismatch")
     tune = _tuning_arg()
-    workspace = _workspace(q.device, lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, D, int(max_kv_len), 0, tune))
+    stream = _stream(q)
+    workspace = _workspace(q.device, lib.mi_prefill_workspace_bytes(T, R, Hq, Hkv, D, int(max_kv_len), 0, tune), stream)
     ws_bytes = 0 if workspace is None else workspace.numel()
     if fp8:
         _lib.check(lib.mi_paged_prefill_attention_fp8(
@@ -516,14 +529,14 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
             k_scales.data_ptr(), v_scales.data_ptr(), block_table.data_ptr(), block_table.stride(0),
             cu_seqlens_q.data_ptr(), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
             _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C, int(max_kv_len), 0, float(softmax_scale), tune,
-            _stream(q)), "mi_paged_prefill_attention_fp8")
+            stream), "mi_paged_prefill_attention_fp8")
         return out
     _lib.check(lib.mi_paged_prefill_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
         block_table.data_ptr(), block_table.stride(0), cu_seqlens_q.data_ptr(), kv_lens.data_ptr(),
         o3.data_ptr(), o3.stride(0), o3.stride(1), _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C,
         int(max_kv_len), 0,
-        float(softmax_scale), _dtype_code(q3, "q"), tune, _stream(q)), "mi_paged_prefill_attention")
+        float(softmax_scale), _dtype_code(q3, "q"), tune, stream), "mi_paged_prefill_attention")
     return out
 
 
@@ -912,3 +925,30 @@ def sample_from_logits(logits: Tensor, *, top_k: int = 0, top_p: float = 0.0, te
         _ptr(kv_length_offsets), _ptr(query_lengths), _ptr(output_lengths),
         int(termination_id) if termination_id is not None else -1, _ptr(mask), stream), "mi_sample_from_logits")
     return (samples, mask, cut) if return_cut else (samples, mask)
+
+
+def linear_decode(x: Tensor, weight: Tensor, bias: Optional[Tensor] = None, out: Optional[Tensor] = None) -> Tensor:
+    """``x @ weight.T (+ bias)`` for a decode-sized step (at most 256 rows of ``x``): the weight matrix streams from
+    HBM once.  ``x`` is ``[..., K]`` (leading dimensions are flattened to rows), ``weight`` ``[N, K]``; the result
+    has ``x``'s leading dimensions and ``N`` columns.  What ``linear_qkv`` / ``linear_proj`` of the attention layer
+    compute at tensor-parallel size 1 (``mi_linear_decode`` of the header)."""
+    _require(weight.dim() == 2 and weight.stride(1) == 1, "weight must be [N, K] with contiguous rows")
+    N, K = weight.shape
+    _require(x.size(-1) == K and x.stride(-1) == 1, "x must be [..., K] with a contiguous last dimension")
+    _require(x.dtype == weight.dtype and (bias is None or bias.dtype == x.dtype), "x, weight and bias share one 16-bit type")
+    x2 = x.reshape(-1, K)
+    T = x2.size(0)
+    if out is None:
+        out = torch.empty(*x.shape[:-1], N, dtype=x.dtype, device=x.device)
+    o2 = out.view(-1, N)
+    _require(o2.size(0) == T and o2.stride(1) == 1, "out must be [..., N] with a contiguous last dimension")
+    if bias is not None:
+        _require(bias.numel() == N and bias.is_contiguous(), "bias must be a contiguous [N] vector")
+    lib = _lib.load()
+    stream = _stream(x)
+    nbytes = lib.mi_linear_decode_workspace_bytes(T, N, K)
+    ws = _workspace(x.device, nbytes, stream)
+    _lib.check(lib.mi_linear_decode(x2.data_ptr(), x2.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
+                                    o2.data_ptr(), o2.stride(0), _ptr(ws), 0 if ws is None else ws.numel(), T, N, K,
+                                    _dtype_code(x, "x"), stream), "mi_linear_decode")
+    return out
