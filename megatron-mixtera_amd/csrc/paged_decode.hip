@@ -1458,12 +1458,23 @@ __global__ __launch_bounds__(256, 1) void paged_mla_decode_heads_kernel(DecodePa
 // shared the request; zero-length rows get zeros.  blockDim.x = HD * S: S groups of HD threads take the
 // segments round-robin in batches of 8 (a request cut over hundreds of workgroups is a chain of dependent
 // memory round trips otherwise) and group 0 folds the S running (maximum, numerator, denominator) triples.
-template <int HD, bool F16>
-__global__ __launch_bounds__(1024) void paged_decode_merge_kernel(DecodeParams p) {
-  constexpr int kMaxGroups = 1024 / HD;
-  __shared__ float red[3][kMaxGroups > 1 ? 1024 : 1];
-  const int r = blockIdx.y, hq = blockIdx.x, d = threadIdx.x % HD, grp = threadIdx.x / HD;
-  const int groups = blockDim.x / HD;
+// One workgroup per (request, block of heads): a thread owns four neighbouring output values of one head (16-byte
+// loads of the fp32 partials, one 8-byte store), `cols` = heads-per-workgroup x head_dim / 4 threads cover the block
+// and `groups` such thread groups take the request's segments round-robin in batches of 8 loads; group 0 folds their
+// (maximum, numerators, denominator) through LDS.
+struct MergeShape {
+  int hd;        // width of the output rows (values per head)
+  int hpw;       // heads per workgroup
+  int cols;      // threads per group = hpw * hd / 4
+  int groups;    // thread groups (blockDim.x = cols * groups)
+};
+template <bool F16>
+__global__ __launch_bounds__(1024) void paged_decode_merge_kernel(DecodeParams p, MergeShape ms) {
+  __shared__ float red[6][1024];
+  const int r = blockIdx.y;
+  const int col = threadIdx.x % ms.cols, grp = threadIdx.x / ms.cols;
+  const int q4 = ms.hd >> 2;
+  const int hq = blockIdx.x * ms.hpw + col / q4, d = 4 * (col % q4);
   int row;
   if (!decode_row(p, r, row)) return;
   // The kernel is a chain of dependent memory round trips, so everything that does not depend
@@ -1471,57 +1482,80 @@ __global__ __launch_bounds__(1024) void paged_decode_merge_kernel(DecodeParams p
   // of every segment together (the running-maximum form below needs no first pass over the LSEs).
   const int len = p.lens[r];
   const int first = p.seg_info[2 * r], last = p.seg_info[2 * r + 1];  // stale for len <= 0: not used then
-  uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)hq * p.o_sh + d;
+  const bool live = hq < p.Hq;                                        // (the last block of heads may be partial)
+  uint16_t* o = p.out + (int64_t)row * p.o_st + (int64_t)(live ? hq : 0) * p.o_sh + d;
   if (len <= 0) {  // (uniform over the workgroup, like the two returns around it)
-    if (grp == 0) *o = 0;
+    if (grp == 0 && live) st8(o, make_uint2(0u, 0u));
     return;
   }
   if (first == last) return;  // written directly by the streaming kernel
-  float mx = -INFINITY, num = 0.f, den = 0.f;
-  for (int w0 = first + 8 * grp; w0 <= last; w0 += 8 * groups) {
-    float lse[8], po[8];
+  float mx = -INFINITY, den = 0.f;
+  float4 num = make_float4(0.f, 0.f, 0.f, 0.f);
+  const int hq_c = live ? hq : p.Hq - 1;
+  for (int w0 = first + 8 * grp; w0 <= last; w0 += 8 * ms.groups) {
+    float lse[8];
+    float4 po[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const int64_t slot = (int64_t)(min(w0 + j, last) + r) * p.Hq + hq;
+      const int64_t slot = (int64_t)(min(w0 + j, last) + r) * p.Hq + hq_c;
       lse[j] = p.part_lse[slot];
-      po[j] = p.part_o[slot * HD + d];
+      po[j] = *reinterpret_cast<const float4*>(p.part_o + slot * ms.hd + d);
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       if (w0 + j <= last) {
         const float m_new = fmaxf(mx, lse[j]);
         const float a = fast_exp2(mx - m_new), wt = fast_exp2(lse[j] - m_new);
-        num = num * a + wt * po[j];
+        num.x = num.x * a + wt * po[j].x; num.y = num.y * a + wt * po[j].y;
+        num.z = num.z * a + wt * po[j].z; num.w = num.w * a + wt * po[j].w;
         den = den * a + wt;
         mx = m_new;
       }
     }
   }
-  if (kMaxGroups > 1 && groups > 1) {
-    red[0][threadIdx.x] = mx; red[1][threadIdx.x] = num; red[2][threadIdx.x] = den;
+  if (ms.groups > 1) {
+    red[0][threadIdx.x] = mx; red[1][threadIdx.x] = den;
+    red[2][threadIdx.x] = num.x; red[3][threadIdx.x] = num.y; red[4][threadIdx.x] = num.z; red[5][threadIdx.x] = num.w;
     __syncthreads();
     if (grp != 0) return;
-    for (int g2 = 1; g2 < groups; ++g2) {
-      const float m2 = red[0][g2 * HD + d];
+    for (int g2 = 1; g2 < ms.groups; ++g2) {
+      const int t = g2 * ms.cols + col;
+      const float m2 = red[0][t];
       if (m2 == -INFINITY) continue;  // that group had no segment
       const float m_new = fmaxf(mx, m2);
       const float a = fast_exp2(mx - m_new), wt = fast_exp2(m2 - m_new);
-      num = num * a + wt * red[1][g2 * HD + d];
-      den = den * a + wt * red[2][g2 * HD + d];
+      num.x = num.x * a + wt * red[2][t]; num.y = num.y * a + wt * red[3][t];
+      num.z = num.z * a + wt * red[4][t]; num.w = num.w * a + wt * red[5][t];
+      den = den * a + wt * red[1][t];
       mx = m_new;
     }
   }
-  *o = f32_to_16<F16>(num / den);
+  if (!live) return;
+  const float inv = 1.f / den;
+  st8(o, make_uint2(pack2<F16>(num.x * inv, num.y * inv), pack2<F16>(num.z * inv, num.w * inv)));
 }
 
-// Thread groups per merge workgroup: one per 8 segments a request is expected to be cut into.
-static int merge_groups(int grid_x, int R, int head_dim) {
+// Shape of the merge launch: about 256 threads per thread group (whole heads), one group per 8 segments a request
+// is expected to be cut into, as far as 1024 threads go.
+static MergeShape merge_shape(int grid_x, int R, int Hq, int head_dim) {
+  MergeShape ms;
+  ms.hd = head_dim;
+  const int q4 = head_dim / 4;
+  ms.hpw = 256 / q4 > 0 ? 256 / q4 : 1;
+  if (ms.hpw > Hq) ms.hpw = Hq;
+  ms.cols = ms.hpw * q4;
   const int per_request = grid_x / (R > 0 ? R : 1) + 2;
   int g = (per_request + 7) / 8;
-  const int cap = 1024 / head_dim;
-  if (g > cap) g = cap;
+  if (g > 1024 / ms.cols) g = 1024 / ms.cols;
   if (g > 8) g = 8;
-  return g < 1 ? 1 : g;
+  ms.groups = g < 1 ? 1 : g;
+  return ms;
+}
+static void launch_merge(const DecodeParams& p, int grid_x, int R, int Hq, int head_dim, bool f16, hipStream_t st) {
+  const MergeShape ms = merge_shape(grid_x, R, Hq, head_dim);
+  const dim3 mgrid((Hq + ms.hpw - 1) / ms.hpw, R), mblock(ms.cols * ms.groups);
+  if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<true>), mgrid, mblock, 0, st, p, ms);
+  else hipLaunchKernelGGL((paged_decode_merge_kernel<false>), mgrid, mblock, 0, st, p, ms);
 }
 
 // Requests one launch of the streaming kernels takes: their tile prefix sums and lengths sit in LDS.
@@ -1738,19 +1772,7 @@ int mi::launch_paged_decode(
 #undef MI_LAUNCH_DECODE_WIDE
 #undef MI_LAUNCH_STEP
   if (timed) (void)hipEventRecord(ev_b, st);
-  dim3 mgrid(Hq, R);
-  const dim3 mblock(head_dim * merge_groups(p.grid, R, head_dim));
-#define MI_LAUNCH_MERGE(HD_)                                                                                          \
-  do {                                                                                                                 \
-    if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<HD_, true>), mgrid, mblock, 0, st, p);                      \
-    else hipLaunchKernelGGL((paged_decode_merge_kernel<HD_, false>), mgrid, mblock, 0, st, p);                         \
-  } while (0)
-  if (head_dim == 128) MI_LAUNCH_MERGE(128);
-  else if (head_dim == 64) MI_LAUNCH_MERGE(64);
-  else if (head_dim == 96) MI_LAUNCH_MERGE(96);
-  else if (head_dim == 192) MI_LAUNCH_MERGE(192);
-  else MI_LAUNCH_MERGE(256);
-#undef MI_LAUNCH_MERGE
+  launch_merge(p, p.grid, R, Hq, head_dim, f16, st);
   return mi_check_launch("mi_paged_decode_attention");
 }
 
@@ -2050,8 +2072,6 @@ extern "C" int mi_paged_mla_decode_attention(
   if (f16) MI_LAUNCH_MLA(true); else MI_LAUNCH_MLA(false);
 #undef MI_LAUNCH_MLA
   if (timed) (void)hipEventRecord(ev_b, st);
-  const dim3 mgrid(Hq, R), mblock(512 * merge_groups(grid_x, R, 512));
-  if (f16) hipLaunchKernelGGL((paged_decode_merge_kernel<512, true>), mgrid, mblock, 0, st, p);
-  else hipLaunchKernelGGL((paged_decode_merge_kernel<512, false>), mgrid, mblock, 0, st, p);
+  launch_merge(p, grid_x, R, Hq, 512, f16, st);
   return mi_check_launch("mi_paged_mla_decode_attention");
 }
