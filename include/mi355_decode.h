@@ -209,8 +209,8 @@ int mi_paged_decode_attention(const void* q, int64_t q_stride_tok, int64_t q_str
  * in its request (what token_to_pos_ids holds on a decode step, and one load fewer on the way to the first
  * product).  Same arithmetic and rounding points as
  * mi_norm_rope_append (faithful_rounding as there); the normed queries are not written anywhere.
- * Limits: 16-bit caches, head_dim 64 or 128, half-split rotary pairs with rot_dim / 2 a multiple of 32 (or
- * interleaved pairs, or no rotary embedding); anything else is MI_ERR_UNSUPPORTED and takes the separate calls.
+ * Limits: 16-bit caches, head_dim 64, 96, 128, 192 or 256, half-split rotary pairs with rot_dim / 2 a multiple of
+ * 32 (or interleaved pairs, or no rotary embedding); anything else is MI_ERR_UNSUPPORTED and takes the separate calls.
  * Workspace as for mi_paged_decode_attention.  Rows with kv_lens[r] == 0 append nothing and produce zeros.
  */
 int mi_decode_step_attention(const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new,

@@ -119,7 +119,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   constexpr int VD = FP8 ? 2 : DV / 2;  // dwords per token and lane of the value operand
   static_assert(HDK % 32 == 0 && HDV % 32 == 0 && HDK >= 64 && HDV >= 64, "head widths: multiples of 32");
   static_assert(!FP8 || (HDK == 128 && HDV == 128 && !F16), "fp8 KV: head_dim 128, bf16 queries");
-  static_assert(!FUSED || (!FP8 && HDK == HDV && (HDK == 64 || HDK == 128)), "fused step: head_dim 64 or 128, 16-bit cache");
+  static_assert(!FUSED || (!FP8 && HDK == HDV && HDK <= 256), "fused step: an ordinary 16-bit cache");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
   // tile base addresses below run on the scalar unit instead of costing vector instructions.
@@ -360,11 +360,19 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
             }
           }
         }
-      } else if (KS == 4 && p.rot == 128) {  // partners 64 elements = two fragments apart
-        rotate_pair(0, 2 % KS);
-        rotate_pair(1, 3 % KS);
-      } else {  // rot_dim 64: fragments 0 and 1 pair up; fragments 2, 3 (head_dim 128) pass through
-        rotate_pair(0, 1);
+      } else {
+        // half-split pairs: partners are rot_dim / 2 elements = nf fragments apart (the entry point admits only
+        // whole numbers of fragments); fragments beyond the rotary width pass through
+        const int nf = p.rot >> 6;
+        if (nf == 1) {
+          rotate_pair(0, 1);
+        } else if (nf == 2) {
+          if constexpr (KS >= 4) { rotate_pair(0, 2); rotate_pair(1, 3); }
+        } else if (nf == 3) {
+          if constexpr (KS >= 6) { rotate_pair(0, 3); rotate_pair(1, 4); rotate_pair(2, 5); }
+        } else {
+          if constexpr (KS >= 8) { rotate_pair(0, 4); rotate_pair(1, 5); rotate_pair(2, 6); rotate_pair(3, 7); }
+        }
       }
     }
 #pragma unroll
@@ -774,8 +782,8 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
 
 // The same stream over the raw queries, keys and values of a decode step: head norm, rotary embedding and the
 // append of the new token ride in the segment prologues (see decode_segment).
-template <int HD, int NT, bool F16>
-__global__ __launch_bounds__(512, 3) void decode_step_stream_kernel(DecodeParams p) {
+template <int HD, int NT, bool F16, int MINW = 3>
+__global__ __launch_bounds__(512, MINW) void decode_step_stream_kernel(DecodeParams p) {
   decode_stream_body<HD, HD, NT, false, F16, true>(p);
 }
 
@@ -1753,10 +1761,17 @@ int mi::launch_paged_decode(
     else hipLaunchKernelGGL((paged_decode_stream_kernel<HD_, 1, false, 2, F16_>), grid, block, lds, st, p);               \
   } while (0)
 #define MI_LAUNCH_STEP(HD_, F16_) hipLaunchKernelGGL((decode_step_stream_kernel<HD_, 1, F16_>), grid, block, lds, st, p)
+#define MI_LAUNCH_STEP_WIDE(HD_, F16_) hipLaunchKernelGGL((decode_step_stream_kernel<HD_, 1, F16_, 2>), grid, block, lds, st, p)
   if (fused && head_dim == 128 && f16) MI_LAUNCH_STEP(128, true);
   else if (fused && head_dim == 128) MI_LAUNCH_STEP(128, false);
-  else if (fused && f16) MI_LAUNCH_STEP(64, true);
-  else if (fused) MI_LAUNCH_STEP(64, false);
+  else if (fused && head_dim == 64 && f16) MI_LAUNCH_STEP(64, true);
+  else if (fused && head_dim == 64) MI_LAUNCH_STEP(64, false);
+  else if (fused && head_dim == 96 && f16) MI_LAUNCH_STEP(96, true);
+  else if (fused && head_dim == 96) MI_LAUNCH_STEP(96, false);
+  else if (fused && head_dim == 192 && f16) MI_LAUNCH_STEP_WIDE(192, true);
+  else if (fused && head_dim == 192) MI_LAUNCH_STEP_WIDE(192, false);
+  else if (fused && f16) MI_LAUNCH_STEP_WIDE(256, true);
+  else if (fused) MI_LAUNCH_STEP_WIDE(256, false);
   else if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true, false);
   else if (head_dim == 128 && f16) MI_LAUNCH_DECODE(128, false, true);
   else if (head_dim == 128) MI_LAUNCH_DECODE(128, false, false);
@@ -1771,6 +1786,7 @@ int mi::launch_paged_decode(
 #undef MI_LAUNCH_DECODE
 #undef MI_LAUNCH_DECODE_WIDE
 #undef MI_LAUNCH_STEP
+#undef MI_LAUNCH_STEP_WIDE
   if (timed) (void)hipEventRecord(ev_b, st);
   launch_merge(p, p.grid, R, Hq, head_dim, f16, st);
   return mi_check_launch("mi_paged_decode_attention");
@@ -1816,8 +1832,8 @@ extern "C" int mi_decode_step_attention(
   if (rc != MI_OK) return rc;
   if (!q || !k_new || !v_new || !k_cache || !v_cache) return fail(MI_ERR_NULL, "null pointer argument");
   if (R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) return fail(MI_ERR_SHAPE, "need R >= 0 and Hq a multiple of Hkv");
-  if (head_dim != 64 && head_dim != 128)
-    return fail(MI_ERR_UNSUPPORTED, "head_dim must be 64 or 128 (other widths: the separate norm / rotary / append and attention calls)");
+  if (head_dim != 64 && head_dim != 96 && head_dim != 128 && head_dim != 192 && head_dim != 256)
+    return fail(MI_ERR_UNSUPPORTED, "head_dim must be 64, 96, 128, 192 or 256");
   if (norm_kind != MI_NORM_NONE && norm_kind != MI_NORM_RMS && norm_kind != MI_NORM_L2)
     return fail(MI_ERR_UNSUPPORTED, "unknown norm kind");
   if (rotary_angles) {

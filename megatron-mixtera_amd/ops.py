@@ -685,7 +685,7 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
 # ---------------------------------------------------------------------------------------------
 def decode_step_supported(head_dim: int, rot_dim: int, rotary_interleaved: bool, fp8_cache: bool) -> bool:
     """Whether :func:`decode_step_attention` has a kernel for these shapes (else: the separate calls)."""
-    if fp8_cache or head_dim not in (64, 128):
+    if fp8_cache or head_dim not in (64, 96, 128, 192, 256):
         return False
     return rot_dim == 0 or rotary_interleaved or (rot_dim // 2) % 32 == 0
 

@@ -103,6 +103,32 @@ def test_fused_step_equals_the_separate_launches(mi, dev, Hq, Hkv, d, rotary, no
     _close(kc_a[:dummy], kc_ref[:dummy], 2e-2, "key cache vs checker")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
+@pytest.mark.parametrize("mixed", [False, True])
+@pytest.mark.parametrize("Hq,Hkv,d,rot,interleaved", [
+    (12, 4, 96, 0, False), (12, 4, 96, 64, False), (12, 4, 96, 96, True), (24, 1, 96, 64, False),
+    (8, 2, 192, 192, False), (8, 2, 192, 128, False), (8, 2, 192, 64, False), (8, 2, 192, 192, True),
+    (16, 2, 256, 256, False), (16, 2, 256, 128, False), (16, 2, 256, 64, False), (16, 2, 256, 0, False),
+    (4, 4, 256, 200, True)])
+def test_fused_step_at_head_widths_96_192_256(mi, dev, Hq, Hkv, d, rot, interleaved, mixed, dtype):
+    """The one-kernel decode step at the other head widths (two wavefronts per SIMD at 192 and 256): half-split
+    rotary pairs a whole number of 32-element fragments apart (rot_dim 64, 128, 192 or 256), interleaved pairs of
+    any even width, no rotary embedding; per-head and mixed (projection-output) inputs."""
+    table = orn.rotary_table(4096, rot, base=500000.0, interleaved=interleaved) if rot else None
+    case, lens, qw, kw, pos = _step_case(mi, dev, Hq=Hq, Hkv=Hkv, d=d, chunk=64, lens=LENS, dtype=dtype, seed=Hq + d + rot)
+    (out_a, kc_a, vc_a), (out_b, kc_b, vc_b) = _run_both(mi, dev, case, lens, qw, kw, pos, norm="rms", table=table,
+                                                         interleaved=interleaved, mixed=mixed,
+                                                         max_kv_len=int(lens.max()))
+    dummy = case.k_cache.size(0) - 1
+    assert torch.equal(kc_a[:dummy], kc_b[:dummy]), "key cache differs from the separate launch"
+    assert torch.equal(vc_a[:dummy], vc_b[:dummy]), "value cache differs from the separate launch"
+    diff = (out_a.float() - out_b.float()).abs().max().item()
+    assert diff <= 8e-3, f"fused and separate outputs differ by {diff:.3e}"
+    ref, kc_ref, vc_ref = _oracle(case, lens, qw, kw, pos, norm="rms", table=table, interleaved=interleaved)
+    _close(out_a, ref, 2e-2, "fused step vs checker")
+    _close(kc_a[:dummy], kc_ref[:dummy], 2e-2, "key cache vs checker")
+
+
 @pytest.mark.parametrize("mixed", [False, True])
 @pytest.mark.parametrize("chunk", [16, 128, 256])
 @pytest.mark.parametrize("grid,split", [(0, 0), (1, 0), (7, 64), (4096, 16)])
@@ -161,14 +187,16 @@ def test_fused_step_rejects_what_it_has_no_kernel_for(mi, dev):
     assert not mi.ops.decode_step_supported(128, 40, False, False)
     assert mi.ops.decode_step_supported(128, 40, True, False) and mi.ops.decode_step_supported(64, 64, False, False)
     assert not mi.ops.decode_step_supported(96, 96, False, False) and not mi.ops.decode_step_supported(128, 128, False, True)
+    assert mi.ops.decode_step_supported(96, 64, False, False) and mi.ops.decode_step_supported(256, 256, False, False)
+    assert not mi.ops.decode_step_supported(80, 0, False, False)
     with pytest.raises(mi._lib.KernelError, match="rot_dim / 2"):
         mi.ops.decode_step_attention(case.q, case.k_new, case.v_new, case.k_cache, case.v_cache, case.kv_lens,
                                      case.block_table, rotary_emb=table.to(dev), positions=pos.to(dev))
-    q96 = torch.zeros(2, 1, 8, 96, dtype=torch.bfloat16, device=dev)
-    k96 = torch.zeros(2, 1, 2, 96, dtype=torch.bfloat16, device=dev)
-    c96 = torch.zeros(4, 64, 2, 96, dtype=torch.bfloat16, device=dev)
+    q80 = torch.zeros(2, 1, 8, 80, dtype=torch.bfloat16, device=dev)
+    k80 = torch.zeros(2, 1, 2, 80, dtype=torch.bfloat16, device=dev)
+    c80 = torch.zeros(4, 64, 2, 80, dtype=torch.bfloat16, device=dev)
     with pytest.raises(mi._lib.KernelError, match="head_dim"):
-        mi.ops.decode_step_attention(q96, k96, k96, c96, c96, case.kv_lens, case.block_table)
+        mi.ops.decode_step_attention(q80, k80, k80, c80, c80, case.kv_lens, case.block_table)
 
 
 def test_fused_step_more_requests_than_one_launch_takes(mi, dev):
