@@ -682,16 +682,17 @@ def run_decode_config(args, mi, lib, torch, dev):
     out = torch.empty_like(case.q)
     use_norm = "rms"
 
-    # the whole step inside the streaming kernel (16-bit caches, head_dim 64 / 128) unless asked otherwise
-    one_kernel = (not cfg.fp8 and not args.attention_only and not args.separate_launches
-                  and mi.ops.decode_step_supported(cfg.d, cfg.d, False, False))
+    # the whole step inside the streaming kernel unless asked otherwise
+    one_kernel = (not args.attention_only and not args.separate_launches
+                  and mi.ops.decode_step_supported(cfg.d, cfg.d, False, cfg.fp8))
 
     def step():
         if one_kernel:
             mi.ops.decode_step_attention(case.q, case.k_new, case.v_new, case.k_cache, case.v_cache, case.kv_lens,
                                          case.block_table, q_weight=qw, k_weight=kw, eps=1e-5, norm=use_norm,
                                          rotary_emb=table, positions=None, out=out, max_kv_len=max_len,
-                                         split_tokens=args.split_tokens)  # (positions: kv_lens - 1)
+                                         split_tokens=args.split_tokens, k_scales=case.k_scales,
+                                         v_scales=case.v_scales)  # (positions: kv_lens - 1)
             return
         if not args.attention_only:
             if cfg.fp8:
@@ -728,12 +729,19 @@ def run_decode_config(args, mi, lib, torch, dev):
     separate = None
     if one_kernel:
         def step_separate():
-            mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_in, value=case.v_new, q_weight=qw, k_weight=kw,
-                                    eps=1e-5, norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos,
-                                    k_cache=case.k_cache, v_cache=case.v_cache, block_table=case.block_table,
-                                    kv_lens=case.kv_lens)
+            if cfg.fp8:
+                mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_in, key_out=k_rot, q_weight=qw, k_weight=kw,
+                                        eps=1e-5, norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos)
+                mi.ops.kv_append_decode_fp8(k_rot, case.v_new, case.k_cache, case.v_cache, case.k_scales,
+                                            case.v_scales, case.block_table, case.kv_lens)
+            else:
+                mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_in, value=case.v_new, q_weight=qw, k_weight=kw,
+                                        eps=1e-5, norm=use_norm, rotary_emb=table, q_positions=pos, k_positions=pos,
+                                        k_cache=case.k_cache, v_cache=case.v_cache, block_table=case.block_table,
+                                        kv_lens=case.kv_lens)
             mi.ops.paged_decode_attention(q_in, case.k_cache, case.v_cache, case.kv_lens, case.block_table, out=out,
-                                          max_kv_len=max_len, split_tokens=args.split_tokens)
+                                          max_kv_len=max_len, split_tokens=args.split_tokens,
+                                          k_scales=case.k_scales, v_scales=case.v_scales)
         for _ in range(args.warmup):
             step_separate()
         torch.cuda.synchronize()

@@ -227,6 +227,30 @@ int mi_decode_step_attention(const void* q, int64_t q_stride_tok, int64_t q_stri
                              int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
+ * The same step over an fp8-e4m3 cache (no counterpart in the reference, like the other fp8 entry points): the
+ * span that ends a request quantises the step's key row (after head norm and rotary embedding, rounded to bf16
+ * first) and value row into their slot with the policy of mi_kv_append_decode_fp8 -- a token that opens a chunk
+ * sets that chunk-head's scale to headroom * amax(token) / 448 (1 for an all-zero row) and stores it, later tokens
+ * reuse the stored scale and saturate -- and then streams the cache as mi_paged_decode_attention does with
+ * kv_dtype MI_KV_FP8_E4M3.  Bytes and scales are those of mi_norm_rope_append (key_out) followed by
+ * mi_kv_append_decode_fp8.  bf16 tensors, head_dim 128; half-split rotary pairs need rot_dim 128 (interleaved
+ * pairs: any even width).
+ */
+int mi_decode_step_attention_fp8(const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new,
+                                 int64_t k_stride_tok, int64_t k_stride_head, const void* v_new,
+                                 int64_t v_stride_tok, int64_t v_stride_head, const void* q_weight,
+                                 const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles,
+                                 int64_t angles_stride, int32_t rot_dim, int32_t rotary_interleaved, float mscale,
+                                 const int64_t* positions, void* k_cache_fp8, void* v_cache_fp8,
+                                 int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
+                                 float* k_scales, float* v_scales, float headroom, const int32_t* block_table,
+                                 int64_t bt_stride, const int32_t* kv_lens, void* out, int64_t o_stride_tok,
+                                 int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R,
+                                 int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
+                                 int32_t split_tokens, float softmax_scale, int32_t faithful_rounding,
+                                 const MiTuning* tuning, void* stream);
+
+/*
  * mi_paged_decode_attention for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments and results as mi_paged_decode_attention, minus the workspace: the

@@ -52,6 +52,11 @@ SIGNATURES = {
         [_P, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F, _P, _P, _P,
          _I64, _I64, _I64, _P, _I64, _P, _P, _I64, _I64, _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32,
          _I32, _P, _P]),
+    "mi_decode_step_attention_fp8": (
+        c_int,
+        [_P, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F, _P, _P, _P,
+         _I64, _I64, _I64, _P, _P, _F, _P, _I64, _P, _P, _I64, _I64, _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _F,
+         _I32, _P, _P]),
     "mi_paged_decode_attention_noalloc": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _I64, _I64,

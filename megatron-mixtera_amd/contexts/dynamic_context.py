@@ -519,13 +519,13 @@ class DynamicInferenceContext:
         return query
 
     def decode_step_fusable(self, head_dim: int, rotary_pos_emb: Optional[Tensor], config=None) -> bool:
-        """Whether this step can run :meth:`fused_decode_step_attention`: a decode-only step over 16-bit per-head
-        caches with shapes the fused kernel has (``ops.decode_step_supported``)."""
-        if not self.is_decode_only() or self.cache_mla_latent or self.kv_cache_fp8:
+        """Whether this step can run :meth:`fused_decode_step_attention`: a decode-only step over per-head caches
+        (16-bit or fp8) with shapes the fused kernel has (``ops.decode_step_supported``)."""
+        if not self.is_decode_only() or self.cache_mla_latent:
             return False
         rot = 0 if rotary_pos_emb is None else rotary_pos_emb.size(-1)
         interleaved = self._rope_flags(config) if config is not None else False
-        return ops.decode_step_supported(head_dim, rot, interleaved, False)
+        return ops.decode_step_supported(head_dim, rot, interleaved, self.kv_cache_fp8)
 
     def fused_decode_step_attention(self, layer_number: int, query: Optional[Tensor] = None,
                                     key: Optional[Tensor] = None, value: Optional[Tensor] = None, *,
@@ -551,6 +551,9 @@ class DynamicInferenceContext:
                       positions=None,  # = kv_seq_lengths - 1, see the docstring
                       rotary_interleaved=self._rope_flags(config) if config is not None else False, mscale=mscale,
                       softmax_scale=softmax_scale, max_kv_len=k_bound, faithful_rounding=faithful_rounding)
+        if self.kv_cache_fp8:  # the quantising append of the step's token rides in the kernel too
+            k_scales, v_scales = self.key_value_scales(layer_number)
+            common.update(k_scales=k_scales, v_scales=v_scales, headroom=self.fp8_append_headroom)
         if mixed_qkv is not None:
             d = self.kv_channels
             out = torch.empty((mixed_qkv.size(0), 1, num_query_heads, d), dtype=mixed_qkv.dtype, device=mixed_qkv.device)

@@ -60,14 +60,6 @@ __global__ __launch_bounds__(256) void kv_append_kernel(AppendParams p) {
   }
 }
 
-// fp32 -> e4m3fn byte, round to nearest even, saturating (no NaN / inf produced).
-static __device__ __forceinline__ uint32_t f32_to_e4m3_sat(float x) {
-  x = fminf(fmaxf(x, -448.f), 448.f);
-  // v_cvt_pk_fp8_f32 packs two conversions into the low 16 bits.
-  const int r = __builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false);
-  return (uint32_t)r & 0xffu;
-}
-
 struct QuantParams {
   const uint16_t* src;   // bf16 rows
   int64_t src_stride;    // elements between tokens (bulk: between chunk tokens)

@@ -39,6 +39,7 @@ struct FusedStepArgs {
   float mscale;
   const int64_t* positions;
   int32_t faithful_rounding;
+  float fp8_headroom;  // fp8 cache: scale of a chunk the step's token opens = headroom * amax(token) / 448
 };
 // Shared by the decode entry point and by the mixed-batch path of the prefill entry point
 // (cu_seqlens_q non-null: only requests with one query row take part, at row cu_seqlens_q[r]).

@@ -298,4 +298,12 @@ static __device__ __forceinline__ uint2 fp8x4_to_bf16x4(uint32_t w) {
   return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
 }
 
+// fp32 -> e4m3fn byte, round to nearest even, saturating (no NaN / inf produced).
+static __device__ __forceinline__ uint32_t f32_to_e4m3_sat(float x) {
+  x = fminf(fmaxf(x, -448.f), 448.f);
+  // v_cvt_pk_fp8_f32 packs two conversions into the low 16 bits.
+  const int r = __builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false);
+  return (uint32_t)r & 0xffu;
+}
+
 }  // namespace mi

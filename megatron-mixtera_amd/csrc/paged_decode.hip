@@ -45,6 +45,8 @@
 
 namespace mi {
 
+constexpr int MI_FUSED_FP8_NT = 2;  // 16-token sub-tiles per iteration of the one-kernel decode step over an fp8 cache
+
 struct DecodeParams {
   const uint16_t* q;
   int64_t q_st, q_sh;  // element strides: token, head
@@ -62,8 +64,9 @@ struct DecodeParams {
   float* part_o;     // [slots][Hq][HD], slots = grid + R
   float* part_lse;   // [slots][Hq]
   int32_t* seg_info;  // [R][2]: first and last workgroup that touched request r
-  const float* k_scale;  // fp8 only: [n_chunks][Hkv]
+  const float* k_scale;  // fp8 only: [n_chunks][Hkv] (written by the fused step when a token opens a chunk)
   const float* v_scale;
+  float headroom;        // fp8 fused step: scale of a chunk a token opens = headroom * amax(token) / 448
   uint64_t chunk_magic;  // ceil(2^40 / chunk)
   int32_t R, Hq, Hkv, G, chunk, min_span_tiles, grid;
   int32_t parts;  // wavefronts per KV head: each takes up to 16 of the G query heads that share it
@@ -119,7 +122,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   constexpr int VD = FP8 ? 2 : DV / 2;  // dwords per token and lane of the value operand
   static_assert(HDK % 32 == 0 && HDV % 32 == 0 && HDK >= 64 && HDV >= 64, "head widths: multiples of 32");
   static_assert(!FP8 || (HDK == 128 && HDV == 128 && !F16), "fp8 KV: head_dim 128, bf16 queries");
-  static_assert(!FUSED || (!FP8 && HDK == HDV && HDK <= 256), "fused step: an ordinary 16-bit cache");
+  static_assert(!FUSED || (HDK == HDV && HDK <= 256), "fused step: an ordinary per-head cache");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
   // tile base addresses below run on the scalar unit instead of costing vector instructions.
@@ -166,6 +169,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   const int64_t chunk_bytes = p.kv_sc * ESZ;
   const uint32_t tok_bytes = (uint32_t)(p.kv_st * ESZ);
 
+  // first element of this lane's 8 of fragment kk (see the query loads above)
+  auto frag_d0 = [&](int kk) { return FP8 ? 64 * (kk >> 1) + 16 * g + 8 * (kk & 1) : 32 * kk + 8 * g; };
   float* const cs = reinterpret_cast<float*>(q_lds);  // fused: [2][HDK]: cos | sin at the request's position
   float* const kx = cs + 2 * HDK;                     // fused: [HDK]: the normalised key row (rotary partners)
   const bool faithful = FUSED && p.faithful != 0;
@@ -189,9 +194,14 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
     }
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk)
-      qwr[kk] = (p.norm == MI_NORM_RMS && p.q_w) ? ld16(p.q_w + 32 * kk + 8 * g)
+      qwr[kk] = (p.norm == MI_NORM_RMS && p.q_w) ? ld16(p.q_w + frag_d0(kk))
                                                  : make_uint4(ones2<F16>(), ones2<F16>(), ones2<F16>(), ones2<F16>());
   }
+  // fp8 fused step: the scales of the chunk that takes the step's token, as this wavefront knows them after its
+  // append (it reads them from these registers, never back from memory: the loads of the cursor below may have
+  // been issued before the store of a scale this very step set)
+  bool own_scale = false;   // the token opened its chunk: own_ksc / own_vsc are that chunk's scales
+  float own_ksc = 1.f, own_vsc = 1.f;
   auto fused_cos_sin = [&] {
     if (p.emb) {
 #pragma unroll
@@ -265,8 +275,58 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
         }
       }
       const int cpos = len - 1, ci = chunk_of(cpos, p.chunk_magic);
-      const int64_t slot_bytes = (int64_t)p.bt[(int64_t)r * p.bt_stride + ci] * chunk_bytes +
-                                 (int64_t)(cpos - ci * p.chunk) * tok_bytes;
+      const int pc_new = p.bt[(int64_t)r * p.bt_stride + ci];
+      const int64_t slot_bytes = (int64_t)pc_new * chunk_bytes + (int64_t)(cpos - ci * p.chunk) * tok_bytes;
+      if constexpr (FP8) {
+        // Quantising append, the policy of the separate launch (kv_append_decode_fp8_kernel): a token that opens a
+        // chunk fixes the chunk-head's scale to headroom * amax(token) / 448, later tokens reuse the stored scale
+        // and saturate; the key row is rounded to bf16 first, as the separate norm / rotary launch hands it over.
+        const bool opens = cpos == ci * p.chunk;  // wave-uniform
+        float* const ksc_p = const_cast<float*>(p.k_scale) + (int64_t)pc_new * p.Hkv + h;
+        float* const vsc_p = const_cast<float*>(p.v_scale) + (int64_t)pc_new * p.Hkv + h;
+        const uint16_t* vsrc = p.nv + (int64_t)row * p.nv_st + (int64_t)h * p.nv_hst;
+        float kq[EPL], vq[EPL];
+#pragma unroll
+        for (int w = 0; w < EPL; ++w) {
+          kq[w] = on ? bf16_to_f32(f32_to_bf16(o[w])) : 0.f;
+          vq[w] = on ? bf16_to_f32(vsrc[i + w * LPV]) : 0.f;
+        }
+        float ksc, vsc;
+        if (opens) {
+          float ka = 0.f, va = 0.f;
+#pragma unroll
+          for (int w = 0; w < EPL; ++w) {
+            ka = fmaxf(ka, fabsf(kq[w]));
+            va = fmaxf(va, fabsf(vq[w]));
+          }
+#pragma unroll
+          for (int off = 32; off > 0; off >>= 1) {
+            ka = fmaxf(ka, __shfl_xor(ka, off, 64));
+            va = fmaxf(va, __shfl_xor(va, off, 64));
+          }
+          ksc = ka > 0.f ? p.headroom * ka / 448.f : 1.f;
+          vsc = va > 0.f ? p.headroom * va / 448.f : 1.f;
+          if (lane == 0) {
+            *ksc_p = ksc;
+            *vsc_p = vsc;
+          }
+          own_scale = true;
+        } else {
+          ksc = *ksc_p;
+          vsc = *vsc_p;
+        }
+        own_ksc = ksc;
+        own_vsc = vsc;
+        uint8_t* kdst8 = const_cast<uint8_t*>(kbase) + slot_bytes;
+        uint8_t* vdst8 = const_cast<uint8_t*>(vbase) + slot_bytes;
+        if (on) {
+#pragma unroll
+          for (int w = 0; w < EPL; ++w) {
+            kdst8[i + w * LPV] = (uint8_t)f32_to_e4m3_sat(kq[w] / ksc);
+            vdst8[i + w * LPV] = (uint8_t)f32_to_e4m3_sat(vq[w] / vsc);
+          }
+        }
+      } else {
       uint16_t* kdst = reinterpret_cast<uint16_t*>(const_cast<uint8_t*>(kbase) + slot_bytes);
       if (on) {
 #pragma unroll
@@ -275,6 +335,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       const uint32_t* vsrc = reinterpret_cast<const uint32_t*>(p.nv + (int64_t)row * p.nv_st + (int64_t)h * p.nv_hst);
       uint32_t* vdst = reinterpret_cast<uint32_t*>(const_cast<uint8_t*>(vbase) + slot_bytes);
       for (int e = lane; e < HDV / 2; e += 64) vdst[e] = vsrc[e];
+      }
       // The rows just written are read back below by other lanes of this same wavefront and by nobody else in
       // this launch (it owns the request's last tiles): wait until the stores have reached the L2 (their
       // acknowledgement), then keep the compiler from moving the loads up.  No cache has to be written back or
@@ -321,10 +382,10 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       auto rotated = [&](float y, float yp, float c, float sn) {
         return faithful ? to_f32<F16>(f32_to_16<F16>(y * c)) + to_f32<F16>(f32_to_16<F16>(yp * sn)) : y * c + yp * sn;
       };
-      // cos | sin of elements 32 kk + 8 g + j .. + 3 (j = 0 or 4)
+      // cos | sin of this lane's elements j .. j + 3 of fragment kk (j = 0 or 4)
       auto cos_sin = [&](int kk, int j, float (&c)[4], float (&sn)[4]) {
-        const float4 c4 = *reinterpret_cast<const float4*>(&cs[32 * kk + 8 * g + j]);
-        const float4 s4 = *reinterpret_cast<const float4*>(&cs[HDK + 32 * kk + 8 * g + j]);
+        const float4 c4 = *reinterpret_cast<const float4*>(&cs[frag_d0(kk) + j]);
+        const float4 s4 = *reinterpret_cast<const float4*>(&cs[HDK + frag_d0(kk) + j]);
         c[0] = c4.x; c[1] = c4.y; c[2] = c4.z; c[3] = c4.w;
         sn[0] = s4.x; sn[1] = s4.y; sn[2] = s4.z; sn[3] = s4.w;
       };
@@ -352,7 +413,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
             cos_sin(kk, j0, c, sn);
 #pragma unroll
             for (int j = 0; j < 4; j += 2) {
-              if (32 * kk + 8 * g + j0 + j < p.rot) {  // (rot_dim is even: a pair lies within it or beyond)
+              if (frag_d0(kk) + j0 + j < p.rot) {  // (rot_dim is even: a pair lies within it or beyond)
                 const float ya = x[kk][j0 + j], yb = x[kk][j0 + j + 1];
                 x[kk][j0 + j] = rotated(ya, -yb, c[j], sn[j]);
                 x[kk][j0 + j + 1] = rotated(yb, ya, c[j + 1], sn[j + 1]);
@@ -470,7 +531,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   auto load_k = [&](int T) {
     int tok0;
     const uint8_t* chunk = tile_chunk(kcur, p.k_scale, kbase, T, tok0);
-    if (FP8) ksc_tile = kcur.sc;
+    if (FP8) ksc_tile = (FUSED && own_scale && kcur.ci == ci_last) ? own_ksc : kcur.sc;
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       const int t0 = min(T + 16 * u, last);
@@ -484,7 +545,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   auto load_v = [&](int T) {
     int tok0;
     const uint8_t* chunk = tile_chunk(vcur, p.v_scale, vbase, T, tok0);
-    if (FP8) vsc_tile = vcur.sc;
+    if (FP8) vsc_tile = (FUSED && own_scale && vcur.ci == ci_last) ? own_vsc : vcur.sc;
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       const int t0 = min(T + 16 * u, last);
@@ -523,6 +584,10 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   if (FP8) {  // the first tile lies in the opening chunk
     kcur.sc = ksc_tile = uniform_f(ksc_first);
     vcur.sc = vsc_tile = uniform_f(vsc_first);
+    if (FUSED && own_scale && kcur.ci == ci_last) {  // ... which the step's token has just opened
+      ksc_tile = own_ksc;
+      vsc_tile = own_vsc;
+    }
   }
   const uint2 ones = make_uint2(ones2<F16>(), ones2<F16>());  // four times 1.0
   for (int T = start; T < end; T += 16 * NT) {
@@ -782,9 +847,9 @@ __global__ __launch_bounds__(512, MINW) void paged_decode_stream_kernel(DecodePa
 
 // The same stream over the raw queries, keys and values of a decode step: head norm, rotary embedding and the
 // append of the new token ride in the segment prologues (see decode_segment).
-template <int HD, int NT, bool F16, int MINW = 3>
+template <int HD, int NT, bool F16, int MINW = 3, bool FP8 = false>
 __global__ __launch_bounds__(512, MINW) void decode_step_stream_kernel(DecodeParams p) {
-  decode_stream_body<HD, HD, NT, false, F16, true>(p);
+  decode_stream_body<HD, HD, NT, FP8, F16, true>(p);
 }
 
 // Multi-latent attention, absorbed form: every query head attends to the same 576-wide latent rows
@@ -1701,7 +1766,7 @@ int mi::launch_paged_decode(
   if (nt != 1 && nt != 2 && nt != 4) nt = kv_dtype == MI_KV_FP8_E4M3 ? 4 : 2;
   if (head_dim == 256) nt = 1;                 // (registers: 64 accumulators + 32 each for queries, keys, values)
   else if (head_dim == 192 && nt > 2) nt = 2;
-  if (fused) nt = 1;  // (the prologue's registers on top of two sub-tiles in flight would spill)
+  if (fused) nt = kv_dtype == MI_KV_FP8_E4M3 ? MI_FUSED_FP8_NT : 1;  // (the prologue's registers on top of two 16-bit sub-tiles in flight would spill)
   while (chunk_tokens % (16 * nt)) nt >>= 1;  // a tile must not straddle two chunks
   const int minw = head_dim > 128 ? 2 : tune.decode_min_waves;
   const int tk = 16 * nt;
@@ -1733,6 +1798,7 @@ int mi::launch_paged_decode(
     p.emb = fused->rotary_angles; p.emb_stride = fused->angles_stride; p.pos = fused->positions;
     p.rot = fused->rot_dim; p.norm = fused->norm_kind; p.interleaved = fused->rotary_interleaved;
     p.faithful = fused->faithful_rounding; p.eps = fused->eps; p.mscale = fused->mscale;
+    p.headroom = fused->fp8_headroom;
   }
 
   const int waves = head_waves(Hq, Hkv);
@@ -1762,7 +1828,9 @@ int mi::launch_paged_decode(
   } while (0)
 #define MI_LAUNCH_STEP(HD_, F16_) hipLaunchKernelGGL((decode_step_stream_kernel<HD_, 1, F16_>), grid, block, lds, st, p)
 #define MI_LAUNCH_STEP_WIDE(HD_, F16_) hipLaunchKernelGGL((decode_step_stream_kernel<HD_, 1, F16_, 2>), grid, block, lds, st, p)
-  if (fused && head_dim == 128 && f16) MI_LAUNCH_STEP(128, true);
+  if (fused && kv_dtype == MI_KV_FP8_E4M3)
+    hipLaunchKernelGGL((decode_step_stream_kernel<128, MI_FUSED_FP8_NT, false, 3, true>), grid, block, lds, st, p);
+  else if (fused && head_dim == 128 && f16) MI_LAUNCH_STEP(128, true);
   else if (fused && head_dim == 128) MI_LAUNCH_STEP(128, false);
   else if (fused && head_dim == 64 && f16) MI_LAUNCH_STEP(64, true);
   else if (fused && head_dim == 64) MI_LAUNCH_STEP(64, false);
@@ -1810,8 +1878,8 @@ extern "C" int mi_paged_decode_attention(
                              split_tokens, softmax_scale, kv_dtype, k_scales, v_scales, dtype, tune, stream);
 }
 
-extern "C" int mi_decode_step_attention(
-    const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new, int64_t k_stride_tok,
+static int decode_step_entry(
+    const char* who, const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new, int64_t k_stride_tok,
     int64_t k_stride_head, const void* v_new, int64_t v_stride_tok, int64_t v_stride_head, const void* q_weight,
     const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles, int64_t angles_stride,
     int32_t rot_dim, int32_t rotary_interleaved, float mscale, const int64_t* positions, void* k_cache, void* v_cache,
@@ -1819,8 +1887,8 @@ extern "C" int mi_decode_step_attention(
     int64_t bt_stride, const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
     int64_t workspace_bytes, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
     int32_t split_tokens, float softmax_scale, int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning,
-    void* stream) {
-  const char* who = "mi_decode_step_attention";
+    void* stream, int32_t kv_dtype, float* k_scales, float* v_scales, float headroom) {
+  const bool fp8 = kv_dtype == MI_KV_FP8_E4M3;
   char msg[160];
   auto fail = [&](int code, const char* what) {
     snprintf(msg, sizeof msg, "%s: %s", who, what);
@@ -1842,7 +1910,12 @@ extern "C" int mi_decode_step_attention(
     // a lane holds 8 consecutive elements of every 32: half-split partners must sit a whole number of 32s away
     if (!rotary_interleaved && (rot_dim / 2) % 32)
       return fail(MI_ERR_UNSUPPORTED, "half-split rotary pairs need rot_dim / 2 to be a multiple of 32 (else: the separate calls)");
+    // (an fp8 cache's key bytes put a lane's 16 consecutive elements of every 64 into two fragments)
+    if (fp8 && !rotary_interleaved && (rot_dim / 2) % 64)
+      return fail(MI_ERR_UNSUPPORTED, "over an fp8 cache half-split rotary pairs need rot_dim / 2 to be a multiple of 64 (else: the separate calls)");
   }
+  if (fp8 && (head_dim != 128 || dtype != MI_DTYPE_BF16 || !k_scales || !v_scales || !(headroom > 0.f)))
+    return fail(MI_ERR_UNSUPPORTED, "an fp8 cache needs head_dim 128, bf16 tensors, both scale arrays and a positive headroom");
   const int G = Hq / Hkv;
   if (q_stride_group < (int64_t)G * head_dim) return fail(MI_ERR_SHAPE, "query group stride smaller than (Hq / Hkv) * head_dim");
   if ((((uintptr_t)q | (uintptr_t)q_weight) & 15) || (q_stride_tok | q_stride_group) % 8)
@@ -1857,12 +1930,50 @@ extern "C" int mi_decode_step_attention(
   fs.rotary_angles = rotary_angles; fs.angles_stride = angles_stride; fs.rot_dim = rot_dim;
   fs.rotary_interleaved = rotary_interleaved; fs.mscale = mscale; fs.positions = positions;
   fs.faithful_rounding = faithful_rounding;
+  fs.fp8_headroom = headroom;
   // (the remaining checks -- cache strides, chunk size, workspace -- are those of the attention entry point; the
   // head stride of q is not used by the fused kernels)
   return launch_paged_decode(q, q_stride_tok, head_dim, k_cache, v_cache, kv_stride_chunk, kv_stride_tok, kv_stride_head,
                              block_table, bt_stride, kv_lens, nullptr, out, o_stride_tok, o_stride_head, workspace,
                              workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens, split_tokens, softmax_scale,
-                             MI_KV_16BIT, nullptr, nullptr, dtype, tune, stream, &fs);
+                             kv_dtype, k_scales, v_scales, dtype, tune, stream, &fs);
+}
+
+extern "C" int mi_decode_step_attention(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new, int64_t k_stride_tok,
+    int64_t k_stride_head, const void* v_new, int64_t v_stride_tok, int64_t v_stride_head, const void* q_weight,
+    const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles, int64_t angles_stride,
+    int32_t rot_dim, int32_t rotary_interleaved, float mscale, const int64_t* positions, void* k_cache, void* v_cache,
+    int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head, const int32_t* block_table,
+    int64_t bt_stride, const int32_t* kv_lens, void* out, int64_t o_stride_tok, int64_t o_stride_head, void* workspace,
+    int64_t workspace_bytes, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
+    int32_t split_tokens, float softmax_scale, int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning,
+    void* stream) {
+  return decode_step_entry("mi_decode_step_attention", q, q_stride_tok, q_stride_group, k_new, k_stride_tok, k_stride_head,
+                           v_new, v_stride_tok, v_stride_head, q_weight, k_weight, eps, norm_kind, rotary_angles,
+                           angles_stride, rot_dim, rotary_interleaved, mscale, positions, k_cache, v_cache, kv_stride_chunk,
+                           kv_stride_tok, kv_stride_head, block_table, bt_stride, kv_lens, out, o_stride_tok, o_stride_head,
+                           workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens, split_tokens, softmax_scale,
+                           faithful_rounding, dtype, tuning, stream, MI_KV_16BIT, nullptr, nullptr, 1.f);
+}
+
+extern "C" int mi_decode_step_attention_fp8(
+    const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new, int64_t k_stride_tok,
+    int64_t k_stride_head, const void* v_new, int64_t v_stride_tok, int64_t v_stride_head, const void* q_weight,
+    const void* k_weight, float eps, int32_t norm_kind, const float* rotary_angles, int64_t angles_stride,
+    int32_t rot_dim, int32_t rotary_interleaved, float mscale, const int64_t* positions, void* k_cache_fp8,
+    void* v_cache_fp8, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head, float* k_scales,
+    float* v_scales, float headroom, const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
+    int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq,
+    int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t split_tokens, float softmax_scale,
+    int32_t faithful_rounding, const MiTuning* tuning, void* stream) {
+  return decode_step_entry("mi_decode_step_attention_fp8", q, q_stride_tok, q_stride_group, k_new, k_stride_tok,
+                           k_stride_head, v_new, v_stride_tok, v_stride_head, q_weight, k_weight, eps, norm_kind,
+                           rotary_angles, angles_stride, rot_dim, rotary_interleaved, mscale, positions, k_cache_fp8,
+                           v_cache_fp8, kv_stride_chunk, kv_stride_tok, kv_stride_head, block_table, bt_stride, kv_lens, out,
+                           o_stride_tok, o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
+                           split_tokens, softmax_scale, faithful_rounding, MI_DTYPE_BF16, tuning, stream, MI_KV_FP8_E4M3,
+                           k_scales, v_scales, headroom);
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -685,9 +685,10 @@ def qkv_norm_rope_append(mixed_qkv: Tensor, *, num_query_heads: int, num_kv_head
 # ---------------------------------------------------------------------------------------------
 def decode_step_supported(head_dim: int, rot_dim: int, rotary_interleaved: bool, fp8_cache: bool) -> bool:
     """Whether :func:`decode_step_attention` has a kernel for these shapes (else: the separate calls)."""
-    if fp8_cache or head_dim not in (64, 96, 128, 192, 256):
+    if head_dim not in (64, 96, 128, 192, 256) or (fp8_cache and head_dim != 128):
         return False
-    return rot_dim == 0 or rotary_interleaved or (rot_dim // 2) % 32 == 0
+    # half-split pairs must sit a whole number of a lane's fragments apart (fp8 key bytes: 64 elements)
+    return rot_dim == 0 or rotary_interleaved or (rot_dim // 2) % (64 if fp8_cache else 32) == 0
 
 
 def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value: Optional[Tensor], k_cache: Tensor,
@@ -698,12 +699,15 @@ def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value:
                           positions: Optional[Tensor] = None, rotary_interleaved: bool = False, mscale: float = 1.0,
                           softmax_scale: Optional[float] = None, max_kv_len: Optional[int] = None,
                           split_tokens: int = 0, out: Optional[Tensor] = None, workspace: Optional[Tensor] = None,
-                          faithful_rounding: bool = True) -> Tensor:
+                          faithful_rounding: bool = True, k_scales: Optional[Tensor] = None,
+                          v_scales: Optional[Tensor] = None, headroom: float = 2.0) -> Tensor:
     """One decode step of a layer in two launches: head norm + RoPE of the raw queries and of the step's new key
     rows, the append of the new key / value rows at position ``kv_lens - 1`` and the attention over the cache --
     what :func:`norm_rope_append` (or :func:`qkv_norm_rope_append`) followed by :func:`paged_decode_attention`
     computes.  Inputs: ``query`` ``[R, (1,) Hq, d]``, ``key`` / ``value`` ``[R, (1,) Hkv, d]``, or ``mixed_qkv``
-    ``[R, (1,) (Hq + 2 Hkv) d]`` (the QKV projection's output) with the head counts.  Returns ``[R, (1,) Hq, d]``."""
+    ``[R, (1,) (Hq + 2 Hkv) d]`` (the QKV projection's output) with the head counts.  Returns ``[R, (1,) Hq, d]``.
+    Byte caches with ``k_scales`` / ``v_scales`` hold e4m3 values: the append then quantises like
+    :func:`kv_append_decode_fp8` (``headroom`` as there)."""
     lib = _lib.load()
     if mixed_qkv is not None:
         _require(query is None and key is None and value is None, "give either query / key / value or mixed_qkv")
@@ -739,7 +743,15 @@ def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value:
     stream = _stream(ref)
     N, C, Hkv_c, Dk = k_cache.shape
     _require(Dk == D and Hkv_c == Hkv and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
-    _require(k_cache.dtype == ref.dtype and v_cache.dtype == ref.dtype, "the caches must have the tensors' 16-bit type")
+    fp8 = k_cache.element_size() == 1
+    if fp8:
+        _require(v_cache.element_size() == 1 and k_scales is not None and v_scales is not None,
+                 "byte caches hold e4m3 values and need k_scales / v_scales")
+        _require(ref.dtype == torch.bfloat16, "an fp8 cache needs bf16 queries / keys / values")
+        for t in (k_scales, v_scales):
+            _require(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (N, Hkv), "scales must be fp32 [n_chunks, Hkv]")
+    else:
+        _require(k_cache.dtype == ref.dtype and v_cache.dtype == ref.dtype, "the caches must have the tensors' 16-bit type")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
     _require(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.stride(1) == 1, "bad block_table")
@@ -764,6 +776,15 @@ def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value:
     if workspace is None:
         workspace = _workspace(ref.device, need, stream)
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    if fp8:
+        _lib.check(lib.mi_decode_step_attention_fp8(
+            q_ptr, q_st, q_gst, k_ptr, k_st, k_hst, v_ptr, v_st, v_hst, _ptr(q_weight), _ptr(k_weight), float(eps),
+            _NORM_KINDS[norm], _ptr(ang), a_stride, rot, int(bool(rotary_interleaved)), float(mscale), _ptr(positions),
+            k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh, k_scales.data_ptr(), v_scales.data_ptr(), float(headroom),
+            block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
+            _ptr(workspace), ws_bytes, R, Hq, Hkv, D, C, int(split_tokens), float(softmax_scale),
+            int(bool(faithful_rounding)), tune, stream), "mi_decode_step_attention_fp8")
+        return out
     _lib.check(lib.mi_decode_step_attention(
         q_ptr, q_st, q_gst, k_ptr, k_st, k_hst, v_ptr, v_st, v_hst, _ptr(q_weight), _ptr(k_weight), float(eps),
         _NORM_KINDS[norm], _ptr(ang), a_stride, rot, int(bool(rotary_interleaved)), float(mscale), _ptr(positions),

@@ -181,12 +181,83 @@ def test_fused_step_without_faithful_rounding_and_repeated_steps(mi, dev):
     _close(kc[:dummy], kc_ref[:dummy], 2e-2, "key cache after three steps")
 
 
+@pytest.mark.parametrize("mixed", [False, True])
+@pytest.mark.parametrize("rotary", ["none", "half", "interleaved", "interleaved40"])
+@pytest.mark.parametrize("norm", [None, "rms"])
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (6, 2), (20, 1)])
+def test_fused_step_over_an_fp8_cache(mi, dev, Hq, Hkv, norm, rotary, mixed):
+    """The one-kernel step over an fp8-e4m3 cache: bytes and scales equal to the separate launches (norm / rotary
+    with key_out, then the quantising append), tokens that open a chunk (lengths 1, 65, 129: they set the scale) and
+    tokens that reuse a stored scale; output within 8e-3 of the separate launches and 6e-2 of the unquantised checker."""
+    d, chunk = 128, 64
+    rot = {"none": 0, "half": d, "interleaved": d, "interleaved40": 40}[rotary]
+    interleaved = rotary.startswith("interleaved")
+    table = orn.rotary_table(4096, rot, base=500000.0, interleaved=interleaved) if rot else None
+    lens_l = [0, 1, 2, 63, 64, 65, 66, 128, 129, 130, 700, 2049, 0, 193]
+    case, lens, qw, kw, pos = _step_case(mi, dev, Hq=Hq, Hkv=Hkv, d=d, chunk=chunk, lens=lens_l, dtype=torch.bfloat16,
+                                         seed=Hq + rot)
+    R = lens.numel()
+    G = Hq // Hkv
+    k8 = torch.empty(case.k_cache.shape, dtype=torch.uint8, device=dev)
+    v8 = torch.empty_like(k8)
+    ks = torch.empty(case.k_cache.size(0), Hkv, dtype=torch.float32, device=dev)
+    vs = torch.empty_like(ks)
+    mi.ops.quantize_chunks_fp8(case.k_cache, k8, ks)
+    mi.ops.quantize_chunks_fp8(case.v_cache, v8, vs)
+    # chunks the step's token is about to open hold no token yet: whatever they held must not matter
+    for r in range(R):
+        L = int(lens[r])
+        if L > 0 and (L - 1) % chunk == 0:
+            c = int(case.block_table[r, (L - 1) // chunk])
+            k8[c] = 0x7e; v8[c] = 0x7e; ks[c] = 1e30; vs[c] = -5.0
+    common = dict(q_weight=qw.to(dev) if norm == "rms" else None, k_weight=kw.to(dev) if norm == "rms" else None,
+                  norm=norm, eps=1e-5, rotary_emb=None if table is None else table.to(dev),
+                  rotary_interleaved=interleaved)
+    posd = pos.to(dev)
+    k8a, v8a, ksa, vsa = k8.clone(), v8.clone(), ks.clone(), vs.clone()
+    k8b, v8b, ksb, vsb = k8.clone(), v8.clone(), ks.clone(), vs.clone()
+    if mixed:
+        grouped = torch.cat([case.q.view(R, Hkv, G * d), case.k_new.view(R, Hkv, d), case.v_new.view(R, Hkv, d)], -1)
+        out_a = mi.ops.decode_step_attention(None, None, None, k8a, v8a, case.kv_lens, case.block_table,
+                                             mixed_qkv=grouped.reshape(R, 1, -1).contiguous(), num_query_heads=Hq,
+                                             num_kv_heads=Hkv, positions=posd, k_scales=ksa, v_scales=vsa, headroom=1.5,
+                                             max_kv_len=int(lens.max()), **common)
+    else:
+        out_a = mi.ops.decode_step_attention(case.q, case.k_new, case.v_new, k8a, v8a, case.kv_lens, case.block_table,
+                                             positions=posd, k_scales=ksa, v_scales=vsa, headroom=1.5,
+                                             max_kv_len=int(lens.max()), **common)
+    q_b, k_b = torch.empty_like(case.q), torch.empty_like(case.k_new)
+    with mi.ops.tuning(norm_rope_vectorised=-1):
+        mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_b, key_out=k_b, q_positions=posd, k_positions=posd, **common)
+    mi.ops.kv_append_decode_fp8(k_b, case.v_new, k8b, v8b, ksb, vsb, case.block_table, case.kv_lens, headroom=1.5)
+    out_b = mi.ops.paged_decode_attention(q_b, k8b, v8b, case.kv_lens, case.block_table, k_scales=ksb, v_scales=vsb,
+                                          max_kv_len=int(lens.max()))
+    torch.cuda.synchronize()
+    assert torch.equal(k8a, k8b) and torch.equal(v8a, v8b), "cache bytes differ from the separate launches"
+    assert torch.equal(ksa, ksb) and torch.equal(vsa, vsb), "scales differ from the separate launches"
+    diff = (out_a.float() - out_b.float()).abs().max().item()
+    assert diff <= 8e-3, f"fused and separate outputs differ by {diff:.3e}"
+    assert (out_a[case.kv_lens == 0] == 0).all()
+    # against the checker: its own norm / rotary chain for the queries, attention over the dequantised cache the
+    # step left behind (2e-2); single values of short rows carry the full e4m3 rounding, so the unquantised
+    # checker is only held to 6e-2 where at least 64 keys average it out
+    w = dict(norm=norm, eps=1e-5, interleaved=interleaved)
+    q_ref = orn.norm_rope(case.q.cpu().squeeze(1), pos, table, weight=qw if norm == "rms" else None, **w)
+    ref8 = oa.paged_decode_attention(q_ref, k8a.cpu(), v8a.cpu(), lens, case.block_table.cpu(), k_scales=ksa.cpu(),
+                                     v_scales=vsa.cpu())
+    _close(out_a, ref8, 2e-2, "fused fp8 step vs the checker over the dequantised cache")
+    ref, _, _ = _oracle(case, lens, qw, kw, pos, norm=norm, table=table, interleaved=interleaved)
+    long_rows = lens >= 64
+    _close(out_a[long_rows.to(dev)], ref[long_rows], 6e-2, "fused fp8 step vs the unquantised checker")
+
+
 def test_fused_step_rejects_what_it_has_no_kernel_for(mi, dev):
     case, lens, qw, kw, pos = _step_case(mi, dev, Hq=8, Hkv=2, d=128, chunk=64, lens=[5, 9], dtype=torch.bfloat16, seed=1)
     table = orn.rotary_table(64, 40, base=10000.0)  # half-split pairs 20 elements apart
     assert not mi.ops.decode_step_supported(128, 40, False, False)
     assert mi.ops.decode_step_supported(128, 40, True, False) and mi.ops.decode_step_supported(64, 64, False, False)
-    assert not mi.ops.decode_step_supported(96, 96, False, False) and not mi.ops.decode_step_supported(128, 128, False, True)
+    assert not mi.ops.decode_step_supported(96, 96, False, False) and mi.ops.decode_step_supported(128, 128, False, True)
+    assert not mi.ops.decode_step_supported(128, 64, False, True) and not mi.ops.decode_step_supported(64, 64, False, True)
     assert mi.ops.decode_step_supported(96, 64, False, False) and mi.ops.decode_step_supported(256, 256, False, False)
     assert not mi.ops.decode_step_supported(80, 0, False, False)
     with pytest.raises(mi._lib.KernelError, match="rot_dim / 2"):

@@ -208,3 +208,57 @@ def test_one_kernel_decode_step_full_size(mi, dev, name, need):
         q_ref = orn.norm_rope(case.q[r:r + 1].cpu().squeeze(1), pos[r:r + 1].cpu(), table, norm="rms", weight=qw, eps=1e-5)
         ref = oa.paged_decode_attention(q_ref, kc, vc, case.kv_lens[r:r + 1].cpu(), rows)
         _close(out_a[r:r + 1], ref, 2e-2, f"{name} row {r}")
+
+
+def test_one_kernel_decode_step_over_the_fp8_cache_full_size(mi, dev):
+    """Configuration 5 at full size (batch 256, U[1024, 32768], fp8-e4m3 cache): the one-kernel decode step --
+    RMSNorm + RoPE + quantising append + attention -- against the separate launches: the appended bytes and every
+    scale bit for bit, the outputs within 8e-3."""
+    _need_free(40)
+    cfg = mi.synthetic.CONFIGS["cfg5"]
+    case = mi.synthetic.make_decode_case(cfg, dev, on_device_rng=True)
+    R, d = case.q.size(0), cfg.d
+    N = case.k_cache.size(0)
+    k8 = torch.empty(case.k_cache.shape, dtype=torch.uint8, device=dev)
+    v8 = torch.empty_like(k8)
+    ks = torch.empty(N, cfg.Hkv, dtype=torch.float32, device=dev)
+    vs = torch.empty_like(ks)
+    mi.ops.quantize_chunks_fp8(case.k_cache, k8, ks)
+    mi.ops.quantize_chunks_fp8(case.v_cache, v8, vs)
+    del case.k_cache, case.v_cache
+    torch.cuda.empty_cache()
+    # a few requests whose step token opens a chunk: shorten them to one token past a chunk boundary
+    lens = case.kv_lens.clone()
+    lens[::37] = (lens[::37] // cfg.chunk) * cfg.chunk + 1
+    mx = int(lens.max())
+    gen = torch.Generator().manual_seed(12)
+    qw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16().to(dev)
+    kw = (1 + 0.02 * torch.randn(d, generator=gen)).bfloat16().to(dev)
+    table = mi.synthetic.rotary_angle_table(mx + 1, d, base=500000.0).to(dev)
+    pos = (lens.long() - 1).contiguous()
+    common = dict(q_weight=qw, k_weight=kw, eps=1e-5, norm="rms", rotary_emb=table)
+    lens_h, bt_h = lens.cpu().long(), case.block_table.cpu().long()
+    slot_chunk = bt_h[torch.arange(R), (lens_h - 1) // cfg.chunk].to(dev)
+    slot_pos = ((lens_h - 1) % cfg.chunk).to(dev)
+    ks0, vs0 = ks.clone(), vs.clone()
+
+    out_a = mi.ops.decode_step_attention(case.q, case.k_new, case.v_new, k8, v8, lens, case.block_table,
+                                         positions=None, max_kv_len=mx, k_scales=ks, v_scales=vs, headroom=2.0, **common)
+    torch.cuda.synchronize()
+    k_rows_a, v_rows_a = k8[slot_chunk, slot_pos].clone(), v8[slot_chunk, slot_pos].clone()
+    ks_a, vs_a = ks.clone(), vs.clone()
+    assert not torch.equal(ks_a, ks0), "no token opened a chunk: the case does not test the scale path"
+    k8[slot_chunk, slot_pos] = 0
+    v8[slot_chunk, slot_pos] = 0
+    ks.copy_(ks0); vs.copy_(vs0)
+    q_b, k_b = torch.empty_like(case.q), torch.empty_like(case.k_new)
+    with mi.ops.tuning(norm_rope_vectorised=-1):
+        mi.ops.norm_rope_append(case.q, case.k_new, query_out=q_b, key_out=k_b, q_positions=pos, k_positions=pos, **common)
+    mi.ops.kv_append_decode_fp8(k_b, case.v_new, k8, v8, ks, vs, case.block_table, lens, headroom=2.0)
+    out_b = mi.ops.paged_decode_attention(q_b, k8, v8, lens, case.block_table, max_kv_len=mx, k_scales=ks, v_scales=vs)
+    torch.cuda.synchronize()
+    assert torch.equal(k8[slot_chunk, slot_pos], k_rows_a) and torch.equal(v8[slot_chunk, slot_pos], v_rows_a), \
+        "appended bytes differ from the separate launches"
+    assert torch.equal(ks, ks_a) and torch.equal(vs, vs_a), "scales differ from the separate launches"
+    diff = (out_a.float() - out_b.float()).abs().max().item()
+    assert diff <= 8e-3, f"one-kernel step and separate launches differ by {diff:.3e}"
