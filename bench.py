@@ -225,6 +225,132 @@ def run_secondary(args, mi, lib, torch, dev):
         "roofline": roofline})
 
 
+def run_bookkeeping(args, mi, lib, torch, dev):
+    """The host-visible bookkeeping of a decode step at serving sizes: mi_add_request per admitted prompt,
+    mi_step_attention_state for the first (prefill) step, then per decode step mi_decode_attention_state and
+    mi_update_requests with its read-back of the new counters.  R requests, a chunk table M columns wide."""
+    from importlib import import_module
+    ops = mi.ops
+    ctx_mod = import_module(mi.__name__ + ".contexts.dynamic_context")
+    chunk = 256
+    timed = {}
+
+    def timing(name):
+        inner = getattr(ops, name)
+
+        def wrapper(*a, **k):
+            ev = (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+            ev[0].record()
+            r = inner(*a, **k)
+            ev[1].record()
+            timed.setdefault(name, []).append(ev)
+            return r
+        return inner, wrapper
+
+    names = ("add_request", "step_attention_state", "decode_attention_state", "update_requests")
+    saved = {}
+    for n in names:
+        saved[n], w = timing(n)
+        setattr(ops, n, w)
+    rows = []
+    try:
+        for R in (64, 256, 1024):
+            for M in (32, 128, 512):
+                timed.clear()
+                gen = torch.Generator().manual_seed(R * 1000 + M)
+                ctx = ctx_mod.DynamicInferenceContext(
+                    params_dtype=torch.bfloat16, num_layers=1, kv_channels=64, num_attention_heads=1,
+                    max_sequence_length=M * chunk, buffer_size_gb=0.75, buffer_guaranteed_fraction=0.1,
+                    chunk_size_tokens=chunk, max_requests_override=R, max_tokens_override=R * 512, device=dev,
+                    fused_bookkeeping=True)
+                assert ctx.request_to_kv_chunk_ids.size(1) == M and ctx.max_requests >= R
+                # prompts end a few tokens before a chunk edge for a share of the requests, so the timed decode steps
+                # cross chunk boundaries (the allocating branch of the update) as well as the plain one
+                lens = torch.randint(100, 500, (R,), generator=gen)
+                lens[::4] = chunk - torch.randint(1, max(2, args.steps), (len(lens[::4]),), generator=gen)
+                prompts = [torch.randint(0, 32000, (int(n),), generator=gen).to(dev) for n in lens]
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for i, pr in enumerate(prompts):
+                    ctx.add_request(i, pr, 4096)
+                torch.cuda.synchronize()
+                add_wall_us = (time.perf_counter() - t0) * 1e6 / R
+                ctx.initialize_attention_state()            # the prefill step's state
+                for _ in range(args.warmup + args.steps - 1):
+                    ops.step_attention_state(ctx, R, ctx.padded_active_request_count, ctx.padded_active_token_count)
+                mask = torch.ones(R, dtype=torch.int32, device=dev)
+                tokens = torch.randint(0, 32000, (R,), generator=gen).to(dev)
+                ctx.update_requests(mask, tokens)
+                wall = []
+                for i in range(args.warmup + args.steps):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    ctx.initialize_attention_state()
+                    ctx.update_requests(mask, tokens)
+                    wall.append((time.perf_counter() - t0) * 1e6)
+                torch.cuda.synchronize()
+                assert ctx.total_request_count == R and ctx.paused_request_count == 0
+                # churn: 8 requests finish in a decode step (their chunks go back, rows from the right fill the holes),
+                # 8 prompts are admitted, and the next step is a mixed one
+                fin, fin_wall, mixed = [], [], []
+                next_id = R
+                for i in range(min(args.steps, 20)):
+                    ctx.initialize_attention_state()
+                    mask_f = mask.clone()
+                    mask_f[torch.randperm(R, generator=gen)[:8].to(dev)] = 0
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    ctx.update_requests(mask_f, tokens)
+                    fin_wall.append((time.perf_counter() - t0) * 1e6)
+                    fin.append(timed["update_requests"][-1])
+                    for k in range(8):
+                        ctx.add_request(next_id, prompts[(next_id * 7) % R], 4096)
+                        next_id += 1
+                    ctx.initialize_attention_state()
+                    mixed.append(timed["step_attention_state"][-1])
+                    ctx.update_requests(mask, tokens)
+                torch.cuda.synchronize()
+                assert ctx.total_request_count == R
+                mean_us = lambda evs: round(sum(a.elapsed_time(b) for a, b in evs) * 1e3 / max(1, len(evs)), 2)
+                w = args.warmup
+                rows.append({
+                    "requests": R, "table_columns": M,
+                    "add_request_us": mean_us(timed["add_request"]), "add_request_wall_us": round(add_wall_us, 2),
+                    "step_attention_state_us": mean_us(timed["step_attention_state"][w:w + args.steps]),
+                    "decode_attention_state_us": mean_us(timed["decode_attention_state"][w:w + args.steps]),
+                    "update_requests_us": mean_us(timed["update_requests"][1 + w:1 + w + args.steps]),
+                    "decode_step_wall_us": round(sum(wall[w:]) / max(1, len(wall[w:])), 2),
+                    "update_requests_8_finished_us": mean_us(fin[2:]),
+                    "update_requests_8_finished_wall_us": round(sum(fin_wall[2:]) / max(1, len(fin_wall[2:])), 2),
+                    "step_attention_state_after_admission_us": mean_us(mixed[2:]),
+                })
+                del ctx
+                torch.cuda.empty_cache()
+    finally:
+        for n in names:
+            setattr(ops, n, saved[n])
+    head = rows[-1]
+    step_us = head["decode_attention_state_us"] + head["update_requests_us"]
+    # what one decode step's two launches must move at the largest size: the block table copied into its mirror
+    # (read + write), 7 request rows read and written, 6 token rows written
+    R, M = head["requests"], head["table_columns"]
+    nbytes = R * M * 4 * 2 + R * 7 * 4 * 2 + R * 6 * 8
+    return {
+        "metric": "bookkeeping_decode_step_us", "value": head["decode_step_wall_us"], "unit": "us", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(head["decode_step_wall_us"] / 1e3, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "int32 / int64", "data": "synthetic",
+        "config": {"workload": "request / token bookkeeping of the dynamic context: value = host-visible time of one "
+                               "decode step's initialize_attention_state + update_requests (two launches, one 32-byte "
+                               "read-back) at 1024 requests and a 512-column chunk table; *_us = HIP events around each "
+                               "launch", "sizes": rows},
+        "roofline": {"bound": "hbm", "kernel": "decode_attention_state_kernel + update_requests_kernel",
+                     "achieved": round(nbytes / step_us / 1e3, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(nbytes / step_us / 1e3 / HBM_PEAK_GBPS, 5), "kernel_ms": round(step_us / 1e3, 5),
+                     "traffic": None,
+                     "note": "launch- and dependency-bound integer work: a few MB per step, so the bandwidth fraction "
+                             "only says that these launches cost microseconds, not how well they stream"}}
+
+
 def run_stream_read(args, mi, torch, dev):
     """Calibration leg: a plain read-only streaming kernel (csrc/bench/stream_read.hip, built into
     libmi355_bench.so) over a buffer of ``--read-mib`` MiB -- what a kernel that does nothing but read reaches
@@ -283,7 +409,8 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="cfg2",
-                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", *SECONDARY_WORKLOADS],
+                    choices=["cfg1", "cfg2", "cfg3", "cfg3_decode", "cfg4", "cfg5", "stream_read", "bookkeeping",
+                             *SECONDARY_WORKLOADS],
                     help="cfg2 (default) is the headline decode step; cfg3 is the mixed prefill+decode batch; the "
                          "mla_* / prefill_d* / sampling_* / log_probs_* workloads time one kernel of the rows built around the path")
     ap.add_argument("--split-tokens", type=int, default=0)
@@ -650,6 +777,8 @@ def run_workload(args, mi, lib, torch, dev):
         return run_mixed_batch(args, mi, lib, torch, dev)
     if args.workload == "stream_read":
         return run_stream_read(args, mi, torch, dev)
+    if args.workload == "bookkeeping":
+        return run_bookkeeping(args, mi, lib, torch, dev)
     if args.workload in SECONDARY_WORKLOADS:
         return run_secondary(args, mi, lib, torch, dev)
     return run_decode_config(args, mi, lib, torch, dev)

@@ -613,7 +613,7 @@ class DynamicInferenceContext:
     def reset_attention_state(self) -> None:
         """Forget the per-step attention metadata (the fixed-address mirrors are zeroed)."""
         self._max_lengths_pending = False
-        note_kv_lengths(None, None)
+        note_kv_lengths(getattr(self, 'cu_kv_seq_lengths', None), None)
         self.max_seqlen_q = None
         self.max_seqlen_k = None
         self.cu_query_seq_lengths = None

@@ -97,6 +97,11 @@ bool mi_profile_next(hipEvent_t* a, hipEvent_t* b) {
   return true;
 }
 
+bool mi_profile_is_on() {
+  std::lock_guard<std::mutex> lock(g_profile_mutex);
+  return g_profile;
+}
+
 extern "C" int mi_profile_enable(int32_t on) {
   std::lock_guard<std::mutex> lock(g_profile_mutex);
   g_profile = on != 0;

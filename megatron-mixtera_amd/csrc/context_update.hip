@@ -11,7 +11,7 @@
 // tensor the reference exposes ends up with the same contents.  The host reads back one small
 // array of counters (a single synchronisation) to refresh its Python integers.
 //
-// One workgroup of 256 threads; rows are distributed over the threads and ordered lists
+// One workgroup of 1024 threads; rows are distributed over the threads and ordered lists
 // (holes, movers, ...) are built with a block-wide prefix sum, so the order of every move and
 // of every chunk id pushed to / popped from the free stack is the reference's.
 #include "mi_common.h"
@@ -35,7 +35,32 @@ struct UpdateParams {
   int32_t total, paused, avail, gtd_chunks, gtd_requests, chunk, max_requests;
 };
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 1024;
+constexpr int kWaves = kThreads / 64;
+
+// Inclusive block-wide prefix sum of one value per thread (thread order); *total receives the sum over the block.
+// Within a wavefront by lane shuffles, across wavefronts through `sh` (at least kWaves ints).  All threads call.
+static __device__ int block_scan(int v, int* sh, int* total) {
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  int x = v;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int y = __shfl_up(x, o, 64);
+    if (lane >= o) x += y;
+  }
+  __syncthreads();  // (an earlier call's readers are done with sh)
+  if (lane == 63) sh[w] = x;
+  __syncthreads();
+  int before = 0, all = 0;
+#pragma unroll
+  for (int i = 0; i < kWaves; ++i) {
+    const int s = sh[i];
+    before += i < w ? s : 0;
+    all += s;
+  }
+  *total = all;
+  return x + before;
+}
 
 // Ordered compaction: out[k] = base + i for the k-th i in [0, n) with pred(i); returns the count.
 // Must be called by all threads of the block.
@@ -46,17 +71,8 @@ static __device__ int compact(int n, int base, int32_t* out, Pred pred, int* sh)
   const int a = min(t * seg, n), b = min(a + seg, n);
   int cnt = 0;
   for (int i = a; i < b; ++i) cnt += pred(i) ? 1 : 0;
-  __syncthreads();
-  sh[t] = cnt;
-  __syncthreads();
-  for (int o = 1; o < kThreads; o <<= 1) {
-    const int v = t >= o ? sh[t - o] : 0;
-    __syncthreads();
-    sh[t] += v;
-    __syncthreads();
-  }
-  const int total = sh[kThreads - 1];
-  int at = sh[t] - cnt;
+  int total;
+  int at = block_scan(cnt, sh, &total) - cnt;
   for (int i = a; i < b; ++i)
     if (pred(i)) out[at++] = base + i;
   __syncthreads();
@@ -76,42 +92,51 @@ static __device__ __forceinline__ void store_row(const UpdateParams& p, int i, c
 }
 
 // Push the chunk ids owned by the listed rows (ascending list order, ascending column) onto the stack.
+// One wavefront per row at a time, its lanes over the columns: the row's ids keep their column order through a
+// ballot and a count of the lower lanes.
 static __device__ int release_rows(const UpdateParams& p, const int32_t* rows, int n_rows, int avail,
                                    int32_t* counts, int* sh) {
-  const int t = threadIdx.x;
-  for (int k = t; k < n_rows; k += kThreads) {
+  const int t = threadIdx.x, lane = t & 63, w = t >> 6;
+  for (int k = w; k < n_rows; k += kWaves) {
     const int32_t* row = p.table + (int64_t)rows[k] * p.table_stride;
     int c = 0;
-    for (int j = 0; j < p.M; ++j) c += row[j] != -1;
-    counts[k] = c;
+    for (int j0 = 0; j0 < p.M; j0 += 64) {
+      const int j = j0 + lane;
+      c += __popcll(__ballot(j < p.M && row[j] != -1));
+    }
+    if (lane == 0) counts[k] = c;
   }
   __syncthreads();
-  // exclusive prefix sum of counts (in place), same block-wide scheme as compact()
+  // counts -> where each row's ids start (exclusive prefix sum, in place)
   const int seg = (n_rows + kThreads - 1) / kThreads;
   const int a = min(t * seg, n_rows), b = min(a + seg, n_rows);
   int cnt = 0;
   for (int k = a; k < b; ++k) cnt += counts[k];
-  sh[t] = cnt;
-  __syncthreads();
-  for (int o = 1; o < kThreads; o <<= 1) {
-    const int v = t >= o ? sh[t - o] : 0;
-    __syncthreads();
-    sh[t] += v;
-    __syncthreads();
-  }
-  const int total = sh[kThreads - 1];
-  int at = sh[t] - cnt;
+  int total;
+  int at = block_scan(cnt, sh, &total) - cnt;
   for (int k = a; k < b; ++k) {
+    const int c = counts[k];
+    counts[k] = at;
+    at += c;
+  }
+  __syncthreads();
+  for (int k = w; k < n_rows; k += kWaves) {
     const int32_t* row = p.table + (int64_t)rows[k] * p.table_stride;
-    for (int j = 0; j < p.M; ++j)
-      if (row[j] != -1) p.bag[avail + at++] = row[j];
+    int start = avail + counts[k];
+    for (int j0 = 0; j0 < p.M; j0 += 64) {
+      const int j = j0 + lane;
+      const int32_t v = j < p.M ? row[j] : -1;
+      const unsigned long long keep = __ballot(v != -1);
+      if (v != -1) p.bag[start + __popcll(keep & ((1ull << lane) - 1))] = v;
+      start += __popcll(keep);
+    }
   }
   __syncthreads();
   return avail + total;
 }
 
 __global__ __launch_bounds__(kThreads) void update_requests_kernel(UpdateParams p) {
-  __shared__ int sh[kThreads];
+  __shared__ int sh[kWaves];
   __shared__ int red[2];
   const int t = threadIdx.x;
   const int P0 = p.paused;
@@ -128,8 +153,15 @@ __global__ __launch_bounds__(kThreads) void update_requests_kernel(UpdateParams 
     c1 += p.mask[i] == 1;
     c0 += p.mask[i] == 0;
   }
-  atomicAdd(&red[0], c1);
-  atomicAdd(&red[1], c0);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    c1 += __shfl_xor(c1, o, 64);
+    c0 += __shfl_xor(c0, o, 64);
+  }
+  if ((t & 63) == 0) {
+    atomicAdd(&red[0], c1);
+    atomicAdd(&red[1], c0);
+  }
   __syncthreads();
   int n_cont = red[0];
   const int n_fin = red[1];
@@ -311,14 +343,15 @@ struct StepStateParams {
 __global__ __launch_bounds__(1024) void step_attention_state_kernel(StepStateParams p) {
   const int t = threadIdx.x;
   if (blockIdx.x > 0) {
-    for (int i = blockIdx.x - 1; i < p.n_active; i += gridDim.x - 1) {
-      const int r = p.paused + i;
-      for (int j = t; j < p.M; j += 1024)
-        p.table_out[(int64_t)i * p.table_out_stride + j] = p.table[(int64_t)r * p.table_stride + j];
+    const int64_t n = (int64_t)p.n_active * p.M, step = (int64_t)(gridDim.x - 1) * 1024;
+    for (int64_t e = (int64_t)(blockIdx.x - 1) * 1024 + t; e < n; e += step) {
+      const int i = (int)(e / p.M), j = (int)(e - (int64_t)i * p.M);
+      p.table_out[(int64_t)i * p.table_out_stride + j] = p.table[(int64_t)(p.paused + i) * p.table_stride + j];
     }
     return;
   }
-  __shared__ int sh_q[1024], sh_k[1024];
+  static_assert(kThreads == 1024, "block_scan covers the workgroup of this kernel");
+  __shared__ int sh_q[kWaves], sh_k[kWaves];
   __shared__ int red[2];
   if (t < 2) red[t] = 0;
   const int seg = (p.R + 1023) / 1024;
@@ -334,25 +367,32 @@ __global__ __launch_bounds__(1024) void step_attention_state_kernel(StepStatePar
     sq += q; sk += k;
     mq = max(mq, q); mk = max(mk, k);
   }
-  sh_q[t] = sq; sh_k[t] = sk;
-  __syncthreads();
-  for (int o = 1; o < 1024; o <<= 1) {
-    const int vq = t >= o ? sh_q[t - o] : 0, vk = t >= o ? sh_k[t - o] : 0;
-    __syncthreads();
-    sh_q[t] += vq; sh_k[t] += vk;
-    __syncthreads();
-  }
-  int cq = sh_q[t] - sq, ck = sh_k[t] - sk;  // sums before this thread's rows
+  int all_q, all_k;
+  int cq = block_scan(sq, sh_q, &all_q) - sq, ck = block_scan(sk, sh_k, &all_k) - sk;  // sums before this thread's rows
   if (t == 0) { p.cu_q_out[0] = 0; p.cu_kv_out[0] = 0; }
-  for (int i = a; i < b; ++i) {
-    const int q = i < p.n_active ? p.q_len[p.paused + i] : 0;
-    const int k = i < p.n_active ? p.kv_off[p.paused + i] + q : 0;
-    cq += q; ck += k;
-    p.cu_q_out[i + 1] = cq;
-    p.cu_kv_out[i + 1] = ck;
+  if (seg == 1) {  // (one row per thread: its lengths are still in sq / sk)
+    if (a < b) {
+      p.cu_q_out[a + 1] = cq + sq;
+      p.cu_kv_out[a + 1] = ck + sk;
+    }
+  } else {
+    for (int i = a; i < b; ++i) {
+      const int q = i < p.n_active ? p.q_len[p.paused + i] : 0;
+      const int k = i < p.n_active ? p.kv_off[p.paused + i] + q : 0;
+      cq += q; ck += k;
+      p.cu_q_out[i + 1] = cq;
+      p.cu_kv_out[i + 1] = ck;
+    }
   }
-  atomicMax(&red[0], mq);
-  atomicMax(&red[1], mk);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {  // one LDS atomic per wavefront instead of one per thread
+    mq = max(mq, __shfl_xor(mq, o, 64));
+    mk = max(mk, __shfl_xor(mk, o, 64));
+  }
+  if ((t & 63) == 0) {
+    atomicMax(&red[0], mq);
+    atomicMax(&red[1], mk);
+  }
   for (int tk = p.active_tokens + t; tk < p.padded; tk += 1024) {
     p.tok_chunk[tk] = p.dummy_chunk;
     p.tok_local[tk] = 0;
@@ -461,8 +501,10 @@ extern "C" int mi_step_attention_state(
   p.tok_in_req = token_to_position_in_request; p.maxes = max_lengths_out;
   p.paused = paused_request_count; p.n_active = active_request_count; p.R = padded_request_count;
   p.padded = padded_active_token_count; p.active_tokens = active_token_count; p.dummy_chunk = dummy_chunk_idx;
-  int copy_blocks = active_request_count < 255 ? active_request_count : 255;
-  hipLaunchKernelGGL(step_attention_state_kernel, dim3(1 + copy_blocks), dim3(1024), 0, (hipStream_t)stream, p);
+  // enough copy workgroups that a thread moves one or two table entries (every load in flight at once)
+  int64_t copy_blocks = ((int64_t)active_request_count * max_kv_chunk_count + 1023) / 1024;
+  if (copy_blocks > 512) copy_blocks = 512;
+  hipLaunchKernelGGL(step_attention_state_kernel, dim3(1 + (int)copy_blocks), dim3(1024), 0, (hipStream_t)stream, p);
   return mi_check_launch("mi_step_attention_state");
 }
 

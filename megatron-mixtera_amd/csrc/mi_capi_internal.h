@@ -19,6 +19,8 @@ int mi_fail(int code, const char* msg);
 int mi_check_launch(const char* where);
 // Next start/stop event pair when kernel timing is enabled (see mi_profile_enable).
 bool mi_profile_next(hipEvent_t* start, hipEvent_t* stop);
+// Whether kernel timing is switched on (timed launches may create events, which allocates).
+bool mi_profile_is_on();
 
 namespace mi {
 int decode_grid_size(int Hq, int Hkv, const MiTuning& tune);
@@ -43,6 +45,10 @@ struct FusedStepArgs {
 };
 // Shared by the decode entry point and by the mixed-batch path of the prefill entry point
 // (cu_seqlens_q non-null: only requests with one query row take part, at row cu_seqlens_q[r]).
+// The workspace checks of launch_paged_decode alone (size for R requests, alignment), for callers that must know
+// the decode launches can go ahead before they enqueue anything else.  MI_OK or a negative code with a message.
+int check_decode_workspace(const void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq, int32_t Hkv,
+                           int32_t head_dim, int32_t split_tokens, const MiTuning& tune, const char* who);
 int launch_paged_decode(const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
                         const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok,
                         int64_t kv_stride_head, const int32_t* block_table, int64_t bt_stride,

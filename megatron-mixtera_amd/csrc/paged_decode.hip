@@ -1685,6 +1685,28 @@ extern "C" int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv,
   return slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
 }
 
+int mi::check_decode_workspace(const void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq, int32_t Hkv,
+                               int32_t head_dim, int32_t split_tokens, const MiTuning& tune, const char* who) {
+  static thread_local char msg[192];
+  if (split_tokens < 0 || split_tokens % 16) {
+    snprintf(msg, sizeof msg, "%s: split_tokens must be a non-negative multiple of 16", who);
+    return mi_fail(MI_ERR_SHAPE, msg);
+  }
+  // a batch above kMaxRequestsPerLaunch runs in slices of that many requests over the same workspace
+  const int64_t n = R < kMaxRequestsPerLaunch ? R : kMaxRequestsPerLaunch;
+  const int64_t slots = (int64_t)decode_grid_size(Hq, Hkv, tune) + n;
+  const int64_t need = slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + n * 2 * (int64_t)sizeof(int32_t);
+  if (!workspace || workspace_bytes < need) {
+    snprintf(msg, sizeof msg, "%s: workspace too small (see mi_decode_workspace_bytes)", who);
+    return mi_fail(MI_ERR_WORKSPACE, msg);
+  }
+  if ((uintptr_t)workspace & 15) {
+    snprintf(msg, sizeof msg, "%s: workspace must be 16-byte aligned", who);
+    return mi_fail(MI_ERR_ALIGN, msg);
+  }
+  return MI_OK;
+}
+
 int mi::launch_paged_decode(
     const void* q, int64_t q_stride_tok, int64_t q_stride_head, const void* k_cache,
     const void* v_cache, int64_t kv_stride_chunk, int64_t kv_stride_tok, int64_t kv_stride_head,
@@ -1721,16 +1743,15 @@ int mi::launch_paged_decode(
     return mi_fail(MI_ERR_ALIGN, "mi_paged_decode_attention: strides must keep rows 16-byte aligned");
   if (kv_stride_tok * (int64_t)chunk_tokens * esz >= (int64_t)1 << 31)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: one chunk must span less than 2 GiB");
-  if (split_tokens < 0 || split_tokens % 16)
-    return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: split_tokens must be a non-negative multiple of 16");
   // The per-request prefix sums and lengths live in LDS (8 bytes per request): a larger batch is streamed in
   // slices of kMaxRequestsPerLaunch requests, one after the other on the same stream and workspace.  Every
   // argument check above is independent of the slice, so either all slices run or none does.
+  {
+    const int rc_w = check_decode_workspace(workspace, workspace_bytes, R, Hq, Hkv, head_dim, split_tokens, tune,
+                                            "mi_paged_decode_attention");
+    if (rc_w != MI_OK) return rc_w;
+  }
   if (R > kMaxRequestsPerLaunch) {
-    const int64_t slots_all = (int64_t)decode_grid_size(Hq, Hkv, tune) + kMaxRequestsPerLaunch;
-    if (!workspace || workspace_bytes < slots_all * Hq * (head_dim + 1) * (int64_t)sizeof(float) +
-                                            (int64_t)kMaxRequestsPerLaunch * 2 * (int64_t)sizeof(int32_t))
-      return mi_fail(MI_ERR_WORKSPACE, "mi_paged_decode_attention: workspace too small (see mi_decode_workspace_bytes)");
     for (int r0 = 0; r0 < R; r0 += kMaxRequestsPerLaunch) {
       const int n = R - r0 < kMaxRequestsPerLaunch ? R - r0 : kMaxRequestsPerLaunch;
       // with cu_seqlens_q the rows of q / out are addressed through it, else request r owns row r
@@ -1755,11 +1776,6 @@ int mi::launch_paged_decode(
 
   const int grid_x = decode_grid_size(Hq, Hkv, tune);
   const int64_t slots = (int64_t)grid_x + R;
-  const int64_t need = slots * Hq * (head_dim + 1) * (int64_t)sizeof(float) + (int64_t)R * 2 * sizeof(int32_t);
-  if (!workspace || workspace_bytes < need)
-    return mi_fail(MI_ERR_WORKSPACE, "mi_paged_decode_attention: workspace too small (see mi_decode_workspace_bytes)");
-  if ((uintptr_t)workspace & 15)
-    return mi_fail(MI_ERR_ALIGN, "mi_paged_decode_attention: workspace must be 16-byte aligned");
 
   // 16-token sub-tiles per loop iteration (0 = automatic).
   int nt = tune.decode_tile_subtiles;
@@ -2023,6 +2039,11 @@ extern "C" int mi_paged_decode_attention_noalloc(
     return mi_fail(MI_ERR_WORKSPACE,
                    "mi_paged_decode_attention_noalloc: these sizes need more than the 16 MiB of built-in scratch "
                    "(see mi_decode_workspace_bytes); use mi_paged_decode_attention with a workspace");
+  // a timed launch takes an event pair from a pool that grows by creating events: not for this entry point
+  if (mi_profile_is_on())
+    return mi_fail(MI_ERR_UNSUPPORTED,
+                   "mi_paged_decode_attention_noalloc: kernel timing is on (mi_profile_enable), and timed launches "
+                   "may create events; switch it off for callers that must not allocate");
   void* ptr = nullptr;
   const int rc = noalloc_scratch(&ptr);
   if (rc != MI_OK) return rc;

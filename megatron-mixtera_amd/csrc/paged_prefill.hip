@@ -1060,6 +1060,8 @@ static int launch_paged_prefill(
     return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention: strides must keep rows 16-byte aligned");
   if (kv_stride_tok * (int64_t)chunk_tokens * 2 >= (int64_t)1 << 31)
     return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: one chunk must span less than 2 GiB");
+  if (fp8 && (kv_stride_chunk | kv_stride_tok | kv_stride_head) % 16)
+    return mi_fail(MI_ERR_ALIGN, "mi_paged_prefill_attention_fp8: cache strides must keep rows 16-byte aligned");
   if (kv_dtype != MI_KV_16BIT && !fp8)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_prefill_attention: unknown kv_dtype");
   if (fp8 && (!k_scales || !v_scales))
@@ -1090,6 +1092,14 @@ static int launch_paged_prefill(
   p.skip_single = workspace != nullptr;
   p.k_scale = k_scales; p.v_scale = v_scales;
   p.split_o = nullptr; p.split_lse = nullptr;
+
+  // The decode part's own argument checks come before the first launch, so that a negative return still means
+  // nothing was enqueued (its remaining checks repeat ones made above).
+  if (p.skip_single) {
+    const int rc_w = check_decode_workspace(workspace, workspace_bytes, R, Hq, Hkv, head_dim, split_tokens, tune,
+                                            "mi_paged_prefill_attention");
+    if (rc_w != MI_OK) return rc_w;
+  }
 
   hipStream_t st = (hipStream_t)stream;
   if (two_phase) {

@@ -9,6 +9,7 @@ silently ignored.
 """
 from __future__ import annotations
 
+import weakref
 from typing import Optional
 
 import torch
@@ -19,23 +20,28 @@ from . import ops
 
 # Per-request kv lengths that belong to a cu_seqlens_k tensor, published by the context that built both
 # (DynamicInferenceContext.initialize_attention_state).  The reference's call site hands flash_attn_varlen_func only
-# the running sums (attention.py:546-557); with this note the lengths need not be recomputed by a
-# subtraction + copy in every layer.  One entry: (data_ptr, numel, version) of the sums -> lengths.
-_kv_lengths_note = None
+# the running sums (attention.py:546-557); with a note the lengths need not be recomputed by a subtraction + copy in
+# every layer.  Notes are keyed by the identity of the sums tensor OBJECT and die with it (a weak reference), so a
+# later tensor that happens to reuse the address never inherits them, and several contexts keep one note each.
+_kv_lengths_notes = {}
 
 
 def note_kv_lengths(cu_seqlens_k: Optional[Tensor], kv_lens: Optional[Tensor]) -> None:
-    """Remember that ``kv_lens`` are the differences of ``cu_seqlens_k`` (``None`` forgets)."""
-    global _kv_lengths_note
-    if cu_seqlens_k is None or kv_lens is None:
-        _kv_lengths_note = None
-    else:
-        _kv_lengths_note = ((cu_seqlens_k.data_ptr(), cu_seqlens_k.numel(), cu_seqlens_k._version), kv_lens)
+    """Remember that ``kv_lens`` are the differences of ``cu_seqlens_k``; ``kv_lens=None`` forgets that tensor's
+    note, ``cu_seqlens_k=None`` is a no-op."""
+    if cu_seqlens_k is None:
+        return
+    key = id(cu_seqlens_k)
+    if kv_lens is None:
+        _kv_lengths_notes.pop(key, None)
+        return
+    ref = weakref.ref(cu_seqlens_k, lambda _r, key=key: _kv_lengths_notes.pop(key, None))
+    _kv_lengths_notes[key] = (ref, kv_lens)
 
 
 def _lengths_of(cu_seqlens_k: Tensor) -> Tensor:
-    note = _kv_lengths_note
-    if note is not None and note[0] == (cu_seqlens_k.data_ptr(), cu_seqlens_k.numel(), cu_seqlens_k._version):
+    note = _kv_lengths_notes.get(id(cu_seqlens_k))
+    if note is not None and note[0]() is cu_seqlens_k:
         return note[1]
     return (cu_seqlens_k[1:] - cu_seqlens_k[:-1]).contiguous()
 

@@ -335,3 +335,26 @@ def test_query_head_groups_that_are_not_powers_of_two(mi, dev, kernel, Hq, Hkv, 
     assert torch.isfinite(got).all() and (got[T:] == 0).all()
     err = (got[:T] - ref).abs()
     assert (err <= 2e-2 + 2e-2 * ref.abs()).all(), f"max err {err.max().item():.4e}"
+
+
+@pytest.mark.parametrize("fault", ["short", "misaligned"])
+def test_a_bad_workspace_is_refused_before_anything_is_launched(mi, dev, fault):
+    """A mixed batch hands its one-row requests to the decode kernels after the tile kernel; a workspace those cannot
+    use must be refused before the tile kernel is enqueued (a negative return = nothing launched)."""
+    lib = mi._lib.load()
+    q, kc, vc, cu_q, lens, bt = mi.synthetic.make_prefill_case(
+        dev, n_prefill=2, new_tokens=100, ctx_lo=0, ctx_hi=200, n_decode=4, dec_lo=1, dec_hi=500,
+        Hq=32, Hkv=8, d=128, chunk=64, seed=5)
+    T, R = q.shape[0], lens.numel()
+    need = lib.mi_prefill_workspace_bytes(T, R, 32, 8, 128, int(lens.max()), 0, None)
+    buf = torch.empty(need + 64, dtype=torch.uint8, device=dev)
+    ws_ptr, ws_bytes = (buf.data_ptr(), 1024) if fault == "short" else (buf.data_ptr() + 4, need)
+    out = torch.full_like(q, float("nan"))
+    ks = kc.stride()
+    rc = lib.mi_paged_prefill_attention(
+        q.data_ptr(), q.stride(0), q.stride(1), kc.data_ptr(), vc.data_ptr(), ks[0], ks[1], ks[2], bt.data_ptr(),
+        bt.stride(0), cu_q.data_ptr(), lens.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1), ws_ptr, ws_bytes,
+        T, R, 32, 8, 128, 64, int(lens.max()), 0, 128 ** -0.5, 0, None, None)
+    torch.cuda.synchronize()
+    assert rc < 0 and b"workspace" in lib.mi_last_error()
+    assert torch.isnan(out.float()).all(), "rows were written although the call was refused"

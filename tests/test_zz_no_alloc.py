@@ -48,11 +48,15 @@ def _with_workspace(lib, case):
 def _no_alloc(lib, case):
     out = torch.full_like(case.q, float("nan"))
     head, tail = _args(case, out)
-    before = torch.cuda.memory_allocated()
+    # the device's own free-memory figure sees every allocation of the process (the library's hipMalloc or event
+    # pools included), torch's counter only its caching allocator's
+    torch.cuda.synchronize()
+    before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
     rc = lib.mi_paged_decode_attention_noalloc(*head, *tail)
     assert rc == 0, lib.mi_last_error()
     torch.cuda.synchronize()
     assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] >= free_before, "device memory was taken during the call"
     return out
 
 
@@ -112,3 +116,24 @@ def test_sizes_beyond_the_scratch_are_rejected(mi, dev):
     rc = lib.mi_paged_decode_attention_noalloc(one, Hq * D, D, one, one, 256 * Hkv * D, Hkv * D, D, one, 16, one, one,
                                                Hq * D, D, R, Hq, Hkv, D, 256, 4096, 0, 0.1, 0, None, None, 0, None, None)
     assert rc == -5 and b"16 MiB" in lib.mi_last_error()
+
+
+def test_refused_while_kernel_timing_is_on(mi, dev):
+    """Timed launches draw event pairs from a pool that grows by creating events, so the entry point that must not
+    allocate returns an error instead while timing is enabled."""
+    lib = mi._lib.load()
+    syn = mi.synthetic
+    case = syn.make_decode_case(syn.DecodeConfig("na-prof", 4, 32, 8, 128, 100, 400, chunk=256, seed=43), dev)
+    out = torch.full_like(case.q, float("nan"))
+    head, tail = _args(case, out)
+    assert lib.mi_profile_enable(1) == 0
+    try:
+        rc = lib.mi_paged_decode_attention_noalloc(*head, *tail)
+        assert rc < 0 and "timing" in lib.mi_last_error().decode()
+    finally:
+        assert lib.mi_profile_enable(0) == 0
+    torch.cuda.synchronize()
+    assert torch.isnan(out.float()).all(), "nothing may have been launched"
+    assert lib.mi_paged_decode_attention_noalloc(*head, *tail) == 0, lib.mi_last_error()
+    torch.cuda.synchronize()
+    _check_vs_oracle(case, out)
