@@ -130,15 +130,24 @@ def run_secondary(args, mi, lib, torch, dev):
     elif kind == "linear":
         T, N, K = prm["T"], prm["N"], prm["K"]
         x = (torch.randn(T, K, generator=gen) * 0.5).bfloat16().to(dev)
-        w = torch.empty(N, K, dtype=torch.bfloat16, device=dev).normal_(0, K ** -0.5)
+        # a model's layers each bring their own matrix from HBM: the step walks a ring of matrices larger than the
+        # 256 MB last-level cache, so that no call finds its weights cached from the call before
+        n_w = max(2, -(-320 * 1024 * 1024 // (N * K * 2)))
+        ws = [torch.empty(N, K, dtype=torch.bfloat16, device=dev).normal_(0, K ** -0.5) for _ in range(n_w)]
+        w = ws[0]
         bias_t = torch.randn(N, generator=gen).bfloat16().to(dev) if prm["bias"] else None
         out = torch.empty(T, N, dtype=torch.bfloat16, device=dev)
-        step = lambda: mi.ops.linear_decode(x, w, bias_t, out=out)
+        ring = {"i": 0}
+
+        def step():
+            ring["i"] = (ring["i"] + 1) % n_w
+            mi.ops.linear_decode(x, ws[ring["i"]], bias_t, out=out)
         nbytes = N * K * 2 + T * K * 2 + T * N * 2 + (N * 2 if prm["bias"] else 0)
         flops = 2 * T * N * K
         kernel = "linear_decode_kernel"
         what = (f"y[{T}, {N}] = x[{T}, {K}] . W[{N}, {K}]^T{' + bias' if prm['bias'] else ''}: the weight matrix streamed "
-                f"once, fp32 partial sums over slices of K and their reduction launch included in the step")
+                f"once (a ring of {n_w} matrices, so every call reads its weights from HBM), fp32 partial sums over slices "
+                f"of K and their reduction launch included in the step")
         dtype = "bf16 (fp32 accumulate)"
         timed_by_library = True
     elif kind == "sampling":
@@ -203,7 +212,9 @@ def run_secondary(args, mi, lib, torch, dev):
     roofline.update({"kernel_ms": round(kernel_ms, 5), "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload)})
     if kind == "linear":
         # the library's GEMM on the same operands, timed the same way (what the reference's linear layers call)
-        lin = lambda: torch.nn.functional.linear(x, w, bias_t)
+        def lin():
+            ring["i"] = (ring["i"] + 1) % n_w
+            torch.nn.functional.linear(x, ws[ring["i"]], bias_t)
         for _ in range(args.warmup):
             lin()
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]

@@ -10,9 +10,10 @@
 //
 // Work split: a workgroup of 8 wavefronts takes 128 rows of W (16 per wavefront, the A operand of mfma 16x16x32)
 // times one slice of at most 512 columns of K, for a block of at most 64 tokens.  Every wavefront asks for its whole
-// share of W at once -- sixteen 16-byte loads per lane, 16 KB per wavefront, non-temporal -- so the launch has the
-// entire matrix in flight from its first microsecond; while those loads travel the workgroup stages its slice of x in
-// LDS (64 tokens x 512 values, read by all 8 wavefronts as the B operand).  Slices of K end in fp32 partial sums
+// share of W at once -- sixteen 16-byte loads per lane, 16 KB per wavefront, non-temporal, whole cache lines per
+// instruction -- so the launch has the entire matrix in flight from its second microsecond, and multiplies each
+// piece as it arrives; before that the workgroup stages its slice of x in LDS (64 tokens x 512 values, read by all 8
+// wavefronts as the B operand).  Slices of K end in fp32 partial sums
 // (one contiguous tile of T x 16 per slice and wavefront) that a second, small kernel adds up in a fixed order (so results do not depend on timing), adds the
 // bias to and rounds; a call whose K fits one slice writes its 16-bit result directly.
 #include "mi_common.h"
@@ -48,15 +49,9 @@ __global__ __launch_bounds__(512, 4) void linear_decode_kernel(LinearParams p) {
   const int nkk = klen >> 5;                            // 32-column steps of the products (<= 16)
   const bool rows_live = n0 < p.N;                      // (wave-uniform; N is a multiple of 16)
 
-  // ---- this wavefront's share of W: lane (m16, g) holds columns k0 + 32 kk + 8 g .. + 7 of row n0 + m16 ----
-  uint4 wf[kLinSlice / 32];
-  {
-    const uint16_t* wrow = p.w + (int64_t)min(n0 + m16, p.N - 1) * p.w_st + k0 + 8 * g;
-#pragma unroll
-    for (int kk = 0; kk < kLinSlice / 32; ++kk)
-      wf[kk] = (rows_live && kk < nkk) ? ld16_stream(wrow + 32 * kk) : make_uint4(0u, 0u, 0u, 0u);
-  }
-  // ---- x[t0 .. t0 + nt)[k0 .. k0 + klen) -> LDS (rows and columns beyond stay zero) ----
+  // ---- x[t0 .. t0 + nt)[k0 .. k0 + klen) -> LDS (rows and columns beyond stay zero).  Before anything of W is asked
+  // for: loads are served in the order a CU issued them, and behind sixteen loads of W per lane these few cache
+  // hits would wait for microseconds ----
   {
     constexpr int PPR = kLinSlice / 8;  // 16-byte pieces per staged row
 #pragma unroll
@@ -68,6 +63,24 @@ __global__ __launch_bounds__(512, 4) void linear_decode_kernel(LinearParams p) {
     }
   }
   __syncthreads();
+  // ---- this wavefront's share of W.  The products want lane (m16, g) to hold columns 32 kk + 8 g .. + 7 of row
+  // n0 + m16; loaded that way an instruction touches 64 bytes of each of 16 rows, half a cache line each.  So a pair
+  // of loads covers whole lines instead -- load 2 j: rows n0 .. + 7, load 2 j + 1: rows n0 + 8 .. + 15, each lane
+  // (m16, g) the 16 bytes at column 64 j + 8 (g + 4 (m16 >> 3)) of row (m16 & 7) -- and two moves per register within
+  // the 16-lane rows put the halves where the products expect them. ----
+  uint4 wf[kLinSlice / 32];
+  {
+    const int lo = m16 & 7, hi = m16 >> 3;
+    const int col = 8 * (g + 4 * hi);   // within a 64-column pair of steps
+    const uint16_t* wrow = p.w + (int64_t)min(n0 + lo, p.N - 1) * p.w_st + k0 + col;
+    const int64_t half = 8 * p.w_st;    // (N is a multiple of 16: rows n0 + 8 .. exist whenever rows_live)
+#pragma unroll
+    for (int j = 0; j < kLinSlice / 64; ++j) {
+      const bool live = rows_live && 64 * j + col < klen;
+      wf[2 * j] = live ? ld16_stream(wrow + 64 * j) : make_uint4(0u, 0u, 0u, 0u);
+      wf[2 * j + 1] = live ? ld16_stream(wrow + half + 64 * j) : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
   if (!rows_live) return;
 
   const int ntile = (nt + 15) >> 4;  // 16-token tiles with a live token
@@ -79,6 +92,15 @@ __global__ __launch_bounds__(512, 4) void linear_decode_kernel(LinearParams p) {
   // would index them at run time)
 #pragma unroll
   for (int kk = 0; kk < kLinSlice / 32; ++kk) {
+    if ((kk & 1) == 0 && kk < nkk) {
+      // lanes 8-15 of every 16 take the rows-8-15 load's lanes 0-7 (columns 8 g ..), lanes 0-7 the rows-0-7 load's
+      // lanes 8-15 (columns 32 + 8 g ..): row_ror:8 with a bank mask writes just those lanes
+      const uint4 a = wf[kk], b = wf[kk + 1];
+      auto upper = [](uint32_t keep, uint32_t from) { return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)from, 0x128, 0xf, 0xc, false); };
+      auto lower = [](uint32_t keep, uint32_t from) { return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)from, 0x128, 0xf, 0x3, false); };
+      wf[kk] = make_uint4(upper(a.x, b.x), upper(a.y, b.y), upper(a.z, b.z), upper(a.w, b.w));
+      wf[kk + 1] = make_uint4(lower(b.x, a.x), lower(b.y, a.y), lower(b.z, a.z), lower(b.w, a.w));
+    }
     if (kk < nkk) {
 #pragma unroll
       for (int i = 0; i < kLinTok / 16; ++i) {
@@ -178,8 +200,9 @@ extern "C" int mi_linear_decode(const void* x, int64_t x_stride_tok, const void*
   p.x = (const uint16_t*)x; p.x_st = x_stride_tok; p.w = (const uint16_t*)weight; p.w_st = w_stride_row;
   p.bias = (const uint16_t*)bias; p.out = (uint16_t*)out; p.o_st = out_stride_tok;
   p.T = T; p.N = N; p.K = K;
-  linear_split(T, N, K, &p.S, &p.kslice);
   p.part = nullptr;
+  hipStream_t st = (hipStream_t)stream;
+  linear_split(T, N, K, &p.S, &p.kslice);
   if (p.S > 1) {
     const int64_t need = (int64_t)p.S * T * N * (int64_t)sizeof(float);
     if (!workspace || workspace_bytes < need)
@@ -187,7 +210,6 @@ extern "C" int mi_linear_decode(const void* x, int64_t x_stride_tok, const void*
     if ((uintptr_t)workspace & 15) return mi_fail(MI_ERR_ALIGN, "mi_linear_decode: the workspace must be 16-byte aligned");
     p.part = (float*)workspace;
   }
-  hipStream_t st = (hipStream_t)stream;
   const dim3 grid((N + kLinRows - 1) / kLinRows, p.S, (T + kLinTok - 1) / kLinTok);
   hipEvent_t ev_a, ev_b;
   const bool timed = mi_profile_next(&ev_a, &ev_b);
