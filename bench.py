@@ -35,22 +35,22 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 # read from inside the benchmark, so the figure is recorded here per workload; None = not collected.
 MEASURED_HBM_TRAFFIC_BYTES = {
     # decode workloads: "<cfg>" = the attention-only streaming kernel, "<cfg>_step" = the one-kernel decode step
-    "cfg2": 1_226_700_000, "cfg2_step": 1_215_100_000, "cfg4": 8_724_600_000, "cfg4_step": 8_635_100_000,
-    "cfg5": 9_070_700_000,
+    "cfg2": 1_226_800_000, "cfg2_step": 1_215_100_000, "cfg4": 8_725_300_000, "cfg4_step": 8_635_100_000,
+    "cfg5": 9_071_100_000, "cfg5_step": 9_049_800_000,
     # the mixed step: tile kernel, stream kernel
-    "cfg3_tile": 401_600_000, "cfg3_stream": 2_195_400_000,
+    "cfg3_tile": 401_700_000, "cfg3_stream": 2_195_700_000,
     # multi-latent decode at 128 heads (reads + the partial results it writes)
     "mla_decode_h128": 454_500_000, "mla_decode_h128_long": 1_305_000_000}
 # Where each figure above was read, so that a reader of the JSON line can tell a stale constant from a fresh one:
 # the summary file and the last commit that touched the kernel when the counters were collected.
 _DECODE_TRAFFIC = ("profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
-                   "kernels as of commit bc375af)")
-_MIXED_TRAFFIC = ("profiles/paged_prefill_pp_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
-                  "commit bc375af)")
+                   "kernels as of commit 74dce26)")
+_MIXED_TRAFFIC = ("profiles/paged_prefill_woven_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
+                  "commit 74dce26)")
 _MLA_HEADS_TRAFFIC = ("profiles/paged_mla_decode_heads_kernel_h128_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                       "kernel as of commit c8e09ff; the row pitch changed since, the traffic does not depend on it)")
 TRAFFIC_SOURCE = {"mla_decode_h128": _MLA_HEADS_TRAFFIC, "mla_decode_h128_long": _MLA_HEADS_TRAFFIC, "cfg2": _DECODE_TRAFFIC, "cfg2_step": _DECODE_TRAFFIC, "cfg4": _DECODE_TRAFFIC,
-                  "cfg4_step": _DECODE_TRAFFIC, "cfg5": _DECODE_TRAFFIC, "cfg3_tile": _MIXED_TRAFFIC,
+                  "cfg4_step": _DECODE_TRAFFIC, "cfg5": _DECODE_TRAFFIC, "cfg5_step": _DECODE_TRAFFIC, "cfg3_tile": _MIXED_TRAFFIC,
                   "cfg3_stream": _MIXED_TRAFFIC}
 
 
@@ -225,6 +225,28 @@ def run_secondary(args, mi, lib, torch, dev):
         torch.cuda.synchronize()
         roofline["library_gemm_ms"] = round(sum(a.elapsed_time(b2) for a, b2 in ev) / args.steps, 5)
         roofline["call_ms"] = round(call_ms, 5)
+        # both again as 3 x n_w calls captured in a HIP graph and replayed: GPU time per call without the host's
+        # launch cost (the eager figures above are bound by it: two launches here, one in the library)
+        nbytes_ws = lib.mi_linear_decode_workspace_bytes(T, N, K)
+        fixed_ws = torch.empty(max(nbytes_ws, 16), dtype=torch.uint8, device=dev)
+
+        def replayed(fn):
+            graph = torch.cuda.CUDAGraph()
+            with mi.ops.use_workspace(fixed_ws), torch.cuda.graph(graph):
+                for _ in range(3 * n_w):
+                    fn()
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize()
+            a, b2 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(10):
+                graph.replay()
+            b2.record()
+            torch.cuda.synchronize()
+            return round(a.elapsed_time(b2) / (30 * n_w), 5)
+        roofline["call_ms_graph"] = replayed(step)
+        roofline["library_gemm_ms_graph"] = replayed(lin)
     if args.workload in TRAFFIC_SOURCE:
         roofline["traffic_source"] = TRAFFIC_SOURCE[args.workload]
     return ({
