@@ -177,7 +177,7 @@ int64_t mi_decode_workspace_bytes(int32_t R, int32_t Hq, int32_t Hkv, int32_t he
  *   out[r,h] = softmax(q[r,h] . K_r[:len_r, h/G]^T * softmax_scale) . V_r[:len_r, h/G]
  *   K_r[j] = k_cache[block_table[r, j / chunk_tokens], j % chunk_tokens], G = Hq/Hkv.
  * q/out: bf16 or fp16 `[R, Hq, d]` with the given token / head strides; d 64, 96, 128, 192 or 256 (an fp8 cache:
- * 128); G any value up to 64 (not only powers of two; every 16 query heads of a KV head take a wavefront).  kv_lens int32 [R] (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] (the reference
+ * 64 or 128); G any value up to 64 (not only powers of two; every 16 query heads of a KV head take a wavefront).  kv_lens int32 [R] (0 => that row's output is zeros).  `max_kv_len` bounds every kv_lens[r] (the reference
  * passes max_sequence_length here, dynamic_context.py:791); the grid does not depend on
  * it.  `split_tokens` = minimum tokens one workgroup streams (0 = default 64).
  * kv_dtype MI_KV_FP8_E4M3 reads byte caches with k_scales/v_scales `[n_chunks, Hkv]`.
@@ -332,8 +332,8 @@ int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_st
 /*
  * The same call over an fp8-e4m3 cache (byte caches `[n_chunks, chunk_tokens, Hkv, d]`, strides in
  * elements = bytes, fp32 scales `[n_chunks, Hkv]`; no counterpart in the reference).  Tiles are
- * multiplied by their chunk's scale and rounded to bf16 on their way into LDS.  Needs head_dim 128
- * and a chunk size that is a multiple of 64.
+ * multiplied by their chunk's scale and rounded to bf16 on their way into LDS.  Needs head_dim 64
+ * or 128, bf16 queries and a chunk size that is a multiple of 64.
  */
 int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
                                    const void* k_cache_fp8, const void* v_cache_fp8,

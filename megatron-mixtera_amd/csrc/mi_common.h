@@ -171,8 +171,10 @@ static __device__ __forceinline__ uint2 ld8_stream(const void* p) {
 typedef uint32_t u32x3a4_t __attribute__((ext_vector_type(3), aligned(4)));
 template <int N>
 static __device__ __forceinline__ void ld_dwords_stream(const void* p, uint32_t (&dst)[N]) {
-  static_assert(N == 3 || N % 2 == 0, "dword counts of the value fragments");
-  if constexpr (N % 4 == 0) {
+  static_assert(N == 1 || N == 3 || N % 2 == 0, "dword counts of the value fragments");
+  if constexpr (N == 1) {
+    dst[0] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p));
+  } else if constexpr (N % 4 == 0) {
 #pragma unroll
     for (int w = 0; w < N / 4; ++w) {
       const uint4 v = ld16_stream(reinterpret_cast<const uint8_t*>(p) + 16 * w);
@@ -191,8 +193,10 @@ static __device__ __forceinline__ void ld_dwords_stream(const void* p, uint32_t 
 }
 template <int N>
 static __device__ __forceinline__ void ld_dwords(const void* p, uint32_t (&dst)[N]) {  // the cacheable form
-  static_assert(N == 3 || N % 2 == 0, "dword counts of the value fragments");
-  if constexpr (N % 4 == 0) {
+  static_assert(N == 1 || N == 3 || N % 2 == 0, "dword counts of the value fragments");
+  if constexpr (N == 1) {
+    dst[0] = *reinterpret_cast<const uint32_t*>(p);
+  } else if constexpr (N % 4 == 0) {
 #pragma unroll
     for (int w = 0; w < N / 4; ++w) {
       const uint4 v = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint8_t*>(p) + 16 * w);

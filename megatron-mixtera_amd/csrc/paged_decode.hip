@@ -119,9 +119,9 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   constexpr bool SHARED_KV = HDK != HDV;
   constexpr int kQPitch = HDK * 2 + 16;
   constexpr int DV = HDV / 16;
-  constexpr int VD = FP8 ? 2 : DV / 2;  // dwords per token and lane of the value operand
+  constexpr int VD = FP8 ? DV / 4 : DV / 2;  // dwords per token and lane of the value operand
   static_assert(HDK % 32 == 0 && HDV % 32 == 0 && HDK >= 64 && HDV >= 64, "head widths: multiples of 32");
-  static_assert(!FP8 || (HDK == 128 && HDV == 128 && !F16), "fp8 KV: head_dim 128, bf16 queries");
+  static_assert(!FP8 || (HDK == HDV && (HDK == 64 || HDK == 128) && !F16), "fp8 KV: head_dim 64 or 128, bf16 queries");
   static_assert(!FUSED || (HDK == HDV && HDK <= 256), "fused step: an ordinary per-head cache");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
@@ -452,7 +452,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   // scores of the current one exist, V of the next tile as soon as the current P.V is done,
   // so every wave keeps loads in flight while it computes.
   uint4 kf[NT][FP8 ? KS / 2 : KS];
-  uint32_t vf[NT][4][VD];  // 16-bit cache: HDV / 8 bytes per token and lane; fp8 (width 128): 8 bytes
+  uint32_t vf[NT][4][VD];  // 16-bit cache: HDV / 8 bytes per token and lane; fp8: HDV / 16 bytes
   float ksc_tile = 1.f, vsc_tile = 1.f;  // fp8: scales of the chunk the staged K / V tile lies in
 
   // Addressing.  A tile of 16*NT tokens never straddles a chunk (the launcher picks NT so that the
@@ -671,15 +671,14 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
           acc[2 * dw + 1] =
               mfma_16x16x16<F16>(make_uint2(high_halves(r1, r0), high_halves(r3, r2)), pf[u], acc[2 * dw + 1]);
         }
-      } else {  // fp8, width 128: eight bytes per token per lane
-        uint2 w[4][2];  // [token j][half] -> two packed bf16 pairs (4 d values)
+      } else {  // fp8: four bytes (width 64) or eight (width 128) per token and lane
+        uint2 w[4][VD];  // [token j][dword] -> two packed bf16 pairs (4 d values)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          w[j][0] = fp8x4_to_bf16x4(vf[u][j][0]);
-          w[j][1] = fp8x4_to_bf16x4(vf[u][j][1]);
-        }
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
+          for (int hf = 0; hf < VD; ++hf) w[j][hf] = fp8x4_to_bf16x4(vf[u][j][hf]);
+#pragma unroll
+        for (int hf = 0; hf < VD; ++hf) {
           acc[4 * hf + 0] = mfma_16x16x16<F16>(
               make_uint2(low_halves(w[1][hf].x, w[0][hf].x), low_halves(w[3][hf].x, w[2][hf].x)), pf[u], acc[4 * hf + 0]);
           acc[4 * hf + 1] = mfma_16x16x16<F16>(
@@ -1733,8 +1732,8 @@ int mi::launch_paged_decode(
     return mi_fail(MI_ERR_SHAPE, "mi_paged_decode_attention: chunk size must be a positive multiple of 16");
   if (kv_dtype != MI_KV_BF16 && kv_dtype != MI_KV_FP8_E4M3)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: unknown kv_dtype");
-  if (kv_dtype == MI_KV_FP8_E4M3 && (head_dim != 128 || !k_scales || !v_scales))
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: fp8 KV needs head_dim 128 and both scale arrays");
+  if (kv_dtype == MI_KV_FP8_E4M3 && ((head_dim != 64 && head_dim != 128) || !k_scales || !v_scales))
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: fp8 KV needs head_dim 64 or 128 and both scale arrays");
   const int esz = kv_dtype == MI_KV_FP8_E4M3 ? 1 : 2;
   if (((uintptr_t)q | (uintptr_t)k_cache | (uintptr_t)v_cache | (uintptr_t)out) & 15)
     return mi_fail(MI_ERR_ALIGN, "mi_paged_decode_attention: q/k/v/out must be 16-byte aligned");
@@ -1856,6 +1855,7 @@ int mi::launch_paged_decode(
   else if (fused && head_dim == 192) MI_LAUNCH_STEP_WIDE(192, false);
   else if (fused && f16) MI_LAUNCH_STEP_WIDE(256, true);
   else if (fused) MI_LAUNCH_STEP_WIDE(256, false);
+  else if (kv_dtype == MI_KV_FP8_E4M3 && head_dim == 64) MI_LAUNCH_DECODE(64, true, false);
   else if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true, false);
   else if (head_dim == 128 && f16) MI_LAUNCH_DECODE(128, false, true);
   else if (head_dim == 128) MI_LAUNCH_DECODE(128, false, false);

@@ -327,9 +327,9 @@ template <int HD> constexpr int pp_tile() { return HD == 256 ? 32 : 64; }
 // caches of multi-latent attention, whose value cache has its own strides.
 template <bool STAGGER, bool FP8, bool SPLIT, int HD, int HDK, bool F16>
 __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams p) {
-  static_assert((HD == 128 && HDK == 128) || ((HD == 64 || HD == 96 || HD == 192 || HD == 256) && HDK == HD && !FP8) ||
-                    (HD == 128 && HDK == 192 && !FP8),
-                "head_dim 128, or 64 / 96 / 192 / 256 with a 16-bit cache, or 192 / 128 with 16-bit caches");
+  static_assert((HD == 128 && HDK == 128) || (HD == 64 && HDK == 64) ||
+                    ((HD == 96 || HD == 192 || HD == 256) && HDK == HD && !FP8) || (HD == 128 && HDK == 192 && !FP8),
+                "head_dim 64 or 128, or 96 / 192 / 256 with a 16-bit cache, or 192 / 128 with 16-bit caches");
   static_assert(!(FP8 && F16), "an fp8 cache is staged as bf16: bf16 queries only");
   constexpr bool MLA = HDK != HD;
   // Wide heads (192, 256): 16 rows per wavefront instead of 32 -- the accumulators of 32 rows (96 / 128 registers)
@@ -523,9 +523,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
       const uint8_t* tb = base + off;
       const uint32_t lim = (uint32_t)room + piece_off;
       if constexpr (FP8) {
-        const uint2 a = ld8(tb + min(row_off0, lim)), b = ld8(tb + min(row_off1, lim));
+        const uint2 a = ld8(tb + min(row_off0, lim));
         reg[0] = make_uint4(a.x, a.y, 0u, 0u);
-        reg[1] = make_uint4(b.x, b.y, 0u, 0u);
+        if constexpr (NPASS == 2) {
+          const uint2 b = ld8(tb + min(row_off1, lim));
+          reg[1] = make_uint4(b.x, b.y, 0u, 0u);
+        }
       } else {
         reg[0] = ld16(tb + min(row_off0, lim));
         if constexpr (NPASS == 2) reg[1] = ld16(tb + min(row_off1, lim));
@@ -1069,9 +1072,9 @@ static int launch_paged_prefill(
   // the two-phase tile kernel stages 64-key tiles that must not straddle chunks; other chunk sizes (and the knob)
   // select the register-only kernel
   const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0;
-  if (fp8 && (head_dim != 128 || !two_phase || f16))
+  if (fp8 && ((head_dim != 64 && head_dim != 128) || !two_phase || f16))
     return mi_fail(MI_ERR_UNSUPPORTED,
-                   "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 128, a chunk size that is a "
+                   "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 64 or 128, a chunk size that is a "
                    "multiple of 64 and the two-phase tile kernel");
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
   // (no limit on the number of requests: the decode part of a mixed batch runs in slices when it has to)
@@ -1126,6 +1129,7 @@ static int launch_paged_prefill(
     }
     // head_dim 128 over a 16-bit cache: the one-stream tile kernel when asked for
     if (!fp8 && head_dim == 128 && tune.prefill_two_phase == 3) launch_prefill_woven(p, lgrid, f16, st);
+    else if (fp8 && head_dim == 64) MI_PP_LAUNCH(true, 64, 64, false);
     else if (fp8) MI_PP_LAUNCH(true, 128, 128, false);
     else if (head_dim == 128 && f16) MI_PP_LAUNCH(false, 128, 128, true);
     else if (head_dim == 128) MI_PP_LAUNCH(false, 128, 128, false);

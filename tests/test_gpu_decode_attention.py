@@ -215,9 +215,11 @@ def test_long_context_split_merge(mi, dev):
     _close(out[:1], ref, 2e-2)
 
 
-def test_fp8_kv_cache(mi, dev):
-    """cfg5 shape at batch 6 / shorter contexts: quantiser is bit-exact, attention within 6e-2."""
-    cfg = mi.synthetic.DecodeConfig("fp8", 6, 32, 8, 128, 1024, 6000, fp8=True, seed=1005)
+@pytest.mark.parametrize("d", [128, 64])
+def test_fp8_kv_cache(mi, dev, d):
+    """cfg5 shape at batch 6 / shorter contexts (and the same at head_dim 64): quantiser is bit-exact, attention
+    within 6e-2."""
+    cfg = mi.synthetic.DecodeConfig("fp8", 6, 32, 8, d, 1024, 6000, fp8=True, seed=1005)
     case = mi.synthetic.make_decode_case(cfg, dev)
     N = case.k_cache.size(0)
     k8 = torch.empty(case.k_cache.shape, dtype=torch.uint8, device=dev)

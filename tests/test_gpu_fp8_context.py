@@ -47,9 +47,12 @@ def test_fp8_sizing_and_buffers(mi, dev):
         mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER = saved
 
 
+@pytest.mark.parametrize("head_dim", [128, 64])
 @pytest.mark.parametrize("entry", ["fused", "unfused", "mixed_qkv"])
-def test_fp8_prefill_then_decode_steps(mi, dev, entry):
-    saved = (mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER)
+def test_fp8_prefill_then_decode_steps(mi, dev, entry, head_dim):
+    global D
+    saved = (mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER, D)
+    D = head_dim   # (head_dim 64: decode steps take the separate launches, half-split pairs sit in other lanes there)
     try:
         ctx = _make_ctx(mi, dev)
         N = ctx.chunk_allocator.chunk_count_total
@@ -115,4 +118,4 @@ def test_fp8_prefill_then_decode_steps(mi, dev, entry):
             ctx.update_requests(mask, torch.randint(0, 100, (n_act,), generator=gen).to(dev))
         assert ctx.total_request_count == 4
     finally:
-        mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER = saved
+        mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER, D = saved

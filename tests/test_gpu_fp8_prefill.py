@@ -23,12 +23,13 @@ def _fp8_case(mi, dev, **kw):
     return q, k8, v8, ks, vs, cu_q, lens, bt
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("pingpong", [1, 2])
 @pytest.mark.parametrize("Hq,Hkv,chunk", [(32, 8, 64), (8, 1, 128), (32, 2, 256), (16, 16, 64)])
-def test_fp8_mixed_prefill_and_decode(mi, dev, Hq, Hkv, chunk, pingpong):
+def test_fp8_mixed_prefill_and_decode(mi, dev, Hq, Hkv, chunk, pingpong, d):
     q, k8, v8, ks, vs, cu_q, lens, bt = _fp8_case(
         mi, dev, n_prefill=3, new_tokens=150, ctx_lo=0, ctx_hi=400, n_decode=5, dec_lo=1, dec_hi=700,
-        Hq=Hq, Hkv=Hkv, d=128, chunk=chunk, seed=Hq + Hkv + chunk)
+        Hq=Hq, Hkv=Hkv, d=d, chunk=chunk, seed=Hq + Hkv + chunk)
     mi.ops.set_tuning("prefill_two_phase", pingpong)
     try:
         out = mi.ops.paged_prefill_attention(q, k8, v8, cu_q, lens, bt, max_kv_len=int(lens.max()),

@@ -67,7 +67,7 @@ def widen_table(bt, extra, fill):
 
 def case_decode(mi, dev, rng, seed, fp8):
     gen = torch.Generator().manual_seed(seed)
-    d = 128 if fp8 else rng.choice([64, 128, 64, 128, 96, 192, 256])
+    d = rng.choice([128, 128, 64]) if fp8 else rng.choice([64, 128, 64, 128, 96, 192, 256])
     Hkv = rng.choice([1, 2, 3, 4, 8, 16])
     G = rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 17, 24, 32] if Hkv <= 2 else [1, 2, 3, 4, 5, 7, 8, 16])
     Hq = Hkv * G
@@ -125,7 +125,7 @@ def case_decode(mi, dev, rng, seed, fp8):
 
 def case_prefill(mi, dev, rng, seed, fp8):
     gen = torch.Generator().manual_seed(seed)
-    d = rng.choice([64, 128, 64, 128, 96, 96, 192, 256]) if not fp8 else 128
+    d = rng.choice([64, 128, 64, 128, 96, 96, 192, 256]) if not fp8 else rng.choice([128, 128, 64])
     Hkv = rng.choice([1, 2, 4, 8])
     G = rng.choice([1, 2, 3, 4, 5, 7, 8, 12, 16, 20, 32] if Hkv <= 2 else [1, 2, 3, 4, 5, 7, 8, 12, 16])
     Hq = Hkv * G
