@@ -45,7 +45,7 @@ enum {
 };
 
 enum { MI_DTYPE_BF16 = 0, MI_DTYPE_FP16 = 1 };
-/* KV storage: the 16-bit type given by `dtype`, or fp8-e4m3 bytes with scales (needs MI_DTYPE_BF16). */
+/* KV storage: the 16-bit type given by `dtype`, or fp8-e4m3 bytes with scales (q / out in either 16-bit type). */
 enum { MI_KV_16BIT = 0, MI_KV_BF16 = 0, MI_KV_FP8_E4M3 = 1 };
 enum { MI_NORM_NONE = 0, MI_NORM_RMS = 1, MI_NORM_L2 = 2 };
 
@@ -132,18 +132,20 @@ int mi_kv_append_decode(const void* key, const void* value, int64_t src_stride_t
  * mi_kv_quantize_chunks_fp8: whole chunks, scale = amax(chunk-head tile) / 448.
  * mi_kv_append_decode_fp8  : one new token per request; a token that opens a chunk
  *   sets scale = headroom * amax(token) / 448, later tokens reuse it (saturating).
+ * `dtype` (MI_DTYPE_BF16 / MI_DTYPE_FP16) is the type of the source rows.
  */
-int mi_kv_quantize_chunks_fp8(const void* src_bf16, int64_t src_stride_chunk,
+int mi_kv_quantize_chunks_fp8(const void* src, int64_t src_stride_chunk,
                               int64_t src_stride_tok, void* dst_fp8, int64_t dst_stride_chunk,
                               int64_t dst_stride_tok, float* scales, int32_t n_chunks,
-                              int32_t chunk_tokens, int32_t Hkv, int32_t head_dim, void* stream);
+                              int32_t chunk_tokens, int32_t Hkv, int32_t head_dim, int32_t dtype,
+                              void* stream);
 
-int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_bf16, int64_t src_stride_tok,
+int mi_kv_append_decode_fp8(const void* key, const void* value, int64_t src_stride_tok,
                             void* k_cache_fp8, void* v_cache_fp8, int64_t kv_stride_chunk,
                             int64_t kv_stride_tok, float* k_scales, float* v_scales,
                             const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens,
                             int32_t R, int32_t chunk_tokens, int32_t Hkv, int32_t head_dim,
-                            float headroom, void* stream);
+                            float headroom, int32_t dtype, void* stream);
 
 /*
  * fp8 append with explicit per-token slots (prefill / mixed steps; no counterpart in the reference).
@@ -152,11 +154,12 @@ int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_bf16, int64_
  * A run that starts at local position 0 opens its chunk: scale = amax(run) / 448, times `headroom`
  * unless the run fills the chunk; any other run reuses the stored scale (saturating).
  */
-int mi_kv_append_fp8(const void* key_bf16, const void* value_bf16, int64_t src_stride_tok,
+int mi_kv_append_fp8(const void* key, const void* value, int64_t src_stride_tok,
                      void* k_cache_fp8, void* v_cache_fp8, int64_t kv_stride_chunk,
                      int64_t kv_stride_tok, float* k_scales, float* v_scales,
                      const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos, int32_t T,
-                     int32_t chunk_tokens, int32_t Hkv, int32_t head_dim, float headroom, void* stream);
+                     int32_t chunk_tokens, int32_t Hkv, int32_t head_dim, float headroom, int32_t dtype,
+                     void* stream);
 
 /*
  * Bytes of workspace mi_paged_decode_attention needs for these sizes on the current
@@ -233,8 +236,8 @@ int mi_decode_step_attention(const void* q, int64_t q_stride_tok, int64_t q_stri
  * sets that chunk-head's scale to headroom * amax(token) / 448 (1 for an all-zero row) and stores it, later tokens
  * reuse the stored scale and saturate -- and then streams the cache as mi_paged_decode_attention does with
  * kv_dtype MI_KV_FP8_E4M3.  Bytes and scales are those of mi_norm_rope_append (key_out) followed by
- * mi_kv_append_decode_fp8.  bf16 tensors, head_dim 128; half-split rotary pairs need rot_dim 128 (interleaved
- * pairs: any even width).
+ * mi_kv_append_decode_fp8.  Tensors of the 16-bit type `dtype`, head_dim 128; half-split rotary pairs need rot_dim 128
+ * (interleaved pairs: any even width).
  */
 int mi_decode_step_attention_fp8(const void* q, int64_t q_stride_tok, int64_t q_stride_group, const void* k_new,
                                  int64_t k_stride_tok, int64_t k_stride_head, const void* v_new,
@@ -248,7 +251,7 @@ int mi_decode_step_attention_fp8(const void* q, int64_t q_stride_tok, int64_t q_
                                  int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R,
                                  int32_t Hq, int32_t Hkv, int32_t head_dim, int32_t chunk_tokens,
                                  int32_t split_tokens, float softmax_scale, int32_t faithful_rounding,
-                                 const MiTuning* tuning, void* stream);
+                                 int32_t dtype, const MiTuning* tuning, void* stream);
 
 /*
  * mi_paged_decode_attention for callers that cannot allocate device memory: code under HIP graph
@@ -333,7 +336,7 @@ int mi_paged_prefill_attention(const void* q, int64_t q_stride_tok, int64_t q_st
  * The same call over an fp8-e4m3 cache (byte caches `[n_chunks, chunk_tokens, Hkv, d]`, strides in
  * elements = bytes, fp32 scales `[n_chunks, Hkv]`; no counterpart in the reference).  Tiles are
  * multiplied by their chunk's scale and rounded to bf16 on their way into LDS.  Needs head_dim 64
- * or 128, bf16 queries and a chunk size that is a multiple of 64.
+ * or 128 and a chunk size that is a multiple of 64; `dtype` is the type of q / out (and of the staged tiles).
  */
 int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t q_stride_head,
                                    const void* k_cache_fp8, const void* v_cache_fp8,
@@ -345,7 +348,8 @@ int mi_paged_prefill_attention_fp8(const void* q, int64_t q_stride_tok, int64_t 
                                    int64_t o_stride_head, void* workspace, int64_t workspace_bytes,
                                    int32_t T, int32_t R, int32_t Hq, int32_t Hkv, int32_t head_dim,
                                    int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
-                                   float softmax_scale, const MiTuning* tuning, void* stream);
+                                   float softmax_scale, int32_t dtype, const MiTuning* tuning,
+                                   void* stream);
 
 /*
  * Paged varlen causal attention with keys wider than values: the prefill / mixed step of

@@ -37,11 +37,11 @@ SIGNATURES = {
     "mi_kv_append_decode": (
         c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _I64, _P, _I32, _I32, _I32, _I32, _P]),
     "mi_kv_quantize_chunks_fp8": (
-        c_int, [_P, _I64, _I64, _P, _I64, _I64, _P, _I32, _I32, _I32, _I32, _P]),
+        c_int, [_P, _I64, _I64, _P, _I64, _I64, _P, _I32, _I32, _I32, _I32, _I32, _P]),
     "mi_kv_append_decode_fp8": (
-        c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _F, _P]),
+        c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _I64, _P, _I32, _I32, _I32, _I32, _F, _I32, _P]),
     "mi_kv_append_fp8": (
-        c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _F, _P]),
+        c_int, [_P, _P, _I64, _P, _P, _I64, _I64, _P, _P, _P, _P, _I32, _I32, _I32, _I32, _F, _I32, _P]),
     "mi_decode_workspace_bytes": (_I64, [_I32, _I32, _I32, _I32, _I32, _I32, _I32, _P]),
     "mi_paged_decode_attention": (
         c_int,
@@ -56,7 +56,7 @@ SIGNATURES = {
         c_int,
         [_P, _I64, _I64, _P, _I64, _I64, _P, _I64, _I64, _P, _P, _F, _I32, _P, _I64, _I32, _I32, _F, _P, _P, _P,
          _I64, _I64, _I64, _P, _P, _F, _P, _I64, _P, _P, _I64, _I64, _P, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _F,
-         _I32, _P, _P]),
+         _I32, _I32, _P, _P]),
     "mi_paged_decode_attention_noalloc": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _I64, _I64,
@@ -73,7 +73,7 @@ SIGNATURES = {
     "mi_paged_prefill_attention_fp8": (
         c_int,
         [_P, _I64, _I64, _P, _P, _I64, _I64, _I64, _P, _P, _P, _I64, _P, _P, _P, _I64, _I64, _P, _I64,
-         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _P, _P]),
+         _I32, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F, _I32, _P, _P]),
     "mi_paged_prefill_attention_mla": (
         c_int,
         [_P, _I64, _I64, _P, _I64, _I64, _I64, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _I64, _I64,

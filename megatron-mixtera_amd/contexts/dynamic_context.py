@@ -144,8 +144,8 @@ class DynamicInferenceContext:
         if kv_cache_dtype in (None, params_dtype):
             self.kv_cache_fp8 = False
         elif kv_cache_dtype in ("fp8", "fp8_e4m3", "float8_e4m3fn", torch.float8_e4m3fn):
-            if params_dtype != torch.bfloat16:
-                raise ValueError("the fp8 KV cache quantises bf16 keys and values: params_dtype must be bfloat16")
+            if params_dtype not in (torch.bfloat16, torch.float16):
+                raise ValueError("the fp8 KV cache quantises 16-bit keys and values: params_dtype must be bfloat16 or float16")
             self.kv_cache_fp8 = True
         else:
             raise ValueError(f"unsupported kv_cache_dtype {kv_cache_dtype!r} (None or 'fp8_e4m3')")

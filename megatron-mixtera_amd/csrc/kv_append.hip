@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void kv_append_kernel(AppendParams p) {
 }
 
 struct QuantParams {
-  const uint16_t* src;   // bf16 rows
+  const uint16_t* src;   // rows in the 16-bit type the kernel is instantiated for
   int64_t src_stride;    // elements between tokens (bulk: between chunk tokens)
   int64_t src_chunk;     // bulk: elements between chunks
   uint8_t* dst;          // fp8 cache
@@ -77,6 +77,7 @@ struct QuantParams {
 // One workgroup (256 threads) per (chunk, KV head): amax over the whole
 // chunk-head tile, scale = amax / 448, then quantise.  Used to fill an fp8 cache
 // from bf16 chunks (prefill-style writes and benchmark set-up).
+template <bool F16>
 __global__ __launch_bounds__(256) void quantize_chunks_fp8_kernel(QuantParams p) {
   const int c = blockIdx.x, h = blockIdx.y;
   const uint16_t* src = p.src + (int64_t)c * p.src_chunk + (int64_t)h * p.d;
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) void quantize_chunks_fp8_kernel(QuantParams p)
   float amax = 0.f;
   for (int i = threadIdx.x; i < n; i += 256) {
     const int tok = i / p.d, e = i - tok * p.d;
-    amax = fmaxf(amax, fabsf(bf16_to_f32(src[(int64_t)tok * p.src_stride + e])));
+    amax = fmaxf(amax, fabsf(to_f32<F16>(src[(int64_t)tok * p.src_stride + e])));
   }
   __shared__ float red[256];
   red[threadIdx.x] = amax;
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(256) void quantize_chunks_fp8_kernel(QuantParams p)
   uint8_t* dst = p.dst + (int64_t)c * p.chunk_bytes + (int64_t)h * p.d;
   for (int i = threadIdx.x; i < n; i += 256) {
     const int tok = i / p.d, e = i - tok * p.d;
-    const float v = bf16_to_f32(src[(int64_t)tok * p.src_stride + e]) / scale;
+    const float v = to_f32<F16>(src[(int64_t)tok * p.src_stride + e]) / scale;
     dst[(int64_t)tok * p.tok_bytes + e] = (uint8_t)f32_to_e4m3_sat(v);
   }
 }
@@ -107,6 +108,7 @@ __global__ __launch_bounds__(256) void quantize_chunks_fp8_kernel(QuantParams p)
 // One workgroup per (request, KV head): quantise the newly generated token.
 // A token that opens a chunk (local position 0) fixes that chunk-head's scale to
 // headroom * amax(token) / 448; later tokens reuse the stored scale and saturate.
+template <bool F16>
 __global__ __launch_bounds__(64) void kv_append_decode_fp8_kernel(QuantParams p) {
   const int r = blockIdx.x, h = blockIdx.y;
   const int len = p.lens[r];
@@ -119,7 +121,7 @@ __global__ __launch_bounds__(64) void kv_append_decode_fp8_kernel(QuantParams p)
   float scale;
   if (l == 0) {
     float amax = 0.f;
-    for (int e = threadIdx.x; e < p.d; e += 64) amax = fmaxf(amax, fabsf(bf16_to_f32(src[e])));
+    for (int e = threadIdx.x; e < p.d; e += 64) amax = fmaxf(amax, fabsf(to_f32<F16>(src[e])));
     for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
     scale = amax > 0.f ? p.headroom * amax / 448.f : 1.f;
     if (threadIdx.x == 0) p.scale[c * p.Hkv + h] = scale;
@@ -127,7 +129,7 @@ __global__ __launch_bounds__(64) void kv_append_decode_fp8_kernel(QuantParams p)
     scale = p.scale[c * p.Hkv + h];
   }
   uint8_t* dst = p.dst + c * p.chunk_bytes + (int64_t)l * p.tok_bytes + (int64_t)h * p.d;
-  for (int e = threadIdx.x; e < p.d; e += 64) dst[e] = (uint8_t)f32_to_e4m3_sat(bf16_to_f32(src[e]) / scale);
+  for (int e = threadIdx.x; e < p.d; e += 64) dst[e] = (uint8_t)f32_to_e4m3_sat(to_f32<F16>(src[e]) / scale);
 }
 
 // ---- fp8 append of many tokens per request (prefill / mixed steps) ----------------------------
@@ -138,7 +140,7 @@ __global__ __launch_bounds__(64) void kv_append_decode_fp8_kernel(QuantParams p)
 // fills the chunk (later tokens of a partly filled chunk reuse the scale and saturate).  A run that
 // starts further in reuses the stored scale.
 struct AppendFp8Params {
-  const uint16_t* src[2];   // key, value rows (bf16)
+  const uint16_t* src[2];   // key, value rows (16-bit)
   int64_t src_stride;       // elements between tokens
   uint8_t* dst[2];          // fp8 caches
   int64_t chunk_bytes, tok_bytes;
@@ -152,6 +154,7 @@ struct AppendFp8Params {
 // grid = (ceil(T / 64), Hkv, 2): a workgroup looks at 64 tokens and, for each of them that opens a
 // chunk (local position 0), computes the scale of (chunk, head) of the key (z = 0) or value (z = 1)
 // cache from the whole run that starts there.
+template <bool F16>
 __global__ __launch_bounds__(256) void kv_append_fp8_scales_kernel(AppendFp8Params p) {
   const int t0 = blockIdx.x * 64, h = blockIdx.y, kv = blockIdx.z;
   __shared__ int open_s[64];
@@ -196,12 +199,12 @@ __global__ __launch_bounds__(256) void kv_append_fp8_scales_kernel(AppendFp8Para
         const uint32_t u[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-          amax = fmaxf(amax, fmaxf(fabsf(bf16lo_to_f32(u[j])), fabsf(bf16hi_to_f32(u[j]))));
+          amax = fmaxf(amax, fmaxf(fabsf(lo_to_f32<F16>(u[j])), fabsf(hi_to_f32<F16>(u[j]))));
       }
     } else {
       for (int i = threadIdx.x; i < n * p.d; i += 256) {
         const int tok = i / p.d, e = i - tok * p.d;
-        amax = fmaxf(amax, fabsf(bf16_to_f32(src[(int64_t)tok * p.src_stride + e])));
+        amax = fmaxf(amax, fabsf(to_f32<F16>(src[(int64_t)tok * p.src_stride + e])));
       }
     }
     red[threadIdx.x] = amax;
@@ -218,6 +221,7 @@ __global__ __launch_bounds__(256) void kv_append_fp8_scales_kernel(AppendFp8Para
 }
 
 // grid = (T, 2): quantise the key (y = 0) or value (y = 1) row of one token with its chunk's scales.
+template <bool F16>
 __global__ __launch_bounds__(256) void kv_append_fp8_rows_kernel(AppendFp8Params p) {
   const int t = blockIdx.x, kv = blockIdx.y;
   const int64_t c = p.tok_chunk[t], l = p.tok_local[t];
@@ -235,14 +239,14 @@ __global__ __launch_bounds__(256) void kv_append_fp8_rows_kernel(AppendFp8Params
       uint32_t out[2] = {0u, 0u};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const uint32_t lo = f32_to_e4m3_sat(bf16lo_to_f32(u[j]) / scale), hi = f32_to_e4m3_sat(bf16hi_to_f32(u[j]) / scale);
+        const uint32_t lo = f32_to_e4m3_sat(lo_to_f32<F16>(u[j]) / scale), hi = f32_to_e4m3_sat(hi_to_f32<F16>(u[j]) / scale);
         out[j >> 1] |= (lo | (hi << 8)) << (16 * (j & 1));
       }
       st8(dst + e, make_uint2(out[0], out[1]));
     }
   } else {
     for (int e = threadIdx.x; e < row; e += 256)
-      dst[e] = (uint8_t)f32_to_e4m3_sat(bf16_to_f32(src[e]) / scales[e / p.d]);
+      dst[e] = (uint8_t)f32_to_e4m3_sat(to_f32<F16>(src[e]) / scales[e / p.d]);
   }
 }
 
@@ -308,32 +312,37 @@ extern "C" int mi_kv_append_decode(const void* key, const void* value, int64_t s
   return mi_check_launch("mi_kv_append_decode");
 }
 
-extern "C" int mi_kv_quantize_chunks_fp8(const void* src_bf16, int64_t src_stride_chunk,
+extern "C" int mi_kv_quantize_chunks_fp8(const void* src, int64_t src_stride_chunk,
                                          int64_t src_stride_tok, void* dst_fp8,
                                          int64_t dst_stride_chunk, int64_t dst_stride_tok,
                                          float* scales, int32_t n_chunks, int32_t chunk_tokens,
-                                         int32_t Hkv, int32_t head_dim, void* stream) {
+                                         int32_t Hkv, int32_t head_dim, int32_t dtype, void* stream) {
   if (n_chunks == 0) return MI_OK;
-  if (!src_bf16 || !dst_fp8 || !scales) return mi_fail(MI_ERR_NULL, "mi_kv_quantize_chunks_fp8: null pointer argument");
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_kv_quantize_chunks_fp8: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  if (!src || !dst_fp8 || !scales) return mi_fail(MI_ERR_NULL, "mi_kv_quantize_chunks_fp8: null pointer argument");
   if (n_chunks < 0 || chunk_tokens <= 0 || Hkv <= 0 || head_dim <= 0 || Hkv > 65535)
     return mi_fail(MI_ERR_SHAPE, "mi_kv_quantize_chunks_fp8: bad sizes");
   QuantParams p = {};
-  p.src = (const uint16_t*)src_bf16; p.src_chunk = src_stride_chunk; p.src_stride = src_stride_tok;
+  p.src = (const uint16_t*)src; p.src_chunk = src_stride_chunk; p.src_stride = src_stride_tok;
   p.dst = (uint8_t*)dst_fp8; p.chunk_bytes = dst_stride_chunk; p.tok_bytes = dst_stride_tok;
   p.scale = scales; p.chunk = chunk_tokens; p.Hkv = Hkv; p.d = head_dim; p.headroom = 1.f;
-  hipLaunchKernelGGL(quantize_chunks_fp8_kernel, dim3(n_chunks, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+  if (dtype == MI_DTYPE_FP16) hipLaunchKernelGGL(quantize_chunks_fp8_kernel<true>, dim3(n_chunks, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+  else hipLaunchKernelGGL(quantize_chunks_fp8_kernel<false>, dim3(n_chunks, Hkv), dim3(256), 0, (hipStream_t)stream, p);
   return mi_check_launch("mi_kv_quantize_chunks_fp8");
 }
 
-extern "C" int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_bf16,
+extern "C" int mi_kv_append_decode_fp8(const void* key, const void* value,
                                        int64_t src_stride_tok, void* k_cache_fp8, void* v_cache_fp8,
                                        int64_t kv_stride_chunk, int64_t kv_stride_tok,
                                        float* k_scales, float* v_scales, const int32_t* block_table,
                                        int64_t bt_stride, const int32_t* kv_lens, int32_t R,
                                        int32_t chunk_tokens, int32_t Hkv, int32_t head_dim,
-                                       float headroom, void* stream) {
+                                       float headroom, int32_t dtype, void* stream) {
   if (R == 0) return MI_OK;
-  if (!key_bf16 || !value_bf16 || !k_cache_fp8 || !v_cache_fp8 || !k_scales || !v_scales || !block_table || !kv_lens)
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_kv_append_decode_fp8: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  if (!key || !value || !k_cache_fp8 || !v_cache_fp8 || !k_scales || !v_scales || !block_table || !kv_lens)
     return mi_fail(MI_ERR_NULL, "mi_kv_append_decode_fp8: null pointer argument");
   if (R < 0 || chunk_tokens <= 0 || Hkv <= 0 || head_dim <= 0 || Hkv > 65535 || !(headroom > 0.f))
     return mi_fail(MI_ERR_SHAPE, "mi_kv_append_decode_fp8: bad sizes");
@@ -341,35 +350,43 @@ extern "C" int mi_kv_append_decode_fp8(const void* key_bf16, const void* value_b
   p.src_stride = src_stride_tok; p.chunk_bytes = kv_stride_chunk; p.tok_bytes = kv_stride_tok;
   p.bt = block_table; p.bt_stride = bt_stride; p.lens = kv_lens;
   p.chunk = chunk_tokens; p.Hkv = Hkv; p.d = head_dim; p.headroom = headroom;
-  p.src = (const uint16_t*)key_bf16; p.dst = (uint8_t*)k_cache_fp8; p.scale = k_scales;
-  hipLaunchKernelGGL(kv_append_decode_fp8_kernel, dim3(R, Hkv), dim3(64), 0, (hipStream_t)stream, p);
-  p.src = (const uint16_t*)value_bf16; p.dst = (uint8_t*)v_cache_fp8; p.scale = v_scales;
-  hipLaunchKernelGGL(kv_append_decode_fp8_kernel, dim3(R, Hkv), dim3(64), 0, (hipStream_t)stream, p);
+  const auto kernel = dtype == MI_DTYPE_FP16 ? kv_append_decode_fp8_kernel<true> : kv_append_decode_fp8_kernel<false>;
+  p.src = (const uint16_t*)key; p.dst = (uint8_t*)k_cache_fp8; p.scale = k_scales;
+  hipLaunchKernelGGL(kernel, dim3(R, Hkv), dim3(64), 0, (hipStream_t)stream, p);
+  p.src = (const uint16_t*)value; p.dst = (uint8_t*)v_cache_fp8; p.scale = v_scales;
+  hipLaunchKernelGGL(kernel, dim3(R, Hkv), dim3(64), 0, (hipStream_t)stream, p);
   return mi_check_launch("mi_kv_append_decode_fp8");
 }
 
-extern "C" int mi_kv_append_fp8(const void* key_bf16, const void* value_bf16, int64_t src_stride_tok,
+extern "C" int mi_kv_append_fp8(const void* key, const void* value, int64_t src_stride_tok,
                                 void* k_cache_fp8, void* v_cache_fp8, int64_t kv_stride_chunk,
                                 int64_t kv_stride_tok, float* k_scales, float* v_scales,
                                 const int64_t* token_to_chunk_idx, const int64_t* token_to_local_pos,
                                 int32_t T, int32_t chunk_tokens, int32_t Hkv, int32_t head_dim,
-                                float headroom, void* stream) {
+                                float headroom, int32_t dtype, void* stream) {
   if (T == 0) return MI_OK;
-  if (!key_bf16 || !value_bf16 || !k_cache_fp8 || !v_cache_fp8 || !k_scales || !v_scales || !token_to_chunk_idx ||
+  if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
+    return mi_fail(MI_ERR_UNSUPPORTED, "mi_kv_append_fp8: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
+  if (!key || !value || !k_cache_fp8 || !v_cache_fp8 || !k_scales || !v_scales || !token_to_chunk_idx ||
       !token_to_local_pos)
     return mi_fail(MI_ERR_NULL, "mi_kv_append_fp8: null pointer argument");
   if (T < 0 || chunk_tokens <= 0 || Hkv <= 0 || head_dim <= 0 || Hkv > 65535 || !(headroom > 0.f) ||
       src_stride_tok < (int64_t)Hkv * head_dim || kv_stride_tok < (int64_t)Hkv * head_dim)
     return mi_fail(MI_ERR_SHAPE, "mi_kv_append_fp8: bad sizes or strides");
   AppendFp8Params p = {};
-  p.src[0] = (const uint16_t*)key_bf16; p.src[1] = (const uint16_t*)value_bf16; p.src_stride = src_stride_tok;
+  p.src[0] = (const uint16_t*)key; p.src[1] = (const uint16_t*)value; p.src_stride = src_stride_tok;
   p.dst[0] = (uint8_t*)k_cache_fp8; p.dst[1] = (uint8_t*)v_cache_fp8;
   p.chunk_bytes = kv_stride_chunk; p.tok_bytes = kv_stride_tok;
   p.scale[0] = k_scales; p.scale[1] = v_scales;
   p.tok_chunk = token_to_chunk_idx; p.tok_local = token_to_local_pos;
   p.T = T; p.chunk = chunk_tokens; p.Hkv = Hkv; p.d = head_dim; p.headroom = headroom;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(kv_append_fp8_scales_kernel, dim3((T + 63) / 64, Hkv, 2), dim3(256), 0, st, p);
-  hipLaunchKernelGGL(kv_append_fp8_rows_kernel, dim3(T, 2), dim3(256), 0, st, p);
+  if (dtype == MI_DTYPE_FP16) {
+    hipLaunchKernelGGL(kv_append_fp8_scales_kernel<true>, dim3((T + 63) / 64, Hkv, 2), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(kv_append_fp8_rows_kernel<true>, dim3(T, 2), dim3(256), 0, st, p);
+  } else {
+    hipLaunchKernelGGL(kv_append_fp8_scales_kernel<false>, dim3((T + 63) / 64, Hkv, 2), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(kv_append_fp8_rows_kernel<false>, dim3(T, 2), dim3(256), 0, st, p);
+  }
   return mi_check_launch("mi_kv_append_fp8");
 }

@@ -302,6 +302,20 @@ static __device__ __forceinline__ uint2 fp8x4_to_bf16x4(uint32_t w) {
   return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
 }
 
+// The same into the operand type of the kernel: bf16 pairs, or fp16 pairs (exact as well: e4m3 has 3 mantissa bits
+// and its exponents lie inside fp16's).
+template <bool F16>
+static __device__ __forceinline__ uint2 fp8x4_to_16x4(uint32_t w) {
+  if constexpr (F16) {
+    typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+    const f16x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+    const f16x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+    return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+  } else {
+    return fp8x4_to_bf16x4(w);
+  }
+}
+
 // fp32 -> e4m3fn byte, round to nearest even, saturating (no NaN / inf produced).
 static __device__ __forceinline__ uint32_t f32_to_e4m3_sat(float x) {
   x = fminf(fmaxf(x, -448.f), 448.f);

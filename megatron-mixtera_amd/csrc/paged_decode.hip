@@ -121,7 +121,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
   constexpr int DV = HDV / 16;
   constexpr int VD = FP8 ? DV / 4 : DV / 2;  // dwords per token and lane of the value operand
   static_assert(HDK % 32 == 0 && HDV % 32 == 0 && HDK >= 64 && HDV >= 64, "head widths: multiples of 32");
-  static_assert(!FP8 || (HDK == HDV && (HDK == 64 || HDK == 128) && !F16), "fp8 KV: head_dim 64 or 128, bf16 queries");
+  static_assert(!FP8 || (HDK == HDV && (HDK == 64 || HDK == 128)), "fp8 KV: head_dim 64 or 128");
   static_assert(!FUSED || (HDK == HDV && HDK <= 256), "fused step: an ordinary per-head cache");
   constexpr int ESZ = FP8 ? 1 : 2;
   // Everything that describes the segment is wave-uniform; as scalars, the chunk lookup and the
@@ -288,8 +288,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
         float kq[EPL], vq[EPL];
 #pragma unroll
         for (int w = 0; w < EPL; ++w) {
-          kq[w] = on ? bf16_to_f32(f32_to_bf16(o[w])) : 0.f;
-          vq[w] = on ? bf16_to_f32(vsrc[i + w * LPV]) : 0.f;
+          kq[w] = on ? to_f32<F16>(f32_to_16<F16>(o[w])) : 0.f;
+          vq[w] = on ? to_f32<F16>(vsrc[i + w * LPV]) : 0.f;
         }
         float ksc, vsc;
         if (opens) {
@@ -604,8 +604,8 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
       if (FP8) {
 #pragma unroll
         for (int kk = 0; kk < KS / 2; ++kk) {
-          const uint2 a0 = fp8x4_to_bf16x4(kf[u][kk].x), a1 = fp8x4_to_bf16x4(kf[u][kk].y);
-          const uint2 b0 = fp8x4_to_bf16x4(kf[u][kk].z), b1 = fp8x4_to_bf16x4(kf[u][kk].w);
+          const uint2 a0 = fp8x4_to_16x4<F16>(kf[u][kk].x), a1 = fp8x4_to_16x4<F16>(kf[u][kk].y);
+          const uint2 b0 = fp8x4_to_16x4<F16>(kf[u][kk].z), b1 = fp8x4_to_16x4<F16>(kf[u][kk].w);
           sacc = mfma_16x16x32<F16>(make_uint4(a0.x, a0.y, a1.x, a1.y), qf[2 * kk], sacc);
           sacc = mfma_16x16x32<F16>(make_uint4(b0.x, b0.y, b1.x, b1.y), qf[2 * kk + 1], sacc);
         }
@@ -676,7 +676,7 @@ static __device__ __forceinline__ void decode_segment(const DecodeParams& p, int
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int hf = 0; hf < VD; ++hf) w[j][hf] = fp8x4_to_bf16x4(vf[u][j][hf]);
+          for (int hf = 0; hf < VD; ++hf) w[j][hf] = fp8x4_to_16x4<F16>(vf[u][j][hf]);
 #pragma unroll
         for (int hf = 0; hf < VD; ++hf) {
           acc[4 * hf + 0] = mfma_16x16x16<F16>(
@@ -1718,8 +1718,6 @@ int mi::launch_paged_decode(
   if (dtype != MI_DTYPE_BF16 && dtype != MI_DTYPE_FP16)
     return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: dtype must be MI_DTYPE_BF16 or MI_DTYPE_FP16");
   const bool f16 = dtype == MI_DTYPE_FP16;
-  if (f16 && kv_dtype == MI_KV_FP8_E4M3)
-    return mi_fail(MI_ERR_UNSUPPORTED, "mi_paged_decode_attention: an fp8 cache needs bf16 queries");
   if (!q || !k_cache || !v_cache || !block_table || !kv_lens || !out)
     return mi_fail(MI_ERR_NULL, "mi_paged_decode_attention: null pointer argument");
   if (R < 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv)
@@ -1843,7 +1841,9 @@ int mi::launch_paged_decode(
   } while (0)
 #define MI_LAUNCH_STEP(HD_, F16_) hipLaunchKernelGGL((decode_step_stream_kernel<HD_, 1, F16_>), grid, block, lds, st, p)
 #define MI_LAUNCH_STEP_WIDE(HD_, F16_) hipLaunchKernelGGL((decode_step_stream_kernel<HD_, 1, F16_, 2>), grid, block, lds, st, p)
-  if (fused && kv_dtype == MI_KV_FP8_E4M3)
+  if (fused && kv_dtype == MI_KV_FP8_E4M3 && f16)
+    hipLaunchKernelGGL((decode_step_stream_kernel<128, MI_FUSED_FP8_NT, true, 3, true>), grid, block, lds, st, p);
+  else if (fused && kv_dtype == MI_KV_FP8_E4M3)
     hipLaunchKernelGGL((decode_step_stream_kernel<128, MI_FUSED_FP8_NT, false, 3, true>), grid, block, lds, st, p);
   else if (fused && head_dim == 128 && f16) MI_LAUNCH_STEP(128, true);
   else if (fused && head_dim == 128) MI_LAUNCH_STEP(128, false);
@@ -1855,7 +1855,9 @@ int mi::launch_paged_decode(
   else if (fused && head_dim == 192) MI_LAUNCH_STEP_WIDE(192, false);
   else if (fused && f16) MI_LAUNCH_STEP_WIDE(256, true);
   else if (fused) MI_LAUNCH_STEP_WIDE(256, false);
+  else if (kv_dtype == MI_KV_FP8_E4M3 && head_dim == 64 && f16) MI_LAUNCH_DECODE(64, true, true);
   else if (kv_dtype == MI_KV_FP8_E4M3 && head_dim == 64) MI_LAUNCH_DECODE(64, true, false);
+  else if (kv_dtype == MI_KV_FP8_E4M3 && f16) MI_LAUNCH_DECODE(128, true, true);
   else if (kv_dtype == MI_KV_FP8_E4M3) MI_LAUNCH_DECODE(128, true, false);
   else if (head_dim == 128 && f16) MI_LAUNCH_DECODE(128, false, true);
   else if (head_dim == 128) MI_LAUNCH_DECODE(128, false, false);
@@ -1930,8 +1932,8 @@ static int decode_step_entry(
     if (fp8 && !rotary_interleaved && (rot_dim / 2) % 64)
       return fail(MI_ERR_UNSUPPORTED, "over an fp8 cache half-split rotary pairs need rot_dim / 2 to be a multiple of 64 (else: the separate calls)");
   }
-  if (fp8 && (head_dim != 128 || dtype != MI_DTYPE_BF16 || !k_scales || !v_scales || !(headroom > 0.f)))
-    return fail(MI_ERR_UNSUPPORTED, "an fp8 cache needs head_dim 128, bf16 tensors, both scale arrays and a positive headroom");
+  if (fp8 && (head_dim != 128 || !k_scales || !v_scales || !(headroom > 0.f)))
+    return fail(MI_ERR_UNSUPPORTED, "an fp8 cache needs head_dim 128, both scale arrays and a positive headroom");
   const int G = Hq / Hkv;
   if (q_stride_group < (int64_t)G * head_dim) return fail(MI_ERR_SHAPE, "query group stride smaller than (Hq / Hkv) * head_dim");
   if ((((uintptr_t)q | (uintptr_t)q_weight) & 15) || (q_stride_tok | q_stride_group) % 8)
@@ -1982,13 +1984,13 @@ extern "C" int mi_decode_step_attention_fp8(
     float* v_scales, float headroom, const int32_t* block_table, int64_t bt_stride, const int32_t* kv_lens, void* out,
     int64_t o_stride_tok, int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t R, int32_t Hq,
     int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t split_tokens, float softmax_scale,
-    int32_t faithful_rounding, const MiTuning* tuning, void* stream) {
+    int32_t faithful_rounding, int32_t dtype, const MiTuning* tuning, void* stream) {
   return decode_step_entry("mi_decode_step_attention_fp8", q, q_stride_tok, q_stride_group, k_new, k_stride_tok,
                            k_stride_head, v_new, v_stride_tok, v_stride_head, q_weight, k_weight, eps, norm_kind,
                            rotary_angles, angles_stride, rot_dim, rotary_interleaved, mscale, positions, k_cache_fp8,
                            v_cache_fp8, kv_stride_chunk, kv_stride_tok, kv_stride_head, block_table, bt_stride, kv_lens, out,
                            o_stride_tok, o_stride_head, workspace, workspace_bytes, R, Hq, Hkv, head_dim, chunk_tokens,
-                           split_tokens, softmax_scale, faithful_rounding, MI_DTYPE_BF16, tuning, stream, MI_KV_FP8_E4M3,
+                           split_tokens, softmax_scale, faithful_rounding, dtype, tuning, stream, MI_KV_FP8_E4M3,
                            k_scales, v_scales, headroom);
 }
 

@@ -330,7 +330,6 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_pp_kernel(PrefillParams 
   static_assert((HD == 128 && HDK == 128) || (HD == 64 && HDK == 64) ||
                     ((HD == 96 || HD == 192 || HD == 256) && HDK == HD && !FP8) || (HD == 128 && HDK == 192 && !FP8),
                 "head_dim 64 or 128, or 96 / 192 / 256 with a 16-bit cache, or 192 / 128 with 16-bit caches");
-  static_assert(!(FP8 && F16), "an fp8 cache is staged as bf16: bf16 queries only");
   constexpr bool MLA = HDK != HD;
   // Wide heads (192, 256): 16 rows per wavefront instead of 32 -- the accumulators of 32 rows (96 / 128 registers)
   // plus query fragments (48 / 64) leave no room for the operand fragments in a wavefront's 256 registers.
@@ -1072,9 +1071,9 @@ static int launch_paged_prefill(
   // the two-phase tile kernel stages 64-key tiles that must not straddle chunks; other chunk sizes (and the knob)
   // select the register-only kernel
   const bool two_phase = tune.prefill_two_phase > 0 && chunk_tokens % 64 == 0;
-  if (fp8 && ((head_dim != 64 && head_dim != 128) || !two_phase || f16))
+  if (fp8 && ((head_dim != 64 && head_dim != 128) || !two_phase))
     return mi_fail(MI_ERR_UNSUPPORTED,
-                   "mi_paged_prefill_attention_fp8: fp8 KV needs bf16 queries, head_dim 64 or 128, a chunk size that is a "
+                   "mi_paged_prefill_attention_fp8: fp8 KV needs head_dim 64 or 128, a chunk size that is a "
                    "multiple of 64 and the two-phase tile kernel");
   if (!(softmax_scale > 0.f)) return mi_fail(MI_ERR_SHAPE, "mi_paged_prefill_attention: softmax_scale must be positive");
   // (no limit on the number of requests: the decode part of a mixed batch runs in slices when it has to)
@@ -1129,7 +1128,9 @@ static int launch_paged_prefill(
     }
     // head_dim 128 over a 16-bit cache: the one-stream tile kernel when asked for
     if (!fp8 && head_dim == 128 && tune.prefill_two_phase == 3) launch_prefill_woven(p, lgrid, f16, st);
+    else if (fp8 && head_dim == 64 && f16) MI_PP_LAUNCH(true, 64, 64, true);
     else if (fp8 && head_dim == 64) MI_PP_LAUNCH(true, 64, 64, false);
+    else if (fp8 && f16) MI_PP_LAUNCH(true, 128, 128, true);
     else if (fp8) MI_PP_LAUNCH(true, 128, 128, false);
     else if (head_dim == 128 && f16) MI_PP_LAUNCH(false, 128, 128, true);
     else if (head_dim == 128) MI_PP_LAUNCH(false, 128, 128, false);
@@ -1207,12 +1208,12 @@ extern "C" int mi_paged_prefill_attention_fp8(
     const int32_t* cu_seqlens_q, const int32_t* kv_lens, void* out, int64_t o_stride_tok,
     int64_t o_stride_head, void* workspace, int64_t workspace_bytes, int32_t T, int32_t R, int32_t Hq,
     int32_t Hkv, int32_t head_dim, int32_t chunk_tokens, int32_t max_kv_len, int32_t split_tokens,
-    float softmax_scale, const MiTuning* tuning, void* stream) {
+    float softmax_scale, int32_t dtype, const MiTuning* tuning, void* stream) {
   return launch_paged_prefill(q, q_stride_tok, q_stride_head, k_cache_fp8, v_cache_fp8, kv_stride_chunk,
                               kv_stride_tok, kv_stride_head, block_table, bt_stride, cu_seqlens_q, kv_lens, out,
                               o_stride_tok, o_stride_head, workspace, workspace_bytes, T, R, Hq, Hkv, head_dim,
                               chunk_tokens, max_kv_len, split_tokens, softmax_scale, MI_KV_FP8_E4M3, k_scales, v_scales,
-                              MI_DTYPE_BF16, tuning, stream);
+                              dtype, tuning, stream);
 }
 
 extern "C" int mi_paged_prefill_attention_mla(

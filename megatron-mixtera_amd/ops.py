@@ -225,10 +225,10 @@ def kv_append_decode(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tenso
 # fp8 KV storage
 # ---------------------------------------------------------------------------------------------
 def quantize_chunks_fp8(src: Tensor, dst: Tensor, scales: Tensor) -> None:
-    """Quantise whole bf16 chunks ``[N, C, Hkv, d]`` into an e4m3fn byte cache + ``[N, Hkv]`` scales."""
+    """Quantise whole 16-bit chunks ``[N, C, Hkv, d]`` into an e4m3fn byte cache + ``[N, Hkv]`` scales."""
     lib = _lib.load()
     _stream(src)  # device check first: there is no CPU path
-    _require(src.dtype == torch.bfloat16, "source chunks must be bf16")
+    _require(src.dtype in (torch.bfloat16, torch.float16), "source chunks must be bf16 or fp16")
     _require(dst.element_size() == 1, "destination cache must hold one byte per element")
     _require(scales.dtype == torch.float32 and scales.is_contiguous(), "scales must be contiguous fp32")
     ssc, sst, ssh = _cache_strides(src)
@@ -237,18 +237,19 @@ def quantize_chunks_fp8(src: Tensor, dst: Tensor, scales: Tensor) -> None:
     _require(tuple(dst.shape) == (N, C, H, D) and tuple(scales.shape) == (N, H), "shape mismatch")
     _require(ssh == D and dsh == D, "heads must be contiguous")
     _lib.check(lib.mi_kv_quantize_chunks_fp8(src.data_ptr(), ssc, sst, dst.data_ptr(), dsc, dst_t,
-                                             scales.data_ptr(), N, C, H, D, _stream(src)),
+                                             scales.data_ptr(), N, C, H, D, _dtype_code(src, "src"), _stream(src)),
                "mi_kv_quantize_chunks_fp8")
 
 
 def kv_append_decode_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor, k_scales: Tensor,
                          v_scales: Tensor, block_table: Tensor, kv_lens: Tensor, headroom: float = 2.0) -> None:
-    """Quantise and append one new bf16 token per request into an fp8 cache."""
+    """Quantise and append one new 16-bit token per request into an fp8 cache."""
     lib = _lib.load()
     _stream(key)  # device check first: there is no CPU path
     key, row, k_st = _rows(key, "key")
     value, _, v_st = _rows(value, "value")
-    _require(key.dtype == torch.bfloat16 and value.dtype == torch.bfloat16 and k_st == v_st, "K/V must be bf16 with equal strides")
+    _require(key.dtype in (torch.bfloat16, torch.float16) and value.dtype == key.dtype and k_st == v_st,
+             "K/V must share one 16-bit type and have equal strides")
     _require(k_cache.element_size() == 1 and v_cache.element_size() == 1, "fp8 caches hold one byte per element")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh) and sh == k_cache.size(3), "cache layout")
@@ -258,20 +259,20 @@ def kv_append_decode_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: T
     _lib.check(lib.mi_kv_append_decode_fp8(key.data_ptr(), value.data_ptr(), k_st, k_cache.data_ptr(), v_cache.data_ptr(),
                                            sc, st, k_scales.data_ptr(), v_scales.data_ptr(), block_table.data_ptr(),
                                            block_table.stride(0), kv_lens.data_ptr(), key.size(0), k_cache.size(1),
-                                           k_cache.size(2), k_cache.size(3), float(headroom), _stream(key)),
-               "mi_kv_append_decode_fp8")
+                                           k_cache.size(2), k_cache.size(3), float(headroom), _dtype_code(key, "key"),
+                                           _stream(key)), "mi_kv_append_decode_fp8")
 
 
 def kv_append_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor, k_scales: Tensor, v_scales: Tensor,
                   token_to_chunk_idx: Tensor, token_to_local_pos: Tensor, headroom: float = 2.0) -> None:
-    """Quantise and append bf16 tokens with explicit slots into an fp8 cache (prefill / mixed steps)."""
+    """Quantise and append 16-bit tokens with explicit slots into an fp8 cache (prefill / mixed steps)."""
     lib = _lib.load()
     _stream(key)  # device check first: there is no CPU path
     key, row, k_st = _rows(key, "key")
     value, _, v_st = _rows(value, "value")
     T = key.size(0)
-    _require(key.dtype == torch.bfloat16 and value.dtype == torch.bfloat16 and k_st == v_st and value.size(0) == T,
-             "K/V must be bf16 with equal shapes and strides")
+    _require(key.dtype in (torch.bfloat16, torch.float16) and value.dtype == key.dtype and k_st == v_st
+             and value.size(0) == T, "K/V must share one 16-bit type and have equal shapes and strides")
     _require(k_cache.element_size() == 1 and v_cache.element_size() == 1, "fp8 caches hold one byte per element")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh) and sh == k_cache.size(3) and row == k_cache.size(2) * sh,
@@ -283,7 +284,8 @@ def kv_append_fp8(key: Tensor, value: Tensor, k_cache: Tensor, v_cache: Tensor, 
     _lib.check(lib.mi_kv_append_fp8(key.data_ptr(), value.data_ptr(), k_st, k_cache.data_ptr(), v_cache.data_ptr(),
                                     sc, st, k_scales.data_ptr(), v_scales.data_ptr(), token_to_chunk_idx.data_ptr(),
                                     token_to_local_pos.data_ptr(), T, k_cache.size(1), k_cache.size(2),
-                                    k_cache.size(3), float(headroom), _stream(key)), "mi_kv_append_fp8")
+                                    k_cache.size(3), float(headroom), _dtype_code(key, "key"), _stream(key)),
+               "mi_kv_append_fp8")
 
 
 # ---------------------------------------------------------------------------------------------
@@ -326,7 +328,6 @@ def paged_decode_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, kv_lens:
     _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
     fp8 = k_cache.element_size() == 1
     _require(fp8 or k_cache.dtype == q3.dtype, "the KV cache must have the queries' 16-bit type, or be a one-byte fp8 type")
-    _require(not fp8 or q3.dtype == torch.bfloat16, "an fp8 cache needs bf16 queries")
     _require(v_cache.dtype == k_cache.dtype, "k_cache / v_cache dtypes differ")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
@@ -375,7 +376,6 @@ def paged_decode_attention_noalloc(q: Tensor, k_cache: Tensor, v_cache: Tensor, 
     _require(Dk == D and tuple(v_cache.shape) == tuple(k_cache.shape), "cache shape mismatch")
     fp8 = k_cache.element_size() == 1
     _require(fp8 or k_cache.dtype == q3.dtype, "the KV cache must have the queries' 16-bit type, or be a one-byte fp8 type")
-    _require(not fp8 or q3.dtype == torch.bfloat16, "an fp8 cache needs bf16 queries")
     _require(v_cache.dtype == k_cache.dtype, "k_cache / v_cache dtypes differ")
     sc, st, sh = _cache_strides(k_cache)
     _require(_cache_strides(v_cache) == (sc, st, sh), "k_cache / v_cache strides differ")
@@ -528,8 +528,8 @@ def paged_prefill_attention(q: Tensor, k_cache: Tensor, v_cache: Tensor, cu_seql
             q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
             k_scales.data_ptr(), v_scales.data_ptr(), block_table.data_ptr(), block_table.stride(0),
             cu_seqlens_q.data_ptr(), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
-            _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C, int(max_kv_len), 0, float(softmax_scale), tune,
-            stream), "mi_paged_prefill_attention_fp8")
+            _ptr(workspace), ws_bytes, T, R, Hq, Hkv, D, C, int(max_kv_len), 0, float(softmax_scale),
+            _dtype_code(q3, "q"), tune, stream), "mi_paged_prefill_attention_fp8")
         return out
     _lib.check(lib.mi_paged_prefill_attention(
         q3.data_ptr(), q3.stride(0), q3.stride(1), k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh,
@@ -747,7 +747,6 @@ def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value:
     if fp8:
         _require(v_cache.element_size() == 1 and k_scales is not None and v_scales is not None,
                  "byte caches hold e4m3 values and need k_scales / v_scales")
-        _require(ref.dtype == torch.bfloat16, "an fp8 cache needs bf16 queries / keys / values")
         for t in (k_scales, v_scales):
             _require(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (N, Hkv), "scales must be fp32 [n_chunks, Hkv]")
     else:
@@ -783,7 +782,7 @@ def decode_step_attention(query: Optional[Tensor], key: Optional[Tensor], value:
             k_cache.data_ptr(), v_cache.data_ptr(), sc, st, sh, k_scales.data_ptr(), v_scales.data_ptr(), float(headroom),
             block_table.data_ptr(), block_table.stride(0), kv_lens.data_ptr(), o3.data_ptr(), o3.stride(0), o3.stride(1),
             _ptr(workspace), ws_bytes, R, Hq, Hkv, D, C, int(split_tokens), float(softmax_scale),
-            int(bool(faithful_rounding)), tune, stream), "mi_decode_step_attention_fp8")
+            int(bool(faithful_rounding)), _dtype_code(ref, "query"), tune, stream), "mi_decode_step_attention_fp8")
         return out
     _lib.check(lib.mi_decode_step_attention(
         q_ptr, q_st, q_gst, k_ptr, k_st, k_hst, v_ptr, v_st, v_hst, _ptr(q_weight), _ptr(k_weight), float(eps),

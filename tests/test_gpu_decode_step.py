@@ -181,11 +181,12 @@ def test_fused_step_without_faithful_rounding_and_repeated_steps(mi, dev):
     _close(kc[:dummy], kc_ref[:dummy], 2e-2, "key cache after three steps")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("mixed", [False, True])
 @pytest.mark.parametrize("rotary", ["none", "half", "interleaved", "interleaved40"])
 @pytest.mark.parametrize("norm", [None, "rms"])
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (6, 2), (20, 1)])
-def test_fused_step_over_an_fp8_cache(mi, dev, Hq, Hkv, norm, rotary, mixed):
+def test_fused_step_over_an_fp8_cache(mi, dev, Hq, Hkv, norm, rotary, mixed, dtype):
     """The one-kernel step over an fp8-e4m3 cache: bytes and scales equal to the separate launches (norm / rotary
     with key_out, then the quantising append), tokens that open a chunk (lengths 1, 65, 129: they set the scale) and
     tokens that reuse a stored scale; output within 8e-3 of the separate launches and 6e-2 of the unquantised checker."""
@@ -194,7 +195,7 @@ def test_fused_step_over_an_fp8_cache(mi, dev, Hq, Hkv, norm, rotary, mixed):
     interleaved = rotary.startswith("interleaved")
     table = orn.rotary_table(4096, rot, base=500000.0, interleaved=interleaved) if rot else None
     lens_l = [0, 1, 2, 63, 64, 65, 66, 128, 129, 130, 700, 2049, 0, 193]
-    case, lens, qw, kw, pos = _step_case(mi, dev, Hq=Hq, Hkv=Hkv, d=d, chunk=chunk, lens=lens_l, dtype=torch.bfloat16,
+    case, lens, qw, kw, pos = _step_case(mi, dev, Hq=Hq, Hkv=Hkv, d=d, chunk=chunk, lens=lens_l, dtype=dtype,
                                          seed=Hq + rot)
     R = lens.numel()
     G = Hq // Hkv

@@ -72,10 +72,50 @@ def test_mismatched_types_are_rejected(mi, dev):
         mi.ops.paged_decode_attention(case.q.bfloat16(), case.k_cache, case.v_cache, case.kv_lens, case.block_table)
     with pytest.raises(ValueError, match="bf16 or fp16"):
         mi.ops.paged_decode_attention(case.q.float(), case.k_cache, case.v_cache, case.kv_lens, case.block_table)
-    k8 = torch.zeros(case.k_cache.shape, dtype=torch.uint8, device=dev)
-    sc = torch.ones(case.k_cache.size(0), 2, device=dev)
-    with pytest.raises(ValueError, match="fp8 cache needs bf16"):
-        mi.ops.paged_decode_attention(case.q, k8, k8, case.kv_lens, case.block_table, k_scales=sc, v_scales=sc)
+
+
+@pytest.mark.parametrize("d", [128, 64])
+def test_fp16_queries_over_an_fp8_cache(mi, dev, d):
+    """fp16 rows quantised to e4m3 (bytes and scales equal to the checker's), then decode attention with fp16
+    queries over the bytes: 2e-2 against the checker on the dequantised cache, 6e-2 against the unquantised one."""
+    cfg = mi.synthetic.DecodeConfig("fp8h", 6, 32, 8, d, 600, 5000, fp8=True, seed=1007)
+    case = mi.synthetic.make_decode_case(cfg, dev, dtype=F16)
+    N = case.k_cache.size(0)
+    k8 = torch.empty(case.k_cache.shape, dtype=torch.uint8, device=dev)
+    v8 = torch.empty_like(k8)
+    ks = torch.empty(N, cfg.Hkv, dtype=torch.float32, device=dev)
+    vs = torch.empty_like(ks)
+    mi.ops.quantize_chunks_fp8(case.k_cache, k8, ks)
+    mi.ops.quantize_chunks_fp8(case.v_cache, v8, vs)
+    torch.cuda.synchronize()
+    k8_ref, ks_ref = oa.quantize_chunks_fp8(case.k_cache.cpu())
+    v8_ref, vs_ref = oa.quantize_chunks_fp8(case.v_cache.cpu())
+    assert torch.equal(ks.cpu(), ks_ref) and torch.equal(vs.cpu(), vs_ref), "scales differ"
+    assert torch.equal(k8.cpu(), k8_ref) and torch.equal(v8.cpu(), v8_ref), "e4m3 bytes differ"
+    out = mi.ops.paged_decode_attention(case.q, k8, v8, case.kv_lens, case.block_table, k_scales=ks, v_scales=vs)
+    torch.cuda.synchronize()
+    assert out.dtype == F16
+    ref_q = oa.paged_decode_attention(case.q.cpu().squeeze(1), k8_ref, v8_ref, case.kv_lens.cpu(), case.block_table.cpu(),
+                                      k_scales=ks_ref, v_scales=vs_ref)
+    _close(out, ref_q, what="fp16 over fp8, dequantised cache")
+    ref = oa.paged_decode_attention(case.q.cpu().squeeze(1), case.k_cache.cpu(), case.v_cache.cpu(), case.kv_lens.cpu(),
+                                    case.block_table.cpu())
+    err = (out.float().cpu().squeeze(1) - ref).abs()
+    assert (err <= 6e-2 + 6e-2 * ref.abs()).all()
+    # the step's token, appended by the quantising decode append with fp16 rows
+    k8a, v8a, ksa, vsa = k8.clone(), v8.clone(), ks.clone(), vs.clone()
+    mi.ops.kv_append_decode_fp8(case.k_new, case.v_new, k8a, v8a, ksa, vsa, case.block_table, case.kv_lens, headroom=2.0)
+    torch.cuda.synchronize()
+    lens, bt = case.kv_lens.cpu(), case.block_table.cpu()
+    for r in range(lens.numel()):
+        pos = int(lens[r]) - 1
+        c, l = int(bt[r, pos // cfg.chunk]), pos % cfg.chunk
+        for src, c8, cs in ((case.k_new, k8a, ksa), (case.v_new, v8a, vsa)):
+            row = src.cpu()[r].view(cfg.Hkv, d)
+            scale = (2.0 * row.float().abs().amax(dim=1) / 448.0) if l == 0 else cs.cpu()[c]
+            if l == 0:
+                assert torch.equal(cs.cpu()[c], scale)
+            assert torch.equal(c8.cpu()[c, l], oa.quantize_token_fp8(row, scale))
 
 
 @pytest.mark.parametrize("kernel", ["two_phase", "two_phase_staggered", "two_phase_lock_step", "registers", "split_keys"])

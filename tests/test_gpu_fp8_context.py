@@ -15,13 +15,14 @@ from oracle import rope_norm as orn
 pytestmark = pytest.mark.gpu
 
 L, HQ, HKV, D, C = 2, 8, 2, 128, 64
+DT = torch.bfloat16   # the parameters' type; a test may switch it to fp16
 
 
 def _make_ctx(mi, dev, **kw):
     mi.DynamicInferenceContext.TOKEN_ROUNDER = 4
     mi.DynamicInferenceContext.REQUEST_ROUNDER = 4
     return mi.DynamicInferenceContext(
-        params_dtype=torch.bfloat16, num_layers=L, kv_channels=D, num_attention_heads=HKV,
+        params_dtype=DT, num_layers=L, kv_channels=D, num_attention_heads=HKV,
         max_sequence_length=256, buffer_size_gb=60 * (2 * L * C * HKV * D + 8 * L * HKV) / 1024**3,
         buffer_guaranteed_fraction=0.1, chunk_size_tokens=C, max_requests_override=16, max_tokens_override=512,
         kv_cache_dtype="fp8_e4m3", device=dev, **kw)
@@ -39,7 +40,7 @@ def test_fp8_sizing_and_buffers(mi, dev):
         assert k8.dtype == torch.uint8 and k8.shape == (60, C, HKV, D)
         ks, vs = ctx.key_value_scales(2)
         assert ks.data_ptr() == ctx.kv_scales[0, 1].data_ptr() and vs.data_ptr() == ctx.kv_scales[1, 1].data_ptr()
-        with pytest.raises(ValueError, match="bfloat16"):
+        with pytest.raises(ValueError, match="bfloat16 or float16"):
             mi.DynamicInferenceContext(params_dtype=torch.float32, num_layers=1, kv_channels=D, num_attention_heads=1,
                                        max_sequence_length=64, buffer_size_gb=0.001, buffer_guaranteed_fraction=0.1,
                                        chunk_size_tokens=C, kv_cache_dtype="fp8_e4m3", device=dev)
@@ -47,12 +48,14 @@ def test_fp8_sizing_and_buffers(mi, dev):
         mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER = saved
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("head_dim", [128, 64])
 @pytest.mark.parametrize("entry", ["fused", "unfused", "mixed_qkv"])
-def test_fp8_prefill_then_decode_steps(mi, dev, entry, head_dim):
-    global D
-    saved = (mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER, D)
+def test_fp8_prefill_then_decode_steps(mi, dev, entry, head_dim, dtype):
+    global D, DT
+    saved = (mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER, D, DT)
     D = head_dim   # (head_dim 64: decode steps take the separate launches, half-split pairs sit in other lanes there)
+    DT = dtype
     try:
         ctx = _make_ctx(mi, dev)
         N = ctx.chunk_allocator.chunk_count_total
@@ -65,9 +68,9 @@ def test_fp8_prefill_then_decode_steps(mi, dev, entry, head_dim):
         table_d = table.to(dev)
         layers, weights = [], []
         for l in range(L):
-            core = mi.PagedSelfAttentionCore(l + 1, D, qk_norm="rms", eps=1e-5, fused=entry != "unfused", device=dev)
-            qw = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
-            kw = (1 + 0.02 * torch.randn(D, generator=gen)).bfloat16()
+            core = mi.PagedSelfAttentionCore(l + 1, D, qk_norm="rms", eps=1e-5, fused=entry != "unfused", dtype=DT, device=dev)
+            qw = (1 + 0.02 * torch.randn(D, generator=gen)).to(DT)
+            kw = (1 + 0.02 * torch.randn(D, generator=gen)).to(DT)
             core.q_layernorm_weight.data.copy_(qw)
             core.k_layernorm_weight.data.copy_(kw)
             layers.append(core)
@@ -85,7 +88,7 @@ def test_fp8_prefill_then_decode_steps(mi, dev, entry, head_dim):
             lo = ctx.token_to_local_position_within_kv_chunk[:act].cpu()
             lens, bt = ctx.kv_seq_lengths.cpu(), ctx.block_table.cpu()
             for l in range(L):
-                mixed = torch.randn(n, 1, (HQ + 2 * HKV) * D, generator=gen).bfloat16()
+                mixed = torch.randn(n, 1, (HQ + 2 * HKV) * D, generator=gen).to(DT)
                 q, k, v = (t.contiguous() for t in orn.split_mixed_qkv(mixed, HQ, HKV))
                 qw, kw = weights[l]
                 qr = orn.norm_rope(q.squeeze(1), qpos, table, norm="rms", weight=qw, eps=1e-5)
@@ -118,4 +121,4 @@ def test_fp8_prefill_then_decode_steps(mi, dev, entry, head_dim):
             ctx.update_requests(mask, torch.randint(0, 100, (n_act,), generator=gen).to(dev))
         assert ctx.total_request_count == 4
     finally:
-        mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER, D = saved
+        mi.DynamicInferenceContext.TOKEN_ROUNDER, mi.DynamicInferenceContext.REQUEST_ROUNDER, D, DT = saved

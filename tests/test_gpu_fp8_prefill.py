@@ -23,13 +23,14 @@ def _fp8_case(mi, dev, **kw):
     return q, k8, v8, ks, vs, cu_q, lens, bt
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("pingpong", [1, 2])
 @pytest.mark.parametrize("Hq,Hkv,chunk", [(32, 8, 64), (8, 1, 128), (32, 2, 256), (16, 16, 64)])
-def test_fp8_mixed_prefill_and_decode(mi, dev, Hq, Hkv, chunk, pingpong, d):
+def test_fp8_mixed_prefill_and_decode(mi, dev, Hq, Hkv, chunk, pingpong, d, dtype):
     q, k8, v8, ks, vs, cu_q, lens, bt = _fp8_case(
         mi, dev, n_prefill=3, new_tokens=150, ctx_lo=0, ctx_hi=400, n_decode=5, dec_lo=1, dec_hi=700,
-        Hq=Hq, Hkv=Hkv, d=d, chunk=chunk, seed=Hq + Hkv + chunk)
+        Hq=Hq, Hkv=Hkv, d=d, chunk=chunk, seed=Hq + Hkv + chunk, dtype=dtype)
     mi.ops.set_tuning("prefill_two_phase", pingpong)
     try:
         out = mi.ops.paged_prefill_attention(q, k8, v8, cu_q, lens, bt, max_kv_len=int(lens.max()),
@@ -86,8 +87,9 @@ def test_fp8_prefill_rejects_what_it_cannot_run(mi, dev):
         mi.ops.paged_prefill_attention(q, k8, v8, cu_q, lens, bt)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "fp16"])
 @pytest.mark.parametrize("headroom", [2.0, 1.5])
-def test_fp8_append_many_tokens_matches_the_policy(mi, dev, headroom):
+def test_fp8_append_many_tokens_matches_the_policy(mi, dev, headroom, dtype):
     """Prompts that fill chunks, end inside a chunk, continue a partly filled chunk, plus padded rows
     that all point at one slot of the dummy chunk."""
     Hkv, d, chunk, N = 4, 128, 64, 24
@@ -104,8 +106,8 @@ def test_fp8_append_many_tokens_matches_the_policy(mi, dev, headroom):
     rows_l += [0] * pad
     T = len(rows_c)
     tc, tl = torch.tensor(rows_c), torch.tensor(rows_l)
-    key = (torch.randn(T, Hkv, d, generator=gen) * 3).bfloat16()
-    val = torch.randn(T, Hkv, d, generator=gen).bfloat16()
+    key = (torch.randn(T, Hkv, d, generator=gen) * 3).to(dtype)
+    val = torch.randn(T, Hkv, d, generator=gen).to(dtype)
     key[5:9, 1] = 0  # a few all-zero head rows
     k8 = torch.randint(0, 255, (N, chunk, Hkv, d), generator=gen, dtype=torch.uint8)
     v8 = torch.randint(0, 255, (N, chunk, Hkv, d), generator=gen, dtype=torch.uint8)
@@ -122,7 +124,7 @@ def test_fp8_append_many_tokens_matches_the_policy(mi, dev, headroom):
         assert torch.equal(got_c.cpu()[: N - 1], want_c[: N - 1])
     assert torch.equal(ksd.cpu()[5], ks[5]) and torch.equal(ksd.cpu()[6], ks[6])  # continued chunks keep their scale
     # a chunk filled by one call gets the same bytes and scale as the whole-chunk quantiser
-    full = torch.full((1, chunk, Hkv, d), 0, dtype=torch.bfloat16)
+    full = torch.full((1, chunk, Hkv, d), 0, dtype=dtype)
     full[0] = key[:64]
     b, s_ = oa.quantize_chunks_fp8(full)
     assert torch.equal(k8d.cpu()[3], b[0]) and torch.equal(ksd.cpu()[3], s_[0])
