@@ -458,6 +458,8 @@ def parse_args():
                     help="stream_read only: buffer size (default: the 1.2 GB one cfg2 launch streams)")
     ap.add_argument("--read-wgs-per-cu", type=int, default=2, help="stream_read only: workgroups per CU")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0, help="seconds of CPU work for the cpu_baseline leg")
+    ap.add_argument("--settle-s", type=float, default=0.25,
+                    help="decode workloads: seconds of untimed steps before the warm-up steps (clock settling; 0 = none)")
     ap.add_argument("--sustained-launches", type=int, default=1000,
                     help="cfg3: back-to-back launches of the tile kernel for the power-capped figure (0 = skip)")
     ap.add_argument("--no-other-configs", action="store_true",
@@ -793,12 +795,14 @@ def main():
                  or args.split_tokens or args.calibrate_copy_mib)
     if args.workload == "cfg2" and plain and not args.no_other_configs:
         others = {}
-        for name, steps in (("cfg3", 20), ("cfg4", 20), ("cfg5", 10)):
+        # (their own step counts, stated in each entry: a step is 1.2-1.4 ms, and the first dozen launches after a
+        # set-up run at a clock that has not settled, so a few more warm-up steps cost nothing and say more)
+        for name, steps, warmup in (("cfg3", 50, 10), ("cfg4", 30, 5), ("cfg5", 30, 5)):
             sub = copy.copy(args)
-            sub.workload, sub.steps, sub.warmup, sub.cpu_budget_s = name, min(args.steps, steps), min(args.warmup, 3), 3.0
+            sub.workload, sub.steps, sub.warmup, sub.cpu_budget_s = name, steps, warmup, 3.0
             torch.cuda.empty_cache()
             r = run_workload(sub, mi, lib, torch, dev)
-            others[name] = {k: r[k] for k in ("value", "unit", "steps", "ms_per_step", "dtype", "config", "roofline",
+            others[name] = {k: r[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "dtype", "config", "roofline",
                                               "roofline_decode_part", "separate_launches", "cpu_baseline") if k in r}
         result["other_configs"] = others
     print(json.dumps(result), flush=True)
@@ -922,6 +926,16 @@ def run_decode_config(args, mi, lib, torch, dev):
                     "frac": round(nbytes / (sep_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                     "traffic": MEASURED_HBM_TRAFFIC_BYTES.get(args.workload),
                     "traffic_source": TRAFFIC_SOURCE.get(args.workload)}
+    # The GPU's clocks take a few hundred launches to settle after the set-up (allocation, input generation, the
+    # host-side CPU legs of earlier workloads): steps until `settle_s` seconds have passed come before the W warm-up
+    # steps and the K timed ones, so that a short run (K = 20) measures the same steady state as a long one.
+    t_settle = time.perf_counter()
+    n_settle = 0
+    while time.perf_counter() - t_settle < args.settle_s:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
+        n_settle += 10
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -983,6 +997,7 @@ def run_decode_config(args, mi, lib, torch, dev):
             "batch": case.q.size(0), "q_heads": cfg.Hq, "kv_heads": cfg.Hkv, "head_dim": cfg.d,
             "chunk_tokens": cfg.chunk, "kv_tokens_total": int(lens_host.sum()), "kv_len_max": max_len,
             "algorithmic_bytes_per_step": nbytes,
+            "untimed_steps_before_warmup": n_settle,
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "decode_steps_per_sec": round(1e3 / ms_per_step, 1),
