@@ -266,3 +266,54 @@ def test_kernel_and_torch_op_sequence_agree_on_a_wide_batch(mi, Ctx, dev):
         if a.paused_request_count:
             assert a.paused_tokens.tolist() == b.paused_tokens.tolist()
     assert widest > 256 and saw_pause and saw_mixed and saw_finished
+
+
+def test_long_requests_release_many_table_columns(mi, Ctx, dev):
+    """Requests that own up to ~190 chunks each (a chunk table 200 columns wide): when they finish, their chunks go
+    back to the allocator's stack in the reference's order (rows ascending, columns ascending) -- more columns than
+    the 64 lanes that walk a row at a time -- and the survivors' table rows move.  Kernel path against the torch op
+    sequence, every state tensor and the stack itself compared after every step."""
+    set_rounder(Ctx, 4)
+    C = 4
+    kw = dict(params_dtype=torch.bfloat16, num_layers=1, kv_channels=8, num_attention_heads=1,
+              max_sequence_length=200 * C, buffer_size_gb=3000 * (2 * 2 * 1 * C * 1 * 8) / 1024**3,
+              buffer_guaranteed_fraction=0.05, chunk_size_tokens=C, max_requests_override=48,
+              max_tokens_override=8192, device=dev)
+    a = Ctx(fused_bookkeeping=True, **kw)
+    b = Ctx(fused_bookkeeping=False, **kw)
+    assert a.request_to_kv_chunk_ids.size(1) == 200
+    rng = random.Random(23)
+    next_id = 0
+    finished_long = 0
+    for step in range(30):
+        for _ in range(rng.randint(0, 6)):
+            n = rng.choice([rng.randint(1, 12), rng.randint(250, 760)])
+            toks = torch.tensor([rng.randint(0, 99) for _ in range(n)], device=dev)
+            outcome = []
+            for c in (a, b):
+                try:
+                    c.add_request(next_id, toks, 30)
+                    outcome.append("")
+                except mi.ContextOverflowError as e:
+                    outcome.append(type(e).__name__)
+            assert outcome[0] == outcome[1]
+            next_id += 1
+        n_act = a.total_request_count - a.paused_request_count
+        if n_act == 0:
+            continue
+        for c in (a, b):
+            c.initialize_attention_state()
+        act = slice(a.paused_request_count, a.total_request_count)
+        seq = (a.request_kv_length_offsets + a.request_query_lengths)[act]
+        budget = a.request_output_lengths[act]
+        mask = torch.tensor([(0 if (x + 1 >= y or rng.random() < 0.2) else 1) for x, y in zip(seq.tolist(), budget.tolist())],
+                            dtype=torch.int32, device=dev)
+        finished_long += int(((mask == 0) & (a.request_kv_chunk_counts[act] > 64)).sum())
+        new = torch.randint(0, 100, (n_act,), device=dev)
+        ga, gb = a.update_requests(mask, new), b.update_requests(mask, new)
+        assert (ga is None) == (gb is None) and (ga is None or ga.tolist() == gb.tolist())
+        assert _snapshot_product(a) == _snapshot_product(b), f"step {step}"
+        avail = a.chunk_allocator.chunk_count_avail
+        assert avail == b.chunk_allocator.chunk_count_avail
+        assert torch.equal(a.chunk_allocator.chunk_bag[:avail], b.chunk_allocator.chunk_bag[:avail]), f"stack order, step {step}"
+    assert finished_long >= 5, "the case this test is for did not occur"
