@@ -178,6 +178,12 @@ def run_secondary(args, mi, lib, torch, dev):
         dtype = "fp32 accumulation"
         timed_by_library = False
 
+    # (untimed steps until the clocks have settled after the set-up, as for the decode workloads)
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < args.settle_s:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -459,7 +465,7 @@ def parse_args():
     ap.add_argument("--read-wgs-per-cu", type=int, default=2, help="stream_read only: workgroups per CU")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0, help="seconds of CPU work for the cpu_baseline leg")
     ap.add_argument("--settle-s", type=float, default=0.25,
-                    help="decode workloads: seconds of untimed steps before the warm-up steps (clock settling; 0 = none)")
+                    help="seconds of untimed steps before the warm-up steps (clock settling; 0 = none)")
     ap.add_argument("--sustained-launches", type=int, default=1000,
                     help="cfg3: back-to-back launches of the tile kernel for the power-capped figure (0 = skip)")
     ap.add_argument("--no-other-configs", action="store_true",
