@@ -122,7 +122,8 @@ def run_secondary(args, mi, lib, torch, dev):
         pairs = n * (new * ctx + new * (new + 1) // 2)          # (query row, visible key) pairs per head
         flops = 2 * Hq * (dk + dv) * pairs
         nbytes = n * (new + ctx) * Hkv * (dk + dv) * 2 + n * new * Hq * (dk + dv) * 2
-        kernel = "paged_prefill_woven_kernel" if (not mla and dk == 128) else "paged_prefill_pp_kernel"
+        kernel = ("paged_prefill_woven_kernel" if (not mla and dk == 128 and args.prefill_kernel in (0, 3))
+                  else "paged_prefill_pp_kernel")
         what = (f"paged varlen causal attention, {n} x {new} new tokens over {ctx} cached, {Hq}/{Hkv} heads, "
                 f"keys {dk} / values {dv} wide, chunk 256")
         dtype = "bf16 (fp32 accumulate)"
@@ -464,6 +465,10 @@ def parse_args():
                     help="stream_read only: buffer size (default: the 1.2 GB one cfg2 launch streams)")
     ap.add_argument("--read-wgs-per-cu", type=int, default=2, help="stream_read only: workgroups per CU")
     ap.add_argument("--cpu-budget-s", type=float, default=12.0, help="seconds of CPU work for the cpu_baseline leg")
+    ap.add_argument("--prefill-kernel", type=int, default=0, choices=[0, 1, 2, 3, -1],
+                    help="MiTuning.prefill_two_phase for this run: 0 = the default (3), 1 = the two-phase tile kernel at "
+                         "every width, 2 = the same with its wave groups in lock-step, 3 = the one-stream kernel at "
+                         "head_dim 128, -1 = the register-only kernel")
     ap.add_argument("--settle-s", type=float, default=0.25,
                     help="seconds of untimed steps before the warm-up steps (clock settling; 0 = none)")
     ap.add_argument("--sustained-launches", type=int, default=1000,
@@ -497,7 +502,10 @@ class BoardPower:
         cap = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"))
         self.path = inp[0] if inp else None
         self.cap_w = self._read(cap[0]) if cap else None
+        clk = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.clk_path = clk[0] if clk else None   # the line marked '*' is the core clock right now
         self.samples = []
+        self.clk_samples = []
         self._stop = False
         self._thread = None
 
@@ -509,12 +517,26 @@ class BoardPower:
         except (OSError, ValueError):
             return None
 
+    @staticmethod
+    def _read_clock(path):
+        try:
+            with open(path) as f:
+                for line in f:
+                    if "*" in line:
+                        return float(line.split(":")[1].lower().replace("mhz", "").replace("*", "").strip())
+        except (OSError, ValueError, IndexError):
+            pass
+        return None
+
     def __enter__(self):
         import threading
         if self.path:
             def loop():
                 while not self._stop:
-                    self.samples.append((time.perf_counter(), self._read(self.path)))
+                    now = time.perf_counter()
+                    self.samples.append((now, self._read(self.path)))
+                    if self.clk_path:
+                        self.clk_samples.append((now, self._read_clock(self.clk_path)))
                     time.sleep(0.01)
             self._thread = threading.Thread(target=loop, daemon=True)
             self._thread.start()
@@ -528,6 +550,10 @@ class BoardPower:
     def mean_w(self, t_from: float, t_to: float):
         vals = [w for t, w in self.samples if w is not None and t_from <= t <= t_to]
         return round(sum(vals) / len(vals), 1) if vals else None
+
+    def mean_clock_mhz(self, t_from: float, t_to: float):
+        vals = [c for t, c in self.clk_samples if c is not None and t_from <= t <= t_to]
+        return round(sum(vals) / len(vals), 0) if vals else None
 
 
 def _time_cpu(torch, one_pass, budget_s: float = 12.0):
@@ -723,8 +749,10 @@ def run_mixed_batch(args, mi, lib, torch, dev):
         sustained = {"launches": args.sustained_launches, "kernel_ms": round(sus_ms, 5),
                      "achieved": None, "board_power_w": power.mean_w(t_a + 0.6 * (t_b - t_a), t_b),
                      "power_cap_w": power.cap_w,
-                     "what": "the prefill requests' tile kernel launched back to back; board power = mean of the "
-                             "driver's hwmon reading over the last 40 % of the run"}
+                     "core_clock_mhz": power.mean_clock_mhz(t_a + 0.6 * (t_b - t_a), t_b),
+                     "what": "the prefill requests' tile kernel launched back to back; board power and core clock = "
+                             "means of the driver's readings (hwmon power1_input, pp_dpm_sclk) over the last 40 % of "
+                             "the run; the clock's ceiling is 2400 MHz"}
 
     lq = (cu_q[1:] - cu_q[:-1]).cpu().long()
     lk = lens.cpu().long()
@@ -747,7 +775,8 @@ def run_mixed_batch(args, mi, lib, torch, dev):
                                + (" (fp8-e4m3 KV cache, quantising append)" if args.fp8_kv else ""),
                    "new_tokens": T, "requests": int(lens.numel()), "algorithmic_bytes_per_step": total_bytes,
                    "prefill_flops_per_step": flops},
-        "roofline": {"bound": "mfma", "kernel": "paged_prefill_pp_kernel" if args.fp8_kv else "paged_prefill_woven_kernel",
+        "roofline": {"bound": "mfma", "kernel": ("paged_prefill_pp_kernel" if (args.fp8_kv or args.prefill_kernel not in (0, 3))
+                                                  else "paged_prefill_woven_kernel"),
                      "achieved": round(flops / tile_ms / 1e9, 1),
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(flops / tile_ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4), "kernel_ms": round(tile_ms, 5),
@@ -793,12 +822,14 @@ def main():
     torch.cuda.set_device(dev)
     if args.subtiles:
         mi.ops.set_tuning("decode_tile_subtiles", args.subtiles)  # (passed with every call of the ops module)
+    if args.prefill_kernel:
+        mi.ops.set_tuning("prefill_two_phase", args.prefill_kernel)
 
     result = run_workload(args, mi, lib, torch, dev)
     # The default run carries the other single-GPU configurations beside the headline one: the mixed batch (cfg3),
     # the long-context batch (cfg4) and the fp8 cache (cfg5), each with its own roofline and a short CPU leg.
     plain = not (args.hip_graph or args.attention_only or args.separate_launches or args.fp8_kv or args.subtiles
-                 or args.split_tokens or args.calibrate_copy_mib)
+                 or args.split_tokens or args.calibrate_copy_mib or args.prefill_kernel)
     if args.workload == "cfg2" and plain and not args.no_other_configs:
         others = {}
         # (their own step counts, stated in each entry: a step is 1.2-1.4 ms, and the first dozen launches after a
