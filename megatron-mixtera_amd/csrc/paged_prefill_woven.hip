@@ -101,8 +101,9 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
   const int kend_wg = min(Lk, shift + min(q0_wg + SBQ, Lq));
   const int ntl_all = (kend_wg + kWvTile - 1) / kWvTile;  // staged tiles the rows of this workgroup can see
   const int n_split = SPLIT ? (int)gridDim.y : 1, split = SPLIT ? (int)blockIdx.y : 0;
-  const int tb = SPLIT ? (int)((int64_t)ntl_all * split / n_split) : 0;
-  const int te = SPLIT ? (int)((int64_t)ntl_all * (split + 1) / n_split) : ntl_all;
+  // (workgroup-uniform values the tile loop's bookkeeping is built from: held in scalar registers)
+  const int tb = __builtin_amdgcn_readfirstlane(SPLIT ? (int)((int64_t)ntl_all * split / n_split) : 0);
+  const int te = __builtin_amdgcn_readfirstlane(SPLIT ? (int)((int64_t)ntl_all * (split + 1) / n_split) : ntl_all);
   const int ntl = te - tb;  // this workgroup walks tiles [tb, te)
 
   const int q0 = q0_wg + wave * BQ;
@@ -137,8 +138,12 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
 
   if (ntl > 0) {
 #define MI_SB() __builtin_amdgcn_sched_barrier(0)
-    const uint8_t* kbase = p.kc + (int64_t)h * p.kv_sh * 2;
-    const uint8_t* vbase = p.vc + (int64_t)h * p.kv_sh * 2;
+    auto uniform64 = [](uint64_t x) {
+      return ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(x >> 32)) << 32) | (uint32_t)__builtin_amdgcn_readfirstlane((int)x);
+    };
+    const uint64_t kbase = uniform64((uint64_t)(uintptr_t)(p.kc + (int64_t)h * p.kv_sh * 2));
+    const uint64_t vbase = uniform64((uint64_t)(uintptr_t)(p.vc + (int64_t)h * p.kv_sh * 2));
+    const int last_key = __builtin_amdgcn_readfirstlane(last);
     const int64_t chunk_bytes = p.kv_sc * 2;
     const int tok_bytes = p.kv_st * 2;
     const int tiles_per_chunk = p.chunk / kWvTile;
@@ -150,32 +155,37 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
     // ---- this wavefront's five direct loads of a tile pair {key tile, value tile} -------------------------------
     // Load k of the pair's 36 (0-17: the key tile's line, 18-35: the value tile's) belongs to wavefront k % 8; the
     // fifth load of wavefronts 4-7 repeats their fourth, so that every wavefront issues five per tile.
+    // Loads 0 and 1 are key loads and loads 3 and 4 value loads for every wavefront; load 2 is a key load for
+    // wavefronts 0 and 1 only.
+    static_assert(kWvLoads == 18, "which of a wavefront's five loads belong to the key tile");
     uint32_t ld_off[5];   // per lane: where its piece of the load comes from, relative to the tile's first row
     uint32_t ld_dst[5];   // scalar: LDS offset of the load's 1 KiB inside its tile buffer
-    bool ld_key[5];       // scalar: the load belongs to the key tile
+    const bool third_is_key = wave < 2;
 #pragma unroll
     for (int i = 0; i < 5; ++i) {
       const int k = wave + 8 * i < 2 * kWvLoads ? wave + 8 * i : wave + 8 * i - 8;
-      ld_key[i] = k < kWvLoads;
-      const int kp = ld_key[i] ? k : k - kWvLoads;
-      ld_dst[i] = 1024u * (uint32_t)kp;
+      const bool is_key = k < kWvLoads;
+      const int kp = is_key ? k : k - kWvLoads;
+      ld_dst[i] = (uint32_t)__builtin_amdgcn_readfirstlane(1024 * kp);
       const uint32_t u = 64u * (uint32_t)kp + (uint32_t)lane;
       const uint32_t prow = (u * 3641u) >> 16, pcol = u - 18u * prow;
       ld_off[i] = prow * (uint32_t)tok_bytes + 16u * min(pcol, 15u);
     }
     // descriptor of a tile: its rows up to the request's last key (reads beyond return zeros)
-    auto tile_rsrc = [&](const uint8_t* base, int64_t off, uint32_t nrec) {
-      const uint64_t a = (uint64_t)(uintptr_t)(base + off);
+    // (pool addresses are user-space addresses: bits 48-63, the descriptor's stride and swizzle fields, are zero)
+    auto tile_rsrc = [&](uint64_t base, int64_t off, uint32_t nrec) {
+      const uint64_t a = base + (uint64_t)off;
       u32x4_t rs;
-      rs.x = __builtin_amdgcn_readfirstlane((uint32_t)a);
-      rs.y = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32) & 0xffffu);
-      rs.z = __builtin_amdgcn_readfirstlane(nrec);
+      rs.x = (uint32_t)a;
+      rs.y = (uint32_t)(a >> 32);
+      rs.z = nrec;
       rs.w = 0x00020000u;
       return rs;
     };
     auto issue_load = [&](int i, const u32x4_t& rs_k, const u32x4_t& rs_v, uint32_t kdst, uint32_t vdst) {
-      const u32x4_t rs = ld_key[i] ? rs_k : rs_v;
-      const uint32_t m0 = __builtin_amdgcn_readfirstlane((ld_key[i] ? kdst : vdst) + ld_dst[i]);
+      const bool is_key = i < 2 || (i == 2 && third_is_key);
+      const u32x4_t rs = is_key ? rs_k : rs_v;
+      const uint32_t m0 = (is_key ? kdst : vdst) + ld_dst[i];
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(m0), "v"(ld_off[i]), "s"(rs)
                    : "memory", "m0");
     };
@@ -183,8 +193,8 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
     struct Cursor { int tile, ci, tin; };
     auto cursor_at = [&](int t) {
       Cursor c;
-      c.tile = min(t, te - 1);
-      c.ci = c.tile / tiles_per_chunk;
+      c.tile = __builtin_amdgcn_readfirstlane(min(t, te - 1));
+      c.ci = __builtin_amdgcn_readfirstlane(c.tile / tiles_per_chunk);
       c.tin = c.tile - c.ci * tiles_per_chunk;
       return c;
     };
@@ -196,7 +206,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
       c.ci += wrap ? 1 : 0;
     };
     auto tile_off = [&](const Cursor& c, int pc) { return (int64_t)pc * chunk_bytes + (int64_t)c.tin * tile_bytes; };
-    auto tile_nrec = [&](const Cursor& c) { return (uint32_t)(min(last - c.tile * kWvTile, kWvTile - 1) + 1) * (uint32_t)tok_bytes; };
+    auto tile_nrec = [&](const Cursor& c) { return (uint32_t)(min(last_key - c.tile * kWvTile, kWvTile - 1) + 1) * (uint32_t)tok_bytes; };
     // block-table entries by scalar loads the compiler does not see (a vector load in the tile loop would make it
     // wait on the vector-memory counter, i.e. for the direct loads in flight)
     auto bt_request = [&](int ci) {
@@ -392,7 +402,7 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
       const u32x4_t rk0 = tile_rsrc(kbase, off_first[0], nrec_first[0]);
 #pragma unroll
       for (int i = 0; i < 5; ++i)
-        if (ld_key[i]) issue_load(i, rk0, rk0, ks_lds, ks_lds);  // key tile 0 -> Ks[0]
+        if (i < 2 || (i == 2 && third_is_key)) issue_load(i, rk0, rk0, ks_lds, ks_lds);  // key tile 0 -> Ks[0]
 #pragma unroll
       for (int t = 1; t <= DEPTH; ++t) {  // the pairs {key tile t -> Ks[t], value tile t - 1 -> Vs[t]}
         const u32x4_t rk = tile_rsrc(kbase, off_first[t], nrec_first[t]);
