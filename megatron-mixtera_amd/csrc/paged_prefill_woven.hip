@@ -82,20 +82,31 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
     }
   }
 
-  // request r's workgroups start at cu_q[r] / SBQ + r; heaviest query blocks first
+  // Query block sb of the batch: request r's blocks are cu_q[r] / SBQ + r onward; last block (most keys) first.
+  // The search takes 64 candidates per pass, one per lane (a pass is one trip to memory, and nothing of the
+  // workgroup's work can start before its request is known): the last request whose first block is not past this
+  // one.  The same pass fetches what is needed of that request.
   const int sb = (int)(gridDim.x / HV) - 1 - rank;
-  int lo = 0, hi = p.R - 1;
-  while (lo < hi) {
-    const int mid = (lo + hi + 1) >> 1;
-    if (p.cu_q[mid] / SBQ + mid <= sb) lo = mid; else hi = mid - 1;
+  int r = 0, q_begin = 0, q_end = 0, Lk = 0;
+  for (int n = p.R;;) {  // the answer lies in [r, r + n)
+    const int stride = (n + 63) >> 6;
+    const int idx = r + lane * stride;
+    const bool in = lane * stride < n;
+    const int cq = in ? p.cu_q[idx] : 0, cq1 = in ? p.cu_q[idx + 1] : 0, len = in ? p.lens[idx] : 0;
+    const int c = __builtin_popcountll(__builtin_amdgcn_ballot_w64(in && cq / SBQ + idx <= sb)) - 1;  // >= 0: the first candidate always qualifies
+    r += c * stride;
+    n = min(stride, n - c * stride);
+    if (stride == 1) {
+      q_begin = __builtin_amdgcn_readlane(cq, c);
+      q_end = __builtin_amdgcn_readlane(cq1, c);
+      Lk = __builtin_amdgcn_readlane(len, c);
+      break;
+    }
   }
-  const int r = lo;
-  const int q_begin = p.cu_q[r];
-  const int Lq = p.cu_q[r + 1] - q_begin;
+  const int Lq = q_end - q_begin;
   const int q0_wg = (sb - (q_begin / SBQ + r)) * SBQ;
   if (q0_wg >= Lq) return;  // workgroup-uniform
   if (p.skip_single && Lq == 1) return;
-  const int Lk = p.lens[r];
   const int shift = Lk - Lq;
   const int last = Lk - 1;
   const int kend_wg = min(Lk, shift + min(q0_wg + SBQ, Lq));
