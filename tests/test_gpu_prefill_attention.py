@@ -358,3 +358,24 @@ def test_a_bad_workspace_is_refused_before_anything_is_launched(mi, dev, fault):
     torch.cuda.synchronize()
     assert rc < 0 and b"workspace" in lib.mi_last_error()
     assert torch.isnan(out.float()).all(), "rows were written although the call was refused"
+
+
+@pytest.mark.parametrize("R", [65, 150, 4200])
+@pytest.mark.parametrize("kernel", [1, 3])
+def test_batches_of_many_requests(mi, dev, R, kernel):
+    """More requests than a wavefront has lanes: a workgroup of the one-stream tile kernel finds its request in
+    passes of 64 candidates (two passes from 65 requests on, three from 4 097 on), the two-phase kernel by bisection;
+    every request has a few new tokens behind a short context."""
+    gen = torch.Generator().manual_seed(R)
+    q_lens = torch.randint(2, 7, (R,), generator=gen)
+    ctx = torch.randint(0, 71, (R,), generator=gen)
+    Hq, Hkv, d, chunk = 8, 2, 128, 64
+    kv_lens = (q_lens + ctx).to(torch.int32)
+    cu_q = torch.zeros(R + 1, dtype=torch.int32)
+    cu_q[1:] = torch.cumsum(q_lens, 0)
+    bt, N = mi.synthetic.build_block_table(kv_lens, chunk, gen)
+    q = torch.randn(int(cu_q[-1]), Hq, d, generator=gen).bfloat16().to(dev)
+    kc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
+    vc = torch.randn(N, chunk, Hkv, d, generator=gen).bfloat16().to(dev)
+    with mi.ops.tuning(prefill_two_phase=kernel):
+        _check(mi, q, kc, vc, cu_q.to(dev), kv_lens.to(dev), bt.to(dev))
