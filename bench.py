@@ -46,7 +46,7 @@ MEASURED_HBM_TRAFFIC_BYTES = {
 _DECODE_TRAFFIC = ("profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                    "kernels as of commit 74dce26)")
 _MIXED_TRAFFIC = ("profiles/paged_prefill_woven_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
-                  "commit 74dce26)")
+                  "commit e60638b)")
 _MLA_HEADS_TRAFFIC = ("profiles/paged_mla_decode_heads_kernel_h128_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                       "kernel as of commit c8e09ff; the row pitch changed since, the traffic does not depend on it)")
 TRAFFIC_SOURCE = {"mla_decode_h128": _MLA_HEADS_TRAFFIC, "mla_decode_h128_long": _MLA_HEADS_TRAFFIC, "cfg2": _DECODE_TRAFFIC, "cfg2_step": _DECODE_TRAFFIC, "cfg4": _DECODE_TRAFFIC,
