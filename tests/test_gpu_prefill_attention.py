@@ -360,11 +360,11 @@ def test_a_bad_workspace_is_refused_before_anything_is_launched(mi, dev, fault):
     assert torch.isnan(out.float()).all(), "rows were written although the call was refused"
 
 
-@pytest.mark.parametrize("R", [65, 150, 4200])
+@pytest.mark.parametrize("R", [64, 65, 150, 4096, 4097, 4200])
 @pytest.mark.parametrize("kernel", [1, 3])
 def test_batches_of_many_requests(mi, dev, R, kernel):
     """More requests than a wavefront has lanes: a workgroup of the one-stream tile kernel finds its request in
-    passes of 64 candidates (two passes from 65 requests on, three from 4 097 on), the two-phase kernel by bisection;
+    passes of 64 candidates (one pass up to 64 requests, two up to 4 096, three beyond), the two-phase kernel by bisection;
     every request has a few new tokens behind a short context."""
     gen = torch.Generator().manual_seed(R)
     q_lens = torch.randint(2, 7, (R,), generator=gen)
