@@ -35,8 +35,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, published
 # read from inside the benchmark, so the figure is recorded here per workload; None = not collected.
 MEASURED_HBM_TRAFFIC_BYTES = {
     # decode workloads: "<cfg>" = the attention-only streaming kernel, "<cfg>_step" = the one-kernel decode step
-    "cfg2": 1_226_800_000, "cfg2_step": 1_215_100_000, "cfg4": 8_725_300_000, "cfg4_step": 8_635_100_000,
-    "cfg5": 9_071_100_000, "cfg5_step": 9_049_800_000,
+    "cfg2": 1_226_700_000, "cfg2_step": 1_215_000_000, "cfg4": 8_724_700_000, "cfg4_step": 8_634_800_000,
+    "cfg5": 9_070_200_000, "cfg5_step": 9_050_500_000,
     # the mixed step: tile kernel, stream kernel
     "cfg3_tile": 401_700_000, "cfg3_stream": 2_195_700_000,
     # multi-latent decode at 128 heads (reads + the partial results it writes)
@@ -44,7 +44,7 @@ MEASURED_HBM_TRAFFIC_BYTES = {
 # Where each figure above was read, so that a reader of the JSON line can tell a stale constant from a fresh one:
 # the summary file and the last commit that touched the kernel when the counters were collected.
 _DECODE_TRAFFIC = ("profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
-                   "kernels as of commit 74dce26)")
+                   "library as of commit b54c9eb)")
 _MIXED_TRAFFIC = ("profiles/paged_prefill_woven_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
                   "commit e60638b)")
 _MLA_HEADS_TRAFFIC = ("profiles/paged_mla_decode_heads_kernel_h128_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
