@@ -152,8 +152,9 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
     auto uniform64 = [](uint64_t x) {
       return ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(x >> 32)) << 32) | (uint32_t)__builtin_amdgcn_readfirstlane((int)x);
     };
-    const uint64_t kbase = uniform64((uint64_t)(uintptr_t)(p.kc + (int64_t)h * p.kv_sh * 2));
-    const uint64_t vbase = uniform64((uint64_t)(uintptr_t)(p.vc + (int64_t)h * p.kv_sh * 2));
+    // (48-bit addresses: what a descriptor's second word holds above them are its stride and swizzle fields)
+    const uint64_t kbase = uniform64((uint64_t)(uintptr_t)(p.kc + (int64_t)h * p.kv_sh * 2)) & 0xffffffffffffull;
+    const uint64_t vbase = uniform64((uint64_t)(uintptr_t)(p.vc + (int64_t)h * p.kv_sh * 2)) & 0xffffffffffffull;
     const int last_key = __builtin_amdgcn_readfirstlane(last);
     const int64_t chunk_bytes = p.kv_sc * 2;
     const int tok_bytes = p.kv_st * 2;
@@ -183,7 +184,6 @@ __global__ __launch_bounds__(512, 2) void paged_prefill_woven_kernel(PrefillPara
       ld_off[i] = prow * (uint32_t)tok_bytes + 16u * min(pcol, 15u);
     }
     // descriptor of a tile: its rows up to the request's last key (reads beyond return zeros)
-    // (pool addresses are user-space addresses: bits 48-63, the descriptor's stride and swizzle fields, are zero)
     auto tile_rsrc = [&](uint64_t base, int64_t off, uint32_t nrec) {
       const uint64_t a = base + (uint64_t)off;
       u32x4_t rs;
