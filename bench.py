@@ -46,7 +46,7 @@ MEASURED_HBM_TRAFFIC_BYTES = {
 _DECODE_TRAFFIC = ("profiles/decode_stream_kernels_hbm_traffic_cfg2_cfg4_cfg5.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                    "library as of commit b54c9eb)")
 _MIXED_TRAFFIC = ("profiles/paged_prefill_woven_kernel_cfg3_mfma.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, kernels as of "
-                  "commit e60638b)")
+                  "commit e60638b; the one later change of the tile kernel, e3f1ea0, masks two base addresses at its set-up)")
 _MLA_HEADS_TRAFFIC = ("profiles/paged_mla_decode_heads_kernel_h128_counters.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, "
                       "kernel as of commit c8e09ff; the row pitch changed since, the traffic does not depend on it)")
 TRAFFIC_SOURCE = {"mla_decode_h128": _MLA_HEADS_TRAFFIC, "mla_decode_h128_long": _MLA_HEADS_TRAFFIC, "cfg2": _DECODE_TRAFFIC, "cfg2_step": _DECODE_TRAFFIC, "cfg4": _DECODE_TRAFFIC,
