@@ -35,6 +35,7 @@ from .contexts import (  # noqa: F401
     WarmupEngineMode,
 )
 from .flash_attn_interface import (  # noqa: F401
+    _flash_attn_forward,
     flash_attn_varlen_func,
     flash_attn_with_kvcache,
     flash_mla_with_kvcache,

@@ -1,4 +1,4 @@
-"""The two flash-attn entry points the reference's dynamic path calls, on MI355X kernels.
+"""The flash-attn entry points the reference's dynamic path calls, on MI355X kernels.
 
 ``Attention.flash_decode_and_prefill`` (megatron/core/transformer/attention.py:470-601)
 resolves the module-level names ``flash_attn_with_kvcache`` and ``flash_attn_varlen_func``;
@@ -47,7 +47,8 @@ def _lengths_of(cu_seqlens_k: Tensor) -> Tensor:
 
 
 def _reject(**unsupported) -> None:
-    bad = [k for k, v in unsupported.items() if v not in (None, False, 0, 0.0, (-1, -1))]
+    # (a tensor is an argument given, whatever it holds: `tensor in (...)` would compare element values)
+    bad = [k for k, v in unsupported.items() if isinstance(v, Tensor) or v not in (None, False, 0, 0.0, (-1, -1))]
     if bad:
         raise NotImplementedError(f"unsupported flash-attn arguments on the paged MI355X path: {bad}")
 
@@ -113,6 +114,36 @@ def flash_attn_varlen_func(q: Tensor, k: Tensor, v: Tensor, cu_seqlens_q: Tensor
     return ops.paged_prefill_attention(q, k, v, cu_seqlens_q, kv_lens.to(torch.int32), block_table,
                                        softmax_scale=softmax_scale, max_kv_len=max_seqlen_k,
                                        k_scales=k_scales, v_scales=v_scales)
+
+
+def _flash_attn_forward(q: Tensor, k: Tensor, v: Tensor, k_new=None, v_new=None, qv=None, out: Optional[Tensor] = None,
+                        cu_seqlens_q: Optional[Tensor] = None, cu_seqlens_k: Optional[Tensor] = None,
+                        cu_seqlens_k_new=None, seqused_q=None, seqused_k: Optional[Tensor] = None,
+                        max_seqlen_q: Optional[int] = None, max_seqlen_k: Optional[int] = None,
+                        page_table: Optional[Tensor] = None, kv_batch_idx=None, leftpad_k=None, rotary_cos=None,
+                        rotary_sin=None, seqlens_rotary=None, q_descale=None, k_descale=None, v_descale=None,
+                        softmax_scale: Optional[float] = None, causal: bool = False, window_size=(-1, -1),
+                        attention_chunk: int = 0, softcap: float = 0.0, rotary_interleaved: bool = True,
+                        scheduler_metadata=None, num_splits: int = 0, pack_gqa=None, sm_margin: int = 0):
+    """The flash-attention-3 form of the paged varlen call (attention.py:510-544, taken when the reference finds
+    ``flashattn_hopper``): ``q`` ``[T, Hq, d]``, paged caches, ``cu_seqlens_q``, per-request key counts in
+    ``seqused_k`` (or the running sums ``cu_seqlens_k``), the block table as ``page_table``.  Returns
+    ``(out, None)``: the reference keeps the first element and discards the rest, and the log-sum-exp is not
+    produced.  Scheduling hints (``scheduler_metadata``, ``num_splits``, ``pack_gqa``, ``sm_margin``) have no
+    meaning here and are ignored; arguments that would change the result are rejected."""
+    _reject(k_new=k_new, v_new=v_new, qv=qv, cu_seqlens_k_new=cu_seqlens_k_new, seqused_q=seqused_q,
+            kv_batch_idx=kv_batch_idx, leftpad_k=leftpad_k, rotary_cos=rotary_cos, rotary_sin=rotary_sin,
+            seqlens_rotary=seqlens_rotary, q_descale=q_descale, k_descale=k_descale, v_descale=v_descale,
+            window_size=window_size, attention_chunk=attention_chunk, softcap=softcap)
+    if cu_seqlens_q is None:
+        raise NotImplementedError("only the varlen form (cu_seqlens_q given) exists on this path")
+    res = flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                                 softmax_scale=softmax_scale, causal=causal, block_table=page_table,
+                                 seqused_k=seqused_k)
+    if out is not None:
+        out.copy_(res)
+        res = out
+    return res, None
 
 
 def get_mla_metadata(cache_seqlens: Tensor, num_heads_per_head_k: int, num_heads_k: int):
